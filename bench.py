@@ -1,0 +1,333 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--sweep]
+
+Headline (BASELINE.json `metric`): fp32 SGEMM TFLOP/s at 8192^3 (alpha 1, beta 0.5,
+kernel 5 = wave tile on fp32 MFMA); the same JSON line carries the int32 scan at 2^30,
+the bf16 MFMA GEMM at 8192^3 and add_m at 2^24 under "also", each with its own roofline
+object. A "step" is one launch of the workload's entry point through the C ABI with
+inputs already resident in HBM. Timing: W untimed steps, then exactly K steps between
+two HIP events on the launch stream, device-synchronised on both sides.
+
+Every timed workload first passes a parity gate against a CPU check on the same data;
+a workload that fails the gate raises and reports nothing.
+
+cpu_baseline: the CPU oracle (oracle/prism_oracle.c, a scalar port, 1 core) timed on a
+bounded sample of the same workload, plus numpy/OpenBLAS and numpy.cumsum lines as
+additional baselines. Baselines, not targets.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+PEAK = {  # MI355X published peaks
+    "hbm_GBps": 8000.0,
+    "fp32_mfma_TFLOPs": 157.3,
+    "bf16_mfma_TFLOPs": 2500.0,
+}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def time_steps(fn, steps: int, warmup: int):
+    """Returns mean milliseconds per step, measured with HIP events on the current stream."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    beg = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    beg.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return beg.elapsed_time(end) / steps
+
+
+# ------------------------------------------------------------------ sgemm --
+
+def bench_sgemm(prism, M, N, K, alpha, beta, variant, steps, warmup, gate=True):
+    import torch
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0)
+    A = torch.rand((M, K), dtype=torch.float32, device="cuda", generator=g) * 2 - 1
+    B = torch.rand((K, N), dtype=torch.float32, device="cuda", generator=g) * 2 - 1
+    C0 = torch.rand((M, N), dtype=torch.float32, device="cuda", generator=g) * 2 - 1
+    C = C0.clone()
+    if gate:
+        prism.sgemm(M, N, K, alpha, A, B, beta, C, variant=variant)
+        torch.cuda.synchronize()
+        rows = torch.tensor(sorted({0, M // 3, M // 2, M - 1}), device="cuda")
+        ref = alpha * (A[rows].double() @ B.double()) + (beta * C0[rows].double() if beta != 0 else 0)
+        err = float((C[rows].double() - ref).abs().max())
+        bound = 1e-5 * np.sqrt(K) + abs(beta) * 2**-22
+        if not err <= bound:
+            raise RuntimeError(f"sgemm kernel {variant} {M}x{N}x{K} failed the parity gate: err {err} > {bound}")
+        C.copy_(C0)
+    # Like the reference's sweep, C accumulates across repeats (evals/4090_sgemm/main.cu:199-203);
+    # with |beta| < 1 it stays bounded.
+    ms = time_steps(lambda: prism.sgemm(M, N, K, alpha, A, B, beta, C, variant=variant), steps, warmup)
+    flops = 2.0 * M * N * K
+    tflops = flops / (ms * 1e-3) / 1e12
+    return {"ms": ms, "tflops": tflops,
+            "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK["fp32_mfma_TFLOPs"], "unit": "TFLOP/s",
+                         "frac": tflops / PEAK["fp32_mfma_TFLOPs"], "traffic": None}}
+
+
+# ------------------------------------------------------------------- scan --
+
+def bench_scan(prism, n, steps, warmup, gate=True):
+    import torch
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0)
+    x = torch.randint(-1000, 1001, (n,), dtype=torch.int32, device="cuda", generator=g)
+    out = torch.empty_like(x)
+    ws = torch.empty(prism.get_workspace_size(n), dtype=torch.uint8, device="cuda")
+    if gate:
+        prism.scan(x, out, ws)
+        torch.cuda.synchronize()
+        ok = int(out[0]) == int(x[0])
+        chunk = 1 << 26
+        total = 0
+        for s in range(0, n, chunk):
+            e = min(n, s + chunk)
+            lo = max(s, 1)
+            ok = ok and bool(torch.equal(out[lo:e] - out[lo - 1:e - 1], x[lo:e]))
+            total += int(x[s:e].sum(dtype=torch.int64))
+        ok = ok and int(out[-1]) == ((total + 2**31) % 2**32) - 2**31
+        if not ok:
+            raise RuntimeError(f"scan n={n} failed the parity gate")
+    # Out of place, so no restore is needed between steps; the workspace reset is part of the step,
+    # as the reference times its launcher's memsets (evals/4090_scan/main.cu:81-82).
+    ms = time_steps(lambda: prism.scan(x, out, ws), steps, warmup)
+    nbytes = 2.0 * 4 * n  # scan_harness.cuh:161
+    gbps = nbytes / (ms * 1e-3) / 1e9
+    return {"ms": ms, "GBps": gbps,
+            "roofline": {"bound": "hbm", "achieved": gbps, "peak": PEAK["hbm_GBps"], "unit": "GB/s",
+                         "frac": gbps / PEAK["hbm_GBps"], "traffic": None}}
+
+
+# ------------------------------------------------------------------ add_m --
+
+def bench_add_m(prism, n, steps, warmup, gate=True):
+    import torch
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0)
+    x = torch.randint(-2**20, 2**20, (n,), dtype=torch.int32, device="cuda", generator=g)
+    y = torch.empty_like(x)
+    if gate:
+        prism.add_m(x, y, 7)
+        torch.cuda.synchronize()
+        if not torch.equal(y, x + 7):
+            raise RuntimeError("add_m failed the parity gate")
+    ms = time_steps(lambda: prism.add_m(x, y, 7), steps, warmup)
+    gbps = 8.0 * n / (ms * 1e-3) / 1e9
+    return {"ms": ms, "GBps": gbps,
+            "roofline": {"bound": "hbm", "achieved": gbps, "peak": PEAK["hbm_GBps"], "unit": "GB/s",
+                         "frac": gbps / PEAK["hbm_GBps"], "traffic": None}}
+
+
+# -------------------------------------------------------------- bf16 gemm --
+
+def bench_gemm_bf16(prism, n, steps, warmup, gate=True):
+    import torch
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0)
+    A = torch.randn((n, n), dtype=torch.float32, device="cuda", generator=g).to(torch.bfloat16)
+    B = torch.randn((n, n), dtype=torch.float32, device="cuda", generator=g).to(torch.bfloat16)
+    D = torch.empty((n, n), dtype=torch.float32, device="cuda")
+    if gate:
+        prism.gemm_bf16(A, B, D)
+        torch.cuda.synchronize()
+        rows = torch.tensor(sorted({0, n // 3, n // 2, n - 1}), device="cuda")
+        ref = A[rows].double() @ B.double().T
+        err = float((D[rows].double() - ref).abs().max())
+        if not err <= 1e-3 * float(ref.abs().max()):
+            raise RuntimeError(f"gemm_bf16 n={n} failed the parity gate: err {err}")
+    ms = time_steps(lambda: prism.gemm_bf16(A, B, D), steps, warmup)
+    tflops = 2.0 * n * n * n / (ms * 1e-3) / 1e12
+    return {"ms": ms, "tflops": tflops,
+            "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK["bf16_mfma_TFLOPs"], "unit": "TFLOP/s",
+                         "frac": tflops / PEAK["bf16_mfma_TFLOPs"], "traffic": None}}
+
+
+# ----------------------------------------------------------- CPU baselines --
+
+def cpu_baseline_sgemm(n=8192, rows=32):
+    """Oracle (scalar fmaf port, 1 core) on the first `rows` rows of the n^3 problem."""
+    import oracle
+    A, B, Cm = oracle.gen_sgemm(rows, n, n, seed=0)
+    t0 = time.perf_counter()
+    oracle.sgemm_fma(1.0, A, B, 0.5, Cm)
+    dt = time.perf_counter() - t0
+    return {"value": 2.0 * rows * n * n / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": f"oracle_sgemm_fma on the first {rows} rows of C ({rows}x{n}x{n}), {dt:.1f} s"}
+
+
+def cpu_blas_sgemm(n=4096):
+    rng = np.random.default_rng(0)
+    A = rng.random((n, n), dtype=np.float32)
+    B = rng.random((n, n), dtype=np.float32)
+    Cm = rng.random((n, n), dtype=np.float32)
+    A @ B  # warm
+    t0 = time.perf_counter()
+    np.float32(1.0) * (A @ B) + np.float32(0.5) * Cm
+    dt = time.perf_counter() - t0
+    threads = None
+    try:
+        from threadpoolctl import threadpool_info
+        threads = max((p.get("num_threads", 0) for p in threadpool_info()), default=None)
+    except Exception:
+        pass
+    return {"value": 2.0 * n**3 / dt / 1e12, "unit": "TFLOP/s", "cores": threads or os.cpu_count(),
+            "kind": "numpy/OpenBLAS sgemm", "sample": f"{n}^3, alpha*(A@B)+beta*C, {dt:.2f} s",
+            "os_cpu_count": os.cpu_count()}
+
+
+def cpu_baseline_scan(n=1 << 28):
+    import oracle
+    x = oracle.gen_scan(n, seed=0)
+    t0 = time.perf_counter()
+    oracle.scan_cpu(x)
+    dt = time.perf_counter() - t0
+    t1 = time.perf_counter()
+    np.cumsum(x, dtype=np.int32)
+    dt_np = time.perf_counter() - t1
+    return {"value": 8.0 * n / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"oracle_scan_cpu (serial loop of scan_harness.cuh:30-36) on n=2^{n.bit_length() - 1}, {dt:.2f} s",
+            "numpy_cumsum_GBps": 8.0 * n / dt_np / 1e9}
+
+
+def cpu_baseline_add_m(n=1 << 24):
+    import oracle
+    x = oracle.gen_add_m(n, seed=0)
+    t0 = time.perf_counter()
+    oracle.add_m(x, 7)
+    dt = time.perf_counter() - t0
+    t1 = time.perf_counter()
+    x + np.int32(7)
+    dt_np = time.perf_counter() - t1
+    return {"value": 8.0 * n / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"oracle_add_m on n=2^24, {dt * 1e3:.1f} ms", "numpy_GBps": 8.0 * n / dt_np / 1e9}
+
+
+# ------------------------------------------------------------------- main --
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="all", choices=["all", "sgemm", "scan", "gemm_bf16", "add_m"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--sweep", action="store_true", help="also time every BASELINE config (table on stderr)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path has no multi-GPU part); run with --gpus 1",
+              file=sys.stderr)
+        return 2
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+    import prism_amd as prism
+    info = prism.device_info()
+    log(f"device: {info}")
+    K, W = args.steps, args.warmup
+    want = lambda w: args.workload in ("all", w)
+
+    res = {}
+    if want("sgemm"):
+        res["sgemm"] = bench_sgemm(prism, 8192, 8192, 8192, 1.0, 0.5, 5, K, W)
+        log("sgemm 8192^3 kernel 5:", res["sgemm"])
+    if want("scan"):
+        res["scan"] = bench_scan(prism, 1 << 30, K, W)
+        log("scan 2^30:", res["scan"])
+    if want("gemm_bf16"):
+        res["gemm_bf16"] = bench_gemm_bf16(prism, 8192, K, W)
+        log("gemm_bf16 8192^3:", res["gemm_bf16"])
+    if want("add_m"):
+        res["add_m"] = bench_add_m(prism, 1 << 24, max(K, 50), W)
+        log("add_m 2^24:", res["add_m"])
+
+    if args.sweep:
+        sweep = {}
+        for n in (1024, 2048, 4096, 8192):
+            for v in (1, 2, 3, 6, 4, 5):
+                if n == 8192 and v in (1, 2, 3):
+                    k, w = 2, 1
+                else:
+                    k, w = (5, 1) if n >= 4096 else (10, 2)
+                r = bench_sgemm(prism, n, n, n, 1.0, 0.5, v, k, w, gate=(v == 5))
+                sweep[f"sgemm_k{v}_{n}"] = r
+                log(f"  sgemm kernel {v} {n}^3: {r['ms']:.3f} ms  {r['tflops']:.2f} TFLOP/s  "
+                    f"({100 * r['roofline']['frac']:.1f}% of fp32 MFMA peak)")
+        for (M, N, Kd) in ((4096, 4096, 128), (128, 4096, 4096), (8191, 4097, 1023), (16384, 16384, 512)):
+            r = bench_sgemm(prism, M, N, Kd, 1.0, 0.0, 5, 10, 2)
+            sweep[f"sgemm_k5_{M}x{N}x{Kd}"] = r
+            log(f"  sgemm kernel 5 {M}x{N}x{Kd}: {r['ms']:.3f} ms  {r['tflops']:.2f} TFLOP/s")
+        for p in (20, 24, 28, 30):
+            r = bench_scan(prism, 1 << p, 20, 3)
+            sweep[f"scan_2p{p}"] = r
+            log(f"  scan 2^{p}: {r['ms']:.4f} ms  {r['GBps']:.1f} GB/s ({100 * r['roofline']['frac']:.1f}% of HBM peak)")
+        for n in (4096, 8192, 16384):
+            r = bench_gemm_bf16(prism, n, 8, 2)
+            sweep[f"gemm_bf16_{n}"] = r
+            log(f"  gemm_bf16 {n}^3: {r['ms']:.3f} ms  {r['tflops']:.1f} TFLOP/s "
+                f"({100 * r['roofline']['frac']:.1f}% of bf16 MFMA peak)")
+        os.makedirs("gpurun_out", exist_ok=True)
+        with open("gpurun_out/sweep.json", "w") as f:
+            json.dump(sweep, f, indent=1)
+
+    cpu = {}
+    if not args.no_cpu_baseline:
+        if want("sgemm"):
+            cpu["sgemm"] = cpu_baseline_sgemm()
+            cpu["sgemm_blas"] = cpu_blas_sgemm()
+        if want("scan"):
+            cpu["scan"] = cpu_baseline_scan()
+        if want("add_m"):
+            cpu["add_m"] = cpu_baseline_add_m()
+        log("cpu baselines:", cpu)
+
+    head_name = "sgemm" if "sgemm" in res else next(iter(res))
+    head = res[head_name]
+    if head_name in ("sgemm", "gemm_bf16"):
+        metric = {"sgemm": "SGEMM TFLOP/s @8192^3 fp32", "gemm_bf16": "bf16 GEMM TFLOP/s @8192^3"}[head_name]
+        value, unit = head["tflops"], "TFLOP/s"
+        dtype = "f32" if head_name == "sgemm" else "bf16"
+    else:
+        metric = {"scan": "int32 scan GB/s @2^30", "add_m": "add_m GB/s @2^24"}[head_name]
+        value, unit = head["GBps"], "GB/s"
+        dtype = "i32"
+    workload = {"sgemm": "sgemm M=N=K=8192 alpha=1 beta=0.5 kernel 5 (wave tile, fp32 MFMA)",
+                "scan": "inclusive scan int32 n=2^30, values in [-1000,1000]",
+                "gemm_bf16": "D=A@B^T bf16 in, fp32 out, M=N=K=8192",
+                "add_m": "y=x+7 int32 n=2^24"}[head_name]
+    line = {
+        "metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": head["ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dtype, "data": "synthetic",
+        "config": {"workload": workload, "device": info["name"], "cu_count": info["cu_count"]},
+        "roofline": head["roofline"],
+        "cpu_baseline": cpu.get(head_name),
+        "also": {k: {kk: vv for kk, vv in v.items()} for k, v in res.items() if k != head_name},
+        "cpu_baselines_also": {k: v for k, v in cpu.items() if k != head_name},
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,159 @@
+/*
+ * prism_amd.h - C ABI of libprism_amd.so: the MI355X (gfx950) kernels behind the
+ * host launchers of manya-bansal/prism's evaluation harnesses.
+ *
+ * Conventions shared by every entry point
+ *   - All data pointers are DEVICE pointers owned by the caller (a raw
+ *     hipMalloc pointer, or tensor.data_ptr() of a PyTorch-ROCm tensor).
+ *   - `stream` is a hipStream_t passed as void*; NULL means the default stream.
+ *   - Calls are asynchronous: they enqueue work and return. The caller
+ *     synchronises, as the reference harnesses do after their launchers.
+ *   - Functions returning int return 0 on success, otherwise a non-zero
+ *     hipError_t value (1 = invalid argument); prism_last_error_string() then
+ *     describes the failure for the calling thread.
+ *   - No entry point reads or keeps host-side state between calls, so all of
+ *     them are re-entrant and may be used from several host threads.
+ *
+ * "Reference" citations below are paths in the manya-bansal/prism tree.
+ */
+#ifndef PRISM_AMD_H
+#define PRISM_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------ misc -- */
+
+/* Library version, "major.minor.patch". */
+const char* prism_version(void);
+
+/* Message for the last failure on the calling thread ("" if none). */
+const char* prism_last_error_string(void);
+
+/*
+ * Properties of the current HIP device, for the roofline report. Any pointer
+ * may be NULL. clock_khz is the device's peak engine clock, lds_bytes the LDS
+ * available to one workgroup, hbm_bytes the total device memory.
+ */
+int prism_device_info(int* cu_count, int* clock_khz, int* wavefront_size,
+                      size_t* lds_bytes, size_t* hbm_bytes, char* name,
+                      size_t name_len);
+
+/*
+ * Host-side evaluation of the workgroup-id -> output-tile map the two MFMA
+ * GEMM kernels use (the role of Schedule, evals/h100_bench/utils.cuh:277-307,
+ * redone for 8 XCDs). Runs on the CPU; lets a caller or test check that the map
+ * visits every tile of a tiles_m x tiles_n grid exactly once.
+ */
+int prism_tile_coords(int workgroup_id, int tiles_m, int tiles_n, int* tile_m, int* tile_n);
+
+/* ----------------------------------------------------------------- add_m -- */
+
+/*
+ * y[i] = x[i] + m for i in [0, n), int32 with two's-complement wrap-around.
+ * Replaces the kernel Prism emits for `add_m_thread`
+ * (examples/add_m_thread.py:10-19, generated text README.md:133-140), whose
+ * signature is add_m(x, y, m) with one thread per element and no bound; here
+ * the element count is explicit. x == y is allowed.
+ */
+int prism_add_m(const int32_t* x, int32_t* y, int32_t m, size_t n, void* stream);
+
+/* ------------------------------------------------------------------ scan -- */
+
+/*
+ * Bytes of device workspace prism_scan_i32 / prism_launch_scan need for n
+ * elements. Replaces scan_gpu::get_workspace_size
+ * (evals/4090_scan/main.cu:63-66). Never 0, so a caller may always allocate it.
+ */
+size_t prism_scan_workspace_bytes(size_t n);
+
+/*
+ * Inclusive prefix sum, out[i] = in[0] + ... + in[i] modulo 2^32 (identical
+ * bit patterns for int32 and uint32). Single pass with decoupled look-back
+ * between tiles. Any n >= 0; in == out is allowed (in-place, as the reference
+ * runs); partial overlap is not. The workspace contents on entry do not
+ * matter: the call resets it itself, as the reference launcher does
+ * (evals/4090_scan/main.cu:81-82). Two calls that share a workspace must be
+ * ordered on one stream.
+ * Replaces scan_kernel + its device helpers (examples/scan.py:23-227,
+ * generated/scan_kernel.cu:1-29).
+ */
+int prism_scan_i32(const int32_t* in, int32_t* out, size_t n, void* workspace,
+                   size_t workspace_bytes, void* stream);
+
+/*
+ * The reference launcher's own shape: in-place on x, default stream, returns
+ * the device pointer that holds the result (x) or NULL on failure.
+ * Replaces scan_gpu::launch_scan (evals/4090_scan/main.cu:68-86). Unlike the
+ * reference, n need not be a multiple of 16384. The workspace must hold at
+ * least prism_scan_workspace_bytes(n) bytes.
+ */
+uint32_t* prism_launch_scan(size_t n, uint32_t* x, void* workspace);
+
+/* ----------------------------------------------------------------- sgemm -- */
+
+/* Kernel numbers accepted by prism_sgemm / prism_run_my_kernel. */
+enum {
+    PRISM_SGEMM_BEST = 0,             /* alias of PRISM_SGEMM_WAVE_TILE                        */
+    PRISM_SGEMM_NAIVE = 1,            /* my_sgemm_kernel_1: one thread per C element            */
+    PRISM_SGEMM_COALESCED = 2,        /* my_sgemm_kernel_2: 32x32 tile thread remap             */
+    PRISM_SGEMM_LDS_BLOCK = 3,        /* sgemm_shared_mem_block<32> (the eval's "kernel 3")     */
+    PRISM_SGEMM_THREAD_TILE = 4,      /* my_sgemm_kernel_4: 8x8 thread tile, vector loads       */
+    PRISM_SGEMM_WAVE_TILE = 5,        /* my_sgemm_kernel_5: wave tile, here on fp32 MFMA        */
+    PRISM_SGEMM_THREAD_TILE_SCALAR = 6 /* my_sgemm_kernel_3: 8x8 thread tile, scalar staging     */
+};
+
+/*
+ * C = alpha * A @ B + beta * C, fp32, row-major, A is MxK, B is KxN, C is MxN,
+ * any M, N, K >= 0. When beta == 0, C is never read (NaN/Inf in it do not
+ * propagate). `variant` selects the kernel (enum above).
+ * Replaces run_my_sgemm_1..5 (evals/4090_sgemm/runner.cu:135-243) and the
+ * kernels they launch (generated/my_sgemm_kernel_{1,2,3,4,5}.cu,
+ * generated/sgemm_shared_mem_block.cu, evals/4090_sgemm/my_kernel_utils.cuh:13-90).
+ */
+int prism_sgemm(int variant, int M, int N, int K, float alpha, const float* A,
+                const float* B, float beta, float* C, void* stream);
+
+/*
+ * The reference dispatcher's own shape: default stream, kernel numbers 1..5.
+ * Replaces run_my_kernel (evals/4090_sgemm/runner.cuh:28-29,
+ * runner.cu:245-267). The reference throws std::invalid_argument for an
+ * unknown number; this returns 1 and sets the error string.
+ */
+int prism_run_my_kernel(int my_kernel_num, int M, int N, int K, float alpha,
+                        float* A, float* B, float beta, float* C);
+
+/* ------------------------------------------------------------- bf16 gemm -- */
+
+/*
+ * D = A @ B^T with bf16 inputs and fp32 accumulation on MFMA.
+ * A is MxK row-major bf16, B is NxK row-major bf16 (both K-contiguous, the
+ * operand layout of the reference's h100_matmul), D is MxN row-major fp32.
+ * Any M, N, K >= 0 (no K tail is dropped). bf16 values are passed as their
+ * 16-bit patterns.
+ * Replaces cutlass_my_h100_match_no_tail (examples/h100_matmul.py:20-297,
+ * generated/cutlass_my_h100_match_no_tail.cu:1-370) with an fp32 result.
+ */
+int prism_gemm_bf16(int M, int N, int K, const uint16_t* A, const uint16_t* B,
+                    float* D, void* stream);
+
+/*
+ * The reference launcher's own shape and output layout: C is bf16,
+ * COLUMN-major MxN (element (m, n) at C[n * M + m],
+ * generated/cutlass_my_h100_match_no_tail.cu:313,347-354), fp32 accumulators
+ * rounded to bf16 (round-to-nearest-even) on store; default stream; DB is
+ * unused, as in the reference. Replaces prism_h100::runmyh100
+ * (evals/h100_bench/utils.cuh:504-533). Holds no cached state, so unlike the
+ * reference it may be called with changing shapes and pointers.
+ */
+int prism_runmyh100(int M, int N, int K, const uint16_t* A, const uint16_t* B,
+                    uint16_t* C, int* DB);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PRISM_AMD_H */

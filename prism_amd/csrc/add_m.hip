@@ -1,0 +1,107 @@
+// add_m: y[i] = x[i] + m over int32 (wrap-around), the streaming plumbing kernel.
+// Semantics follow the kernel Prism prints for add_m_thread
+// (examples/add_m_thread.py:10-19; text in README.md:133-140): one element per
+// thread id, y[tid] = x[tid] + m. Here every lane moves 16 B per access and the
+// element count is an argument, so any n is legal.
+//
+// HBM-bound: 8 algorithmic bytes per element (one 4 B read, one 4 B write).
+#include "common.h"
+
+namespace prism {
+namespace {
+
+constexpr int kAddBlock = 256;
+constexpr int kAddUnroll = 4;  // 16 B accesses per lane per block pass
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// Each block owns kAddBlock * kAddUnroll consecutive 16 B packets; within the
+// block, access u of lane t is packet (u * kAddBlock + t), so a wavefront always
+// touches 1 KiB of contiguous memory per instruction.
+__global__ __launch_bounds__(kAddBlock) void add_m_vec4_kernel(const u32x4* __restrict__ x,
+                                                               u32x4* __restrict__ y, uint32_t m,
+                                                               size_t n_vec) {
+    const size_t base = static_cast<size_t>(blockIdx.x) * (kAddBlock * kAddUnroll) + threadIdx.x;
+    u32x4 v[kAddUnroll];
+#pragma unroll
+    for (int u = 0; u < kAddUnroll; ++u) {
+        const size_t i = base + static_cast<size_t>(u) * kAddBlock;
+        if (i < n_vec) v[u] = __builtin_nontemporal_load(&x[i]);
+    }
+#pragma unroll
+    for (int u = 0; u < kAddUnroll; ++u) {
+        const size_t i = base + static_cast<size_t>(u) * kAddBlock;
+        if (i < n_vec) __builtin_nontemporal_store(v[u] + m, &y[i]);
+    }
+}
+
+// Same as above when x and y are the same buffer (no __restrict__ promise).
+__global__ __launch_bounds__(kAddBlock) void add_m_vec4_inplace_kernel(u32x4* xy, uint32_t m,
+                                                                       size_t n_vec) {
+    const size_t base = static_cast<size_t>(blockIdx.x) * (kAddBlock * kAddUnroll) + threadIdx.x;
+    u32x4 v[kAddUnroll];
+#pragma unroll
+    for (int u = 0; u < kAddUnroll; ++u) {
+        const size_t i = base + static_cast<size_t>(u) * kAddBlock;
+        if (i < n_vec) v[u] = xy[i];
+    }
+#pragma unroll
+    for (int u = 0; u < kAddUnroll; ++u) {
+        const size_t i = base + static_cast<size_t>(u) * kAddBlock;
+        if (i < n_vec) xy[i] = v[u] + m;
+    }
+}
+
+// One element per thread: the tail of a vector launch, or the whole array when
+// a pointer is not 16 B aligned. x may alias y.
+__global__ __launch_bounds__(kAddBlock) void add_m_scalar_kernel(const uint32_t* x, uint32_t* y,
+                                                                 uint32_t m, size_t first,
+                                                                 size_t n) {
+    const size_t i = first + static_cast<size_t>(blockIdx.x) * kAddBlock + threadIdx.x;
+    if (i < n) y[i] = x[i] + m;
+}
+
+}  // namespace
+
+int launch_add_m(const int32_t* x_, int32_t* y_, int32_t m_, size_t n, hipStream_t s) {
+    if (n == 0) return 0;
+    if (x_ == nullptr || y_ == nullptr) return fail(1, "prism_add_m: null pointer with n=%zu", n);
+    if (!aligned4(x_) || !aligned4(y_)) return fail(1, "prism_add_m: pointers must be 4-byte aligned");
+    const uint32_t* x = reinterpret_cast<const uint32_t*>(x_);
+    uint32_t* y = reinterpret_cast<uint32_t*>(y_);
+    const uint32_t m = static_cast<uint32_t>(m_);
+    // Overlap other than exact aliasing would make the result depend on the
+    // order blocks run in.
+    if (x != y) {
+        const uintptr_t xa = reinterpret_cast<uintptr_t>(x), ya = reinterpret_cast<uintptr_t>(y);
+        const uintptr_t bytes = n * sizeof(uint32_t);
+        if (xa < ya + bytes && ya < xa + bytes)
+            return fail(1, "prism_add_m: x and y overlap without being equal");
+    }
+
+    size_t n_vec = 0;
+    if (aligned16(x) && aligned16(y)) n_vec = n / 4;
+    if (n_vec > 0) {
+        const size_t per_block = static_cast<size_t>(kAddBlock) * kAddUnroll;
+        const size_t blocks = ceil_div(n_vec, per_block);
+        if (blocks > 0x7fffffffull) return fail(1, "prism_add_m: n=%zu too large", n);
+        if (x == y)
+            add_m_vec4_inplace_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(kAddBlock), 0, s>>>(
+                reinterpret_cast<u32x4*>(y), m, n_vec);
+        else
+            add_m_vec4_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(kAddBlock), 0, s>>>(
+                reinterpret_cast<const u32x4*>(x), reinterpret_cast<u32x4*>(y), m, n_vec);
+        if (int rc = check_launch("add_m_vec4_kernel")) return rc;
+    }
+    const size_t first = n_vec * 4;
+    if (first < n) {
+        const size_t blocks = ceil_div(n - first, static_cast<size_t>(kAddBlock));
+        if (blocks > 0x7fffffffull) return fail(1, "prism_add_m: n=%zu too large", n);
+        add_m_scalar_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(kAddBlock), 0, s>>>(x, y, m,
+                                                                                            first, n);
+        if (int rc = check_launch("add_m_scalar_kernel")) return rc;
+    }
+    return 0;
+}
+
+}  // namespace prism

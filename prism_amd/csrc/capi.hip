@@ -1,0 +1,94 @@
+// extern "C" surface of libprism_amd.so; declarations and the reference
+// interfaces they replace are in include/prism_amd.h.
+#include "../../include/prism_amd.h"
+
+#include <cstring>
+
+#include "common.h"
+#include "tile_map.h"
+
+namespace prism {
+char* error_buffer() {
+    static thread_local char buf[kErrorBufferLen] = {0};
+    return buf;
+}
+}  // namespace prism
+
+using namespace prism;
+
+extern "C" {
+
+const char* prism_version(void) { return "0.1.0"; }
+
+const char* prism_last_error_string(void) { return error_buffer(); }
+
+int prism_device_info(int* cu_count, int* clock_khz, int* wavefront_size, size_t* lds_bytes,
+                      size_t* hbm_bytes, char* name, size_t name_len) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    hipDeviceProp_t p;
+    e = hipGetDeviceProperties(&p, dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDeviceProperties");
+    if (cu_count) *cu_count = p.multiProcessorCount;
+    if (clock_khz) *clock_khz = p.clockRate;
+    if (wavefront_size) *wavefront_size = p.warpSize;
+    if (lds_bytes) *lds_bytes = p.sharedMemPerBlock;
+    if (hbm_bytes) *hbm_bytes = p.totalGlobalMem;
+    if (name && name_len) {
+        strncpy(name, p.gcnArchName, name_len - 1);
+        name[name_len - 1] = 0;
+    }
+    return 0;
+}
+
+int prism_tile_coords(int workgroup_id, int tiles_m, int tiles_n, int* tile_m, int* tile_n) {
+    if (tiles_m <= 0 || tiles_n <= 0 || workgroup_id < 0 ||
+        static_cast<long long>(workgroup_id) >= static_cast<long long>(tiles_m) * tiles_n)
+        return fail(1, "prism_tile_coords: id %d outside a %d x %d tile grid", workgroup_id, tiles_m, tiles_n);
+    if (!tile_m || !tile_n) return fail(1, "prism_tile_coords: null output");
+    xcd_tile_coords(workgroup_id, tiles_m, tiles_n, *tile_m, *tile_n);
+    return 0;
+}
+
+int prism_add_m(const int32_t* x, int32_t* y, int32_t m, size_t n, void* stream) {
+    return launch_add_m(x, y, m, n, static_cast<hipStream_t>(stream));
+}
+
+size_t prism_scan_workspace_bytes(size_t n) { return scan_workspace_bytes(n); }
+
+int prism_scan_i32(const int32_t* in, int32_t* out, size_t n, void* workspace,
+                   size_t workspace_bytes, void* stream) {
+    return launch_scan(reinterpret_cast<const uint32_t*>(in), reinterpret_cast<uint32_t*>(out), n,
+                       workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+uint32_t* prism_launch_scan(size_t n, uint32_t* x, void* workspace) {
+    int rc = launch_scan(x, x, n, workspace, scan_workspace_bytes(n), nullptr);
+    return rc == 0 ? x : nullptr;
+}
+
+int prism_sgemm(int variant, int M, int N, int K, float alpha, const float* A, const float* B,
+                float beta, float* C, void* stream) {
+    return launch_sgemm(variant, M, N, K, alpha, A, B, beta, C, static_cast<hipStream_t>(stream));
+}
+
+int prism_run_my_kernel(int my_kernel_num, int M, int N, int K, float alpha, float* A, float* B,
+                        float beta, float* C) {
+    if (my_kernel_num < 1 || my_kernel_num > 5)
+        return fail(1, "Unknown my_kernel number %d (expected 1..5)", my_kernel_num);
+    return launch_sgemm(my_kernel_num, M, N, K, alpha, A, B, beta, C, nullptr);
+}
+
+int prism_gemm_bf16(int M, int N, int K, const uint16_t* A, const uint16_t* B, float* D,
+                    void* stream) {
+    return launch_gemm_bf16(M, N, K, A, B, D, nullptr, static_cast<hipStream_t>(stream));
+}
+
+int prism_runmyh100(int M, int N, int K, const uint16_t* A, const uint16_t* B, uint16_t* C,
+                    int* DB) {
+    (void)DB;
+    return launch_gemm_bf16(M, N, K, A, B, nullptr, C, nullptr);
+}
+
+}  // extern "C"

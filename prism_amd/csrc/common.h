@@ -1,0 +1,54 @@
+// Shared host-side helpers for libprism_amd.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+
+namespace prism {
+
+constexpr int kWave = 64;  // CDNA wavefront width; every kernel here assumes it
+
+// Thread-local error text behind prism_last_error_string().
+char* error_buffer();
+constexpr size_t kErrorBufferLen = 512;
+
+inline int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(error_buffer(), kErrorBufferLen, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+inline int hip_fail(hipError_t e, const char* what) {
+    return fail(static_cast<int>(e), "%s: %s", what, hipGetErrorString(e));
+}
+
+// Launch check: hipGetLastError() clears and returns the launch error, if any.
+inline int check_launch(const char* kernel) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(e, kernel);
+    return 0;
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
+inline bool aligned2(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 1u) == 0; }
+
+template <typename T>
+constexpr T ceil_div(T a, T b) { return (a + b - 1) / b; }
+
+// Internal launchers, one per kernel family (defined in the .hip files).
+int launch_add_m(const int32_t* x, int32_t* y, int32_t m, size_t n, hipStream_t s);
+size_t scan_workspace_bytes(size_t n);
+int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, hipStream_t s);
+int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, const float* B,
+                 float beta, float* C, hipStream_t s);
+int launch_gemm_bf16(int M, int N, int K, const uint16_t* A, const uint16_t* B, float* D_f32,
+                     uint16_t* C_bf16_colmajor, hipStream_t s);
+
+}  // namespace prism

@@ -1,0 +1,281 @@
+// Single-pass inclusive prefix sum with decoupled look-back, uint32 modulo 2^32.
+//
+// What the reference does (examples/scan.py:200-227, generated/scan_kernel.cu):
+// every block takes a ticket, scans 16384 elements as 512 rows of 32 staged in
+// shared memory, scans the 512 row totals, publishes its aggregate, walks back
+// over its predecessors' {ready,data} records with one thread, publishes its
+// inclusive prefix and writes the tile back.
+//
+// What this file does on 64-lane wavefronts:
+//   * a tile lives in registers: every lane owns VPT packets of 4 consecutive
+//     elements (16 B loads/stores, 1 KiB contiguous per wave instruction);
+//   * lane-local serial sums, then one 6-step DPP scan per packet row across
+//     the wave (row_shr 1/2/4/8, row_bcast 15, row_bcast 31) - the wave64
+//     counterpart of scan_warps + shfl_up_sync_wrapper
+//     (examples/scan.py:23-29,106-128);
+//   * wave totals meet in LDS (<= 16 words) instead of the 512-entry
+//     Hillis-Steele pass (examples/scan.py:131-171);
+//   * one 64-bit status word per tile, {state, value}, written and polled with
+//     agent-scope atomics so that the word is coherent across the eight XCD
+//     L2s (the reference's volatile accesses assume one device-wide L2:
+//     evals/4090_scan/main.cu:21-37, generated/lookback_to_prev_blocks.cu:12-21);
+//   * the look-back is wave-parallel: 64 predecessors per poll, a ballot finds
+//     the nearest published prefix (examples/scan.py:60-85 walks them one by one).
+//
+// HBM-bound: 8 algorithmic bytes per element (4 B read + 4 B write); status
+// traffic is 8 B per tile.
+#include "common.h"
+
+#ifndef PRISM_SCAN_BLOCK
+#define PRISM_SCAN_BLOCK 256
+#endif
+#ifndef PRISM_SCAN_VPT
+#define PRISM_SCAN_VPT 4
+#endif
+// 1: release stores / acquire loads on the status words; 0: relaxed. The value
+// travels inside the atomic word itself, so no other memory needs ordering.
+#ifndef PRISM_SCAN_ACQ_REL
+#define PRISM_SCAN_ACQ_REL 0
+#endif
+
+namespace prism {
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned long long u64;
+
+constexpr int kScanBlock = PRISM_SCAN_BLOCK;
+constexpr int kScanVpt = PRISM_SCAN_VPT;                 // 16 B packets per lane
+constexpr int kScanTile = kScanBlock * kScanVpt * 4;     // elements per tile
+constexpr size_t kHeaderBytes = 256;                     // ticket counter lives here
+static_assert(kScanBlock % kWave == 0 && kScanBlock <= 1024, "block must be whole waves");
+
+// Tile states, the three-valued form of the reference's two ready flags
+// (BlockInfo::prefix.ready / aggregate.ready, evals/4090_scan/main.cu:21-37).
+constexpr uint32_t kInvalid = 0;    // nothing published yet
+constexpr uint32_t kAggregate = 1;  // value = sum of this tile only
+constexpr uint32_t kPrefix = 2;     // value = sum of everything up to and including this tile
+
+__device__ __forceinline__ u64 pack_status(uint32_t state, uint32_t value) {
+    return static_cast<u64>(state) | (static_cast<u64>(value) << 32);
+}
+
+__device__ __forceinline__ void publish(u64* word, uint32_t state, uint32_t value) {
+    __hip_atomic_store(word, pack_status(state, value),
+                       PRISM_SCAN_ACQ_REL ? __ATOMIC_RELEASE : __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ u64 poll(const u64* word) {
+    return __hip_atomic_load(word, PRISM_SCAN_ACQ_REL ? __ATOMIC_ACQUIRE : __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// DPP controls (gfx9): row_shr:n = 0x110 + n, row_bcast:15 = 0x142, row_bcast:31 = 0x143.
+template <int CTRL, int ROW_MASK, bool ZERO_FILL>
+__device__ __forceinline__ uint32_t dpp(uint32_t x) {
+    return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(x), CTRL, ROW_MASK,
+                                                             0xf, ZERO_FILL));
+}
+
+// Inclusive scan across the 64 lanes of a wavefront, no LDS.
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t x) {
+    x += dpp<0x111, 0xf, true>(x);   // within each row of 16 lanes
+    x += dpp<0x112, 0xf, true>(x);
+    x += dpp<0x114, 0xf, true>(x);
+    x += dpp<0x118, 0xf, true>(x);
+    x += dpp<0x142, 0xa, false>(x);  // lane 15 of rows 0,2 into rows 1,3
+    x += dpp<0x143, 0xc, false>(x);  // lane 31 into rows 2,3
+    return x;
+}
+
+__device__ __forceinline__ uint32_t wave_last_lane(uint32_t x) {
+    return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(x), 63));
+}
+
+// Exclusive prefix of tile `tile` (> 0): the sum of all earlier tiles. Run by
+// one whole wavefront; lane l inspects tile (window_end - l). Every tile below
+// `tile` has taken its ticket earlier, so it is running or finished and will
+// publish without waiting for anything later: the loop terminates.
+__device__ __forceinline__ uint32_t look_back(const u64* status, uint32_t tile, int lane) {
+    uint32_t sum = 0;
+    long long window_end = static_cast<long long>(tile) - 1;
+    while (true) {
+        const long long t = window_end - lane;
+        // Tiles "before the first" count as a published prefix of 0.
+        const u64 w = (t >= 0) ? poll(&status[t]) : pack_status(kPrefix, 0);
+        const uint32_t state = static_cast<uint32_t>(w);
+        const uint32_t value = static_cast<uint32_t>(w >> 32);
+        const u64 has_prefix = __ballot(state == kPrefix);
+        const u64 is_invalid = __ballot(state == kInvalid);
+        // Lanes 0..first-prefix-lane are needed; all 64 when no prefix is in the window.
+        const u64 needed = has_prefix ? ((2ull << __builtin_ctzll(has_prefix)) - 1ull) : ~0ull;
+        if (is_invalid & needed) {
+            __builtin_amdgcn_s_sleep(1);
+            continue;
+        }
+        const uint32_t contrib = ((needed >> lane) & 1ull) ? value : 0u;
+        sum += wave_last_lane(wave_inclusive_scan(contrib));
+        if (has_prefix) break;
+        window_end -= kWave;
+    }
+    return sum;
+}
+
+// VEC: in and out are 16 B aligned, full tiles use 16 B accesses.
+template <int BLOCK, int VPT, bool VEC>
+__global__ __launch_bounds__(BLOCK) void scan_lookback_kernel(const uint32_t* in, uint32_t* out,
+                                                              size_t n, uint32_t* ticket,
+                                                              u64* status) {
+    constexpr int WAVES = BLOCK / kWave;
+    constexpr int TILE = BLOCK * VPT * 4;
+    constexpr int WAVE_ELEMS = kWave * VPT * 4;
+    constexpr int ROW_ELEMS = kWave * 4;  // elements one wave instruction covers
+
+    __shared__ uint32_t s_tile;
+    __shared__ uint32_t s_wave_total[WAVES];
+    __shared__ uint32_t s_tile_prefix;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
+
+    // Dynamic tile id: tiles are numbered in the order blocks start running
+    // (examples/scan.py:88-99), which is what makes the look-back deadlock-free.
+    if (tid == 0)
+        s_tile = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const uint32_t tile = s_tile;
+
+    const size_t tile_base = static_cast<size_t>(tile) * TILE;
+    const size_t lane_base = tile_base + static_cast<size_t>(wave) * WAVE_ELEMS + lane * 4;
+    const bool full = VEC && (tile_base + TILE <= n);
+
+    u32x4 v[VPT];
+    if (full) {
+#pragma unroll
+        for (int j = 0; j < VPT; ++j)
+            v[j] = *reinterpret_cast<const u32x4*>(in + lane_base + j * ROW_ELEMS);
+    } else {
+#pragma unroll
+        for (int j = 0; j < VPT; ++j) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const size_t i = lane_base + j * ROW_ELEMS + c;
+                v[j][c] = (i < n) ? in[i] : 0u;
+            }
+        }
+    }
+
+    // Lane-local inclusive sums of each packet, then the packet totals are
+    // scanned across the wave; rows are chained by the wave-uniform carry.
+    uint32_t offset[VPT];
+    uint32_t carry = 0;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        v[j].y += v[j].x;
+        v[j].z += v[j].y;
+        v[j].w += v[j].z;
+        const uint32_t inclusive = wave_inclusive_scan(v[j].w);
+        offset[j] = carry + (inclusive - v[j].w);
+        carry += wave_last_lane(inclusive);
+    }
+    if (lane == 0) s_wave_total[wave] = carry;
+    __syncthreads();
+
+    uint32_t wave_prefix = 0;
+    uint32_t aggregate = 0;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+        const uint32_t t = s_wave_total[w];
+        if (w < wave) wave_prefix += t;
+        aggregate += t;
+    }
+
+    if (wave == 0) {
+        uint32_t prefix = 0;
+        if (tile == 0) {
+            if (lane == 0) publish(&status[0], kPrefix, aggregate);
+        } else {
+            if (lane == 0) publish(&status[tile], kAggregate, aggregate);
+            prefix = look_back(status, tile, lane);
+            if (lane == 0) publish(&status[tile], kPrefix, aggregate + prefix);
+        }
+        if (lane == 0) s_tile_prefix = prefix;
+    }
+    __syncthreads();
+    const uint32_t base_sum = s_tile_prefix + wave_prefix;
+
+    if (full) {
+#pragma unroll
+        for (int j = 0; j < VPT; ++j) {
+            const u32x4 r = v[j] + (offset[j] + base_sum);
+            *reinterpret_cast<u32x4*>(out + lane_base + j * ROW_ELEMS) = r;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < VPT; ++j) {
+            const uint32_t add = offset[j] + base_sum;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const size_t i = lane_base + j * ROW_ELEMS + c;
+                if (i < n) out[i] = v[j][c] + add;
+            }
+        }
+    }
+}
+
+// Clears the ticket counter and every status word (the two memsets of the
+// reference launcher, evals/4090_scan/main.cu:81-82, as one fill kernel).
+__global__ __launch_bounds__(256) void scan_reset_kernel(u64* words, size_t n_words) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i < n_words) words[i] = 0ull;
+}
+
+inline size_t num_tiles_for(size_t n) { return ceil_div(n, static_cast<size_t>(kScanTile)); }
+
+}  // namespace
+
+size_t scan_workspace_bytes(size_t n) {
+    return kHeaderBytes + sizeof(u64) * (num_tiles_for(n) > 0 ? num_tiles_for(n) : 1);
+}
+
+int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes,
+                hipStream_t s) {
+    if (n == 0) return 0;
+    if (in == nullptr || out == nullptr || ws == nullptr)
+        return fail(1, "prism_scan: null pointer with n=%zu", n);
+    if (!aligned4(in) || !aligned4(out)) return fail(1, "prism_scan: data pointers must be 4-byte aligned");
+    if ((reinterpret_cast<uintptr_t>(ws) & 7u) != 0)
+        return fail(1, "prism_scan: workspace must be 8-byte aligned");
+    const size_t need = scan_workspace_bytes(n);
+    if (ws_bytes < need)
+        return fail(1, "prism_scan: workspace of %zu bytes is smaller than the %zu needed for n=%zu",
+                    ws_bytes, need, n);
+    if (in != out) {
+        const uintptr_t a = reinterpret_cast<uintptr_t>(in), b = reinterpret_cast<uintptr_t>(out);
+        const uintptr_t bytes = n * sizeof(uint32_t);
+        if (a < b + bytes && b < a + bytes)
+            return fail(1, "prism_scan: in and out overlap without being equal");
+    }
+    const size_t tiles = num_tiles_for(n);
+    if (tiles > 0x7fffffffull) return fail(1, "prism_scan: n=%zu too large", n);
+
+    u64* words = reinterpret_cast<u64*>(ws);
+    const size_t n_words = need / sizeof(u64);
+    uint32_t* ticket = reinterpret_cast<uint32_t*>(ws);
+    u64* status = reinterpret_cast<u64*>(static_cast<char*>(ws) + kHeaderBytes);
+
+    scan_reset_kernel<<<dim3(static_cast<unsigned>(ceil_div(n_words, size_t{256}))), dim3(256), 0, s>>>(
+        words, n_words);
+    if (int rc = check_launch("scan_reset_kernel")) return rc;
+
+    const dim3 grid(static_cast<unsigned>(tiles)), block(kScanBlock);
+    if (aligned16(in) && aligned16(out))
+        scan_lookback_kernel<kScanBlock, kScanVpt, true><<<grid, block, 0, s>>>(in, out, n, ticket, status);
+    else
+        scan_lookback_kernel<kScanBlock, kScanVpt, false><<<grid, block, 0, s>>>(in, out, n, ticket, status);
+    return check_launch("scan_lookback_kernel");
+}
+
+}  // namespace prism

@@ -1,0 +1,456 @@
+// fp32 SGEMM progression, C = alpha * A @ B + beta * C, row-major, gfx950.
+//
+// The six kernels follow the reference's progression one to one
+// (launch shapes: evals/4090_sgemm/runner.cu:135-243):
+//   1  naive            generated/my_sgemm_kernel_1.cu       one thread per C element
+//   2  coalesced        generated/my_sgemm_kernel_2.cu       32x32-tile thread remap
+//   3  LDS block tile   generated/sgemm_shared_mem_block.cu  32x32 tiles in LDS
+//   6  thread tile      generated/my_sgemm_kernel_3.cu       8x8 per thread, scalar staging
+//   4  thread tile vec  generated/my_sgemm_kernel_4.cu       + 16 B loads, A tile transposed
+//   5  wave tile        generated/my_sgemm_kernel_5.cu,
+//                       evals/4090_sgemm/my_kernel_utils.cuh:13-90
+// Kernels 1, 2, 3, 4 and 6 accumulate every C element with one fused
+// multiply-add per k, in increasing k, and finish with
+// fma(alpha, acc, beta * c): they are bit-identical to each other and to a
+// serial host loop written the same way. Kernel 5 keeps the reference's
+// block -> wave -> sub-tile decomposition, but a 64-lane wave computes its
+// sub-tiles with v_mfma_f32_32x32x2_f32 instead of per-thread outer products;
+// its summation order inside the matrix unit is not specified, so it is
+// checked against an fp64 product within a tolerance.
+//
+// Unlike the reference kernels (no guards in kernels 1, 3, 4, 5), every kernel
+// here accepts any M, N, K: full tiles take a guard-free path, edge tiles a
+// predicated one. When beta == 0, C is not read.
+#include "common.h"
+#include "tile_map.h"
+
+namespace prism {
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ float epilogue(float alpha, float acc, float beta, const float* c) {
+    return beta == 0.0f ? alpha * acc : __builtin_fmaf(alpha, acc, beta * (*c));
+}
+
+// ---------------------------------------------------------------- kernel 1 --
+// Thread id -> (row, col) = (tid / N, tid % N) as in
+// generated/my_sgemm_kernel_1.cu:11-23, plus the bound the reference lacks.
+__global__ __launch_bounds__(256) void sgemm_naive_kernel(int M, int N, int K, float alpha,
+                                                          const float* __restrict__ A,
+                                                          const float* __restrict__ B, float beta,
+                                                          float* C) {
+    const size_t tid = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (tid >= static_cast<size_t>(M) * N) return;
+    const size_t row = tid / N, col = tid % N;
+    float acc = 0.0f;
+    for (int k = 0; k < K; ++k) acc = __builtin_fmaf(A[row * K + k], B[static_cast<size_t>(k) * N + col], acc);
+    float* c = &C[row * N + col];
+    *c = epilogue(alpha, acc, beta, c);
+}
+
+// ---------------------------------------------------------------- kernel 2 --
+// Consecutive thread ids fill 32x32 tiles of C row by row
+// (generated/my_sgemm_kernel_2.cu:5-16); block = one tile = 1024 threads.
+__global__ __launch_bounds__(1024) void sgemm_coalesced_kernel(int M, int N, int K, float alpha,
+                                                               const float* __restrict__ A,
+                                                               const float* __restrict__ B,
+                                                               float beta, float* C) {
+    constexpr int TS = 32;
+    const int tiles_per_row = (N + TS - 1) / TS;
+    const int tile_row = blockIdx.x / tiles_per_row, tile_col = blockIdx.x % tiles_per_row;
+    const int row = tile_row * TS + threadIdx.x / TS;
+    const int col = tile_col * TS + threadIdx.x % TS;
+    if (row >= M || col >= N) return;
+    const float* a = A + static_cast<size_t>(row) * K;
+    float acc = 0.0f;
+    for (int k = 0; k < K; ++k) acc = __builtin_fmaf(a[k], B[static_cast<size_t>(k) * N + col], acc);
+    float* c = &C[static_cast<size_t>(row) * N + col];
+    *c = epilogue(alpha, acc, beta, c);
+}
+
+// ---------------------------------------------------------------- kernel 3 --
+// 32x32 tiles of A and B staged in LDS, one accumulator per thread, two
+// barriers per K tile exactly where the reference's sync pass puts them
+// (generated/sgemm_shared_mem_block.cu:34,38). Out-of-range elements are
+// staged as zeros. A wave reads one As word per row (broadcast) and 32
+// consecutive Bs words, so neither tile needs padding.
+__global__ __launch_bounds__(1024) void sgemm_lds_block_kernel(int M, int N, int K, float alpha,
+                                                               const float* __restrict__ A,
+                                                               const float* __restrict__ B,
+                                                               float beta, float* C,
+                                                               int num_blocks_n) {
+    constexpr int BS = 32;
+    __shared__ float As[BS * BS];
+    __shared__ float Bs[BS * BS];
+    const int c_row = blockIdx.x / num_blocks_n, c_col = blockIdx.x % num_blocks_n;
+    const int t_row = threadIdx.x / BS, t_col = threadIdx.x % BS;
+    const int row = c_row * BS + t_row, col = c_col * BS + t_col;
+    float acc = 0.0f;
+    for (int k0 = 0; k0 < K; k0 += BS) {
+        const int ka = k0 + t_col, kb = k0 + t_row;
+        As[t_row * BS + t_col] = (row < M && ka < K) ? A[static_cast<size_t>(row) * K + ka] : 0.0f;
+        Bs[t_row * BS + t_col] = (kb < K && col < N) ? B[static_cast<size_t>(kb) * N + col] : 0.0f;
+        __syncthreads();
+        // Always the whole tile: the zero-filled tail adds exact +0 products, so
+        // the result still equals the serial loop over k < K bit for bit.
+#pragma unroll
+        for (int d = 0; d < BS; ++d) acc = __builtin_fmaf(As[t_row * BS + d], Bs[d * BS + t_col], acc);
+        __syncthreads();
+    }
+    if (row < M && col < N) {
+        float* c = &C[static_cast<size_t>(row) * N + col];
+        *c = epilogue(alpha, acc, beta, c);
+    }
+}
+
+// ----------------------------------------------------------- kernels 4 / 6 --
+// Block tile BM x BN, K step BK, TM x TN accumulators per thread.
+//   VEC = false: kernel 6 (generated/my_sgemm_kernel_3.cu): A tile row-major
+//                [BM][BK], scalar staging.
+//   VEC = true : kernel 4 (generated/my_sgemm_kernel_4.cu:41-46,74-79): A tile
+//                stored transposed [BK][BM], 16 B global loads, 16 B C epilogue.
+//   EDGE       : predicated scalar staging and stores for tiles that hang over
+//                M, N or K, or when rows are not 16 B aligned.
+// The register-fill loops are bounded by TM for regM and TN for regN; the
+// reference bounds both by TN (examples/sgemm_kernel_3.py:66-67), which is only
+// right because TM == TN there.
+template <int BM, int BN, int BK, int TM, int TN, bool VEC, bool EDGE>
+__global__ __launch_bounds__((BM * BN) / (TM * TN)) void sgemm_thread_tile_kernel(
+    int M, int N, int K, float alpha, const float* __restrict__ A, const float* __restrict__ B,
+    float beta, float* C, int num_blocks_n) {
+    constexpr int THREADS = (BM * BN) / (TM * TN);
+    static_assert(TN % 4 == 0 && BK % 4 == 0 && BN % 4 == 0, "16 B packets");
+    __shared__ __attribute__((aligned(16))) float As[BM * BK];
+    __shared__ __attribute__((aligned(16))) float Bs[BK * BN];
+
+    const int c_row = blockIdx.x / num_blocks_n, c_col = blockIdx.x % num_blocks_n;
+    const int row0 = c_row * BM, col0 = c_col * BN;
+    const int tid = threadIdx.x;
+    const int t_row = tid / (BN / TN), t_col = tid % (BN / TN);
+
+    float acc[TM * TN] = {0.0f};
+    float reg_m[TM], reg_n[TN];
+
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        if constexpr (VEC && !EDGE) {
+            // 16 B packets: A along k, stored transposed; B along n, stored as is.
+            for (int p = tid; p < BM * BK / 4; p += THREADS) {
+                const int r = p / (BK / 4), kc = p % (BK / 4);
+                const f32x4 a = *reinterpret_cast<const f32x4*>(
+                    &A[static_cast<size_t>(row0 + r) * K + k0 + kc * 4]);
+                As[(kc * 4 + 0) * BM + r] = a.x;
+                As[(kc * 4 + 1) * BM + r] = a.y;
+                As[(kc * 4 + 2) * BM + r] = a.z;
+                As[(kc * 4 + 3) * BM + r] = a.w;
+            }
+            for (int p = tid; p < BK * BN / 4; p += THREADS) {
+                const int r = p / (BN / 4), nc = p % (BN / 4);
+                *reinterpret_cast<f32x4*>(&Bs[r * BN + nc * 4]) = *reinterpret_cast<const f32x4*>(
+                    &B[static_cast<size_t>(k0 + r) * N + col0 + nc * 4]);
+            }
+        } else {
+            for (int p = tid; p < BM * BK; p += THREADS) {
+                const int r = p / BK, kk = p % BK;
+                float a;
+                if constexpr (EDGE)
+                    a = (row0 + r < M && k0 + kk < K) ? A[static_cast<size_t>(row0 + r) * K + k0 + kk] : 0.0f;
+                else
+                    a = A[static_cast<size_t>(row0 + r) * K + k0 + kk];
+                if constexpr (VEC) As[kk * BM + r] = a; else As[r * BK + kk] = a;
+            }
+            for (int p = tid; p < BK * BN; p += THREADS) {
+                const int r = p / BN, nn = p % BN;
+                float b;
+                if constexpr (EDGE)
+                    b = (k0 + r < K && col0 + nn < N) ? B[static_cast<size_t>(k0 + r) * N + col0 + nn] : 0.0f;
+                else
+                    b = B[static_cast<size_t>(k0 + r) * N + col0 + nn];
+                Bs[r * BN + nn] = b;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int d = 0; d < BK; ++d) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                reg_m[i] = VEC ? As[d * BM + t_row * TM + i] : As[(t_row * TM + i) * BK + d];
+#pragma unroll
+            for (int j = 0; j < TN; ++j) reg_n[j] = Bs[d * BN + t_col * TN + j];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i * TN + j] = __builtin_fmaf(reg_m[i], reg_n[j], acc[i * TN + j]);
+        }
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int row = row0 + t_row * TM + i;
+        if constexpr (VEC && !EDGE) {
+#pragma unroll
+            for (int j = 0; j < TN; j += 4) {
+                f32x4* c = reinterpret_cast<f32x4*>(&C[static_cast<size_t>(row) * N + col0 + t_col * TN + j]);
+                f32x4 r;
+                if (beta == 0.0f) {
+                    r.x = alpha * acc[i * TN + j + 0];
+                    r.y = alpha * acc[i * TN + j + 1];
+                    r.z = alpha * acc[i * TN + j + 2];
+                    r.w = alpha * acc[i * TN + j + 3];
+                } else {
+                    const f32x4 old = *c;
+                    r.x = __builtin_fmaf(alpha, acc[i * TN + j + 0], beta * old.x);
+                    r.y = __builtin_fmaf(alpha, acc[i * TN + j + 1], beta * old.y);
+                    r.z = __builtin_fmaf(alpha, acc[i * TN + j + 2], beta * old.z);
+                    r.w = __builtin_fmaf(alpha, acc[i * TN + j + 3], beta * old.w);
+                }
+                *c = r;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int col = col0 + t_col * TN + j;
+                if (!EDGE || (row < M && col < N)) {
+                    float* c = &C[static_cast<size_t>(row) * N + col];
+                    *c = epilogue(alpha, acc[i * TN + j], beta, c);
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------- kernel 5 --
+// Block tile BM x BN split over (BM/WM) x (BN/WN) waves; a wave's WM x WN tile
+// is a grid of 32x32 sub-tiles (the WMITER x WNITER sub-tiles of
+// generated/my_sgemm_kernel_5.cu:8-10 with WSUBM = WSUBN = 32), each held as the
+// 16 accumulator registers of one v_mfma_f32_32x32x2_f32.
+//
+// LDS tiles (double-buffered, one barrier per K step):
+//   As[k][m], transposed like the reference's loadFromGmem
+//   (evals/4090_sgemm/my_kernel_utils.cuh:23-31): row length BM + 2 words so
+//   that the four k-rows a 16 B global packet scatters to hit distinct banks;
+//   Bs[k][n] as in global memory.
+// MFMA operands: lane l supplies A[m = l % 32][k = l / 32] and
+// B[k = l / 32][n = l % 32]: both are 32 consecutive LDS words per half-wave.
+// Result register v of lane l is C[8 * (v / 4) + 4 * (l / 32) + v % 4][l % 32].
+//
+// Global loads for K step t+1 are issued before the MFMAs of step t and written
+// to the other LDS buffer after them.
+//
+// Workgroups are dealt to the 8 XCDs round-robin by id; the id is remapped so
+// that every XCD walks its own contiguous band of C tiles in columns of 8, and
+// the tiles resident on one XCD share A and B panels in that XCD's L2.
+template <int BM, int BN, int BK, int WM, int WN, bool EDGE>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile_kernel(
+    int M, int N, int K, float alpha, const float* __restrict__ A, const float* __restrict__ B,
+    float beta, float* C, int tiles_m, int tiles_n) {
+    constexpr int WAVES_N = BN / WN;
+    constexpr int THREADS = (BM / WM) * WAVES_N * kWave;
+    constexpr int MI = WM / 32, NI = WN / 32;  // sub-tiles per wave
+    constexpr int LDA = BM + 2, LDB = BN;
+    constexpr int A_PACKETS = BM * BK / 4, B_PACKETS = BK * BN / 4;
+    static_assert(A_PACKETS % THREADS == 0 && B_PACKETS % THREADS == 0, "whole packets per thread");
+    constexpr int A_PER = A_PACKETS / THREADS, B_PER = B_PACKETS / THREADS;
+    static_assert(BK % 4 == 0 && WM % 32 == 0 && WN % 32 == 0, "tile shapes");
+
+    __shared__ __attribute__((aligned(16))) float As[2][BK * LDA];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB];
+
+    int tm, tn;
+    xcd_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+    const int row0 = tm * BM, col0 = tn * BN;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1), wave = tid / kWave;
+    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+    const int l32 = lane & 31, lhi = lane >> 5;
+
+    f32x16 acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    f32x4 a_stage[A_PER], b_stage[B_PER];
+
+    auto load_global = [&](int k0) {
+#pragma unroll
+        for (int u = 0; u < A_PER; ++u) {
+            const int p = tid + u * THREADS;
+            const int r = p / (BK / 4), kc = p % (BK / 4);
+            const int row = row0 + r, k = k0 + kc * 4;
+            if constexpr (!EDGE) {
+                a_stage[u] = *reinterpret_cast<const f32x4*>(&A[static_cast<size_t>(row) * K + k]);
+            } else {
+                const float* src = &A[static_cast<size_t>(row) * K + k];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) a_stage[u][c] = (row < M && k + c < K) ? src[c] : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < B_PER; ++u) {
+            const int p = tid + u * THREADS;
+            const int r = p / (BN / 4), nc = p % (BN / 4);
+            const int k = k0 + r, col = col0 + nc * 4;
+            if constexpr (!EDGE) {
+                b_stage[u] = *reinterpret_cast<const f32x4*>(&B[static_cast<size_t>(k) * N + col]);
+            } else {
+                const float* src = &B[static_cast<size_t>(k) * N + col];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) b_stage[u][c] = (k < K && col + c < N) ? src[c] : 0.0f;
+            }
+        }
+    };
+    auto store_lds = [&](int buf) {
+#pragma unroll
+        for (int u = 0; u < A_PER; ++u) {
+            const int p = tid + u * THREADS;
+            const int r = p / (BK / 4), kc = p % (BK / 4);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) As[buf][(kc * 4 + c) * LDA + r] = a_stage[u][c];
+        }
+#pragma unroll
+        for (int u = 0; u < B_PER; ++u) {
+            const int p = tid + u * THREADS;
+            const int r = p / (BN / 4), nc = p % (BN / 4);
+            *reinterpret_cast<f32x4*>(&Bs[buf][r * LDB + nc * 4]) = b_stage[u];
+        }
+    };
+
+    const int k_tiles = (K + BK - 1) / BK;
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+
+    for (int t = 0; t < k_tiles; ++t) {
+        const int buf = t & 1;
+        const bool more = (t + 1 < k_tiles);
+        if (more) load_global((t + 1) * BK);
+
+        const float* as = &As[buf][wave_m * WM + l32];
+        const float* bs = &Bs[buf][wave_n * WN + l32];
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 2) {
+            float a[MI], b[NI];
+#pragma unroll
+            for (int i = 0; i < MI; ++i) a[i] = as[(kk + lhi) * LDA + i * 32];
+#pragma unroll
+            for (int j = 0; j < NI; ++j) b[j] = bs[(kk + lhi) * LDB + j * 32];
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+
+        if (more) store_lds(buf ^ 1);
+        __syncthreads();
+    }
+
+    // Epilogue: each store instruction writes two 128 B row segments.
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+            const int col = col0 + wave_n * WN + j * 32 + l32;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = row0 + wave_m * WM + i * 32 + 8 * (v / 4) + 4 * lhi + (v % 4);
+                if (!EDGE || (row < M && col < N)) {
+                    float* c = &C[static_cast<size_t>(row) * N + col];
+                    *c = epilogue(alpha, acc[i][j][v], beta, c);
+                }
+            }
+        }
+    }
+}
+
+// --------------------------------------------------------------- launchers --
+
+template <int BM, int BN, int BK, int TM, int TN, bool VEC>
+int run_thread_tile(int M, int N, int K, float alpha, const float* A, const float* B, float beta,
+                    float* C, hipStream_t s) {
+    const int nbm = ceil_div(M, BM), nbn = ceil_div(N, BN);
+    const dim3 grid(static_cast<unsigned>(nbm) * nbn), block((BM * BN) / (TM * TN));
+    const bool whole = (M % BM == 0) && (N % BN == 0) && (K % BK == 0);
+    const bool vec_ok = aligned16(A) && aligned16(B) && aligned16(C) && (K % 4 == 0) && (N % 4 == 0);
+    if (whole && (!VEC || vec_ok))
+        sgemm_thread_tile_kernel<BM, BN, BK, TM, TN, VEC, false><<<grid, block, 0, s>>>(
+            M, N, K, alpha, A, B, beta, C, nbn);
+    else
+        sgemm_thread_tile_kernel<BM, BN, BK, TM, TN, VEC, true><<<grid, block, 0, s>>>(
+            M, N, K, alpha, A, B, beta, C, nbn);
+    return check_launch("sgemm_thread_tile_kernel");
+}
+
+template <int BM, int BN, int BK, int WM, int WN>
+int run_wave_tile(int M, int N, int K, float alpha, const float* A, const float* B, float beta,
+                  float* C, hipStream_t s) {
+    const int tiles_m = ceil_div(M, BM), tiles_n = ceil_div(N, BN);
+    const dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n), block((BM / WM) * (BN / WN) * kWave);
+    const bool fast = (M % BM == 0) && (N % BN == 0) && (K % BK == 0) && aligned16(A) && aligned16(B);
+    if (fast)
+        sgemm_wave_tile_kernel<BM, BN, BK, WM, WN, false><<<grid, block, 0, s>>>(
+            M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n);
+    else
+        sgemm_wave_tile_kernel<BM, BN, BK, WM, WN, true><<<grid, block, 0, s>>>(
+            M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n);
+    return check_launch("sgemm_wave_tile_kernel");
+}
+
+}  // namespace
+
+int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, const float* B,
+                 float beta, float* C, hipStream_t s) {
+    if (variant < 0 || variant > 6) return fail(1, "prism_sgemm: unknown kernel number %d", variant);
+    if (M < 0 || N < 0 || K < 0) return fail(1, "prism_sgemm: negative dimension (%d,%d,%d)", M, N, K);
+    if (M == 0 || N == 0) return 0;
+    if (C == nullptr || (K > 0 && (A == nullptr || B == nullptr)))
+        return fail(1, "prism_sgemm: null matrix pointer");
+    if (!aligned4(A) || !aligned4(B) || !aligned4(C))
+        return fail(1, "prism_sgemm: matrices must be 4-byte aligned");
+    const size_t mn = static_cast<size_t>(M) * N;
+    if (variant == 0) variant = 5;
+    // K == 0 leaves C = beta * C; the naive kernel does exactly that.
+    if (K == 0) variant = 1;
+
+    switch (variant) {
+        case 1: {
+            const size_t blocks = ceil_div(mn, size_t{256});
+            if (blocks > 0x7fffffffull) return fail(1, "prism_sgemm: M*N too large for kernel 1");
+            sgemm_naive_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s>>>(M, N, K, alpha, A, B, beta, C);
+            return check_launch("sgemm_naive_kernel");
+        }
+        case 2: {
+            const size_t blocks = static_cast<size_t>(ceil_div(M, 32)) * ceil_div(N, 32);
+            sgemm_coalesced_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(1024), 0, s>>>(M, N, K, alpha, A, B, beta, C);
+            return check_launch("sgemm_coalesced_kernel");
+        }
+        case 3: {
+            const int nbn = ceil_div(N, 32);
+            const size_t blocks = static_cast<size_t>(ceil_div(M, 32)) * nbn;
+            sgemm_lds_block_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(1024), 0, s>>>(M, N, K, alpha, A, B, beta, C, nbn);
+            return check_launch("sgemm_lds_block_kernel");
+        }
+        case 4:
+            // Tile choice of run_my_sgemm_4 (evals/4090_sgemm/runner.cu:163-189).
+            if (M >= 128 && N >= 128) return run_thread_tile<128, 128, 8, 8, 8, true>(M, N, K, alpha, A, B, beta, C, s);
+            return run_thread_tile<64, 64, 8, 8, 8, true>(M, N, K, alpha, A, B, beta, C, s);
+        case 6:
+            if (M >= 128 && N >= 128) return run_thread_tile<128, 128, 8, 8, 8, false>(M, N, K, alpha, A, B, beta, C, s);
+            return run_thread_tile<64, 64, 8, 8, 8, false>(M, N, K, alpha, A, B, beta, C, s);
+        case 5:
+            // BM = BN = 128, BK = 16, WM = WN = 64: the tile shape of
+            // run_my_sgemm_5 (evals/4090_sgemm/runner.cu:194-202), with four
+            // 64-lane waves in place of four 32-lane warps.
+            return run_wave_tile<128, 128, 16, 64, 64>(M, N, K, alpha, A, B, beta, C, s);
+    }
+    return fail(1, "prism_sgemm: unknown kernel number %d", variant);
+}
+
+}  // namespace prism

@@ -1,0 +1,191 @@
+"""Host-side mirror of the reference's launchers, over libprism_amd.so.
+
+Names, argument order and meaning follow the C++ entry points of the
+reference's evaluation harnesses so that a test written against those reads the
+same here:
+
+  get_workspace_size / launch_scan   evals/4090_scan/main.cu:63-86
+  run_my_kernel                      evals/4090_sgemm/runner.cu:245-267
+  runmyh100                          evals/h100_bench/utils.cuh:504-533
+  add_m                              kernel signature in README.md:133-140
+
+plus tensor-shaped conveniences (scan, sgemm, gemm_bf16). Device memory is a
+PyTorch-ROCm tensor (or a raw integer device pointer where noted); torch is
+only the allocator and the stream provider, every computation is a HIP kernel
+in the shared library. All calls are asynchronous on torch's current stream
+unless the reference's shape fixes the default stream.
+"""
+from __future__ import annotations
+
+from typing import Optional, Union
+
+import torch
+
+from . import _lib
+
+SGEMM_KERNELS = {
+    1: "naive",
+    2: "coalesced",
+    3: "lds_block",
+    4: "thread_tile_vec",
+    5: "wave_tile_mfma",
+    6: "thread_tile_scalar",
+}
+
+Ptr = Union[int, "torch.Tensor"]
+
+
+class PrismError(RuntimeError):
+    """A launcher in libprism_amd.so reported a failure."""
+
+
+def _check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = _lib.last_error()
+        if rc == 1:
+            raise ValueError(f"{what}: {msg}")
+        raise PrismError(f"{what}: HIP error {rc}: {msg}")
+
+
+def _ptr(t: Ptr) -> int:
+    if isinstance(t, int):
+        return t
+    if t is None:
+        return 0
+    if not t.is_cuda:
+        raise ValueError("expected a tensor in device memory (cuda), got a host tensor")
+    if not t.is_contiguous():
+        raise ValueError("expected a contiguous tensor")
+    return t.data_ptr()
+
+
+def _need(t: "torch.Tensor", dtypes, numel: int, name: str) -> None:
+    if t.dtype not in dtypes:
+        raise TypeError(f"{name}: dtype {t.dtype} not in {tuple(dtypes)}")
+    if t.numel() < numel:
+        raise ValueError(f"{name}: holds {t.numel()} elements, {numel} needed")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+# ------------------------------------------------------------------- add_m --
+
+def add_m(x: "torch.Tensor", y: "torch.Tensor", m: int) -> "torch.Tensor":
+    """y[i] = x[i] + m (int32 wrap-around) for every element of x; returns y."""
+    _need(x, (torch.int32,), 0, "x")
+    _need(y, (torch.int32,), x.numel(), "y")
+    m = ((int(m) + 2**31) % 2**32) - 2**31  # wrap m itself like an int32 argument
+    _check(_lib.load().prism_add_m(_ptr(x), _ptr(y), m, x.numel(), _stream()), "add_m")
+    return y
+
+
+# -------------------------------------------------------------------- scan --
+
+def get_workspace_size(n: int) -> int:
+    """Workspace bytes for an n-element scan (scan_gpu::get_workspace_size)."""
+    if n < 0:
+        raise ValueError("n must be >= 0")
+    return int(_lib.load().prism_scan_workspace_bytes(n))
+
+
+def launch_scan(n: int, x: "torch.Tensor", workspace: "torch.Tensor") -> "torch.Tensor":
+    """In-place inclusive scan of the first n elements of x (scan_gpu::launch_scan).
+
+    Returns the tensor that holds the result (x itself), as the reference
+    returns its device pointer. Runs on the default stream like the reference.
+    """
+    _need(x, (torch.int32, torch.uint32), n, "x")
+    if workspace.numel() * workspace.element_size() < get_workspace_size(n):
+        raise ValueError("workspace smaller than get_workspace_size(n)")
+    out =_lib.load().prism_launch_scan(n, _ptr(x), _ptr(workspace))
+    if n > 0 and not out:
+        raise PrismError(f"launch_scan: {_lib.last_error()}")
+    return x
+
+
+def scan(inp: "torch.Tensor", out: Optional["torch.Tensor"] = None,
+         workspace: Optional["torch.Tensor"] = None) -> "torch.Tensor":
+    """Inclusive prefix sum modulo 2^32 of a 1-D int32/uint32 tensor; out may be inp."""
+    _need(inp, (torch.int32, torch.uint32), 0, "inp")
+    n = inp.numel()
+    if out is None:
+        out = torch.empty_like(inp)
+    _need(out, (inp.dtype,), n, "out")
+    need = get_workspace_size(n)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=inp.device)
+    ws_bytes = workspace.numel() * workspace.element_size()
+    _check(_lib.load().prism_scan_i32(_ptr(inp), _ptr(out), n, _ptr(workspace), ws_bytes, _stream()), "scan")
+    return out
+
+
+# ------------------------------------------------------------------- sgemm --
+
+def run_my_kernel(my_kernel_num: int, M: int, N: int, K: int, alpha: float, A: Ptr, B: Ptr,
+                  beta: float, C: Ptr) -> None:
+    """C = alpha*A@B + beta*C with kernel 1..5 on the default stream (run_my_kernel).
+
+    Raises ValueError for an unknown kernel number, where the reference throws
+    std::invalid_argument.
+    """
+    if my_kernel_num not in (1, 2, 3, 4, 5):
+        raise ValueError("Unknown my_kernel number")
+    _check(_lib.load().prism_run_my_kernel(my_kernel_num, M, N, K, alpha, _ptr(A), _ptr(B), beta, _ptr(C)),
+           "run_my_kernel")
+
+
+def sgemm(M: int, N: int, K: int, alpha: float, A: "torch.Tensor", B: "torch.Tensor", beta: float,
+          C: "torch.Tensor", variant: int = 5) -> "torch.Tensor":
+    """sgemm(M,N,K,alpha,A,B,beta,C): the kernel signature of generated/my_sgemm_kernel_*.cu."""
+    if variant not in (0, 1, 2, 3, 4, 5, 6):
+        raise ValueError("Unknown my_kernel number")
+    _need(A, (torch.float32,), M * K, "A")
+    _need(B, (torch.float32,), K * N, "B")
+    _need(C, (torch.float32,), M * N, "C")
+    _check(_lib.load().prism_sgemm(variant, M, N, K, alpha, _ptr(A), _ptr(B), beta, _ptr(C), _stream()), "sgemm")
+    return C
+
+
+# --------------------------------------------------------------- bf16 gemm --
+
+def gemm_bf16(A: "torch.Tensor", B: "torch.Tensor", D: Optional["torch.Tensor"] = None) -> "torch.Tensor":
+    """D[M,N] (fp32) = A[M,K] @ B[N,K]^T for bf16 A and B."""
+    _need(A, (torch.bfloat16,), 0, "A")
+    _need(B, (torch.bfloat16,), 0, "B")
+    if A.dim() != 2 or B.dim() != 2 or A.shape[1] != B.shape[1]:
+        raise ValueError("A must be MxK and B NxK")
+    M, K = A.shape
+    N = B.shape[0]
+    if D is None:
+        D = torch.empty((M, N), dtype=torch.float32, device=A.device)
+    _need(D, (torch.float32,), M * N, "D")
+    _check(_lib.load().prism_gemm_bf16(M, N, K, _ptr(A), _ptr(B), _ptr(D), _stream()), "gemm_bf16")
+    return D
+
+
+def runmyh100(M: int, N: int, K: int, A: Ptr, B: Ptr, C: Ptr, DB: Optional[Ptr] = None) -> None:
+    """bf16 C, column-major MxN, = A[M,K] @ B[N,K]^T on the default stream (runmyh100)."""
+    _check(_lib.load().prism_runmyh100(M, N, K, _ptr(A), _ptr(B), _ptr(C), _ptr(DB) if DB is not None else 0),
+           "runmyh100")
+
+
+# -------------------------------------------------------------------- misc --
+
+def device_info() -> dict:
+    import ctypes as C
+    cu, khz, wave = C.c_int(), C.c_int(), C.c_int()
+    lds, hbm = C.c_size_t(), C.c_size_t()
+    name = C.create_string_buffer(128)
+    _check(_lib.load().prism_device_info(C.byref(cu), C.byref(khz), C.byref(wave), C.byref(lds), C.byref(hbm),
+                                         name, 128), "device_info")
+    return {"cu_count": cu.value, "clock_khz": khz.value, "wavefront_size": wave.value,
+            "lds_bytes": lds.value, "hbm_bytes": hbm.value, "name": name.value.decode()}
+
+
+def tile_coords(workgroup_id: int, tiles_m: int, tiles_n: int) -> tuple:
+    import ctypes as C
+    tm, tn = C.c_int(), C.c_int()
+    _check(_lib.load().prism_tile_coords(workgroup_id, tiles_m, tiles_n, C.byref(tm), C.byref(tn)), "tile_coords")
+    return tm.value, tn.value

@@ -1,0 +1,119 @@
+"""GPU parity tests for the bf16 MFMA GEMM (the h100_matmul analogue), through the C ABI.
+
+Oracle: fp64 product of the bf16-rounded inputs. Tolerance (written out here):
+  fp32 output   |got - ref| <= 1e-3 * max|ref|            (relative, max-norm)  and
+                |got - ref| <= 1e-3 * sum_k |a_k||b_k|    (element-wise, where computed)
+  bf16 output   the same plus one bf16 rounding: |got - ref| <= 2^-8 |ref| + 1e-3 * max|ref|
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+REL = 1e-3
+
+
+def dev16(a16: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(np.ascontiguousarray(a16).view(np.int16)).to(DEV).view(torch.bfloat16)
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def check_f32(oracle, got, A16, B16):
+    ref = oracle.gemm_bf16_f64(A16, B16)
+    err = np.abs(got - ref)
+    scale = float(np.abs(ref).max(initial=0.0))
+    assert err.max(initial=0.0) <= REL * scale + 1e-30
+    mag = np.abs(oracle.bf16_to_f32(A16)).astype(np.float64) @ np.abs(oracle.bf16_to_f32(B16)).astype(np.float64).T
+    assert np.all(err <= REL * mag + 1e-30)
+
+
+SHAPES = [(1, 1, 1), (32, 32, 16), (40, 24, 75), (128, 128, 64), (128, 128, 128), (256, 384, 192),
+          (130, 200, 72), (64, 64, 8), (100, 36, 1000), (257, 129, 65)]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_fp32_output_vs_fp64_oracle(prism, oracle, shape):
+    M, N, K = shape
+    A16, B16 = oracle.gen_gemm_bf16(M, N, K, seed=M * 7 + N + K)
+    D = prism.gemm_bf16(dev16(A16), dev16(B16))
+    assert D.shape == (M, N) and D.dtype == torch.float32
+    check_f32(oracle, host(D), A16, B16)
+
+
+def test_fixture(prism, golden, oracle):
+    A16, B16 = golden["bf16_A"], golden["bf16_B"]
+    D = host(prism.gemm_bf16(dev16(A16), dev16(B16)))
+    ref = golden["bf16_D_f64"]
+    assert np.max(np.abs(D - ref)) <= REL * np.abs(ref).max()
+
+
+def test_exact_on_small_integers(prism, oracle):
+    """Small integers are exact in bf16 and their dot products exact in fp32: the result must be
+    exact whatever the summation order; a wrong operand layout (B read as K x N) fails."""
+    rng = np.random.default_rng(2)
+    M, N, K = 96, 160, 200
+    A = rng.integers(-4, 5, (M, K)).astype(np.float32)
+    B = rng.integers(-4, 5, (N, K)).astype(np.float32)
+    A16, B16 = oracle.np_f32_to_bf16(A), oracle.np_f32_to_bf16(B)
+    D = host(prism.gemm_bf16(dev16(A16), dev16(B16)))
+    assert np.array_equal(D, (A.astype(np.float64) @ B.astype(np.float64).T).astype(np.float32))
+
+
+@pytest.mark.parametrize("shape", [(128, 256, 256), (96, 40, 75), (256, 128, 64)])
+def test_runmyh100_layout_and_rounding(prism, oracle, shape):
+    """Reference launcher shape: bf16 output, column-major (C[n*M + m])."""
+    M, N, K = shape
+    A16, B16 = oracle.gen_gemm_bf16(M, N, K, seed=K)
+    C = torch.zeros(M * N + 64, dtype=torch.bfloat16, device=DEV)
+    prism.runmyh100(M, N, K, dev16(A16), dev16(B16), C[:M * N], None)
+    raw = host(C.view(torch.int16)).view(np.uint16)
+    assert np.all(raw[M * N:] == 0)
+    got = oracle.bf16_to_f32(raw[:M * N]).reshape(N, M).T  # column-major M x N
+    ref = oracle.gemm_bf16_f64(A16, B16)
+    assert np.all(np.abs(got - ref) <= 2.0**-8 * np.abs(ref) + REL * np.abs(ref).max())
+    # identical to rounding the fp32-output kernel's result (same accumulation, different store)
+    D = host(prism.gemm_bf16(dev16(A16), dev16(B16)))
+    assert np.array_equal(oracle.np_f32_to_bf16(D), raw[:M * N].reshape(N, M).T)
+
+
+def test_no_write_outside_and_k_zero(prism, oracle):
+    M, N, K = 70, 45, 33
+    A16, B16 = oracle.gen_gemm_bf16(M, N, K, seed=1)
+    buf = torch.full((M * N + 512,), 777.0, dtype=torch.float32, device=DEV)
+    D = buf[256:256 + M * N].view(M, N)
+    prism.gemm_bf16(dev16(A16), dev16(B16), D)
+    out = host(buf)
+    assert np.all(out[:256] == 777.0) and np.all(out[256 + M * N:] == 777.0)
+    check_f32(oracle, out[256:256 + M * N].reshape(M, N), A16, B16)
+    Z = prism.gemm_bf16(torch.zeros((M, 0), dtype=torch.bfloat16, device=DEV),
+                        torch.zeros((N, 0), dtype=torch.bfloat16, device=DEV),
+                        torch.full((M, N), 5.0, dtype=torch.float32, device=DEV))
+    assert np.all(host(Z) == 0.0)
+
+
+@pytest.mark.parametrize("n", [4096, 8192, 16384])
+def test_baseline_sizes_sampled(prism, oracle, n):
+    """BASELINE sizes: N(0,1) inputs rounded to bf16; 32 sampled rows against fp64."""
+    g = torch.Generator(device=DEV)
+    g.manual_seed(0)
+    A = torch.randn((n, n), dtype=torch.float32, device=DEV, generator=g).to(torch.bfloat16)
+    B = torch.randn((n, n), dtype=torch.float32, device=DEV, generator=g).to(torch.bfloat16)
+    D = prism.gemm_bf16(A, B)
+    torch.cuda.synchronize()
+    idx = np.sort(np.random.default_rng(0).choice(n, 32, replace=False))
+    idx[0], idx[-1] = 0, n - 1
+    it = torch.from_numpy(idx).to(DEV)
+    a_rows = A[it].float().cpu().numpy().astype(np.float64)
+    b_all = B.float().cpu().numpy()
+    ref = a_rows @ b_all.astype(np.float64).T
+    got = D[it].cpu().numpy()
+    assert np.max(np.abs(got - ref)) <= REL * np.abs(ref).max()
+    # scaling an input by 2 (exact in bf16) scales the output exactly
+    D2 = prism.gemm_bf16((A.float() * 2).to(torch.bfloat16), B)
+    assert torch.equal(D2, 2.0 * D)

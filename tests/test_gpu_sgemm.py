@@ -1,0 +1,194 @@
+"""GPU parity tests for the fp32 SGEMM progression, through the C ABI.
+
+Kernels 1, 2, 3, 4, 6 compute each element as a serial chain of fused
+multiply-adds over increasing k, so they must equal the fmaf oracle BIT FOR BIT.
+Kernel 5 (MFMA) is checked against the fp64 oracle with the tolerance
+max|err| <= 1e-5 * sqrt(K) * max|A| * max|B| (plus the rounding of the beta*C term).
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+EXACT = (1, 2, 3, 4, 6)
+ALL = (1, 2, 3, 4, 5, 6)
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def run(prism, variant, alpha, A, B, beta, Cm):
+    M, K = A.shape
+    N = B.shape[1]
+    c = dev(Cm).clone()
+    prism.sgemm(M, N, K, alpha, dev(A), dev(B), beta, c, variant=variant)
+    return host(c)
+
+
+def tol(oracle, K, A, B, beta, Cm):
+    extra = abs(beta) * float(np.abs(Cm).max(initial=0.0)) * 2**-22 if beta != 0 else 0.0
+    return oracle.sgemm_tolerance(K, A, B) + extra
+
+
+SMALL = [(1, 1, 1), (16, 16, 16), (33, 47, 29), (127, 129, 17), (64, 64, 64), (128, 128, 128),
+         (130, 70, 33), (256, 128, 64), (64, 200, 8), (200, 64, 250), (129, 257, 100)]
+
+
+@pytest.mark.parametrize("shape", SMALL)
+def test_exact_kernels_match_fma_oracle_bitwise(prism, oracle, shape):
+    M, N, K = shape
+    A, B, Cm = oracle.gen_sgemm(M, N, K, seed=M + N + K)
+    want = oracle.sgemm_fma(0.5, A, B, 3.0, Cm)
+    for v in EXACT:
+        got = run(prism, v, 0.5, A, B, 3.0, Cm)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), f"kernel {v} shape {shape}"
+
+
+@pytest.mark.parametrize("shape", SMALL)
+def test_wave_tile_kernel_within_tolerance(prism, oracle, shape):
+    M, N, K = shape
+    A, B, Cm = oracle.gen_sgemm(M, N, K, seed=M + N + K)
+    want = oracle.sgemm_f64(1.0, A, B, 0.5, Cm)
+    got = run(prism, 5, 1.0, A, B, 0.5, Cm)
+    assert np.max(np.abs(got - want)) <= tol(oracle, K, A, B, 0.5, Cm)
+    # variant 0 is the alias of the best kernel
+    assert np.array_equal(run(prism, 0, 1.0, A, B, 0.5, Cm), got)
+
+
+def test_fixture(prism, golden, oracle):
+    a, b = (float(v) for v in golden["sgemm_alpha_beta"])
+    A, B, Cm = golden["sgemm_A"], golden["sgemm_B"], golden["sgemm_C"]
+    for v in EXACT:
+        assert np.array_equal(run(prism, v, a, A, B, b, Cm), golden["sgemm_out_fma"])
+    got = run(prism, 5, a, A, B, b, Cm)
+    assert np.max(np.abs(got - golden["sgemm_out_f64"])) <= tol(oracle, A.shape[1], A, B, b, Cm)
+
+
+def test_reference_harness_configuration(prism, oracle):
+    """The reference's own correctness run: 1024^3, alpha 0.5, beta 3.0, entries +-(k + 0.01 j),
+    k, j in 0..4, every kernel within 0.01 of the oracle (evals/4090_sgemm/main.cu:48,84-147,
+    runner.cu:54-65,105-117), through run_my_kernel."""
+    n = 1024
+    rng = np.random.default_rng(1)
+
+    def randomize(shape):
+        v = rng.integers(0, 5, shape).astype(np.float32) + np.float32(0.01) * rng.integers(0, 5, shape).astype(np.float32)
+        return np.where(rng.integers(0, 2, shape) == 0, v, -v).astype(np.float32)
+
+    A, B, Cm = randomize((n, n)), randomize((n, n)), randomize((n, n))
+    want = oracle.np_sgemm_f64(0.5, A, B, 3.0, Cm)
+    for k in (1, 2, 3, 4, 5):
+        c = dev(Cm).clone()
+        prism.run_my_kernel(k, n, n, n, 0.5, dev(A), dev(B), 3.0, c)
+        got = host(c)
+        assert np.max(np.abs(got - want)) <= 0.01, f"kernel {k}"
+        assert np.max(np.abs(got - want)) <= tol(oracle, n, A, B, 3.0, Cm), f"kernel {k}"
+    with pytest.raises(ValueError):
+        prism.run_my_kernel(6, n, n, n, 0.5, dev(A), dev(B), 3.0, dev(Cm))
+
+
+def test_special_cases_all_kernels(prism, oracle):
+    M, N, K = 96, 160, 72
+    A, B, Cm = oracle.gen_sgemm(M, N, K, seed=3)
+    poison = np.full((M, N), np.nan, dtype=np.float32)
+    eye = np.eye(K, dtype=np.float32)
+    for v in ALL:
+        # beta == 0 never reads C
+        got = run(prism, v, 1.0, A, B, 0.0, poison)
+        assert np.isfinite(got).all(), f"kernel {v} read C with beta == 0"
+        assert np.max(np.abs(got - oracle.sgemm_f64(1.0, A, B, 0.0))) <= oracle.sgemm_tolerance(K, A, B)
+        # alpha == 0: C = beta * C exactly
+        assert np.array_equal(run(prism, v, 0.0, A, B, 0.5, Cm), np.float32(0.5) * Cm), f"kernel {v}"
+        # B = I: C = A exactly (0 and 1 products are exact in every summation order)
+        assert np.array_equal(run(prism, v, 1.0, A, eye, 0.0, np.zeros((M, K), np.float32)), A), f"kernel {v}"
+        # K == 1 outer product, K == 0 scaling
+        a1, b1 = A[:, :1].copy(), B[:1, :].copy()
+        assert np.array_equal(run(prism, v, 1.0, a1, b1, 0.0, poison), a1 * b1), f"kernel {v}"
+        a0, b0 = np.zeros((M, 0), np.float32), np.zeros((0, N), np.float32)
+        assert np.array_equal(run(prism, v, 1.0, a0, b0, 2.0, Cm), 2.0 * Cm), f"kernel {v}"
+
+
+def test_does_not_write_outside_c(prism, oracle):
+    M, N, K = 70, 45, 33
+    A, B, Cm = oracle.gen_sgemm(M, N, K, seed=5)
+    for v in ALL:
+        buf = torch.full((M * N + 512,), 777.0, dtype=torch.float32, device=DEV)
+        c = buf[256:256 + M * N]
+        c.copy_(dev(Cm).reshape(-1))
+        prism.sgemm(M, N, K, 1.0, dev(A), dev(B), 0.5, c, variant=v)
+        out = host(buf)
+        assert np.all(out[:256] == 777.0) and np.all(out[256 + M * N:] == 777.0), f"kernel {v}"
+
+
+@pytest.mark.parametrize("n", [1024, 2048])
+def test_baseline_square_all_kernels(prism, oracle, n):
+    A, B, Cm = oracle.gen_sgemm(n, n, n, seed=0)
+    want = oracle.np_sgemm_f64(1.0, A, B, 0.5, Cm)
+    t = tol(oracle, n, A, B, 0.5, Cm)
+    first = None
+    for v in ALL:
+        got = run(prism, v, 1.0, A, B, 0.5, Cm)
+        assert np.max(np.abs(got - want)) <= t, f"kernel {v} n {n}"
+        if v in EXACT:
+            first = got if first is None else first
+            assert np.array_equal(got, first), f"kernel {v} differs from kernel 1 bitwise"
+
+
+@pytest.mark.parametrize("shape", [(4096, 4096, 128), (128, 4096, 4096), (8191, 4097, 1023)])
+def test_baseline_tail_shapes(prism, oracle, shape):
+    M, N, K = shape
+    A, B, _ = oracle.gen_sgemm(M, N, K, seed=1)
+    want = oracle.np_sgemm_f64(1.0, A, B, 0.0)
+    poison = np.full((M, N), np.nan, dtype=np.float32)
+    t = oracle.sgemm_tolerance(K, A, B)
+    for v in (4, 5):
+        got = run(prism, v, 1.0, A, B, 0.0, poison)
+        assert np.max(np.abs(got - want)) <= t, f"kernel {v} shape {shape}"
+
+
+def _sampled_check(prism, oracle, M, N, K, alpha, beta, variant, rows=48):
+    """Full-size run, checked on `rows` random rows against an fp64 product."""
+    g = torch.Generator(device=DEV)
+    g.manual_seed(0)
+    A = torch.rand((M, K), dtype=torch.float32, device=DEV, generator=g) * 2 - 1
+    B = torch.rand((K, N), dtype=torch.float32, device=DEV, generator=g) * 2 - 1
+    C0 = torch.rand((M, N), dtype=torch.float32, device=DEV, generator=g) * 2 - 1
+    c = C0.clone()
+    prism.sgemm(M, N, K, alpha, A, B, beta, c, variant=variant)
+    torch.cuda.synchronize()
+    idx = np.sort(np.random.default_rng(0).choice(M, rows, replace=False))
+    idx[0], idx[-1] = 0, M - 1
+    it = torch.from_numpy(idx).to(DEV)
+    a_rows = A[it].cpu().numpy()
+    b_host = B.cpu().numpy()
+    want = oracle.np_sgemm_f64(alpha, a_rows, b_host, beta, C0[it].cpu().numpy())
+    got = c[it].cpu().numpy()
+    bound = 1e-5 * np.sqrt(K) * 1.0 * 1.0 + (abs(beta) * 2**-22 if beta else 0.0)
+    assert np.max(np.abs(got - want)) <= bound
+    # linearity in alpha: doubling alpha with beta = 0 doubles every element exactly
+    c1 = torch.empty_like(c)
+    c2 = torch.empty_like(c)
+    prism.sgemm(M, N, K, 1.0, A, B, 0.0, c1, variant=variant)
+    prism.sgemm(M, N, K, 2.0, A, B, 0.0, c2, variant=variant)
+    assert torch.equal(c2, 2.0 * c1)
+
+
+def test_wave_tile_4096_and_8192(prism, oracle):
+    _sampled_check(prism, oracle, 4096, 4096, 4096, 1.0, 0.5, 5)
+    _sampled_check(prism, oracle, 8192, 8192, 8192, 1.0, 0.5, 5)
+
+
+def test_wave_tile_16384x16384x512(prism, oracle):
+    _sampled_check(prism, oracle, 16384, 16384, 512, 1.0, 0.0, 5)
+
+
+def test_thread_tile_4096(prism, oracle):
+    _sampled_check(prism, oracle, 4096, 4096, 4096, 1.0, 0.5, 4, rows=16)
