@@ -20,23 +20,27 @@
 //     L2s (the reference's volatile accesses assume one device-wide L2:
 //     evals/4090_scan/main.cu:21-37, generated/lookback_to_prev_blocks.cu:12-21);
 //   * the look-back is wave-parallel: 64 predecessors per poll, a ballot finds
-//     the nearest published prefix (examples/scan.py:60-85 walks them one by one).
+//     the nearest published prefix (examples/scan.py:60-85 walks them one by
+//     one with a single thread).
+//
+// Two measured facts about MI355X shape the tile size. Tickets are atomic adds
+// on one address and retire at about one per 12 ns, so a 2^30-element scan can
+// afford at most ~10^5 tiles. A status word takes a few microseconds to travel
+// between XCDs, during which hundreds of small tiles would start, and the
+// nearest published prefix would sit hundreds of tiles back. Large inputs
+// therefore use 256 KiB tiles (few tiles in flight, one or two polls per
+// look-back); small inputs use 64 KiB tiles so that more CUs get work. Polling
+// with more than one wave per tile was measured slower: the extra status
+// traffic costs more than the round trips it saves.
+//
+// Status words use RELAXED agent-scope atomics: the value travels inside the
+// atomic word, no other memory is communicated between tiles, so no fence is
+// needed (acquire/release here would write back and invalidate a whole L2 per
+// poll, measured 10x slower).
 //
 // HBM-bound: 8 algorithmic bytes per element (4 B read + 4 B write); status
-// traffic is 8 B per tile.
+// traffic is 8 B per tile plus the polls.
 #include "common.h"
-
-#ifndef PRISM_SCAN_BLOCK
-#define PRISM_SCAN_BLOCK 256
-#endif
-#ifndef PRISM_SCAN_VPT
-#define PRISM_SCAN_VPT 4
-#endif
-// 1: release stores / acquire loads on the status words; 0: relaxed. The value
-// travels inside the atomic word itself, so no other memory needs ordering.
-#ifndef PRISM_SCAN_ACQ_REL
-#define PRISM_SCAN_ACQ_REL 0
-#endif
 
 namespace prism {
 namespace {
@@ -44,11 +48,26 @@ namespace {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned long long u64;
 
-constexpr int kScanBlock = PRISM_SCAN_BLOCK;
-constexpr int kScanVpt = PRISM_SCAN_VPT;                 // 16 B packets per lane
-constexpr int kScanTile = kScanBlock * kScanVpt * 4;     // elements per tile
-constexpr size_t kHeaderBytes = 256;                     // ticket counter lives here
-static_assert(kScanBlock % kWave == 0 && kScanBlock <= 1024, "block must be whole waves");
+constexpr size_t kHeaderBytes = 256;  // ticket counter lives here
+
+// Tile shapes: {threads, 16 B packets per lane}.
+struct SmallCfg { static constexpr int BLOCK = 1024, VPT = 4; };
+#ifndef PRISM_SCAN_BIG_BLOCK
+#define PRISM_SCAN_BIG_BLOCK 1024
+#endif
+#ifndef PRISM_SCAN_BIG_VPT
+#define PRISM_SCAN_BIG_VPT 16
+#endif
+#ifndef PRISM_SCAN_SLEEP
+#define PRISM_SCAN_SLEEP 1
+#endif
+struct BigCfg { static constexpr int BLOCK = PRISM_SCAN_BIG_BLOCK, VPT = PRISM_SCAN_BIG_VPT; };
+template <typename Cfg> constexpr int tile_elems() { return Cfg::BLOCK * Cfg::VPT * 4; }
+// Inputs up to this many elements use the small tile.
+#ifndef PRISM_SCAN_SMALL_MAX
+#define PRISM_SCAN_SMALL_MAX ((size_t{1} << 24) - 1)
+#endif
+constexpr size_t kSmallMax = PRISM_SCAN_SMALL_MAX;
 
 // Tile states, the three-valued form of the reference's two ready flags
 // (BlockInfo::prefix.ready / aggregate.ready, evals/4090_scan/main.cu:21-37).
@@ -61,14 +80,11 @@ __device__ __forceinline__ u64 pack_status(uint32_t state, uint32_t value) {
 }
 
 __device__ __forceinline__ void publish(u64* word, uint32_t state, uint32_t value) {
-    __hip_atomic_store(word, pack_status(state, value),
-                       PRISM_SCAN_ACQ_REL ? __ATOMIC_RELEASE : __ATOMIC_RELAXED,
-                       __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(word, pack_status(state, value), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __device__ __forceinline__ u64 poll(const u64* word) {
-    return __hip_atomic_load(word, PRISM_SCAN_ACQ_REL ? __ATOMIC_ACQUIRE : __ATOMIC_RELAXED,
-                             __HIP_MEMORY_SCOPE_AGENT);
+    return __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // DPP controls (gfx9): row_shr:n = 0x110 + n, row_bcast:15 = 0x142, row_bcast:31 = 0x143.
@@ -111,7 +127,7 @@ __device__ __forceinline__ uint32_t look_back(const u64* status, uint32_t tile, 
         // Lanes 0..first-prefix-lane are needed; all 64 when no prefix is in the window.
         const u64 needed = has_prefix ? ((2ull << __builtin_ctzll(has_prefix)) - 1ull) : ~0ull;
         if (is_invalid & needed) {
-            __builtin_amdgcn_s_sleep(1);
+            __builtin_amdgcn_s_sleep(PRISM_SCAN_SLEEP);
             continue;
         }
         const uint32_t contrib = ((needed >> lane) & 1ull) ? value : 0u;
@@ -123,14 +139,16 @@ __device__ __forceinline__ uint32_t look_back(const u64* status, uint32_t tile, 
 }
 
 // VEC: in and out are 16 B aligned, full tiles use 16 B accesses.
-template <int BLOCK, int VPT, bool VEC>
-__global__ __launch_bounds__(BLOCK) void scan_lookback_kernel(const uint32_t* in, uint32_t* out,
-                                                              size_t n, uint32_t* ticket,
-                                                              u64* status) {
+template <typename Cfg, bool VEC>
+__global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_t* in, uint32_t* out,
+                                                                   size_t n, uint32_t* ticket,
+                                                                   u64* status) {
+    constexpr int BLOCK = Cfg::BLOCK, VPT = Cfg::VPT;
     constexpr int WAVES = BLOCK / kWave;
     constexpr int TILE = BLOCK * VPT * 4;
     constexpr int WAVE_ELEMS = kWave * VPT * 4;
     constexpr int ROW_ELEMS = kWave * 4;  // elements one wave instruction covers
+    static_assert(BLOCK % kWave == 0 && BLOCK <= 1024, "block must be whole waves");
 
     __shared__ uint32_t s_tile;
     __shared__ uint32_t s_wave_total[WAVES];
@@ -155,7 +173,7 @@ __global__ __launch_bounds__(BLOCK) void scan_lookback_kernel(const uint32_t* in
     if (full) {
 #pragma unroll
         for (int j = 0; j < VPT; ++j)
-            v[j] = *reinterpret_cast<const u32x4*>(in + lane_base + j * ROW_ELEMS);
+            v[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(in + lane_base + j * ROW_ELEMS));
     } else {
 #pragma unroll
         for (int j = 0; j < VPT; ++j) {
@@ -210,7 +228,7 @@ __global__ __launch_bounds__(BLOCK) void scan_lookback_kernel(const uint32_t* in
 #pragma unroll
         for (int j = 0; j < VPT; ++j) {
             const u32x4 r = v[j] + (offset[j] + base_sum);
-            *reinterpret_cast<u32x4*>(out + lane_base + j * ROW_ELEMS) = r;
+            __builtin_nontemporal_store(r, reinterpret_cast<u32x4*>(out + lane_base + j * ROW_ELEMS));
         }
     } else {
 #pragma unroll
@@ -232,12 +250,29 @@ __global__ __launch_bounds__(256) void scan_reset_kernel(u64* words, size_t n_wo
     if (i < n_words) words[i] = 0ull;
 }
 
-inline size_t num_tiles_for(size_t n) { return ceil_div(n, static_cast<size_t>(kScanTile)); }
+inline bool use_small(size_t n) { return n <= kSmallMax; }
+
+inline size_t num_tiles_for(size_t n) {
+    const size_t tile = use_small(n) ? tile_elems<SmallCfg>() : tile_elems<BigCfg>();
+    return ceil_div(n, tile);
+}
+
+template <typename Cfg>
+int launch_cfg(const uint32_t* in, uint32_t* out, size_t n, uint32_t* ticket, u64* status, size_t tiles,
+               hipStream_t s) {
+    const dim3 grid(static_cast<unsigned>(tiles)), block(Cfg::BLOCK);
+    if (aligned16(in) && aligned16(out))
+        scan_lookback_kernel<Cfg, true><<<grid, block, 0, s>>>(in, out, n, ticket, status);
+    else
+        scan_lookback_kernel<Cfg, false><<<grid, block, 0, s>>>(in, out, n, ticket, status);
+    return check_launch("scan_lookback_kernel");
+}
 
 }  // namespace
 
 size_t scan_workspace_bytes(size_t n) {
-    return kHeaderBytes + sizeof(u64) * (num_tiles_for(n) > 0 ? num_tiles_for(n) : 1);
+    const size_t tiles = num_tiles_for(n);
+    return kHeaderBytes + sizeof(u64) * (tiles > 0 ? tiles : 1);
 }
 
 int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes,
@@ -270,12 +305,8 @@ int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws
         words, n_words);
     if (int rc = check_launch("scan_reset_kernel")) return rc;
 
-    const dim3 grid(static_cast<unsigned>(tiles)), block(kScanBlock);
-    if (aligned16(in) && aligned16(out))
-        scan_lookback_kernel<kScanBlock, kScanVpt, true><<<grid, block, 0, s>>>(in, out, n, ticket, status);
-    else
-        scan_lookback_kernel<kScanBlock, kScanVpt, false><<<grid, block, 0, s>>>(in, out, n, ticket, status);
-    return check_launch("scan_lookback_kernel");
+    if (use_small(n)) return launch_cfg<SmallCfg>(in, out, n, ticket, status, tiles, s);
+    return launch_cfg<BigCfg>(in, out, n, ticket, status, tiles, s);
 }
 
 }  // namespace prism

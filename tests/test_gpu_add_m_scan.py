@@ -73,7 +73,8 @@ def test_scan_fixtures(prism, golden):
 
 
 TILE_EDGES = [1, 2, 63, 64, 65, 255, 256, 257, 1023, 1024, 1025, 4095, 4096, 4097, 8191, 8192, 8193,
-              16383, 16384, 16385, 32768, 100_003]
+              16383, 16384, 16385, 32768, 65535, 65536, 65537, 100_003, 262_145,
+              (1 << 24) - 1, (1 << 24) + 1, (1 << 24) + 65536 * 3 + 5]
 
 
 @pytest.mark.parametrize("n", TILE_EDGES)
@@ -151,11 +152,12 @@ def test_scan_workspace_reuse_and_unaligned(prism, oracle):
         x = oracle.gen_scan(m, seed=seed)
         out = prism.scan(dev(x), workspace=ws)
         assert np.array_equal(host(out), oracle.scan_cpu(x))
-    x = oracle.gen_scan(n + 1, seed=42)
-    xd = dev(x)
-    out = torch.zeros(n + 3, dtype=torch.int32, device=DEV)
-    prism.scan(xd[1:], out[3:3 + n])  # 4-byte-aligned only: scalar path
-    assert np.array_equal(host(out)[3:], oracle.scan_cpu(x[1:]))
+    for n in (n, (1 << 24) + 12_345):  # small-tile and large-tile kernels
+        x = oracle.gen_scan(n + 1, seed=42)
+        xd = dev(x)
+        out = torch.zeros(n + 3, dtype=torch.int32, device=DEV)
+        prism.scan(xd[1:], out[3:3 + n])  # 4-byte-aligned only: scalar path
+        assert np.array_equal(host(out)[3:], oracle.scan_cpu(x[1:]))
 
 
 def test_scan_on_a_side_stream(prism, oracle):
