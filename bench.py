@@ -34,8 +34,28 @@ PEAK = {  # MI355X published peaks
 }
 
 
+# HBM-side bytes per launch (L2 misses: TCC fetches + write-backs), measured with
+# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over this script and scaled by what the same
+# counters read for a 1 GiB copy (`--workload calibrate`): FETCH_SIZE x 2.0, WRITE_SIZE x 1.0
+# (summaries under profiles/). None where not measured for that shape.
+TRAFFIC_BYTES = {
+    ("sgemm", 8192, 5): (8105032 + 262144) * 1024,
+    ("scan", 1 << 30): (4198548 + 4217260) * 1024,
+    ("gemm_bf16", 8192): (1573592 + 262144) * 1024,
+    ("add_m", 1 << 24): (65567 + 65606) * 1024,
+}
+
+
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
+
+
+def _capi():
+    """The C-ABI library and the current stream handle: timed loops call the entry points
+    directly so that Python-side argument checks are not part of a step."""
+    import torch
+    from prism_amd import _lib
+    return _lib.load(), torch.cuda.current_stream().cuda_stream
 
 
 def time_steps(fn, steps: int, warmup: int):
@@ -76,12 +96,15 @@ def bench_sgemm(prism, M, N, K, alpha, beta, variant, steps, warmup, gate=True):
         C.copy_(C0)
     # Like the reference's sweep, C accumulates across repeats (evals/4090_sgemm/main.cu:199-203);
     # with |beta| < 1 it stays bounded.
-    ms = time_steps(lambda: prism.sgemm(M, N, K, alpha, A, B, beta, C, variant=variant), steps, warmup)
+    lib, st = _capi()
+    a, b, c = A.data_ptr(), B.data_ptr(), C.data_ptr()
+    ms = time_steps(lambda: lib.prism_sgemm(variant, M, N, K, alpha, a, b, beta, c, st), steps, warmup)
     flops = 2.0 * M * N * K
     tflops = flops / (ms * 1e-3) / 1e12
     return {"ms": ms, "tflops": tflops,
             "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK["fp32_mfma_TFLOPs"], "unit": "TFLOP/s",
-                         "frac": tflops / PEAK["fp32_mfma_TFLOPs"], "traffic": None}}
+                         "frac": tflops / PEAK["fp32_mfma_TFLOPs"],
+                         "traffic": TRAFFIC_BYTES.get(("sgemm", M, variant)) if M == N == K else None}}
 
 
 # ------------------------------------------------------------------- scan --
@@ -109,12 +132,14 @@ def bench_scan(prism, n, steps, warmup, gate=True):
             raise RuntimeError(f"scan n={n} failed the parity gate")
     # Out of place, so no restore is needed between steps; the workspace reset is part of the step,
     # as the reference times its launcher's memsets (evals/4090_scan/main.cu:81-82).
-    ms = time_steps(lambda: prism.scan(x, out, ws), steps, warmup)
+    lib, st = _capi()
+    xp, op, wp, wb = x.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel()
+    ms = time_steps(lambda: lib.prism_scan_i32(xp, op, n, wp, wb, st), steps, warmup)
     nbytes = 2.0 * 4 * n  # scan_harness.cuh:161
     gbps = nbytes / (ms * 1e-3) / 1e9
     return {"ms": ms, "GBps": gbps,
             "roofline": {"bound": "hbm", "achieved": gbps, "peak": PEAK["hbm_GBps"], "unit": "GB/s",
-                         "frac": gbps / PEAK["hbm_GBps"], "traffic": None}}
+                         "frac": gbps / PEAK["hbm_GBps"], "traffic": TRAFFIC_BYTES.get(("scan", n))}}
 
 
 # ------------------------------------------------------------------ add_m --
@@ -130,11 +155,13 @@ def bench_add_m(prism, n, steps, warmup, gate=True):
         torch.cuda.synchronize()
         if not torch.equal(y, x + 7):
             raise RuntimeError("add_m failed the parity gate")
-    ms = time_steps(lambda: prism.add_m(x, y, 7), steps, warmup)
+    lib, st = _capi()
+    xp, yp = x.data_ptr(), y.data_ptr()
+    ms = time_steps(lambda: lib.prism_add_m(xp, yp, 7, n, st), steps, warmup)
     gbps = 8.0 * n / (ms * 1e-3) / 1e9
     return {"ms": ms, "GBps": gbps,
             "roofline": {"bound": "hbm", "achieved": gbps, "peak": PEAK["hbm_GBps"], "unit": "GB/s",
-                         "frac": gbps / PEAK["hbm_GBps"], "traffic": None}}
+                         "frac": gbps / PEAK["hbm_GBps"], "traffic": TRAFFIC_BYTES.get(("add_m", n))}}
 
 
 # -------------------------------------------------------------- bf16 gemm --
@@ -154,11 +181,13 @@ def bench_gemm_bf16(prism, n, steps, warmup, gate=True):
         err = float((D[rows].double() - ref).abs().max())
         if not err <= 1e-3 * float(ref.abs().max()):
             raise RuntimeError(f"gemm_bf16 n={n} failed the parity gate: err {err}")
-    ms = time_steps(lambda: prism.gemm_bf16(A, B, D), steps, warmup)
+    lib, st = _capi()
+    a, b, d = A.data_ptr(), B.data_ptr(), D.data_ptr()
+    ms = time_steps(lambda: lib.prism_gemm_bf16(n, n, n, a, b, d, st), steps, warmup)
     tflops = 2.0 * n * n * n / (ms * 1e-3) / 1e12
     return {"ms": ms, "tflops": tflops,
             "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK["bf16_mfma_TFLOPs"], "unit": "TFLOP/s",
-                         "frac": tflops / PEAK["bf16_mfma_TFLOPs"], "traffic": None}}
+                         "frac": tflops / PEAK["bf16_mfma_TFLOPs"], "traffic": TRAFFIC_BYTES.get(("gemm_bf16", n))}}
 
 
 # ----------------------------------------------------------- CPU baselines --
@@ -228,7 +257,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="all", choices=["all", "sgemm", "scan", "gemm_bf16", "add_m"])
+    ap.add_argument("--workload", default="all", choices=["all", "sgemm", "scan", "gemm_bf16", "add_m", "calibrate"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--sweep", action="store_true", help="also time every BASELINE config (table on stderr)")
     args = ap.parse_args()
@@ -246,6 +275,17 @@ def main() -> int:
     log(f"device: {info}")
     K, W = args.steps, args.warmup
     want = lambda w: args.workload in ("all", w)
+
+    if args.workload == "calibrate":
+        # A plain copy of known size (1 GiB read + 1 GiB written per launch) for scaling the
+        # FETCH_SIZE / WRITE_SIZE counters of a `rocprofv3 --pmc` run of this same script.
+        n = 1 << 28
+        x = torch.randint(-1000, 1001, (n,), dtype=torch.int32, device="cuda")
+        y = torch.empty_like(x)
+        ms = time_steps(lambda: y.copy_(x), K, W)
+        print(json.dumps({"workload": "calibrate", "kernel": "torch copy_ int32", "bytes_read": 4 * n,
+                          "bytes_written": 4 * n, "ms_per_step": ms, "GBps": 8.0 * n / ms / 1e6}), flush=True)
+        return 0
 
     res = {}
     if want("sgemm"):

@@ -267,6 +267,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_kerne
 // the other. Step t: issue the loads of tile t+1 into the idle stage, multiply
 // tile t, barrier (which also waits for the loads), prefetch the first operands
 // of tile t+1.
+#ifndef PRISM_BF16_DMA_SPLIT
+#define PRISM_BF16_DMA_SPLIT 1
+#endif
 #ifndef PRISM_BF16_SWZ
 #define PRISM_BF16_SWZ 1
 #endif
@@ -382,11 +385,18 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_dma_k
             mfma_all(kk & 1);
         }
 #if PRISM_BF16_SCHED
+        // The direct loads are spread over the first DMA_SPLIT groups of MFMAs.
         constexpr int LOADS = prefetch ? (P_PER + Q_PER) : 0;
+        constexpr int L_PER = (LOADS + PRISM_BF16_DMA_SPLIT - 1) / PRISM_BF16_DMA_SPLIT;
         __builtin_amdgcn_sched_group_barrier(0x100, MI + NI, 0);
-        sched_substep<0, 0, LOADS, MI * NI>();
+        sched_substep<0, 0, L_PER, MI * NI>();
 #pragma unroll
-        for (int kk = 0; kk + 1 < KS; ++kk) sched_substep<MI + NI, 0, 0, MI * NI>();
+        for (int kk = 0; kk + 1 < KS; ++kk) {
+            if (kk + 1 < PRISM_BF16_DMA_SPLIT)
+                sched_substep<MI + NI, 0, L_PER, MI * NI>();
+            else
+                sched_substep<MI + NI, 0, 0, MI * NI>();
+        }
 #endif
         __syncthreads();
     };
