@@ -112,3 +112,18 @@ def test_tile_map_keeps_an_xcd_on_a_compact_patch(lib):
             rows.add(tm.value)
             cols.add(tn.value)
         assert len(rows) <= 8 and len(cols) <= 8
+
+
+def test_header_is_valid_c_and_cxx(tmp_path):
+    """include/prism_amd.h must compile as plain C99 and as C++ (it is the FFI contract)."""
+    import shutil
+    import subprocess
+    src_c = tmp_path / "t.c"
+    src_c.write_text('#include "prism_amd.h"\nint main(void) { return (int)sizeof(&prism_scan_i32) == 0; }\n')
+    src_cc = tmp_path / "t.cpp"
+    src_cc.write_text('#include "prism_amd.h"\nint main() { return PRISM_SGEMM_WAVE_TILE == 5 ? 0 : 1; }\n')
+    inc = str(ROOT / "include")
+    if shutil.which("gcc"):
+        subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-fsyntax-only", "-I", inc, str(src_c)], check=True)
+    if shutil.which("g++"):
+        subprocess.run(["g++", "-std=c++11", "-Wall", "-Werror", "-fsyntax-only", "-I", inc, str(src_cc)], check=True)
