@@ -24,6 +24,11 @@
 #include "common.h"
 #include "tile_map.h"
 
+// Kernel 5 tile shape: BM, BN, BK, WM, WN.
+#ifndef PRISM_SGEMM5_CFG
+#define PRISM_SGEMM5_CFG 128, 128, 16, 64, 64
+#endif
+
 namespace prism {
 namespace {
 
@@ -448,7 +453,7 @@ int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, 
             // BM = BN = 128, BK = 16, WM = WN = 64: the tile shape of
             // run_my_sgemm_5 (evals/4090_sgemm/runner.cu:194-202), with four
             // 64-lane waves in place of four 32-lane warps.
-            return run_wave_tile<128, 128, 16, 64, 64>(M, N, K, alpha, A, B, beta, C, s);
+            return run_wave_tile<PRISM_SGEMM5_CFG>(M, N, K, alpha, A, B, beta, C, s);
     }
     return fail(1, "prism_sgemm: unknown kernel number %d", variant);
 }

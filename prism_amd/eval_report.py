@@ -1,0 +1,186 @@
+"""Evaluation sweeps in the reference harnesses' own methodology and text format.
+
+    python -m prism_amd.eval_report [sgemm] [scan] [h100]      (default: all three)
+
+The counterpart of the reference's three benchmark mains, so that the text it
+prints can be fed to the reference's plotting script unchanged:
+
+  sgemm  evals/4090_sgemm/main.cu:43,154-217  sizes 256..8192, alpha 0.5, beta 3.0, 10 back-to-back
+         launches between two events, GFLOPS = 2 m n k / t; blocks "[cuBLAS FP32]" / "[My Kernel k]"
+         (parsed by evals/plot_results.py:37-79)
+  scan   evals/4090_scan/bench.cu:157-262     n = 2^20..2^30, best wall-clock of launch + device sync over
+         repeats until 500 ms have elapsed, GB/s = n * 4 * 2 / t; table "Size | CUB ... | Ours ..."
+         (parsed by plot_results.py:82-108)
+  h100   evals/h100_bench/main.cu:112-167     8 back-to-back launches between two events, TFLOPS;
+         lines "Kernel: ..." / "cuBLAS: ..." (parsed by plot_results.py:18-34)
+
+The vendor-library slots ("cuBLAS", "CUB") are filled with what the ROCm stack
+offers through PyTorch: rocBLAS/hipBLASLt `torch.matmul` and rocPRIM
+`torch.cumsum`. They are comparison lines, like the reference's.
+"""
+from __future__ import annotations
+
+import sys
+import time
+
+SGEMM_SIZES = (256, 512, 1024, 2048, 4096, 8192)            # evals/4090_sgemm/main.cu:43
+SCAN_LOG2_SIZES = tuple(range(20, 31))                       # evals/4090_scan/bench.cu:157-169
+H100_SIZES = (2048, 4096, 6144, 8192, 12288, 16384)          # evals/run_h100.sh:12
+
+
+# ------------------------------------------------------------- formatting --
+
+def sgemm_line(seconds_per_call: float, gflops: float, size: int) -> str:
+    # printf format of evals/4090_sgemm/main.cu:182-186
+    return ("Average elapsed time: (%7.6f) s, performance: (%7.1f) GFLOPS. size: (%ld)." % (seconds_per_call, gflops, size))
+
+
+def h100_line(who: str, seconds_per_call: float, tflops: float, size: int) -> str:
+    # printf format of evals/h100_bench/main.cu:149-152 ("Kernel:" / "cuBLAS:")
+    return ("%s  Average elapsed time: (%7.6f) s, performance: (%7.1f) TFLOPS. size: (%ld)." % (who, seconds_per_call, tflops, size))
+
+
+def scan_header() -> str:
+    # evals/4090_scan/bench.cu:175-179
+    return ("%12s | %10s %10s | %10s %10s\n%s" % ("Size", "CUB (ms)", "CUB (GB/s)", "Ours (ms)", "Ours (GB/s)", "-" * 62))
+
+
+def scan_row(n: int, lib_ms: float, lib_gbps: float, ours_ms: float, ours_gbps: float) -> str:
+    # evals/4090_scan/bench.cu:261-262
+    return "%12d | %10.4f %10.2f | %10.4f %10.2f" % (n, lib_ms, lib_gbps, ours_ms, ours_gbps)
+
+
+# ----------------------------------------------------------------- timing --
+
+def _events_ms(fn, repeats: int) -> float:
+    import torch
+    beg, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    beg.record()
+    for _ in range(repeats):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return beg.elapsed_time(end)
+
+
+def _best_wall_ms(fn, target_ms: float) -> float:
+    """benchmark_ms of evals/4090_scan/scan_harness.cuh:84-100: best of repeated (launch + sync)."""
+    import torch
+    best, elapsed = float("inf"), 0.0
+    while elapsed < target_ms:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        fn()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3
+        elapsed += ms
+        best = min(best, ms)
+    return best
+
+
+# ----------------------------------------------------------------- sweeps --
+
+def sweep_sgemm(out=sys.stdout, sizes=SGEMM_SIZES, repeats: int = 10) -> None:
+    import torch
+    from . import _lib
+    lib = _lib.load()
+    alpha, beta = 0.5, 3.0
+    top = max(sizes)
+    A = torch.rand((top, top), device="cuda") * 2 - 1
+    B = torch.rand((top, top), device="cuda") * 2 - 1
+    C = torch.rand((top, top), device="cuda") * 2 - 1
+    print("\n====================================\nStarting Performance Sweep\n====================================", file=out)
+    for n in sizes:
+        a, b = A.flatten()[: n * n].view(n, n), B.flatten()[: n * n].view(n, n)
+        c = C.flatten()[: n * n].view(n, n).clone()
+        flops = 2.0 * n * n * n
+        print(f"\n====================================\nSize: {n}x{n}x{n}\n====================================", file=out)
+        print("\n[cuBLAS FP32]", file=out)  # slot of the vendor BLAS: rocBLAS/hipBLASLt through torch
+        ref = c.clone()
+        torch.addmm(ref, a, b, beta=beta, alpha=alpha, out=ref)
+        ms = _events_ms(lambda: torch.addmm(ref, a, b, beta=beta, alpha=alpha, out=ref), repeats)
+        print(sgemm_line(ms / 1e3 / repeats, repeats * flops * 1e-9 / (ms / 1e3), n), file=out)
+        for k in (1, 2, 3, 4, 5):
+            print(f"\n[My Kernel {k}]", file=out)
+            c.copy_(C.flatten()[: n * n].view(n, n))
+            fn = lambda: lib.prism_run_my_kernel(k, n, n, n, alpha, a.data_ptr(), b.data_ptr(), beta, c.data_ptr())
+            fn()
+            ms = _events_ms(fn, repeats)
+            print(sgemm_line(ms / 1e3 / repeats, repeats * flops * 1e-9 / (ms / 1e3), n), file=out)
+        out.flush()
+
+
+def sweep_scan(out=sys.stdout, log2_sizes=SCAN_LOG2_SIZES, target_ms: float = 500.0) -> None:
+    import torch
+    from . import _lib
+    lib = _lib.load()
+    top = 1 << max(log2_sizes)
+    x = torch.randint(0, 101, (top,), dtype=torch.int32, device="cuda")  # U{0..100}, scan_harness.cuh:172
+    work = torch.empty_like(x)
+    ws = torch.empty(lib.prism_scan_workspace_bytes(top), dtype=torch.uint8, device="cuda")
+    print(scan_header(), file=out)
+    for p in log2_sizes:
+        n = 1 << p
+        xin, buf = x[:n], work[:n]
+        # the reference scans in place and restores the input outside the timed region
+        def ours():
+            lib.prism_launch_scan(n, buf.data_ptr(), ws.data_ptr())
+        def vendor():
+            torch.cumsum(xin, 0, dtype=torch.int32, out=buf)
+        results = []
+        for fn in (vendor, ours):
+            best, elapsed = float("inf"), 0.0
+            while elapsed < target_ms:
+                buf.copy_(xin)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                fn()
+                torch.cuda.synchronize()
+                ms = (time.perf_counter() - t0) * 1e3
+                elapsed += max(ms, 0.05)
+                best = min(best, ms)
+            results.append(best)
+        bytes_ = n * 4 * 2
+        print(scan_row(n, results[0], bytes_ / results[0] / 1e6, results[1], bytes_ / results[1] / 1e6), file=out)
+        out.flush()
+    print("", file=out)
+
+
+def sweep_h100(out=sys.stdout, sizes=H100_SIZES, repeats: int = 8) -> None:
+    import torch
+    from . import _lib
+    lib = _lib.load()
+    for n in sizes:
+        A = torch.randn((n, n), device="cuda").to(torch.bfloat16)
+        B = torch.randn((n, n), device="cuda").to(torch.bfloat16)
+        Cc = torch.empty((n, n), dtype=torch.bfloat16, device="cuda")  # column-major M x N, as the reference
+        flops = 2.0 * n * n * n
+        fn = lambda: lib.prism_runmyh100(n, n, n, A.data_ptr(), B.data_ptr(), Cc.data_ptr(), None)
+        fn()
+        ms = _events_ms(fn, repeats)
+        print(h100_line("Kernel:", ms / 1e3 / repeats, repeats * flops * 1e-9 / ms, n), file=out)
+        vend = lambda: torch.matmul(A, B.T)
+        vend()
+        ms = _events_ms(vend, repeats)
+        print(h100_line("cuBLAS:", ms / 1e3 / repeats, repeats * flops * 1e-9 / ms, n) + "\n", file=out)
+        out.flush()
+        del A, B, Cc
+
+
+def main(argv=None) -> int:
+    which = [a for a in (argv if argv is not None else sys.argv[1:])] or ["sgemm", "scan", "h100"]
+    for w in which:
+        if w == "sgemm":
+            sweep_sgemm()
+        elif w == "scan":
+            sweep_scan()
+        elif w == "h100":
+            sweep_h100()
+        else:
+            print(f"unknown sweep {w!r}; expected sgemm, scan or h100", file=sys.stderr)
+            return 2
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

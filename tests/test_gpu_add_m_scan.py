@@ -74,7 +74,8 @@ def test_scan_fixtures(prism, golden):
 
 TILE_EDGES = [1, 2, 63, 64, 65, 255, 256, 257, 1023, 1024, 1025, 4095, 4096, 4097, 8191, 8192, 8193,
               16383, 16384, 16385, 32768, 65535, 65536, 65537, 100_003, 262_145,
-              (1 << 24) - 1, (1 << 24) + 1, (1 << 24) + 65536 * 3 + 5]
+              (1 << 24) - 1, (1 << 24) + 1, (1 << 24) + 65536 * 3 + 5,
+              65536 * 300 - 1, 65536 * 300, 65536 * 300 + 1]
 
 
 @pytest.mark.parametrize("n", TILE_EDGES)
