@@ -248,8 +248,12 @@ __global__ __launch_bounds__((BM * BN) / (TM * TN)) void sgemm_thread_tile_kerne
 // Workgroups are dealt to the 8 XCDs round-robin by id; the id is remapped so
 // that every XCD walks its own contiguous band of C tiles in columns of 8, and
 // the tiles resident on one XCD share A and B panels in that XCD's L2.
+#ifndef PRISM_SGEMM5_WAVES_PER_EU
+#define PRISM_SGEMM5_WAVES_PER_EU 4
+#endif
 template <int BM, int BN, int BK, int WM, int WN, bool EDGE>
-__global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile_kernel(
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave)
+__attribute__((amdgpu_waves_per_eu(PRISM_SGEMM5_WAVES_PER_EU))) void sgemm_wave_tile_kernel(
     int M, int N, int K, float alpha, const float* __restrict__ A, const float* __restrict__ B,
     float beta, float* C, int tiles_m, int tiles_n) {
     constexpr int WAVES_N = BN / WN;
@@ -375,6 +379,258 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
     }
 }
 
+// ------------------------------------------------- kernel 5, whole tiles --
+// The same product for problems made of whole 256 x 256 tiles: global data goes
+// straight into LDS (global_load_lds_dwordx4: no staging registers, no LDS
+// write instructions), four waves each own a 128 x 128 corner held in 256
+// accumulator registers, and one workgroup occupies a CU. With a single wave
+// per SIMD nothing else hides a stall, so the K loop is written as phases that
+// run from barrier to barrier with the matrix pipe fed throughout.
+//
+// LDS layout of one K tile (two stages, separate arrays so that the compiler's
+// wait-count logic knows loads into one stage do not feed reads of the other):
+//   As[m][k]  as in global memory, BK floats per row. A wave-wide direct load
+//             writes 1 KiB of contiguous LDS (lane l lands at base + 16 l), so
+//             rows cannot be padded; the 16 B chunk c of row m is kept in slot
+//             c ^ ((m >> SWZ) & (chunks - 1)) instead, which spreads the 16 rows
+//             a quarter-wave reads with ds_read_b128 over all 64 banks.
+//   Bs[k][n]  as in global memory, one 1 KiB row per direct load.
+// MFMA operands, per group of 8 k values starting at k8: lane (l32, lhi) reads
+// the A chunk k8 + 4 lhi .. + 3 of row l32 (one ds_read_b128 per 32-row block)
+// and, for jj = 0..3, B[k8 + 4 lhi + jj][4 l32 .. 4 l32 + 3] (one ds_read_b128
+// each). MFMA jj multiplies element jj of the A chunk by element j of the B
+// chunk into sub-tile j: the two k values of a 32x32x2 instruction are
+// k8 + jj and k8 + 4 + jj, and lane l32 of sub-tile j holds column 4 l32 + j,
+// so a lane owns 4 consecutive columns of C and stores them as one 16 B packet.
+#ifndef PRISM_SGEMM5_SCHED
+#define PRISM_SGEMM5_SCHED 1
+#endif
+#ifndef PRISM_SGEMM5_LATE_BARRIER
+#define PRISM_SGEMM5_LATE_BARRIER 1
+#endif
+#ifndef PRISM_SGEMM5_LOAD_GAP
+#define PRISM_SGEMM5_LOAD_GAP 4
+#endif
+// One wave-wide 16 B-per-lane load from global memory straight into LDS: lane l
+// reads base + offset(l) and lands at lds_dst + 16 l. Written as inline assembly
+// for its addressing mode: a scalar base plus a 32-bit vector offset, which the
+// compiler's own selection for the direct-load builtin does not use (it builds a
+// 64-bit vector address with vector ALU instructions for every load). M0 carries
+// the LDS address; a scalar write of M0 needs one wait state before the load
+// reads it. The compiler does not see these loads in its wait counts: the caller
+// waits with an explicit vmcnt before the barrier that publishes the tile.
+__device__ __forceinline__ void direct_load16(const char* base, uint32_t lane_offset, const float* lds_dst) {
+    const uint32_t lds_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+        (const __attribute__((address_space(3))) void*)lds_dst));
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(lane_offset), "s"(base), "s"(lds_addr)
+                 : "memory", "m0");
+}
+
+template <int BM, int BN, int BK, int WM, int WN>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile_dma_kernel(
+    int M, int N, int K, float alpha, const float* __restrict__ A, const float* __restrict__ B,
+    float beta, float* C, int tiles_m, int tiles_n) {
+    constexpr int WAVES_N = BN / WN;
+    constexpr int WAVES = (BM / WM) * WAVES_N;
+    constexpr int MI = WM / 32, NI = 4;
+    static_assert(WN == 128 && BN == 256, "a lane owns 4 columns of a 128-wide wave tile; a B row is one direct load");
+    constexpr int KP = BK / 4;                        // 16 B chunks per A row
+    constexpr int SWZ = KP == 4 ? 2 : 1;
+    static_assert(KP == 4 || KP == 8, "BK is 16 or 32");
+    constexpr int KS = BK / 8;                        // operand groups (8 k values) per tile
+    constexpr int ROWS_PER_LOAD = kWave / KP;         // A rows one wave-wide load covers
+    constexpr int ROWS_PER_PASS = ROWS_PER_LOAD * WAVES;
+    static_assert(BM % ROWS_PER_PASS == 0 && BK % WAVES == 0, "whole load passes");
+    constexpr int A_PER = BM / ROWS_PER_PASS, B_PER = BK / WAVES;  // loads per wave per tile
+    constexpr int LOAD_GAP = PRISM_SGEMM5_LOAD_GAP;                  // MFMAs between two direct loads
+    static_assert((A_PER + B_PER) * LOAD_GAP <= 4 * MI * 4, "the loads of a tile fit among the MFMAs of one group");
+    static_assert(((ROWS_PER_PASS >> SWZ) % KP) == 0 && ((32 >> SWZ) % KP) == 0,
+                  "the swizzle term must repeat with the load pass and the 32-row MFMA block");
+
+    __shared__ __attribute__((aligned(1024))) float As0[BM * BK];
+    __shared__ __attribute__((aligned(1024))) float As1[BM * BK];
+    __shared__ __attribute__((aligned(1024))) float Bs0[BK * BN];
+    __shared__ __attribute__((aligned(1024))) float Bs1[BK * BN];
+
+    int tm, tn;
+    xcd_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+    const int row0 = tm * BM, col0 = tn * BN;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // wave-uniform, lives in an SGPR
+    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+    const int l32 = lane & 31, lhi = lane >> 5;
+
+    f32x16 acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    // Load side. A: in pass u this wave fills rows [(u * WAVES + wave) * ROWS_PER_LOAD, + ROWS_PER_LOAD);
+    // lane l owns row l / KP of those and slot l % KP. The swizzle term is the same in every pass.
+    // B: in pass u this wave fills k-row u * WAVES + wave; lane l owns columns 4 l .. 4 l + 3.
+    // Addresses are a wave-uniform base (scalar registers, advanced by scalar adds) plus a
+    // loop-invariant 32-bit lane offset, so that the K loop holds no vector address arithmetic:
+    // a vector ALU instruction between two MFMAs delays the second one.
+    const int ld_row = wave * ROWS_PER_LOAD + lane / KP;
+    const int ld_chunk = (lane % KP) ^ ((ld_row >> SWZ) & (KP - 1));
+    const uint32_t a_lane = (static_cast<uint32_t>(lane / KP) * static_cast<uint32_t>(K) + ld_chunk * 4) * 4u;  // bytes
+    const uint32_t b_lane = static_cast<uint32_t>(lane) * 16u;
+    const char* a_wave = reinterpret_cast<const char*>(A + static_cast<size_t>(row0 + wave * ROWS_PER_LOAD) * K);
+    const char* b_wave = reinterpret_cast<const char*>(B + static_cast<size_t>(wave) * N + col0);
+    const size_t a_pass = static_cast<size_t>(ROWS_PER_PASS) * K * 4;
+    const size_t b_pass = static_cast<size_t>(WAVES) * N * 4;
+
+    // Load number m (0 .. A_PER + B_PER - 1) of the tile that starts at k0.
+    auto issue_load = [&](float* as, float* bs, int k0, int m) {
+        if (m < A_PER)
+            direct_load16(a_wave + static_cast<size_t>(k0) * 4 + m * a_pass, a_lane,
+                          as + (m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK);
+        else
+            direct_load16(b_wave + static_cast<size_t>(k0) * N * 4 + (m - A_PER) * b_pass, b_lane,
+                          bs + ((m - A_PER) * WAVES + wave) * BN);
+    };
+    constexpr int LOADS = A_PER + B_PER;
+
+    // Operand side.
+    const int sw = (l32 >> SWZ) & (KP - 1);
+    int a_off[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) a_off[s] = (wave_m * WM + l32) * BK + ((2 * s + lhi) ^ sw) * 4;
+    const int b_off = (4 * lhi) * BN + wave_n * WN + 4 * l32;
+
+    f32x4 fa[2][MI], fb[2][4];
+    auto read_frags = [&](const float* as, const float* bs, int s, int slot) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i) fa[slot][i] = *reinterpret_cast<const f32x4*>(&as[a_off[s] + i * 32 * BK]);
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj)
+            fb[slot][jj] = *reinterpret_cast<const f32x4*>(&bs[b_off + (8 * s + jj) * BN]);
+    };
+    // `between(m)` runs after the m-th MFMA of the group.
+    auto mfma_all = [&](int slot, auto between) {
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[slot][i][jj], fb[slot][jj][j], acc[i][j], 0, 0, 0);
+                    between((jj * MI + i) * NI + j);
+                }
+    };
+    auto nothing = [](int) {};
+
+    // One phase = everything between two barriers. It is entered right after the
+    // barrier that says "tile t is complete in (as, bs), nobody reads (as_n, bs_n)
+    // any more", while operand slot 1 still holds the last group of tile t-1:
+    //   read group 0 of tile t           -> slot 0
+    //   MFMAs of the last group of t-1   <- slot 1, with the direct loads of tile t+1 issued among them
+    //   groups 0 .. KS-2 of tile t, each preceded by the reads of the next group
+    //   wait for this wave's direct loads, barrier
+    auto phase = [&](float* as, float* bs, float* as_n, float* bs_n, int k_next, auto prefetch) {
+        read_frags(as, bs, 0, 0);
+        mfma_all(1, [&](int m) {
+            if constexpr (prefetch) {
+                if (m % LOAD_GAP == 0 && m / LOAD_GAP < LOADS) {
+                    issue_load(as_n, bs_n, k_next, m / LOAD_GAP);
+                    // The scheduler would otherwise bunch the loads together, and a burst of
+                    // them holds the wave (and with it the next MFMA) at the memory pipeline.
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        });
+#pragma unroll
+        for (int s = 0; s + 1 < KS; ++s) {
+            read_frags(as, bs, s + 1, (s + 1) & 1);
+            mfma_all(s & 1, nothing);
+        }
+#if PRISM_SGEMM5_SCHED
+        constexpr int G = 4 * MI * NI;  // MFMAs per group
+        constexpr int PLACED = prefetch ? (LOADS - 1) * LOAD_GAP + 1 : 0;  // MFMAs above the last sched_barrier
+        if constexpr (!prefetch) __builtin_amdgcn_sched_group_barrier(0x100, MI + 4, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, G - PLACED, 0);
+#pragma unroll
+        for (int s = 0; s + 1 < KS; ++s) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, MI + 4, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, G - 4, 0);
+        }
+#endif
+#if PRISM_SGEMM5_LATE_BARRIER
+        __builtin_amdgcn_sched_barrier(0);  // keep the MFMAs above the barrier: the direct loads get a whole tile to land
+#endif
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the direct loads are invisible to the compiler's wait counts
+        __syncthreads();
+    };
+    using yes = std::integral_constant<bool, true>;
+    using no = std::integral_constant<bool, false>;
+
+    // Slot 1 starts as zeros, so the "previous tile" MFMAs of the first phase add nothing.
+#pragma unroll
+    for (int i = 0; i < MI; ++i) fa[1][i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) fb[1][jj] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    auto load_tile0 = [&](float* as, float* bs) {
+#pragma unroll
+        for (int m = 0; m < LOADS; ++m) issue_load(as, bs, 0, m);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+    };
+
+    // The launcher guarantees K % BK == 0 and K > 0. Tiles alternate between the
+    // two stages such that the last tile always sits in stage 1.
+    const int k_tiles = K / BK;
+    int t = 0;
+    if (k_tiles & 1) {
+        load_tile0(As1, Bs1);
+        if (k_tiles > 1) {
+            phase(As1, Bs1, As0, Bs0, BK, yes{});
+            t = 1;
+        }
+    } else {
+        load_tile0(As0, Bs0);
+    }
+    for (; t + 2 < k_tiles; t += 2) {
+        phase(As0, Bs0, As1, Bs1, (t + 1) * BK, yes{});
+        phase(As1, Bs1, As0, Bs0, (t + 2) * BK, yes{});
+    }
+    if (k_tiles > 1) phase(As0, Bs0, As1, Bs1, (t + 1) * BK, yes{});
+    phase(As1, Bs1, As0, Bs0, 0, no{});
+    mfma_all(1, nothing);  // last group of the last tile
+
+    // Epilogue: a lane holds columns 4 l32 .. 4 l32 + 3 of 16 rows per 32-row block.
+    float* c_lane = C + static_cast<size_t>(row0 + wave_m * WM + 4 * lhi) * N + col0 + wave_n * WN + 4 * l32;
+    auto write_back = [&](auto read_c) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                f32x4* c = reinterpret_cast<f32x4*>(c_lane + static_cast<size_t>(i * 32 + 8 * (v / 4) + (v % 4)) * N);
+                f32x4 r;
+                if constexpr (read_c) {
+                    const f32x4 old = *c;
+#pragma unroll
+                    for (int j = 0; j < NI; ++j) r[j] = __builtin_fmaf(alpha, acc[i][j][v], beta * old[j]);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < NI; ++j) r[j] = alpha * acc[i][j][v];
+                }
+                *c = r;
+            }
+            __builtin_amdgcn_sched_barrier(0);  // at most one 32-row block of C reads in flight (64 registers)
+        }
+    };
+    if (beta == 0.0f) write_back(no{}); else write_back(yes{});
+}
+
 // --------------------------------------------------------------- launchers --
 
 template <int BM, int BN, int BK, int TM, int TN, bool VEC>
@@ -406,6 +662,28 @@ int run_wave_tile(int M, int N, int K, float alpha, const float* A, const float*
         sgemm_wave_tile_kernel<BM, BN, BK, WM, WN, true><<<grid, block, 0, s>>>(
             M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n);
     return check_launch("sgemm_wave_tile_kernel");
+}
+
+// Whole-tile kernel when the problem is made of 256 x 256 tiles and there are
+// enough of them to give every CU one; otherwise the general kernel.
+#ifndef PRISM_SGEMM5_DMA
+#define PRISM_SGEMM5_DMA 1
+#endif
+#ifndef PRISM_SGEMM5_DMA_MIN_TILES
+#define PRISM_SGEMM5_DMA_MIN_TILES 256
+#endif
+template <int BM, int BN, int BK, int WM, int WN>
+bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const float* B, float beta,
+                       float* C, hipStream_t s, int* rc) {
+    if (!PRISM_SGEMM5_DMA) return false;
+    if (K <= 0 || M % BM || N % BN || K % BK || !aligned16(A) || !aligned16(B) || !aligned16(C)) return false;
+    const int tiles_m = M / BM, tiles_n = N / BN;
+    if (static_cast<long long>(tiles_m) * tiles_n < PRISM_SGEMM5_DMA_MIN_TILES) return false;
+    const dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n), block((BM / WM) * (BN / WN) * kWave);
+    sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN><<<grid, block, 0, s>>>(M, N, K, alpha, A, B, beta, C,
+                                                                          tiles_m, tiles_n);
+    *rc = check_launch("sgemm_wave_tile_dma_kernel");
+    return true;
 }
 
 }  // namespace
@@ -453,6 +731,12 @@ int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, 
             // BM = BN = 128, BK = 16, WM = WN = 64: the tile shape of
             // run_my_sgemm_5 (evals/4090_sgemm/runner.cu:194-202), with four
             // 64-lane waves in place of four 32-lane warps.
+            {
+                // K tiles of 32 (128 KiB of LDS) when K allows, else of 16.
+                int rc = 0;
+                if (try_wave_tile_dma<256, 256, 32, 128, 128>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
+                if (try_wave_tile_dma<256, 256, 16, 128, 128>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
+            }
             return run_wave_tile<PRISM_SGEMM5_CFG>(M, N, K, alpha, A, B, beta, C, s);
     }
     return fail(1, "prism_sgemm: unknown kernel number %d", variant);

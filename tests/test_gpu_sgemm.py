@@ -154,6 +154,29 @@ def test_baseline_tail_shapes(prism, oracle, shape):
         assert np.max(np.abs(got - want)) <= t, f"kernel {v} shape {shape}"
 
 
+@pytest.mark.parametrize("shape", [(4096, 4096, 16), (4096, 4096, 32), (4096, 4096, 48), (4096, 4096, 80),
+                                   (2048, 8192, 96), (8192, 2048, 64)])
+def test_wave_tile_whole_tile_path(prism, oracle, shape):
+    """Shapes made of at least 256 whole 256 x 256 tiles take kernel 5's direct-to-LDS path; K covers
+    one, an even and an odd number of K tiles. Every element is checked, with and without reading C,
+    and against the general path (same data at a 4-byte offset, which the whole-tile path rejects)."""
+    M, N, K = shape
+    A, B, Cm = oracle.gen_sgemm(M, N, K, seed=K)
+    t = tol(oracle, K, A, B, -0.5, Cm)
+    got = run(prism, 5, 1.5, A, B, -0.5, Cm)
+    assert np.max(np.abs(got - oracle.np_sgemm_f64(1.5, A, B, -0.5, Cm))) <= t
+    poison = np.full((M, N), np.nan, dtype=np.float32)
+    got0 = run(prism, 5, 1.0, A, B, 0.0, poison)
+    assert np.max(np.abs(got0 - oracle.np_sgemm_f64(1.0, A, B, 0.0))) <= oracle.sgemm_tolerance(K, A, B)
+    buf = torch.full((M * N + 8,), 777.0, dtype=torch.float32, device=DEV)
+    c = buf[1:1 + M * N]
+    c.copy_(dev(Cm).reshape(-1))
+    prism.sgemm(M, N, K, 1.5, dev(A), dev(B), -0.5, c, variant=5)
+    out = host(buf)
+    assert out[0] == 777.0 and np.all(out[1 + M * N:] == 777.0)
+    assert np.max(np.abs(out[1:1 + M * N].reshape(M, N) - got)) <= 2 * t
+
+
 def _sampled_check(prism, oracle, M, N, K, alpha, beta, variant, rows=48):
     """Full-size run, checked on `rows` random rows against an fp64 product."""
     g = torch.Generator(device=DEV)
