@@ -1,0 +1,52 @@
+// Global memory -> LDS without staging registers (gfx950 global_load_lds_dwordx4).
+#pragma once
+
+#include <cstdint>
+
+#include <hip/hip_runtime.h>
+
+namespace prism {
+
+// One wave-wide load of 16 B per lane from global memory straight into LDS: lane l
+// reads base + lane_offset(l) and lands at lds_dst + 16 l (1 KiB of contiguous LDS
+// per instruction). Written as inline assembly for its addressing mode: a scalar
+// base plus a 32-bit vector offset. The compiler's own selection for the
+// direct-load builtin builds a 64-bit vector address with vector ALU instructions
+// for every load, and a vector ALU instruction between two MFMAs delays the second
+// one (about 12 clocks each, measured with one wave per SIMD). M0 carries the LDS
+// address; a scalar write of M0 needs one wait state before the load reads it.
+//
+// The compiler does not see these loads in its wait counts: the caller waits with an
+// explicit s_waitcnt (waitcnt_imm below) before the barrier that publishes the data.
+__device__ __forceinline__ void direct_load16(const char* base, uint32_t lane_offset, const void* lds_dst) {
+    const uint32_t lds_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+        (const __attribute__((address_space(3))) void*)lds_dst));
+    // M0 is listed as clobbered so that the compiler does not assume a value of its own survives
+    // (clang warns that M0 is a reserved register; the kernels here have no other user of it).
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(lane_offset), "s"(base), "s"(lds_addr)
+                 : "memory", "m0");
+#pragma clang diagnostic pop
+}
+
+// s_waitcnt immediate (gfx9 encoding): at most `vm` vector-memory and `lgkm`
+// LDS/scalar operations outstanding; vmcnt[3:0] in bits 3:0 and vmcnt[5:4] in bits
+// 15:14, lgkmcnt in bits 11:8, the export counter left at its maximum.
+constexpr int kVmMax = 63, kLgkmMax = 15;
+constexpr int waitcnt_imm(int vm, int lgkm) {
+    return (vm & 0xF) | ((vm >> 4) << 14) | (0x7 << 4) | ((lgkm & 0xF) << 8);
+}
+
+// Workgroup barrier that orders LDS traffic only: waits for this wave's LDS
+// operations, not for its outstanding global loads (__syncthreads() waits for
+// both, which would drain a software pipeline of loads at every barrier).
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+}  // namespace prism

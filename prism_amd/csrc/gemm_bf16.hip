@@ -4,12 +4,18 @@
 // This is the gfx950 counterpart of the reference's Hopper kernel
 // (examples/h100_matmul.py:20-297, generated/cutlass_my_h100_match_no_tail.cu):
 //   reference                                   here
-//   wgmma m64n256k16 from swizzled smem     ->  v_mfma_f32_32x32x16_bf16 from padded LDS rows
-//   TMA bulk copies + mbarrier ring (4 x)   ->  16 B global loads staged in registers one K
-//                                               step ahead, two LDS buffers, one barrier a step
+//   wgmma m64n256k16 from swizzled smem     ->  v_mfma_f32_32x32x16_bf16, 4 waves x 128x128, swizzled LDS
+//   TMA bulk copies + mbarrier ring (4 x)   ->  long K: buffer loads into two register sets two K tiles
+//                                               ahead, two LDS stages (gemm_bf16_staged_kernel);
+//                                               short K: direct-to-LDS loads, ring of two stages
+//                                               (gemm_bf16_ring_kernel)
 //   1 producer + 2 consumer warpgroups      ->  every wave loads and multiplies
-//   persistent CTAs + 16x8 super-tiles      ->  one workgroup per tile, XCD-aware tile order
-//   K tail dropped, M/N multiples required  ->  any M, N, K (zero-filled edge tiles)
+//   persistent CTAs + 16x8 super-tiles      ->  one workgroup per tile, 16x16 super-blocks with an
+//                                               8x4 patch per XCD (tile_map.h)
+//   K tail dropped, M/N multiples required  ->  any M, N, K: problems that are not whole 256x256x64
+//                                               tiles take gemm_bf16_kernel (zero-filled edge tiles,
+//                                               16 B global loads staged in registers one K step
+//                                               ahead, padded LDS rows)
 //
 // prism_gemm_bf16 calls it with (P, Q) = (A, B) and an fp32 OUT = D[M][N].
 // prism_runmyh100 needs the reference's column-major bf16 C (C[n * M + m],
@@ -21,19 +27,17 @@
 // P[r = l % 32][k = 8 * (l / 32) .. + 7] and Q[c = l % 32][same k]; result
 // register v of lane l is OUT[8 * (v / 4) + 4 * (l / 32) + v % 4][l % 32].
 //
-// LDS rows are BK + 8 elements (144 B for BK = 64): eight lanes reading 16 B from
-// eight consecutive rows then cover all banks exactly once.
+// In gemm_bf16_kernel LDS rows are BK + 8 elements (144 B for BK = 64): eight lanes
+// reading 16 B from eight consecutive rows then cover all banks exactly once.
 #include <type_traits>
 
 #include "common.h"
+#include "direct_load.h"
 #include "tile_map.h"
 
 // Block tile BM x BN x BK and wave tile WM x WN.
 #ifndef PRISM_BF16_SCHED
 #define PRISM_BF16_SCHED 1
-#endif
-#ifndef PRISM_BF16_DMA
-#define PRISM_BF16_DMA 1
 #endif
 #ifndef PRISM_BF16_CFG
 #define PRISM_BF16_CFG 256, 256, 64, 128, 128
@@ -249,52 +253,56 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_kerne
     }
 }
 
-// ------------------------------------------------------- full-tile kernel --
-// Same product for problems made of whole tiles with 16 B aligned rows; global
-// data goes straight into LDS (global_load_lds_dwordx4, no staging registers,
-// no LDS-write instructions), which is the role TMA plays in the reference
-// (evals/h100_bench/utils.cuh:238-273).
+// ------------------------------------------------- direct-to-LDS ring kernel --
+// Whole tiles, K a multiple of BK and at least STAGES K tiles. Global data goes
+// straight into LDS (global_load_lds_dwordx4: no staging registers, no LDS write
+// instructions), the role TMA plays in the reference
+// (evals/h100_bench/utils.cuh:238-273). K tiles travel through a ring of STAGES
+// LDS stages; the direct loads of tile t + STAGES - 1 are issued while tile t is
+// multiplied, into the stage tile t-1 has just left.
 //
 // A wave-wide direct load writes 1 KiB of contiguous LDS (lane l lands at
 // base + 16 l), so rows cannot be padded. Bank conflicts are avoided the way the
 // reference's 128 B swizzle does it (utils.cuh:6-16): the 16 B chunk c of row r
-// is stored in slot c ^ ((r >> SWZ) & (chunks_per_row - 1)); the load side
-// applies the permutation to the global address, the MFMA operand reads apply it
-// to the LDS address.
+// sits in slot c ^ ((r >> SWZ) & (chunks_per_row - 1)); the load side applies the
+// permutation to the global address, the operand reads to the LDS address.
 //
-// Two LDS stages of one K tile each, declared as separate arrays so that the
-// compiler's wait-count logic knows loads into one stage do not feed reads of
-// the other. Step t: issue the loads of tile t+1 into the idle stage, multiply
-// tile t, barrier (which also waits for the loads), prefetch the first operands
-// of tile t+1.
-#ifndef PRISM_BF16_DMA_SPLIT
-#define PRISM_BF16_DMA_SPLIT 1
-#endif
-#ifndef PRISM_BF16_SWZ
-#define PRISM_BF16_SWZ 1
-#endif
-
-template <int BM, int BN, int BK, int WM, int WN, int SWZ, typename OutT>
-__global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_dma_kernel(
+// With one wave per SIMD nothing hides a stall and every vector ALU instruction a
+// wave issues between two MFMAs delays the second one, so the K loop is laid out
+// by hand and pinned with scheduling barriers: MFMA, one LDS read, MFMA, one LDS
+// read, ...; the operands of a group of 16 MFMAs are read behind the first half
+// of the group before it; loads use a scalar base and a fixed lane offset (no
+// vector ALU work in the loop).
+//
+// Two shapes are compiled. 64 x 2 stages is the one used (short K): a direct load
+// cannot be issued before its stage is free, so it has less than one tile time to
+// land, and for long K the register-staged kernel below is faster. 32 x 4 stages
+// gives loads three tile times but reads half cache lines (64 B per row and
+// tile) and measured slower than both.
+template <int BM, int BN, int BK, int STAGES, int WM, int WN, typename OutT>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_kernel(
     int R, int Cn, int K, const uint16_t* __restrict__ P, const uint16_t* __restrict__ Q,
     OutT* __restrict__ OUT, int tiles_m, int tiles_n) {
+    static_assert((BK == 32 || BK == 64) && (STAGES == 2 || STAGES == 4), "ring shape");
+    constexpr int KP = BK / 8;                        // 16 B chunks per row
+    constexpr int SWZ = KP == 4 ? 2 : 1;
+    constexpr int KS = BK / 16;                       // k-groups (one MFMA deep) per tile
+    constexpr int AHEAD = STAGES - 1;                 // tiles in flight ahead of the one being multiplied
     constexpr int WAVES_N = BN / WN;
     constexpr int WAVES = (BM / WM) * WAVES_N;
     constexpr int MI = WM / 32, NI = WN / 32;
-    constexpr int KP = BK / 8;                       // 16 B chunks per row
-    constexpr int KS = BK / 16;                      // k-substeps per tile
-    constexpr int ROWS_PER_LOAD = kWave / KP;        // rows one wave-wide load covers
+    constexpr int ROWS_PER_LOAD = kWave / KP;         // rows one wave-wide load covers
     constexpr int ROWS_PER_PASS = ROWS_PER_LOAD * WAVES;
     static_assert(BM % ROWS_PER_PASS == 0 && BN % ROWS_PER_PASS == 0, "whole load passes");
     constexpr int P_PER = BM / ROWS_PER_PASS, Q_PER = BN / ROWS_PER_PASS;  // loads per wave per tile
-    static_assert(KS % 2 == 0 && (KP & (KP - 1)) == 0, "tile shape");
-    static_assert(((ROWS_PER_PASS >> SWZ) % KP) == 0 && ((32 >> SWZ) % KP == 0 || KP <= (32 >> SWZ)),
+    constexpr int LOADS = P_PER + Q_PER, READS = MI + NI, GROUP = MI * NI;
+    constexpr int GAPS = GROUP - READS;               // MFMAs of a group with nothing behind them yet
+    static_assert(GAPS > 0 && LOADS <= GAPS * KS, "the loads of a tile fit between the MFMAs of a phase");
+    static_assert(((ROWS_PER_PASS >> SWZ) % KP) == 0 && ((32 >> SWZ) % KP) == 0,
                   "the swizzle term must repeat with the load pass and the 32-row MFMA block");
 
-    __shared__ __attribute__((aligned(1024))) uint16_t Ps0[BM * BK];
-    __shared__ __attribute__((aligned(1024))) uint16_t Ps1[BM * BK];
-    __shared__ __attribute__((aligned(1024))) uint16_t Qs0[BN * BK];
-    __shared__ __attribute__((aligned(1024))) uint16_t Qs1[BN * BK];
+    __shared__ __attribute__((aligned(1024))) uint16_t Ps[STAGES][BM * BK];
+    __shared__ __attribute__((aligned(1024))) uint16_t Qs[STAGES][BN * BK];
 
     int tm, tn;
     xcd_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
@@ -302,7 +310,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_dma_k
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
-    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // wave-uniform, lives in an SGPR
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
     const int l32 = lane & 31, lhi = lane >> 5;
 
@@ -314,33 +322,26 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_dma_k
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    // Load side: in pass u this wave fills LDS rows [u * ROWS_PER_PASS + wave * ROWS_PER_LOAD, + ROWS_PER_LOAD);
-    // lane l owns row (l / KP) of those and slot (l % KP), which holds global chunk
-    // slot ^ swizzle(row). The swizzle term is the same in every pass, so the lane's
-    // byte offset from the pass's first row is loop-invariant and everything else is scalar.
+    // Load side: lane l of a wave-wide load owns row l / KP of its rows and slot l % KP.
     const int ld_row = wave * ROWS_PER_LOAD + lane / KP;
     const int ld_chunk = (lane % KP) ^ ((ld_row >> SWZ) & (KP - 1));
-    const uint32_t lane_off = static_cast<uint32_t>((lane / KP) * K + ld_chunk * 8) * 2u;  // bytes
+    const uint32_t lane_off = (static_cast<uint32_t>(lane / KP) * static_cast<uint32_t>(K) + ld_chunk * 8) * 2u;  // bytes
     const char* p_wave = reinterpret_cast<const char*>(P + static_cast<size_t>(row0 + wave * ROWS_PER_LOAD) * K);
     const char* q_wave = reinterpret_cast<const char*>(Q + static_cast<size_t>(col0 + wave * ROWS_PER_LOAD) * K);
     const size_t pass_bytes = static_cast<size_t>(ROWS_PER_PASS) * K * 2;
-
-    typedef const __attribute__((address_space(1))) void* gptr_t;
-    typedef __attribute__((address_space(3))) void* lptr_t;
-    auto issue_loads = [&](uint16_t* ps, uint16_t* qs, int k0) {
-#pragma unroll
-        for (int u = 0; u < P_PER; ++u)
-            __builtin_amdgcn_global_load_lds((gptr_t)(p_wave + u * pass_bytes + static_cast<size_t>(k0) * 2 + lane_off),
-                                             (lptr_t)(ps + (u * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK), 16, 0, 0);
-#pragma unroll
-        for (int u = 0; u < Q_PER; ++u)
-            __builtin_amdgcn_global_load_lds((gptr_t)(q_wave + u * pass_bytes + static_cast<size_t>(k0) * 2 + lane_off),
-                                             (lptr_t)(qs + (u * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK), 16, 0, 0);
+    // Load number m (0 .. LOADS - 1) of the tile that starts at k0, into stage `stage`.
+    auto issue_load = [&](int stage, int k0, int m) {
+        if (m < P_PER)
+            direct_load16(p_wave + static_cast<size_t>(k0) * 2 + m * pass_bytes, lane_off,
+                          &Ps[stage][(m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]);
+        else
+            direct_load16(q_wave + static_cast<size_t>(k0) * 2 + (m - P_PER) * pass_bytes, lane_off,
+                          &Qs[stage][((m - P_PER) * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]);
     };
 
-    // Operand side: row (wave tile origin + 32 i + l32), chunk (2 kk + lhi) -> slot.
+    // Operand side: row (wave tile origin + 32 i + l32), chunk 2 kk + lhi of the row.
     const int sw = (l32 >> SWZ) & (KP - 1);
-    int p_off[KS], q_off[KS];  // element offsets inside a stage for i = 0 / j = 0
+    int p_off[KS], q_off[KS];
 #pragma unroll
     for (int kk = 0; kk < KS; ++kk) {
         const int slot = (2 * kk + lhi) ^ sw;
@@ -348,60 +349,57 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_dma_k
         q_off[kk] = (wave_n * WN + l32) * BK + slot * 8;
     }
     bf16x8 fa[2][MI], fb[2][NI];
-    auto read_frags = [&](const uint16_t* ps, const uint16_t* qs, int kk, int slot) {
-#pragma unroll
-        for (int i = 0; i < MI; ++i)
-            fa[slot][i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&ps[p_off[kk] + i * 32 * BK]));
-#pragma unroll
-        for (int j = 0; j < NI; ++j)
-            fb[slot][j] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&qs[q_off[kk] + j * 32 * BK]));
+    // Read number r (0 .. READS - 1) of k-group kk of the tile in `stage`, into operand slot kk & 1.
+    auto read_one = [&](int stage, int kk, int r) {
+        if (r < MI)
+            fa[kk & 1][r] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&Ps[stage][p_off[kk] + r * 32 * BK]));
+        else
+            fb[kk & 1][r - MI] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&Qs[stage][q_off[kk] + (r - MI) * 32 * BK]));
     };
-
-    auto mfma_all = [&](int slot) {
+    // The MFMAs of operand slot `slot`; `after(m)` is issued right behind the m-th.
+    auto mfma_group = [&](int slot, auto after) {
 #pragma unroll
         for (int i = 0; i < MI; ++i)
 #pragma unroll
-            for (int j = 0; j < NI; ++j)
+            for (int j = 0; j < NI; ++j) {
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[slot][i], fb[slot][j], acc[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                after(i * NI + j);
+                __builtin_amdgcn_sched_barrier(0);
+            }
     };
 
-    // One phase = everything between two barriers. It is entered right after the
-    // barrier that says "tile t is complete in (ps, qs), nobody reads (ps_n, qs_n)
-    // any more", and while operand slot 1 still holds the last k-substep of tile
-    // t-1. That substep's MFMAs are issued here, after the barrier, so that they
-    // cover the barrier skew and the latency of the first operand reads of tile t:
-    //   read substep 0 of tile t          -> slot 0
-    //   MFMAs of the last substep of t-1  <- slot 1, with the direct loads of tile t+1 issued between them
-    //   substeps 0 .. KS-2 of tile t, each preceded by the reads of the next substep
-    //   barrier (also waits for the direct loads)
-    // `prefetch`: tile t+1 exists and goes to (ps_n, qs_n).
-    auto phase = [&](uint16_t* ps, uint16_t* qs, uint16_t* ps_n, uint16_t* qs_n, int k_next, auto prefetch) {
-        read_frags(ps, qs, 0, 0);
-        mfma_all(1);
-        if constexpr (prefetch) issue_loads(ps_n, qs_n, k_next);
+    // One phase = everything between two barriers. Entered right after the barrier
+    // that says "tile t is complete in stage S and nobody reads the stage of tile t-1
+    // any more", while operand slot 1 holds the last k-group of tile t-1. Group g of
+    // the phase (g = 0 .. KS-1) issues the MFMAs of the k-group read one group earlier
+    // (g = 0: the last one of tile t-1); behind its first READS MFMAs go the reads of
+    // k-group g of tile t, behind the others the direct loads of tile t+AHEAD into the
+    // stage tile t-1 has left. Then: wait until at most the loads of the younger tiles
+    // are in flight, barrier.
+    auto phase = [&](auto stage_c, auto prefetch, int k_next) {
+        constexpr int S = decltype(stage_c)::value;
 #pragma unroll
-        for (int kk = 0; kk + 1 < KS; ++kk) {
-            read_frags(ps, qs, kk + 1, (kk + 1) & 1);
-            mfma_all(kk & 1);
+        for (int g = 0; g < KS; ++g) {
+            mfma_group((g + 1) & 1, [&](int m) {
+                if (m < READS) {
+                    read_one(S, g, m);
+                } else if constexpr (prefetch) {
+                    const int ld = g * GAPS + (m - READS);
+                    if (ld < LOADS) issue_load((S + AHEAD) % STAGES, k_next, ld);
+                }
+            });
         }
-#if PRISM_BF16_SCHED
-        // The direct loads are spread over the first DMA_SPLIT groups of MFMAs.
-        constexpr int LOADS = prefetch ? (P_PER + Q_PER) : 0;
-        constexpr int L_PER = (LOADS + PRISM_BF16_DMA_SPLIT - 1) / PRISM_BF16_DMA_SPLIT;
-        __builtin_amdgcn_sched_group_barrier(0x100, MI + NI, 0);
-        sched_substep<0, 0, L_PER, MI * NI>();
-#pragma unroll
-        for (int kk = 0; kk + 1 < KS; ++kk) {
-            if (kk + 1 < PRISM_BF16_DMA_SPLIT)
-                sched_substep<MI + NI, 0, L_PER, MI * NI>();
-            else
-                sched_substep<MI + NI, 0, 0, MI * NI>();
-        }
-#endif
-        __syncthreads();
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(prefetch ? (AHEAD - 1) * LOADS : 0, 0));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
     };
     using yes = std::integral_constant<bool, true>;
     using no = std::integral_constant<bool, false>;
+    using s0 = std::integral_constant<int, 0>;
+    using s1 = std::integral_constant<int, 1>;
+    using s2 = std::integral_constant<int, 2>;
+    using s3 = std::integral_constant<int, 3>;
 
     // Slot 1 starts as zeros, so the "previous tile" MFMAs of the first phase add nothing.
 #pragma unroll
@@ -409,28 +407,48 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_dma_k
 #pragma unroll
     for (int j = 0; j < NI; ++j) fb[1][j] = bf16x8{};
 
-    // The launcher guarantees K % BK == 0 and K > 0. Tiles alternate between the
-    // two stages such that the last tile always sits in stage 1.
+    // The launcher guarantees K % BK == 0 and at least STAGES tiles. Tile t lives in
+    // stage (first + t) % STAGES with `first` chosen such that the last tile sits in the
+    // last stage: the ragged part of the tile count is handled up front and the rest
+    // runs in whole rings.
     const int k_tiles = K / BK;
-    int t = 0;
-    if (k_tiles & 1) {
-        issue_loads(Ps1, Qs1, 0);
-        __syncthreads();
-        if (k_tiles > 1) {
-            phase(Ps1, Qs1, Ps0, Qs0, BK, yes{});
-            t = 1;
+    const int ragged = k_tiles % STAGES;
+    const int first = (STAGES - ragged) % STAGES;
+#pragma unroll
+    for (int t = 0; t < AHEAD; ++t)
+#pragma unroll
+        for (int m = 0; m < LOADS; ++m) issue_load((first + t) % STAGES, t * BK, m);
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm((AHEAD - 1) * LOADS, 0));
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+
+    int k_next = AHEAD * BK;  // first k of the tile the next phase prefetches
+    if constexpr (STAGES == 4) {
+        if (ragged == 3) { phase(s1{}, yes{}, k_next); k_next += BK; }
+        if (ragged >= 2) { phase(s2{}, yes{}, k_next); k_next += BK; }
+        if (ragged >= 1) { phase(s3{}, yes{}, k_next); k_next += BK; }
+        for (int ring = k_tiles / STAGES; ring > 1; --ring) {
+            phase(s0{}, yes{}, k_next);
+            phase(s1{}, yes{}, k_next + BK);
+            phase(s2{}, yes{}, k_next + 2 * BK);
+            phase(s3{}, yes{}, k_next + 3 * BK);
+            k_next += 4 * BK;
         }
+        phase(s0{}, yes{}, k_next);
+        phase(s1{}, no{}, 0);
+        phase(s2{}, no{}, 0);
+        phase(s3{}, no{}, 0);
     } else {
-        issue_loads(Ps0, Qs0, 0);
-        __syncthreads();
+        if (ragged == 1) { phase(s1{}, yes{}, k_next); k_next += BK; }
+        for (int ring = k_tiles / STAGES; ring > 1; --ring) {
+            phase(s0{}, yes{}, k_next);
+            phase(s1{}, yes{}, k_next + BK);
+            k_next += 2 * BK;
+        }
+        phase(s0{}, yes{}, k_next);
+        phase(s1{}, no{}, 0);
     }
-    for (; t + 2 < k_tiles; t += 2) {
-        phase(Ps0, Qs0, Ps1, Qs1, (t + 1) * BK, yes{});
-        phase(Ps1, Qs1, Ps0, Qs0, (t + 2) * BK, yes{});
-    }
-    if (k_tiles > 1) phase(Ps0, Qs0, Ps1, Qs1, (t + 1) * BK, yes{});
-    phase(Ps1, Qs1, Ps0, Qs0, 0, no{});
-    mfma_all(1);  // last k-substep of the last tile
+    mfma_group(1, [](int) {});  // last k-group of the last tile
 
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
@@ -446,6 +464,230 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_dma_k
     }
 }
 
+// ------------------------------------------- register-staged pipeline kernel --
+// Whole tiles, K a multiple of 64 and at least 5 K tiles. Two LDS stages of one
+// 256 x 256 x 64 tile pair each (128 KiB), plus two register sets that each hold
+// a wave's share of one more tile pair (16 x 16 B per lane). Tile t+3 is loaded
+// from global memory into registers while tile t is multiplied, and is written
+// to LDS two tiles later, so a load has two tile times (about 4000 clocks) to
+// land. A direct-to-LDS load cannot be issued before its LDS stage is free,
+// which with two stages leaves it less than one tile time; measured with
+// all-zero operands (no power throttling), waiting for those loads cost 35 % of
+// the run time. This is the depth the reference gets from its four-stage
+// mbarrier ring (QSIZE = 4, generated/cutlass_my_h100_match_no_tail.cu:117);
+// 160 KiB of LDS cannot hold four such stages, registers can hold two.
+//
+// Every barrier orders LDS traffic only (lds_barrier), so global loads stay in
+// flight across it. The K loop is laid out by hand and pinned with scheduling
+// barriers: between two barriers a wave issues 64 MFMAs; behind the first 8 of
+// every group of 16 go the LDS reads of the next group's operands, behind the
+// other 8 alternately one LDS write of a staged 16 B packet (tile t+1) and the
+// global load that refills its registers (tile t+3).
+//
+// LDS rows are 128 B (8 chunks of 16 B); chunk c of row r sits in slot
+// c ^ ((r >> 1) & 7): a wave writes 1 KiB of contiguous LDS per instruction, and
+// the 16 rows a quarter-wave reads with ds_read_b128 cover all 64 banks.
+template <int BM, int BN, int WM, int WN, typename OutT>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_staged_kernel(
+    int R, int Cn, int K, const uint16_t* __restrict__ P, const uint16_t* __restrict__ Q,
+    OutT* __restrict__ OUT, int tiles_m, int tiles_n) {
+    constexpr int BK = 64, KP = 8, SWZ = 1, KS = 4;
+    constexpr int WAVES_N = BN / WN;
+    constexpr int WAVES = (BM / WM) * WAVES_N;
+    constexpr int MI = WM / 32, NI = WN / 32;
+    constexpr int ROWS_PER_LOAD = kWave / KP;         // 8 rows of 128 B per wave-wide access
+    constexpr int ROWS_PER_PASS = ROWS_PER_LOAD * WAVES;
+    static_assert(BM % ROWS_PER_PASS == 0 && BN % ROWS_PER_PASS == 0, "whole load passes");
+    constexpr int P_PER = BM / ROWS_PER_PASS, Q_PER = BN / ROWS_PER_PASS;
+    constexpr int PACKETS = P_PER + Q_PER;            // 16 B packets per lane per tile pair
+    constexpr int READS = MI + NI, GROUP = MI * NI;
+    static_assert(2 * PACKETS == (GROUP - READS) * KS, "one write and one load behind every free MFMA of a phase");
+
+    __shared__ __attribute__((aligned(1024))) uint16_t Ps[2][BM * BK];
+    __shared__ __attribute__((aligned(1024))) uint16_t Qs[2][BN * BK];
+
+    int tm, tn;
+    xcd_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+    const int row0 = tm * BM, col0 = tn * BN;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+    const int l32 = lane & 31, lhi = lane >> 5;
+
+    f32x16 acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    // Global side: packet m of a tile pair is rows [(m * WAVES + wave) * 8, + 8) of P (m < P_PER) or Q;
+    // lane l owns row l / 8 of those and the chunk that belongs in slot l % 8. Addresses are a
+    // wave-uniform base plus a loop-invariant 32-bit lane offset.
+    const int ld_row = wave * ROWS_PER_LOAD + lane / KP;
+    const int ld_chunk = (lane % KP) ^ ((ld_row >> SWZ) & (KP - 1));
+    const uint32_t lane_off = (static_cast<uint32_t>(lane / KP) * static_cast<uint32_t>(K) + ld_chunk * 8) * 2u;  // bytes
+    // Buffer loads: the address is (descriptor base) + (vector offset) + (scalar offset), so a load
+    // needs no vector ALU work; offsets stay inside this workgroup's 256-row panel (the launcher
+    // checks that a panel is below 2 GiB).
+    const auto p_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(P + static_cast<size_t>(row0 + wave * ROWS_PER_LOAD) * K), 0, 0x7fffffff, 0x00020000);
+    const auto q_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(Q + static_cast<size_t>(col0 + wave * ROWS_PER_LOAD) * K), 0, 0x7fffffff, 0x00020000);
+    const int pass_bytes = ROWS_PER_PASS * K * 2;
+    u32x4 staged[2][PACKETS];
+    auto load_packet = [&](int set, int k0, int m) {
+        if (m < P_PER)
+            staged[set][m] = __builtin_amdgcn_raw_buffer_load_b128(p_rsrc, lane_off, m * pass_bytes + k0 * 2, 0);
+        else
+            staged[set][m] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, lane_off, (m - P_PER) * pass_bytes + k0 * 2, 0);
+    };
+    // LDS side: the same packet lands at (its first row) * 128 B + 16 B * lane.
+    auto write_packet = [&](int set, int m) {
+        uint16_t* dst = (m < P_PER) ? &Ps[set][(m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]
+                                    : &Qs[set][((m - P_PER) * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK];
+        *reinterpret_cast<u32x4*>(dst + lane * 8) = staged[set][m];
+    };
+
+    // Operand side: row (wave tile origin + 32 i + l32), chunk 2 kk + lhi of the row.
+    const int sw = (l32 >> SWZ) & (KP - 1);
+    int p_off[KS], q_off[KS];
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk) {
+        const int slot = (2 * kk + lhi) ^ sw;
+        p_off[kk] = (wave_m * WM + l32) * BK + slot * 8;
+        q_off[kk] = (wave_n * WN + l32) * BK + slot * 8;
+    }
+    bf16x8 fa[2][MI], fb[2][NI];
+    auto read_one = [&](int stage, int kk, int r) {
+        if (r < MI)
+            fa[kk & 1][r] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&Ps[stage][p_off[kk] + r * 32 * BK]));
+        else
+            fb[kk & 1][r - MI] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&Qs[stage][q_off[kk] + (r - MI) * 32 * BK]));
+    };
+    auto mfma_group = [&](int slot, auto after) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[slot][i], fb[slot][j], acc[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                after(i * NI + j);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+    };
+
+    // One phase = everything between two barriers, for the tile in stage S (tile t). Entered
+    // right after the barrier that says "tile t is complete in stage S and nobody reads stage
+    // S^1 any more", while operand slot 1 holds the last k-group of tile t-1. Register set S^1
+    // holds tile t+1 (loaded two phases ago): it is written to stage S^1 (`write`) and refilled
+    // with tile t+3, which starts at k_load (`load`).
+    auto phase = [&](auto stage_c, auto write, auto load, int k_load) {
+        constexpr int S = decltype(stage_c)::value;
+#pragma unroll
+        for (int g = 0; g < KS; ++g) {
+            mfma_group((g + 1) & 1, [&](int m) {
+                if (m < READS) {
+                    read_one(S, g, m);
+                } else {
+                    const int packet = (g * (GROUP - READS) + (m - READS)) / 2;
+                    if ((m - READS) % 2 == 0) {
+                        if constexpr (write) write_packet(S ^ 1, packet);
+                    } else {
+                        if constexpr (load) load_packet(S ^ 1, k_load, packet);
+                    }
+                }
+            });
+        }
+        lds_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    using yes = std::integral_constant<bool, true>;
+    using no = std::integral_constant<bool, false>;
+    using s0 = std::integral_constant<int, 0>;
+    using s1 = std::integral_constant<int, 1>;
+
+    // Slot 1 starts as zeros, so the "previous tile" MFMAs of the first phase add nothing.
+#pragma unroll
+    for (int i = 0; i < MI; ++i) fa[1][i] = bf16x8{};
+#pragma unroll
+    for (int j = 0; j < NI; ++j) fb[1][j] = bf16x8{};
+
+    // The launcher guarantees K % 64 == 0 and at least 5 tiles. Tiles alternate between the two
+    // stages (and register sets) such that the last tile always sits in stage 1: an odd tile
+    // count starts in stage 1 and runs one phase up front.
+    const int k_tiles = K / BK;
+    int k_load;  // first k of the tile the next phase loads
+    if (k_tiles & 1) {
+#pragma unroll
+        for (int m = 0; m < PACKETS; ++m) load_packet(1, 0, m);
+#pragma unroll
+        for (int m = 0; m < PACKETS; ++m) load_packet(0, BK, m);
+#pragma unroll
+        for (int m = 0; m < PACKETS; ++m) write_packet(1, m);
+        __builtin_amdgcn_sched_barrier(0);  // the set is reloaded only after it has been written out
+#pragma unroll
+        for (int m = 0; m < PACKETS; ++m) load_packet(1, 2 * BK, m);
+        lds_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        phase(s1{}, yes{}, yes{}, 3 * BK);
+        k_load = 4 * BK;
+    } else {
+#pragma unroll
+        for (int m = 0; m < PACKETS; ++m) load_packet(0, 0, m);
+#pragma unroll
+        for (int m = 0; m < PACKETS; ++m) load_packet(1, BK, m);
+#pragma unroll
+        for (int m = 0; m < PACKETS; ++m) write_packet(0, m);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int m = 0; m < PACKETS; ++m) load_packet(0, 2 * BK, m);
+        lds_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        k_load = 3 * BK;
+    }
+    // An even number of tiles remains, the first of them in stage 0; all but the last four run in
+    // pairs that write and load; the last four wind the pipeline down.
+    for (; k_load + BK < K; k_load += 2 * BK) {
+        phase(s0{}, yes{}, yes{}, k_load);
+        phase(s1{}, yes{}, yes{}, k_load + BK);
+    }
+    phase(s0{}, yes{}, yes{}, k_load);
+    phase(s1{}, yes{}, no{}, 0);
+    phase(s0{}, yes{}, no{}, 0);
+    phase(s1{}, no{}, no{}, 0);
+    mfma_group(1, [](int) {});  // last k-group of the last tile
+
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+            const int col = col0 + wave_n * WN + j * 32 + l32;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = row0 + wave_m * WM + i * 32 + 8 * (v / 4) + 4 * lhi + (v % 4);
+                store_out(&OUT[static_cast<size_t>(row) * Cn + col], acc[i][j][v]);
+            }
+        }
+    }
+}
+
+// Kernel choice for whole-tile problems: K tiles of 64; from PRISM_BF16_STAGED_MIN_K on the
+// register-staged pipeline (its two-tile load lead pays once the operands no longer sit in the
+// caches next to the CUs), below it the direct-to-LDS ring (lighter prologue).
+#ifndef PRISM_BF16_STAGED_MIN_K
+#define PRISM_BF16_STAGED_MIN_K 6144
+#endif
+#ifndef PRISM_BF16_RING_BK
+#define PRISM_BF16_RING_BK 64
+#endif
+#ifndef PRISM_BF16_RING_STAGES
+#define PRISM_BF16_RING_STAGES 2
+#endif
+
 template <int BM, int BN, int BK, int WM, int WN, typename OutT>
 int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, OutT* OUT,
                   hipStream_t s) {
@@ -453,24 +695,24 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
     constexpr size_t lds_bytes = 2ull * (BM + BN) * LD * sizeof(uint16_t);
     const int tiles_m = ceil_div(R, BM), tiles_n = ceil_div(Cn, BN);
     const dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n), block((BM / WM) * (BN / WN) * kWave);
-    const bool fast = (K > 0) && (R % BM == 0) && (Cn % BN == 0) && (K % BK == 0) && aligned16(P) && aligned16(Q);
-    auto launch = [&](auto kernel) -> int {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           static_cast<int>(lds_bytes));
-        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(gemm_bf16_kernel)");
-        kernel<<<grid, block, lds_bytes, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
-        return check_launch("gemm_bf16_kernel");
-    };
-    if (fast) {
-#if PRISM_BF16_DMA
-        gemm_bf16_dma_kernel<BM, BN, BK, WM, WN, PRISM_BF16_SWZ, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
-        return check_launch("gemm_bf16_dma_kernel");
-#else
-        return launch(gemm_bf16_kernel<BM, BN, BK, WM, WN, false, OutT>);
-#endif
+    const bool whole = (R % BM == 0) && (Cn % BN == 0) && aligned16(P) && aligned16(Q);
+    // The staged kernel addresses a 256-row panel with 32-bit offsets.
+    if (whole && K % 64 == 0 && K >= 5 * 64 && K >= PRISM_BF16_STAGED_MIN_K &&
+        static_cast<long long>(BM > BN ? BM : BN) * K * 2 < (1ll << 31)) {
+        gemm_bf16_staged_kernel<BM, BN, WM, WN, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
+        return check_launch("gemm_bf16_staged_kernel");
     }
-    return launch(gemm_bf16_kernel<BM, BN, BK, WM, WN, true, OutT>);
+    if (whole && K % PRISM_BF16_RING_BK == 0 && K >= PRISM_BF16_RING_BK * PRISM_BF16_RING_STAGES &&
+        static_cast<long long>(K) * 2 * 64 < (1ll << 32)) {  // 32-bit lane offsets inside a load's rows
+        gemm_bf16_ring_kernel<BM, BN, PRISM_BF16_RING_BK, PRISM_BF16_RING_STAGES, WM, WN, OutT>
+            <<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
+        return check_launch("gemm_bf16_ring_kernel");
+    }
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<BM, BN, BK, WM, WN, true, OutT>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+    if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(gemm_bf16_kernel)");
+    gemm_bf16_kernel<BM, BN, BK, WM, WN, true, OutT><<<grid, block, lds_bytes, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
+    return check_launch("gemm_bf16_kernel");
 }
 
 }  // namespace

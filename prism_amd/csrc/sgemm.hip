@@ -22,6 +22,7 @@
 // here accepts any M, N, K: full tiles take a guard-free path, edge tiles a
 // predicated one. When beta == 0, C is not read.
 #include "common.h"
+#include "direct_load.h"
 #include "tile_map.h"
 
 // Kernel 5 tile shape: BM, BN, BK, WM, WN.
@@ -411,23 +412,6 @@ __attribute__((amdgpu_waves_per_eu(PRISM_SGEMM5_WAVES_PER_EU))) void sgemm_wave_
 #ifndef PRISM_SGEMM5_LOAD_GAP
 #define PRISM_SGEMM5_LOAD_GAP 4
 #endif
-// One wave-wide 16 B-per-lane load from global memory straight into LDS: lane l
-// reads base + offset(l) and lands at lds_dst + 16 l. Written as inline assembly
-// for its addressing mode: a scalar base plus a 32-bit vector offset, which the
-// compiler's own selection for the direct-load builtin does not use (it builds a
-// 64-bit vector address with vector ALU instructions for every load). M0 carries
-// the LDS address; a scalar write of M0 needs one wait state before the load
-// reads it. The compiler does not see these loads in its wait counts: the caller
-// waits with an explicit vmcnt before the barrier that publishes the tile.
-__device__ __forceinline__ void direct_load16(const char* base, uint32_t lane_offset, const float* lds_dst) {
-    const uint32_t lds_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
-        (const __attribute__((address_space(3))) void*)lds_dst));
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :
-                 : "v"(lane_offset), "s"(base), "s"(lds_addr)
-                 : "memory", "m0");
-}
-
 template <int BM, int BN, int BK, int WM, int WN>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile_dma_kernel(
     int M, int N, int K, float alpha, const float* __restrict__ A, const float* __restrict__ B,
@@ -566,7 +550,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
 #if PRISM_SGEMM5_LATE_BARRIER
         __builtin_amdgcn_sched_barrier(0);  // keep the MFMAs above the barrier: the direct loads get a whole tile to land
 #endif
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the direct loads are invisible to the compiler's wait counts
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));  // the direct loads are invisible to the compiler's wait counts
         __syncthreads();
     };
     using yes = std::integral_constant<bool, true>;
@@ -581,7 +565,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
     auto load_tile0 = [&](float* as, float* bs) {
 #pragma unroll
         for (int m = 0; m < LOADS; ++m) issue_load(as, bs, 0, m);
-        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));
         __syncthreads();
     };
 

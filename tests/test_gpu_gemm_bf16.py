@@ -46,6 +46,26 @@ def test_fp32_output_vs_fp64_oracle(prism, oracle, shape):
     check_f32(oracle, host(D), A16, B16)
 
 
+@pytest.mark.parametrize("shape", [(256, 256, 128), (256, 512, 192), (512, 256, 256), (256, 256, 320), (512, 512, 1024),
+                                   (256, 512, 6144), (512, 256, 6208), (256, 256, 6272)])
+def test_whole_tile_paths(prism, oracle, shape):
+    """Problems made of whole 256 x 256 x 64 tiles leave the general kernel: K below 6144 takes the
+    direct-to-LDS ring (2, 3, 4, 5 and 16 K tiles here: even and odd ring counts), K from 6144 on the
+    register-staged pipeline (96, 97 and 98 K tiles). Every element is checked, for both output types."""
+    M, N, K = shape
+    A16, B16 = oracle.gen_gemm_bf16(M, N, K, seed=K + M)
+    D = prism.gemm_bf16(dev16(A16), dev16(B16))
+    check_f32(oracle, host(D), A16, B16)
+    Cc = torch.full((N * M + 64,), -7.0, dtype=torch.bfloat16, device=DEV)
+    prism.runmyh100(M, N, K, dev16(A16), dev16(B16), Cc[32:32 + N * M])
+    got = host(Cc.view(torch.int16)).view(np.uint16)
+    guard = np.float32(-7.0).view(np.uint32) >> 16
+    assert np.all(got[:32] == guard) and np.all(got[32 + N * M:] == guard)
+    ref = oracle.gemm_bf16_f64(A16, B16)
+    c = oracle.bf16_to_f32(got[32:32 + N * M]).reshape(N, M).T
+    assert np.all(np.abs(c - ref) <= 2.0**-8 * np.abs(ref) + REL * np.abs(ref).max())
+
+
 def test_fixture(prism, golden, oracle):
     A16, B16 = golden["bf16_A"], golden["bf16_B"]
     D = host(prism.gemm_bf16(dev16(A16), dev16(B16)))
