@@ -33,6 +33,21 @@
 // with more than one wave per tile was measured slower: the extra status
 // traffic costs more than the round trips it saves.
 //
+// Tile order. A tile may only wait for tiles that are already running. The
+// reference gets that from a ticket counter (examples/scan.py:88-99): tiles are
+// numbered in the order blocks start. The ticket is an agent-scope atomic on one
+// address, and its round trip (about 2 us) sits in front of every block's first
+// load: measured 5 % of the run time at 2^30. The default here is therefore
+// tile = workgroup id, which is deadlock-free as long as the dispatcher starts the
+// workgroups of a 1-D grid in id order on every XCD (then the lowest unfinished
+// tile is always running; this is the same assumption CUB's look-back scan makes
+// on NVIDIA hardware). PRISM_SCAN_ORDER=ticket in the environment selects the
+// reference's ticket order instead. In both modes the look-back wait is bounded
+// (kSpinLimit polls, several seconds): a wave that runs out stores the tile number
+// plus one into the workspace header (word 2) and carries on with a wrong prefix,
+// so that a broken ordering assumption shows up as a wrong result, not as a hung
+// GPU.
+//
 // Status words use RELAXED agent-scope atomics: the value travels inside the
 // atomic word, no other memory is communicated between tiles, so no fence is
 // needed (acquire/release here would write back and invalidate a whole L2 per
@@ -40,6 +55,9 @@
 //
 // HBM-bound: 8 algorithmic bytes per element (4 B read + 4 B write); status
 // traffic is 8 B per tile plus the polls.
+#include <cstdlib>
+#include <cstring>
+
 #include "common.h"
 
 namespace prism {
@@ -48,7 +66,8 @@ namespace {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned long long u64;
 
-constexpr size_t kHeaderBytes = 256;  // ticket counter lives here
+constexpr size_t kHeaderBytes = 256;  // word 0: ticket counter, word 2: look-back time-out report
+constexpr uint32_t kSpinLimit = 1u << 22;  // polls of one look-back window before giving up
 
 // Tile shapes: {threads, 16 B packets per lane}.
 struct SmallCfg { static constexpr int BLOCK = 1024, VPT = 4; };
@@ -111,10 +130,12 @@ __device__ __forceinline__ uint32_t wave_last_lane(uint32_t x) {
 
 // Exclusive prefix of tile `tile` (> 0): the sum of all earlier tiles. Run by
 // one whole wavefront; lane l inspects tile (window_end - l). Every tile below
-// `tile` has taken its ticket earlier, so it is running or finished and will
-// publish without waiting for anything later: the loop terminates.
-__device__ __forceinline__ uint32_t look_back(const u64* status, uint32_t tile, int lane) {
+// `tile` is running or finished (see "Tile order" above) and will publish without
+// waiting for anything later, so the loop terminates; the spin limit is a guard.
+__device__ __forceinline__ uint32_t look_back(const u64* status, uint32_t tile, int lane, uint32_t spin_limit,
+                                              uint32_t* timed_out) {
     uint32_t sum = 0;
+    uint32_t spins = 0;
     long long window_end = static_cast<long long>(tile) - 1;
     while (true) {
         const long long t = window_end - lane;
@@ -127,6 +148,10 @@ __device__ __forceinline__ uint32_t look_back(const u64* status, uint32_t tile, 
         // Lanes 0..first-prefix-lane are needed; all 64 when no prefix is in the window.
         const u64 needed = has_prefix ? ((2ull << __builtin_ctzll(has_prefix)) - 1ull) : ~0ull;
         if (is_invalid & needed) {
+            if (++spins > spin_limit) {
+                if (lane == 0) __hip_atomic_store(timed_out, tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                break;
+            }
             __builtin_amdgcn_s_sleep(PRISM_SCAN_SLEEP);
             continue;
         }
@@ -139,10 +164,11 @@ __device__ __forceinline__ uint32_t look_back(const u64* status, uint32_t tile, 
 }
 
 // VEC: in and out are 16 B aligned, full tiles use 16 B accesses.
-template <typename Cfg, bool VEC>
+// TICKET: tiles are numbered by the ticket counter, else by workgroup id.
+template <typename Cfg, bool VEC, bool TICKET>
 __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_t* in, uint32_t* out,
-                                                                   size_t n, uint32_t* ticket,
-                                                                   u64* status) {
+                                                                   size_t n, uint32_t* header,
+                                                                   u64* status, uint32_t spin_limit) {
     constexpr int BLOCK = Cfg::BLOCK, VPT = Cfg::VPT;
     constexpr int WAVES = BLOCK / kWave;
     constexpr int TILE = BLOCK * VPT * 4;
@@ -158,12 +184,14 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
 
-    // Dynamic tile id: tiles are numbered in the order blocks start running
-    // (examples/scan.py:88-99), which is what makes the look-back deadlock-free.
-    if (tid == 0)
-        s_tile = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    const uint32_t tile = s_tile;
+    uint32_t tile = blockIdx.x;
+    if constexpr (TICKET) {
+        // Dynamic tile id: tiles are numbered in the order blocks start running (examples/scan.py:88-99).
+        if (tid == 0)
+            s_tile = __hip_atomic_fetch_add(&header[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        tile = s_tile;
+    }
 
     const size_t tile_base = static_cast<size_t>(tile) * TILE;
     const size_t lane_base = tile_base + static_cast<size_t>(wave) * WAVE_ELEMS + lane * 4;
@@ -216,7 +244,7 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
             if (lane == 0) publish(&status[0], kPrefix, aggregate);
         } else {
             if (lane == 0) publish(&status[tile], kAggregate, aggregate);
-            prefix = look_back(status, tile, lane);
+            prefix = look_back(status, tile, lane, spin_limit, &header[2]);
             if (lane == 0) publish(&status[tile], kPrefix, aggregate + prefix);
         }
         if (lane == 0) s_tile_prefix = prefix;
@@ -257,14 +285,31 @@ inline size_t num_tiles_for(size_t n) {
     return ceil_div(n, tile);
 }
 
+// PRISM_SCAN_ORDER=ticket selects the reference's ticket order (read at every call, so a process can
+// switch); PRISM_SCAN_SPIN_LIMIT overrides the look-back bound (0 makes every wait time out at once:
+// the kernel's way out can then be exercised without a stuck predecessor).
+inline bool ticket_order() {
+    const char* v = getenv("PRISM_SCAN_ORDER");
+    return v != nullptr && strcmp(v, "ticket") == 0;
+}
+inline uint32_t spin_limit() {
+    const char* v = getenv("PRISM_SCAN_SPIN_LIMIT");
+    return v != nullptr ? static_cast<uint32_t>(strtoul(v, nullptr, 10)) : kSpinLimit;
+}
+
 template <typename Cfg>
-int launch_cfg(const uint32_t* in, uint32_t* out, size_t n, uint32_t* ticket, u64* status, size_t tiles,
+int launch_cfg(const uint32_t* in, uint32_t* out, size_t n, uint32_t* header, u64* status, size_t tiles,
                hipStream_t s) {
     const dim3 grid(static_cast<unsigned>(tiles)), block(Cfg::BLOCK);
-    if (aligned16(in) && aligned16(out))
-        scan_lookback_kernel<Cfg, true><<<grid, block, 0, s>>>(in, out, n, ticket, status);
-    else
-        scan_lookback_kernel<Cfg, false><<<grid, block, 0, s>>>(in, out, n, ticket, status);
+    const bool vec = aligned16(in) && aligned16(out);
+    const uint32_t limit = spin_limit();
+    if (ticket_order()) {
+        if (vec) scan_lookback_kernel<Cfg, true, true><<<grid, block, 0, s>>>(in, out, n, header, status, limit);
+        else scan_lookback_kernel<Cfg, false, true><<<grid, block, 0, s>>>(in, out, n, header, status, limit);
+    } else {
+        if (vec) scan_lookback_kernel<Cfg, true, false><<<grid, block, 0, s>>>(in, out, n, header, status, limit);
+        else scan_lookback_kernel<Cfg, false, false><<<grid, block, 0, s>>>(in, out, n, header, status, limit);
+    }
     return check_launch("scan_lookback_kernel");
 }
 

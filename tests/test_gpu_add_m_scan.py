@@ -108,6 +108,56 @@ def test_scan_baseline_sizes(prism, oracle, n):
     assert np.array_equal(host(out), oracle.scan_cpu(x))
 
 
+@pytest.fixture
+def scan_env(monkeypatch):
+    """The library reads PRISM_SCAN_ORDER / PRISM_SCAN_SPIN_LIMIT at every call."""
+    def set_(order=None, spin_limit=None):
+        for key, val in (("PRISM_SCAN_ORDER", order), ("PRISM_SCAN_SPIN_LIMIT", spin_limit)):
+            if val is None:
+                monkeypatch.delenv(key, raising=False)
+            else:
+                monkeypatch.setenv(key, str(val))
+    yield set_
+    set_()
+
+
+@pytest.mark.parametrize("n", [1, 4097, 65536 * 3 + 5, (1 << 24) + 1, 1 << 26, (1 << 28) + 12345])
+def test_scan_ticket_order_matches_dispatch_order(prism, oracle, scan_env, n):
+    """Tiles numbered by the ticket counter (the reference's get_block_idx_from_global_counter,
+    examples/scan.py:88-99) and tiles numbered by workgroup id give the same bits."""
+    x = oracle.gen_scan(n, seed=n % 1000)
+    want = oracle.scan_cpu(x)
+    xd = dev(x)
+    for order in ("ticket", None):
+        scan_env(order=order)
+        out = prism.scan(xd)
+        assert np.array_equal(host(out), want), order
+
+
+def test_scan_look_back_wait_is_bounded(prism, oracle, scan_env):
+    """With the spin limit forced to 0 a look-back that has to wait even once gives up: the kernel
+    must still finish, and a wave that gave up reports its tile + 1 in word 2 of the workspace.
+    With the default limit the same workspace reports nothing and the result is exact."""
+    n = 1 << 26
+    x = oracle.gen_scan(n, seed=3)
+    xd = dev(x)
+    out = torch.empty_like(xd)
+    ws = torch.empty(prism.get_workspace_size(n), dtype=torch.uint8, device=DEV)
+    for order in ("ticket", None):
+        scan_env(order=order, spin_limit=0)
+        prism.scan(xd, out, ws)
+        torch.cuda.synchronize()  # the point of the test: this returns
+        report = int(ws[8:12].view(torch.int32).item())
+        tiles = -(-n // 16384)
+        assert 0 <= report <= tiles
+        if report == 0:  # nobody had to wait: then the result must be right
+            assert np.array_equal(host(out), oracle.scan_cpu(x))
+        scan_env(order=order)
+        prism.scan(xd, out, ws)
+        assert int(ws[8:12].view(torch.int32).item()) == 0
+        assert np.array_equal(host(out), oracle.scan_cpu(x))
+
+
 def test_scan_2pow30_properties(prism):
     """Full BASELINE size (4 GiB in, 4 GiB out): checked on the device through
     size-independent properties - first element, the difference invariant
