@@ -5,10 +5,10 @@
 // (examples/h100_matmul.py:20-297, generated/cutlass_my_h100_match_no_tail.cu):
 //   reference                                   here
 //   wgmma m64n256k16 from swizzled smem     ->  v_mfma_f32_32x32x16_bf16, 4 waves x 128x128, swizzled LDS
-//   TMA bulk copies + mbarrier ring (4 x)   ->  long K: buffer loads into two register sets two K tiles
-//                                               ahead, two LDS stages (gemm_bf16_staged_kernel);
-//                                               short K: direct-to-LDS loads, ring of two stages
-//                                               (gemm_bf16_ring_kernel)
+//   TMA bulk copies + mbarrier ring (4 x)   ->  buffer loads into two register sets two K tiles ahead,
+//                                               two LDS stages (gemm_bf16_staged_kernel); odd or
+//                                               small K tile counts: direct-to-LDS loads, ring of two
+//                                               stages (gemm_bf16_ring_kernel)
 //   1 producer + 2 consumer warpgroups      ->  every wave loads and multiplies
 //   persistent CTAs + 16x8 super-tiles      ->  one workgroup per tile, 16x16 super-blocks with an
 //                                               8x4 patch per XCD (tile_map.h)
@@ -274,11 +274,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_kerne
 // of the group before it; loads use a scalar base and a fixed lane offset (no
 // vector ALU work in the loop).
 //
-// Two shapes are compiled. 64 x 2 stages is the one used (short K): a direct load
-// cannot be issued before its stage is free, so it has less than one tile time to
-// land, and for long K the register-staged kernel below is faster. 32 x 4 stages
-// gives loads three tile times but reads half cache lines (64 B per row and
-// tile) and measured slower than both.
+// 64 x 2 stages is the shape used, for the K tile counts the register-staged kernel
+// below does not take: a direct load cannot be issued before its stage is free, so
+// it has less than one tile time to land, which the staged kernel avoids. 32 x 4
+// stages (also supported by the template) gives loads three tile times but reads
+// half cache lines (64 B per row and tile) and measured slower than both.
 template <int BM, int BN, int BK, int STAGES, int WM, int WN, typename OutT>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_kernel(
     int R, int Cn, int K, const uint16_t* __restrict__ P, const uint16_t* __restrict__ Q,
@@ -465,7 +465,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_
 }
 
 // ------------------------------------------- register-staged pipeline kernel --
-// Whole tiles, K a multiple of 64 and at least 5 K tiles. Two LDS stages of one
+// Whole tiles, K a multiple of 128 (an even number of K tiles, at least 6). Two LDS stages of one
 // 256 x 256 x 64 tile pair each (128 KiB), plus two register sets that each hold
 // a wave's share of one more tile pair (16 x 16 B per lane). Tile t+3 is loaded
 // from global memory into registers while tile t is multiplied, and is written
@@ -616,45 +616,27 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
 #pragma unroll
     for (int j = 0; j < NI; ++j) fb[1][j] = bf16x8{};
 
-    // The launcher guarantees K % 64 == 0 and at least 5 tiles. Tiles alternate between the two
-    // stages (and register sets) such that the last tile always sits in stage 1: an odd tile
-    // count starts in stage 1 and runs one phase up front.
-    const int k_tiles = K / BK;
-    int k_load;  // first k of the tile the next phase loads
-    if (k_tiles & 1) {
+    // The launcher guarantees an even number of K tiles, at least 6: tiles alternate between the
+    // two stages (and register sets), the first in stage 0 and the last in stage 1.
 #pragma unroll
-        for (int m = 0; m < PACKETS; ++m) load_packet(1, 0, m);
+    for (int m = 0; m < PACKETS; ++m) load_packet(0, 0, m);
 #pragma unroll
-        for (int m = 0; m < PACKETS; ++m) load_packet(0, BK, m);
+    for (int m = 0; m < PACKETS; ++m) load_packet(1, BK, m);
 #pragma unroll
-        for (int m = 0; m < PACKETS; ++m) write_packet(1, m);
-        __builtin_amdgcn_sched_barrier(0);  // the set is reloaded only after it has been written out
+    for (int m = 0; m < PACKETS; ++m) write_packet(0, m);
+    __builtin_amdgcn_sched_barrier(0);  // the set is reloaded only after it has been written out
 #pragma unroll
-        for (int m = 0; m < PACKETS; ++m) load_packet(1, 2 * BK, m);
-        lds_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-        phase(s1{}, yes{}, yes{}, 3 * BK);
-        k_load = 4 * BK;
-    } else {
-#pragma unroll
-        for (int m = 0; m < PACKETS; ++m) load_packet(0, 0, m);
-#pragma unroll
-        for (int m = 0; m < PACKETS; ++m) load_packet(1, BK, m);
-#pragma unroll
-        for (int m = 0; m < PACKETS; ++m) write_packet(0, m);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int m = 0; m < PACKETS; ++m) load_packet(0, 2 * BK, m);
-        lds_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-        k_load = 3 * BK;
-    }
-    // An even number of tiles remains, the first of them in stage 0; all but the last four run in
-    // pairs that write and load; the last four wind the pipeline down.
-    for (; k_load + BK < K; k_load += 2 * BK) {
+    for (int m = 0; m < PACKETS; ++m) load_packet(0, 2 * BK, m);
+    lds_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    int k_load = 3 * BK;  // first k of the tile the next phase loads
+    // All but the last four tiles run in pairs of phases that write and load; the last four wind
+    // the pipeline down.
+    do {  // runs at least once: 4 tiles are loaded by now and at least 6 exist
         phase(s0{}, yes{}, yes{}, k_load);
         phase(s1{}, yes{}, yes{}, k_load + BK);
-    }
+        k_load += 2 * BK;
+    } while (k_load + BK < K);
     phase(s0{}, yes{}, yes{}, k_load);
     phase(s1{}, yes{}, no{}, 0);
     phase(s0{}, yes{}, no{}, 0);
@@ -675,11 +657,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
     }
 }
 
-// Kernel choice for whole-tile problems: K tiles of 64; from PRISM_BF16_STAGED_MIN_K on the
-// register-staged pipeline (its two-tile load lead pays once the operands no longer sit in the
-// caches next to the CUs), below it the direct-to-LDS ring (lighter prologue).
+// Kernel choice for whole-tile problems, K tiles of 64: the register-staged pipeline whenever the
+// K tile count is even and at least 6 (measured faster than the ring from 2048^3 up), else the
+// direct-to-LDS ring (any count from 2).
 #ifndef PRISM_BF16_STAGED_MIN_K
-#define PRISM_BF16_STAGED_MIN_K 6144
+#define PRISM_BF16_STAGED_MIN_K 384
 #endif
 #ifndef PRISM_BF16_RING_BK
 #define PRISM_BF16_RING_BK 64
@@ -697,7 +679,7 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
     const dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n), block((BM / WM) * (BN / WN) * kWave);
     const bool whole = (R % BM == 0) && (Cn % BN == 0) && aligned16(P) && aligned16(Q);
     // The staged kernel addresses a 256-row panel with 32-bit offsets.
-    if (whole && K % 64 == 0 && K >= 5 * 64 && K >= PRISM_BF16_STAGED_MIN_K &&
+    if (whole && K % 128 == 0 && K >= 6 * 64 && K >= PRISM_BF16_STAGED_MIN_K &&
         static_cast<long long>(BM > BN ? BM : BN) * K * 2 < (1ll << 31)) {
         gemm_bf16_staged_kernel<BM, BN, WM, WN, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
         return check_launch("gemm_bf16_staged_kernel");

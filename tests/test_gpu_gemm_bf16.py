@@ -46,12 +46,12 @@ def test_fp32_output_vs_fp64_oracle(prism, oracle, shape):
     check_f32(oracle, host(D), A16, B16)
 
 
-@pytest.mark.parametrize("shape", [(256, 256, 128), (256, 512, 192), (512, 256, 256), (256, 256, 320), (512, 512, 1024),
+@pytest.mark.parametrize("shape", [(256, 256, 128), (256, 512, 192), (512, 256, 256), (256, 256, 320), (512, 512, 1024), (256, 256, 384), (256, 256, 448),
                                    (256, 512, 6144), (512, 256, 6208), (256, 256, 6272)])
 def test_whole_tile_paths(prism, oracle, shape):
-    """Problems made of whole 256 x 256 x 64 tiles leave the general kernel: K below 6144 takes the
-    direct-to-LDS ring (2, 3, 4, 5 and 16 K tiles here: even and odd ring counts), K from 6144 on the
-    register-staged pipeline (96, 97 and 98 K tiles). Every element is checked, for both output types."""
+    """Problems made of whole 256 x 256 x 64 tiles leave the general kernel: an even K tile count from
+    6 up takes the register-staged pipeline (16, 96 and 98 K tiles here), the others the direct-to-LDS
+    ring (2, 3, 4, 5 and 97 K tiles). Every element is checked, for both output types."""
     M, N, K = shape
     A16, B16 = oracle.gen_gemm_bf16(M, N, K, seed=K + M)
     D = prism.gemm_bf16(dev16(A16), dev16(B16))
