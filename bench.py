@@ -39,10 +39,10 @@ PEAK = {  # MI355X published peaks
 # counters read for a 1 GiB copy (`--workload calibrate`): FETCH_SIZE x 2.0, WRITE_SIZE x 1.0
 # (summaries under profiles/). None where not measured for that shape.
 TRAFFIC_BYTES = {
-    ("sgemm", 8192, 5): (8105032 + 262144) * 1024,
-    ("scan", 1 << 30): (4198548 + 4217260) * 1024,
-    ("gemm_bf16", 8192): (1573592 + 262144) * 1024,
-    ("add_m", 1 << 24): (65567 + 65606) * 1024,
+    ("sgemm", 8192, 5): (4048474 + 262144) * 1024,
+    ("scan", 1 << 30): (4204765 + 4201577) * 1024,
+    ("gemm_bf16", 8192): (1591115 + 262144) * 1024,
+    ("add_m", 1 << 24): (65567 + 65601) * 1024,
 }
 
 
@@ -58,9 +58,21 @@ def _capi():
     return _lib.load(), torch.cuda.current_stream().cuda_stream
 
 
+SETTLE_MS = 150.0  # untimed run of the workload before the warm-up steps, see time_steps
+
+
 def time_steps(fn, steps: int, warmup: int):
-    """Returns mean milliseconds per step, measured with HIP events on the current stream."""
+    """Returns mean milliseconds per step, measured with HIP events on the current stream.
+
+    Before the W warm-up steps the workload runs untimed for SETTLE_MS: the chip's clock and power
+    management take tens of milliseconds to settle under a new load (the first launches of the bf16
+    GEMM after an idle or memory-bound phase measured up to 15 % off the sustained rate), and three
+    sub-millisecond warm-up steps do not cover that."""
     import torch
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < SETTLE_MS:
+        fn()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -356,7 +368,7 @@ def main() -> int:
                 "gemm_bf16": "D=A@B^T bf16 in, fp32 out, M=N=K=8192",
                 "add_m": "y=x+7 int32 n=2^24"}[head_name]
     line = {
-        "metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": K, "warmup": W,
+        "metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": K, "warmup": W, "settle_ms": SETTLE_MS,
         "ms_per_step": head["ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype, "data": "synthetic",
         "config": {"workload": workload, "device": info["name"], "cu_count": info["cu_count"]},
