@@ -79,6 +79,12 @@ size_t prism_scan_workspace_bytes(size_t n);
  * matter: the call resets it itself, as the reference launcher does
  * (evals/4090_scan/main.cu:81-82). Two calls that share a workspace must be
  * ordered on one stream.
+ * Tiles are numbered by workgroup id; with PRISM_SCAN_ORDER=ticket in the
+ * environment (read at every call) by the reference's ticket counter
+ * (get_block_idx_from_global_counter, examples/scan.py:88-99). A tile's wait
+ * for its predecessors is bounded: should it ever run out, the kernel still
+ * finishes, ((uint32_t*)workspace)[2] holds the tile number + 1 and the output
+ * is not valid; after every normal call that word is 0.
  * Replaces scan_kernel + its device helpers (examples/scan.py:23-227,
  * generated/scan_kernel.cu:1-29).
  */
