@@ -392,6 +392,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_
         }
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(prefetch ? (AHEAD - 1) * LOADS : 0, 0));
         __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");  // the compiler does not know that the loads write LDS: no read moves above the barrier
         __builtin_amdgcn_sched_barrier(0);
     };
     using yes = std::integral_constant<bool, true>;
@@ -420,6 +421,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_
         for (int m = 0; m < LOADS; ++m) issue_load((first + t) % STAGES, t * BK, m);
     __builtin_amdgcn_s_waitcnt(waitcnt_imm((AHEAD - 1) * LOADS, 0));
     __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
 
     int k_next = AHEAD * BK;  // first k of the tile the next phase prefetches

@@ -615,6 +615,221 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
     if (beta == 0.0f) write_back(no{}); else write_back(yes{});
 }
 
+// -------------------------------------------- kernel 5, one wave per tile --
+// Problems too small to give every CU a 256 x 256 tile: the tile is one wave's
+// tile (WT x WT, WT = 64 or 32) and the workgroup is one wave, so there are no
+// barriers at all; a CU runs four or more such workgroups side by side. Same
+// ingredients as the whole-tile kernel above: direct-to-LDS loads with a scalar
+// base, swizzled A rows read 16 B per lane, the k / n permutation that lets a
+// lane read NI consecutive B columns per k and own NI consecutive C columns, and
+// the previous tile's last MFMA group issued first. The K tiles of 16 travel
+// through a ring of STAGES private LDS stages; the loads of tile t + STAGES - 1
+// go into the stage of tile t - 1 once this wave's own reads of it have returned
+// (lgkmcnt), and a tile is read once this wave's loads of it have (vmcnt).
+//
+// B stage layout. WT = 64: [k][64], a k-row is 256 B, four rows per direct load.
+// WT = 32: a k-row is 128 B, and the two half-waves of an operand read (k and
+// k + 4) would hit the same 32 banks; rows k and k + 4 therefore share a 256 B
+// line (k & 3 selects the line, bit 2 of k the half), which the load side gets by
+// permuting which k-row a lane fetches.
+template <int WT, int STAGES>
+__global__ __launch_bounds__(kWave) void sgemm_single_wave_kernel(
+    int M, int N, int K, float alpha, const float* __restrict__ A, const float* __restrict__ B,
+    float beta, float* C, int tiles_m, int tiles_n) {
+    constexpr int BK = 16, KP = 4, SWZ = 2, KS = 2;
+    constexpr int MI = WT / 32, NI = WT / 32;
+    static_assert(WT == 32 || WT == 64, "wave tile");
+    constexpr int A_LOADS = WT / 16;                  // 16 rows of 64 B per load
+    constexpr int B_ROWS_PER_LOAD = 1024 / (WT * 4);  // k-rows per load
+    constexpr int B_LOADS = BK / B_ROWS_PER_LOAD;
+    constexpr int LOADS = A_LOADS + B_LOADS;
+    constexpr int GROUP = 4 * MI * NI;                // MFMAs per group of 8 k values
+    static_assert(LOADS <= GROUP, "the loads of a tile fit among the MFMAs of one group");
+    static_assert((STAGES - 1) * LOADS < 64, "outstanding loads fit the vmcnt counter");
+
+    __shared__ __attribute__((aligned(1024))) float As[STAGES][WT * BK];
+    __shared__ __attribute__((aligned(1024))) float Bs[STAGES][BK * WT];
+
+    int tm, tn;
+    xcd_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+    const int row0 = tm * WT, col0 = tn * WT;
+    const int lane = threadIdx.x;
+    const int l32 = lane & 31, lhi = lane >> 5;
+
+    f32x16 acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    // Load side (lane offsets in bytes, loop-invariant).
+    const int a_chunk = (lane % KP) ^ (((lane / KP) >> SWZ) & (KP - 1));
+    const uint32_t a_lane = (static_cast<uint32_t>(lane / KP) * static_cast<uint32_t>(K) + a_chunk * 4) * 4u;
+    // B: WT = 64: lane l fetches k-row l / 16, columns 4 (l % 16) ..; WT = 32: LDS position l holds
+    // k-row (l / 16) + 4 ((l / 8) & 1), columns 4 (l % 8) .. (see the layout note above).
+    const int b_krow = WT == 64 ? lane / 16 : (lane / 16) + 4 * ((lane / 8) & 1);
+    const int b_col = WT == 64 ? 4 * (lane % 16) : 4 * (lane % 8);
+    const uint32_t b_lane = (static_cast<uint32_t>(b_krow) * static_cast<uint32_t>(N) + b_col) * 4u;
+    const char* a_base = reinterpret_cast<const char*>(A + static_cast<size_t>(row0) * K);
+    const char* b_base = reinterpret_cast<const char*>(B + col0);
+    auto issue_load = [&](int stage, int k0, int m) {
+        if (m < A_LOADS)
+            direct_load16(a_base + (static_cast<size_t>(m) * 16 * K + k0) * 4, a_lane, &As[stage][m * 16 * BK]);
+        else
+            direct_load16(b_base + static_cast<size_t>(k0 + (m - A_LOADS) * B_ROWS_PER_LOAD) * N * 4, b_lane,
+                          &Bs[stage][(m - A_LOADS) * B_ROWS_PER_LOAD * WT]);
+    };
+
+    // Operand side.
+    const int sw = (l32 >> SWZ) & (KP - 1);
+    int a_off[KS];
+#pragma unroll
+    for (int g = 0; g < KS; ++g) a_off[g] = l32 * BK + ((2 * g + lhi) ^ sw) * 4;
+    // B element (k = 8 g + 4 lhi + jj, column NI * l32 + j).
+    auto b_index = [&](int g, int jj) {
+        if constexpr (WT == 64) return (8 * g + 4 * lhi + jj) * WT + NI * l32;
+        else return (4 * g + jj) * 64 + lhi * 32 + l32;  // line (k & 3) + 4 (k >> 3), half = bit 2 of k
+    };
+    typedef float fvec __attribute__((ext_vector_type(NI == 2 ? 2 : 1)));
+    f32x4 fa[2][MI];
+    float fb[2][4][NI];
+    auto read_frags = [&](int stage, int g, int slot) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i) fa[slot][i] = *reinterpret_cast<const f32x4*>(&As[stage][a_off[g] + i * 32 * BK]);
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            if constexpr (NI == 2) {
+                const fvec b = *reinterpret_cast<const fvec*>(&Bs[stage][b_index(g, jj)]);
+                fb[slot][jj][0] = b[0];
+                fb[slot][jj][1] = b[1];
+            } else {
+                fb[slot][jj][0] = Bs[stage][b_index(g, jj)];
+            }
+        }
+    };
+    auto mfma_group = [&](int slot, auto after) {
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[slot][i][jj], fb[slot][jj][j], acc[i][j], 0, 0, 0);
+                    after((jj * MI + i) * NI + j);
+                }
+    };
+    auto nothing = [](int) {};
+
+    // Phase t (tile t sits in stage S): the last group of tile t-1 is multiplied from slot 1 while
+    // group 0 of tile t is read into slot 0 and the loads of tile t+STAGES-1 are issued into the
+    // stage tile t-1 leaves; then group 0 is multiplied while group 1 is read into slot 1.
+    auto phase = [&](auto stage_c, auto prefetch, int k_next) {
+        constexpr int S = decltype(stage_c)::value;
+        // Reads of tile t-1 have all returned (their values are in slot 1 / were used), so its stage
+        // may be overwritten; the explicit wait below keeps that true whatever the compiler schedules.
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(kVmMax, 0));
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(S, 0, 0);
+        mfma_group(1, [&](int m) {
+            if constexpr (prefetch) {
+                if (m < LOADS) {
+                    issue_load((S + STAGES - 1) % STAGES, k_next, m);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        });
+        read_frags(S, 1, 1);
+        mfma_group(0, nothing);
+        __builtin_amdgcn_sched_barrier(0);
+        // Tile t+1 has landed when at most the loads of the younger tiles are outstanding.
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(prefetch ? (STAGES - 2) * LOADS : 0, kLgkmMax));
+        asm volatile("" ::: "memory");  // the compiler does not know that the loads write LDS: no read moves above the wait
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    using yes = std::integral_constant<bool, true>;
+    using no = std::integral_constant<bool, false>;
+
+#pragma unroll
+    for (int i = 0; i < MI; ++i) fa[1][i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) fb[1][jj][j] = 0.0f;
+
+    // The launcher guarantees K % 16 == 0 and at least STAGES tiles. Tile t lives in stage
+    // (first + t) % STAGES with `first` chosen such that the last tile sits in the last stage.
+    const int k_tiles = K / BK;
+    const int ragged = k_tiles % STAGES;
+    const int first = (STAGES - ragged) % STAGES;
+#pragma unroll
+    for (int t = 0; t < STAGES - 1; ++t)
+#pragma unroll
+        for (int m = 0; m < LOADS; ++m) issue_load((first + t) % STAGES, t * BK, m);
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm((STAGES - 2) * LOADS, kLgkmMax));
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+
+    int k_next = (STAGES - 1) * BK;
+    static_assert(STAGES == 4, "the phase sequence below is written out for four stages");
+    using s0 = std::integral_constant<int, 0>;
+    using s1 = std::integral_constant<int, 1>;
+    using s2 = std::integral_constant<int, 2>;
+    using s3 = std::integral_constant<int, 3>;
+    if (ragged == 3) { phase(s1{}, yes{}, k_next); k_next += BK; }
+    if (ragged >= 2) { phase(s2{}, yes{}, k_next); k_next += BK; }
+    if (ragged >= 1) { phase(s3{}, yes{}, k_next); k_next += BK; }
+    for (int ring = k_tiles / STAGES; ring > 1; --ring) {
+        phase(s0{}, yes{}, k_next);
+        phase(s1{}, yes{}, k_next + BK);
+        phase(s2{}, yes{}, k_next + 2 * BK);
+        phase(s3{}, yes{}, k_next + 3 * BK);
+        k_next += 4 * BK;
+    }
+    phase(s0{}, yes{}, k_next);
+    phase(s1{}, no{}, 0);
+    phase(s2{}, no{}, 0);
+    phase(s3{}, no{}, 0);
+    mfma_group(1, nothing);  // last group of the last tile
+
+    // Epilogue: a lane holds columns NI l32 .. NI l32 + NI - 1 of 16 rows per 32-row block.
+    float* c_lane = C + static_cast<size_t>(row0 + 4 * lhi) * N + col0 + NI * l32;
+    auto write_back = [&](auto read_c) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                float* c = c_lane + static_cast<size_t>(i * 32 + 8 * (v / 4) + (v % 4)) * N;
+                float r[NI];
+                if constexpr (read_c) {
+                    float old[NI];
+                    if constexpr (NI == 2) {
+                        const fvec o = *reinterpret_cast<const fvec*>(c);
+                        old[0] = o[0];
+                        old[1] = o[1];
+                    } else {
+                        old[0] = *c;
+                    }
+#pragma unroll
+                    for (int j = 0; j < NI; ++j) r[j] = __builtin_fmaf(alpha, acc[i][j][v], beta * old[j]);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < NI; ++j) r[j] = alpha * acc[i][j][v];
+                }
+                if constexpr (NI == 2) {
+                    fvec o;
+                    o[0] = r[0];
+                    o[1] = r[1];
+                    *reinterpret_cast<fvec*>(c) = o;
+                } else {
+                    *c = r[0];
+                }
+            }
+    };
+    if (beta == 0.0f) write_back(no{}); else write_back(yes{});
+}
+
 // --------------------------------------------------------------- launchers --
 
 template <int BM, int BN, int BK, int TM, int TN, bool VEC>
@@ -648,13 +863,21 @@ int run_wave_tile(int M, int N, int K, float alpha, const float* A, const float*
     return check_launch("sgemm_wave_tile_kernel");
 }
 
+inline int cu_count() {
+    static int cached[64] = {};  // per device; a racing first call writes the same value
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+        cached[dev] = cus;
+    }
+    return cached[dev];
+}
 // Whole-tile kernel when the problem is made of 256 x 256 tiles and there are
-// enough of them to give every CU one; otherwise the general kernel.
+// enough of them for three quarters of the CUs.
 #ifndef PRISM_SGEMM5_DMA
 #define PRISM_SGEMM5_DMA 1
-#endif
-#ifndef PRISM_SGEMM5_DMA_MIN_TILES
-#define PRISM_SGEMM5_DMA_MIN_TILES 256
 #endif
 template <int BM, int BN, int BK, int WM, int WN>
 bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const float* B, float beta,
@@ -662,11 +885,28 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
     if (!PRISM_SGEMM5_DMA) return false;
     if (K <= 0 || M % BM || N % BN || K % BK || !aligned16(A) || !aligned16(B) || !aligned16(C)) return false;
     const int tiles_m = M / BM, tiles_n = N / BN;
-    if (static_cast<long long>(tiles_m) * tiles_n < PRISM_SGEMM5_DMA_MIN_TILES) return false;
+    if (static_cast<long long>(tiles_m) * tiles_n * 4 < 3ll * cu_count()) return false;
     const dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n), block((BM / WM) * (BN / WN) * kWave);
     sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN><<<grid, block, 0, s>>>(M, N, K, alpha, A, B, beta, C,
                                                                           tiles_m, tiles_n);
     *rc = check_launch("sgemm_wave_tile_dma_kernel");
+    return true;
+}
+
+#ifndef PRISM_SGEMM5_SINGLE
+#define PRISM_SGEMM5_SINGLE 1
+#endif
+template <int WT>
+bool try_single_wave(int M, int N, int K, float alpha, const float* A, const float* B, float beta, float* C,
+                     hipStream_t s, int* rc) {
+    constexpr int STAGES = 4;
+    if (!PRISM_SGEMM5_SINGLE) return false;
+    if (M % WT || N % WT || K % 16 || K < 16 * STAGES || !aligned16(A) || !aligned16(B) || !aligned16(C)) return false;
+    if (static_cast<long long>(K) * 64 >= (1ll << 30) || static_cast<long long>(N) * 64 >= (1ll << 30)) return false;
+    const int tiles_m = M / WT, tiles_n = N / WT;
+    sgemm_single_wave_kernel<WT, STAGES><<<dim3(static_cast<unsigned>(tiles_m) * tiles_n), dim3(kWave), 0, s>>>(
+        M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n);
+    *rc = check_launch("sgemm_single_wave_kernel");
     return true;
 }
 
@@ -716,10 +956,20 @@ int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, 
             // run_my_sgemm_5 (evals/4090_sgemm/runner.cu:194-202), with four
             // 64-lane waves in place of four 32-lane warps.
             {
+                // Whole 256 x 256 tiles for at least three quarters of the CUs: the direct-to-LDS kernel,
                 // K tiles of 32 (128 KiB of LDS) when K allows, else of 16.
                 int rc = 0;
                 if (try_wave_tile_dma<256, 256, 32, 128, 128>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
                 if (try_wave_tile_dma<256, 256, 16, 128, 128>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
+                // Small problems (at most one 64 x 64 tile per SIMD): one wave per tile, 32 x 32 tiles when
+                // 64 x 64 ones would leave SIMDs without work. In between, the general kernel's 128 x 128
+                // tiles quantise best.
+                const long long simds = 4ll * cu_count();
+                const long long tiles64 = static_cast<long long>(M / 64) * (N / 64);
+                if (tiles64 <= simds) {
+                    if (tiles64 < simds && try_single_wave<32>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
+                    if (try_single_wave<64>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
+                }
             }
             return run_wave_tile<PRISM_SGEMM5_CFG>(M, N, K, alpha, A, B, beta, C, s);
     }

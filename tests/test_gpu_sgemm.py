@@ -157,7 +157,7 @@ def test_baseline_tail_shapes(prism, oracle, shape):
 @pytest.mark.parametrize("shape", [(4096, 4096, 16), (4096, 4096, 32), (4096, 4096, 48), (4096, 4096, 80),
                                    (2048, 8192, 96), (8192, 2048, 64)])
 def test_wave_tile_whole_tile_path(prism, oracle, shape):
-    """Shapes made of at least 256 whole 256 x 256 tiles take kernel 5's direct-to-LDS path; K covers
+    """Shapes made of whole 256 x 256 tiles, enough for three quarters of the CUs, take kernel 5's direct-to-LDS path; K covers
     one, an even and an odd number of K tiles. Every element is checked, with and without reading C,
     and against the general path (same data at a 4-byte offset, which the whole-tile path rejects)."""
     M, N, K = shape
@@ -175,6 +175,21 @@ def test_wave_tile_whole_tile_path(prism, oracle, shape):
     out = host(buf)
     assert out[0] == 777.0 and np.all(out[1 + M * N:] == 777.0)
     assert np.max(np.abs(out[1:1 + M * N].reshape(M, N) - got)) <= 2 * t
+
+
+@pytest.mark.parametrize("shape", [(512, 512, 64), (1024, 1024, 80), (1024, 1024, 96), (1024, 1024, 112), (1024, 512, 256),
+                                   (2048, 2048, 128), (128, 4096, 256), (64, 64, 2048), (96, 160, 64)])
+def test_wave_tile_one_wave_per_tile_path(prism, oracle, shape):
+    """Problems with at most one 64 x 64 tile per SIMD take kernel 5's one-wave-per-tile path (32 x 32
+    tiles below that, 64 x 64 at exactly that); K covers every residue of the 4-stage ring. Every element is
+    checked, with and without reading C."""
+    M, N, K = shape
+    A, B, Cm = oracle.gen_sgemm(M, N, K, seed=K + N)
+    got = run(prism, 5, -0.75, A, B, 2.0, Cm)
+    assert np.max(np.abs(got - oracle.np_sgemm_f64(-0.75, A, B, 2.0, Cm))) <= tol(oracle, K, A, B, 2.0, Cm)
+    poison = np.full((M, N), np.nan, dtype=np.float32)
+    got0 = run(prism, 5, 1.0, A, B, 0.0, poison)
+    assert np.max(np.abs(got0 - oracle.np_sgemm_f64(1.0, A, B, 0.0))) <= oracle.sgemm_tolerance(K, A, B)
 
 
 def _sampled_check(prism, oracle, M, N, K, alpha, beta, variant, rows=48):
