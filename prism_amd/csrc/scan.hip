@@ -38,10 +38,11 @@
 // numbered in the order blocks start. The ticket is an agent-scope atomic on one
 // address, and its round trip (about 2 us) sits in front of every block's first
 // load: measured 5 % of the run time at 2^30. The default here is therefore
-// tile = workgroup id, which is deadlock-free as long as the dispatcher starts the
-// workgroups of a 1-D grid in id order on every XCD (then the lowest unfinished
-// tile is always running; this is the same assumption CUB's look-back scan makes
-// on NVIDIA hardware). PRISM_SCAN_ORDER=ticket in the environment selects the
+// tile = a fixed function of the workgroup id (chunks of 4 consecutive tiles go to
+// workgroups of one XCD, see the kernel), which is deadlock-free as long as the
+// dispatcher starts the workgroups of a 1-D grid in id order on every XCD (then
+// the lowest unfinished tile is always running; this is the same assumption
+// CUB's look-back scan makes on NVIDIA hardware). PRISM_SCAN_ORDER=ticket in the environment selects the
 // reference's ticket order instead. In both modes the look-back wait is bounded
 // (kSpinLimit polls, several seconds): a wave that runs out stores the tile number
 // plus one into the workspace header (word 2) and carries on with a wrong prefix,
@@ -76,6 +77,9 @@ struct SmallCfg { static constexpr int BLOCK = 1024, VPT = 4; };
 #endif
 #ifndef PRISM_SCAN_BIG_VPT
 #define PRISM_SCAN_BIG_VPT 16
+#endif
+#ifndef PRISM_SCAN_CHUNK
+#define PRISM_SCAN_CHUNK 4  // consecutive tiles per XCD in workgroup-id order; 4-5 measured best, 1 and 32 worst
 #endif
 #ifndef PRISM_SCAN_SLEEP
 #define PRISM_SCAN_SLEEP 1
@@ -185,6 +189,22 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
     const int wave = tid / kWave;
 
     uint32_t tile = blockIdx.x;
+#if PRISM_SCAN_CHUNK > 1
+    {
+        // Consecutive workgroup ids go to the 8 XCDs in turn, and the XCDs drift apart, so in plain id
+        // order half of all tiles start before their predecessor and wait longer for it. Chunks of
+        // PRISM_SCAN_CHUNK consecutive tiles are given to workgroups of one XCD instead (every 8th id),
+        // which start in order; only chunk boundaries cross XCDs. A tile's predecessors then have ids at
+        // most 8 * PRISM_SCAN_CHUNK above its own, far fewer than the workgroups resident at once, so
+        // the lowest unfinished tile is still always running.
+        constexpr uint32_t G = PRISM_SCAN_CHUNK, SPAN = 8 * G;
+        const uint32_t whole = (gridDim.x / SPAN) * SPAN;
+        if (tile < whole) {
+            const uint32_t xcd = tile % 8, j = tile / 8;
+            tile = (j / G) * SPAN + xcd * G + (j % G);
+        }
+    }
+#endif
     if constexpr (TICKET) {
         // Dynamic tile id: tiles are numbered in the order blocks start running (examples/scan.py:88-99).
         if (tid == 0)
