@@ -296,8 +296,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_
     static_assert(BM % ROWS_PER_PASS == 0 && BN % ROWS_PER_PASS == 0, "whole load passes");
     constexpr int P_PER = BM / ROWS_PER_PASS, Q_PER = BN / ROWS_PER_PASS;  // loads per wave per tile
     constexpr int LOADS = P_PER + Q_PER, READS = MI + NI, GROUP = MI * NI;
-    constexpr int GAPS = GROUP - READS;               // MFMAs of a group with nothing behind them yet
-    static_assert(GAPS > 0 && LOADS <= GAPS * KS, "the loads of a tile fit between the MFMAs of a phase");
+    static_assert(READS <= GROUP && LOADS <= GROUP, "reads and loads of a tile fit behind the MFMAs of one group");
     static_assert(((ROWS_PER_PASS >> SWZ) % KP) == 0 && ((32 >> SWZ) % KP) == 0,
                   "the swizzle term must repeat with the load pass and the 32-row MFMA block");
 
@@ -374,19 +373,20 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_
     // any more", while operand slot 1 holds the last k-group of tile t-1. Group g of
     // the phase (g = 0 .. KS-1) issues the MFMAs of the k-group read one group earlier
     // (g = 0: the last one of tile t-1); behind its first READS MFMAs go the reads of
-    // k-group g of tile t, behind the others the direct loads of tile t+AHEAD into the
-    // stage tile t-1 has left. Then: wait until at most the loads of the younger tiles
-    // are in flight, barrier.
+    // k-group g of tile t, and behind the MFMAs of group 0 also the direct loads of tile
+    // t+AHEAD into the stage tile t-1 has left. Then: wait until at most the loads of the
+    // younger tiles are in flight, barrier.
     auto phase = [&](auto stage_c, auto prefetch, int k_next) {
         constexpr int S = decltype(stage_c)::value;
 #pragma unroll
         for (int g = 0; g < KS; ++g) {
             mfma_group((g + 1) & 1, [&](int m) {
-                if (m < READS) {
-                    read_one(S, g, m);
-                } else if constexpr (prefetch) {
-                    const int ld = g * GAPS + (m - READS);
-                    if (ld < LOADS) issue_load((S + AHEAD) % STAGES, k_next, ld);
+                // Reads of k-group g behind the first MFMAs of every group; all loads of the next tile behind
+                // the MFMAs of the first group, one each, so that every load has most of the phase to land
+                // (spreading them over two groups was slower for long K, issuing two per MFMA too).
+                if (m < READS) read_one(S, g, m);
+                if constexpr (prefetch) {
+                    if (g == 0 && m < LOADS) issue_load((S + AHEAD) % STAGES, k_next, m);
                 }
             });
         }
