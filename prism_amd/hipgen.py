@@ -1,0 +1,377 @@
+"""A HIP emitter for the thread-level subset of the Prism DSL (gfx950).
+
+The reference's product is a source-to-source compiler: kernels are Python
+functions decorated with ``@prism("global")`` whose parameters and locals carry a
+perspective (``@ grid[1]``, ``@ thread[1]``), and ``generate(name)`` prints CUDA
+(prism/codegen.py:321-384,758-849; surface syntax in examples/add_m_thread.py:10-19,
+expected text in README.md:133-140). This module is the first slice of a HIP
+back-end for that front end: it accepts the same surface syntax for kernels whose
+work is expressed per thread --
+
+    @requires(grid[1], thread[1])
+    @prism("global")
+    def add_m_thread(x: ptr(const(int)) @ grid[1], y: ptr(int) @ grid[1], m: int @ grid[1]):
+        tid: int @ thread[1] = id()
+        with partition(x, p=thread[1], offset=tid) as x_thread:
+            with partition(y, p=thread[1], offset=tid) as y_thread:
+                with group(thread[1]):
+                    y_thread[0] = x_thread[0] + m
+
+-- and prints a HIP kernel, optionally with an element count and a bounds guard
+(the reference kernel has neither and must be launched with exactly n threads),
+plus an ``extern "C"`` launcher that picks the grid. ``build()`` compiles the text
+with hipcc for gfx950 and returns a ctypes handle; nothing is interpreted on the
+CPU and there is no fallback.
+
+Supported: scalar and pointer parameters of int / float / unsigned, ``id()`` at
+thread perspective, nested ``partition(..., p=thread[1], offset=e)`` views,
+``group(thread[1])`` bodies with assignments, augmented assignments, arithmetic,
+comparisons and ``if``. Anything else raises ``HipgenError`` naming the construct:
+block- and warp-level perspectives, shared memory and the automatic barrier
+placement are not part of this slice.
+
+The decorators only register the function's source; annotations are evaluated by
+Python at definition time, so the perspective objects below implement ``[]`` and
+``@`` and nothing else.
+"""
+from __future__ import annotations
+
+import ast
+import ctypes
+import inspect
+import subprocess
+import tempfile
+import textwrap
+from dataclasses import dataclass, field
+from pathlib import Path
+from typing import Callable, Dict, List, Optional
+
+__all__ = ["prism", "requires", "grid", "block", "warp", "thread", "ptr", "const", "group", "partition",
+           "generate", "generate_launcher", "build", "HipgenError"]
+
+
+class HipgenError(Exception):
+    """The kernel uses something outside the supported subset."""
+
+
+# ------------------------------------------------------------ surface syntax --
+
+@dataclass(frozen=True)
+class Perspective:
+    level: str
+    size: int = 1
+
+    def __getitem__(self, size: int) -> "Perspective":
+        return Perspective(self.level, int(size))
+
+    def __rmatmul__(self, other):  # `int @ thread[1]`
+        return Located(other, self)
+
+
+@dataclass(frozen=True)
+class Located:
+    ctype: object
+    where: Perspective
+
+
+@dataclass(frozen=True)
+class CType:
+    text: str
+
+    def __matmul__(self, where: Perspective):  # `ptr(int) @ grid[1]`
+        return Located(self, where)
+
+
+grid, block, warp, thread = (Perspective(n) for n in ("grid", "block", "warp", "thread"))
+
+_SCALARS = {"int": "int", "float": "float", "unsigned": "unsigned int", "uint": "unsigned int", "bool": "bool"}
+
+
+def _ctype_text(t) -> str:
+    if isinstance(t, CType):
+        return t.text
+    name = getattr(t, "__name__", str(t))
+    if name in _SCALARS:
+        return _SCALARS[name]
+    raise HipgenError(f"unsupported element type {t!r}")
+
+
+def const(t) -> CType:
+    return CType("const " + _ctype_text(t))
+
+
+def ptr(t) -> CType:
+    return CType(_ctype_text(t) + "*")
+
+
+def group(_where):  # only ever appears inside kernel bodies, which are parsed, not run
+    raise HipgenError("group() is part of a kernel body; kernels are compiled with generate(), not called")
+
+
+partition = group
+
+_REGISTRY: Dict[str, "Kernel"] = {}
+
+
+@dataclass
+class Kernel:
+    name: str
+    kind: str
+    source: str
+    requires: tuple = ()
+    fn: Optional[Callable] = field(default=None, repr=False)
+
+
+def prism(kind: str):
+    if kind not in ("global", "device"):
+        raise HipgenError(f'@prism("{kind}"): expected "global" or "device"')
+
+    def deco(fn):
+        _REGISTRY[fn.__name__] = Kernel(fn.__name__, kind, textwrap.dedent(inspect.getsource(fn)), fn=fn)
+        return fn
+    return deco
+
+
+def requires(*perspectives: Perspective):
+    def deco(fn):
+        k = _REGISTRY.get(fn.__name__)
+        if k is None:
+            raise HipgenError("@requires must be applied above @prism")
+        k.requires = tuple(perspectives)
+        return fn
+    return deco
+
+
+# ------------------------------------------------------------------ emitter --
+
+_BINOPS = {ast.Add: "+", ast.Sub: "-", ast.Mult: "*", ast.Div: "/", ast.Mod: "%", ast.LShift: "<<",
+           ast.RShift: ">>", ast.BitAnd: "&", ast.BitOr: "|", ast.BitXor: "^", ast.FloorDiv: "/"}
+_CMPOPS = {ast.Lt: "<", ast.LtE: "<=", ast.Gt: ">", ast.GtE: ">=", ast.Eq: "==", ast.NotEq: "!="}
+_UNOPS = {ast.USub: "-", ast.Invert: "~", ast.Not: "!"}
+
+
+def _perspective_of(node: ast.AST) -> Perspective:
+    """`thread[1]` / `grid[1]` as written in the source."""
+    if isinstance(node, ast.Subscript) and isinstance(node.value, ast.Name) and node.value.id in (
+            "grid", "block", "warp", "thread"):
+        size = node.slice
+        if isinstance(size, ast.Constant) and isinstance(size.value, int):
+            return Perspective(node.value.id, size.value)
+    raise HipgenError(f"line {getattr(node, 'lineno', '?')}: expected a perspective such as thread[1]")
+
+
+def _type_of(node: ast.AST) -> str:
+    """`ptr(const(int))`, `int` ... as written in the source."""
+    if isinstance(node, ast.Name):
+        if node.id in _SCALARS:
+            return _SCALARS[node.id]
+        raise HipgenError(f"line {node.lineno}: unsupported type {node.id}")
+    if isinstance(node, ast.Call) and isinstance(node.func, ast.Name) and len(node.args) == 1:
+        inner = _type_of(node.args[0])
+        if node.func.id == "ptr":
+            return inner + "*"
+        if node.func.id == "const":
+            return "const " + inner
+    raise HipgenError(f"line {getattr(node, 'lineno', '?')}: unsupported type expression")
+
+
+def _split_annotation(node: ast.AST):
+    """`T @ where` -> (C type text, Perspective)."""
+    if isinstance(node, ast.BinOp) and isinstance(node.op, ast.MatMult):
+        return _type_of(node.left), _perspective_of(node.right)
+    raise HipgenError(f"line {getattr(node, 'lineno', '?')}: annotation must be `type @ perspective`")
+
+
+class _Emitter:
+    def __init__(self, kernel: Kernel, bounded: bool):
+        self.k = kernel
+        self.bounded = bounded
+        self.lines: List[str] = []
+        self.views: Dict[str, tuple] = {}   # view name -> (base expression text, offset expression text)
+        self.params: List[tuple] = []       # (ctype, name)
+        self.thread_ids: List[str] = []
+
+    # expressions
+    def expr(self, n: ast.AST) -> str:
+        if isinstance(n, ast.Constant):
+            if isinstance(n.value, bool):
+                return "true" if n.value else "false"
+            if isinstance(n.value, int):
+                return str(n.value)
+            if isinstance(n.value, float):
+                return repr(n.value) + "f"
+            raise HipgenError(f"line {n.lineno}: unsupported constant {n.value!r}")
+        if isinstance(n, ast.Name):
+            if n.id in self.views:
+                raise HipgenError(f"line {n.lineno}: view {n.id} must be indexed")
+            return n.id
+        if isinstance(n, ast.BinOp) and type(n.op) in _BINOPS:
+            return f"{self.operand(n.left)} {_BINOPS[type(n.op)]} {self.operand(n.right)}"
+        if isinstance(n, ast.UnaryOp) and type(n.op) in _UNOPS:
+            return f"{_UNOPS[type(n.op)]}{self.operand(n.operand)}"
+        if isinstance(n, ast.Compare) and len(n.ops) == 1 and type(n.ops[0]) in _CMPOPS:
+            return f"{self.operand(n.left)} {_CMPOPS[type(n.ops[0])]} {self.operand(n.comparators[0])}"
+        if isinstance(n, ast.Subscript):
+            return self.element(n)
+        raise HipgenError(f"line {getattr(n, 'lineno', '?')}: unsupported expression {ast.dump(n)[:60]}")
+
+    def operand(self, n: ast.AST) -> str:
+        text = self.expr(n)
+        return f"({text})" if isinstance(n, (ast.BinOp, ast.Compare)) else text
+
+    def element(self, n: ast.Subscript) -> str:
+        if not isinstance(n.value, ast.Name):
+            raise HipgenError(f"line {n.lineno}: only named arrays and views can be indexed")
+        idx = self.expr(n.slice)
+        name = n.value.id
+        if name in self.views:
+            base, off = self.views[name]
+            return f"{base}[{off}]" if idx == "0" else f"{base}[{off} + {idx}]"
+        return f"{name}[{idx}]"
+
+    # statements
+    def stmt(self, n: ast.stmt, depth: int) -> None:
+        pad = "    " * depth
+        if isinstance(n, ast.AnnAssign) and isinstance(n.target, ast.Name):
+            ctype, where = _split_annotation(n.annotation)
+            if isinstance(n.value, ast.Call) and isinstance(n.value.func, ast.Name) and n.value.func.id == "id":
+                if where != Perspective("thread", 1):
+                    raise HipgenError(f"line {n.lineno}: id() is supported at thread[1] only (got {where.level}[{where.size}])")
+                self.lines.append(f"{pad}{ctype} {n.target.id} = blockIdx.x * blockDim.x + threadIdx.x;")
+                self.thread_ids.append(n.target.id)
+                if self.bounded and len(self.thread_ids) == 1:
+                    self.lines.append(f"{pad}if ({n.target.id} >= prism_n) return;")
+                return
+            if n.value is None:
+                self.lines.append(f"{pad}{ctype} {n.target.id};")
+            else:
+                self.lines.append(f"{pad}{ctype} {n.target.id} = {self.expr(n.value)};")
+            return
+        if isinstance(n, ast.With) and len(n.items) == 1:
+            call = n.items[0].context_expr
+            if isinstance(call, ast.Call) and isinstance(call.func, ast.Name):
+                if call.func.id == "partition":
+                    self.partition(call, n.items[0].optional_vars, n)
+                    for s in n.body:
+                        self.stmt(s, depth)
+                    return
+                if call.func.id == "group":
+                    where = _perspective_of(call.args[0]) if call.args else None
+                    if where != Perspective("thread", 1):
+                        raise HipgenError(f"line {n.lineno}: group() is supported at thread[1] only")
+                    for s in n.body:
+                        self.stmt(s, depth)
+                    return
+            raise HipgenError(f"line {n.lineno}: unsupported with-statement")
+        if isinstance(n, ast.Assign) and len(n.targets) == 1:
+            self.lines.append(f"{pad}{self.expr(n.targets[0])} = {self.expr(n.value)};")
+            return
+        if isinstance(n, ast.AugAssign) and type(n.op) in _BINOPS:
+            self.lines.append(f"{pad}{self.expr(n.target)} {_BINOPS[type(n.op)]}= {self.expr(n.value)};")
+            return
+        if isinstance(n, ast.If):
+            self.lines.append(f"{pad}if ({self.expr(n.test)}) {{")
+            for s in n.body:
+                self.stmt(s, depth + 1)
+            if n.orelse:
+                self.lines.append(f"{pad}}} else {{")
+                for s in n.orelse:
+                    self.stmt(s, depth + 1)
+            self.lines.append(f"{pad}}}")
+            return
+        if isinstance(n, ast.Expr) and isinstance(n.value, ast.Constant) and isinstance(n.value.value, str):
+            return  # docstring
+        if isinstance(n, ast.Pass):
+            return
+        raise HipgenError(f"line {n.lineno}: unsupported statement {type(n).__name__}")
+
+    def partition(self, call: ast.Call, target, node) -> None:
+        if not isinstance(target, ast.Name) or not call.args or not isinstance(call.args[0], ast.Name):
+            raise HipgenError(f"line {node.lineno}: expected `with partition(array, p=..., offset=...) as view`")
+        kw = {k.arg: k.value for k in call.keywords}
+        if set(kw) != {"p", "offset"}:
+            raise HipgenError(f"line {node.lineno}: partition() takes p= and offset=")
+        where = _perspective_of(kw["p"])
+        if where != Perspective("thread", 1):
+            raise HipgenError(f"line {node.lineno}: partition() is supported at p=thread[1] only (got {where.level}[{where.size}])")
+        off = self.operand(kw["offset"])
+        parent = call.args[0].id
+        if parent in self.views:  # a view of a view: offsets add up
+            base, parent_off = self.views[parent]
+            self.views[target.id] = (base, f"{parent_off} + {off}")
+        else:
+            self.views[target.id] = (parent, off)
+
+    def emit(self) -> str:
+        tree = ast.parse(self.k.source)
+        fn = tree.body[0]
+        if not isinstance(fn, ast.FunctionDef):
+            raise HipgenError("expected a function definition")
+        for a in fn.args.args:
+            if a.annotation is None:
+                raise HipgenError(f"parameter {a.arg} needs a `type @ perspective` annotation")
+            ctype, where = _split_annotation(a.annotation)
+            if where.level != "grid":
+                raise HipgenError(f"parameter {a.arg}: kernel parameters live at grid perspective")
+            self.params.append((ctype, a.arg))
+        for s in fn.body:
+            self.stmt(s, 1)
+        if self.bounded and not self.thread_ids:
+            raise HipgenError("a bounded kernel needs a thread id (`tid: int @ thread[1] = id()`)")
+        params = ", ".join(f"{t} {n}" for t, n in self.params)
+        if self.bounded:
+            params += (", " if params else "") + "size_t prism_n"
+        qualifier = "__global__" if self.k.kind == "global" else "__device__"
+        head = f"{qualifier} void {self.k.name}({params}) {{"
+        return "\n".join([head, *self.lines, "}"]) + "\n"
+
+
+def _kernel(name: str) -> Kernel:
+    try:
+        return _REGISTRY[name]
+    except KeyError:
+        raise HipgenError(f"no kernel named {name!r} has been defined with @prism") from None
+
+
+def generate(name: str, bounded: bool = False) -> str:
+    """HIP text of kernel `name`. bounded=False prints what the reference prints for the same
+    source (one thread per element, no guard); bounded=True appends a `size_t prism_n` parameter and
+    returns early for thread ids beyond it, so that any grid covering n is legal."""
+    return _Emitter(_kernel(name), bounded).emit()
+
+
+def generate_launcher(name: str, block_size: int = 256) -> str:
+    """Bounded kernel plus `extern "C" int <name>_launch(<params>, size_t n, void* stream)`:
+    ceil(n / block_size) workgroups of block_size threads (a multiple of the 64-lane wavefront)."""
+    if block_size % 64 or not 64 <= block_size <= 1024:
+        raise HipgenError("block_size must be a multiple of 64 between 64 and 1024")
+    em = _Emitter(_kernel(name), True)
+    text = em.emit()
+    params = ", ".join(f"{t} {n}" for t, n in em.params)
+    args = ", ".join(n for _, n in em.params)
+    sep = ", " if params else ""
+    return (
+        "#include <hip/hip_runtime.h>\n#include <cstddef>\n\n" + text + "\n"
+        f'extern "C" int {name}_launch({params}{sep}size_t n, void* stream) {{\n'
+        "    if (n == 0) return 0;\n"
+        f"    const size_t blocks = (n + {block_size - 1}) / {block_size};\n"
+        "    if (blocks > 0x7fffffffull) return 1;\n"
+        f"    {name}<<<dim3(static_cast<unsigned>(blocks)), dim3({block_size}), 0, static_cast<hipStream_t>(stream)>>>"
+        f"({args}{sep}n);\n"
+        "    return static_cast<int>(hipGetLastError());\n"
+        "}\n")
+
+
+def build(name: str, out_dir: Optional[str] = None, block_size: int = 256) -> ctypes.CDLL:
+    """Compile `generate_launcher(name)` for gfx950 and load it. The handle's `<name>_launch` takes the
+    kernel's parameters (device pointers as integers), the element count and a stream handle."""
+    from .build import HIPCC_FLAGS, hipcc_path
+    d = Path(out_dir) if out_dir else Path(tempfile.mkdtemp(prefix="prism_hipgen_"))
+    d.mkdir(parents=True, exist_ok=True)
+    src, lib = d / f"{name}.hip", d / f"lib{name}.so"
+    src.write_text(generate_launcher(name, block_size))
+    proc = subprocess.run([hipcc_path(), *HIPCC_FLAGS, "-shared", "-o", str(lib), str(src)],
+                          capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise HipgenError(f"hipcc failed for {name}:\n{proc.stderr}")
+    return ctypes.CDLL(str(lib))
