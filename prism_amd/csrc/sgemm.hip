@@ -16,7 +16,10 @@
 // block -> wave -> sub-tile decomposition, but a 64-lane wave computes its
 // sub-tiles with v_mfma_f32_32x32x2_f32 instead of per-thread outer products;
 // its summation order inside the matrix unit is not specified, so it is
-// checked against an fp64 product within a tolerance.
+// checked against an fp64 product within a tolerance. It comes in three forms,
+// chosen by the launcher from the tile count: the general 128 x 128 block kernel
+// (any shape), a 256 x 256 direct-to-LDS kernel for problems made of whole tiles
+// that fill the chip, and a one-wave-per-tile kernel for small problems.
 //
 // Unlike the reference kernels (no guards in kernels 1, 3, 4, 5), every kernel
 // here accepts any M, N, K: full tiles take a guard-free path, edge tiles a
@@ -25,7 +28,7 @@
 #include "direct_load.h"
 #include "tile_map.h"
 
-// Kernel 5 tile shape: BM, BN, BK, WM, WN.
+// General kernel 5 tile shape: BM, BN, BK, WM, WN.
 #ifndef PRISM_SGEMM5_CFG
 #define PRISM_SGEMM5_CFG 128, 128, 16, 64, 64
 #endif
