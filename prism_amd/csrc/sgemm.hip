@@ -391,8 +391,14 @@ __attribute__((amdgpu_waves_per_eu(PRISM_SGEMM5_WAVES_PER_EU))) void sgemm_wave_
 // per SIMD nothing else hides a stall, so the K loop is written as phases that
 // run from barrier to barrier with the matrix pipe fed throughout.
 //
-// LDS layout of one K tile (two stages, separate arrays so that the compiler's
-// wait-count logic knows loads into one stage do not feed reads of the other):
+// A vector ALU instruction between two MFMAs delays the second one by about 12
+// clocks (measured with one wave per SIMD; LDS reads cost about 5, scalar
+// instructions and barriers nothing), so the loop contains none: the direct
+// loads take a scalar base and a fixed lane offset (direct_load.h), one load
+// behind every PRISM_SGEMM5_LOAD_GAP-th MFMA of the first group, pinned there
+// with scheduling barriers (bunched loads hold the wave at the memory pipeline).
+//
+// LDS layout of one K tile (two stages):
 //   As[m][k]  as in global memory, BK floats per row. A wave-wide direct load
 //             writes 1 KiB of contiguous LDS (lane l lands at base + 16 l), so
 //             rows cannot be padded; the 16 B chunk c of row m is kept in slot
