@@ -644,7 +644,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
 template <int WT, int STAGES>
 __global__ __launch_bounds__(kWave) void sgemm_single_wave_kernel(
     int M, int N, int K, float alpha, const float* __restrict__ A, const float* __restrict__ B,
-    float beta, float* C, int tiles_m, int tiles_n) {
+    float beta, float* C, int tiles_m, int tiles_n, int first_big) {
     constexpr int BK = 16, KP = 4, SWZ = 2, KS = 2;
     constexpr int MI = WT / 32, NI = WT / 32;
     static_assert(WT == 32 || WT == 64, "wave tile");
@@ -659,9 +659,24 @@ __global__ __launch_bounds__(kWave) void sgemm_single_wave_kernel(
     __shared__ __attribute__((aligned(1024))) float As[STAGES][WT * BK];
     __shared__ __attribute__((aligned(1024))) float Bs[STAGES][BK * WT];
 
-    int tm, tn;
-    xcd_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
-    const int row0 = tm * WT, col0 = tn * WT;
+    // first_big < 0: the grid covers the whole tiles_m x tiles_n grid of WT x WT tiles. Otherwise this
+    // launch finishes what a launch of the 256 x 256 kernel left over: tiles_m x tiles_n is that kernel's
+    // grid, first_big the first tile number it did not take, and every leftover tile is cut into
+    // (256 / WT)^2 wave tiles.
+    int row0, col0;
+    if (first_big < 0) {
+        int tm, tn;
+        xcd_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+        row0 = tm * WT;
+        col0 = tn * WT;
+    } else {
+        constexpr int SUB = 256 / WT;
+        int tm, tn;
+        xcd_tile_coords(first_big + blockIdx.x / (SUB * SUB), tiles_m, tiles_n, tm, tn);
+        const int sub = blockIdx.x % (SUB * SUB);
+        row0 = tm * 256 + (sub / SUB) * WT;
+        col0 = tn * 256 + (sub % SUB) * WT;
+    }
     const int lane = threadIdx.x;
     const int l32 = lane & 31, lhi = lane >> 5;
 
@@ -888,6 +903,9 @@ inline int cu_count() {
 #ifndef PRISM_SGEMM5_DMA
 #define PRISM_SGEMM5_DMA 1
 #endif
+#ifndef PRISM_SGEMM5_LEFTOVER
+#define PRISM_SGEMM5_LEFTOVER 1
+#endif
 template <int BM, int BN, int BK, int WM, int WN>
 bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const float* B, float beta,
                        float* C, hipStream_t s, int* rc) {
@@ -895,10 +913,36 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
     if (K <= 0 || M % BM || N % BN || K % BK || !aligned16(A) || !aligned16(B) || !aligned16(C)) return false;
     const int tiles_m = M / BM, tiles_n = N / BN;
     if (static_cast<long long>(tiles_m) * tiles_n * 4 < 3ll * cu_count()) return false;
-    const dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n), block((BM / WM) * (BN / WN) * kWave);
-    sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN><<<grid, block, 0, s>>>(M, N, K, alpha, A, B, beta, C,
-                                                                          tiles_m, tiles_n);
+    const dim3 block((BM / WM) * (BN / WN) * kWave);
+    // Tile counts that do not fill whole rounds of CUs: the 256 x 256 kernel takes the whole rounds, and
+    // the tiles of the last, partial round are cut into 64 x 64 wave tiles that spread over all SIMDs
+    // (6144^3: 2 rounds + 64 tiles instead of 3 rounds). Not worth it when the last round is nearly full.
+    static_assert(BM == 256 && BN == 256, "the leftover launch cuts 256 x 256 tiles");
+    const int tiles = tiles_m * tiles_n, cus = cu_count();
+    int main_tiles = tiles, leftover_wt = 0;
+    if (PRISM_SGEMM5_LEFTOVER && tiles > cus && tiles % cus != 0 && K >= 64) {
+        // Cost of the last round in units of one full round of 256 x 256 tiles: a wave tile of 64 (32)
+        // is 1/4 (1/16) of a SIMD's share of a big tile and runs at about 0.87 (0.72) of its rate.
+        const int left = tiles % cus, simds = 4 * cus;
+        const double cost64 = ceil_div(left * 16, simds) * 0.25 / 0.87;
+        const double cost32 = ceil_div(left * 64, simds) * 0.0625 / 0.72;
+        if (cost64 < 0.9 || cost32 < 0.9) {
+            main_tiles = tiles - left;
+            leftover_wt = cost64 <= cost32 ? 64 : 32;
+        }
+    }
+    sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
+        M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n);
     *rc = check_launch("sgemm_wave_tile_dma_kernel");
+    if (*rc == 0 && leftover_wt == 64) {
+        sgemm_single_wave_kernel<64, 4><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 16), dim3(kWave), 0, s>>>(
+            M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, main_tiles);
+        *rc = check_launch("sgemm_single_wave_kernel");
+    } else if (*rc == 0 && leftover_wt == 32) {
+        sgemm_single_wave_kernel<32, 4><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 64), dim3(kWave), 0, s>>>(
+            M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, main_tiles);
+        *rc = check_launch("sgemm_single_wave_kernel");
+    }
     return true;
 }
 
@@ -914,7 +958,7 @@ bool try_single_wave(int M, int N, int K, float alpha, const float* A, const flo
     if (static_cast<long long>(K) * 64 >= (1ll << 30) || static_cast<long long>(N) * 64 >= (1ll << 30)) return false;
     const int tiles_m = M / WT, tiles_n = N / WT;
     sgemm_single_wave_kernel<WT, STAGES><<<dim3(static_cast<unsigned>(tiles_m) * tiles_n), dim3(kWave), 0, s>>>(
-        M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n);
+        M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
     *rc = check_launch("sgemm_single_wave_kernel");
     return true;
 }
