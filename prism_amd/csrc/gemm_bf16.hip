@@ -489,7 +489,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_
 // LDS rows are 128 B (8 chunks of 16 B); chunk c of row r sits in slot
 // c ^ ((r >> 1) & 7): a wave writes 1 KiB of contiguous LDS per instruction, and
 // the 16 rows a quarter-wave reads with ds_read_b128 cover all 64 banks.
-template <int BM, int BN, int WM, int WN, typename OutT>
+template <int BM, int BN, int WM, int WN, bool EDGE, typename OutT>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_staged_kernel(
     int R, int Cn, int K, const uint16_t* __restrict__ P, const uint16_t* __restrict__ Q,
     OutT* __restrict__ OUT, int tiles_m, int tiles_n) {
@@ -535,17 +535,42 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
     // Buffer loads: the address is (descriptor base) + (vector offset) + (scalar offset), so a load
     // needs no vector ALU work; offsets stay inside this workgroup's 256-row panel (the launcher
     // checks that a panel is below 2 GiB).
+    //
+    // EDGE: the matrices need not be whole tiles. A buffer load returns zero for every dword at or
+    // beyond the descriptor's extent (vector + scalar offset are both checked), so with the extent set
+    // to the end of the matrix the rows below it read as zeros. Columns k >= K of a row are the
+    // next row's data and in range, so there the lane offset is replaced by one beyond any extent
+    // (kBeyond); K is a multiple of 8, so a 16 B chunk is either whole or absent. The K loop runs
+    // over an even number (at least 6) of K tiles, the ones past K reading zeros.
+    constexpr uint32_t kBeyond = 0x80000000u;
+    auto extent = [&](int first_row, int rows) -> int {  // bytes from a wave's first row to the end of the matrix
+        if (!EDGE) return 0x7fffffff;
+        const long long left = static_cast<long long>(rows - first_row) * K * 2;
+        return static_cast<int>(left < 0 ? 0 : (left > 0x7fffffff ? 0x7fffffff : left));
+    };
+    const int p_first = row0 + wave * ROWS_PER_LOAD, q_first = col0 + wave * ROWS_PER_LOAD;
+    // A wave whose first row is already outside the matrix gets extent 0 on a valid base address.
     const auto p_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t*>(P + static_cast<size_t>(row0 + wave * ROWS_PER_LOAD) * K), 0, 0x7fffffff, 0x00020000);
+        const_cast<uint16_t*>(P + (EDGE && p_first >= R ? size_t{0} : static_cast<size_t>(p_first) * K)), 0,
+        extent(p_first, R), 0x00020000);
     const auto q_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t*>(Q + static_cast<size_t>(col0 + wave * ROWS_PER_LOAD) * K), 0, 0x7fffffff, 0x00020000);
+        const_cast<uint16_t*>(Q + (EDGE && q_first >= Cn ? size_t{0} : static_cast<size_t>(q_first) * K)), 0,
+        extent(q_first, Cn), 0x00020000);
     const int pass_bytes = ROWS_PER_PASS * K * 2;
+    const int k_full = K - K % BK;                                   // tiles that start below it are whole
+    const int k_end = EDGE ? ((K + 2 * BK - 1) / (2 * BK) < 3 ? 6 * BK : (K + 2 * BK - 1) / (2 * BK) * 2 * BK) : K;
+    const uint32_t tail_off = (EDGE && k_full + ld_chunk * 8 < K) ? lane_off : kBeyond;  // lane offset in the partial tile
     u32x4 staged[2][PACKETS];
-    auto load_packet = [&](int set, int k0, int m) {
+    // Lane offset for the loads of the tile that starts at k0: two selects on scalar conditions.
+    auto offset_for = [&](int k0) -> uint32_t {
+        if (!EDGE) return lane_off;
+        return k0 < k_full ? lane_off : (k0 < K ? tail_off : kBeyond);
+    };
+    auto load_packet = [&](int set, int k0, int m, uint32_t off) {
         if (m < P_PER)
-            staged[set][m] = __builtin_amdgcn_raw_buffer_load_b128(p_rsrc, lane_off, m * pass_bytes + k0 * 2, 0);
+            staged[set][m] = __builtin_amdgcn_raw_buffer_load_b128(p_rsrc, off, m * pass_bytes + k0 * 2, 0);
         else
-            staged[set][m] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, lane_off, (m - P_PER) * pass_bytes + k0 * 2, 0);
+            staged[set][m] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, off, (m - P_PER) * pass_bytes + k0 * 2, 0);
     };
     // LDS side: the same packet lands at (its first row) * 128 B + 16 B * lane.
     auto write_packet = [&](int set, int m) {
@@ -589,6 +614,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
     // with tile t+3, which starts at k_load (`load`).
     auto phase = [&](auto stage_c, auto write, auto load, int k_load) {
         constexpr int S = decltype(stage_c)::value;
+        const uint32_t off = offset_for(k_load);
 #pragma unroll
         for (int g = 0; g < KS; ++g) {
             mfma_group((g + 1) & 1, [&](int m) {
@@ -599,7 +625,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
                     if ((m - READS) % 2 == 0) {
                         if constexpr (write) write_packet(S ^ 1, packet);
                     } else {
-                        if constexpr (load) load_packet(S ^ 1, k_load, packet);
+                        if constexpr (load) load_packet(S ^ 1, k_load, packet, off);
                     }
                 }
             });
@@ -621,14 +647,14 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
     // The launcher guarantees an even number of K tiles, at least 6: tiles alternate between the
     // two stages (and register sets), the first in stage 0 and the last in stage 1.
 #pragma unroll
-    for (int m = 0; m < PACKETS; ++m) load_packet(0, 0, m);
+    for (int m = 0; m < PACKETS; ++m) load_packet(0, 0, m, offset_for(0));
 #pragma unroll
-    for (int m = 0; m < PACKETS; ++m) load_packet(1, BK, m);
+    for (int m = 0; m < PACKETS; ++m) load_packet(1, BK, m, offset_for(BK));
 #pragma unroll
     for (int m = 0; m < PACKETS; ++m) write_packet(0, m);
     __builtin_amdgcn_sched_barrier(0);  // the set is reloaded only after it has been written out
 #pragma unroll
-    for (int m = 0; m < PACKETS; ++m) load_packet(0, 2 * BK, m);
+    for (int m = 0; m < PACKETS; ++m) load_packet(0, 2 * BK, m, offset_for(2 * BK));
     lds_barrier();
     __builtin_amdgcn_sched_barrier(0);
     int k_load = 3 * BK;  // first k of the tile the next phase loads
@@ -638,7 +664,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
         phase(s0{}, yes{}, yes{}, k_load);
         phase(s1{}, yes{}, yes{}, k_load + BK);
         k_load += 2 * BK;
-    } while (k_load + BK < K);
+    } while (k_load + BK < k_end);
     phase(s0{}, yes{}, yes{}, k_load);
     phase(s1{}, yes{}, no{}, 0);
     phase(s0{}, yes{}, no{}, 0);
@@ -653,7 +679,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int row = row0 + wave_m * WM + i * 32 + 8 * (v / 4) + 4 * lhi + (v % 4);
-                store_out(&OUT[static_cast<size_t>(row) * Cn + col], acc[i][j][v]);
+                if (!EDGE || (row < R && col < Cn))
+                    store_out(&OUT[static_cast<size_t>(row) * Cn + col], acc[i][j][v]);
             }
         }
     }
@@ -664,6 +691,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
 // direct-to-LDS ring (any count from 2).
 #ifndef PRISM_BF16_STAGED_MIN_K
 #define PRISM_BF16_STAGED_MIN_K 384
+#endif
+#ifndef PRISM_BF16_STAGED_EDGES
+#define PRISM_BF16_STAGED_EDGES 1
 #endif
 #ifndef PRISM_BF16_RING_BK
 #define PRISM_BF16_RING_BK 64
@@ -679,11 +709,12 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
     constexpr size_t lds_bytes = 2ull * (BM + BN) * LD * sizeof(uint16_t);
     const int tiles_m = ceil_div(R, BM), tiles_n = ceil_div(Cn, BN);
     const dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n), block((BM / WM) * (BN / WN) * kWave);
-    const bool whole = (R % BM == 0) && (Cn % BN == 0) && aligned16(P) && aligned16(Q);
-    // The staged kernel addresses a 256-row panel with 32-bit offsets.
-    if (whole && K % 128 == 0 && K >= 6 * 64 && K >= PRISM_BF16_STAGED_MIN_K &&
-        static_cast<long long>(BM > BN ? BM : BN) * K * 2 < (1ll << 31)) {
-        gemm_bf16_staged_kernel<BM, BN, WM, WN, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
+    const bool aligned = aligned16(P) && aligned16(Q);
+    const bool whole = (R % BM == 0) && (Cn % BN == 0) && aligned;
+    // The staged kernel addresses a 256-row panel (plus up to six K tiles of padding) with 32-bit offsets.
+    const bool panel_ok = static_cast<long long>(BM > BN ? BM : BN) * (static_cast<long long>(K) + 6 * 64) * 2 < (1ll << 31);
+    if (whole && K % 128 == 0 && K >= 6 * 64 && K >= PRISM_BF16_STAGED_MIN_K && panel_ok) {
+        gemm_bf16_staged_kernel<BM, BN, WM, WN, false, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
         return check_launch("gemm_bf16_staged_kernel");
     }
     if (whole && K % PRISM_BF16_RING_BK == 0 && K >= PRISM_BF16_RING_BK * PRISM_BF16_RING_STAGES &&
@@ -691,6 +722,11 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
         gemm_bf16_ring_kernel<BM, BN, PRISM_BF16_RING_BK, PRISM_BF16_RING_STAGES, WM, WN, OutT>
             <<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
         return check_launch("gemm_bf16_ring_kernel");
+    }
+    // Ragged M, N or K with 16 B-aligned rows: the staged kernel with zero-filled edges.
+    if (PRISM_BF16_STAGED_EDGES && aligned && K % 8 == 0 && K > 0 && panel_ok) {
+        gemm_bf16_staged_kernel<BM, BN, WM, WN, true, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
+        return check_launch("gemm_bf16_staged_kernel (edges)");
     }
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<BM, BN, BK, WM, WN, true, OutT>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));

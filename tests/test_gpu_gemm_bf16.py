@@ -66,6 +66,38 @@ def test_whole_tile_paths(prism, oracle, shape):
     assert np.all(np.abs(c - ref) <= 2.0**-8 * np.abs(ref) + REL * np.abs(ref).max())
 
 
+def nan_fenced(a16: np.ndarray) -> torch.Tensor:
+    """The matrix as a view into a device buffer whose other elements are bf16 NaN patterns (16 B-aligned start)."""
+    buf = torch.full((a16.size + 2048,), 0x7FC0, dtype=torch.int16, device=DEV)
+    buf[1024:1024 + a16.size] = torch.from_numpy(np.ascontiguousarray(a16).view(np.int16).ravel()).to(DEV)
+    return buf[1024:1024 + a16.size].view(torch.bfloat16).view(a16.shape)
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 8), (257, 255, 8), (300, 520, 392), (255, 513, 456), (512, 512, 72), (1000, 1000, 1000),
+                                   (256, 256, 64), (8, 8, 1032), (264, 24, 6152), (777, 300, 128)])
+def test_ragged_shapes_with_aligned_rows(prism, oracle, shape):
+    """M, N not multiples of 256 or K not a multiple of 64, K a multiple of 8: the register-staged
+    kernel with zero-filled edges (rows beyond the matrix and K tiles beyond K read as zeros through the
+    buffer descriptor's range check). The matrices sit between NaNs, so one element read from outside a
+    matrix, or from the next row in the partial K tile, would poison the output; stores are fenced too."""
+    M, N, K = shape
+    A16, B16 = oracle.gen_gemm_bf16(M, N, K, seed=3 * M + N + K)
+    buf = torch.full((M * N + 512,), 777.0, dtype=torch.float32, device=DEV)
+    D = buf[256:256 + M * N].view(M, N)
+    prism.gemm_bf16(nan_fenced(A16), nan_fenced(B16), D)
+    out = host(buf)
+    assert np.all(out[:256] == 777.0) and np.all(out[256 + M * N:] == 777.0)
+    check_f32(oracle, out[256:256 + M * N].reshape(M, N), A16, B16)
+    Cc = torch.full((N * M + 64,), -7.0, dtype=torch.bfloat16, device=DEV)
+    prism.runmyh100(M, N, K, nan_fenced(A16), nan_fenced(B16), Cc[32:32 + N * M])
+    got = host(Cc.view(torch.int16)).view(np.uint16)
+    guard = np.float32(-7.0).view(np.uint32) >> 16
+    assert np.all(got[:32] == guard) and np.all(got[32 + N * M:] == guard)
+    ref = oracle.gemm_bf16_f64(A16, B16)
+    c = oracle.bf16_to_f32(got[32:32 + N * M]).reshape(N, M).T
+    assert np.all(np.abs(c - ref) <= 2.0**-8 * np.abs(ref) + REL * np.abs(ref).max())
+
+
 def test_fixture(prism, golden, oracle):
     A16, B16 = golden["bf16_A"], golden["bf16_B"]
     D = host(prism.gemm_bf16(dev16(A16), dev16(B16)))
