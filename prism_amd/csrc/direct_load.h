@@ -32,6 +32,37 @@ __device__ __forceinline__ void direct_load16(const char* base, uint32_t lane_of
 #pragma clang diagnostic pop
 }
 
+// The same load through a buffer descriptor: lane l reads descriptor base + lane_offset(l) +
+// scalar_offset. Every dword whose offset (lane + scalar part) is at or beyond the descriptor's
+// extent arrives as zero, which is how ragged matrix edges are filled: the extent ends with the
+// matrix, and a lane whose element lies outside for another reason (past the row end) passes
+// kBeyondExtent as its offset.
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+constexpr uint32_t kBeyondExtent = 0x80000000u;  // extents here stay below 2 GiB
+// Raw buffer descriptor (stride 0) for `extent_bytes` bytes at `base`: base address, extent, and the
+// data-format word of an untyped 32-bit buffer. Wave-uniform by construction (forced into scalar registers).
+__device__ __forceinline__ i32x4 buffer_descriptor(const void* base, uint32_t extent_bytes) {
+    const uint64_t a = reinterpret_cast<uint64_t>(base);
+    i32x4 d;
+    d[0] = __builtin_amdgcn_readfirstlane(static_cast<int>(a & 0xffffffffu));
+    d[1] = __builtin_amdgcn_readfirstlane(static_cast<int>((a >> 32) & 0xffffu));
+    d[2] = __builtin_amdgcn_readfirstlane(static_cast<int>(extent_bytes));
+    d[3] = 0x00020000;
+    return d;
+}
+__device__ __forceinline__ void direct_load16_buffer(i32x4 rsrc, uint32_t lane_offset, uint32_t scalar_offset,
+                                                     const void* lds_dst) {
+    const uint32_t lds_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+        (const __attribute__((address_space(3))) void*)lds_dst));
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+    asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
+                 :
+                 : "v"(lane_offset), "s"(rsrc), "s"(scalar_offset), "s"(lds_addr)
+                 : "memory", "m0");
+#pragma clang diagnostic pop
+}
+
 // s_waitcnt immediate (gfx9 encoding): at most `vm` vector-memory and `lgkm`
 // LDS/scalar operations outstanding; vmcnt[3:0] in bits 3:0 and vmcnt[5:4] in bits
 // 15:14, lgkmcnt in bits 11:8, the export counter left at its maximum.

@@ -421,7 +421,7 @@ __attribute__((amdgpu_waves_per_eu(PRISM_SGEMM5_WAVES_PER_EU))) void sgemm_wave_
 #ifndef PRISM_SGEMM5_LOAD_GAP
 #define PRISM_SGEMM5_LOAD_GAP 4
 #endif
-template <int BM, int BN, int BK, int WM, int WN>
+template <int BM, int BN, int BK, int WM, int WN, bool EDGE>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile_dma_kernel(
     int M, int N, int K, float alpha, const float* __restrict__ A, const float* __restrict__ B,
     float beta, float* C, int tiles_m, int tiles_n) {
@@ -480,14 +480,40 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
     const size_t a_pass = static_cast<size_t>(ROWS_PER_PASS) * K * 4;
     const size_t b_pass = static_cast<size_t>(WAVES) * N * 4;
 
+    // EDGE: M, N, K need not be whole tiles (N and K multiples of 4, so that rows stay 16 B aligned and
+    // a 16 B chunk is whole or absent). The loads go through buffer descriptors whose extents end with
+    // the matrices: A rows >= M and B rows >= K lie beyond them and arrive as zeros. What lies past
+    // the end of a row is the next row, so there the lane offset is replaced by one beyond any extent:
+    // B columns >= N (fixed per lane) and, in the partial K tile, A chunks with k >= K.
+    const int a_first = row0 + wave * ROWS_PER_LOAD;              // this wave's first A row
+    const long long a_left = static_cast<long long>(M - a_first) * K * 4;
+    const long long b_left = (static_cast<long long>(K - wave) * N - col0) * 4;
+    const i32x4 a_rsrc = buffer_descriptor(EDGE && a_left > 0 ? static_cast<const void*>(a_wave) : static_cast<const void*>(A),
+                                           EDGE && a_left > 0 ? static_cast<uint32_t>(a_left) : 0u);
+    const i32x4 b_rsrc = buffer_descriptor(EDGE && b_left > 0 ? static_cast<const void*>(b_wave) : static_cast<const void*>(B),
+                                           EDGE && b_left > 0 ? static_cast<uint32_t>(b_left) : 0u);
+    const int k_full = K - K % BK;
+    const uint32_t a_tail = (k_full + ld_chunk * 4 < K) ? a_lane : kBeyondExtent;
+    const uint32_t b_edge = (col0 + 4 * lane < N) ? b_lane : kBeyondExtent;
     // Load number m (0 .. A_PER + B_PER - 1) of the tile that starts at k0.
     auto issue_load = [&](float* as, float* bs, int k0, int m) {
-        if (m < A_PER)
-            direct_load16(a_wave + static_cast<size_t>(k0) * 4 + m * a_pass, a_lane,
-                          as + (m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK);
-        else
-            direct_load16(b_wave + static_cast<size_t>(k0) * N * 4 + (m - A_PER) * b_pass, b_lane,
-                          bs + ((m - A_PER) * WAVES + wave) * BN);
+        if constexpr (EDGE) {
+            if (m < A_PER)
+                direct_load16_buffer(a_rsrc, k0 < k_full ? a_lane : a_tail,
+                                     static_cast<uint32_t>(k0) * 4u + m * static_cast<uint32_t>(a_pass),
+                                     as + (m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK);
+            else
+                direct_load16_buffer(b_rsrc, b_edge,
+                                     (static_cast<uint32_t>(k0) + (m - A_PER) * WAVES) * static_cast<uint32_t>(N) * 4u,
+                                     bs + ((m - A_PER) * WAVES + wave) * BN);
+        } else {
+            if (m < A_PER)
+                direct_load16(a_wave + static_cast<size_t>(k0) * 4 + m * a_pass, a_lane,
+                              as + (m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK);
+            else
+                direct_load16(b_wave + static_cast<size_t>(k0) * N * 4 + (m - A_PER) * b_pass, b_lane,
+                              bs + ((m - A_PER) * WAVES + wave) * BN);
+        }
     };
     constexpr int LOADS = A_PER + B_PER;
 
@@ -578,9 +604,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
         __syncthreads();
     };
 
-    // The launcher guarantees K % BK == 0 and K > 0. Tiles alternate between the
+    // The launcher guarantees K > 0 and, unless EDGE, K % BK == 0. Tiles alternate between the
     // two stages such that the last tile always sits in stage 1.
-    const int k_tiles = K / BK;
+    const int k_tiles = (K + BK - 1) / BK;
     int t = 0;
     if (k_tiles & 1) {
         load_tile0(As1, Bs1);
@@ -600,13 +626,16 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
     mfma_all(1, nothing);  // last group of the last tile
 
     // Epilogue: a lane holds columns 4 l32 .. 4 l32 + 3 of 16 rows per 32-row block.
-    float* c_lane = C + static_cast<size_t>(row0 + wave_m * WM + 4 * lhi) * N + col0 + wave_n * WN + 4 * l32;
+    const int c_row = row0 + wave_m * WM + 4 * lhi, c_col = col0 + wave_n * WN + 4 * l32;
+    float* c_lane = C + static_cast<size_t>(c_row) * N + c_col;
     auto write_back = [&](auto read_c) {
 #pragma unroll
         for (int i = 0; i < MI; ++i) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                f32x4* c = reinterpret_cast<f32x4*>(c_lane + static_cast<size_t>(i * 32 + 8 * (v / 4) + (v % 4)) * N);
+                const int r_in = i * 32 + 8 * (v / 4) + (v % 4);
+                if (EDGE && (c_row + r_in >= M || c_col >= N)) continue;
+                f32x4* c = reinterpret_cast<f32x4*>(c_lane + static_cast<size_t>(r_in) * N);
                 f32x4 r;
                 if constexpr (read_c) {
                     const f32x4 old = *c;
@@ -906,14 +935,32 @@ inline int cu_count() {
 #ifndef PRISM_SGEMM5_LEFTOVER
 #define PRISM_SGEMM5_LEFTOVER 1
 #endif
-template <int BM, int BN, int BK, int WM, int WN>
+#ifndef PRISM_SGEMM5_EDGES
+#define PRISM_SGEMM5_EDGES 1
+#endif
+template <int BM, int BN, int BK, int WM, int WN, bool ALLOW_EDGES>
 bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const float* B, float beta,
                        float* C, hipStream_t s, int* rc) {
     if (!PRISM_SGEMM5_DMA) return false;
-    if (K <= 0 || M % BM || N % BN || K % BK || !aligned16(A) || !aligned16(B) || !aligned16(C)) return false;
-    const int tiles_m = M / BM, tiles_n = N / BN;
+    if (K <= 0 || !aligned16(A) || !aligned16(B) || !aligned16(C)) return false;
+    const bool whole = M % BM == 0 && N % BN == 0 && K % BK == 0;
+    // Ragged edges: rows must stay 16 B aligned, and the kernel's buffer offsets are 32 bits wide
+    // (a 256-row panel of A plus one K tile; all of B plus one K tile).
+    if (!whole && (!PRISM_SGEMM5_EDGES || !ALLOW_EDGES || N % 4 || K % 4 ||
+                   (static_cast<long long>(BM) + 64) * K * 4 >= (1ll << 31) ||
+                   (static_cast<long long>(K) + 64) * N * 4 >= (1ll << 31)))
+        return false;
+    const int tiles_m = ceil_div(M, BM), tiles_n = ceil_div(N, BN);
     if (static_cast<long long>(tiles_m) * tiles_n * 4 < 3ll * cu_count()) return false;
     const dim3 block((BM / WM) * (BN / WN) * kWave);
+    if constexpr (ALLOW_EDGES) {
+        if (!whole) {
+            sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, true><<<dim3(static_cast<unsigned>(tiles_m) * tiles_n), block, 0, s>>>(
+                M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n);
+            *rc = check_launch("sgemm_wave_tile_dma_kernel (edges)");
+            return true;
+        }
+    }
     // Tile counts that do not fill whole rounds of CUs: the 256 x 256 kernel takes the whole rounds, and
     // the tiles of the last, partial round are cut into 64 x 64 wave tiles that spread over all SIMDs
     // (6144^3: 2 rounds + 64 tiles instead of 3 rounds). Not worth it when the last round is nearly full.
@@ -931,7 +978,7 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
             leftover_wt = cost64 <= cost32 ? 64 : 32;
         }
     }
-    sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
+    sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, false><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
         M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n);
     *rc = check_launch("sgemm_wave_tile_dma_kernel");
     if (*rc == 0 && leftover_wt == 64) {
@@ -1012,8 +1059,9 @@ int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, 
                 // Whole 256 x 256 tiles for at least three quarters of the CUs: the direct-to-LDS kernel,
                 // K tiles of 32 (128 KiB of LDS) when K allows, else of 16.
                 int rc = 0;
-                if (try_wave_tile_dma<256, 256, 32, 128, 128>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
-                if (try_wave_tile_dma<256, 256, 16, 128, 128>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
+                // Ragged M, N, K (N and K multiples of 4) take the K-tile-of-32 kernel with zero-filled edges.
+                if (try_wave_tile_dma<256, 256, 32, 128, 128, true>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
+                if (try_wave_tile_dma<256, 256, 16, 128, 128, false>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
                 // Small problems (at most one 64 x 64 tile per SIMD): one wave per tile, 32 x 32 tiles when
                 // 64 x 64 ones would leave SIMDs without work. In between, the general kernel's 128 x 128
                 // tiles quantise best.

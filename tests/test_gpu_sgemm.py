@@ -203,6 +203,34 @@ def test_wave_tile_leftover_round(prism, oracle, shape):
     assert np.max(np.abs(got - oracle.np_sgemm_f64(1.25, A, B, 0.5, Cm))) <= tol(oracle, K, A, B, 0.5, Cm)
 
 
+def nan_fenced(a: np.ndarray) -> torch.Tensor:
+    """The matrix as a view into a device buffer whose other elements are NaN (16 B-aligned start)."""
+    buf = torch.full((a.size + 2048,), float("nan"), dtype=torch.float32, device=DEV)
+    buf[1024:1024 + a.size] = torch.from_numpy(np.ascontiguousarray(a).ravel()).to(DEV)
+    return buf[1024:1024 + a.size].view(a.shape)
+
+
+@pytest.mark.parametrize("shape", [(3581, 3580, 100), (3584, 3588, 64), (3585, 3584, 36), (3500, 3600, 4), (3841, 3332, 232)])
+def test_wave_tile_ragged_edges(prism, oracle, shape):
+    """M, N, K that are not whole 256 x 256 x 32 tiles (N and K multiples of 4, enough tiles for the CUs):
+    the whole-tile kernel with zero-filled edges (rows beyond a matrix arrive as zeros through the buffer
+    descriptor's range check, columns beyond N and k beyond K through an out-of-range lane offset).
+    A and B sit between NaNs, so one element read from outside a matrix, or from the next row, would
+    poison the output; C is fenced against stores outside it. Every element is checked, with and
+    without reading C."""
+    M, N, K = shape
+    A, B, Cm = oracle.gen_sgemm(M, N, K, seed=M + 3 * K)
+    for beta in (0.5, 0.0):
+        buf = torch.full((M * N + 512,), 777.0, dtype=torch.float32, device=DEV)
+        c = buf[256:256 + M * N].view(M, N)
+        c.copy_(dev(Cm))
+        prism.sgemm(M, N, K, 1.25, nan_fenced(A), nan_fenced(B), beta, c, variant=5)
+        out = host(buf)
+        assert np.all(out[:256] == 777.0) and np.all(out[256 + M * N:] == 777.0)
+        got = out[256:256 + M * N].reshape(M, N)
+        assert np.max(np.abs(got - oracle.np_sgemm_f64(1.25, A, B, beta, Cm))) <= tol(oracle, K, A, B, beta, Cm)
+
+
 def _sampled_check(prism, oracle, M, N, K, alpha, beta, variant, rows=48):
     """Full-size run, checked on `rows` random rows against an fp64 product."""
     g = torch.Generator(device=DEV)
