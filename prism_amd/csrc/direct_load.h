@@ -54,6 +54,8 @@ __device__ __forceinline__ void direct_load16_buffer(i32x4 rsrc, uint32_t lane_o
                                                      const void* lds_dst) {
     const uint32_t lds_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
         (const __attribute__((address_space(3))) void*)lds_dst));
+    // Wave-uniform by contract; said explicitly because the operand must be a scalar register.
+    scalar_offset = __builtin_amdgcn_readfirstlane(scalar_offset);
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
     asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"

@@ -291,6 +291,17 @@ __attribute__((amdgpu_waves_per_eu(PRISM_SGEMM5_WAVES_PER_EU))) void sgemm_wave_
 
     f32x4 a_stage[A_PER], b_stage[B_PER];
 
+    // EDGE (any M, N, K; rows only 4 B aligned): 16 B buffer loads. The descriptor of A covers this
+    // tile's row panel up to the end of the matrix and that of B is rebuilt per K tile from its first
+    // row, so every dword at or beyond the end of a matrix (A rows >= M, B rows >= K) arrives as zero
+    // from the range check and vector offsets stay small. What lies past the end of a row is the next
+    // row: those elements (k >= K in A, columns >= N in B) are replaced by zeros after the load.
+    auto clamp_extent = [](long long bytes) -> int {
+        return static_cast<int>(bytes < 0 ? 0 : (bytes > 0x7fffffff ? 0x7fffffff : bytes));
+    };
+    const long long a_left = static_cast<long long>(M - row0) * K * 4;
+    const auto a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(A + (a_left > 0 ? static_cast<size_t>(row0) * K : size_t{0})), 0, clamp_extent(a_left), 0x00020000);
     auto load_global = [&](int k0) {
 #pragma unroll
         for (int u = 0; u < A_PER; ++u) {
@@ -300,11 +311,18 @@ __attribute__((amdgpu_waves_per_eu(PRISM_SGEMM5_WAVES_PER_EU))) void sgemm_wave_
             if constexpr (!EDGE) {
                 a_stage[u] = *reinterpret_cast<const f32x4*>(&A[static_cast<size_t>(row) * K + k]);
             } else {
-                const float* src = &A[static_cast<size_t>(row) * K + k];
+                a_stage[u] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                    a_rsrc, (static_cast<uint32_t>(r) * static_cast<uint32_t>(K) + kc * 4) * 4u, k0 * 4, 0));
+                if (k0 + BK > K) {
 #pragma unroll
-                for (int c = 0; c < 4; ++c) a_stage[u][c] = (row < M && k + c < K) ? src[c] : 0.0f;
+                    for (int c = 0; c < 4; ++c) a_stage[u][c] = (k + c < K) ? a_stage[u][c] : 0.0f;
+                }
             }
         }
+        const long long b_left = (static_cast<long long>(K - k0) * N - col0) * 4;
+        const auto b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float*>(B + (EDGE && b_left > 0 ? static_cast<size_t>(k0) * N + col0 : size_t{0})), 0,
+            clamp_extent(b_left), 0x00020000);
 #pragma unroll
         for (int u = 0; u < B_PER; ++u) {
             const int p = tid + u * THREADS;
@@ -313,9 +331,10 @@ __attribute__((amdgpu_waves_per_eu(PRISM_SGEMM5_WAVES_PER_EU))) void sgemm_wave_
             if constexpr (!EDGE) {
                 b_stage[u] = *reinterpret_cast<const f32x4*>(&B[static_cast<size_t>(k) * N + col]);
             } else {
-                const float* src = &B[static_cast<size_t>(k) * N + col];
+                b_stage[u] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                    b_rsrc, (static_cast<uint32_t>(r) * static_cast<uint32_t>(N) + nc * 4) * 4u, 0, 0));
 #pragma unroll
-                for (int c = 0; c < 4; ++c) b_stage[u][c] = (k < K && col + c < N) ? src[c] : 0.0f;
+                for (int c = 0; c < 4; ++c) b_stage[u][c] = (col + c < N) ? b_stage[u][c] : 0.0f;
             }
         }
     };
@@ -670,7 +689,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
 // k + 4) would hit the same 32 banks; rows k and k + 4 therefore share a 256 B
 // line (k & 3 selects the line, bit 2 of k the half), which the load side gets by
 // permuting which k-row a lane fetches.
-template <int WT, int STAGES>
+//
+// EDGE: M, N, K need not be whole tiles (N and K multiples of 4); edges are zero-filled as in the
+// whole-tile kernel above (buffer descriptors that end with the matrices, an out-of-range lane
+// offset past a row's end), and the K loop runs over at least STAGES tiles, those beyond K all zeros.
+template <int WT, int STAGES, bool EDGE>
 __global__ __launch_bounds__(kWave) void sgemm_single_wave_kernel(
     int M, int N, int K, float alpha, const float* __restrict__ A, const float* __restrict__ B,
     float beta, float* C, int tiles_m, int tiles_n, int first_big) {
@@ -727,12 +750,28 @@ __global__ __launch_bounds__(kWave) void sgemm_single_wave_kernel(
     const uint32_t b_lane = (static_cast<uint32_t>(b_krow) * static_cast<uint32_t>(N) + b_col) * 4u;
     const char* a_base = reinterpret_cast<const char*>(A + static_cast<size_t>(row0) * K);
     const char* b_base = reinterpret_cast<const char*>(B + col0);
+    const i32x4 a_rsrc = buffer_descriptor(a_base, EDGE ? static_cast<uint32_t>(static_cast<long long>(M - row0) * K * 4) : 0u);
+    const i32x4 b_rsrc = buffer_descriptor(b_base, EDGE ? static_cast<uint32_t>((static_cast<long long>(K) * N - col0) * 4) : 0u);
+    const int k_full = K - K % BK;
+    const uint32_t a_tail = (k_full + a_chunk * 4 < K) ? a_lane : kBeyondExtent;
+    const uint32_t b_edge = (col0 + b_col < N) ? b_lane : kBeyondExtent;
     auto issue_load = [&](int stage, int k0, int m) {
-        if (m < A_LOADS)
-            direct_load16(a_base + (static_cast<size_t>(m) * 16 * K + k0) * 4, a_lane, &As[stage][m * 16 * BK]);
-        else
-            direct_load16(b_base + static_cast<size_t>(k0 + (m - A_LOADS) * B_ROWS_PER_LOAD) * N * 4, b_lane,
-                          &Bs[stage][(m - A_LOADS) * B_ROWS_PER_LOAD * WT]);
+        if constexpr (EDGE) {
+            if (m < A_LOADS)
+                direct_load16_buffer(a_rsrc, k0 < k_full ? a_lane : (k0 < K ? a_tail : kBeyondExtent),
+                                     (static_cast<uint32_t>(m) * 16u * static_cast<uint32_t>(K) + k0) * 4u,
+                                     &As[stage][m * 16 * BK]);
+            else
+                direct_load16_buffer(b_rsrc, b_edge,
+                                     static_cast<uint32_t>(k0 + (m - A_LOADS) * B_ROWS_PER_LOAD) * static_cast<uint32_t>(N) * 4u,
+                                     &Bs[stage][(m - A_LOADS) * B_ROWS_PER_LOAD * WT]);
+        } else {
+            if (m < A_LOADS)
+                direct_load16(a_base + (static_cast<size_t>(m) * 16 * K + k0) * 4, a_lane, &As[stage][m * 16 * BK]);
+            else
+                direct_load16(b_base + static_cast<size_t>(k0 + (m - A_LOADS) * B_ROWS_PER_LOAD) * N * 4, b_lane,
+                              &Bs[stage][(m - A_LOADS) * B_ROWS_PER_LOAD * WT]);
+        }
     };
 
     // Operand side.
@@ -811,9 +850,9 @@ __global__ __launch_bounds__(kWave) void sgemm_single_wave_kernel(
 #pragma unroll
         for (int j = 0; j < NI; ++j) fb[1][jj][j] = 0.0f;
 
-    // The launcher guarantees K % 16 == 0 and at least STAGES tiles. Tile t lives in stage
+    // Unless EDGE, the launcher guarantees K % 16 == 0 and at least STAGES tiles. Tile t lives in stage
     // (first + t) % STAGES with `first` chosen such that the last tile sits in the last stage.
-    const int k_tiles = K / BK;
+    const int k_tiles = EDGE ? ((K + BK - 1) / BK < STAGES ? STAGES : (K + BK - 1) / BK) : K / BK;
     const int ragged = k_tiles % STAGES;
     const int first = (STAGES - ragged) % STAGES;
 #pragma unroll
@@ -853,7 +892,9 @@ __global__ __launch_bounds__(kWave) void sgemm_single_wave_kernel(
         for (int i = 0; i < MI; ++i)
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                float* c = c_lane + static_cast<size_t>(i * 32 + 8 * (v / 4) + (v % 4)) * N;
+                const int r_in = i * 32 + 8 * (v / 4) + (v % 4);
+                if (EDGE && (row0 + 4 * lhi + r_in >= M || col0 + NI * l32 >= N)) continue;
+                float* c = c_lane + static_cast<size_t>(r_in) * N;
                 float r[NI];
                 if constexpr (read_c) {
                     float old[NI];
@@ -910,6 +951,10 @@ int run_wave_tile(int M, int N, int K, float alpha, const float* A, const float*
     if (fast)
         sgemm_wave_tile_kernel<BM, BN, BK, WM, WN, false><<<grid, block, 0, s>>>(
             M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n);
+    else if (static_cast<long long>(BM) * K * 4 >= (1ll << 31) || static_cast<long long>(BK) * N * 4 >= (1ll << 31))
+        // The edge path addresses a row panel of A and a K tile of B with 32-bit byte offsets.
+        return fail(1, "prism_sgemm: kernel 5 with ragged or unaligned operands needs K < %lld and N < %lld",
+                    (1ll << 29) / BM, (1ll << 29) / BK);
     else
         sgemm_wave_tile_kernel<BM, BN, BK, WM, WN, true><<<grid, block, 0, s>>>(
             M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n);
@@ -938,6 +983,12 @@ inline int cu_count() {
 #ifndef PRISM_SGEMM5_EDGES
 #define PRISM_SGEMM5_EDGES 1
 #endif
+#ifndef PRISM_SGEMM5_DMA_MIN_QUARTERS
+#define PRISM_SGEMM5_DMA_MIN_QUARTERS 3
+#endif
+#ifndef PRISM_SGEMM5_SINGLE_ROUNDS
+#define PRISM_SGEMM5_SINGLE_ROUNDS 1
+#endif
 template <int BM, int BN, int BK, int WM, int WN, bool ALLOW_EDGES>
 bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const float* B, float beta,
                        float* C, hipStream_t s, int* rc) {
@@ -951,7 +1002,7 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
                    (static_cast<long long>(K) + 64) * N * 4 >= (1ll << 31)))
         return false;
     const int tiles_m = ceil_div(M, BM), tiles_n = ceil_div(N, BN);
-    if (static_cast<long long>(tiles_m) * tiles_n * 4 < 3ll * cu_count()) return false;
+    if (static_cast<long long>(tiles_m) * tiles_n * 4 < static_cast<long long>(PRISM_SGEMM5_DMA_MIN_QUARTERS) * cu_count()) return false;
     const dim3 block((BM / WM) * (BN / WN) * kWave);
     if constexpr (ALLOW_EDGES) {
         if (!whole) {
@@ -982,11 +1033,11 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
         M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n);
     *rc = check_launch("sgemm_wave_tile_dma_kernel");
     if (*rc == 0 && leftover_wt == 64) {
-        sgemm_single_wave_kernel<64, 4><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 16), dim3(kWave), 0, s>>>(
+        sgemm_single_wave_kernel<64, 4, false><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 16), dim3(kWave), 0, s>>>(
             M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, main_tiles);
         *rc = check_launch("sgemm_single_wave_kernel");
     } else if (*rc == 0 && leftover_wt == 32) {
-        sgemm_single_wave_kernel<32, 4><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 64), dim3(kWave), 0, s>>>(
+        sgemm_single_wave_kernel<32, 4, false><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 64), dim3(kWave), 0, s>>>(
             M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, main_tiles);
         *rc = check_launch("sgemm_single_wave_kernel");
     }
@@ -1001,12 +1052,22 @@ bool try_single_wave(int M, int N, int K, float alpha, const float* A, const flo
                      hipStream_t s, int* rc) {
     constexpr int STAGES = 4;
     if (!PRISM_SGEMM5_SINGLE) return false;
-    if (M % WT || N % WT || K % 16 || K < 16 * STAGES || !aligned16(A) || !aligned16(B) || !aligned16(C)) return false;
+    if (K <= 0 || !aligned16(A) || !aligned16(B) || !aligned16(C)) return false;
     if (static_cast<long long>(K) * 64 >= (1ll << 30) || static_cast<long long>(N) * 64 >= (1ll << 30)) return false;
-    const int tiles_m = M / WT, tiles_n = N / WT;
-    sgemm_single_wave_kernel<WT, STAGES><<<dim3(static_cast<unsigned>(tiles_m) * tiles_n), dim3(kWave), 0, s>>>(
+    const int tiles_m = ceil_div(M, WT), tiles_n = ceil_div(N, WT);
+    const dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n);
+    if (M % WT == 0 && N % WT == 0 && K % 16 == 0 && K >= 16 * STAGES) {
+        sgemm_single_wave_kernel<WT, STAGES, false><<<grid, dim3(kWave), 0, s>>>(
+            M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
+        *rc = check_launch("sgemm_single_wave_kernel");
+        return true;
+    }
+    // Ragged edges: rows must stay 16 B aligned; all of B plus the padding K tiles is addressed with
+    // 32-bit byte offsets.
+    if (!PRISM_SGEMM5_EDGES || N % 4 || K % 4 || (static_cast<long long>(K) + 16 * STAGES) * N * 4 >= (1ll << 31)) return false;
+    sgemm_single_wave_kernel<WT, STAGES, true><<<grid, dim3(kWave), 0, s>>>(
         M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
-    *rc = check_launch("sgemm_single_wave_kernel");
+    *rc = check_launch("sgemm_single_wave_kernel (edges)");
     return true;
 }
 
@@ -1066,8 +1127,8 @@ int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, 
                 // 64 x 64 ones would leave SIMDs without work. In between, the general kernel's 128 x 128
                 // tiles quantise best.
                 const long long simds = 4ll * cu_count();
-                const long long tiles64 = static_cast<long long>(M / 64) * (N / 64);
-                if (tiles64 <= simds) {
+                const long long tiles64 = static_cast<long long>(ceil_div(M, 64)) * ceil_div(N, 64);
+                if (tiles64 <= PRISM_SGEMM5_SINGLE_ROUNDS * simds) {
                     if (tiles64 < simds && try_single_wave<32>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
                     if (try_single_wave<64>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
                 }

@@ -203,17 +203,39 @@ def test_wave_tile_leftover_round(prism, oracle, shape):
     assert np.max(np.abs(got - oracle.np_sgemm_f64(1.25, A, B, 0.5, Cm))) <= tol(oracle, K, A, B, 0.5, Cm)
 
 
-def nan_fenced(a: np.ndarray) -> torch.Tensor:
-    """The matrix as a view into a device buffer whose other elements are NaN (16 B-aligned start)."""
+def nan_fenced(a: np.ndarray, start: int = 1024) -> torch.Tensor:
+    """The matrix as a view into a device buffer whose other elements are NaN; `start` is its first
+    element's index (a multiple of 4 keeps it 16 B aligned)."""
     buf = torch.full((a.size + 2048,), float("nan"), dtype=torch.float32, device=DEV)
-    buf[1024:1024 + a.size] = torch.from_numpy(np.ascontiguousarray(a).ravel()).to(DEV)
-    return buf[1024:1024 + a.size].view(a.shape)
+    buf[start:start + a.size] = torch.from_numpy(np.ascontiguousarray(a).ravel()).to(DEV)
+    return buf[start:start + a.size].view(a.shape)
 
 
-@pytest.mark.parametrize("shape", [(3581, 3580, 100), (3584, 3588, 64), (3585, 3584, 36), (3500, 3600, 4), (3841, 3332, 232)])
+@pytest.mark.parametrize("shape", [(1000, 1001, 999), (515, 777, 130), (128, 128, 16), (1, 1500, 7), (1500, 2, 3), (640, 640, 64)])
+def test_wave_tile_any_shape_between_nans(prism, oracle, shape):
+    """The general kernel 5 path: any M, N, K, operands only 4 B aligned (their first element sits at an
+    odd index). Its edge tiles are filled by range-checked 16 B buffer loads plus masks for what lies past
+    a row's end; A and B sit between NaNs, so a read outside a matrix or a missing mask poisons the output."""
+    M, N, K = shape
+    A, B, Cm = oracle.gen_sgemm(M, N, K, seed=M + 5 * K)
+    for start in (1024, 1021):
+        buf = torch.full((M * N + 512,), 777.0, dtype=torch.float32, device=DEV)
+        c = buf[255:255 + M * N].view(M, N)
+        c.copy_(dev(Cm))
+        prism.sgemm(M, N, K, 1.25, nan_fenced(A, start), nan_fenced(B, start), 0.5, c, variant=5)
+        out = host(buf)
+        assert np.all(out[:255] == 777.0) and np.all(out[255 + M * N:] == 777.0)
+        got = out[255:255 + M * N].reshape(M, N)
+        assert np.max(np.abs(got - oracle.np_sgemm_f64(1.25, A, B, 0.5, Cm))) <= tol(oracle, K, A, B, 0.5, Cm)
+
+
+@pytest.mark.parametrize("shape", [(3581, 3580, 100), (3584, 3588, 64), (3585, 3584, 36), (3500, 3600, 4), (3841, 3332, 232),
+                                   (1000, 1000, 1000), (2000, 1996, 200), (100, 36, 8), (70, 2044, 52), (1, 4, 4)])
 def test_wave_tile_ragged_edges(prism, oracle, shape):
-    """M, N, K that are not whole 256 x 256 x 32 tiles (N and K multiples of 4, enough tiles for the CUs):
-    the whole-tile kernel with zero-filled edges (rows beyond a matrix arrive as zeros through the buffer
+    """M, N, K that are not whole tiles, N and K multiples of 4: with enough 256 x 256 tiles for the CUs
+    (the first five shapes) the whole-tile kernel, for small problems the one-wave-per-tile kernel
+    (64 x 64 or 32 x 32 tiles, at least four K tiles of 16, those beyond K all zeros), both with
+    zero-filled edges (rows beyond a matrix arrive as zeros through the buffer
     descriptor's range check, columns beyond N and k beyond K through an out-of-range lane offset).
     A and B sit between NaNs, so one element read from outside a matrix, or from the next row, would
     poison the output; C is fenced against stores outside it. Every element is checked, with and
