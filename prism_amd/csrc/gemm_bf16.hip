@@ -12,9 +12,12 @@
 //   1 producer + 2 consumer warpgroups      ->  every wave loads and multiplies
 //   persistent CTAs + 16x8 super-tiles      ->  one workgroup per tile, 16x16 super-blocks with an
 //                                               8x4 patch per XCD (tile_map.h)
-//   K tail dropped, M/N multiples required  ->  any M, N, K: problems that are not whole 256x256x64
-//                                               tiles take gemm_bf16_kernel (zero-filled edge tiles,
-//                                               16 B global loads staged in registers one K step
+//   K tail dropped, M/N multiples required  ->  any M, N, K. Ragged M, N, K with K a multiple of 8
+//                                               (16 B-aligned rows): the staged kernel, edges zero-filled
+//                                               by the buffer loads' range check. Anything else (K not a
+//                                               multiple of 8, operands not 16 B aligned):
+//                                               gemm_bf16_kernel (guarded loads, 16 B where a packet
+//                                               lies inside its row; staged in registers one K step
 //                                               ahead, padded LDS rows)
 //
 // prism_gemm_bf16 calls it with (P, Q) = (A, B) and an fp32 OUT = D[M][N].
@@ -132,13 +135,18 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_kerne
         if constexpr (!EDGE) {
             return *reinterpret_cast<const u32x4*>(&base[static_cast<size_t>(row) * K + k]);
         } else {
-            uint16_t e[8];
+            u32x4 r = {0u, 0u, 0u, 0u};
+            if (row < rows && k + 8 <= K) {
+                // Whole packet inside the row: one 16 B access (rows may be only 2 B aligned).
+                __builtin_memcpy(&r, &base[static_cast<size_t>(row) * K + k], 16);
+            } else if (row < rows && k < K) {
+                // The packet that straddles the end of the row: element by element.
+                uint16_t e[8];
 #pragma unroll
-            for (int c = 0; c < 8; ++c)
-                e[c] = (row < rows && k + c < K) ? base[static_cast<size_t>(row) * K + k + c] : uint16_t{0};
-            u32x4 r;
+                for (int c = 0; c < 8; ++c) e[c] = (k + c < K) ? base[static_cast<size_t>(row) * K + k + c] : uint16_t{0};
 #pragma unroll
-            for (int c = 0; c < 4; ++c) r[c] = static_cast<uint32_t>(e[2 * c]) | (static_cast<uint32_t>(e[2 * c + 1]) << 16);
+                for (int c = 0; c < 4; ++c) r[c] = static_cast<uint32_t>(e[2 * c]) | (static_cast<uint32_t>(e[2 * c + 1]) << 16);
+            }
             return r;
         }
     };
@@ -686,9 +694,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
     }
 }
 
-// Kernel choice for whole-tile problems, K tiles of 64: the register-staged pipeline whenever the
-// K tile count is even and at least 6 (measured faster than the ring from 2048^3 up), else the
-// direct-to-LDS ring (any count from 2).
+// Kernel choice. Whole 256 x 256 x 64 tiles: the register-staged pipeline whenever the K tile count
+// is even and at least 6 (measured faster than the ring from 2048^3 up), else the direct-to-LDS ring
+// (any count from 2). Ragged M, N or K with K a multiple of 8 and 16 B-aligned operands: the staged
+// pipeline's edge variant (K tiles padded with zeros to an even count of at least 6). Everything
+// else: the general kernel.
 #ifndef PRISM_BF16_STAGED_MIN_K
 #define PRISM_BF16_STAGED_MIN_K 384
 #endif
