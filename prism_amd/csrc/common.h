@@ -42,6 +42,19 @@ inline bool aligned2(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 1
 template <typename T>
 constexpr T ceil_div(T a, T b) { return (a + b - 1) / b; }
 
+// Compute units of the current device (the launchers size their tile choices by it).
+inline int cu_count() {
+    static int cached[64] = {};  // per device; a racing first call writes the same value
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+        cached[dev] = cus;
+    }
+    return cached[dev];
+}
+
 // Internal launchers, one per kernel family (defined in the .hip files).
 int launch_add_m(const int32_t* x, int32_t* y, int32_t m, size_t n, hipStream_t s);
 size_t scan_workspace_bytes(size_t n);

@@ -287,7 +287,13 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_kerne
 // it has less than one tile time to land, which the staged kernel avoids. 32 x 4
 // stages (also supported by the template) gives loads three tile times but reads
 // half cache lines (64 B per row and tile) and measured slower than both.
-template <int BM, int BN, int BK, int STAGES, int WM, int WN, typename OutT>
+//
+// EDGE: M, N, K need not be whole tiles (K a multiple of 8, so that rows stay 16 B aligned and a
+// 16 B chunk is whole or absent). The direct loads then go through buffer descriptors whose extents
+// end with the matrices: rows beyond them arrive as zeros. Columns k >= K of a row are the next
+// row's data, so in the partial K tile those lanes use an offset beyond any extent; the K loop
+// runs over at least STAGES tiles, those beyond K all zeros.
+template <int BM, int BN, int BK, int STAGES, int WM, int WN, bool EDGE, typename OutT>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_kernel(
     int R, int Cn, int K, const uint16_t* __restrict__ P, const uint16_t* __restrict__ Q,
     OutT* __restrict__ OUT, int tiles_m, int tiles_n) {
@@ -304,7 +310,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_
     static_assert(BM % ROWS_PER_PASS == 0 && BN % ROWS_PER_PASS == 0, "whole load passes");
     constexpr int P_PER = BM / ROWS_PER_PASS, Q_PER = BN / ROWS_PER_PASS;  // loads per wave per tile
     constexpr int LOADS = P_PER + Q_PER, READS = MI + NI, GROUP = MI * NI;
-    static_assert(READS <= GROUP && LOADS <= GROUP, "reads and loads of a tile fit behind the MFMAs of one group");
+    static_assert(READS <= GROUP && LOADS <= GROUP * KS, "the reads of a group and the loads of a tile fit behind the MFMAs");
     static_assert(((ROWS_PER_PASS >> SWZ) % KP) == 0 && ((32 >> SWZ) % KP) == 0,
                   "the swizzle term must repeat with the load pass and the 32-row MFMA block");
 
@@ -337,13 +343,30 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_
     const char* q_wave = reinterpret_cast<const char*>(Q + static_cast<size_t>(col0 + wave * ROWS_PER_LOAD) * K);
     const size_t pass_bytes = static_cast<size_t>(ROWS_PER_PASS) * K * 2;
     // Load number m (0 .. LOADS - 1) of the tile that starts at k0, into stage `stage`.
+    const int p_first = row0 + wave * ROWS_PER_LOAD, q_first = col0 + wave * ROWS_PER_LOAD;
+    const long long p_left = static_cast<long long>(R - p_first) * K * 2, q_left = static_cast<long long>(Cn - q_first) * K * 2;
+    auto extent = [](long long left) -> uint32_t { return static_cast<uint32_t>(left < 0 ? 0 : (left > 0x7fffffff ? 0x7fffffff : left)); };
+    const i32x4 p_rsrc = buffer_descriptor(EDGE && p_left > 0 ? static_cast<const void*>(p_wave) : static_cast<const void*>(P), EDGE ? extent(p_left) : 0u);
+    const i32x4 q_rsrc = buffer_descriptor(EDGE && q_left > 0 ? static_cast<const void*>(q_wave) : static_cast<const void*>(Q), EDGE ? extent(q_left) : 0u);
+    const int k_full = K - K % BK;
+    const uint32_t tail_off = (k_full + ld_chunk * 8 < K) ? lane_off : kBeyondExtent;
     auto issue_load = [&](int stage, int k0, int m) {
-        if (m < P_PER)
-            direct_load16(p_wave + static_cast<size_t>(k0) * 2 + m * pass_bytes, lane_off,
-                          &Ps[stage][(m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]);
-        else
-            direct_load16(q_wave + static_cast<size_t>(k0) * 2 + (m - P_PER) * pass_bytes, lane_off,
-                          &Qs[stage][((m - P_PER) * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]);
+        if constexpr (EDGE) {
+            const uint32_t off = k0 < k_full ? lane_off : (k0 < K ? tail_off : kBeyondExtent);
+            if (m < P_PER)
+                direct_load16_buffer(p_rsrc, off, static_cast<uint32_t>(k0) * 2u + m * static_cast<uint32_t>(pass_bytes),
+                                     &Ps[stage][(m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]);
+            else
+                direct_load16_buffer(q_rsrc, off, static_cast<uint32_t>(k0) * 2u + (m - P_PER) * static_cast<uint32_t>(pass_bytes),
+                                     &Qs[stage][((m - P_PER) * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]);
+        } else {
+            if (m < P_PER)
+                direct_load16(p_wave + static_cast<size_t>(k0) * 2 + m * pass_bytes, lane_off,
+                              &Ps[stage][(m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]);
+            else
+                direct_load16(q_wave + static_cast<size_t>(k0) * 2 + (m - P_PER) * pass_bytes, lane_off,
+                              &Qs[stage][((m - P_PER) * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]);
+        }
     };
 
     // Operand side: row (wave tile origin + 32 i + l32), chunk 2 kk + lhi of the row.
@@ -389,12 +412,13 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_
 #pragma unroll
         for (int g = 0; g < KS; ++g) {
             mfma_group((g + 1) & 1, [&](int m) {
-                // Reads of k-group g behind the first MFMAs of every group; all loads of the next tile behind
-                // the MFMAs of the first group, one each, so that every load has most of the phase to land
-                // (spreading them over two groups was slower for long K, issuing two per MFMA too).
+                // Reads of k-group g behind the first MFMAs of every group; the loads of the next tile one
+                // behind each MFMA from the start of the phase (with 16 MFMAs per group all of them fall
+                // into the first group), so that every load has most of the phase to land (spreading them
+                // over two groups was slower for long K, issuing two per MFMA too).
                 if (m < READS) read_one(S, g, m);
                 if constexpr (prefetch) {
-                    if (g == 0 && m < LOADS) issue_load((S + AHEAD) % STAGES, k_next, m);
+                    if (g * GROUP + m < LOADS) issue_load((S + AHEAD) % STAGES, k_next, g * GROUP + m);
                 }
             });
         }
@@ -420,7 +444,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_
     // stage (first + t) % STAGES with `first` chosen such that the last tile sits in the
     // last stage: the ragged part of the tile count is handled up front and the rest
     // runs in whole rings.
-    const int k_tiles = K / BK;
+    const int k_tiles = EDGE ? ((K + BK - 1) / BK < STAGES ? STAGES : (K + BK - 1) / BK) : K / BK;
     const int ragged = k_tiles % STAGES;
     const int first = (STAGES - ragged) % STAGES;
 #pragma unroll
@@ -468,7 +492,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int row = row0 + wave_m * WM + i * 32 + 8 * (v / 4) + 4 * lhi + (v % 4);
-                store_out(&OUT[static_cast<size_t>(row) * Cn + col], acc[i][j][v]);
+                if (!EDGE || (row < R && col < Cn))
+                    store_out(&OUT[static_cast<size_t>(row) * Cn + col], acc[i][j][v]);
             }
         }
     }
@@ -705,6 +730,12 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
 #ifndef PRISM_BF16_STAGED_EDGES
 #define PRISM_BF16_STAGED_EDGES 1
 #endif
+#ifndef PRISM_BF16_SMALL_TILES
+#define PRISM_BF16_SMALL_TILES 1
+#endif
+#ifndef PRISM_BF16_SMALL_MAX_QUARTERS
+#define PRISM_BF16_SMALL_MAX_QUARTERS 2
+#endif
 #ifndef PRISM_BF16_RING_BK
 #define PRISM_BF16_RING_BK 64
 #endif
@@ -723,13 +754,25 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
     const bool whole = (R % BM == 0) && (Cn % BN == 0) && aligned;
     // The staged kernel addresses a 256-row panel (plus up to six K tiles of padding) with 32-bit offsets.
     const bool panel_ok = static_cast<long long>(BM > BN ? BM : BN) * (static_cast<long long>(K) + 6 * 64) * 2 < (1ll << 31);
-    if (whole && K % 128 == 0 && K >= 6 * 64 && K >= PRISM_BF16_STAGED_MIN_K && panel_ok) {
+    const bool few_tiles = PRISM_BF16_SMALL_TILES && static_cast<long long>(tiles_m) * tiles_n * 4 <
+                                                         static_cast<long long>(PRISM_BF16_SMALL_MAX_QUARTERS) * cu_count();
+    if (whole && !few_tiles && K % 128 == 0 && K >= 6 * 64 && K >= PRISM_BF16_STAGED_MIN_K && panel_ok) {
         gemm_bf16_staged_kernel<BM, BN, WM, WN, false, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
         return check_launch("gemm_bf16_staged_kernel");
     }
+    // Too few 256 x 256 tiles for the CUs: 128 x 128 tiles (four waves of 64 x 64), two workgroups per CU.
+    if (few_tiles && aligned && K % 8 == 0 && K > 0 && panel_ok) {
+        const int tm = ceil_div(R, 128), tn = ceil_div(Cn, 128);
+        const dim3 grid128(static_cast<unsigned>(tm) * tn);
+        if (R % 128 == 0 && Cn % 128 == 0 && K % 64 == 0 && K >= 128)
+            gemm_bf16_ring_kernel<128, 128, 64, 2, 64, 64, false, OutT><<<grid128, dim3(256), 0, s>>>(R, Cn, K, P, Q, OUT, tm, tn);
+        else
+            gemm_bf16_ring_kernel<128, 128, 64, 2, 64, 64, true, OutT><<<grid128, dim3(256), 0, s>>>(R, Cn, K, P, Q, OUT, tm, tn);
+        return check_launch("gemm_bf16_ring_kernel (128 x 128)");
+    }
     if (whole && K % PRISM_BF16_RING_BK == 0 && K >= PRISM_BF16_RING_BK * PRISM_BF16_RING_STAGES &&
         static_cast<long long>(K) * 2 * 64 < (1ll << 32)) {  // 32-bit lane offsets inside a load's rows
-        gemm_bf16_ring_kernel<BM, BN, PRISM_BF16_RING_BK, PRISM_BF16_RING_STAGES, WM, WN, OutT>
+        gemm_bf16_ring_kernel<BM, BN, PRISM_BF16_RING_BK, PRISM_BF16_RING_STAGES, WM, WN, false, OutT>
             <<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
         return check_launch("gemm_bf16_ring_kernel");
     }

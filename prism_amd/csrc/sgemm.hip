@@ -961,17 +961,6 @@ int run_wave_tile(int M, int N, int K, float alpha, const float* A, const float*
     return check_launch("sgemm_wave_tile_kernel");
 }
 
-inline int cu_count() {
-    static int cached[64] = {};  // per device; a racing first call writes the same value
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    if (cached[dev] == 0) {
-        int cus = 0;
-        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
-        cached[dev] = cus;
-    }
-    return cached[dev];
-}
 // Whole-tile kernel when the problem is made of 256 x 256 tiles and there are
 // enough of them for three quarters of the CUs.
 #ifndef PRISM_SGEMM5_DMA
