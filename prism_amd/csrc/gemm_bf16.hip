@@ -42,6 +42,10 @@
 #ifndef PRISM_BF16_SCHED
 #define PRISM_BF16_SCHED 1
 #endif
+#ifndef PRISM_BF16_MFMA_ORDER
+#define PRISM_BF16_MFMA_ORDER 2  // issue order of a group's MFMAs in the staged kernel (see mfma_group there);
+                                 // 8192^3: 1431-1437 / 1434 / 1438-1442 TFLOP/s for 0 / 1 / 2
+#endif
 #ifndef PRISM_BF16_CFG
 #define PRISM_BF16_CFG 256, 256, 64, 128, 128
 #endif
@@ -630,14 +634,19 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
     };
     auto mfma_group = [&](int slot, auto after) {
 #pragma unroll
-        for (int i = 0; i < MI; ++i)
-#pragma unroll
-            for (int j = 0; j < NI; ++j) {
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[slot][i], fb[slot][j], acc[i][j], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-                after(i * NI + j);
-                __builtin_amdgcn_sched_barrier(0);
-            }
+        for (int m = 0; m < MI * NI; ++m) {
+#if PRISM_BF16_MFMA_ORDER == 1   // column-major: B operand fixed for MI instructions
+            const int j = m / MI, i = m % MI;
+#elif PRISM_BF16_MFMA_ORDER == 2  // serpentine: consecutive instructions always share one operand
+            const int i = m / NI, j = (i & 1) ? NI - 1 - m % NI : m % NI;
+#else                             // row-major: A operand fixed for NI instructions
+            const int i = m / NI, j = m % NI;
+#endif
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[slot][i], fb[slot][j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            after(m);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     };
 
     // One phase = everything between two barriers, for the tile in stage S (tile t). Entered
