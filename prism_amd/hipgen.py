@@ -23,12 +23,14 @@ plus an ``extern "C"`` launcher that picks the grid. ``build()`` compiles the te
 with hipcc for gfx950 and returns a ctypes handle; nothing is interpreted on the
 CPU and there is no fallback.
 
-Supported: scalar and pointer parameters of int / float / unsigned, ``id()`` at
+Supported here: scalar and pointer parameters of int / float / unsigned, ``id()`` at
 thread perspective, nested ``partition(..., p=thread[1], offset=e)`` views,
 ``group(thread[1])`` bodies with assignments, augmented assignments, arithmetic,
-comparisons and ``if``. Anything else raises ``HipgenError`` naming the construct:
-block- and warp-level perspectives, shared memory and the automatic barrier
-placement are not part of this slice.
+comparisons and ``if``. Kernels that declare a block perspective (block-level ids
+and views, LDS arrays with automatic barriers, loops, templates, device functions)
+are handed to hipgen_blocks.py, which keeps the reference's nested structure.
+Anything else raises ``HipgenError`` naming the construct; warp-shaped groups
+(``thread[32]``) are not built.
 
 The decorators only register the function's source; annotations are evaluated by
 Python at definition time, so the perspective objects below implement ``[]`` and
@@ -46,7 +48,8 @@ from dataclasses import dataclass, field
 from pathlib import Path
 from typing import Callable, Dict, List, Optional
 
-__all__ = ["prism", "requires", "grid", "block", "warp", "thread", "ptr", "const", "group", "partition",
+__all__ = ["prism", "requires", "attr", "grid", "block", "warp", "thread", "ptr", "const", "restrict", "constexpr",
+           "shared", "uint", "double", "uint32_t", "uint64_t", "group", "partition",
            "generate", "generate_launcher", "build", "HipgenError"]
 
 
@@ -84,7 +87,8 @@ class CType:
 
 grid, block, warp, thread = (Perspective(n) for n in ("grid", "block", "warp", "thread"))
 
-_SCALARS = {"int": "int", "float": "float", "unsigned": "unsigned int", "uint": "unsigned int", "bool": "bool"}
+_SCALARS = {"int": "int", "float": "float", "unsigned": "unsigned int", "uint": "unsigned int", "bool": "bool",
+            "double": "double", "uint32_t": "uint32_t", "uint64_t": "uint64_t"}
 
 
 def _ctype_text(t) -> str:
@@ -98,6 +102,35 @@ def _ctype_text(t) -> str:
 
 def const(t) -> CType:
     return CType("const " + _ctype_text(t))
+
+
+def restrict(t) -> CType:
+    return CType(_ctype_text(t) + " __restrict__")
+
+
+def constexpr(t) -> CType:
+    return CType("constexpr " + _ctype_text(t))
+
+
+class _TypeName:
+    """A type that Python has no builtin name for (`uint`, `double`, ...): annotations are parsed from
+    the source, so these only have to exist, be callable and be indexable."""
+
+    def __init__(self, name: str):
+        self.__name__ = name
+
+    def __getitem__(self, _size):
+        return self
+
+    def __call__(self, *args, **kwargs):
+        return self
+
+    def __matmul__(self, where):
+        return Located(self, where)
+
+
+uint, double, uint32_t, uint64_t = (_TypeName(n) for n in ("uint", "double", "uint32_t", "uint64_t"))
+shared = _TypeName("shared")
 
 
 def ptr(t) -> CType:
@@ -119,6 +152,8 @@ class Kernel:
     kind: str
     source: str
     requires: tuple = ()
+    smem: Optional[int] = None   # @requires(..., smem=bytes): LDS budget the author states
+    attr: str = ""               # @attr("..."): text between the qualifier and the return type
     fn: Optional[Callable] = field(default=None, repr=False)
 
 
@@ -132,12 +167,24 @@ def prism(kind: str):
     return deco
 
 
-def requires(*perspectives: Perspective):
+def requires(*perspectives: Perspective, smem: Optional[int] = None):
     def deco(fn):
         k = _REGISTRY.get(fn.__name__)
         if k is None:
             raise HipgenError("@requires must be applied above @prism")
         k.requires = tuple(perspectives)
+        k.smem = smem
+        return fn
+    return deco
+
+
+def attr(text: str):
+    """`@attr("__launch_bounds__(256)")`, above @prism: printed between the qualifier and the return type."""
+    def deco(fn):
+        k = _REGISTRY.get(fn.__name__)
+        if k is None:
+            raise HipgenError("@attr must be applied above @prism")
+        k.attr = str(text)
         return fn
     return deco
 
@@ -333,25 +380,72 @@ def _kernel(name: str) -> Kernel:
         raise HipgenError(f"no kernel named {name!r} has been defined with @prism") from None
 
 
-def generate(name: str, bounded: bool = False) -> str:
-    """HIP text of kernel `name`. bounded=False prints what the reference prints for the same
-    source (one thread per element, no guard); bounded=True appends a `size_t prism_n` parameter and
-    returns early for thread ids beyond it, so that any grid covering n is legal."""
-    return _Emitter(_kernel(name), bounded).emit()
+def _structured(k: Kernel) -> bool:
+    """Kernels with a block perspective (or device functions) keep the nested form of hipgen_blocks.py."""
+    return k.kind == "device" or any(p.level == "block" for p in k.requires)
 
 
-def generate_launcher(name: str, block_size: int = 256) -> str:
-    """Bounded kernel plus `extern "C" int <name>_launch(<params>, size_t n, void* stream)`:
-    ceil(n / block_size) workgroups of block_size threads (a multiple of the 64-lane wavefront)."""
+def generate(name: str, bounded: bool = False, auto_sync: bool = True) -> str:
+    """HIP text of kernel `name`.
+
+    Thread-level kernels (@requires without a block perspective) are printed flat. bounded=False prints
+    what the reference prints for the same source (one thread per element, no guard); bounded=True
+    appends a `size_t prism_n` parameter and returns early for thread ids beyond it, so that any grid
+    covering n is legal. Kernels with a block perspective are printed by hipgen_blocks.generate_blocks
+    (auto_sync places the barriers); they carry their own guards, so bounded does not apply."""
+    k = _kernel(name)
+    if _structured(k):
+        if bounded:
+            raise HipgenError("bounded=True applies to thread-level kernels only")
+        from .hipgen_blocks import generate_blocks
+        return generate_blocks(name, auto_sync)
+    return _Emitter(k, bounded).emit()
+
+
+def generate_launcher(name: str, block_size: int = 256, template: Optional[List[int]] = None) -> str:
+    """The kernel plus an `extern "C"` launcher.
+
+    Thread-level kernel: bounded kernel and `int <name>_launch(<params>, size_t n, void* stream)`, which
+    starts ceil(n / block_size) workgroups. Kernel with a block perspective:
+    `int <name>_launch(<params>, unsigned grid_blocks, void* stream)`, which starts grid_blocks workgroups
+    of block_size threads with the dynamic LDS the kernel's shared() arrays need; `template` gives the
+    values of its template parameters. block_size is a multiple of the 64-lane wavefront."""
     if block_size % 64 or not 64 <= block_size <= 1024:
         raise HipgenError("block_size must be a multiple of 64 between 64 and 1024")
-    em = _Emitter(_kernel(name), True)
+    k = _kernel(name)
+    head = "#include <hip/hip_runtime.h>\n#include <cstddef>\n#include <cstdint>\n\n"
+    if _structured(k):
+        from .hipgen_blocks import BlockEmitter, device_functions_used, generate_blocks
+        if k.kind != "global":
+            raise HipgenError("only global kernels have launchers")
+        em = BlockEmitter(k, True)
+        text = em.emit_function()
+        if len(template or []) != len(em.template):
+            raise HipgenError(f"{name} has {len(em.template)} template parameters, {len(template or [])} values given")
+        if k.smem is not None and em.smem_offset > k.smem:
+            raise HipgenError(f"{name} declares smem={k.smem} but its shared() arrays take {em.smem_offset} bytes")
+        helpers = "".join(generate_blocks(d) + "\n" for d in device_functions_used(name))
+        targs = "<" + ", ".join(str(int(v)) for v in template) + ">" if template else ""
+        params = ", ".join(f"{t} {n}" for t, n in em.params)
+        args = ", ".join(n for _, n in em.params)
+        sep = ", " if params else ""
+        return (
+            head + helpers + text + "\n"
+            f'extern "C" int {name}_launch({params}{sep}unsigned grid_blocks, void* stream) {{\n'
+            "    if (grid_blocks == 0) return 0;\n"
+            f"    {name}{targs}<<<dim3(grid_blocks), dim3({block_size}), {em.smem_offset}, static_cast<hipStream_t>(stream)>>>"
+            f"({args});\n"
+            "    return static_cast<int>(hipGetLastError());\n"
+            "}\n")
+    if template:
+        raise HipgenError("thread-level kernels take no template values")
+    em = _Emitter(k, True)
     text = em.emit()
     params = ", ".join(f"{t} {n}" for t, n in em.params)
     args = ", ".join(n for _, n in em.params)
     sep = ", " if params else ""
     return (
-        "#include <hip/hip_runtime.h>\n#include <cstddef>\n\n" + text + "\n"
+        head + text + "\n"
         f'extern "C" int {name}_launch({params}{sep}size_t n, void* stream) {{\n'
         "    if (n == 0) return 0;\n"
         f"    const size_t blocks = (n + {block_size - 1}) / {block_size};\n"
@@ -362,14 +456,16 @@ def generate_launcher(name: str, block_size: int = 256) -> str:
         "}\n")
 
 
-def build(name: str, out_dir: Optional[str] = None, block_size: int = 256) -> ctypes.CDLL:
-    """Compile `generate_launcher(name)` for gfx950 and load it. The handle's `<name>_launch` takes the
-    kernel's parameters (device pointers as integers), the element count and a stream handle."""
+def build(name: str, out_dir: Optional[str] = None, block_size: int = 256,
+          template: Optional[List[int]] = None) -> ctypes.CDLL:
+    """Compile `generate_launcher(name, block_size, template)` for gfx950 and load it. The handle's
+    `<name>_launch` takes the kernel's parameters (device pointers as integers), then the element count
+    (thread-level kernels) or the number of workgroups (kernels with a block perspective), then a stream."""
     from .build import HIPCC_FLAGS, hipcc_path
     d = Path(out_dir) if out_dir else Path(tempfile.mkdtemp(prefix="prism_hipgen_"))
     d.mkdir(parents=True, exist_ok=True)
     src, lib = d / f"{name}.hip", d / f"lib{name}.so"
-    src.write_text(generate_launcher(name, block_size))
+    src.write_text(generate_launcher(name, block_size, template))
     proc = subprocess.run([hipcc_path(), *HIPCC_FLAGS, "-shared", "-o", str(lib), str(src)],
                           capture_output=True, text=True)
     if proc.returncode != 0:

@@ -1,0 +1,647 @@
+"""HIP emitter for Prism kernels with block- and thread-level structure (gfx950).
+
+The second slice of the HIP back-end for the reference's front end (prism/codegen.py:321-384 prologue,
+:422-530 declarations, :700-738 loops, :744-849 group/partition; surface syntax in
+examples/sgemm_kernel_1.py, examples/sgemm_shared_mem_block.py, examples/sgemm_kernel_3.py,
+examples/add_m_block_thread.py, examples/function_call.py). hipgen.py's first slice folds a purely
+per-thread kernel into a flat body; this one keeps the reference's structure:
+
+  * every kernel starts from `__block_id_0 = blockIdx.x` and
+    `__thread_id_0 = __block_id_0 * blockDim.x + threadIdx.x`; `with group(level[n])` opens a scope with
+    the ids of the next depth (block: `__block_id_d = outer % n`, thread id rebuilt from it; thread:
+    `__thread_id_d = outer % n`), and `id()` in a declaration `@ level[n]` reads the id of that level
+    at the current depth (divided by n when n > 1);
+  * `with partition(a, p=..., offset=e) as v` opens a scope with `T* v = a + (e);`;
+  * `shared(T[n], static=True)` is a `__shared__` array, `shared(T[n])` a window of the dynamic LDS
+    block `__smem` at the running offset; `T[n] @ thread[1]` is a private array;
+  * `template=[("BM", int), ...]` becomes `template<int BM, ...>`, `@attr("...")` goes between
+    `__global__` and the return type; `@prism("device")` functions take the caller's ids and `__smem`
+    as three leading arguments, which calls to them pass along.
+
+Barriers. The reference derives `__syncthreads()` placement from an analysis of which threads touch
+which elements (prism/sync_analysis.py, prism/sync_transform.py). Here placement is conservative and
+array-granular: walking a block's statements in program order, a barrier goes in front of the first
+statement that reads an LDS array written since the last barrier (by any thread), or writes one read
+since then (in front of the whole loop when that statement sits in one); a loop whose body would meet
+such a hazard with its own previous iteration gets a barrier at the end of the body. A barrier is never placed inside an `if` (threads may disagree on the branch):
+the hazard is resolved in front of the `if`, and one that lies wholly inside an `if` is an error.
+Two writes to one array without a read in between are taken to hit different elements. For the
+reference's LDS-tiled SGEMM example this gives the two barriers the reference prints
+(generated/sgemm_shared_mem_block.cu:38,42).
+
+Not part of this slice, refused by name: warp-shaped groups (`thread[32]`; a wavefront has 64 lanes,
+so shuffles and their masks need a design of their own), `claim`, `split`, `f=lambda` partitions,
+inline PTX (`intrinsic`, `unsafe`), asynchronous copies.
+"""
+from __future__ import annotations
+
+import ast
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Set, Tuple
+
+from .hipgen import HipgenError, Kernel, _BINOPS, _CMPOPS, _REGISTRY, _UNOPS
+
+_TYPES = {"int": ("int", 4), "float": ("float", 4), "double": ("double", 8), "bool": ("bool", 1),
+          "uint": ("unsigned int", 4), "unsigned": ("unsigned int", 4), "uint32_t": ("uint32_t", 4),
+          "uint64_t": ("uint64_t", 8), "void": ("void", 0)}
+_LEVELS = ("grid", "block", "thread")
+
+
+@dataclass(frozen=True)
+class _Ids:
+    block_id: str
+    thread_id: str
+    depth: int
+
+
+def _line(node: ast.AST) -> str:
+    return f"line {getattr(node, 'lineno', '?')}"
+
+
+def _level(node: ast.AST) -> Tuple[str, int]:
+    """`block[16]` as written -> ("block", 16)."""
+    if (isinstance(node, ast.Subscript) and isinstance(node.value, ast.Name) and node.value.id in _LEVELS
+            and isinstance(node.slice, ast.Constant) and isinstance(node.slice.value, int)):
+        return node.value.id, node.slice.value
+    if isinstance(node, ast.Subscript) and isinstance(node.value, ast.Name) and node.value.id == "warp":
+        raise HipgenError(f"{_line(node)}: warp-level perspectives are not part of this slice")
+    raise HipgenError(f"{_line(node)}: expected a perspective such as block[1]")
+
+
+def _is_call(node: ast.AST, name: str) -> bool:
+    return isinstance(node, ast.Call) and isinstance(node.func, ast.Name) and node.func.id == name
+
+
+class _Scalar:
+    """C text of a type expression as written in an annotation."""
+
+    @staticmethod
+    def text(node: ast.AST) -> str:
+        if isinstance(node, ast.Name):
+            if node.id in _TYPES:
+                return _TYPES[node.id][0]
+            raise HipgenError(f"{_line(node)}: unsupported type {node.id}")
+        if isinstance(node, ast.Call) and isinstance(node.func, ast.Name) and node.args:
+            inner = _Scalar.text(node.args[0])
+            if node.func.id == "ptr":
+                return inner + "*"
+            if node.func.id == "const":
+                return "const " + inner
+            if node.func.id == "restrict":
+                return inner + " __restrict__"
+            if node.func.id == "constexpr":
+                return "constexpr " + inner
+        raise HipgenError(f"{_line(node)}: unsupported type expression")
+
+
+def _annotation(node: ast.AST) -> Tuple[ast.AST, Optional[Tuple[str, int]]]:
+    """`T @ level[n]` -> (T, (level, n)); a bare `T` -> (T, None)."""
+    if isinstance(node, ast.BinOp) and isinstance(node.op, ast.MatMult):
+        return node.left, _level(node.right)
+    return node, None
+
+
+# --------------------------------------------------------------- barrier plan --
+
+class _SyncPlan:
+    """Which statements get a barrier in front of them / at the end of their body."""
+
+    def __init__(self, fn: ast.FunctionDef):
+        self.before: Set[int] = set()     # id(stmt)
+        self.at_end: Set[int] = set()     # id(loop stmt)
+        self.root: Dict[str, str] = {}    # LDS array or view of one -> the array
+        self._collect(fn.body)
+        self._walk(fn.body, (set(), set()), True)
+
+    def _collect(self, stmts: List[ast.stmt]) -> None:
+        for s in stmts:
+            if isinstance(s, ast.AnnAssign) and isinstance(s.target, ast.Name):
+                t, _ = _annotation(s.annotation)
+                if _is_call(t, "shared"):
+                    self.root[s.target.id] = s.target.id
+            elif isinstance(s, ast.With):
+                call = s.items[0].context_expr
+                target = s.items[0].optional_vars
+                if (_is_call(call, "partition") and call.args and isinstance(call.args[0], ast.Name)
+                        and isinstance(target, ast.Name) and call.args[0].id in self.root):
+                    self.root[target.id] = self.root[call.args[0].id]
+            for field in ("body", "orelse"):
+                self._collect(getattr(s, field, []) or [])
+
+    # read / write sets of LDS arrays
+    def _reads(self, node: Optional[ast.AST]) -> Set[str]:
+        out: Set[str] = set()
+        if node is None:
+            return out
+        for n in ast.walk(node):
+            if isinstance(n, ast.Name) and n.id in self.root:
+                out.add(self.root[n.id])  # an element read, or the array handed to a function
+        return out
+
+    def _with_reads(self, s: ast.With) -> Set[str]:
+        """A view is pointer arithmetic; only its offset expression can read memory."""
+        out: Set[str] = set()
+        for item in s.items:
+            call = item.context_expr
+            if isinstance(call, ast.Call):
+                for kw in call.keywords:
+                    if kw.arg == "offset":
+                        out |= self._reads(kw.value)
+        return out
+
+    def _access(self, s: ast.stmt) -> Tuple[Set[str], Set[str]]:
+        """(reads, writes) of a statement that holds no other statements."""
+        if isinstance(s, ast.Assign):
+            r, w = self._reads(s.value), set()
+            for t in s.targets:
+                if isinstance(t, ast.Subscript) and isinstance(t.value, ast.Name) and t.value.id in self.root:
+                    w.add(self.root[t.value.id])
+                    r |= self._reads(t.slice)
+                else:
+                    r |= self._reads(t)
+            return r, w
+        if isinstance(s, ast.AugAssign):
+            r = self._reads(s.value) | self._reads(s.target)
+            w = set()
+            if isinstance(s.target, ast.Subscript) and isinstance(s.target.value, ast.Name) and s.target.value.id in self.root:
+                w.add(self.root[s.target.value.id])
+            return r, w
+        if isinstance(s, ast.AnnAssign):
+            return self._reads(s.value), set()
+        if isinstance(s, ast.Expr):
+            r = self._reads(s.value)
+            # A call that is handed an LDS array may write it as well.
+            return r, (set(r) if isinstance(s.value, ast.Call) else set())
+        if isinstance(s, ast.Return):
+            return self._reads(s.value), set()
+        return set(), set()
+
+    def _whole(self, stmts: List[ast.stmt]) -> Tuple[Set[str], Set[str]]:
+        r: Set[str] = set()
+        w: Set[str] = set()
+        for s in stmts:
+            if isinstance(s, ast.With):
+                r |= self._with_reads(s)
+                a, b = self._whole(s.body)
+            elif isinstance(s, (ast.For, ast.While)):
+                r |= self._reads(s.iter if isinstance(s, ast.For) else s.test)
+                a, b = self._whole(s.body)
+            elif isinstance(s, ast.If):
+                r |= self._reads(s.test)
+                a, b = self._whole(s.body + s.orelse)
+            else:
+                a, b = self._access(s)
+            r |= a
+            w |= b
+        return r, w
+
+    @staticmethod
+    def _hazard(r: Set[str], w: Set[str], pending: Tuple[Set[str], Set[str]]) -> bool:
+        pr, pw = pending
+        return bool((r & pw) or (w & pr))
+
+    def _walk(self, stmts: List[ast.stmt], pending: Tuple[Set[str], Set[str]], may_sync: bool) -> Tuple[Set[str], Set[str]]:
+        """Plans barriers for `stmts` entered with `pending` = (reads, writes) since the last barrier;
+        returns the same pair at the end."""
+        pr, pw = set(pending[0]), set(pending[1])
+        for s in stmts:
+            if isinstance(s, ast.With):
+                r = self._with_reads(s)
+                if self._hazard(r, set(), (pr, pw)):
+                    self._mark(s, may_sync)
+                    pr, pw = set(), set()
+                pr |= r
+                pr, pw = self._walk(s.body, (pr, pw), may_sync)
+            elif isinstance(s, (ast.For, ast.While)):
+                # A hazard between what is pending and anything in the loop is resolved once, in front
+                # of the loop, not in every iteration.
+                r, w = self._whole([s])
+                if self._hazard(r, w, (pr, pw)):
+                    self._mark(s, may_sync)
+                    pr, pw = set(), set()
+                pr |= self._reads(s.iter if isinstance(s, ast.For) else s.test)
+                pr, pw = self._walk(s.body, (pr, pw), may_sync)
+                if self._probe(s.body, (pr, pw)) == "hazard":
+                    if not may_sync:
+                        raise HipgenError(f"{_line(s)}: a loop inside an `if` needs a barrier between its iterations")
+                    self.at_end.add(id(s))
+                    pr, pw = set(), set()
+            elif isinstance(s, ast.If):
+                r, w = self._whole([s])
+                if self._hazard(r, w, (pr, pw)):
+                    self._mark(s, may_sync)
+                    pr, pw = set(), set()
+                # Inside the branches no barrier may be placed; hazards there are errors.
+                a = self._walk(s.body, (set(), set()), False)
+                b = self._walk(s.orelse, (set(), set()), False)
+                pr |= r | a[0] | b[0]
+                pw |= w | a[1] | b[1]
+            else:
+                r, w = self._access(s)
+                if self._hazard(r, w, (pr, pw)):
+                    self._mark(s, may_sync)
+                    pr, pw = set(), set()
+                pr |= r
+                pw |= w
+        return pr, pw
+
+    def _mark(self, s: ast.stmt, may_sync: bool) -> None:
+        if not may_sync:
+            raise HipgenError(f"{_line(s)}: LDS is written and read inside one `if`; the barrier between "
+                              "them cannot be placed in divergent code")
+        self.before.add(id(s))
+
+    def _probe(self, stmts: List[ast.stmt], pending: Tuple[Set[str], Set[str]]) -> str:
+        """Runs the next iteration's statements against what the previous one left pending:
+        "hazard" if one is met before the first planned barrier, "barrier" if a barrier comes first,
+        "none" if the body ends without either."""
+        for s in stmts:
+            if id(s) in self.before:
+                return "barrier"
+            if isinstance(s, ast.With):
+                if self._hazard(self._with_reads(s), set(), pending):
+                    return "hazard"
+                got = self._probe(s.body, pending)
+            elif isinstance(s, (ast.For, ast.While)):
+                r, w = self._whole([s])
+                got = "hazard" if self._hazard(r, w, pending) else ("barrier" if id(s) in self.at_end else "none")
+            elif isinstance(s, ast.If):
+                r, w = self._whole([s])
+                got = "hazard" if self._hazard(r, w, pending) else "none"
+            else:
+                r, w = self._access(s)
+                got = "hazard" if self._hazard(r, w, pending) else "none"
+            if got != "none":
+                return got
+        return "none"
+
+
+# -------------------------------------------------------------------- emitter --
+
+class BlockEmitter:
+    def __init__(self, kernel: Kernel, auto_sync: bool = True):
+        self.k = kernel
+        self.auto_sync = auto_sync
+        self.out: List[str] = []
+        self.indent = 0
+        self.ids = _Ids("__block_id_0", "__thread_id_0", 0)
+        self.pointer_type: Dict[str, str] = {}   # name -> C pointer type text (parameters, views, arrays)
+        self.smem_offset = 0                     # bytes of __smem handed out so far
+        self.template: List[Tuple[str, str]] = []
+        self.params: List[Tuple[str, str]] = []
+        self.id_level: Optional[Tuple[str, int]] = None  # perspective `id()` resolves against
+        self.plan: Optional[_SyncPlan] = None
+
+    # -- text helpers
+    def emit(self, text: str) -> None:
+        self.out.append("    " * self.indent + text)
+
+    def open(self) -> None:
+        self.emit("{")
+        self.indent += 1
+
+    def close(self) -> None:
+        self.indent -= 1
+        self.emit("}")
+
+    # -- expressions (every binary operation parenthesised, like the reference prints them)
+    def expr(self, n: ast.AST) -> str:
+        if isinstance(n, ast.Constant):
+            if isinstance(n.value, bool):
+                return "true" if n.value else "false"
+            if isinstance(n.value, (int, float)):
+                return str(n.value)
+            raise HipgenError(f"{_line(n)}: unsupported constant {n.value!r}")
+        if isinstance(n, ast.Name):
+            return n.id
+        if isinstance(n, ast.BinOp) and type(n.op) in _BINOPS:
+            return f"({self.expr(n.left)} {_BINOPS[type(n.op)]} {self.expr(n.right)})"
+        if isinstance(n, ast.UnaryOp) and type(n.op) in _UNOPS:
+            return f"({_UNOPS[type(n.op)]}{self.expr(n.operand)})"
+        if isinstance(n, ast.Compare) and all(type(o) in _CMPOPS for o in n.ops):
+            text = self.expr(n.left)
+            for op, right in zip(n.ops, n.comparators):
+                text = f"({text} {_CMPOPS[type(op)]} {self.expr(right)})"
+            return text
+        if isinstance(n, ast.BoolOp):
+            joiner = " && " if isinstance(n.op, ast.And) else " || "
+            return "(" + joiner.join(self.expr(v) for v in n.values) + ")"
+        if isinstance(n, ast.IfExp):
+            return f"({self.expr(n.test)} ? {self.expr(n.body)} : {self.expr(n.orelse)})"
+        if isinstance(n, ast.Subscript):
+            return f"{self.expr(n.value)}[{self.expr(n.slice)}]"
+        if isinstance(n, ast.Attribute):
+            return f"{self.expr(n.value)}.{n.attr}"
+        if isinstance(n, ast.Call):
+            return self.call(n)
+        raise HipgenError(f"{_line(n)}: unsupported expression {type(n).__name__}")
+
+    def level_id(self, level: str, size: int) -> str:
+        if level == "grid":
+            return "0"
+        base = self.ids.block_id if level == "block" else self.ids.thread_id
+        return base if size == 1 else f"({base} / {size})"
+
+    def call(self, n: ast.Call) -> str:
+        if not isinstance(n.func, ast.Name):
+            raise HipgenError(f"{_line(n)}: unsupported call (inline PTX and method calls are not part of this slice)")
+        name = n.func.id
+        if name == "id":
+            if n.args:
+                return self.level_id(*_level(n.args[0]))
+            if self.id_level is None:
+                raise HipgenError(f"{_line(n)}: id() needs a perspective: use it in a declaration `x: T @ level[n] = ...`")
+            return self.level_id(*self.id_level)
+        if name in ("unsafe", "intrinsic", "float4_cast", "claim", "split"):
+            raise HipgenError(f"{_line(n)}: {name}() is not part of this slice")
+        targs = ""
+        for kw in n.keywords:
+            if kw.arg == "template" and isinstance(kw.value, ast.List):
+                targs = "<" + ", ".join(self.expr(e) for e in kw.value.elts) + ">"
+            else:
+                raise HipgenError(f"{_line(n)}: unsupported keyword argument {kw.arg}")
+        args = [self.expr(a) for a in n.args]
+        if name in _REGISTRY and _REGISTRY[name].kind == "device":
+            args = [self.ids.block_id, self.ids.thread_id, "__smem"] + args
+        return f"{name}{targs}({', '.join(args)})"
+
+    # -- statements
+    def block(self, stmts: List[ast.stmt]) -> None:
+        for s in stmts:
+            if self.plan is not None and id(s) in self.plan.before:
+                self.emit("__syncthreads();")
+            self.stmt(s)
+
+    def stmt(self, s: ast.stmt) -> None:
+        if isinstance(s, ast.AnnAssign) and isinstance(s.target, ast.Name):
+            return self.declare(s)
+        if isinstance(s, ast.With) and len(s.items) == 1 and isinstance(s.items[0].context_expr, ast.Call):
+            call = s.items[0].context_expr
+            if _is_call(call, "group"):
+                return self.group(s, call)
+            if _is_call(call, "partition"):
+                return self.partition(s, call, s.items[0].optional_vars)
+            raise HipgenError(f"{_line(s)}: `with {getattr(call.func, 'id', '?')}(...)` is not part of this slice")
+        if isinstance(s, ast.Assign) and len(s.targets) == 1:
+            return self.emit(f"{self.expr(s.targets[0])} = {self.expr(s.value)};")
+        if isinstance(s, ast.AugAssign) and type(s.op) in _BINOPS:
+            return self.emit(f"{self.expr(s.target)} {_BINOPS[type(s.op)]}= {self.expr(s.value)};")
+        if isinstance(s, ast.For):
+            return self.loop(s)
+        if isinstance(s, ast.While):
+            self.emit(f"while ({self.expr(s.test)}) {{")
+            return self.body_and_close(s)
+        if isinstance(s, ast.If):
+            return self.branch(s)
+        if isinstance(s, ast.Return):
+            return self.emit("return;" if s.value is None else f"return {self.expr(s.value)};")
+        if isinstance(s, ast.Break):
+            return self.emit("break;")
+        if isinstance(s, ast.Continue):
+            return self.emit("continue;")
+        if isinstance(s, ast.Pass):
+            return None
+        if isinstance(s, ast.Expr):
+            if isinstance(s.value, ast.Constant) and isinstance(s.value.value, str):
+                return None  # docstring
+            return self.emit(f"{self.expr(s.value)};")
+        raise HipgenError(f"{_line(s)}: unsupported statement {type(s).__name__}")
+
+    def body_and_close(self, s) -> None:
+        self.indent += 1
+        self.block(s.body)
+        if self.plan is not None and id(s) in self.plan.at_end:
+            self.emit("__syncthreads();")
+        self.indent -= 1
+        self.emit("}")
+
+    def loop(self, s: ast.For) -> None:
+        if not (isinstance(s.target, ast.Name) and _is_call(s.iter, "range") and 1 <= len(s.iter.args) <= 3):
+            raise HipgenError(f"{_line(s)}: loops are `for i in range(...)`")
+        a = [self.expr(x) for x in s.iter.args]
+        start, stop, step = ("0", a[0], "1") if len(a) == 1 else (a[0], a[1], "1") if len(a) == 2 else a
+        i = s.target.id
+        bump = f"{i}++" if step == "1" else f"{i} += {step}"
+        self.emit(f"for (int {i} = {start}; {i} < {stop}; {bump}) {{")
+        self.body_and_close(s)
+
+    def branch(self, s: ast.If) -> None:
+        self.emit(f"if ({self.expr(s.test)}) {{")
+        self.indent += 1
+        self.block(s.body)
+        self.indent -= 1
+        rest = s.orelse
+        while rest:
+            if len(rest) == 1 and isinstance(rest[0], ast.If):
+                self.emit(f"}} else if ({self.expr(rest[0].test)}) {{")
+                self.indent += 1
+                self.block(rest[0].body)
+                self.indent -= 1
+                rest = rest[0].orelse
+            else:
+                self.emit("} else {")
+                self.indent += 1
+                self.block(rest)
+                self.indent -= 1
+                rest = []
+        self.emit("}")
+
+    def declare(self, s: ast.AnnAssign) -> None:
+        name = s.target.id
+        t, where = _annotation(s.annotation)
+        if _is_call(t, "shared"):
+            return self.shared(name, t)
+        if isinstance(t, ast.Subscript):  # T[n] or T[a][b]: a private array
+            dims = []
+            base = t
+            while isinstance(base, ast.Subscript):
+                dims.append(base.slice)
+                base = base.value
+            if not (isinstance(base, ast.Name) and base.id in _TYPES):
+                raise HipgenError(f"{_line(s)}: unsupported array type")
+            ctype = _TYPES[base.id][0]
+            extent = "".join(f"[{self.expr(d)}]" for d in reversed(dims))
+            zero = (isinstance(s.value, ast.Set) and len(s.value.elts) == 1
+                    and isinstance(s.value.elts[0], ast.Constant) and s.value.elts[0].value == 0)
+            if s.value is not None and not zero:
+                raise HipgenError(f"{_line(s)}: a private array is declared bare or with `= {{0}}`")
+            self.emit(f"{ctype} {name}{extent}{' = {0}' if zero else ''};")
+            self.pointer_type[name] = ctype + "*"
+            return
+        ctype = _Scalar.text(t)
+        if ctype.endswith("*"):
+            self.pointer_type[name] = ctype
+        if s.value is None:
+            return self.emit(f"{ctype} {name};")
+        saved, self.id_level = self.id_level, where or self.id_level
+        self.emit(f"{ctype} {name} = {self.expr(s.value)};")
+        self.id_level = saved
+
+    def shared(self, name: str, t: ast.Call) -> None:
+        arg = t.args[0] if t.args else None
+        if not (isinstance(arg, ast.Subscript) and isinstance(arg.value, ast.Name) and arg.value.id in _TYPES):
+            raise HipgenError(f"{_line(t)}: expected shared(type[size])")
+        ctype, nbytes = _TYPES[arg.value.id]
+        size = self.expr(arg.slice)
+        align, static = None, False
+        for kw in t.keywords:
+            if kw.arg == "align" and isinstance(kw.value, ast.Constant):
+                align = int(kw.value.value)
+            elif kw.arg == "static" and isinstance(kw.value, ast.Constant):
+                static = bool(kw.value.value)
+            else:
+                raise HipgenError(f"{_line(t)}: shared() takes align= and static=")
+        self.pointer_type[name] = ctype + "*"
+        if static:
+            return self.emit(f"__shared__ {f'__align__({align}) ' if align else ''}{ctype} {name}[{size}];")
+        count = self.constant(arg.slice)
+        if align:
+            self.smem_offset = (self.smem_offset + align - 1) // align * align
+        self.emit(f"{f'__align__({align}) ' if align else ''}{ctype} (&{name})[{size}] = "
+                  f"*(({ctype} (*)[{size}])(__smem + {self.smem_offset}));")
+        self.smem_offset += count * nbytes
+
+    def constant(self, n: ast.AST) -> int:
+        """Element count of a dynamic LDS window: it fixes the next window's offset, so it must be a number."""
+        if isinstance(n, ast.Constant) and isinstance(n.value, int) and not isinstance(n.value, bool):
+            return n.value
+        if isinstance(n, ast.BinOp) and type(n.op) in (ast.Add, ast.Sub, ast.Mult, ast.FloorDiv, ast.Div):
+            a, b = self.constant(n.left), self.constant(n.right)
+            if isinstance(n.op, ast.Add):
+                return a + b
+            if isinstance(n.op, ast.Sub):
+                return a - b
+            if isinstance(n.op, ast.Mult):
+                return a * b
+            return a // b
+        raise HipgenError(f"{_line(n)}: the size of a dynamic shared() array must be a constant "
+                          "(use static=True for sizes that depend on template parameters)")
+
+    def group(self, s: ast.With, call: ast.Call) -> None:
+        if not call.args:
+            raise HipgenError(f"{_line(s)}: group() takes a perspective")
+        level, size = _level(call.args[0])
+        if level == "thread" and size > 1:
+            raise HipgenError(f"{_line(s)}: group(thread[{size}]) is a warp-shaped group: a wavefront has 64 lanes, "
+                              "and warp-level code is not part of this slice")
+        outer = self.ids
+        inner = _Ids(f"__block_id_{outer.depth + 1}", f"__thread_id_{outer.depth + 1}", outer.depth + 1)
+        self.open()
+        if level == "block":
+            self.emit(f"int {inner.block_id} = {outer.block_id} % {size};")
+            self.emit(f"int {inner.thread_id} = {inner.block_id} * blockDim.x + threadIdx.x;")
+        elif level == "thread":
+            self.emit(f"int {inner.block_id} = {outer.block_id};")
+            self.emit(f"int {inner.thread_id} = {outer.thread_id} % {size};")
+        else:
+            self.emit(f"int {inner.block_id} = {outer.block_id};")
+            self.emit(f"int {inner.thread_id} = {outer.thread_id};")
+        saved_level, self.id_level = self.id_level, (level, size)
+        self.ids = inner
+        self.block(s.body)
+        self.ids = outer
+        self.id_level = saved_level
+        self.close()
+
+    def partition(self, s: ast.With, call: ast.Call, target) -> None:
+        if not (isinstance(target, ast.Name) and call.args and isinstance(call.args[0], ast.Name)):
+            raise HipgenError(f"{_line(s)}: expected `with partition(array, p=..., offset=...) as view`")
+        kw = {k.arg: k.value for k in call.keywords}
+        if "f" in kw:
+            raise HipgenError(f"{_line(s)}: partition(f=lambda ...) is not part of this slice")
+        if not set(kw) <= {"p", "offset"}:
+            raise HipgenError(f"{_line(s)}: partition() takes p= and offset=")
+        if "p" in kw:
+            _level(kw["p"])  # checked for shape only: the view is plain pointer arithmetic
+        parent = call.args[0].id
+        ctype = self.pointer_type.get(parent)
+        if ctype is None:
+            raise HipgenError(f"{_line(s)}: {parent} is not a pointer or array")
+        saved, self.id_level = self.id_level, (_level(kw["p"]) if "p" in kw else self.id_level)
+        offset = self.expr(kw["offset"]) if "offset" in kw else "0"
+        self.id_level = saved
+        self.open()
+        self.emit(f"{ctype} {target.id} = {parent} + ({offset});")
+        self.pointer_type[target.id] = ctype
+        self.block(s.body)
+        self.close()
+
+    # -- the function
+    def emit_function(self) -> str:
+        tree = ast.parse(self.k.source)
+        fn = tree.body[0]
+        if not isinstance(fn, ast.FunctionDef):
+            raise HipgenError("expected a function definition")
+        args = fn.args.args
+        defaults = dict(zip([a.arg for a in args[len(args) - len(fn.args.defaults):]], fn.args.defaults))
+        for a in args:
+            if a.arg == "template":
+                d = defaults.get("template")
+                if not isinstance(d, ast.List):
+                    raise HipgenError("template= takes a list of (name, type) pairs")
+                for item in d.elts:
+                    if not (isinstance(item, ast.Tuple) and len(item.elts) == 2 and isinstance(item.elts[0], ast.Constant)):
+                        raise HipgenError("template= takes a list of (name, type) pairs")
+                    self.template.append((_Scalar.text(item.elts[1]), str(item.elts[0].value)))
+                continue
+            if a.annotation is None:
+                raise HipgenError(f"parameter {a.arg} needs a `type @ perspective` annotation")
+            t, _ = _annotation(a.annotation)
+            ctype = _Scalar.text(t)
+            self.params.append((ctype, a.arg))
+            if ctype.endswith("*") or ctype.endswith("__restrict__"):
+                self.pointer_type[a.arg] = ctype
+        device = self.k.kind == "device"
+        ret = "void"
+        if fn.returns is not None:
+            ret = _Scalar.text(_annotation(fn.returns)[0])
+        elif not device and any(isinstance(n, ast.Return) and n.value is not None for n in ast.walk(fn)):
+            raise HipgenError("a global kernel returns nothing")
+        if self.auto_sync:
+            self.plan = _SyncPlan(fn)
+        plist = (["int __block_id", "int __thread_id", "char* __smem"] if device else []) + [f"{t} {n}" for t, n in self.params]
+        if self.template:
+            self.emit("template<" + ", ".join(f"{t} {n}" for t, n in self.template) + ">")
+        attr = f" {self.k.attr}" if getattr(self.k, "attr", "") else ""
+        self.emit(f"{'__device__' if device else '__global__'}{attr} {ret} {self.k.name}({', '.join(plist)}) {{")
+        self.indent += 1
+        if device:
+            self.emit(f"int {self.ids.block_id} = __block_id;")
+            self.emit(f"int {self.ids.thread_id} = __thread_id;")
+        else:
+            self.emit("extern __shared__ __align__(128) char __smem[];")
+            self.emit(f"int {self.ids.block_id} = blockIdx.x;")
+            self.emit(f"int {self.ids.thread_id} = {self.ids.block_id} * blockDim.x + threadIdx.x;")
+        self.block(fn.body)
+        self.indent -= 1
+        self.emit("}")
+        return "\n".join(self.out) + "\n"
+
+
+def generate_blocks(name: str, auto_sync: bool = True) -> str:
+    """HIP text of kernel or device function `name` in the structured form described above."""
+    if name not in _REGISTRY:
+        raise HipgenError(f"no kernel named {name!r} has been defined with @prism")
+    return BlockEmitter(_REGISTRY[name], auto_sync).emit_function()
+
+
+def dynamic_lds_bytes(name: str) -> int:
+    """Bytes of the dynamic LDS block (`__smem`) the kernel's non-static shared() arrays take."""
+    em = BlockEmitter(_REGISTRY[name], False)
+    em.emit_function()
+    return em.smem_offset
+
+
+def device_functions_used(name: str) -> List[str]:
+    """Names of the @prism("device") functions kernel `name` calls, callees first."""
+    order: List[str] = []
+
+    def visit(n: str) -> None:
+        tree = ast.parse(_REGISTRY[n].source)
+        for node in ast.walk(tree):
+            if (isinstance(node, ast.Call) and isinstance(node.func, ast.Name) and node.func.id in _REGISTRY
+                    and _REGISTRY[node.func.id].kind == "device" and node.func.id not in order and node.func.id != n):
+                visit(node.func.id)
+                order.append(node.func.id)
+    visit(name)
+    return order

@@ -1,4 +1,5 @@
-"""The HIP emitter for the thread-level subset of the Prism DSL (prism_amd/hipgen.py).
+"""The HIP emitter for the thread-level subset of the Prism DSL (prism_amd/hipgen.py); kernels with a
+block perspective are covered by test_hipgen_blocks.py.
 
 CPU: the text printed for the reference's add_m_thread example (examples/add_m_thread.py:10-19) equals
 the text the reference documents for it (README.md:133-140); bounded and launcher forms; constructs
@@ -40,9 +41,10 @@ def clipped_axpy(x: ptr(const(float)) @ grid[1], y: ptr(float) @ grid[1], a: flo
                 yv[0] = t
 
 
-@requires(grid[1], block[1], thread[1])
+@requires(grid[1], thread[1])
 @prism("global")
 def block_level(x: ptr(int) @ grid[1]):
+    """Declares no block perspective (so it is printed flat) but asks for a block id."""
     bid: int @ block[1] = id()
 
 

@@ -1,0 +1,337 @@
+"""The HIP emitter for Prism kernels with block-level structure (prism_amd/hipgen_blocks.py).
+
+The kernels below are written in the reference's surface syntax (block and thread perspectives, views,
+LDS arrays without hand-placed barriers, templates, private arrays, a device function) in the manner of
+its examples (examples/sgemm_kernel_1.py, examples/sgemm_shared_mem_block.py, examples/sgemm_kernel_3.py,
+examples/add_m_block_thread.py, examples/function_call.py).
+CPU: structure of the printed text (id chain, scopes, LDS declarations, where the barriers land), refusals
+by name, and that every launcher cross-compiles for gfx950.
+GPU: the compiled kernels run through their C launchers; add_m bit for bit against numpy, the SGEMMs
+within 1e-5 * sqrt(K) * max|A| * max|B| of the fp64 oracle (the compiler is free to contract a * b + c).
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+from prism_amd import hipgen
+from prism_amd.hipgen import (HipgenError, attr, block, const, generate, generate_launcher, grid, group, partition,
+                              prism, ptr, requires, shared, thread)
+from prism_amd.hipgen_blocks import dynamic_lds_bytes
+
+
+@requires(grid[1], block[1], thread[1])
+@prism("global")
+def add_m_blocks(x: ptr(const(int)) @ grid[1], y: ptr(int) @ grid[1], m: int @ grid[1],
+                 per_block: int @ grid[1], n: int @ grid[1]):
+    first: int @ block[1] = id() * per_block
+    with partition(x, p=block[1], offset=first) as x_blk:
+        with partition(y, p=block[1], offset=first) as y_blk:
+            with group(block[1]):
+                lane: int @ thread[1] = id()
+                with partition(x_blk, p=thread[1], offset=lane) as x_one:
+                    with partition(y_blk, p=thread[1], offset=lane) as y_one:
+                        with group(thread[1]):
+                            if first + lane < n:
+                                y_one[0] = x_one[0] + m
+
+
+@requires(grid[1], block[1], thread[1])
+@prism("global")
+def naive_sgemm(M: int @ grid[1], N: int @ grid[1], K: int @ grid[1], alpha: float @ grid[1],
+                A: ptr(const(float)) @ grid[1], B: ptr(const(float)) @ grid[1], beta: float @ grid[1],
+                C: ptr(float) @ grid[1], per_block: int @ grid[1]):
+    blk: int @ block[1] = id()
+    with partition(C, p=block[1], offset=0) as C_of_block:
+        with group(block[1]):
+            e: int @ thread[1] = blk * per_block + id()
+            row: const(int) @ thread[1] = e / N
+            col: const(int) @ thread[1] = e % N
+            with partition(C_of_block, p=thread[1], offset=0) as C_mine:
+                with group(thread[1]):
+                    if e < M * N:
+                        acc: float @ thread[1] = 0
+                        for k in range(K):
+                            acc += A[row * K + k] * B[k * N + col]
+                        C_mine[row * N + col] = alpha * acc + beta * C_mine[row * N + col]
+
+
+@requires(grid[1], block[1], thread[1])
+@prism("global")
+def tiled_sgemm(M: int @ grid[1], N: int @ grid[1], K: int @ grid[1], alpha: float @ grid[1],
+                A: ptr(const(float)) @ grid[1], B: ptr(const(float)) @ grid[1], beta: float @ grid[1],
+                C: ptr(float) @ grid[1], tiles_n: int @ grid[1], template=[("TILE", int)]):
+    tile_r: const(int) @ block[1] = id() / tiles_n
+    tile_c: const(int) @ block[1] = id() % tiles_n
+    with partition(A, p=block[1], offset=tile_r * TILE * K) as A_rows:
+        with partition(B, p=block[1], offset=tile_c * TILE) as B_cols:
+            with partition(C, p=block[1], offset=tile_r * TILE * N + tile_c * TILE) as C_tile:
+                with group(block[1]):
+                    a_lds: shared(float[TILE * TILE], static=True) @ block[1]
+                    b_lds: shared(float[TILE * TILE], static=True) @ block[1]
+                    r: const(int) @ thread[1] = id() / TILE
+                    c: const(int) @ thread[1] = id() % TILE
+                    acc: float @ thread[1] = 0
+                    with group(thread[1]):
+                        for k0 in range(0, K, TILE):
+                            a_lds[r * TILE + c] = A_rows[r * K + k0 + c]
+                            b_lds[r * TILE + c] = B_cols[(k0 + r) * N + c]
+                            for d in range(TILE):
+                                acc += a_lds[r * TILE + d] * b_lds[d * TILE + c]
+                        C_tile[r * N + c] = alpha * acc + beta * C_tile[r * N + c]
+
+
+@attr("__launch_bounds__((BM * BN) / (TM * TN))")
+@requires(grid[1], block[1], thread[1], smem=8192)
+@prism("global")
+def thread_tile_sgemm(M: int @ grid[1], N: int @ grid[1], K: int @ grid[1], alpha: float @ grid[1],
+                      A: ptr(const(float)) @ grid[1], B: ptr(const(float)) @ grid[1], beta: float @ grid[1],
+                      C: ptr(float) @ grid[1], tiles_n: int @ grid[1],
+                      template=[("BM", int), ("BN", int), ("BK", int), ("TM", int), ("TN", int)]):
+    tile_r: const(int) @ block[1] = id() / tiles_n
+    tile_c: const(int) @ block[1] = id() % tiles_n
+    with partition(A, p=block[1], offset=tile_r * BM * K) as A_rows:
+        with partition(B, p=block[1], offset=tile_c * BN) as B_cols:
+            with partition(C, p=block[1], offset=tile_r * BM * N + tile_c * BN) as C_tile:
+                with group(block[1]):
+                    a_lds: shared(float[1024]) @ block[1]
+                    b_lds: shared(float[1024]) @ block[1]
+                    t: const(int) @ thread[1] = id()
+                    threads: const(int) @ thread[1] = (BM * BN) / (TM * TN)
+                    out_r: const(int) @ thread[1] = t / (BN / TN)
+                    out_c: const(int) @ thread[1] = t % (BN / TN)
+                    acc: float[16] @ thread[1] = {0}
+                    a_reg: float[4] @ thread[1] = {0}
+                    b_reg: float[4] @ thread[1] = {0}
+                    for k0 in range(0, K, BK):
+                        with group(thread[1]):
+                            for e in range(t, BM * BK, threads):
+                                a_lds[e] = A_rows[(e / BK) * K + k0 + e % BK]
+                            for e in range(t, BK * BN, threads):
+                                b_lds[e] = B_cols[(k0 + e / BN) * N + e % BN]
+                            for kk in range(BK):
+                                for i in range(TM):
+                                    a_reg[i] = a_lds[(out_r * TM + i) * BK + kk]
+                                for j in range(TN):
+                                    b_reg[j] = b_lds[kk * BN + out_c * TN + j]
+                                for i in range(TM):
+                                    for j in range(TN):
+                                        acc[i * TN + j] += a_reg[i] * b_reg[j]
+                    with group(thread[1]):
+                        for i in range(TM):
+                            for j in range(TN):
+                                C_tile[(out_r * TM + i) * N + out_c * TN + j] = \
+                                    alpha * acc[i * TN + j] + beta * C_tile[(out_r * TM + i) * N + out_c * TN + j]
+
+
+@requires(thread[1])
+@prism("device")
+def scaled_sum(a: float @ thread[1], b: float @ thread[1], s: float @ thread[1]) -> float @ thread[1]:
+    return s * (a + b)
+
+
+@requires(grid[1], block[1], thread[1])
+@prism("global")
+def scaled_sum_all(x: ptr(const(float)) @ grid[1], y: ptr(float) @ grid[1], s: float @ grid[1], n: int @ grid[1]):
+    i: int @ thread[1] = id()  # outside every group: the thread's number in the whole grid
+    with group(block[1]):
+        with group(thread[1]):
+            if i < n:
+                y[i] = scaled_sum(x[i], y[i], s)
+
+
+@requires(grid[1], block[1], thread[1])
+@prism("global")
+def hazard_in_branch(x: ptr(float) @ grid[1]):
+    with group(block[1]):
+        buf: shared(float[64], static=True) @ block[1]
+        t: int @ thread[1] = id()
+        if t < 32:
+            buf[t] = x[t]
+            x[t] = buf[31 - t]
+
+
+@requires(grid[1], block[1], thread[32])
+@prism("global")
+def warp_shaped(x: ptr(float) @ grid[1]):
+    with group(block[1]):
+        with group(thread[32]):
+            w: int @ thread[32] = id()
+
+
+def lines(text):
+    return [ln.strip() for ln in text.splitlines()]
+
+
+def test_id_chain_and_scopes_of_a_block_thread_kernel():
+    text = generate("add_m_blocks")
+    got = lines(text)
+    assert got[0] == "__global__ void add_m_blocks(const int* x, int* y, int m, int per_block, int n) {"
+    assert got[1:4] == ["extern __shared__ __align__(128) char __smem[];", "int __block_id_0 = blockIdx.x;",
+                        "int __thread_id_0 = __block_id_0 * blockDim.x + threadIdx.x;"]
+    assert "int first = (__block_id_0 * per_block);" in got
+    assert "const int* x_blk = x + (first);" in got and "int* y_blk = y + (first);" in got
+    # group(block[1]) opens depth 1: the thread id inside it is the id within the block
+    i = got.index("int __block_id_1 = __block_id_0 % 1;")
+    assert got[i + 1] == "int __thread_id_1 = __block_id_1 * blockDim.x + threadIdx.x;"
+    assert got[i + 2] == "int lane = __thread_id_1;"
+    j = got.index("int __block_id_2 = __block_id_1;")
+    assert got[j + 1] == "int __thread_id_2 = __thread_id_1 % 1;"
+    assert "if (((first + lane) < n)) {" in got and "y_one[0] = (x_one[0] + m);" in got
+    assert text.count("{") == text.count("}") and "__syncthreads();" not in got
+
+
+def test_loops_guards_and_expressions():
+    got = lines(generate("naive_sgemm"))
+    assert "int e = ((blk * per_block) + __thread_id_1);" in got
+    assert "const int row = (e / N);" in got and "const int col = (e % N);" in got
+    assert "for (int k = 0; k < K; k++) {" in got
+    assert "acc += (A[((row * K) + k)] * B[((k * N) + col)]);" in got
+    assert "C_mine[((row * N) + col)] = ((alpha * acc) + (beta * C_mine[((row * N) + col)]));" in got
+
+
+def test_barriers_of_the_lds_tiled_kernel():
+    """Stores into both LDS tiles, barrier, the dot-product loop that reads them, barrier at the end of the
+    K loop's body (the next iteration overwrites what this one read): the two barriers the reference
+    prints for its LDS-tiled example (generated/sgemm_shared_mem_block.cu:38,42)."""
+    got = lines(generate("tiled_sgemm"))
+    assert got[0] == "template<int TILE>"
+    assert "__shared__ float a_lds[(TILE * TILE)];" in got and "__shared__ float b_lds[(TILE * TILE)];" in got
+    assert got.count("__syncthreads();") == 2
+    first = got.index("__syncthreads();")
+    assert got[first - 1].startswith("b_lds[") and got[first + 1] == "for (int d = 0; d < TILE; d++) {"
+    second = got.index("__syncthreads();", first + 1)
+    assert got[second - 1] == "}" and got[second + 1] == "}"          # closes the d loop, then the k0 loop
+    assert got[second + 2].startswith("C_tile[")
+    assert "for (int k0 = 0; k0 < K; k0 += TILE) {" in got
+    assert "__syncthreads();" not in lines(generate("tiled_sgemm", auto_sync=False))
+
+
+def test_dynamic_lds_windows_private_arrays_and_attr():
+    text = generate("thread_tile_sgemm")
+    got = lines(text)
+    assert got[0] == "template<int BM, int BN, int BK, int TM, int TN>"
+    assert got[1].startswith("__global__ __launch_bounds__((BM * BN) / (TM * TN)) void thread_tile_sgemm(")
+    assert "float (&a_lds)[1024] = *((float (*)[1024])(__smem + 0));" in got
+    assert "float (&b_lds)[1024] = *((float (*)[1024])(__smem + 4096));" in got
+    assert dynamic_lds_bytes("thread_tile_sgemm") == 8192
+    assert "float acc[16] = {0};" in got and "float a_reg[4] = {0};" in got
+    assert "for (int e = t; e < (BM * BK); e += threads) {" in got
+    # one barrier between the two staging loops and the compute loop, one before the next K step
+    assert got.count("__syncthreads();") == 2
+    first = got.index("__syncthreads();")
+    assert got[first + 1] == "for (int kk = 0; kk < BK; kk++) {"
+    launcher = generate_launcher("thread_tile_sgemm", block_size=256, template=[64, 64, 8, 4, 4])
+    assert "thread_tile_sgemm<64, 64, 8, 4, 4><<<dim3(grid_blocks), dim3(256), 8192," in launcher
+    with pytest.raises(HipgenError, match="template parameters"):
+        generate_launcher("thread_tile_sgemm", block_size=256)
+
+
+def test_device_function_gets_the_callers_ids():
+    helper = lines(generate("scaled_sum"))
+    assert helper[0] == "__device__ float scaled_sum(int __block_id, int __thread_id, char* __smem, float a, float b, float s) {"
+    assert helper[1:3] == ["int __block_id_0 = __block_id;", "int __thread_id_0 = __thread_id;"]
+    assert "return (s * (a + b));" in helper
+    caller = generate("scaled_sum_all")
+    assert "y[i] = scaled_sum(__block_id_2, __thread_id_2, __smem, x[i], y[i], s);" in caller
+    launcher = generate_launcher("scaled_sum_all")
+    assert launcher.index("__device__ float scaled_sum(") < launcher.index("__global__ void scaled_sum_all(")
+
+
+def test_refusals_name_the_construct():
+    with pytest.raises(HipgenError, match="inside one `if`"):
+        generate("hazard_in_branch")
+    with pytest.raises(HipgenError, match="64 lanes"):
+        generate("warp_shaped")
+    with pytest.raises(HipgenError, match="thread-level kernels only"):
+        generate("naive_sgemm", bounded=True)
+
+
+BUILDS = {"add_m_blocks": (256, None), "naive_sgemm": (256, None), "tiled_sgemm": (1024, [32]),
+          "thread_tile_sgemm": (256, [64, 64, 8, 4, 4]), "scaled_sum_all": (256, None)}
+
+
+@pytest.fixture(scope="module")
+def built(tmp_path_factory):
+    """Every kernel above, generated and cross-compiled for gfx950 once for this module."""
+    d = tmp_path_factory.mktemp("hipgen_blocks")
+    return {name: hipgen.build(name, out_dir=str(d), block_size=bs, template=targs) for name, (bs, targs) in BUILDS.items()}
+
+
+def test_launchers_compile_for_gfx950(built):
+    for name in BUILDS:
+        assert hasattr(built[name], f"{name}_launch")
+
+
+SGEMM_ARGS = [ctypes.c_int] * 3 + [ctypes.c_float, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p,
+                                   ctypes.c_int, ctypes.c_uint, ctypes.c_void_p]
+
+
+def run_sgemm(lib, name, oracle, M, N, K, last_arg, grid_blocks):
+    import torch
+    fn = getattr(lib, f"{name}_launch")
+    fn.argtypes = SGEMM_ARGS
+    A, B, Cm = oracle.gen_sgemm(M, N, K, seed=M + N + K)
+    a, b = torch.from_numpy(A).to("cuda:0"), torch.from_numpy(B).to("cuda:0")
+    buf = torch.full((M * N + 128,), 777.0, dtype=torch.float32, device="cuda:0")
+    c = buf[64:64 + M * N].view(M, N)
+    c.copy_(torch.from_numpy(Cm))
+    assert fn(M, N, K, 0.5, a.data_ptr(), b.data_ptr(), 3.0, c.data_ptr(), last_arg, grid_blocks, None) == 0
+    torch.cuda.synchronize()
+    out = buf.cpu().numpy()
+    assert np.all(out[:64] == 777.0) and np.all(out[64 + M * N:] == 777.0)
+    want = oracle.np_sgemm_f64(0.5, A, B, 3.0, Cm)
+    tol = oracle.sgemm_tolerance(K, A, B) + 3.0 * float(np.abs(Cm).max()) * 2**-22
+    assert np.max(np.abs(out[64:64 + M * N].reshape(M, N) - want)) <= tol
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n", [1, 255, 256, 1000, (1 << 20) + 5])
+def test_generated_block_thread_add_m_is_bit_exact(built, n):
+    import torch
+    fn = built["add_m_blocks"].add_m_blocks_launch
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_uint, ctypes.c_void_p]
+    x = np.random.default_rng(n).integers(-2**20, 2**20, n, dtype=np.int32)
+    x[0] = 2**31 - 2
+    xd = torch.from_numpy(x).to("cuda:0")
+    yd = torch.full((n + 4,), -1, dtype=torch.int32, device="cuda:0")
+    assert fn(xd.data_ptr(), yd.data_ptr(), 7, 256, n, (n + 255) // 256, None) == 0
+    torch.cuda.synchronize()
+    y = yd.cpu().numpy()
+    assert np.array_equal(y[:n], x + np.int32(7)) and np.all(y[n:] == -1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(1, 1, 1), (33, 47, 29), (128, 96, 200)])
+def test_generated_naive_sgemm(built, oracle, shape):
+    M, N, K = shape
+    run_sgemm(built["naive_sgemm"], "naive_sgemm", oracle, M, N, K, 256, (M * N + 255) // 256)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(32, 32, 32), (64, 96, 160), (256, 128, 64)])
+def test_generated_lds_tiled_sgemm(built, oracle, shape):
+    """Needs the barriers to be where they belong: without them the tiles are read half-written."""
+    M, N, K = shape
+    run_sgemm(built["tiled_sgemm"], "tiled_sgemm", oracle, M, N, K, N // 32, (M // 32) * (N // 32))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(64, 64, 8), (128, 192, 72), (256, 64, 256)])
+def test_generated_thread_tile_sgemm(built, oracle, shape):
+    M, N, K = shape
+    run_sgemm(built["thread_tile_sgemm"], "thread_tile_sgemm", oracle, M, N, K, N // 64, (M // 64) * (N // 64))
+
+
+@pytest.mark.gpu
+def test_generated_kernel_calls_its_device_function(built):
+    import torch
+    fn = built["scaled_sum_all"].scaled_sum_all_launch
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float, ctypes.c_int, ctypes.c_uint, ctypes.c_void_p]
+    n = 10_001
+    rng = np.random.default_rng(5)
+    x, y = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+    xd, yd = torch.from_numpy(x).to("cuda:0"), torch.from_numpy(y).to("cuda:0")
+    assert fn(xd.data_ptr(), yd.data_ptr(), 0.25, n, (n + 255) // 256, None) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(yd.cpu().numpy(), np.float32(0.25) * (x + y))
