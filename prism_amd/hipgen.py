@@ -29,8 +29,7 @@ thread perspective, nested ``partition(..., p=thread[1], offset=e)`` views,
 comparisons and ``if``. Kernels that declare a block perspective (block-level ids
 and views, LDS arrays with automatic barriers, loops, templates, device functions)
 are handed to hipgen_blocks.py, which keeps the reference's nested structure.
-Anything else raises ``HipgenError`` naming the construct; warp-shaped groups
-(``thread[32]``) are not built.
+Anything else raises ``HipgenError`` naming the construct.
 
 The decorators only register the function's source; annotations are evaluated by
 Python at definition time, so the perspective objects below implement ``[]`` and
@@ -49,7 +48,7 @@ from pathlib import Path
 from typing import Callable, Dict, List, Optional
 
 __all__ = ["prism", "requires", "attr", "grid", "block", "warp", "thread", "ptr", "const", "restrict", "constexpr",
-           "shared", "uint", "double", "uint32_t", "uint64_t", "group", "partition",
+           "shared", "uint", "double", "uint32_t", "uint64_t", "group", "partition", "unsafe",
            "generate", "generate_launcher", "build", "HipgenError"]
 
 
@@ -142,6 +141,7 @@ def group(_where):  # only ever appears inside kernel bodies, which are parsed, 
 
 
 partition = group
+unsafe = group
 
 _REGISTRY: Dict[str, "Kernel"] = {}
 

@@ -29,9 +29,17 @@ Two writes to one array without a read in between are taken to hit different ele
 reference's LDS-tiled SGEMM example this gives the two barriers the reference prints
 (generated/sgemm_shared_mem_block.cu:38,42).
 
-Not part of this slice, refused by name: warp-shaped groups (`thread[32]`; a wavefront has 64 lanes,
-so shuffles and their masks need a design of their own), `claim`, `split`, `f=lambda` partitions,
-inline PTX (`intrinsic`, `unsafe`), asynchronous copies.
+Thread groups (`group(thread[n])`, the reference's warps for n = 32) are index arithmetic only
+(`__thread_id_d = outer % n`), so they carry over to 64-lane wavefronts unchanged as long as a group
+does not straddle two wavefronts: n is a power of two up to 64, and a 32-wide group is one half of a
+wavefront. Cross-lane traffic inside a group comes from `unsafe("...")` statements, whose text is
+printed as it stands and must therefore be HIP: the counterpart of the reference's
+`__shfl_up_sync(static_cast<uint32_t>(-1), val, delta)` (examples/scan.py:23-29) is
+`__shfl_up(val, delta, 32)`, which shifts within each aligned group of 32 lanes. The barrier plan
+does not look into unsafe() text.
+
+Not part of this slice, refused by name: `claim`, `split`, `f=lambda` partitions, inline PTX
+(`intrinsic`), vector casts, asynchronous copies.
 """
 from __future__ import annotations
 
@@ -84,6 +92,8 @@ class _Scalar:
         if isinstance(node, ast.Call) and isinstance(node.func, ast.Name) and node.args:
             inner = _Scalar.text(node.args[0])
             if node.func.id == "ptr":
+                return inner if inner.endswith("*") and _is_call(node.args[0], "shared") else inner + "*"
+            if node.func.id == "shared":  # ptr(shared(T)): a pointer into LDS is a plain pointer in the text
                 return inner + "*"
             if node.func.id == "const":
                 return "const " + inner
@@ -290,6 +300,7 @@ class BlockEmitter:
         self.template: List[Tuple[str, str]] = []
         self.params: List[Tuple[str, str]] = []
         self.id_level: Optional[Tuple[str, int]] = None  # perspective `id()` resolves against
+        self.returns_value = False
         self.plan: Optional[_SyncPlan] = None
 
     # -- text helpers
@@ -352,7 +363,9 @@ class BlockEmitter:
             if self.id_level is None:
                 raise HipgenError(f"{_line(n)}: id() needs a perspective: use it in a declaration `x: T @ level[n] = ...`")
             return self.level_id(*self.id_level)
-        if name in ("unsafe", "intrinsic", "float4_cast", "claim", "split"):
+        if name == "unsafe":
+            raise HipgenError(f"{_line(n)}: unsafe() is a statement")
+        if name in ("intrinsic", "float4_cast", "claim", "split"):
             raise HipgenError(f"{_line(n)}: {name}() is not part of this slice")
         targs = ""
         for kw in n.keywords:
@@ -394,7 +407,11 @@ class BlockEmitter:
         if isinstance(s, ast.If):
             return self.branch(s)
         if isinstance(s, ast.Return):
-            return self.emit("return;" if s.value is None else f"return {self.expr(s.value)};")
+            if s.value is None:
+                # A value-returning function whose value comes from unsafe() text ends in a bare `return`
+                # in the source; printing it would not compile.
+                return None if self.returns_value else self.emit("return;")
+            return self.emit(f"return {self.expr(s.value)};")
         if isinstance(s, ast.Break):
             return self.emit("break;")
         if isinstance(s, ast.Continue):
@@ -404,6 +421,14 @@ class BlockEmitter:
         if isinstance(s, ast.Expr):
             if isinstance(s.value, ast.Constant) and isinstance(s.value.value, str):
                 return None  # docstring
+            if _is_call(s.value, "unsafe"):
+                # Target text, printed as it stands (HIP here, where the reference's examples hold CUDA).
+                a = s.value.args
+                if len(a) != 1 or not (isinstance(a[0], ast.Constant) and isinstance(a[0].value, str)):
+                    raise HipgenError(f"{_line(s)}: unsafe() takes one string")
+                for text in a[0].value.strip().splitlines():
+                    self.emit(text.rstrip())
+                return None
             return self.emit(f"{self.expr(s.value)};")
         raise HipgenError(f"{_line(s)}: unsupported statement {type(s).__name__}")
 
@@ -521,9 +546,11 @@ class BlockEmitter:
         if not call.args:
             raise HipgenError(f"{_line(s)}: group() takes a perspective")
         level, size = _level(call.args[0])
-        if level == "thread" and size > 1:
-            raise HipgenError(f"{_line(s)}: group(thread[{size}]) is a warp-shaped group: a wavefront has 64 lanes, "
-                              "and warp-level code is not part of this slice")
+        if size < 1:
+            raise HipgenError(f"{_line(s)}: a group has at least one member")
+        if level == "thread" and size > 1 and (size & (size - 1) or size > 64):
+            raise HipgenError(f"{_line(s)}: group(thread[{size}]): thread groups are powers of two up to the 64-lane "
+                              "wavefront, so that a group never straddles two wavefronts")
         outer = self.ids
         inner = _Ids(f"__block_id_{outer.depth + 1}", f"__thread_id_{outer.depth + 1}", outer.depth + 1)
         self.open()
@@ -595,6 +622,7 @@ class BlockEmitter:
         ret = "void"
         if fn.returns is not None:
             ret = _Scalar.text(_annotation(fn.returns)[0])
+            self.returns_value = ret != "void"
         elif not device and any(isinstance(n, ast.Return) and n.value is not None for n in ast.walk(fn)):
             raise HipgenError("a global kernel returns nothing")
         if self.auto_sync:

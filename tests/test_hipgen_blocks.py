@@ -16,7 +16,7 @@ import pytest
 
 from prism_amd import hipgen
 from prism_amd.hipgen import (HipgenError, attr, block, const, generate, generate_launcher, grid, group, partition,
-                              prism, ptr, requires, shared, thread)
+                              prism, ptr, requires, shared, thread, uint32_t, unsafe)
 from prism_amd.hipgen_blocks import dynamic_lds_bytes
 
 
@@ -151,12 +151,48 @@ def hazard_in_branch(x: ptr(float) @ grid[1]):
             x[t] = buf[31 - t]
 
 
+@requires(grid[1], block[1], thread[48])
+@prism("global")
+def straddling_groups(x: ptr(float) @ grid[1]):
+    with group(block[1]):
+        with group(thread[48]):
+            w: int @ thread[48] = id()
+
+
+@requires(thread[1])
+@prism("device")
+def lane_shift_up(val: uint32_t @ thread[1], delta: uint32_t @ thread[1]) -> uint32_t @ thread[1]:
+    with group(thread[1]):
+        unsafe("return __shfl_up(val, delta, 32);")
+    return
+
+
 @requires(grid[1], block[1], thread[32])
 @prism("global")
-def warp_shaped(x: ptr(float) @ grid[1]):
-    with group(block[1]):
-        with group(thread[32]):
-            w: int @ thread[32] = id()
+def row_scan32(x: ptr(const(uint32_t)) @ grid[1], y: ptr(uint32_t) @ grid[1], rows: int @ grid[1]):
+    """Inclusive scan of every row of 32 elements by a group of 32 threads (half a wavefront), the
+    building block of the reference's scan (scan_warps, examples/scan.py:106-128)."""
+    first_row: int @ block[1] = id() * 8
+    with partition(x, p=block[1], offset=first_row * 32) as x_blk:
+        with partition(y, p=block[1], offset=first_row * 32) as y_blk:
+            with group(block[1]):
+                g: int @ thread[32] = id()
+                with partition(x_blk, p=thread[32], offset=g * 32) as x_row:
+                    with partition(y_blk, p=thread[32], offset=g * 32) as y_row:
+                        with group(thread[32]):
+                            lane: uint32_t @ thread[1] = id()
+                            with group(thread[1]):
+                                v: uint32_t @ thread[1] = 0
+                                if first_row + g < rows:
+                                    v = x_row[lane]
+                                step: uint32_t @ thread[1] = 1
+                                while step < 32:
+                                    got: uint32_t @ thread[1] = lane_shift_up(v, step)
+                                    if lane >= step:
+                                        v = got + v
+                                    step *= 2
+                                if first_row + g < rows:
+                                    y_row[lane] = v
 
 
 def lines(text):
@@ -241,13 +277,27 @@ def test_device_function_gets_the_callers_ids():
 def test_refusals_name_the_construct():
     with pytest.raises(HipgenError, match="inside one `if`"):
         generate("hazard_in_branch")
-    with pytest.raises(HipgenError, match="64 lanes"):
-        generate("warp_shaped")
+    with pytest.raises(HipgenError, match="powers of two"):
+        generate("straddling_groups")
     with pytest.raises(HipgenError, match="thread-level kernels only"):
         generate("naive_sgemm", bounded=True)
 
 
-BUILDS = {"add_m_blocks": (256, None), "naive_sgemm": (256, None), "tiled_sgemm": (1024, [32]),
+def test_thread_groups_of_32_and_target_text():
+    """A group of 32 threads is index arithmetic (`% 32`, `/ 32`); unsafe() text is printed as it stands, and
+    the bare `return` that follows it in a value-returning function is dropped."""
+    helper = lines(generate("lane_shift_up"))
+    assert helper[0] == "__device__ uint32_t lane_shift_up(int __block_id, int __thread_id, char* __smem, uint32_t val, uint32_t delta) {"
+    assert "return __shfl_up(val, delta, 32);" in helper and "return;" not in helper
+    got = lines(generate("row_scan32"))
+    assert "int g = (__thread_id_1 / 32);" in got
+    i = got.index("int __thread_id_2 = __thread_id_1 % 32;")
+    assert got[i - 1] == "int __block_id_2 = __block_id_1;" and got[i + 1] == "uint32_t lane = __thread_id_2;"
+    assert "while ((step < 32)) {" in got
+    assert "uint32_t got = lane_shift_up(__block_id_3, __thread_id_3, __smem, v, step);" in got
+
+
+BUILDS = {"row_scan32": (256, None), "add_m_blocks": (256, None), "naive_sgemm": (256, None), "tiled_sgemm": (1024, [32]),
           "thread_tile_sgemm": (256, [64, 64, 8, 4, 4]), "scaled_sum_all": (256, None)}
 
 
@@ -321,6 +371,23 @@ def test_generated_lds_tiled_sgemm(built, oracle, shape):
 def test_generated_thread_tile_sgemm(built, oracle, shape):
     M, N, K = shape
     run_sgemm(built["thread_tile_sgemm"], "thread_tile_sgemm", oracle, M, N, K, N // 64, (M // 64) * (N // 64))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows", [1, 8, 9, 1000])
+def test_generated_row_scan_on_half_wavefronts(built, rows):
+    """Groups of 32 threads on 64-lane wavefronts: two rows per wavefront, the shuffle stays inside each."""
+    import torch
+    fn = built["row_scan32"].row_scan32_launch
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_uint, ctypes.c_void_p]
+    x = np.random.default_rng(rows).integers(0, 2**32, (rows, 32), dtype=np.uint32)
+    xd = torch.from_numpy(x.view(np.int32)).to("cuda:0")
+    yd = torch.full((rows * 32 + 64,), -1, dtype=torch.int32, device="cuda:0")
+    assert fn(xd.data_ptr(), yd.data_ptr(), rows, (rows + 7) // 8, None) == 0
+    torch.cuda.synchronize()
+    y = yd.cpu().numpy().view(np.uint32)
+    assert np.array_equal(y[:rows * 32].reshape(rows, 32), np.cumsum(x, axis=1, dtype=np.uint32))
+    assert np.all(y[rows * 32:] == 0xFFFFFFFF)
 
 
 @pytest.mark.gpu
