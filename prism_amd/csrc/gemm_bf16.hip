@@ -300,7 +300,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_kerne
 template <int BM, int BN, int BK, int STAGES, int WM, int WN, bool EDGE, typename OutT>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_kernel(
     int R, int Cn, int K, const uint16_t* __restrict__ P, const uint16_t* __restrict__ Q,
-    OutT* __restrict__ OUT, int tiles_m, int tiles_n) {
+    OutT* __restrict__ OUT, int tiles_m, int tiles_n, int first_big) {
     static_assert((BK == 32 || BK == 64) && (STAGES == 2 || STAGES == 4), "ring shape");
     constexpr int KP = BK / 8;                        // 16 B chunks per row
     constexpr int SWZ = KP == 4 ? 2 : 1;
@@ -321,9 +321,24 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_
     __shared__ __attribute__((aligned(1024))) uint16_t Ps[STAGES][BM * BK];
     __shared__ __attribute__((aligned(1024))) uint16_t Qs[STAGES][BN * BK];
 
-    int tm, tn;
-    xcd_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
-    const int row0 = tm * BM, col0 = tn * BN;
+    // first_big < 0: the grid covers the tiles_m x tiles_n grid of BM x BN tiles. Otherwise this launch
+    // finishes what a launch of a 256 x 256 kernel left over: tiles_m x tiles_n is that kernel's grid,
+    // first_big the first tile number it did not take, and every leftover tile is cut into
+    // (256 / BM) x (256 / BN) tiles of this kernel.
+    int row0, col0;
+    if (first_big < 0) {
+        int tm, tn;
+        xcd_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+        row0 = tm * BM;
+        col0 = tn * BN;
+    } else {
+        constexpr int SUB_M = 256 / BM, SUB_N = 256 / BN;
+        int tm, tn;
+        xcd_tile_coords(first_big + blockIdx.x / (SUB_M * SUB_N), tiles_m, tiles_n, tm, tn);
+        const int sub = blockIdx.x % (SUB_M * SUB_N);
+        row0 = tm * 256 + (sub / SUB_N) * BM;
+        col0 = tn * 256 + (sub % SUB_N) * BN;
+    }
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -739,6 +754,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
 #ifndef PRISM_BF16_STAGED_EDGES
 #define PRISM_BF16_STAGED_EDGES 1
 #endif
+#ifndef PRISM_BF16_LEFTOVER
+#define PRISM_BF16_LEFTOVER 1
+#endif
 #ifndef PRISM_BF16_SMALL_TILES
 #define PRISM_BF16_SMALL_TILES 1
 #endif
@@ -766,23 +784,39 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
     const bool few_tiles = PRISM_BF16_SMALL_TILES && static_cast<long long>(tiles_m) * tiles_n * 4 <
                                                          static_cast<long long>(PRISM_BF16_SMALL_MAX_QUARTERS) * cu_count();
     if (whole && !few_tiles && K % 128 == 0 && K >= 6 * 64 && K >= PRISM_BF16_STAGED_MIN_K && panel_ok) {
-        gemm_bf16_staged_kernel<BM, BN, WM, WN, false, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
-        return check_launch("gemm_bf16_staged_kernel");
+        // Tile counts that do not fill whole rounds of CUs: the staged kernel takes the whole rounds and
+        // the tiles of the last, partial round are cut into 128 x 128 tiles (two workgroups per CU), when
+        // that gives every CU at most two of them (6144^3: 2 rounds + 64 tiles instead of 3 rounds).
+        static_assert(BM == 256 && BN == 256, "the leftover launch cuts 256 x 256 tiles");
+        const int tiles = tiles_m * tiles_n, cus = cu_count();
+        const int left = tiles % cus;
+        const bool cut = PRISM_BF16_LEFTOVER && tiles > cus && left != 0 && left * 4 <= 2 * cus &&
+                         static_cast<long long>(K) * 2 * 64 < (1ll << 32);
+        const int main_tiles = cut ? tiles - left : tiles;
+        gemm_bf16_staged_kernel<BM, BN, WM, WN, false, OutT><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
+            R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
+        if (int rc = check_launch("gemm_bf16_staged_kernel")) return rc;
+        if (cut) {
+            gemm_bf16_ring_kernel<128, 128, 64, 2, 64, 64, false, OutT><<<dim3(static_cast<unsigned>(left) * 4), dim3(256), 0, s>>>(
+                R, Cn, K, P, Q, OUT, tiles_m, tiles_n, main_tiles);
+            return check_launch("gemm_bf16_ring_kernel (leftover)");
+        }
+        return 0;
     }
     // Too few 256 x 256 tiles for the CUs: 128 x 128 tiles (four waves of 64 x 64), two workgroups per CU.
     if (few_tiles && aligned && K % 8 == 0 && K > 0 && panel_ok) {
         const int tm = ceil_div(R, 128), tn = ceil_div(Cn, 128);
         const dim3 grid128(static_cast<unsigned>(tm) * tn);
         if (R % 128 == 0 && Cn % 128 == 0 && K % 64 == 0 && K >= 128)
-            gemm_bf16_ring_kernel<128, 128, 64, 2, 64, 64, false, OutT><<<grid128, dim3(256), 0, s>>>(R, Cn, K, P, Q, OUT, tm, tn);
+            gemm_bf16_ring_kernel<128, 128, 64, 2, 64, 64, false, OutT><<<grid128, dim3(256), 0, s>>>(R, Cn, K, P, Q, OUT, tm, tn, -1);
         else
-            gemm_bf16_ring_kernel<128, 128, 64, 2, 64, 64, true, OutT><<<grid128, dim3(256), 0, s>>>(R, Cn, K, P, Q, OUT, tm, tn);
+            gemm_bf16_ring_kernel<128, 128, 64, 2, 64, 64, true, OutT><<<grid128, dim3(256), 0, s>>>(R, Cn, K, P, Q, OUT, tm, tn, -1);
         return check_launch("gemm_bf16_ring_kernel (128 x 128)");
     }
     if (whole && K % PRISM_BF16_RING_BK == 0 && K >= PRISM_BF16_RING_BK * PRISM_BF16_RING_STAGES &&
         static_cast<long long>(K) * 2 * 64 < (1ll << 32)) {  // 32-bit lane offsets inside a load's rows
         gemm_bf16_ring_kernel<BM, BN, PRISM_BF16_RING_BK, PRISM_BF16_RING_STAGES, WM, WN, false, OutT>
-            <<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
+            <<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n, -1);
         return check_launch("gemm_bf16_ring_kernel");
     }
     // Ragged M, N or K with 16 B-aligned rows: the staged kernel with zero-filled edges.

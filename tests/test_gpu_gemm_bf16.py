@@ -48,12 +48,15 @@ def test_fp32_output_vs_fp64_oracle(prism, oracle, shape):
 
 @pytest.mark.parametrize("shape", [(256, 256, 128), (256, 512, 192), (512, 256, 256), (256, 256, 320), (512, 512, 1024), (256, 256, 384), (256, 256, 448),
                                    (256, 512, 6144), (512, 256, 6208), (128, 384, 6272),
-                                   (3072, 3072, 384), (3072, 3072, 192), (2816, 3328, 448), (3072, 3328, 512)])
+                                   (3072, 3072, 384), (3072, 3072, 192), (2816, 3328, 448), (3072, 3328, 512),
+                                   (4352, 4352, 384)])
 def test_whole_tile_paths(prism, oracle, shape):
     """Problems made of whole tiles leave the general kernel. Fewer than 128 tiles of 256 x 256 (the first
     ten shapes): 128 x 128 tiles, direct-to-LDS ring. From 128 tiles up: an even K tile count from 6 up
     takes the register-staged pipeline (6 and 8 K tiles here), the others the direct-to-LDS ring of
-    256 x 256 tiles (3 and 7 K tiles). Every element is checked, for both output types."""
+    256 x 256 tiles (3 and 7 K tiles). The last shape has 289 tiles for 256 CUs: the 33 tiles of the partial
+    second round are cut into 128 x 128 tiles by a second launch. Every element is checked, for both
+    output types."""
     M, N, K = shape
     A16, B16 = oracle.gen_gemm_bf16(M, N, K, seed=K + M)
     D = prism.gemm_bf16(dev16(A16), dev16(B16))
