@@ -729,6 +729,7 @@ __global__ __launch_bounds__(kWave) void sgemm_single_wave_kernel(
         row0 = tm * 256 + (sub / SUB) * WT;
         col0 = tn * 256 + (sub % SUB) * WT;
     }
+    if (EDGE && (row0 >= M || col0 >= N)) return;  // a piece of an edge tile that lies wholly outside C
     const int lane = threadIdx.x;
     const int l32 = lane & 31, lhi = lane >> 5;
 
@@ -993,21 +994,14 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
     const int tiles_m = ceil_div(M, BM), tiles_n = ceil_div(N, BN);
     if (static_cast<long long>(tiles_m) * tiles_n * 4 < static_cast<long long>(PRISM_SGEMM5_DMA_MIN_QUARTERS) * cu_count()) return false;
     const dim3 block((BM / WM) * (BN / WN) * kWave);
-    if constexpr (ALLOW_EDGES) {
-        if (!whole) {
-            sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, true><<<dim3(static_cast<unsigned>(tiles_m) * tiles_n), block, 0, s>>>(
-                M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n);
-            *rc = check_launch("sgemm_wave_tile_dma_kernel (edges)");
-            return true;
-        }
-    }
     // Tile counts that do not fill whole rounds of CUs: the 256 x 256 kernel takes the whole rounds, and
     // the tiles of the last, partial round are cut into 64 x 64 wave tiles that spread over all SIMDs
     // (6144^3: 2 rounds + 64 tiles instead of 3 rounds). Not worth it when the last round is nearly full.
     static_assert(BM == 256 && BN == 256, "the leftover launch cuts 256 x 256 tiles");
     const int tiles = tiles_m * tiles_n, cus = cu_count();
     int main_tiles = tiles, leftover_wt = 0;
-    if (PRISM_SGEMM5_LEFTOVER && tiles > cus && tiles % cus != 0 && K >= 64) {
+    const bool lane_offsets_fit = static_cast<long long>(K) * 64 < (1ll << 30) && static_cast<long long>(N) * 64 < (1ll << 30);
+    if (PRISM_SGEMM5_LEFTOVER && lane_offsets_fit && tiles > cus && tiles % cus != 0 && K >= 64) {
         // Cost of the last round in units of one full round of 256 x 256 tiles: a wave tile of 64 (32)
         // is 1/4 (1/16) of a SIMD's share of a big tile and runs at about 0.87 (0.72) of its rate.
         const int left = tiles % cus, simds = 4 * cus;
@@ -1018,17 +1012,26 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
             leftover_wt = cost64 <= cost32 ? 64 : 32;
         }
     }
-    sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, false><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
-        M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n);
-    *rc = check_launch("sgemm_wave_tile_dma_kernel");
-    if (*rc == 0 && leftover_wt == 64) {
-        sgemm_single_wave_kernel<64, 4, false><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 16), dim3(kWave), 0, s>>>(
-            M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, main_tiles);
-        *rc = check_launch("sgemm_single_wave_kernel");
-    } else if (*rc == 0 && leftover_wt == 32) {
-        sgemm_single_wave_kernel<32, 4, false><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 64), dim3(kWave), 0, s>>>(
-            M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, main_tiles);
-        *rc = check_launch("sgemm_single_wave_kernel");
+    // `edge` selects the zero-filling variants of both kernels (sub-tiles that lie wholly outside C exit at once).
+    auto launch = [&](auto edge) {
+        constexpr bool EDGE = decltype(edge)::value;
+        sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, EDGE><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
+            M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n);
+        *rc = check_launch("sgemm_wave_tile_dma_kernel");
+        if (*rc == 0 && leftover_wt == 64) {
+            sgemm_single_wave_kernel<64, 4, EDGE><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 16), dim3(kWave), 0, s>>>(
+                M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, main_tiles);
+            *rc = check_launch("sgemm_single_wave_kernel");
+        } else if (*rc == 0 && leftover_wt == 32) {
+            sgemm_single_wave_kernel<32, 4, EDGE><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 64), dim3(kWave), 0, s>>>(
+                M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, main_tiles);
+            *rc = check_launch("sgemm_single_wave_kernel");
+        }
+    };
+    if (whole) {
+        launch(std::false_type{});
+    } else {
+        if constexpr (ALLOW_EDGES) launch(std::true_type{});
     }
     return true;
 }

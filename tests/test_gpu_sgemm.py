@@ -230,12 +230,14 @@ def test_wave_tile_any_shape_between_nans(prism, oracle, shape):
 
 
 @pytest.mark.parametrize("shape", [(3581, 3580, 100), (3584, 3588, 64), (3585, 3584, 36), (3500, 3600, 4), (3841, 3332, 232),
-                                   (1000, 1000, 1000), (2000, 1996, 200), (100, 36, 8), (70, 2044, 52), (1, 4, 4)])
+                                   (1000, 1000, 1000), (2000, 1996, 200), (100, 36, 8), (70, 2044, 52), (1, 4, 4),
+                                   (4300, 4348, 100), (4090, 5116, 68)])
 def test_wave_tile_ragged_edges(prism, oracle, shape):
     """M, N, K that are not whole tiles, N and K multiples of 4: with enough 256 x 256 tiles for the CUs
     (the first five shapes) the whole-tile kernel, for small problems the one-wave-per-tile kernel
     (64 x 64 or 32 x 32 tiles, at least four K tiles of 16, those beyond K all zeros), both with
-    zero-filled edges (rows beyond a matrix arrive as zeros through the buffer
+    zero-filled edges; the last two shapes have 289 and 320 tiles for 256 CUs, so the ragged tiles of
+    the partial second round are cut into one-wave tiles (32 x 32 and 64 x 64), pieces outside C included (rows beyond a matrix arrive as zeros through the buffer
     descriptor's range check, columns beyond N and k beyond K through an out-of-range lane offset).
     A and B sit between NaNs, so one element read from outside a matrix, or from the next row, would
     poison the output; C is fenced against stores outside it. Every element is checked, with and
