@@ -39,6 +39,12 @@ __device__ __forceinline__ void direct_load16(const char* base, uint32_t lane_of
 // kBeyondExtent as its offset.
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 constexpr uint32_t kBeyondExtent = 0x80000000u;  // extents here stay below 2 GiB
+// Extent of a descriptor that should end `bytes_left` bytes after its base: descriptors hold 32 bits, and
+// every offset used here stays below 2 GiB, so anything beyond that is cut to 2 GiB - 1 (kBeyondExtent
+// stays out of range).
+__host__ __device__ __forceinline__ uint32_t clamped_extent(long long bytes_left) {
+    return static_cast<uint32_t>(bytes_left < 0 ? 0 : (bytes_left > 0x7fffffffll ? 0x7fffffffll : bytes_left));
+}
 // Raw buffer descriptor (stride 0) for `extent_bytes` bytes at `base`: base address, extent, and the
 // data-format word of an untyped 32-bit buffer. Wave-uniform by construction (forced into scalar registers).
 __device__ __forceinline__ i32x4 buffer_descriptor(const void* base, uint32_t extent_bytes) {

@@ -364,9 +364,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_
     // Load number m (0 .. LOADS - 1) of the tile that starts at k0, into stage `stage`.
     const int p_first = row0 + wave * ROWS_PER_LOAD, q_first = col0 + wave * ROWS_PER_LOAD;
     const long long p_left = static_cast<long long>(R - p_first) * K * 2, q_left = static_cast<long long>(Cn - q_first) * K * 2;
-    auto extent = [](long long left) -> uint32_t { return static_cast<uint32_t>(left < 0 ? 0 : (left > 0x7fffffff ? 0x7fffffff : left)); };
-    const i32x4 p_rsrc = buffer_descriptor(EDGE && p_left > 0 ? static_cast<const void*>(p_wave) : static_cast<const void*>(P), EDGE ? extent(p_left) : 0u);
-    const i32x4 q_rsrc = buffer_descriptor(EDGE && q_left > 0 ? static_cast<const void*>(q_wave) : static_cast<const void*>(Q), EDGE ? extent(q_left) : 0u);
+    const i32x4 p_rsrc = buffer_descriptor(EDGE && p_left > 0 ? static_cast<const void*>(p_wave) : static_cast<const void*>(P), EDGE ? clamped_extent(p_left) : 0u);
+    const i32x4 q_rsrc = buffer_descriptor(EDGE && q_left > 0 ? static_cast<const void*>(q_wave) : static_cast<const void*>(Q), EDGE ? clamped_extent(q_left) : 0u);
     const int k_full = K - K % BK;
     const uint32_t tail_off = (k_full + ld_chunk * 8 < K) ? lane_off : kBeyondExtent;
     auto issue_load = [&](int stage, int k0, int m) {

@@ -508,9 +508,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
     const long long a_left = static_cast<long long>(M - a_first) * K * 4;
     const long long b_left = (static_cast<long long>(K - wave) * N - col0) * 4;
     const i32x4 a_rsrc = buffer_descriptor(EDGE && a_left > 0 ? static_cast<const void*>(a_wave) : static_cast<const void*>(A),
-                                           EDGE && a_left > 0 ? static_cast<uint32_t>(a_left) : 0u);
+                                           EDGE ? clamped_extent(a_left) : 0u);
     const i32x4 b_rsrc = buffer_descriptor(EDGE && b_left > 0 ? static_cast<const void*>(b_wave) : static_cast<const void*>(B),
-                                           EDGE && b_left > 0 ? static_cast<uint32_t>(b_left) : 0u);
+                                           EDGE ? clamped_extent(b_left) : 0u);
     const int k_full = K - K % BK;
     const uint32_t a_tail = (k_full + ld_chunk * 4 < K) ? a_lane : kBeyondExtent;
     const uint32_t b_edge = (col0 + 4 * lane < N) ? b_lane : kBeyondExtent;
@@ -751,8 +751,8 @@ __global__ __launch_bounds__(kWave) void sgemm_single_wave_kernel(
     const uint32_t b_lane = (static_cast<uint32_t>(b_krow) * static_cast<uint32_t>(N) + b_col) * 4u;
     const char* a_base = reinterpret_cast<const char*>(A + static_cast<size_t>(row0) * K);
     const char* b_base = reinterpret_cast<const char*>(B + col0);
-    const i32x4 a_rsrc = buffer_descriptor(a_base, EDGE ? static_cast<uint32_t>(static_cast<long long>(M - row0) * K * 4) : 0u);
-    const i32x4 b_rsrc = buffer_descriptor(b_base, EDGE ? static_cast<uint32_t>((static_cast<long long>(K) * N - col0) * 4) : 0u);
+    const i32x4 a_rsrc = buffer_descriptor(a_base, EDGE ? clamped_extent(static_cast<long long>(M - row0) * K * 4) : 0u);
+    const i32x4 b_rsrc = buffer_descriptor(b_base, EDGE ? clamped_extent((static_cast<long long>(K) * N - col0) * 4) : 0u);
     const int k_full = K - K % BK;
     const uint32_t a_tail = (k_full + a_chunk * 4 < K) ? a_lane : kBeyondExtent;
     const uint32_t b_edge = (col0 + b_col < N) ? b_lane : kBeyondExtent;

@@ -256,6 +256,30 @@ def test_wave_tile_ragged_edges(prism, oracle, shape):
         assert np.max(np.abs(got - oracle.np_sgemm_f64(1.25, A, B, beta, Cm))) <= tol(oracle, K, A, B, beta, Cm)
 
 
+def test_wave_tile_ragged_tall_matrix(prism, oracle):
+    """A ragged A of more than 4 GiB: the bytes from a tile's first row to the end of A do not fit the 32 bits
+    of a buffer descriptor's extent and are cut to 2 GiB - 1 (a tile only reaches 256 rows ahead). Rows are
+    sampled from the first and last tiles and from the tile whose remaining byte count is smallest modulo
+    2^32, where an extent that wrapped around instead would zero-fill rows that exist."""
+    M, N, K = 1_100_003, 260, 1000
+    g = torch.Generator(device=DEV)
+    g.manual_seed(1)
+    A = torch.rand((M, K), dtype=torch.float32, device=DEV, generator=g) * 2 - 1
+    B = torch.rand((K, N), dtype=torch.float32, device=DEV, generator=g) * 2 - 1
+    C = torch.full((M, N), 3.0, dtype=torch.float32, device=DEV)
+    prism.sgemm(M, N, K, 1.0, A, B, 0.0, C, variant=5)
+    torch.cuda.synchronize()
+    left = [(M - 256 * t) * K * 4 for t in range((M + 255) // 256)]
+    worst = min((t for t in range(len(left)) if left[t] >= 2**32), key=lambda t: left[t] % 2**32)
+    assert left[worst] % 2**32 < 256 * K * 4  # a wrapped extent would end inside this tile
+    rows = np.unique(np.concatenate([np.arange(0, 256, 37), np.arange(worst * 256, worst * 256 + 256, 5),
+                                     np.arange(M - 300, M, 7)]))
+    it = torch.from_numpy(rows).to(DEV)
+    want = A[it].cpu().numpy().astype(np.float64) @ B.cpu().numpy().astype(np.float64)
+    got = C[it].cpu().numpy()
+    assert np.max(np.abs(got - want)) <= 1e-5 * np.sqrt(K)
+
+
 def _sampled_check(prism, oracle, M, N, K, alpha, beta, variant, rows=48):
     """Full-size run, checked on `rows` random rows against an fp64 product."""
     g = torch.Generator(device=DEV)
