@@ -92,6 +92,16 @@ int prism_scan_i32(const int32_t* in, int32_t* out, size_t n, void* workspace,
                    size_t workspace_bytes, void* stream);
 
 /*
+ * Exclusive prefix sum, out[i] = in[0] + ... + in[i-1] modulo 2^32, out[0] = 0: the same single-pass
+ * kernel with a different write-back stage (the stage of update_with_new_data_and_writeback,
+ * examples/scan.py:174-193). Arguments, workspace and aliasing rules as for prism_scan_i32. The
+ * reference's harness only times inclusive sums (evals/4090_scan/bench.cu:96-116); this form is what
+ * callers that turn counts into offsets need.
+ */
+int prism_scan_exclusive_i32(const int32_t* in, int32_t* out, size_t n, void* workspace,
+                             size_t workspace_bytes, void* stream);
+
+/*
  * The reference launcher's own shape: in-place on x, default stream, returns
  * the device pointer that holds the result (x) or NULL on failure.
  * Replaces scan_gpu::launch_scan (evals/4090_scan/main.cu:68-86). Unlike the

@@ -39,6 +39,8 @@ def lib() -> C.CDLL:
         L.oracle_add_m.restype = None
         L.oracle_scan_cpu.argtypes = [sz, vp, vp]
         L.oracle_scan_cpu.restype = None
+        L.oracle_scan_exclusive_cpu.argtypes = [sz, vp, vp]
+        L.oracle_scan_exclusive_cpu.restype = None
         L.oracle_scan_lookback.argtypes = [sz, vp, C.c_uint]
         L.oracle_scan_lookback.restype = sz
         L.oracle_sgemm_fma.argtypes = [C.c_int, C.c_int, C.c_int, f32, vp, vp, f32, vp]
@@ -90,6 +92,15 @@ def scan_cpu(x: np.ndarray) -> np.ndarray:
     xu = _c(x, dt).view(np.uint32)
     out = np.empty_like(xu)
     lib().oracle_scan_cpu(xu.size, _p(xu), _p(out))
+    return out.view(dt)
+
+
+def scan_exclusive_cpu(x: np.ndarray) -> np.ndarray:
+    """Serial uint32 exclusive scan: out[0] = 0, out[i] = x[0] + ... + x[i-1]."""
+    dt = x.dtype
+    xu = _c(x, dt).view(np.uint32)
+    out = np.empty_like(xu)
+    lib().oracle_scan_exclusive_cpu(xu.size, _p(xu), _p(out))
     return out.view(dt)
 
 

@@ -14,6 +14,7 @@
  *   oracle_add_m            closed form y = x + m on hand-computed wrap cases; numpy int32 add
  *   oracle_scan_cpu         closed forms (all-ones -> i+1, wrap cases), numpy.cumsum(int32),
  *                           difference invariant out[i]-out[i-1] == x[i]
+ *   oracle_scan_exclusive_cpu  closed forms (all-ones -> i, wrap), inclusive[i] - x[i], shifted numpy.cumsum
  *   oracle_scan_lookback    equality with oracle_scan_cpu on the reference's own test sizes
  *                           and distribution; tail beyond the last full block left untouched
  *   oracle_sgemm_fma        brute-force exact rational/fp64 check on small integer-valued
@@ -47,6 +48,18 @@ void oracle_scan_cpu(size_t n, const uint32_t* x, uint32_t* out) {
     for (size_t i = 0; i < n; i++) {
         accumulator = accumulator + x[i];
         out[i] = accumulator;
+    }
+}
+
+/* Exclusive form of the loop above (same accumulator, written before it takes the element in):
+ * out[0] = 0, out[i] = x[0] + ... + x[i-1]. No reference counterpart; it is the serial definition
+ * the exclusive entry point of the library is checked against. */
+void oracle_scan_exclusive_cpu(size_t n, const uint32_t* x, uint32_t* out) {
+    uint32_t accumulator = 0;
+    for (size_t i = 0; i < n; i++) {
+        const uint32_t element = x[i];  /* x may be out */
+        out[i] = accumulator;
+        accumulator = accumulator + element;
     }
 }
 

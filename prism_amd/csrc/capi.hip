@@ -60,11 +60,17 @@ size_t prism_scan_workspace_bytes(size_t n) { return scan_workspace_bytes(n); }
 int prism_scan_i32(const int32_t* in, int32_t* out, size_t n, void* workspace,
                    size_t workspace_bytes, void* stream) {
     return launch_scan(reinterpret_cast<const uint32_t*>(in), reinterpret_cast<uint32_t*>(out), n,
-                       workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+                       workspace, workspace_bytes, false, static_cast<hipStream_t>(stream));
+}
+
+int prism_scan_exclusive_i32(const int32_t* in, int32_t* out, size_t n, void* workspace,
+                             size_t workspace_bytes, void* stream) {
+    return launch_scan(reinterpret_cast<const uint32_t*>(in), reinterpret_cast<uint32_t*>(out), n,
+                       workspace, workspace_bytes, true, static_cast<hipStream_t>(stream));
 }
 
 uint32_t* prism_launch_scan(size_t n, uint32_t* x, void* workspace) {
-    int rc = launch_scan(x, x, n, workspace, scan_workspace_bytes(n), nullptr);
+    int rc = launch_scan(x, x, n, workspace, scan_workspace_bytes(n), false, nullptr);
     return rc == 0 ? x : nullptr;
 }
 

@@ -58,6 +58,7 @@
 // traffic is 8 B per tile plus the polls.
 #include <cstdlib>
 #include <cstring>
+#include <type_traits>
 
 #include "common.h"
 
@@ -169,7 +170,9 @@ __device__ __forceinline__ uint32_t look_back(const u64* status, uint32_t tile, 
 
 // VEC: in and out are 16 B aligned, full tiles use 16 B accesses.
 // TICKET: tiles are numbered by the ticket counter, else by workgroup id.
-template <typename Cfg, bool VEC, bool TICKET>
+// EXCLUSIVE: out[i] is the sum of the elements before i (out[0] = 0) instead of up to and including i;
+// only the write-back differs.
+template <typename Cfg, bool VEC, bool TICKET, bool EXCLUSIVE>
 __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_t* in, uint32_t* out,
                                                                    size_t n, uint32_t* header,
                                                                    u64* status, uint32_t spin_limit) {
@@ -275,7 +278,9 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
     if (full) {
 #pragma unroll
         for (int j = 0; j < VPT; ++j) {
-            const u32x4 r = v[j] + (offset[j] + base_sum);
+            // v[j] holds the running sums inside the packet; shifted by one element they are the exclusive ones.
+            const u32x4 sums = EXCLUSIVE ? u32x4{0u, v[j].x, v[j].y, v[j].z} : v[j];
+            const u32x4 r = sums + (offset[j] + base_sum);
             __builtin_nontemporal_store(r, reinterpret_cast<u32x4*>(out + lane_base + j * ROW_ELEMS));
         }
     } else {
@@ -285,7 +290,7 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const size_t i = lane_base + j * ROW_ELEMS + c;
-                if (i < n) out[i] = v[j][c] + add;
+                if (i < n) out[i] = (EXCLUSIVE ? (c ? v[j][c - 1] : 0u) : v[j][c]) + add;
             }
         }
     }
@@ -317,19 +322,26 @@ inline uint32_t spin_limit() {
     return v != nullptr ? static_cast<uint32_t>(strtoul(v, nullptr, 10)) : kSpinLimit;
 }
 
+// Calls f with std::true_type or std::false_type for a run-time flag.
+template <typename F>
+void with_flag(bool flag, F&& f) {
+    if (flag) f(std::true_type{});
+    else f(std::false_type{});
+}
+
 template <typename Cfg>
 int launch_cfg(const uint32_t* in, uint32_t* out, size_t n, uint32_t* header, u64* status, size_t tiles,
-               hipStream_t s) {
+               bool exclusive, hipStream_t s) {
     const dim3 grid(static_cast<unsigned>(tiles)), block(Cfg::BLOCK);
-    const bool vec = aligned16(in) && aligned16(out);
     const uint32_t limit = spin_limit();
-    if (ticket_order()) {
-        if (vec) scan_lookback_kernel<Cfg, true, true><<<grid, block, 0, s>>>(in, out, n, header, status, limit);
-        else scan_lookback_kernel<Cfg, false, true><<<grid, block, 0, s>>>(in, out, n, header, status, limit);
-    } else {
-        if (vec) scan_lookback_kernel<Cfg, true, false><<<grid, block, 0, s>>>(in, out, n, header, status, limit);
-        else scan_lookback_kernel<Cfg, false, false><<<grid, block, 0, s>>>(in, out, n, header, status, limit);
-    }
+    with_flag(aligned16(in) && aligned16(out), [&](auto vec) {
+        with_flag(ticket_order(), [&](auto ticket) {
+            with_flag(exclusive, [&](auto excl) {
+                scan_lookback_kernel<Cfg, decltype(vec)::value, decltype(ticket)::value, decltype(excl)::value>
+                    <<<grid, block, 0, s>>>(in, out, n, header, status, limit);
+            });
+        });
+    });
     return check_launch("scan_lookback_kernel");
 }
 
@@ -340,7 +352,7 @@ size_t scan_workspace_bytes(size_t n) {
     return kHeaderBytes + sizeof(u64) * (tiles > 0 ? tiles : 1);
 }
 
-int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes,
+int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, bool exclusive,
                 hipStream_t s) {
     if (n == 0) return 0;
     if (in == nullptr || out == nullptr || ws == nullptr)
@@ -370,8 +382,8 @@ int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws
         words, n_words);
     if (int rc = check_launch("scan_reset_kernel")) return rc;
 
-    if (use_small(n)) return launch_cfg<SmallCfg>(in, out, n, ticket, status, tiles, s);
-    return launch_cfg<BigCfg>(in, out, n, ticket, status, tiles, s);
+    if (use_small(n)) return launch_cfg<SmallCfg>(in, out, n, ticket, status, tiles, exclusive, s);
+    return launch_cfg<BigCfg>(in, out, n, ticket, status, tiles, exclusive, s);
 }
 
 }  // namespace prism

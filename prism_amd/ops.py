@@ -106,8 +106,9 @@ def launch_scan(n: int, x: "torch.Tensor", workspace: "torch.Tensor") -> "torch.
 
 
 def scan(inp: "torch.Tensor", out: Optional["torch.Tensor"] = None,
-         workspace: Optional["torch.Tensor"] = None) -> "torch.Tensor":
-    """Inclusive prefix sum modulo 2^32 of a 1-D int32/uint32 tensor; out may be inp."""
+         workspace: Optional["torch.Tensor"] = None, exclusive: bool = False) -> "torch.Tensor":
+    """Prefix sum modulo 2^32 of a 1-D int32/uint32 tensor; out may be inp. Inclusive (out[i] includes
+    inp[i]) unless exclusive=True (out[0] = 0, out[i] = inp[0] + ... + inp[i-1])."""
     _need(inp, (torch.int32, torch.uint32), 0, "inp")
     n = inp.numel()
     if out is None:
@@ -117,7 +118,8 @@ def scan(inp: "torch.Tensor", out: Optional["torch.Tensor"] = None,
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=inp.device)
     ws_bytes = workspace.numel() * workspace.element_size()
-    _check(_lib.load().prism_scan_i32(_ptr(inp), _ptr(out), n, _ptr(workspace), ws_bytes, _stream()), "scan")
+    fn = _lib.load().prism_scan_exclusive_i32 if exclusive else _lib.load().prism_scan_i32
+    _check(fn(_ptr(inp), _ptr(out), n, _ptr(workspace), ws_bytes, _stream()), "scan")
     return out
 
 

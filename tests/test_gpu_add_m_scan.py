@@ -88,6 +88,27 @@ def test_scan_tile_boundaries(prism, oracle, n):
     assert np.all(got[n:] == -7)
 
 
+@pytest.mark.parametrize("n", [1, 2, 255, 256, 257, 4096, 16385, 65536, 65537, 100_003, (1 << 24) - 1, (1 << 24) + 65536 * 3 + 5,
+                               1 << 26])
+def test_exclusive_scan(prism, oracle, n):
+    """The exclusive form (out[0] = 0, out[i] = in[0] + ... + in[i-1]) on both tile shapes, out of place with a
+    fenced output and in place; and exclusive + element == inclusive, element for element."""
+    x = oracle.gen_scan(n, seed=n + 1)
+    want = oracle.scan_exclusive_cpu(x)
+    out = torch.full((n + 8,), -7, dtype=torch.int32, device=DEV)
+    xd = dev(x)
+    prism.scan(xd, out[:n], exclusive=True)
+    got = host(out)
+    assert np.array_equal(got[:n], want) and np.all(got[n:] == -7)
+    assert np.array_equal(got[:n].view(np.uint32) + x.view(np.uint32), host(prism.scan(xd)).view(np.uint32))
+    prism.scan(xd, xd, exclusive=True)
+    assert np.array_equal(host(xd), want)
+    if n >= 256:  # only 4 B aligned views take the scalar path
+        y = torch.zeros(n + 1, dtype=torch.int32, device=DEV)
+        prism.scan(dev(np.concatenate([[0], x]).astype(np.int32))[1:], y[1:], exclusive=True)
+        assert np.array_equal(host(y)[1:], want)
+
+
 @pytest.mark.parametrize("n", [16384, 32768, 1 << 20, 1 << 24, 1 << 26])
 def test_scan_reference_test_sizes_inplace(prism, oracle, n):
     """The reference's own correctness sizes and distribution (evals/4090_scan/main.cu:97-109),

@@ -55,6 +55,21 @@ def test_scan_wraps_like_uint32(oracle):
     assert oracle.scan_cpu(np.array([-5], dtype=np.int32)).tolist() == [-5]
 
 
+def test_exclusive_scan_closed_forms_and_relation_to_inclusive(oracle):
+    ones = np.ones(70_000, dtype=np.int32)
+    assert np.array_equal(oracle.scan_exclusive_cpu(ones), np.arange(0, 70_000, dtype=np.int32))
+    x = np.full(6, 2**31 - 1, dtype=np.int32)  # wraps at the third element
+    assert oracle.scan_exclusive_cpu(x).view(np.uint32).tolist() == [((2**31 - 1) * i) % 2**32 for i in range(6)]
+    assert oracle.scan_exclusive_cpu(np.array([], dtype=np.int32)).size == 0
+    assert oracle.scan_exclusive_cpu(np.array([-5], dtype=np.int32)).tolist() == [0]
+    for n in (1, 2, 63, 64, 65, 4097, 100_003):
+        x = oracle.gen_scan(n, seed=n)
+        ex = oracle.scan_exclusive_cpu(x)
+        inc = np.cumsum(x, dtype=np.int32)
+        assert ex[0] == 0 and np.array_equal(ex[1:], inc[:-1])                        # shifted inclusive sums
+        assert np.array_equal(ex.view(np.uint32) + x.view(np.uint32), inc.view(np.uint32))  # exclusive + element
+
+
 def test_scan_vs_numpy_cumsum_and_difference_invariant(oracle):
     for n in (1, 63, 64, 65, 4095, 4096, 4097, 16384, 100_003):
         x = oracle.gen_scan(n, seed=n)
