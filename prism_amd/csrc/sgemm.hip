@@ -17,13 +17,18 @@
 // sub-tiles with v_mfma_f32_32x32x2_f32 instead of per-thread outer products;
 // its summation order inside the matrix unit is not specified, so it is
 // checked against an fp64 product within a tolerance. It comes in three forms,
-// chosen by the launcher from the tile count: the general 128 x 128 block kernel
-// (any shape), a 256 x 256 direct-to-LDS kernel for problems made of whole tiles
-// that fill the chip, and a one-wave-per-tile kernel for small problems.
+// chosen by the launcher from the tile count: a 256 x 256 direct-to-LDS kernel
+// for problems with enough such tiles to fill the chip, a one-wave-per-tile
+// kernel for small problems and for the tiles of a partial last round of the
+// big kernel, and the general 128 x 128 block kernel for what lies in between.
+// The two direct-to-LDS kernels have edge variants for ragged M, N, K with N and K
+// multiples of 4 (16 B-aligned rows): their loads go through buffer descriptors
+// whose range check zero-fills everything beyond the matrices. Other shapes and
+// alignments take the general kernel, whose edge variant uses range-checked
+// 16 B buffer loads plus masks.
 //
 // Unlike the reference kernels (no guards in kernels 1, 3, 4, 5), every kernel
-// here accepts any M, N, K: full tiles take a guard-free path, edge tiles a
-// predicated one. When beta == 0, C is not read.
+// here accepts any M, N, K. When beta == 0, C is not read.
 #include "common.h"
 #include "direct_load.h"
 #include "tile_map.h"
