@@ -4,7 +4,8 @@
 // This is the gfx950 counterpart of the reference's Hopper kernel
 // (examples/h100_matmul.py:20-297, generated/cutlass_my_h100_match_no_tail.cu):
 //   reference                                   here
-//   wgmma m64n256k16 from swizzled smem     ->  v_mfma_f32_32x32x16_bf16, 4 waves x 128x128, swizzled LDS
+//   wgmma m64n256k16 from swizzled smem     ->  v_mfma_f32_16x16x32_bf16 (32x32x16 in the small-tile and
+//                                               general kernels), 4 waves x 128x128, swizzled LDS
 //   TMA bulk copies + mbarrier ring (4 x)   ->  buffer loads into two register sets two K tiles ahead,
 //                                               two LDS stages (gemm_bf16_staged_kernel); odd or
 //                                               small K tile counts: direct-to-LDS loads, ring of two
@@ -56,6 +57,7 @@ namespace {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // fp32 -> bf16, round to nearest even; NaN stays NaN (quiet bit forced).
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
@@ -742,6 +744,233 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
     }
 }
 
+// ------------------------------ register-staged pipeline, 16x16x32 matrix instructions --
+// The same pipeline (two LDS stages, two register sets, tile t+3 loaded while tile t is multiplied,
+// LDS-only barriers, the edge handling) around v_mfma_f32_16x16x32_bf16 instead of 32x32x16. Both forms
+// have the same peak rate; on random operands, where the chip is power-limited, a register-only loop
+// of the 16x16x32 form sustains 2.04 PFLOP/s against 1.82 for 32x32x16 (2.47 / 2.50 on all-zero
+// operands), so the same schedule runs at a higher clock.
+//
+// Operand layout of the instruction: lane l supplies P[row l % 16][k = 8 (l / 16) .. + 7] and
+// Q[col l % 16][same k] (one 16 B chunk each, 32 k values per instruction over the four lane
+// groups); result register v of lane l is OUT[4 (l / 16) + v][l % 16]. A wave's 128 x 128 tile is
+// 8 x 8 such sub-tiles (64 accumulators of 4 registers). A K tile of 64 is two k-steps of 32; a k-step
+// is eight "rows" of eight instructions (one P fragment against the eight Q fragments).
+//
+// Fragments: the eight Q fragments of a k-step are double-buffered by k-step parity; the eight P
+// fragments of a k-step have one register slot per row, and the fragment of row i of the next k-step
+// is read four rows after row i of the current one has been issued. The last four rows of a tile
+// are issued after the barrier that ends its phase, from fragments read before it; behind them go the
+// first reads of the next tile (four P fragments, all eight Q fragments of its first k-step), so that
+// no read is needed sooner than about 200 clocks after it is issued: with 48 LDS instructions of
+// 1 KiB per wave and K tile the LDS pipeline of a CU is busy three quarters of the time, and a design
+// with 128 clocks of slack ran its matrix pipe only 73 % of the cycles. Behind the instructions of
+// every row: one P read (j = 0), one LDS write of a staged packet (j = 2), one Q read for the next
+// k-step (j = 4; after a barrier three per row, j odd), one global load (j = 6).
+//
+// The matrix instruction is issued from inline assembly with the accumulator as a read-write operand:
+// written with the builtin, the compiler gave result and addend different registers, and with all 256
+// accumulation registers taken by the 64 accumulators that meant moving them around in every
+// iteration (hundreds of copies and spills). The compiler does not know the instruction's result
+// latency then; the only place a result is read soon after it is produced is the write-back, which
+// therefore waits first (mfma_results_settle).
+__device__ __forceinline__ void mfma_16x16x32_in_place(f32x4& c, bf16x8 a, bf16x8 b) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_results_settle() {
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+}
+
+template <int BM, int BN, int WM, int WN, bool EDGE, typename OutT>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_staged16_kernel(
+    int R, int Cn, int K, const uint16_t* __restrict__ P, const uint16_t* __restrict__ Q,
+    OutT* __restrict__ OUT, int tiles_m, int tiles_n) {
+    constexpr int BK = 64, KP = 8, SWZ = 1;
+    constexpr int WAVES_N = BN / WN;
+    constexpr int WAVES = (BM / WM) * WAVES_N;
+    constexpr int MI = WM / 16, NI = WN / 16;
+    static_assert(MI == 8 && NI == 8, "the row schedule below is written for 128 x 128 wave tiles");
+    constexpr int ROWS_PER_LOAD = kWave / KP;
+    constexpr int ROWS_PER_PASS = ROWS_PER_LOAD * WAVES;
+    static_assert(BM % ROWS_PER_PASS == 0 && BN % ROWS_PER_PASS == 0, "whole load passes");
+    constexpr int P_PER = BM / ROWS_PER_PASS, Q_PER = BN / ROWS_PER_PASS;
+    constexpr int PACKETS = P_PER + Q_PER;
+    static_assert(PACKETS == 16, "one LDS write and one global load per row of a phase");
+
+    __shared__ __attribute__((aligned(1024))) uint16_t Ps[2][BM * BK];
+    __shared__ __attribute__((aligned(1024))) uint16_t Qs[2][BN * BK];
+
+    int tm, tn;
+    xcd_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+    const int row0 = tm * BM, col0 = tn * BN;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+    const int l16 = lane & 15, lq = lane >> 4;
+
+    f32x4 acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // Global and LDS-write side: as in gemm_bf16_staged_kernel.
+    const int ld_row = wave * ROWS_PER_LOAD + lane / KP;
+    const int ld_chunk = (lane % KP) ^ ((ld_row >> SWZ) & (KP - 1));
+    const uint32_t lane_off = (static_cast<uint32_t>(lane / KP) * static_cast<uint32_t>(K) + ld_chunk * 8) * 2u;
+    constexpr uint32_t kBeyond = 0x80000000u;
+    auto extent = [&](int first_row, int rows) -> int {
+        if (!EDGE) return 0x7fffffff;
+        return static_cast<int>(clamped_extent(static_cast<long long>(rows - first_row) * K * 2));
+    };
+    const int p_first = row0 + wave * ROWS_PER_LOAD, q_first = col0 + wave * ROWS_PER_LOAD;
+    const auto p_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(P + (EDGE && p_first >= R ? size_t{0} : static_cast<size_t>(p_first) * K)), 0,
+        extent(p_first, R), 0x00020000);
+    const auto q_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(Q + (EDGE && q_first >= Cn ? size_t{0} : static_cast<size_t>(q_first) * K)), 0,
+        extent(q_first, Cn), 0x00020000);
+    const int pass_bytes = ROWS_PER_PASS * K * 2;
+    const int k_full = K - K % BK;
+    const int k_end = EDGE ? ((K + 2 * BK - 1) / (2 * BK) < 3 ? 6 * BK : (K + 2 * BK - 1) / (2 * BK) * 2 * BK) : K;
+    const uint32_t tail_off = (EDGE && k_full + ld_chunk * 8 < K) ? lane_off : kBeyond;
+    u32x4 staged[2][PACKETS];
+    auto offset_for = [&](int k0) -> uint32_t {
+        if (!EDGE) return lane_off;
+        return k0 < k_full ? lane_off : (k0 < K ? tail_off : kBeyond);
+    };
+    auto load_packet = [&](int set, int k0, int m, uint32_t off) {
+        if (m < P_PER)
+            staged[set][m] = __builtin_amdgcn_raw_buffer_load_b128(p_rsrc, off, m * pass_bytes + k0 * 2, 0);
+        else
+            staged[set][m] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, off, (m - P_PER) * pass_bytes + k0 * 2, 0);
+    };
+    auto write_packet = [&](int set, int m) {
+        uint16_t* dst = (m < P_PER) ? &Ps[set][(m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]
+                                    : &Qs[set][((m - P_PER) * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK];
+        *reinterpret_cast<u32x4*>(dst + lane * 8) = staged[set][m];
+    };
+
+    // Operand side: row (wave tile origin + 16 i + l16), chunk 4 kk + lq of the row, kept in slot
+    // chunk ^ ((row >> 1) & 7) (the row term is that of l16: 16 i is a multiple of 16).
+    const int sw = (l16 >> SWZ) & (KP - 1);
+    int p_off[2], q_off[2];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+        const int slot = (4 * kk + lq) ^ sw;
+        p_off[kk] = (wave_m * WM + l16) * BK + slot * 8;
+        q_off[kk] = (wave_n * WN + l16) * BK + slot * 8;
+    }
+    bf16x8 fp[MI], fq[2][NI];  // P fragments: one slot per row; Q fragments: by k-step parity
+    auto read_p = [&](int stage, int kk, int i) {
+        fp[i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&Ps[stage][p_off[kk] + i * 16 * BK]));
+    };
+    auto read_q = [&](int stage, int kk, int j) {
+        fq[kk][j] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&Qs[stage][q_off[kk] + j * 16 * BK]));
+    };
+    // Row i of k-step kk: eight instructions; `after(j)` is issued right behind the j-th.
+    auto mfma_row = [&](int kk, int i, auto after) {
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+            mfma_16x16x32_in_place(acc[i][j], fp[i], fq[kk][j]);
+            __builtin_amdgcn_sched_barrier(0);
+            after(j);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // One phase = everything between two barriers, for the tile in stage S (tile t). Entered right after
+    // the barrier that says "tile t is complete in stage S and nobody reads stage S^1 any more", with
+    // rows 4..7 of tile t-1's second k-step still to do (their fragments are in registers). Register set
+    // S^1 holds tile t+1: packet n is written to stage S^1 behind row n of the phase (`write`) and
+    // refilled with tile t+3, which starts at k_load (`load`).
+    auto phase = [&](auto stage_c, auto write, auto load, int k_load) {
+        constexpr int S = decltype(stage_c)::value;
+        const uint32_t off = offset_for(k_load);
+        auto staging = [&](int n, int j) {  // the LDS write and the global load of row n of the phase
+            if (j == 2) { if constexpr (write) write_packet(S ^ 1, n); }
+            if (j == 6) { if constexpr (load) load_packet(S ^ 1, k_load, n, off); }
+        };
+        // rows 4..7 of the previous tile; behind them the first reads of this tile
+#pragma unroll
+        for (int i = 4; i < 8; ++i)
+            mfma_row(1, i, [&](int j) {
+                if (j == 0) read_p(S, 0, i - 4);
+                if (j % 2 == 1 && j < 6 && 3 * (i - 4) + j / 2 < NI) read_q(S, 0, 3 * (i - 4) + j / 2);
+                staging(i - 4, j);
+            });
+        // k-step 0: rows 0..7
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            mfma_row(0, i, [&](int j) {
+                if (j == 0) { if (i < 4) read_p(S, 0, i + 4); else read_p(S, 1, i - 4); }
+                if (j == 4) read_q(S, 1, i);
+                staging(4 + i, j);
+            });
+        // k-step 1: rows 0..3 (4..7 follow the barrier)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            mfma_row(1, i, [&](int j) {
+                if (j == 0) read_p(S, 1, i + 4);
+                staging(12 + i, j);
+            });
+        lds_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    using yes = std::integral_constant<bool, true>;
+    using no = std::integral_constant<bool, false>;
+    using s0 = std::integral_constant<int, 0>;
+    using s1 = std::integral_constant<int, 1>;
+
+    // "Rows 4..7 of the tile before the first" multiply zeros.
+#pragma unroll
+    for (int i = 4; i < 8; ++i) fp[i] = bf16x8{};
+#pragma unroll
+    for (int j = 0; j < NI; ++j) fq[1][j] = bf16x8{};
+
+    // Even number of K tiles, at least 6; the first in stage 0 and the last in stage 1 (as above).
+#pragma unroll
+    for (int m = 0; m < PACKETS; ++m) load_packet(0, 0, m, offset_for(0));
+#pragma unroll
+    for (int m = 0; m < PACKETS; ++m) load_packet(1, BK, m, offset_for(BK));
+#pragma unroll
+    for (int m = 0; m < PACKETS; ++m) write_packet(0, m);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int m = 0; m < PACKETS; ++m) load_packet(0, 2 * BK, m, offset_for(2 * BK));
+    lds_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    int k_load = 3 * BK;
+    do {
+        phase(s0{}, yes{}, yes{}, k_load);
+        phase(s1{}, yes{}, yes{}, k_load + BK);
+        k_load += 2 * BK;
+    } while (k_load + BK < k_end);
+    phase(s0{}, yes{}, yes{}, k_load);
+    phase(s1{}, yes{}, no{}, 0);
+    phase(s0{}, yes{}, no{}, 0);
+    phase(s1{}, no{}, no{}, 0);
+#pragma unroll
+    for (int i = 4; i < 8; ++i) mfma_row(1, i, [](int) {});  // the last four rows of the last tile
+    mfma_results_settle();
+
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+            const int col = col0 + wave_n * WN + j * 16 + l16;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int row = row0 + wave_m * WM + i * 16 + 4 * lq + v;
+                if (!EDGE || (row < R && col < Cn))
+                    store_out(&OUT[static_cast<size_t>(row) * Cn + col], acc[i][j][v]);
+            }
+        }
+    }
+}
+
 // Kernel choice. Whole 256 x 256 x 64 tiles: the register-staged pipeline whenever the K tile count
 // is even and at least 6 (measured faster than the ring from 2048^3 up), else the direct-to-LDS ring
 // (any count from 2). Ragged M, N or K with K a multiple of 8 and 16 B-aligned operands: the staged
@@ -755,6 +984,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
 #endif
 #ifndef PRISM_BF16_LEFTOVER
 #define PRISM_BF16_LEFTOVER 1
+#endif
+#ifndef PRISM_BF16_MFMA16
+#define PRISM_BF16_MFMA16 1  // the staged pipeline on 16x16x32 instructions (0: on 32x32x16)
 #endif
 #ifndef PRISM_BF16_SMALL_TILES
 #define PRISM_BF16_SMALL_TILES 1
@@ -792,8 +1024,12 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
         const bool cut = PRISM_BF16_LEFTOVER && tiles > cus && left != 0 && left * 4 <= 2 * cus &&
                          static_cast<long long>(K) * 2 * 64 < (1ll << 32);
         const int main_tiles = cut ? tiles - left : tiles;
-        gemm_bf16_staged_kernel<BM, BN, WM, WN, false, OutT><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
-            R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
+        if (PRISM_BF16_MFMA16)
+            gemm_bf16_staged16_kernel<BM, BN, WM, WN, false, OutT><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
+                R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
+        else
+            gemm_bf16_staged_kernel<BM, BN, WM, WN, false, OutT><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
+                R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
         if (int rc = check_launch("gemm_bf16_staged_kernel")) return rc;
         if (cut) {
             gemm_bf16_ring_kernel<128, 128, 64, 2, 64, 64, false, OutT><<<dim3(static_cast<unsigned>(left) * 4), dim3(256), 0, s>>>(
@@ -820,7 +1056,10 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
     }
     // Ragged M, N or K with 16 B-aligned rows: the staged kernel with zero-filled edges.
     if (PRISM_BF16_STAGED_EDGES && aligned && K % 8 == 0 && K > 0 && panel_ok) {
-        gemm_bf16_staged_kernel<BM, BN, WM, WN, true, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
+        if (PRISM_BF16_MFMA16)
+            gemm_bf16_staged16_kernel<BM, BN, WM, WN, true, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
+        else
+            gemm_bf16_staged_kernel<BM, BN, WM, WN, true, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
         return check_launch("gemm_bf16_staged_kernel (edges)");
     }
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<BM, BN, BK, WM, WN, true, OutT>),
