@@ -43,6 +43,13 @@
 #ifndef PRISM_BF16_SCHED
 #define PRISM_BF16_SCHED 1
 #endif
+#ifndef PRISM_BF16_M16_WRITE_J
+#define PRISM_BF16_M16_WRITE_J 2  // in the 16x16x32 kernel: the instruction of a row behind which the LDS write goes
+#endif
+#ifndef PRISM_BF16_M16_LOAD_J
+#define PRISM_BF16_M16_LOAD_J 3   // ... and the global load, which must come after the write of the same packet
+                                  // (2/3, 2/6, 1/5, 3/7 all within 0.5 % of each other; 6/7 is 5 % slower at 8192^3)
+#endif
 #ifndef PRISM_BF16_MFMA_ORDER
 #define PRISM_BF16_MFMA_ORDER 2  // issue order of a group's MFMAs in the staged kernel (see mfma_group there);
                                  // 8192^3: 1431-1437 / 1434 / 1438-1442 TFLOP/s for 0 / 1 / 2
@@ -764,9 +771,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
 // first reads of the next tile (four P fragments, all eight Q fragments of its first k-step), so that
 // no read is needed sooner than about 200 clocks after it is issued: with 48 LDS instructions of
 // 1 KiB per wave and K tile the LDS pipeline of a CU is busy three quarters of the time, and a design
-// with 128 clocks of slack ran its matrix pipe only 73 % of the cycles. Behind the instructions of
-// every row: one P read (j = 0), one LDS write of a staged packet (j = 2), one Q read for the next
-// k-step (j = 4; after a barrier three per row, j odd), one global load (j = 6).
+// with 128 clocks of slack was no faster. Behind the instructions of every row: one P read (j = 0),
+// one LDS write of a staged packet (j = 2) and the global load that refills its registers (j = 3), one
+// Q read for the next k-step (j = 4; after a barrier three per row, j odd).
 //
 // The matrix instruction is issued from inline assembly with the accumulator as a read-write operand:
 // written with the builtin, the compiler gave result and addend different registers, and with all 256
@@ -796,6 +803,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
     constexpr int P_PER = BM / ROWS_PER_PASS, Q_PER = BN / ROWS_PER_PASS;
     constexpr int PACKETS = P_PER + Q_PER;
     static_assert(PACKETS == 16, "one LDS write and one global load per row of a phase");
+    static_assert(PRISM_BF16_M16_WRITE_J < PRISM_BF16_M16_LOAD_J && PRISM_BF16_M16_LOAD_J < 8, "a packet is written out before its registers are reloaded");
 
     __shared__ __attribute__((aligned(1024))) uint16_t Ps[2][BM * BK];
     __shared__ __attribute__((aligned(1024))) uint16_t Qs[2][BN * BK];
@@ -890,8 +898,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
         constexpr int S = decltype(stage_c)::value;
         const uint32_t off = offset_for(k_load);
         auto staging = [&](int n, int j) {  // the LDS write and the global load of row n of the phase
-            if (j == 2) { if constexpr (write) write_packet(S ^ 1, n); }
-            if (j == 6) { if constexpr (load) load_packet(S ^ 1, k_load, n, off); }
+            if (j == PRISM_BF16_M16_WRITE_J) { if constexpr (write) write_packet(S ^ 1, n); }
+            if (j == PRISM_BF16_M16_LOAD_J) { if constexpr (load) load_packet(S ^ 1, k_load, n, off); }
         };
         // rows 4..7 of the previous tile; behind them the first reads of this tile
 #pragma unroll
