@@ -48,7 +48,7 @@ from pathlib import Path
 from typing import Callable, Dict, List, Optional
 
 __all__ = ["prism", "requires", "attr", "grid", "block", "warp", "thread", "ptr", "const", "restrict", "constexpr",
-           "shared", "uint", "double", "uint32_t", "uint64_t", "group", "partition", "unsafe",
+           "shared", "uint", "double", "uint32_t", "uint64_t", "group", "partition", "claim", "split", "unsafe",
            "generate", "generate_launcher", "build", "HipgenError"]
 
 
@@ -141,6 +141,8 @@ def group(_where):  # only ever appears inside kernel bodies, which are parsed, 
 
 
 partition = group
+claim = group
+split = group
 unsafe = group
 
 _REGISTRY: Dict[str, "Kernel"] = {}

@@ -38,8 +38,13 @@ printed as it stands and must therefore be HIP: the counterpart of the reference
 `__shfl_up(val, delta, 32)`, which shifts within each aligned group of 32 lanes. The barrier plan
 does not look into unsafe() text.
 
-Not part of this slice, refused by name: `claim`, `split`, `f=lambda` partitions, inline PTX
-(`intrinsic`), vector casts, asynchronous copies.
+`match split(level): case n: ...` hands the first n members of a level one body and the next ones
+another (ids restart in every case; the reference's producer / consumer split,
+examples/h100_matmul.py:203-206); `claim(...)` prints like `partition(...)`. A split's cases are treated
+like the branches of an `if` by the barrier plan.
+
+Not part of this slice, refused by name: `f=lambda` partitions, inline PTX (`intrinsic`), vector
+casts, asynchronous copies.
 """
 from __future__ import annotations
 
@@ -132,11 +137,15 @@ class _SyncPlan:
             elif isinstance(s, ast.With):
                 call = s.items[0].context_expr
                 target = s.items[0].optional_vars
-                if (_is_call(call, "partition") and call.args and isinstance(call.args[0], ast.Name)
-                        and isinstance(target, ast.Name) and call.args[0].id in self.root):
+                if ((_is_call(call, "partition") or _is_call(call, "claim")) and call.args
+                        and isinstance(call.args[0], ast.Name) and isinstance(target, ast.Name)
+                        and call.args[0].id in self.root):
                     self.root[target.id] = self.root[call.args[0].id]
             for field in ("body", "orelse"):
                 self._collect(getattr(s, field, []) or [])
+            if isinstance(s, ast.Match):
+                for case in s.cases:
+                    self._collect(case.body)
 
     # read / write sets of LDS arrays
     def _reads(self, node: Optional[ast.AST]) -> Set[str]:
@@ -199,6 +208,8 @@ class _SyncPlan:
             elif isinstance(s, ast.If):
                 r |= self._reads(s.test)
                 a, b = self._whole(s.body + s.orelse)
+            elif isinstance(s, ast.Match):
+                a, b = self._whole([x for c in s.cases for x in c.body])
             else:
                 a, b = self._access(s)
             r |= a
@@ -236,16 +247,20 @@ class _SyncPlan:
                         raise HipgenError(f"{_line(s)}: a loop inside an `if` needs a barrier between its iterations")
                     self.at_end.add(id(s))
                     pr, pw = set(), set()
-            elif isinstance(s, ast.If):
+            elif isinstance(s, (ast.If, ast.Match)):
                 r, w = self._whole([s])
                 if self._hazard(r, w, (pr, pw)):
                     self._mark(s, may_sync)
                     pr, pw = set(), set()
-                # Inside the branches no barrier may be placed; hazards there are errors.
-                a = self._walk(s.body, (set(), set()), False)
-                b = self._walk(s.orelse, (set(), set()), False)
-                pr |= r | a[0] | b[0]
-                pw |= w | a[1] | b[1]
+                # Inside the branches (or the cases of a split) no barrier may be placed: not every thread
+                # gets there. Hazards inside are errors.
+                bodies = [s.body, s.orelse] if isinstance(s, ast.If) else [c.body for c in s.cases]
+                for body in bodies:
+                    a = self._walk(body, (set(), set()), False)
+                    pr |= a[0]
+                    pw |= a[1]
+                pr |= r
+                pw |= w
             else:
                 r, w = self._access(s)
                 if self._hazard(r, w, (pr, pw)):
@@ -275,7 +290,7 @@ class _SyncPlan:
             elif isinstance(s, (ast.For, ast.While)):
                 r, w = self._whole([s])
                 got = "hazard" if self._hazard(r, w, pending) else ("barrier" if id(s) in self.at_end else "none")
-            elif isinstance(s, ast.If):
+            elif isinstance(s, (ast.If, ast.Match)):
                 r, w = self._whole([s])
                 got = "hazard" if self._hazard(r, w, pending) else "none"
             else:
@@ -365,7 +380,7 @@ class BlockEmitter:
             return self.level_id(*self.id_level)
         if name == "unsafe":
             raise HipgenError(f"{_line(n)}: unsafe() is a statement")
-        if name in ("intrinsic", "float4_cast", "claim", "split"):
+        if name in ("intrinsic", "float4_cast"):
             raise HipgenError(f"{_line(n)}: {name}() is not part of this slice")
         targs = ""
         for kw in n.keywords:
@@ -392,7 +407,7 @@ class BlockEmitter:
             call = s.items[0].context_expr
             if _is_call(call, "group"):
                 return self.group(s, call)
-            if _is_call(call, "partition"):
+            if _is_call(call, "partition") or _is_call(call, "claim"):  # both are pointer arithmetic in the text
                 return self.partition(s, call, s.items[0].optional_vars)
             raise HipgenError(f"{_line(s)}: `with {getattr(call.func, 'id', '?')}(...)` is not part of this slice")
         if isinstance(s, ast.Assign) and len(s.targets) == 1:
@@ -406,6 +421,8 @@ class BlockEmitter:
             return self.body_and_close(s)
         if isinstance(s, ast.If):
             return self.branch(s)
+        if isinstance(s, ast.Match):
+            return self.split(s)
         if isinstance(s, ast.Return):
             if s.value is None:
                 # A value-returning function whose value comes from unsafe() text ends in a bare `return`
@@ -470,6 +487,46 @@ class BlockEmitter:
                 self.indent -= 1
                 rest = []
         self.emit("}")
+
+    def split(self, s: ast.Match) -> None:
+        """`match split(level): case n: ... case m: ...` gives the first n members of the level one body, the
+        next m another, ...; inside a case ids restart at 0 (prism/codegen.py:936-993)."""
+        if not (_is_call(s.subject, "split") and len(s.subject.args) == 1 and isinstance(s.subject.args[0], ast.Name)
+                and s.subject.args[0].id in _LEVELS):
+            raise HipgenError(f"{_line(s)}: expected `match split(block)` or `match split(thread)`")
+        level = s.subject.args[0].id
+        outer, before = self.ids, 0
+        for case in s.cases:
+            pat = case.pattern
+            if not (isinstance(pat, ast.MatchValue) and isinstance(pat.value, ast.Constant)
+                    and isinstance(pat.value.value, int) and pat.value.value > 0) or case.guard is not None:
+                raise HipgenError(f"{_line(case.pattern)}: a case of split() is a positive member count")
+            count = pat.value.value
+            inner = _Ids(f"__block_id_{outer.depth + 1}", f"__thread_id_{outer.depth + 1}", outer.depth + 1)
+            shift = f" - {before}" if before else ""
+            self.open()
+            if level == "block":
+                self.emit(f"int {inner.block_id} = {outer.block_id}{shift};")
+                self.emit(f"int {inner.thread_id} = {inner.block_id} * blockDim.x + threadIdx.x;")
+                self.emit(f"if ({inner.block_id} >= 0 && {inner.block_id} < {count}) {{")
+            elif level == "thread":
+                self.emit(f"int {inner.block_id} = {outer.block_id};")
+                self.emit(f"int {inner.thread_id} = {outer.thread_id}{shift};")
+                self.emit(f"if ({inner.thread_id} >= 0 && {inner.thread_id} < {count}) {{")
+            else:
+                self.emit(f"int {inner.block_id} = {outer.block_id};")
+                self.emit(f"int {inner.thread_id} = {outer.thread_id};")
+                self.emit("if (true) {")
+            self.indent += 1
+            saved_level, self.id_level = self.id_level, (level, 1)
+            self.ids = inner
+            self.block(case.body)
+            self.ids = outer
+            self.id_level = saved_level
+            self.indent -= 1
+            self.emit("}")
+            self.close()
+            before += count
 
     def declare(self, s: ast.AnnAssign) -> None:
         name = s.target.id

@@ -16,7 +16,7 @@ import pytest
 
 from prism_amd import hipgen
 from prism_amd.hipgen import (HipgenError, attr, block, const, generate, generate_launcher, grid, group, partition,
-                              prism, ptr, requires, shared, thread, uint32_t, unsafe)
+                              prism, ptr, requires, shared, split, thread, uint32_t, unsafe)
 from prism_amd.hipgen_blocks import dynamic_lds_bytes
 
 
@@ -151,6 +151,36 @@ def hazard_in_branch(x: ptr(float) @ grid[1]):
             x[t] = buf[31 - t]
 
 
+@requires(grid[1], block[1], thread[1])
+@prism("global")
+def two_roles(x: ptr(const(int)) @ grid[1], y: ptr(int) @ grid[1], n: int @ grid[1]):
+    """The first 128 threads of a block double their element, the next 128 add one to theirs (the shape of
+    the reference's producer / consumer split, examples/h100_matmul.py:203-206)."""
+    base: int @ block[1] = id() * 256
+    with group(block[1]):
+        match split(thread):
+            case 128:
+                t: int @ thread[1] = id()
+                if base + t < n:
+                    y[base + t] = x[base + t] * 2
+            case 128:
+                t: int @ thread[1] = id()
+                if base + 128 + t < n:
+                    y[base + 128 + t] = x[base + 128 + t] + 1
+
+
+@requires(grid[1], block[1], thread[1])
+@prism("global")
+def split_with_hazard(x: ptr(float) @ grid[1]):
+    with group(block[1]):
+        buf: shared(float[256], static=True) @ block[1]
+        match split(thread):
+            case 128:
+                t: int @ thread[1] = id()
+                buf[t] = x[t]
+                x[t] = buf[127 - t]
+
+
 @requires(grid[1], block[1], thread[48])
 @prism("global")
 def straddling_groups(x: ptr(float) @ grid[1]):
@@ -274,6 +304,18 @@ def test_device_function_gets_the_callers_ids():
     assert launcher.index("__device__ float scaled_sum(") < launcher.index("__global__ void scaled_sum_all(")
 
 
+def test_split_restarts_ids_in_every_case():
+    got = lines(generate("two_roles"))
+    i = got.index("int __thread_id_2 = __thread_id_1;")
+    assert got[i - 1] == "int __block_id_2 = __block_id_1;"
+    assert got[i + 1] == "if (__thread_id_2 >= 0 && __thread_id_2 < 128) {" and got[i + 2] == "int t = __thread_id_2;"
+    k = got.index("int __thread_id_2 = __thread_id_1 - 128;")
+    assert got[k + 1] == "if (__thread_id_2 >= 0 && __thread_id_2 < 128) {" and k > i
+    assert "y[((base + 128) + t)] = (x[((base + 128) + t)] + 1);" in got
+    with pytest.raises(HipgenError, match="inside one `if`"):
+        generate("split_with_hazard")  # a barrier inside a case would not be reached by the other threads
+
+
 def test_refusals_name_the_construct():
     with pytest.raises(HipgenError, match="inside one `if`"):
         generate("hazard_in_branch")
@@ -297,7 +339,7 @@ def test_thread_groups_of_32_and_target_text():
     assert "uint32_t got = lane_shift_up(__block_id_3, __thread_id_3, __smem, v, step);" in got
 
 
-BUILDS = {"row_scan32": (256, None), "add_m_blocks": (256, None), "naive_sgemm": (256, None), "tiled_sgemm": (1024, [32]),
+BUILDS = {"two_roles": (256, None), "row_scan32": (256, None), "add_m_blocks": (256, None), "naive_sgemm": (256, None), "tiled_sgemm": (1024, [32]),
           "thread_tile_sgemm": (256, [64, 64, 8, 4, 4]), "scaled_sum_all": (256, None)}
 
 
@@ -388,6 +430,22 @@ def test_generated_row_scan_on_half_wavefronts(built, rows):
     y = yd.cpu().numpy().view(np.uint32)
     assert np.array_equal(y[:rows * 32].reshape(rows, 32), np.cumsum(x, axis=1, dtype=np.uint32))
     assert np.all(y[rows * 32:] == 0xFFFFFFFF)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n", [1, 128, 129, 256, 1000])
+def test_generated_split_runs_both_roles(built, n):
+    import torch
+    fn = built["two_roles"].two_roles_launch
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_uint, ctypes.c_void_p]
+    x = np.random.default_rng(n).integers(-1000, 1000, n, dtype=np.int32)
+    xd = torch.from_numpy(x).to("cuda:0")
+    yd = torch.full((n + 4,), -1, dtype=torch.int32, device="cuda:0")
+    assert fn(xd.data_ptr(), yd.data_ptr(), n, (n + 255) // 256, None) == 0
+    torch.cuda.synchronize()
+    first_role = (np.arange(n) % 256) < 128
+    y = yd.cpu().numpy()
+    assert np.array_equal(y[:n], np.where(first_role, x * 2, x + 1)) and np.all(y[n:] == -1)
 
 
 @pytest.mark.gpu
