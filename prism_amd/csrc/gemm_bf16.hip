@@ -7,9 +7,11 @@
 //   wgmma m64n256k16 from swizzled smem     ->  v_mfma_f32_16x16x32_bf16 (32x32x16 in the small-tile and
 //                                               general kernels), 4 waves x 128x128, swizzled LDS
 //   TMA bulk copies + mbarrier ring (4 x)   ->  buffer loads into two register sets two K tiles ahead,
-//                                               two LDS stages (gemm_bf16_staged_kernel); odd or
-//                                               small K tile counts: direct-to-LDS loads, ring of two
-//                                               stages (gemm_bf16_ring_kernel)
+//                                               two LDS stages (gemm_bf16_staged16_kernel, _staged_kernel);
+//                                               odd or small K tile counts: direct-to-LDS loads, ring of
+//                                               two stages (gemm_bf16_ring_kernel); selectable:
+//                                               direct-to-LDS loads with the stage freed in mid-phase
+//                                               (gemm_bf16_early_kernel)
 //   1 producer + 2 consumer warpgroups      ->  every wave loads and multiplies
 //   persistent CTAs + 16x8 super-tiles      ->  one workgroup per tile, 16x16 super-blocks with an
 //                                               8x4 patch per XCD (tile_map.h)
@@ -33,6 +35,8 @@
 //
 // In gemm_bf16_kernel LDS rows are BK + 8 elements (144 B for BK = 64): eight lanes
 // reading 16 B from eight consecutive rows then cover all banks exactly once.
+#include <cstdlib>
+#include <cstring>
 #include <type_traits>
 
 #include "common.h"
@@ -49,6 +53,10 @@
 #ifndef PRISM_BF16_M16_LOAD_J
 #define PRISM_BF16_M16_LOAD_J 3   // ... and the global load, which must come after the write of the same packet
                                   // (2/3, 2/6, 1/5, 3/7 all within 0.5 % of each other; 6/7 is 5 % slower at 8192^3)
+#endif
+#ifndef PRISM_BF16_EARLY_LOAD_GAP
+#define PRISM_BF16_EARLY_LOAD_GAP 4  // matrix instructions between two direct loads in gemm_bf16_early_kernel
+                                     // (8192^3: 1.32-1.37 / 1.36-1.38 / 1.40-1.42 PFLOP/s for 1-2 / 3 / 4)
 #endif
 #ifndef PRISM_BF16_MFMA_ORDER
 #define PRISM_BF16_MFMA_ORDER 2  // issue order of a group's MFMAs in the staged kernel (see mfma_group there);
@@ -979,6 +987,177 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
     }
 }
 
+// ------------------------------ direct-to-LDS loads with early fragment reads, 16x16x32 --
+// Whole tiles, an even number (at least 4) of K tiles. The staged kernels above pay for their lead time
+// with 16 LDS write instructions per wave and K tile; this one has none: global data goes straight into
+// LDS (direct_load.h) as in the ring kernel, whose problem was that a stage had to be free before the
+// load into it could be issued, which left a load less than one tile time. Here all 32 fragments of a K
+// tile are read into registers behind the first 32 matrix instructions of its phase (three sets of
+// 8 + 8 fragments: k-step 0 of this tile, k-step 1 of this tile, k-step 1 of the previous tile, which is
+// what those instructions multiply), a barrier in mid-phase then says that nobody reads the stage any
+// more, and the loads of the tile after next are issued into it right away: about one and a half tile
+// times before they are needed.
+template <int BM, int BN, int WM, int WN, typename OutT>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early_kernel(
+    int R, int Cn, int K, const uint16_t* __restrict__ P, const uint16_t* __restrict__ Q,
+    OutT* __restrict__ OUT, int tiles_m, int tiles_n) {
+    constexpr int BK = 64, KP = 8, SWZ = 1;
+    constexpr int WAVES_N = BN / WN;
+    constexpr int WAVES = (BM / WM) * WAVES_N;
+    constexpr int MI = WM / 16, NI = WN / 16;
+    static_assert(MI == 8 && NI == 8, "written for 128 x 128 wave tiles");
+    constexpr int ROWS_PER_LOAD = kWave / KP;
+    constexpr int ROWS_PER_PASS = ROWS_PER_LOAD * WAVES;
+    constexpr int P_PER = BM / ROWS_PER_PASS, Q_PER = BN / ROWS_PER_PASS;
+    constexpr int LOADS = P_PER + Q_PER;
+    static_assert(LOADS == 16, "sixteen direct loads per wave and K tile");
+
+    __shared__ __attribute__((aligned(1024))) uint16_t Ps[2][BM * BK];
+    __shared__ __attribute__((aligned(1024))) uint16_t Qs[2][BN * BK];
+
+    int tm, tn;
+    xcd_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+    const int row0 = tm * BM, col0 = tn * BN;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+    const int l16 = lane & 15, lq = lane >> 4;
+
+    f32x4 acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // Load side, as in gemm_bf16_ring_kernel.
+    const int ld_row = wave * ROWS_PER_LOAD + lane / KP;
+    const int ld_chunk = (lane % KP) ^ ((ld_row >> SWZ) & (KP - 1));
+    const uint32_t lane_off = (static_cast<uint32_t>(lane / KP) * static_cast<uint32_t>(K) + ld_chunk * 8) * 2u;
+    const char* p_wave = reinterpret_cast<const char*>(P + static_cast<size_t>(row0 + wave * ROWS_PER_LOAD) * K);
+    const char* q_wave = reinterpret_cast<const char*>(Q + static_cast<size_t>(col0 + wave * ROWS_PER_LOAD) * K);
+    const size_t pass_bytes = static_cast<size_t>(ROWS_PER_PASS) * K * 2;
+    auto issue_load = [&](int stage, int k0, int m) {
+        if (m < P_PER)
+            direct_load16(p_wave + static_cast<size_t>(k0) * 2 + m * pass_bytes, lane_off,
+                          &Ps[stage][(m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]);
+        else
+            direct_load16(q_wave + static_cast<size_t>(k0) * 2 + (m - P_PER) * pass_bytes, lane_off,
+                          &Qs[stage][((m - P_PER) * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]);
+    };
+
+    // Operand side, as in gemm_bf16_staged16_kernel.
+    const int sw = (l16 >> SWZ) & (KP - 1);
+    int p_off[2], q_off[2];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+        const int slot = (4 * kk + lq) ^ sw;
+        p_off[kk] = (wave_m * WM + l16) * BK + slot * 8;
+        q_off[kk] = (wave_n * WN + l16) * BK + slot * 8;
+    }
+    // Fragment sets: [0] k-step 0 of the current tile; [1], [2] k-step 1 of the tiles in stage 0 / stage 1.
+    bf16x8 fp[3][MI], fq[3][NI];
+    auto read_fragment = [&](int set, int stage, int kk, int r) {  // r = 0..7: P fragment r; 8..15: Q fragment r - 8
+        if (r < MI)
+            fp[set][r] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&Ps[stage][p_off[kk] + r * 16 * BK]));
+        else
+            fq[set][r - MI] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&Qs[stage][q_off[kk] + (r - MI) * 16 * BK]));
+    };
+    // The 64 instructions of one k-step from fragment set `set`; `after(m)` is issued right behind the m-th.
+    auto mfma_block = [&](int set, auto after) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+                mfma_16x16x32_in_place(acc[i][j], fp[set][i], fq[set][j]);
+                __builtin_amdgcn_sched_barrier(0);
+                after(i * NI + j);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+    };
+
+    // One phase, for the tile in stage S (tile t). Entered right after the barrier that says "tile t is
+    // complete in stage S".
+    //   k-step 1 of tile t-1 (set 2 - S... the set of the other stage); behind its first 32 instructions the
+    //     32 fragment reads of tile t: k-step 0 into set 0, k-step 1 into the set of stage S
+    //   wait for those reads; barrier: nobody reads stage S any more
+    //   k-step 0 of tile t (set 0); behind its first instructions the direct loads of tile t+2 into stage S
+    //   wait until at most those loads are in flight (tile t+1 has landed); barrier
+    // Every phase issues its sixteen loads, the last two as well (they fetch the last two tiles once
+    // more, into stages nobody reads again): all phases are then the same straight-line code inside one
+    // loop, and the compiler keeps every accumulator in one place for the whole K loop. (With separate
+    // code for the last two phases it moved accumulators between registers right behind matrix
+    // instructions whose latency it does not know, see mfma_16x16x32_in_place, and read them too early;
+    // with the loads under a run-time condition the branches cost 5 %.)
+    auto phase = [&](auto stage_c, int k_next) {
+        constexpr int S = decltype(stage_c)::value;
+        constexpr int MINE = 1 + S, OTHER = 2 - S;  // fragment sets of k-step 1: this stage's, the other stage's
+        mfma_block(OTHER, [&](int m) {
+            if (m < 16) read_fragment(0, S, 0, m);
+            else if (m < 32) read_fragment(MINE, S, 1, m - 16);
+        });
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(kVmMax, 0));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_block(0, [&](int m) {
+            if (m % PRISM_BF16_EARLY_LOAD_GAP == 0 && m / PRISM_BF16_EARLY_LOAD_GAP < LOADS)
+                issue_load(S, k_next, m / PRISM_BF16_EARLY_LOAD_GAP);
+        });
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(LOADS, kLgkmMax));
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");  // the compiler does not know that the loads write LDS: no read moves above the barrier
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    using s0 = std::integral_constant<int, 0>;
+    using s1 = std::integral_constant<int, 1>;
+
+    // "k-step 1 of the tile before the first" multiplies zeros (set 2 is what the first phase, stage 0, uses).
+#pragma unroll
+    for (int i = 0; i < MI; ++i) fp[2][i] = bf16x8{};
+#pragma unroll
+    for (int j = 0; j < NI; ++j) fq[2][j] = bf16x8{};
+
+    // Tile t lives in stage t % 2; the launcher guarantees an even number of K tiles, at least 4.
+    const int k_tiles = K / BK;
+#pragma unroll
+    for (int m = 0; m < LOADS; ++m) issue_load(0, 0, m);
+#pragma unroll
+    for (int m = 0; m < LOADS; ++m) issue_load(1, BK, m);
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(LOADS, kLgkmMax));
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    for (int t = 0; t < k_tiles; t += 2) {
+        const int next = t + 2 < k_tiles ? t + 2 : k_tiles - 2;
+        phase(s0{}, next * BK);
+        phase(s1{}, (next + 1) * BK);
+    }
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));  // the last, redundant loads: nothing is in flight when the wave ends
+    // k-step 1 of the last tile (stage 1 -> set 2). Outside the loop the compiler is free to move accumulators
+    // to other registers; it does so between these instructions, so here they are issued through the builtin,
+    // whose result latency it knows.
+    mfma_results_settle();
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fp[2][i], fq[2][j], acc[i][j], 0, 0, 0);
+
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+            const int col = col0 + wave_n * WN + j * 16 + l16;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int row = row0 + wave_m * WM + i * 16 + 4 * lq + v;
+                store_out(&OUT[static_cast<size_t>(row) * Cn + col], acc[i][j][v]);
+            }
+        }
+    }
+}
+
 // Kernel choice. Whole 256 x 256 x 64 tiles: the register-staged pipeline whenever the K tile count
 // is even and at least 6 (measured faster than the ring from 2048^3 up), else the direct-to-LDS ring
 // (any count from 2). Ragged M, N or K with K a multiple of 8 and 16 B-aligned operands: the staged
@@ -992,6 +1171,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
 #endif
 #ifndef PRISM_BF16_LEFTOVER
 #define PRISM_BF16_LEFTOVER 1
+#endif
+#ifndef PRISM_BF16_EARLY
+#define PRISM_BF16_EARLY 0  // 1: whole-tile problems take gemm_bf16_early_kernel instead of the staged pipeline
 #endif
 #ifndef PRISM_BF16_MFMA16
 #define PRISM_BF16_MFMA16 1  // the staged pipeline on 16x16x32 instructions (0: on 32x32x16)
@@ -1008,6 +1190,21 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
 #ifndef PRISM_BF16_RING_STAGES
 #define PRISM_BF16_RING_STAGES 2
 #endif
+
+// Which of the three pipelines takes problems made of whole 256 x 256 x 64 tiles (and, for the two
+// staged ones, ragged problems): PRISM_BF16_KERNEL in the environment, read at every call.
+//   staged16 (default)  register-staged, 16x16x32 instructions
+//   staged32            register-staged, 32x32x16 instructions
+//   early               direct-to-LDS with early fragment reads, 16x16x32 instructions
+// Measured within 1 % of each other at 8192^3 (1.43-1.45 PFLOP/s under bench.py); early is 4 % ahead at
+// 4096^3, staged16 3 % ahead at 16384^3.
+inline int whole_tile_kernel() {
+    const char* v = getenv("PRISM_BF16_KERNEL");
+    if (v == nullptr) return PRISM_BF16_EARLY ? 2 : (PRISM_BF16_MFMA16 ? 1 : 0);
+    if (strcmp(v, "staged32") == 0) return 0;
+    if (strcmp(v, "early") == 0) return 2;
+    return 1;
+}
 
 template <int BM, int BN, int BK, int WM, int WN, typename OutT>
 int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, OutT* OUT,
@@ -1032,7 +1229,11 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
         const bool cut = PRISM_BF16_LEFTOVER && tiles > cus && left != 0 && left * 4 <= 2 * cus &&
                          static_cast<long long>(K) * 2 * 64 < (1ll << 32);
         const int main_tiles = cut ? tiles - left : tiles;
-        if (PRISM_BF16_MFMA16)
+        const int which = whole_tile_kernel();
+        if (which == 2 && static_cast<long long>(K) * 2 * 64 < (1ll << 32))
+            gemm_bf16_early_kernel<BM, BN, WM, WN, OutT><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
+                R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
+        else if (which != 0)
             gemm_bf16_staged16_kernel<BM, BN, WM, WN, false, OutT><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
                 R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
         else
@@ -1064,7 +1265,7 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
     }
     // Ragged M, N or K with 16 B-aligned rows: the staged kernel with zero-filled edges.
     if (PRISM_BF16_STAGED_EDGES && aligned && K % 8 == 0 && K > 0 && panel_ok) {
-        if (PRISM_BF16_MFMA16)
+        if (whole_tile_kernel() != 0)
             gemm_bf16_staged16_kernel<BM, BN, WM, WN, true, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
         else
             gemm_bf16_staged_kernel<BM, BN, WM, WN, true, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
