@@ -54,9 +54,15 @@
 #define PRISM_BF16_M16_LOAD_J 3   // ... and the global load, which must come after the write of the same packet
                                   // (2/3, 2/6, 1/5, 3/7 all within 0.5 % of each other; 6/7 is 5 % slower at 8192^3)
 #endif
+#ifndef PRISM_BF16_EARLY_BARRIER_AT
+#define PRISM_BF16_EARLY_BARRIER_AT 36  // gemm_bf16_early_kernel: instructions of a phase before the barrier that frees its stage
+#endif
 #ifndef PRISM_BF16_EARLY_LOAD_GAP
-#define PRISM_BF16_EARLY_LOAD_GAP 4  // matrix instructions between two direct loads in gemm_bf16_early_kernel
-                                     // (8192^3: 1.32-1.37 / 1.36-1.38 / 1.40-1.42 PFLOP/s for 1-2 / 3 / 4)
+#define PRISM_BF16_EARLY_LOAD_GAP 6  // matrix instructions between two direct loads in gemm_bf16_early_kernel.
+// Barrier position / gap, PFLOP/s at 8192^3 and 16384^3: 64/2 1.33-1.37, 1.32; 64/4 1.41-1.42, 1.42; 48/5 1.43-1.44,
+// 1.47; 40/5 1.44-1.45, 1.47; 36/6 1.44, 1.49 (the staged kernel in the same run: 1.38-1.42, 1.45). A wave-wide
+// 16 B load keeps the CU's vector memory path busy for 16 clocks, and the 64 loads of a K tile are half of a
+// phase's clocks: the more evenly they are spread, the less they hold up the matrix instructions behind them.
 #endif
 #ifndef PRISM_BF16_MFMA_ORDER
 #define PRISM_BF16_MFMA_ORDER 2  // issue order of a group's MFMAs in the staged kernel (see mfma_group there);
@@ -1093,17 +1099,25 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     auto phase = [&](auto stage_c, int k_next) {
         constexpr int S = decltype(stage_c)::value;
         constexpr int MINE = 1 + S, OTHER = 2 - S;  // fragment sets of k-step 1: this stage's, the other stage's
+        // Load number n goes behind instruction BARRIER_AT + n * GAP of the phase's 128 (counted from the
+        // start of the first block); the barrier that frees the stage sits behind instruction BARRIER_AT - 1.
+        constexpr int BARRIER_AT = PRISM_BF16_EARLY_BARRIER_AT, GAP = PRISM_BF16_EARLY_LOAD_GAP;
+        static_assert(BARRIER_AT >= 33 && BARRIER_AT <= 64 && BARRIER_AT + (LOADS - 1) * GAP < 128, "loads fit the phase");
+        auto maybe_load = [&](int at) {  // `at` = number of the instruction just issued, 0..127
+            if (at >= BARRIER_AT && (at - BARRIER_AT) % GAP == 0 && (at - BARRIER_AT) / GAP < LOADS)
+                issue_load(S, k_next, (at - BARRIER_AT) / GAP);
+        };
         mfma_block(OTHER, [&](int m) {
             if (m < 16) read_fragment(0, S, 0, m);
             else if (m < 32) read_fragment(MINE, S, 1, m - 16);
+            if (m == BARRIER_AT - 1) {
+                __builtin_amdgcn_s_waitcnt(waitcnt_imm(kVmMax, 0));
+                __builtin_amdgcn_s_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            maybe_load(m);
         });
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(kVmMax, 0));
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_block(0, [&](int m) {
-            if (m % PRISM_BF16_EARLY_LOAD_GAP == 0 && m / PRISM_BF16_EARLY_LOAD_GAP < LOADS)
-                issue_load(S, k_next, m / PRISM_BF16_EARLY_LOAD_GAP);
-        });
+        mfma_block(0, [&](int m) { maybe_load(64 + m); });
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(LOADS, kLgkmMax));
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");  // the compiler does not know that the loads write LDS: no read moves above the barrier
@@ -1173,7 +1187,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
 #define PRISM_BF16_LEFTOVER 1
 #endif
 #ifndef PRISM_BF16_EARLY
-#define PRISM_BF16_EARLY 0  // 1: whole-tile problems take gemm_bf16_early_kernel instead of the staged pipeline
+#define PRISM_BF16_EARLY 1  // 1: whole-tile problems take gemm_bf16_early_kernel, 0: the staged pipeline
 #endif
 #ifndef PRISM_BF16_MFMA16
 #define PRISM_BF16_MFMA16 1  // the staged pipeline on 16x16x32 instructions (0: on 32x32x16)
@@ -1191,19 +1205,20 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
 #define PRISM_BF16_RING_STAGES 2
 #endif
 
-// Which of the three pipelines takes problems made of whole 256 x 256 x 64 tiles (and, for the two
-// staged ones, ragged problems): PRISM_BF16_KERNEL in the environment, read at every call.
-//   staged16 (default)  register-staged, 16x16x32 instructions
-//   staged32            register-staged, 32x32x16 instructions
-//   early               direct-to-LDS with early fragment reads, 16x16x32 instructions
-// Measured within 1 % of each other at 8192^3 (1.43-1.45 PFLOP/s under bench.py); early is 4 % ahead at
-// 4096^3, staged16 3 % ahead at 16384^3.
+// Which of the three pipelines takes problems made of whole 256 x 256 x 64 tiles: PRISM_BF16_KERNEL in the
+// environment, read at every call.
+//   early (default)  direct-to-LDS with early fragment reads, 16x16x32 instructions
+//   staged16         register-staged, 16x16x32 instructions (also the kernel for ragged problems)
+//   staged32         register-staged, 32x32x16 instructions (then also for ragged problems)
+// Under bench.py at 8192^3, alternating on one box: early 1.43 PFLOP/s, staged16 1.39-1.41; early is also
+// 2-3 % ahead at 16384^3 and level at 4096^3.
 inline int whole_tile_kernel() {
     const char* v = getenv("PRISM_BF16_KERNEL");
     if (v == nullptr) return PRISM_BF16_EARLY ? 2 : (PRISM_BF16_MFMA16 ? 1 : 0);
     if (strcmp(v, "staged32") == 0) return 0;
+    if (strcmp(v, "staged16") == 0) return 1;
     if (strcmp(v, "early") == 0) return 2;
-    return 1;
+    return PRISM_BF16_EARLY ? 2 : (PRISM_BF16_MFMA16 ? 1 : 0);
 }
 
 template <int BM, int BN, int BK, int WM, int WN, typename OutT>
