@@ -130,6 +130,8 @@ class _TypeName:
 
 uint, double, uint32_t, uint64_t = (_TypeName(n) for n in ("uint", "double", "uint32_t", "uint64_t"))
 shared = _TypeName("shared")
+float4 = _TypeName("float4")
+float4_cast = _TypeName("float4_cast")  # float4_cast(x[i]) reads, float4_cast[x[i]] = v writes 16 bytes at &x[i]
 
 
 def ptr(t) -> CType:
@@ -144,6 +146,16 @@ partition = group
 claim = group
 split = group
 unsafe = group
+
+
+class _Intrinsics:
+    """`intrinsic.<name>(...)` statements in kernel bodies (parsed, never run)."""
+
+    def __getattr__(self, name):
+        return group
+
+
+intrinsic = _Intrinsics()
 
 _REGISTRY: Dict[str, "Kernel"] = {}
 

@@ -43,8 +43,26 @@ another (ids restart in every case; the reference's producer / consumer split,
 examples/h100_matmul.py:203-206); `claim(...)` prints like `partition(...)`. A split's cases are treated
 like the branches of an `if` by the barrier plan.
 
-Not part of this slice, refused by name: `f=lambda` partitions, inline PTX (`intrinsic`), vector
-casts, asynchronous copies.
+Vector accesses (prism/codegen.py:239-242,544-549; examples/sgemm_kernel_4.py:53-60,78-84):
+`float4_cast(a[i])` reads and `float4_cast[a[i]] = v` writes the 16 bytes at `&a[i]`
+(`reinterpret_cast<float4 *>(&a[i])[0]`, one `global_load_dwordx4` / `ds_read_b128` when the address is
+16-byte aligned, which is the kernel author's responsibility as in the reference); a `float4` variable's
+`.x .y .z .w` read and assign like scalars. The barrier plan counts the cast as an access of the array
+inside it.
+
+`with partition(a, p=..., f=lambda i: e) as v` declares no pointer: every `v[i]` is printed as `a[e(i)]`
+(prism/codegen.py:816-826,552-562), also through a chain of such views.
+
+Matrix instructions. The reference's `intrinsic.mma(a0..a3, b0, b1, c0..c3, out=[d0..d3])` prints one
+`mma.sync.aligned.m16n8k8` of inline PTX for a warp (prism/codegen.py:627-661, used by
+examples/simple_mma.py and examples/mmaTF32NaiveKernel.py). The counterparts here are wavefront-wide
+fp32 MFMAs, printed as compiler builtins:
+`intrinsic.mfma_f32_16x16x4_f32(a, b, c0, c1, c2, c3, out=[d0, d1, d2, d3])` (lane l supplies
+a = A[l % 16][l / 16] and b = B[l / 16][l % 16] of a 16 x 4 by 4 x 16 product and holds
+C[4 (l / 16) + v][l % 16] in c<v>) and `intrinsic.mfma_f32_32x32x2_f32(a, b, c0..c15, out=[d0..d15])`
+(a = A[l % 32][l / 32], b = B[l / 32][l % 32], c<v> = C[8 (v / 4) + 4 (l / 32) + v % 4][l % 32]). All 64
+lanes of the wavefront must reach the statement together. Inline PTX itself (`intrinsic.mma`,
+`intrinsic.wgmma256`) has no meaning on this target and is refused by name, like asynchronous copies.
 """
 from __future__ import annotations
 
@@ -56,8 +74,11 @@ from .hipgen import HipgenError, Kernel, _BINOPS, _CMPOPS, _REGISTRY, _UNOPS
 
 _TYPES = {"int": ("int", 4), "float": ("float", 4), "double": ("double", 8), "bool": ("bool", 1),
           "uint": ("unsigned int", 4), "unsigned": ("unsigned int", 4), "uint32_t": ("uint32_t", 4),
-          "uint64_t": ("uint64_t", 8), "void": ("void", 0)}
+          "uint64_t": ("uint64_t", 8), "float4": ("float4", 16), "void": ("void", 0)}
 _LEVELS = ("grid", "block", "thread")
+# intrinsic.<name> -> (compiler builtin, accumulator registers per lane)
+_MFMA = {"mfma_f32_16x16x4_f32": ("__builtin_amdgcn_mfma_f32_16x16x4f32", 4),
+         "mfma_f32_32x32x2_f32": ("__builtin_amdgcn_mfma_f32_32x32x2f32", 16)}
 
 
 @dataclass(frozen=True)
@@ -173,6 +194,9 @@ class _SyncPlan:
         if isinstance(s, ast.Assign):
             r, w = self._reads(s.value), set()
             for t in s.targets:
+                if (isinstance(t, ast.Subscript) and isinstance(t.value, ast.Name) and t.value.id == "float4_cast"
+                        and isinstance(t.slice, ast.Subscript)):
+                    t = t.slice  # float4_cast[a[i]] = v stores through a[i]
                 if isinstance(t, ast.Subscript) and isinstance(t.value, ast.Name) and t.value.id in self.root:
                     w.add(self.root[t.value.id])
                     r |= self._reads(t.slice)
@@ -317,6 +341,8 @@ class BlockEmitter:
         self.id_level: Optional[Tuple[str, int]] = None  # perspective `id()` resolves against
         self.returns_value = False
         self.plan: Optional[_SyncPlan] = None
+        self.views: Dict[str, Tuple[str, ast.Lambda]] = {}  # f=lambda view -> (array it indexes, the lambda)
+        self.bound: Dict[str, str] = {}                     # lambda parameter -> text of the index in hand
 
     # -- text helpers
     def emit(self, text: str) -> None:
@@ -339,7 +365,9 @@ class BlockEmitter:
                 return str(n.value)
             raise HipgenError(f"{_line(n)}: unsupported constant {n.value!r}")
         if isinstance(n, ast.Name):
-            return n.id
+            if n.id in self.views:
+                raise HipgenError(f"{_line(n)}: {n.id} is an index-mapped view; only its elements can be named")
+            return self.bound.get(n.id, n.id)
         if isinstance(n, ast.BinOp) and type(n.op) in _BINOPS:
             return f"({self.expr(n.left)} {_BINOPS[type(n.op)]} {self.expr(n.right)})"
         if isinstance(n, ast.UnaryOp) and type(n.op) in _UNOPS:
@@ -355,12 +383,27 @@ class BlockEmitter:
         if isinstance(n, ast.IfExp):
             return f"({self.expr(n.test)} ? {self.expr(n.body)} : {self.expr(n.orelse)})"
         if isinstance(n, ast.Subscript):
+            if isinstance(n.value, ast.Name) and n.value.id in self.views:
+                return self.view_element(n.value.id, self.expr(n.slice))
             return f"{self.expr(n.value)}[{self.expr(n.slice)}]"
         if isinstance(n, ast.Attribute):
             return f"{self.expr(n.value)}.{n.attr}"
         if isinstance(n, ast.Call):
             return self.call(n)
         raise HipgenError(f"{_line(n)}: unsupported expression {type(n).__name__}")
+
+    def view_element(self, view: str, index: str) -> str:
+        """`view[index]` for a view declared with f=lambda: the element of the underlying array."""
+        parent, fn = self.views[view]
+        param = fn.args.args[0].arg
+        saved = self.bound.get(param)
+        self.bound[param] = index
+        mapped = self.expr(fn.body)
+        if saved is None:
+            del self.bound[param]
+        else:
+            self.bound[param] = saved
+        return self.view_element(parent, mapped) if parent in self.views else f"{parent}[{mapped}]"
 
     def level_id(self, level: str, size: int) -> str:
         if level == "grid":
@@ -370,7 +413,8 @@ class BlockEmitter:
 
     def call(self, n: ast.Call) -> str:
         if not isinstance(n.func, ast.Name):
-            raise HipgenError(f"{_line(n)}: unsupported call (inline PTX and method calls are not part of this slice)")
+            raise HipgenError(f"{_line(n)}: unsupported call (intrinsic.<name>(...) is a statement; method calls are "
+                              "not part of this slice)")
         name = n.func.id
         if name == "id":
             if n.args:
@@ -380,8 +424,11 @@ class BlockEmitter:
             return self.level_id(*self.id_level)
         if name == "unsafe":
             raise HipgenError(f"{_line(n)}: unsafe() is a statement")
-        if name in ("intrinsic", "float4_cast"):
-            raise HipgenError(f"{_line(n)}: {name}() is not part of this slice")
+        if name == "float4_cast":
+            if len(n.args) != 1 or n.keywords or not isinstance(n.args[0], ast.Subscript):
+                raise HipgenError(f"{_line(n)}: float4_cast() takes one array element")
+            return f"reinterpret_cast<float4 *>(&{self.expr(n.args[0])})[0]"
+
         targs = ""
         for kw in n.keywords:
             if kw.arg == "template" and isinstance(kw.value, ast.List):
@@ -411,7 +458,12 @@ class BlockEmitter:
                 return self.partition(s, call, s.items[0].optional_vars)
             raise HipgenError(f"{_line(s)}: `with {getattr(call.func, 'id', '?')}(...)` is not part of this slice")
         if isinstance(s, ast.Assign) and len(s.targets) == 1:
-            return self.emit(f"{self.expr(s.targets[0])} = {self.expr(s.value)};")
+            t = s.targets[0]
+            if isinstance(t, ast.Subscript) and isinstance(t.value, ast.Name) and t.value.id == "float4_cast":
+                if not isinstance(t.slice, ast.Subscript):
+                    raise HipgenError(f"{_line(s)}: float4_cast[...] takes one array element")
+                return self.emit(f"reinterpret_cast<float4 *>(&{self.expr(t.slice)})[0] = {self.expr(s.value)};")
+            return self.emit(f"{self.expr(t)} = {self.expr(s.value)};")
         if isinstance(s, ast.AugAssign) and type(s.op) in _BINOPS:
             return self.emit(f"{self.expr(s.target)} {_BINOPS[type(s.op)]}= {self.expr(s.value)};")
         if isinstance(s, ast.For):
@@ -438,6 +490,9 @@ class BlockEmitter:
         if isinstance(s, ast.Expr):
             if isinstance(s.value, ast.Constant) and isinstance(s.value.value, str):
                 return None  # docstring
+            if (isinstance(s.value, ast.Call) and isinstance(s.value.func, ast.Attribute)
+                    and isinstance(s.value.func.value, ast.Name) and s.value.func.value.id == "intrinsic"):
+                return self.matrix_instruction(s.value)
             if _is_call(s.value, "unsafe"):
                 # Target text, printed as it stands (HIP here, where the reference's examples hold CUDA).
                 a = s.value.args
@@ -448,6 +503,26 @@ class BlockEmitter:
                 return None
             return self.emit(f"{self.expr(s.value)};")
         raise HipgenError(f"{_line(s)}: unsupported statement {type(s).__name__}")
+
+    def matrix_instruction(self, n: ast.Call) -> None:
+        name = n.func.attr
+        if name not in _MFMA:
+            raise HipgenError(f"{_line(n)}: intrinsic.{name} is not an instruction of this target "
+                              f"(available: {', '.join(sorted(_MFMA))})")
+        builtin, regs = _MFMA[name]
+        out = [kw.value for kw in n.keywords if kw.arg == "out"]
+        if (len(n.args) != 2 + regs or len(n.keywords) != 1 or len(out) != 1 or not isinstance(out[0], ast.List)
+                or len(out[0].elts) != regs):
+            raise HipgenError(f"{_line(n)}: intrinsic.{name}(a, b, c0..c{regs - 1}, out=[d0..d{regs - 1}])")
+        a, b = self.expr(n.args[0]), self.expr(n.args[1])
+        acc = ", ".join(self.expr(c) for c in n.args[2:])
+        self.open()
+        self.emit(f"typedef float __acc_t __attribute__((ext_vector_type({regs})));")
+        self.emit(f"__acc_t __acc = {{{acc}}};")
+        self.emit(f"__acc = {builtin}({a}, {b}, __acc, 0, 0, 0);")
+        for v, d in enumerate(out[0].elts):
+            self.emit(f"{self.expr(d)} = __acc[{v}];")
+        self.close()
 
     def body_and_close(self, s) -> None:
         self.indent += 1
@@ -631,16 +706,30 @@ class BlockEmitter:
         if not (isinstance(target, ast.Name) and call.args and isinstance(call.args[0], ast.Name)):
             raise HipgenError(f"{_line(s)}: expected `with partition(array, p=..., offset=...) as view`")
         kw = {k.arg: k.value for k in call.keywords}
-        if "f" in kw:
-            raise HipgenError(f"{_line(s)}: partition(f=lambda ...) is not part of this slice")
-        if not set(kw) <= {"p", "offset"}:
-            raise HipgenError(f"{_line(s)}: partition() takes p= and offset=")
+        if not set(kw) <= {"p", "offset", "f"} or ("f" in kw and "offset" in kw):
+            raise HipgenError(f"{_line(s)}: partition() takes p= and one of offset= and f=")
         if "p" in kw:
             _level(kw["p"])  # checked for shape only: the view is plain pointer arithmetic
         parent = call.args[0].id
         ctype = self.pointer_type.get(parent)
         if ctype is None:
             raise HipgenError(f"{_line(s)}: {parent} is not a pointer or array")
+        if "f" in kw:
+            fn = kw["f"]
+            if not (isinstance(fn, ast.Lambda) and len(fn.args.args) == 1 and not fn.args.defaults):
+                raise HipgenError(f"{_line(s)}: f= takes a lambda of one index")
+            if target.id in self.views or target.id in self.pointer_type:
+                raise HipgenError(f"{_line(s)}: {target.id} is already the name of an array or view")
+            # No pointer is declared: every element access goes through the index map.
+            self.views[target.id] = (parent, fn)
+            self.pointer_type[target.id] = ctype
+            self.block(s.body)
+            del self.views[target.id]
+            del self.pointer_type[target.id]
+            return
+        if parent in self.views:
+            raise HipgenError(f"{_line(s)}: {parent} is an index-mapped view; it has no address to offset "
+                              "(use f=lambda i: i + offset)")
         saved, self.id_level = self.id_level, (_level(kw["p"]) if "p" in kw else self.id_level)
         offset = self.expr(kw["offset"]) if "offset" in kw else "0"
         self.id_level = saved

@@ -3,7 +3,7 @@
 The kernels below are written in the reference's surface syntax (block and thread perspectives, views,
 LDS arrays without hand-placed barriers, templates, private arrays, a device function) in the manner of
 its examples (examples/sgemm_kernel_1.py, examples/sgemm_shared_mem_block.py, examples/sgemm_kernel_3.py,
-examples/add_m_block_thread.py, examples/function_call.py).
+examples/add_m_block_thread.py, examples/function_call.py; 16-byte accesses as in examples/sgemm_kernel_4.py).
 CPU: structure of the printed text (id chain, scopes, LDS declarations, where the barriers land), refusals
 by name, and that every launcher cross-compiles for gfx950.
 GPU: the compiled kernels run through their C launchers; add_m bit for bit against numpy, the SGEMMs
@@ -15,8 +15,8 @@ import numpy as np
 import pytest
 
 from prism_amd import hipgen
-from prism_amd.hipgen import (HipgenError, attr, block, const, generate, generate_launcher, grid, group, partition,
-                              prism, ptr, requires, shared, split, thread, uint32_t, unsafe)
+from prism_amd.hipgen import (HipgenError, attr, block, const, float4, float4_cast, generate, generate_launcher, grid,
+                              group, intrinsic, partition, prism, ptr, requires, shared, split, thread, uint32_t, unsafe)
 from prism_amd.hipgen_blocks import dynamic_lds_bytes
 
 
@@ -225,6 +225,183 @@ def row_scan32(x: ptr(const(uint32_t)) @ grid[1], y: ptr(uint32_t) @ grid[1], ro
                                     y_row[lane] = v
 
 
+@attr("__launch_bounds__((BM * BN) / (TM * TN))")
+@requires(grid[1], block[1], thread[1], smem=8192)
+@prism("global")
+def vector_tile_sgemm(M: int @ grid[1], N: int @ grid[1], K: int @ grid[1], alpha: float @ grid[1],
+                      A: ptr(float) @ grid[1], B: ptr(float) @ grid[1], beta: float @ grid[1],
+                      C: ptr(float) @ grid[1], tiles_n: int @ grid[1],
+                      template=[("BM", int), ("BN", int), ("BK", int), ("TM", int), ("TN", int)]):
+    """Thread-tile SGEMM with 16-byte global loads and stores; the A tile is stored transposed (BK x BM)
+    through an index-mapped view, so that a K slice of it is contiguous. One packet of A and one of B per
+    thread: BM * BK = BK * BN = 4 * threads."""
+    tile_r: const(int) @ block[1] = id() / tiles_n
+    tile_c: const(int) @ block[1] = id() % tiles_n
+    with partition(A, p=block[1], offset=tile_r * BM * K) as A_rows:
+        with partition(B, p=block[1], offset=tile_c * BN) as B_cols:
+            with partition(C, p=block[1], offset=tile_r * BM * N + tile_c * BN) as C_tile:
+                with group(block[1]):
+                    a_lds: shared(float[1024]) @ block[1]
+                    b_lds: shared(float[1024]) @ block[1]
+                    t: const(int) @ thread[1] = id()
+                    out_r: const(int) @ thread[1] = t / (BN / TN)
+                    out_c: const(int) @ thread[1] = t % (BN / TN)
+                    a_row: const(int) @ thread[1] = t / (BK / 4)
+                    a_quad: const(int) @ thread[1] = t % (BK / 4)
+                    b_row: const(int) @ thread[1] = t / (BN / 4)
+                    b_quad: const(int) @ thread[1] = t % (BN / 4)
+                    acc: float[64] @ thread[1] = {0}
+                    a_reg: float[8] @ thread[1] = {0}
+                    b_reg: float[8] @ thread[1] = {0}
+                    for k0 in range(0, K, BK):
+                        with partition(a_lds, p=thread[1], f=lambda e: (e % BK) * BM + e / BK) as a_by_row:
+                            with group(thread[1]):
+                                quad: float4 @ thread[1] = float4_cast(A_rows[a_row * K + k0 + a_quad * 4])
+                                a_by_row[a_row * BK + a_quad * 4] = quad.x
+                                a_by_row[a_row * BK + a_quad * 4 + 1] = quad.y
+                                a_by_row[a_row * BK + a_quad * 4 + 2] = quad.z
+                                a_by_row[a_row * BK + a_quad * 4 + 3] = quad.w
+                                float4_cast[b_lds[b_row * BN + b_quad * 4]] = \
+                                    float4_cast(B_cols[(k0 + b_row) * N + b_quad * 4])
+                                for kk in range(BK):
+                                    for i in range(TM):
+                                        a_reg[i] = a_lds[kk * BM + out_r * TM + i]
+                                    for j in range(TN):
+                                        b_reg[j] = b_lds[kk * BN + out_c * TN + j]
+                                    for i in range(TM):
+                                        for j in range(TN):
+                                            acc[i * TN + j] += a_reg[i] * b_reg[j]
+                    with group(thread[1]):
+                        for i in range(TM):
+                            for j in range(0, TN, 4):
+                                with partition(C_tile, p=thread[1], offset=(out_r * TM + i) * N + out_c * TN + j) as c4:
+                                    was: float4 @ thread[1] = float4_cast(c4[0])
+                                    was.x = alpha * acc[i * TN + j] + beta * was.x
+                                    was.y = alpha * acc[i * TN + j + 1] + beta * was.y
+                                    was.z = alpha * acc[i * TN + j + 2] + beta * was.z
+                                    was.w = alpha * acc[i * TN + j + 3] + beta * was.w
+                                    float4_cast[c4[0]] = was
+
+
+@requires(grid[1], block[1], thread[1])
+@prism("global")
+def gather_columns(x: ptr(const(int)) @ grid[1], y: ptr(int) @ grid[1], rows: int @ grid[1], cols: int @ grid[1]):
+    """y = x transposed, written through two stacked index-mapped views: `column` picks every cols-th element
+    starting at the thread's column, `shifted` skips its first element; thread c writes column c."""
+    c: int @ thread[1] = id()
+    with partition(x, p=thread[1], f=lambda r: r * cols + c) as column:
+        with partition(column, p=thread[1], f=lambda r: r + 1) as shifted:
+            with partition(y, p=thread[1], offset=c * rows) as mine:
+                with group(block[1]):
+                    with group(thread[1]):
+                        if c < cols:
+                            mine[0] = column[0]
+                            for r in range(rows - 1):
+                                mine[r + 1] = shifted[r]
+
+
+@requires(grid[1], block[1], thread[1])
+@prism("global")
+def view_without_address(x: ptr(int) @ grid[1]):
+    with partition(x, p=thread[1], f=lambda i: 2 * i) as evens:
+        with partition(evens, p=thread[1], offset=4) as later:
+            later[0] = 1
+
+
+@requires(thread[1])
+@prism("device")
+def lane_load(src: ptr(const(int)) @ thread[1], dst: ptr(int) @ thread[1], items: int @ thread[1]):
+    with group(thread[1]):
+        for i in range(items):
+            dst[i] = src[i]
+
+
+@requires(thread[1])
+@prism("device")
+def lane_store(src: ptr(const(int)) @ thread[1], dst: ptr(int) @ thread[1], items: int @ thread[1]):
+    with group(thread[1]):
+        for i in range(items):
+            dst[i] = src[i]
+
+
+@requires(thread[64])
+@prism("device")
+def wave_load(src: ptr(const(int)) @ thread[64], dst: ptr(int) @ thread[1], items: int @ thread[64]):
+    """Blocked arrangement: lane l of the wavefront takes items l * items .. l * items + items - 1 of the
+    wavefront's range (the reference's warp_load, examples/warp_load.py:13-22, on 64 lanes)."""
+    with group(thread[64]):
+        lane: int @ thread[1] = id()
+        with partition(src, p=thread[1], offset=lane * items) as mine:
+            with group(thread[1]):
+                lane_load(mine, dst, items)
+
+
+@requires(thread[64])
+@prism("device")
+def wave_store(src: ptr(const(int)) @ thread[1], dst: ptr(int) @ thread[64], items: int @ thread[64]):
+    with group(thread[64]):
+        lane: int @ thread[1] = id()
+        with partition(dst, p=thread[1], offset=lane * items) as mine:
+            with group(thread[1]):
+                lane_store(src, mine, items)
+
+
+@requires(grid[1], block[1], thread[64])
+@prism("global")
+def add_m_by_wavefronts(x: ptr(const(int)) @ grid[1], y: ptr(int) @ grid[1], m: int @ grid[1], wavefronts: int @ grid[1]):
+    """Every wavefront loads 64 x 4 consecutive elements into registers, adds m and stores them."""
+    w: int @ thread[64] = id()
+    with partition(x, p=thread[64], offset=w * 256) as x_wave:
+        with partition(y, p=thread[64], offset=w * 256) as y_wave:
+            with group(block[1]):
+                with group(thread[64]):
+                    held: int[4] @ thread[1]
+                    if w < wavefronts:
+                        wave_load(x_wave, held, 4)
+                        for i in range(4):
+                            held[i] += m
+                        wave_store(held, y_wave, 4)
+
+
+@requires(grid[1], block[1], thread[64])
+@prism("global")
+def one_mfma_per_wavefront(A: ptr(const(float)) @ grid[1], B: ptr(const(float)) @ grid[1], C: ptr(float) @ grid[1],
+                           M: int @ grid[1], N: int @ grid[1], K: int @ grid[1]):
+    """C = A B with one wavefront per 16 x 16 tile of C and one 16x16x4 fp32 MFMA per K step of 4, operands
+    straight from global memory (the teaching kernel of examples/mmaTF32NaiveKernel.py:14-85, for whole tiles)."""
+    tiles_n: const(int) @ grid[1] = N / 16
+    w: const(int) @ thread[64] = id()
+    tile_r: const(int) @ thread[64] = w / tiles_n
+    tile_c: const(int) @ thread[64] = w % tiles_n
+    with partition(A, p=thread[64], offset=tile_r * 16 * K) as A_rows:
+        with partition(B, p=thread[64], offset=tile_c * 16) as B_cols:
+            with partition(C, p=thread[64], offset=tile_r * 16 * N + tile_c * 16) as C_tile:
+                with group(block[1]):
+                    with group(thread[64]):
+                        lane: const(int) @ thread[1] = id()
+                        r: const(int) @ thread[1] = lane % 16
+                        q: const(int) @ thread[1] = lane / 16
+                        c0: float @ thread[1] = 0
+                        c1: float @ thread[1] = 0
+                        c2: float @ thread[1] = 0
+                        c3: float @ thread[1] = 0
+                        if w < (M / 16) * tiles_n:
+                            for k0 in range(0, K, 4):
+                                intrinsic.mfma_f32_16x16x4_f32(A_rows[r * K + k0 + q], B_cols[(k0 + q) * N + r],
+                                                               c0, c1, c2, c3, out=[c0, c1, c2, c3])
+                            C_tile[(4 * q + 0) * N + r] = c0
+                            C_tile[(4 * q + 1) * N + r] = c1
+                            C_tile[(4 * q + 2) * N + r] = c2
+                            C_tile[(4 * q + 3) * N + r] = c3
+
+
+@requires(grid[1], block[1], thread[64])
+@prism("global")
+def foreign_instruction(x: ptr(float) @ grid[1]):
+    a: float @ thread[1] = 0
+    intrinsic.mma(a, a, a, a, a, a, a, a, a, a, out=[a, a, a, a])
+
+
 def lines(text):
     return [ln.strip() for ln in text.splitlines()]
 
@@ -293,6 +470,57 @@ def test_dynamic_lds_windows_private_arrays_and_attr():
         generate_launcher("thread_tile_sgemm", block_size=256)
 
 
+def test_vector_casts_and_index_mapped_views():
+    got = lines(generate("vector_tile_sgemm"))
+    assert "float4 quad = reinterpret_cast<float4 *>(&A_rows[(((a_row * K) + k0) + (a_quad * 4))])[0];" in got
+    # the view declares no pointer; its elements are elements of a_lds at the mapped index
+    assert not any("a_by_row" in ln for ln in got)
+    e = "(((a_row * BK) + (a_quad * 4)) + 1)"
+    assert f"a_lds[((({e} % BK) * BM) + ({e} / BK))] = quad.y;" in got
+    assert ("reinterpret_cast<float4 *>(&b_lds[((b_row * BN) + (b_quad * 4))])[0] = "
+            "reinterpret_cast<float4 *>(&B_cols[(((k0 + b_row) * N) + (b_quad * 4))])[0];") in got
+    assert "float4 was = reinterpret_cast<float4 *>(&c4[0])[0];" in got
+    assert "was.w = ((alpha * acc[(((i * TN) + j) + 3)]) + (beta * was.w));" in got
+    assert "reinterpret_cast<float4 *>(&c4[0])[0] = was;" in got
+    # stores through the cast and through the view count as writes of the LDS arrays: a barrier between them
+    # and the loop that reads the tiles, and one before the next K step overwrites them
+    assert got.count("__syncthreads();") == 2
+    first = got.index("__syncthreads();")
+    assert got[first + 1] == "for (int kk = 0; kk < BK; kk++) {"
+    assert got[first - 1].startswith("reinterpret_cast<float4 *>(&b_lds[")
+    chain = lines(generate("gather_columns"))
+    assert "mine[0] = x[((0 * cols) + c)];" in chain
+    assert "mine[(r + 1)] = x[(((r + 1) * cols) + c)];" in chain
+    with pytest.raises(HipgenError, match="no address to offset"):
+        generate("view_without_address")
+
+
+def test_wavefront_load_and_store_primitives():
+    got = lines(generate("wave_load"))
+    assert got[0] == "__device__ void wave_load(int __block_id, int __thread_id, char* __smem, const int* src, int* dst, int items) {"
+    i = got.index("int __thread_id_1 = __thread_id_0 % 64;")
+    assert got[i + 1] == "int lane = __thread_id_1;"
+    assert "const int* mine = src + ((lane * items));" in got
+    assert "lane_load(__block_id_2, __thread_id_2, __smem, mine, dst, items);" in got
+    caller = lines(generate("add_m_by_wavefronts"))
+    assert "int w = (__thread_id_0 / 64);" in caller and "int held[4];" in caller
+    launcher = generate_launcher("add_m_by_wavefronts")
+    order = [launcher.index(f"void {name}(") for name in ("lane_load", "wave_load", "add_m_by_wavefronts")]
+    assert order == sorted(order)  # callees are defined before their callers
+
+
+def test_matrix_instruction_statement():
+    got = lines(generate("one_mfma_per_wavefront"))
+    i = got.index("typedef float __acc_t __attribute__((ext_vector_type(4)));")
+    assert got[i + 1] == "__acc_t __acc = {c0, c1, c2, c3};"
+    assert got[i + 2] == ("__acc = __builtin_amdgcn_mfma_f32_16x16x4f32(A_rows[(((r * K) + k0) + q)], "
+                          "B_cols[(((k0 + q) * N) + r)], __acc, 0, 0, 0);")
+    assert got[i + 3:i + 7] == [f"c{v} = __acc[{v}];" for v in range(4)]
+    assert "const int w = (__thread_id_0 / 64);" in got
+    with pytest.raises(HipgenError, match="intrinsic.mma is not an instruction of this target"):
+        generate("foreign_instruction")
+
+
 def test_device_function_gets_the_callers_ids():
     helper = lines(generate("scaled_sum"))
     assert helper[0] == "__device__ float scaled_sum(int __block_id, int __thread_id, char* __smem, float a, float b, float s) {"
@@ -340,7 +568,9 @@ def test_thread_groups_of_32_and_target_text():
 
 
 BUILDS = {"two_roles": (256, None), "row_scan32": (256, None), "add_m_blocks": (256, None), "naive_sgemm": (256, None), "tiled_sgemm": (1024, [32]),
-          "thread_tile_sgemm": (256, [64, 64, 8, 4, 4]), "scaled_sum_all": (256, None)}
+          "thread_tile_sgemm": (256, [64, 64, 8, 4, 4]), "scaled_sum_all": (256, None),
+          "vector_tile_sgemm": (256, [128, 128, 8, 8, 8]), "gather_columns": (256, None),
+          "add_m_by_wavefronts": (256, None), "one_mfma_per_wavefront": (256, None)}
 
 
 @pytest.fixture(scope="module")
@@ -460,3 +690,63 @@ def test_generated_kernel_calls_its_device_function(built):
     assert fn(xd.data_ptr(), yd.data_ptr(), 0.25, n, (n + 255) // 256, None) == 0
     torch.cuda.synchronize()
     assert np.array_equal(yd.cpu().numpy(), np.float32(0.25) * (x + y))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(128, 128, 8), (256, 384, 72), (384, 128, 256)])
+def test_generated_vector_tile_sgemm(built, oracle, shape):
+    """16-byte loads of A and B, a transposed A tile behind an index-mapped view, 16-byte read-modify-write of C."""
+    M, N, K = shape
+    run_sgemm(built["vector_tile_sgemm"], "vector_tile_sgemm", oracle, M, N, K, N // 128, (M // 128) * (N // 128))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(1, 1), (7, 300), (33, 256), (50, 1000)])
+def test_generated_stacked_views_transpose(built, shape):
+    import torch
+    rows, cols = shape
+    fn = built["gather_columns"].gather_columns_launch
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_uint, ctypes.c_void_p]
+    x = np.random.default_rng(rows * cols).integers(-2**31, 2**31 - 1, (rows, cols), dtype=np.int32)
+    xd = torch.from_numpy(x).to("cuda:0")
+    yd = torch.full((rows * cols + 8,), -5, dtype=torch.int32, device="cuda:0")
+    assert fn(xd.data_ptr(), yd.data_ptr(), rows, cols, (cols + 255) // 256, None) == 0
+    torch.cuda.synchronize()
+    y = yd.cpu().numpy()
+    assert np.array_equal(y[:rows * cols].reshape(cols, rows), x.T) and np.all(y[rows * cols:] == -5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("wavefronts", [1, 4, 5, 1000])
+def test_generated_wavefront_load_store(built, wavefronts):
+    import torch
+    fn = built["add_m_by_wavefronts"].add_m_by_wavefronts_launch
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_uint, ctypes.c_void_p]
+    n = wavefronts * 256
+    x = np.random.default_rng(wavefronts).integers(-2**30, 2**30, n, dtype=np.int32)
+    xd = torch.from_numpy(x).to("cuda:0")
+    yd = torch.full((n + 8,), -5, dtype=torch.int32, device="cuda:0")
+    assert fn(xd.data_ptr(), yd.data_ptr(), 7, wavefronts, (wavefronts + 3) // 4, None) == 0
+    torch.cuda.synchronize()
+    y = yd.cpu().numpy()
+    assert np.array_equal(y[:n], x + np.int32(7)) and np.all(y[n:] == -5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(16, 16, 4), (48, 80, 36), (256, 128, 512)])
+def test_generated_one_mfma_per_wavefront(built, oracle, shape):
+    import torch
+    M, N, K = shape
+    fn = built["one_mfma_per_wavefront"].one_mfma_per_wavefront_launch
+    fn.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int] * 3 + [ctypes.c_uint, ctypes.c_void_p]
+    A, B, _ = oracle.gen_sgemm(M, N, K, seed=M + K)
+    a, b = torch.from_numpy(A).to("cuda:0"), torch.from_numpy(B).to("cuda:0")
+    buf = torch.full((M * N + 128,), 777.0, dtype=torch.float32, device="cuda:0")
+    c = buf[64:64 + M * N]
+    tiles = (M // 16) * (N // 16)
+    assert fn(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, (tiles + 3) // 4, None) == 0
+    torch.cuda.synchronize()
+    out = buf.cpu().numpy()
+    assert np.all(out[:64] == 777.0) and np.all(out[64 + M * N:] == 777.0)
+    want = oracle.np_sgemm_f64(1.0, A, B, 0.0, np.zeros((M, N), np.float32))
+    assert np.max(np.abs(out[64:64 + M * N].reshape(M, N) - want)) <= oracle.sgemm_tolerance(K, A, B)
