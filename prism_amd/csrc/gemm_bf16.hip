@@ -1043,14 +1043,27 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     const uint32_t lane_off = (static_cast<uint32_t>(lane / KP) * static_cast<uint32_t>(K) + ld_chunk * 8) * 2u;
     const char* p_wave = reinterpret_cast<const char*>(P + static_cast<size_t>(row0 + wave * ROWS_PER_LOAD) * K);
     const char* q_wave = reinterpret_cast<const char*>(Q + static_cast<size_t>(col0 + wave * ROWS_PER_LOAD) * K);
-    const size_t pass_bytes = static_cast<size_t>(ROWS_PER_PASS) * K * 2;
-    auto issue_load = [&](int stage, int k0, int m) {
+    // The loads go through two buffer descriptors (this wave's first P row, its first Q row) for their
+    // addressing mode, not for range checks: descriptor base + scalar offset + lane offset, where the scalar
+    // offset (load number x rows per pass) and the lane offset are loop-invariant and only the two bases
+    // move along K. With one 64-bit scalar base per load instead, the compiler keeps 32 pointers as
+    // induction variables: some 90 scalar additions and a dozen reloads of spilled scalar registers in one
+    // run at the head of every iteration, with the matrix pipe idle behind them.
+    const uint32_t pass_bytes = static_cast<uint32_t>(ROWS_PER_PASS) * static_cast<uint32_t>(K) * 2u;  // the launcher keeps BM * K * 2 below 2^31
+    const i32x4 p_rsrc = buffer_descriptor(p_wave, 0x7fffffffu);
+    const i32x4 q_rsrc = buffer_descriptor(q_wave, 0x7fffffffu);
+    auto advanced = [](i32x4 d, uint32_t bytes) {  // the descriptor with its base moved up
+        const uint64_t a = ((static_cast<uint64_t>(static_cast<uint32_t>(d[1])) << 32) | static_cast<uint32_t>(d[0])) + bytes;
+        d[0] = static_cast<int>(a & 0xffffffffu);
+        d[1] = static_cast<int>(a >> 32);
+        return d;
+    };
+    auto issue_load = [&](int stage, const i32x4& pd, const i32x4& qd, int m) {
         if (m < P_PER)
-            direct_load16(p_wave + static_cast<size_t>(k0) * 2 + m * pass_bytes, lane_off,
-                          &Ps[stage][(m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]);
+            direct_load16_buffer(pd, lane_off, m * pass_bytes, &Ps[stage][(m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]);
         else
-            direct_load16(q_wave + static_cast<size_t>(k0) * 2 + (m - P_PER) * pass_bytes, lane_off,
-                          &Qs[stage][((m - P_PER) * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]);
+            direct_load16_buffer(qd, lane_off, (m - P_PER) * pass_bytes,
+                                 &Qs[stage][((m - P_PER) * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]);
     };
 
     // Operand side, as in gemm_bf16_staged16_kernel.
@@ -1096,16 +1109,17 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     // code for the last two phases it moved accumulators between registers right behind matrix
     // instructions whose latency it does not know, see mfma_16x16x32_in_place, and read them too early;
     // with the loads under a run-time condition the branches cost 5 %.)
-    auto phase = [&](auto stage_c, int k_next) {
+    auto phase = [&](auto stage_c, uint32_t k_next_bytes) {
         constexpr int S = decltype(stage_c)::value;
         constexpr int MINE = 1 + S, OTHER = 2 - S;  // fragment sets of k-step 1: this stage's, the other stage's
         // Load number n goes behind instruction BARRIER_AT + n * GAP of the phase's 128 (counted from the
         // start of the first block); the barrier that frees the stage sits behind instruction BARRIER_AT - 1.
         constexpr int BARRIER_AT = PRISM_BF16_EARLY_BARRIER_AT, GAP = PRISM_BF16_EARLY_LOAD_GAP;
         static_assert(BARRIER_AT >= 33 && BARRIER_AT <= 64 && BARRIER_AT + (LOADS - 1) * GAP < 128, "loads fit the phase");
+        const i32x4 pd = advanced(p_rsrc, k_next_bytes), qd = advanced(q_rsrc, k_next_bytes);
         auto maybe_load = [&](int at) {  // `at` = number of the instruction just issued, 0..127
             if (at >= BARRIER_AT && (at - BARRIER_AT) % GAP == 0 && (at - BARRIER_AT) / GAP < LOADS)
-                issue_load(S, k_next, (at - BARRIER_AT) / GAP);
+                issue_load(S, pd, qd, (at - BARRIER_AT) / GAP);
         };
         mfma_block(OTHER, [&](int m) {
             if (m < 16) read_fragment(0, S, 0, m);
@@ -1135,17 +1149,20 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     // Tile t lives in stage t % 2; the launcher guarantees an even number of K tiles, at least 4.
     const int k_tiles = K / BK;
 #pragma unroll
-    for (int m = 0; m < LOADS; ++m) issue_load(0, 0, m);
+    for (int m = 0; m < LOADS; ++m) issue_load(0, p_rsrc, q_rsrc, m);
+    {
+        const i32x4 pd = advanced(p_rsrc, BK * 2), qd = advanced(q_rsrc, BK * 2);
 #pragma unroll
-    for (int m = 0; m < LOADS; ++m) issue_load(1, BK, m);
+        for (int m = 0; m < LOADS; ++m) issue_load(1, pd, qd, m);
+    }
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(LOADS, kLgkmMax));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     for (int t = 0; t < k_tiles; t += 2) {
         const int next = t + 2 < k_tiles ? t + 2 : k_tiles - 2;
-        phase(s0{}, next * BK);
-        phase(s1{}, (next + 1) * BK);
+        phase(s0{}, static_cast<uint32_t>(next) * (BK * 2));
+        phase(s1{}, static_cast<uint32_t>(next + 1) * (BK * 2));
     }
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));  // the last, redundant loads: nothing is in flight when the wave ends
     // k-step 1 of the last tile (stage 1 -> set 2). Outside the loop the compiler is free to move accumulators
