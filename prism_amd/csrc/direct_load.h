@@ -71,6 +71,27 @@ __device__ __forceinline__ void direct_load16_buffer(i32x4 rsrc, uint32_t lane_o
 #pragma clang diagnostic pop
 }
 
+// The same load in two parts, for loops in which matrix instructions run back to back: M0 is written
+// one matrix instruction ahead of the load that reads it. Measured with one wave per SIMD between
+// independent 16-clock MFMAs: `s_mov m0; s_nop 0; buffer_load ... lds` in one place holds the next MFMA
+// up by 10 clocks (6 for the global_load_lds form), the M0 write alone by none, and the load alone,
+// with M0 written one MFMA earlier (which is also the wait state the load needs), by none at six
+// instructions between loads and 1 clock at four. Nothing else may write M0 between the two parts: the
+// compiler has no use for M0 in these loops (no indexed register access, no spills); the callers'
+// kernels are checked for that in the generated code.
+__device__ __forceinline__ void set_direct_load_destination(const void* lds_dst) {
+    const uint32_t lds_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+        (const __attribute__((address_space(3))) void*)lds_dst));
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+    asm volatile("s_mov_b32 m0, %0" : : "s"(lds_addr) : "memory", "m0");
+#pragma clang diagnostic pop
+}
+__device__ __forceinline__ void direct_load16_buffer_to_destination(i32x4 rsrc, uint32_t lane_offset, uint32_t scalar_offset) {
+    scalar_offset = __builtin_amdgcn_readfirstlane(scalar_offset);
+    asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(lane_offset), "s"(rsrc), "s"(scalar_offset) : "memory");
+}
+
 // s_waitcnt immediate (gfx9 encoding): at most `vm` vector-memory and `lgkm`
 // LDS/scalar operations outstanding; vmcnt[3:0] in bits 3:0 and vmcnt[5:4] in bits
 // 15:14, lgkmcnt in bits 11:8, the export counter left at its maximum.

@@ -1020,7 +1020,6 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
 
     __shared__ __attribute__((aligned(1024))) uint16_t Ps[2][BM * BK];
     __shared__ __attribute__((aligned(1024))) uint16_t Qs[2][BN * BK];
-
     int tm, tn;
     xcd_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
     const int row0 = tm * BM, col0 = tn * BN;
@@ -1057,6 +1056,16 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
         d[0] = static_cast<int>(a & 0xffffffffu);
         d[1] = static_cast<int>(a >> 32);
         return d;
+    };
+    // The two parts of a load in the K loop: the LDS destination goes into M0 one matrix instruction
+    // before the load is issued (see set_direct_load_destination).
+    auto aim_load = [&](int stage, int m) {
+        set_direct_load_destination(m < P_PER ? &Ps[stage][(m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]
+                                              : &Qs[stage][((m - P_PER) * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]);
+    };
+    auto fire_load = [&](const i32x4& pd, const i32x4& qd, int m) {
+        if (m < P_PER) direct_load16_buffer_to_destination(pd, lane_off, m * pass_bytes);
+        else direct_load16_buffer_to_destination(qd, lane_off, (m - P_PER) * pass_bytes);
     };
     auto issue_load = [&](int stage, const i32x4& pd, const i32x4& qd, int m) {
         if (m < P_PER)
@@ -1118,8 +1127,10 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
         static_assert(BARRIER_AT >= 33 && BARRIER_AT <= 64 && BARRIER_AT + (LOADS - 1) * GAP < 128, "loads fit the phase");
         const i32x4 pd = advanced(p_rsrc, k_next_bytes), qd = advanced(q_rsrc, k_next_bytes);
         auto maybe_load = [&](int at) {  // `at` = number of the instruction just issued, 0..127
+            if (at + 1 >= BARRIER_AT && (at + 1 - BARRIER_AT) % GAP == 0 && (at + 1 - BARRIER_AT) / GAP < LOADS)
+                aim_load(S, (at + 1 - BARRIER_AT) / GAP);
             if (at >= BARRIER_AT && (at - BARRIER_AT) % GAP == 0 && (at - BARRIER_AT) / GAP < LOADS)
-                issue_load(S, pd, qd, (at - BARRIER_AT) / GAP);
+                fire_load(pd, qd, (at - BARRIER_AT) / GAP);
         };
         mfma_block(OTHER, [&](int m) {
             if (m < 16) read_fragment(0, S, 0, m);
@@ -1164,7 +1175,6 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
         phase(s0{}, static_cast<uint32_t>(next) * (BK * 2));
         phase(s1{}, static_cast<uint32_t>(next + 1) * (BK * 2));
     }
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));  // the last, redundant loads: nothing is in flight when the wave ends
     // k-step 1 of the last tile (stage 1 -> set 2). Outside the loop the compiler is free to move accumulators
     // to other registers; it does so between these instructions, so here they are issued through the builtin,
     // whose result latency it knows.
@@ -1174,7 +1184,6 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
 #pragma unroll
         for (int j = 0; j < NI; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fp[2][i], fq[2][j], acc[i][j], 0, 0, 0);
-
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
 #pragma unroll
@@ -1187,6 +1196,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
             }
         }
     }
+    // The last, redundant loads write LDS: they must have landed before the wave ends and its LDS goes to
+    // the next workgroup. Behind the write-back the wait is covered by the stores.
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));
 }
 
 // Kernel choice. Whole 256 x 256 x 64 tiles: the register-staged pipeline whenever the K tile count
