@@ -56,8 +56,17 @@ __device__ __forceinline__ i32x4 buffer_descriptor(const void* base, uint32_t ex
     d[3] = 0x00020000;
     return d;
 }
+// A descriptor is wave-uniform by contract; said explicitly, dword by dword, because the operand must be a
+// tuple of scalar registers (a descriptor that went through 64-bit arithmetic may otherwise be handed over in
+// vector registers, which does not assemble). No instruction results when the value is scalar already.
+__device__ __forceinline__ i32x4 scalar_descriptor(i32x4 d) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) d[c] = __builtin_amdgcn_readfirstlane(d[c]);
+    return d;
+}
 __device__ __forceinline__ void direct_load16_buffer(i32x4 rsrc, uint32_t lane_offset, uint32_t scalar_offset,
                                                      const void* lds_dst) {
+    rsrc = scalar_descriptor(rsrc);
     const uint32_t lds_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
         (const __attribute__((address_space(3))) void*)lds_dst));
     // Wave-uniform by contract; said explicitly because the operand must be a scalar register.
@@ -89,6 +98,7 @@ __device__ __forceinline__ void set_direct_load_destination(const void* lds_dst)
 }
 __device__ __forceinline__ void direct_load16_buffer_to_destination(i32x4 rsrc, uint32_t lane_offset, uint32_t scalar_offset) {
     scalar_offset = __builtin_amdgcn_readfirstlane(scalar_offset);
+    rsrc = scalar_descriptor(rsrc);
     asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(lane_offset), "s"(rsrc), "s"(scalar_offset) : "memory");
 }
 

@@ -6,17 +6,18 @@
 //   reference                                   here
 //   wgmma m64n256k16 from swizzled smem     ->  v_mfma_f32_16x16x32_bf16 (32x32x16 in the small-tile and
 //                                               general kernels), 4 waves x 128x128, swizzled LDS
-//   TMA bulk copies + mbarrier ring (4 x)   ->  buffer loads into two register sets two K tiles ahead,
-//                                               two LDS stages (gemm_bf16_staged16_kernel, _staged_kernel);
-//                                               odd or small K tile counts: direct-to-LDS loads, ring of
-//                                               two stages (gemm_bf16_ring_kernel); selectable:
-//                                               direct-to-LDS loads with the stage freed in mid-phase
-//                                               (gemm_bf16_early_kernel)
+//   TMA bulk copies + mbarrier ring (4 x)   ->  direct-to-LDS loads two K tiles ahead into two LDS stages,
+//                                               a stage freed in mid-phase once its fragments are in
+//                                               registers (gemm_bf16_early_kernel); odd or small K tile
+//                                               counts: direct-to-LDS ring of two stages
+//                                               (gemm_bf16_ring_kernel); selectable: buffer loads into two
+//                                               register sets two K tiles ahead, written to LDS by the
+//                                               waves (gemm_bf16_staged16_kernel, _staged_kernel)
 //   1 producer + 2 consumer warpgroups      ->  every wave loads and multiplies
 //   persistent CTAs + 16x8 super-tiles      ->  one workgroup per tile, 16x16 super-blocks with an
 //                                               8x4 patch per XCD (tile_map.h)
 //   K tail dropped, M/N multiples required  ->  any M, N, K. Ragged M, N, K with K a multiple of 8
-//                                               (16 B-aligned rows): the staged kernel, edges zero-filled
+//                                               (16 B-aligned rows): the same kernels, edges zero-filled
 //                                               by the buffer loads' range check. Anything else (K not a
 //                                               multiple of 8, operands not 16 B aligned):
 //                                               gemm_bf16_kernel (guarded loads, 16 B where a packet
@@ -1003,7 +1004,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
 // what those instructions multiply), a barrier in mid-phase then says that nobody reads the stage any
 // more, and the loads of the tile after next are issued into it right away: about one and a half tile
 // times before they are needed.
-template <int BM, int BN, int WM, int WN, typename OutT>
+template <int BM, int BN, int WM, int WN, bool EDGE, typename OutT>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early_kernel(
     int R, int Cn, int K, const uint16_t* __restrict__ P, const uint16_t* __restrict__ Q,
     OutT* __restrict__ OUT, int tiles_m, int tiles_n) {
@@ -1048,14 +1049,36 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     // move along K. With one 64-bit scalar base per load instead, the compiler keeps 32 pointers as
     // induction variables: some 90 scalar additions and a dozen reloads of spilled scalar registers in one
     // run at the head of every iteration, with the matrix pipe idle behind them.
+    //
+    // EDGE: R, Cn, K need not be whole tiles (K a multiple of 8, operands 16 B aligned). Then the range check
+    // is used as well: the descriptors' extents end with the matrices, so rows beyond them arrive as zeros
+    // (a descriptor whose base moves up by some bytes loses as many from its extent); what follows a row's
+    // last column is the next row, so in the partial K tile lanes with k >= K use an offset beyond any
+    // extent, and in the K tiles that pad the count to an even number of at least 4 all lanes do.
     const uint32_t pass_bytes = static_cast<uint32_t>(ROWS_PER_PASS) * static_cast<uint32_t>(K) * 2u;  // the launcher keeps BM * K * 2 below 2^31
-    const i32x4 p_rsrc = buffer_descriptor(p_wave, 0x7fffffffu);
-    const i32x4 q_rsrc = buffer_descriptor(q_wave, 0x7fffffffu);
+    const int p_first = row0 + wave * ROWS_PER_LOAD, q_first = col0 + wave * ROWS_PER_LOAD;
+    const long long p_left = static_cast<long long>(R - p_first) * K * 2, q_left = static_cast<long long>(Cn - q_first) * K * 2;
+    const i32x4 p_rsrc = buffer_descriptor(EDGE && p_left <= 0 ? reinterpret_cast<const char*>(P) : p_wave, EDGE ? clamped_extent(p_left) : 0x7fffffffu);
+    const i32x4 q_rsrc = buffer_descriptor(EDGE && q_left <= 0 ? reinterpret_cast<const char*>(Q) : q_wave, EDGE ? clamped_extent(q_left) : 0x7fffffffu);
     auto advanced = [](i32x4 d, uint32_t bytes) {  // the descriptor with its base moved up
         const uint64_t a = ((static_cast<uint64_t>(static_cast<uint32_t>(d[1])) << 32) | static_cast<uint32_t>(d[0])) + bytes;
         d[0] = static_cast<int>(a & 0xffffffffu);
         d[1] = static_cast<int>(a >> 32);
+        if constexpr (EDGE) {
+            // Signed subtract and maximum (extents stay below 2^31), which the scalar ALU has: written as an
+            // unsigned saturating subtraction this becomes a vector instruction plus v_readfirstlane, and
+            // a scalar register written by the vector ALU is not safe to read in the load's inline assembly
+            // a few cycles later (the compiler does not insert the wait states there).
+            const int rest = d[2] - static_cast<int>(bytes);
+            d[2] = rest > 0 ? rest : 0;
+        }
         return d;
+    };
+    const int k_full = K - K % BK;
+    const uint32_t tail_off = (k_full + ld_chunk * 8 < K) ? lane_off : kBeyondExtent;
+    auto lane_offset_at = [&](int k0) -> uint32_t {  // k0 wave-uniform: the select costs one vector instruction per K tile
+        if constexpr (!EDGE) return lane_off;
+        return k0 < k_full ? lane_off : (k0 < K ? tail_off : kBeyondExtent);
     };
     // The two parts of a load in the K loop: the LDS destination goes into M0 one matrix instruction
     // before the load is issued (see set_direct_load_destination).
@@ -1063,15 +1086,15 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
         set_direct_load_destination(m < P_PER ? &Ps[stage][(m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]
                                               : &Qs[stage][((m - P_PER) * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]);
     };
-    auto fire_load = [&](const i32x4& pd, const i32x4& qd, int m) {
-        if (m < P_PER) direct_load16_buffer_to_destination(pd, lane_off, m * pass_bytes);
-        else direct_load16_buffer_to_destination(qd, lane_off, (m - P_PER) * pass_bytes);
+    auto fire_load = [&](const i32x4& pd, const i32x4& qd, uint32_t off, int m) {
+        if (m < P_PER) direct_load16_buffer_to_destination(pd, off, m * pass_bytes);
+        else direct_load16_buffer_to_destination(qd, off, (m - P_PER) * pass_bytes);
     };
-    auto issue_load = [&](int stage, const i32x4& pd, const i32x4& qd, int m) {
+    auto issue_load = [&](int stage, const i32x4& pd, const i32x4& qd, uint32_t off, int m) {
         if (m < P_PER)
-            direct_load16_buffer(pd, lane_off, m * pass_bytes, &Ps[stage][(m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]);
+            direct_load16_buffer(pd, off, m * pass_bytes, &Ps[stage][(m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]);
         else
-            direct_load16_buffer(qd, lane_off, (m - P_PER) * pass_bytes,
+            direct_load16_buffer(qd, off, (m - P_PER) * pass_bytes,
                                  &Qs[stage][((m - P_PER) * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]);
     };
 
@@ -1126,11 +1149,12 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
         constexpr int BARRIER_AT = PRISM_BF16_EARLY_BARRIER_AT, GAP = PRISM_BF16_EARLY_LOAD_GAP;
         static_assert(BARRIER_AT >= 33 && BARRIER_AT <= 64 && BARRIER_AT + (LOADS - 1) * GAP < 128, "loads fit the phase");
         const i32x4 pd = advanced(p_rsrc, k_next_bytes), qd = advanced(q_rsrc, k_next_bytes);
+        const uint32_t off = lane_offset_at(static_cast<int>(k_next_bytes / 2));
         auto maybe_load = [&](int at) {  // `at` = number of the instruction just issued, 0..127
             if (at + 1 >= BARRIER_AT && (at + 1 - BARRIER_AT) % GAP == 0 && (at + 1 - BARRIER_AT) / GAP < LOADS)
                 aim_load(S, (at + 1 - BARRIER_AT) / GAP);
             if (at >= BARRIER_AT && (at - BARRIER_AT) % GAP == 0 && (at - BARRIER_AT) / GAP < LOADS)
-                fire_load(pd, qd, (at - BARRIER_AT) / GAP);
+                fire_load(pd, qd, off, (at - BARRIER_AT) / GAP);
         };
         mfma_block(OTHER, [&](int m) {
             if (m < 16) read_fragment(0, S, 0, m);
@@ -1157,14 +1181,19 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
 #pragma unroll
     for (int j = 0; j < NI; ++j) fq[2][j] = bf16x8{};
 
-    // Tile t lives in stage t % 2; the launcher guarantees an even number of K tiles, at least 4.
-    const int k_tiles = K / BK;
+    // Tile t lives in stage t % 2. Whole tiles: the launcher guarantees an even number of K tiles, at least 4;
+    // EDGE: the count is padded to one (the padding tiles load zeros).
+    const int k_tiles = EDGE ? (ceil_div(K, BK) < 4 ? 4 : (ceil_div(K, BK) + 1) / 2 * 2) : K / BK;
+    {
+        const uint32_t off = lane_offset_at(0);
 #pragma unroll
-    for (int m = 0; m < LOADS; ++m) issue_load(0, p_rsrc, q_rsrc, m);
+        for (int m = 0; m < LOADS; ++m) issue_load(0, p_rsrc, q_rsrc, off, m);
+    }
     {
         const i32x4 pd = advanced(p_rsrc, BK * 2), qd = advanced(q_rsrc, BK * 2);
+        const uint32_t off = lane_offset_at(BK);
 #pragma unroll
-        for (int m = 0; m < LOADS; ++m) issue_load(1, pd, qd, m);
+        for (int m = 0; m < LOADS; ++m) issue_load(1, pd, qd, off, m);
     }
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(LOADS, kLgkmMax));
     __builtin_amdgcn_s_barrier();
@@ -1184,28 +1213,33 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
 #pragma unroll
         for (int j = 0; j < NI; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fp[2][i], fq[2][j], acc[i][j], 0, 0, 0);
+    // Write-back. Tiles that lie wholly inside the matrix (all of them unless EDGE) store without guards.
+    auto write_back = [&](auto guarded) {
 #pragma unroll
-    for (int i = 0; i < MI; ++i) {
+        for (int i = 0; i < MI; ++i) {
 #pragma unroll
-        for (int j = 0; j < NI; ++j) {
-            const int col = col0 + wave_n * WN + j * 16 + l16;
+            for (int j = 0; j < NI; ++j) {
+                const int col = col0 + wave_n * WN + j * 16 + l16;
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int row = row0 + wave_m * WM + i * 16 + 4 * lq + v;
-                store_out(&OUT[static_cast<size_t>(row) * Cn + col], acc[i][j][v]);
+                for (int v = 0; v < 4; ++v) {
+                    const int row = row0 + wave_m * WM + i * 16 + 4 * lq + v;
+                    if (!guarded || (row < R && col < Cn)) store_out(&OUT[static_cast<size_t>(row) * Cn + col], acc[i][j][v]);
+                }
             }
         }
-    }
+    };
+    if (!EDGE || (row0 + BM <= R && col0 + BN <= Cn)) write_back(std::false_type{});
+    else write_back(std::true_type{});
     // The last, redundant loads write LDS: they must have landed before the wave ends and its LDS goes to
     // the next workgroup. Behind the write-back the wait is covered by the stores.
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));
 }
 
-// Kernel choice. Whole 256 x 256 x 64 tiles: the register-staged pipeline whenever the K tile count
-// is even and at least 6 (measured faster than the ring from 2048^3 up), else the direct-to-LDS ring
-// (any count from 2). Ragged M, N or K with K a multiple of 8 and 16 B-aligned operands: the staged
-// pipeline's edge variant (K tiles padded with zeros to an even count of at least 6). Everything
-// else: the general kernel.
+// Kernel choice. Whole 256 x 256 x 64 tiles: the early-read pipeline (or, on request, a register-staged
+// one) whenever the K tile count is even and at least 6, else the direct-to-LDS ring (any count from 2).
+// Ragged M, N or K with K a multiple of 8 and 16 B-aligned operands: the same pipeline's edge variant
+// (K tiles padded with zeros to an even count). Fewer than 128 tiles: 128 x 128 tiles of the ring.
+// Everything else: the general kernel.
 #ifndef PRISM_BF16_STAGED_MIN_K
 #define PRISM_BF16_STAGED_MIN_K 384
 #endif
@@ -1275,7 +1309,7 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
         const int main_tiles = cut ? tiles - left : tiles;
         const int which = whole_tile_kernel();
         if (which == 2 && static_cast<long long>(K) * 2 * 64 < (1ll << 32))
-            gemm_bf16_early_kernel<BM, BN, WM, WN, OutT><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
+            gemm_bf16_early_kernel<BM, BN, WM, WN, false, OutT><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
                 R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
         else if (which != 0)
             gemm_bf16_staged16_kernel<BM, BN, WM, WN, false, OutT><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
@@ -1309,7 +1343,9 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
     }
     // Ragged M, N or K with 16 B-aligned rows: the staged kernel with zero-filled edges.
     if (PRISM_BF16_STAGED_EDGES && aligned && K % 8 == 0 && K > 0 && panel_ok) {
-        if (whole_tile_kernel() != 0)
+        if (whole_tile_kernel() == 2 && static_cast<long long>(K) * 2 * 64 < (1ll << 32))
+            gemm_bf16_early_kernel<BM, BN, WM, WN, true, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
+        else if (whole_tile_kernel() != 0)
             gemm_bf16_staged16_kernel<BM, BN, WM, WN, true, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
         else
             gemm_bf16_staged_kernel<BM, BN, WM, WN, true, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
