@@ -1,0 +1,112 @@
+"""Checks on the machine code hipcc generates for the two GEMM sources (CPU only: cross-compiles to assembly).
+
+The direct-to-LDS loads are inline assembly, which the compiler does not look into. Three things it would
+otherwise take care of are therefore checked on the generated text:
+
+* M0 carries a load's LDS destination. Every `s_mov_b32 m0` in these files is one of ours, so the number of M0
+  mentions must equal the number of direct loads, and walking back from every direct load the first M0 write
+  must come before the previous direct load (each load has its own write, nothing else touches M0 in between).
+* A scalar register written by the vector ALU (`v_readfirstlane`, `v_readlane`) needs five wait states before
+  a vector-memory instruction reads it. The compiler inserts them for instructions it knows; in front of an
+  inline-assembly load nothing does. No direct load may read such a register within five instructions unless a
+  scalar instruction has rewritten it in between.
+* The kernels whose K loops keep all 256 accumulation registers pinned (`gemm_bf16_early_kernel` for whole
+  tiles, `sgemm_wave_tile_dma_kernel`) must not spill: a spill there means the compiler has started to move
+  accumulators, which with matrix instructions in inline assembly is also a correctness hazard.
+"""
+import re
+import subprocess
+from concurrent.futures import ThreadPoolExecutor
+
+import pytest
+
+from prism_amd import build as pbuild
+
+SOURCES = ["gemm_bf16.hip", "sgemm.hip"]
+
+
+@pytest.fixture(scope="module")
+def assembly(tmp_path_factory):
+    out_dir = tmp_path_factory.mktemp("asm")
+
+    def compile_one(name):
+        out = out_dir / (name + ".s")
+        cmd = [pbuild.hipcc_path(), *pbuild.HIPCC_FLAGS, "-S", "--cuda-device-only", "-o", str(out), str(pbuild.CSRC / name)]
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        return out.read_text()
+
+    with ThreadPoolExecutor(max_workers=2) as pool:
+        return dict(zip(SOURCES, pool.map(compile_one, SOURCES)))
+
+
+def instructions(text):
+    """(kernel symbol, instruction text) for every instruction line, in order."""
+    out, kernel = [], None
+    for raw in text.splitlines():
+        line = raw.split(";")[0].strip()
+        if not line or line.startswith((".", "#")):
+            continue
+        if line.endswith(":"):
+            if line.startswith("_Z"):
+                kernel = line[:-1]
+            continue
+        out.append((kernel, line))
+    return out
+
+
+def is_direct_load(ins):
+    return ins.startswith("global_load_lds_") or (ins.startswith("buffer_load_") and ins.endswith(" lds"))
+
+
+def scalar_registers(text):
+    regs = set()
+    for m in re.finditer(r"s\[(\d+):(\d+)\]", text):
+        regs |= set(range(int(m.group(1)), int(m.group(2)) + 1))
+    for m in re.finditer(r"(?<![\w\[])s(\d+)\b", text):
+        regs.add(int(m.group(1)))
+    return regs
+
+
+@pytest.mark.parametrize("source", SOURCES)
+def test_every_direct_load_has_its_own_m0_write(assembly, source):
+    ins = [i for _, i in instructions(assembly[source])]
+    loads = [n for n, i in enumerate(ins) if is_direct_load(i)]
+    m0 = [n for n, i in enumerate(ins) if re.search(r"\bm0\b", i)]
+    assert loads and all(ins[n].startswith("s_mov_b32 m0,") for n in m0), "something other than s_mov_b32 touches M0"
+    assert len(m0) == len(loads)
+    previous = -1
+    for n in loads:
+        writes = [w for w in m0 if previous < w < n]
+        assert len(writes) == 1, f"direct load without an M0 write of its own: {ins[n]}"
+        previous = n
+
+
+@pytest.mark.parametrize("source", SOURCES)
+def test_no_vector_written_scalar_is_read_by_a_direct_load_too_soon(assembly, source):
+    ins = [i for _, i in instructions(assembly[source])]
+    for n, i in enumerate(ins):
+        if not is_direct_load(i):
+            continue
+        wanted = scalar_registers(i)
+        for back in range(1, 6):
+            if n - back < 0:
+                break
+            p = ins[n - back]
+            written = scalar_registers(p.split(",")[0]) if p.startswith(("s_", "v_readfirstlane", "v_readlane")) else set()
+            if p.startswith(("v_readfirstlane", "v_readlane")):
+                assert not (written & wanted), f"{p}  ...  {i}  ({back} instructions apart)"
+            wanted -= written  # rewritten by a scalar instruction: the load reads that result instead
+
+
+def test_pinned_accumulator_kernels_do_not_spill(assembly):
+    pinned = {"gemm_bf16.hip": r"gemm_bf16_early_kernelILi256ELi256ELi128ELi128ELb0E", "sgemm.hip": r"sgemm_wave_tile_dma_kernelILi256ELi256E"}
+    for source, pattern in pinned.items():
+        text = assembly[source]
+        found = 0
+        for m in re.finditer(r"^\s*\.amdhsa_kernel\s+(\S+)(.*?)\.end_amdhsa_kernel", text, re.S | re.M):
+            if re.search(pattern, m.group(1)):
+                found += 1
+                size = re.search(r"\.amdhsa_private_segment_fixed_size\s+(\d+)", m.group(2))
+                assert size and int(size.group(1)) == 0, f"{m.group(1)} uses {size.group(1) if size else '?'} bytes of scratch"
+        assert found >= 2, f"no kernel matching {pattern} in {source}"
