@@ -87,7 +87,8 @@ class CType:
 grid, block, warp, thread = (Perspective(n) for n in ("grid", "block", "warp", "thread"))
 
 _SCALARS = {"int": "int", "float": "float", "unsigned": "unsigned int", "uint": "unsigned int", "bool": "bool",
-            "double": "double", "uint32_t": "uint32_t", "uint64_t": "uint64_t"}
+            "double": "double", "uint32_t": "uint32_t", "uint64_t": "uint64_t", "bf16": "__bf16", "float4": "float4",
+            "void": "void"}
 
 
 def _ctype_text(t) -> str:
@@ -130,6 +131,7 @@ class _TypeName:
 
 uint, double, uint32_t, uint64_t = (_TypeName(n) for n in ("uint", "double", "uint32_t", "uint64_t"))
 shared = _TypeName("shared")
+bf16, void = _TypeName("bf16"), _TypeName("void")
 float4 = _TypeName("float4")
 float4_cast = _TypeName("float4_cast")  # float4_cast(x[i]) reads, float4_cast[x[i]] = v writes 16 bytes at &x[i]
 

@@ -60,7 +60,11 @@ fp32 MFMAs, printed as compiler builtins:
 `intrinsic.mfma_f32_16x16x4_f32(a, b, c0, c1, c2, c3, out=[d0, d1, d2, d3])` (lane l supplies
 a = A[l % 16][l / 16] and b = B[l / 16][l % 16] of a 16 x 4 by 4 x 16 product and holds
 C[4 (l / 16) + v][l % 16] in c<v>) and `intrinsic.mfma_f32_32x32x2_f32(a, b, c0..c15, out=[d0..d15])`
-(a = A[l % 32][l / 32], b = B[l / 32][l % 32], c<v> = C[8 (v / 4) + 4 (l / 32) + v % 4][l % 32]). All 64
+(a = A[l % 32][l / 32], b = B[l / 32][l % 32], c<v> = C[8 (v / 4) + 4 (l / 32) + v % 4][l % 32]). The bf16
+forms, `intrinsic.mfma_f32_16x16x32_bf16(a, b, c0..c3, out=[...])` and `intrinsic.mfma_f32_32x32x16_bf16(a, b,
+c0..c15, out=[...])`, take `float4` operands that carry eight consecutive bf16 of a row, the way
+`float4_cast(P[i])` reads them from a `ptr(bf16)`: a = P[l % 16][8 (l / 16) .. + 7], b = Q[l % 16][same k] for
+C = P Q^T (32-row form: l % 32 and 8 (l / 32)); accumulators as in the fp32 forms. All 64
 lanes of the wavefront must reach the statement together. Inline PTX itself (`intrinsic.mma`,
 `intrinsic.wgmma256`) has no meaning on this target and is refused by name, like asynchronous copies.
 """
@@ -74,11 +78,13 @@ from .hipgen import HipgenError, Kernel, _BINOPS, _CMPOPS, _REGISTRY, _UNOPS
 
 _TYPES = {"int": ("int", 4), "float": ("float", 4), "double": ("double", 8), "bool": ("bool", 1),
           "uint": ("unsigned int", 4), "unsigned": ("unsigned int", 4), "uint32_t": ("uint32_t", 4),
-          "uint64_t": ("uint64_t", 8), "float4": ("float4", 16), "void": ("void", 0)}
+          "uint64_t": ("uint64_t", 8), "float4": ("float4", 16), "bf16": ("__bf16", 2), "void": ("void", 0)}
 _LEVELS = ("grid", "block", "thread")
-# intrinsic.<name> -> (compiler builtin, accumulator registers per lane)
-_MFMA = {"mfma_f32_16x16x4_f32": ("__builtin_amdgcn_mfma_f32_16x16x4f32", 4),
-         "mfma_f32_32x32x2_f32": ("__builtin_amdgcn_mfma_f32_32x32x2f32", 16)}
+# intrinsic.<name> -> (compiler builtin, accumulator registers per lane, operands are 16-byte packets of 8 bf16)
+_MFMA = {"mfma_f32_16x16x4_f32": ("__builtin_amdgcn_mfma_f32_16x16x4f32", 4, False),
+         "mfma_f32_32x32x2_f32": ("__builtin_amdgcn_mfma_f32_32x32x2f32", 16, False),
+         "mfma_f32_16x16x32_bf16": ("__builtin_amdgcn_mfma_f32_16x16x32_bf16", 4, True),
+         "mfma_f32_32x32x16_bf16": ("__builtin_amdgcn_mfma_f32_32x32x16_bf16", 16, True)}
 
 
 @dataclass(frozen=True)
@@ -427,7 +433,13 @@ class BlockEmitter:
         if name == "float4_cast":
             if len(n.args) != 1 or n.keywords or not isinstance(n.args[0], ast.Subscript):
                 raise HipgenError(f"{_line(n)}: float4_cast() takes one array element")
-            return f"reinterpret_cast<float4 *>(&{self.expr(n.args[0])})[0]"
+            # Reading through a pointer to const needs the const in the cast (the reference prints the
+            # plain form, which only compiles for non-const arrays; its examples declare theirs that way).
+            base = n.args[0].value
+            while isinstance(base, ast.Name) and base.id in self.views:
+                base = ast.Name(id=self.views[base.id][0])
+            const = isinstance(base, ast.Name) and self.pointer_type.get(base.id, "").startswith("const ")
+            return f"reinterpret_cast<{'const ' if const else ''}float4 *>(&{self.expr(n.args[0])})[0]"
 
         targs = ""
         for kw in n.keywords:
@@ -509,7 +521,7 @@ class BlockEmitter:
         if name not in _MFMA:
             raise HipgenError(f"{_line(n)}: intrinsic.{name} is not an instruction of this target "
                               f"(available: {', '.join(sorted(_MFMA))})")
-        builtin, regs = _MFMA[name]
+        builtin, regs, packets = _MFMA[name]
         out = [kw.value for kw in n.keywords if kw.arg == "out"]
         if (len(n.args) != 2 + regs or len(n.keywords) != 1 or len(out) != 1 or not isinstance(out[0], ast.List)
                 or len(out[0].elts) != regs):
@@ -519,6 +531,9 @@ class BlockEmitter:
         self.open()
         self.emit(f"typedef float __acc_t __attribute__((ext_vector_type({regs})));")
         self.emit(f"__acc_t __acc = {{{acc}}};")
+        if packets:  # a float4 carries eight consecutive bf16 of a row, as float4_cast reads them
+            self.emit("typedef __bf16 __packet_t __attribute__((ext_vector_type(8)));")
+            a, b = f"__builtin_bit_cast(__packet_t, {a})", f"__builtin_bit_cast(__packet_t, {b})"
         self.emit(f"__acc = {builtin}({a}, {b}, __acc, 0, 0, 0);")
         for v, d in enumerate(out[0].elts):
             self.emit(f"{self.expr(d)} = __acc[{v}];")

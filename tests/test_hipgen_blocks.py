@@ -15,7 +15,7 @@ import numpy as np
 import pytest
 
 from prism_amd import hipgen
-from prism_amd.hipgen import (HipgenError, attr, block, const, float4, float4_cast, generate, generate_launcher, grid,
+from prism_amd.hipgen import (HipgenError, attr, bf16, block, const, float4, float4_cast, generate, generate_launcher, grid,
                               group, intrinsic, partition, prism, ptr, requires, shared, split, thread, uint32_t, unsafe)
 from prism_amd.hipgen_blocks import dynamic_lds_bytes
 
@@ -402,6 +402,40 @@ def foreign_instruction(x: ptr(float) @ grid[1]):
     intrinsic.mma(a, a, a, a, a, a, a, a, a, a, out=[a, a, a, a])
 
 
+@requires(grid[1], block[1], thread[64])
+@prism("global")
+def one_bf16_mfma_per_wavefront(P: ptr(const(bf16)) @ grid[1], Q: ptr(const(bf16)) @ grid[1], D: ptr(float) @ grid[1],
+                                M: int @ grid[1], N: int @ grid[1], K: int @ grid[1]):
+    """D = P Q^T (P is M x K, Q is N x K, both bf16 with K contiguous: the operand layout of
+    examples/h100_matmul.py) with one wavefront per 16 x 16 tile of D and one 16x16x32 bf16 MFMA per K step of
+    32; every lane fetches 16-byte packets of eight bf16 straight from global memory."""
+    tiles_n: const(int) @ grid[1] = N / 16
+    w: const(int) @ thread[64] = id()
+    tile_r: const(int) @ thread[64] = w / tiles_n
+    tile_c: const(int) @ thread[64] = w % tiles_n
+    with partition(P, p=thread[64], offset=tile_r * 16 * K) as P_rows:
+        with partition(Q, p=thread[64], offset=tile_c * 16 * K) as Q_rows:
+            with partition(D, p=thread[64], offset=tile_r * 16 * N + tile_c * 16) as D_tile:
+                with group(block[1]):
+                    with group(thread[64]):
+                        lane: const(int) @ thread[1] = id()
+                        r: const(int) @ thread[1] = lane % 16
+                        q: const(int) @ thread[1] = lane / 16
+                        c0: float @ thread[1] = 0
+                        c1: float @ thread[1] = 0
+                        c2: float @ thread[1] = 0
+                        c3: float @ thread[1] = 0
+                        if w < (M / 16) * tiles_n:
+                            for k0 in range(0, K, 32):
+                                a: float4 @ thread[1] = float4_cast(P_rows[r * K + k0 + 8 * q])
+                                b: float4 @ thread[1] = float4_cast(Q_rows[r * K + k0 + 8 * q])
+                                intrinsic.mfma_f32_16x16x32_bf16(a, b, c0, c1, c2, c3, out=[c0, c1, c2, c3])
+                            D_tile[(4 * q + 0) * N + r] = c0
+                            D_tile[(4 * q + 1) * N + r] = c1
+                            D_tile[(4 * q + 2) * N + r] = c2
+                            D_tile[(4 * q + 3) * N + r] = c3
+
+
 def lines(text):
     return [ln.strip() for ln in text.splitlines()]
 
@@ -519,6 +553,12 @@ def test_matrix_instruction_statement():
     assert "const int w = (__thread_id_0 / 64);" in got
     with pytest.raises(HipgenError, match="intrinsic.mma is not an instruction of this target"):
         generate("foreign_instruction")
+    half = lines(generate("one_bf16_mfma_per_wavefront"))
+    assert half[0].startswith("__global__ void one_bf16_mfma_per_wavefront(const __bf16* P, const __bf16* Q, float* D,")
+    assert "float4 a = reinterpret_cast<const float4 *>(&P_rows[(((r * K) + k0) + (8 * q))])[0];" in half
+    i = half.index("typedef __bf16 __packet_t __attribute__((ext_vector_type(8)));")
+    assert half[i + 1] == ("__acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(__packet_t, a), "
+                           "__builtin_bit_cast(__packet_t, b), __acc, 0, 0, 0);")
 
 
 def test_device_function_gets_the_callers_ids():
@@ -570,7 +610,8 @@ def test_thread_groups_of_32_and_target_text():
 BUILDS = {"two_roles": (256, None), "row_scan32": (256, None), "add_m_blocks": (256, None), "naive_sgemm": (256, None), "tiled_sgemm": (1024, [32]),
           "thread_tile_sgemm": (256, [64, 64, 8, 4, 4]), "scaled_sum_all": (256, None),
           "vector_tile_sgemm": (256, [128, 128, 8, 8, 8]), "gather_columns": (256, None),
-          "add_m_by_wavefronts": (256, None), "one_mfma_per_wavefront": (256, None)}
+          "add_m_by_wavefronts": (256, None), "one_mfma_per_wavefront": (256, None),
+          "one_bf16_mfma_per_wavefront": (256, None)}
 
 
 @pytest.fixture(scope="module")
@@ -750,3 +791,24 @@ def test_generated_one_mfma_per_wavefront(built, oracle, shape):
     assert np.all(out[:64] == 777.0) and np.all(out[64 + M * N:] == 777.0)
     want = oracle.np_sgemm_f64(1.0, A, B, 0.0, np.zeros((M, N), np.float32))
     assert np.max(np.abs(out[64:64 + M * N].reshape(M, N) - want)) <= oracle.sgemm_tolerance(K, A, B)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(16, 16, 32), (48, 80, 96), (256, 128, 512)])
+def test_generated_one_bf16_mfma_per_wavefront(built, oracle, shape):
+    import torch
+    M, N, K = shape
+    fn = built["one_bf16_mfma_per_wavefront"].one_bf16_mfma_per_wavefront_launch
+    fn.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int] * 3 + [ctypes.c_uint, ctypes.c_void_p]
+    P16, Q16 = oracle.gen_gemm_bf16(M, N, K, seed=M + K)
+    p = torch.from_numpy(P16.view(np.int16)).to("cuda:0")
+    q = torch.from_numpy(Q16.view(np.int16)).to("cuda:0")
+    buf = torch.full((M * N + 128,), 777.0, dtype=torch.float32, device="cuda:0")
+    d = buf[64:64 + M * N]
+    tiles = (M // 16) * (N // 16)
+    assert fn(p.data_ptr(), q.data_ptr(), d.data_ptr(), M, N, K, (tiles + 3) // 4, None) == 0
+    torch.cuda.synchronize()
+    out = buf.cpu().numpy()
+    assert np.all(out[:64] == 777.0) and np.all(out[64 + M * N:] == 777.0)
+    ref = oracle.gemm_bf16_f64(P16, Q16)
+    assert np.max(np.abs(out[64:64 + M * N].reshape(M, N) - ref)) <= 1e-3 * np.abs(ref).max()
