@@ -96,9 +96,10 @@ __device__ __forceinline__ void set_direct_load_destination(const void* lds_dst)
     asm volatile("s_mov_b32 m0, %0" : : "s"(lds_addr) : "memory", "m0");
 #pragma clang diagnostic pop
 }
+// The descriptor and the scalar offset must be in scalar registers already (made so where they are
+// computed, away from the loads): a v_readfirstlane here would sit right in front of the load, which would
+// then read a scalar register the vector ALU has just written, without the wait states that needs.
 __device__ __forceinline__ void direct_load16_buffer_to_destination(i32x4 rsrc, uint32_t lane_offset, uint32_t scalar_offset) {
-    scalar_offset = __builtin_amdgcn_readfirstlane(scalar_offset);
-    rsrc = scalar_descriptor(rsrc);
     asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(lane_offset), "s"(rsrc), "s"(scalar_offset) : "memory");
 }
 

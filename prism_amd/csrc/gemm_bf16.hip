@@ -967,6 +967,10 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_stage
     __builtin_amdgcn_sched_barrier(0);
     int k_load = 3 * BK;
     do {
+        // Wait states between vector-ALU writes of fragment registers (the zeros above, the compiler's
+        // copies of them in front of the loop) and the inline-assembly matrix instructions that read
+        // them; see the note at the head of gemm_bf16_early_kernel's loop.
+        asm volatile("s_nop 4");
         phase(s0{}, yes{}, yes{}, k_load);
         phase(s1{}, yes{}, yes{}, k_load + BK);
         k_load += 2 * BK;
@@ -1055,7 +1059,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     // (a descriptor whose base moves up by some bytes loses as many from its extent); what follows a row's
     // last column is the next row, so in the partial K tile lanes with k >= K use an offset beyond any
     // extent, and in the K tiles that pad the count to an even number of at least 4 all lanes do.
-    const uint32_t pass_bytes = static_cast<uint32_t>(ROWS_PER_PASS) * static_cast<uint32_t>(K) * 2u;  // the launcher keeps BM * K * 2 below 2^31
+    // (Forced into a scalar register here: direct_load16_buffer_to_destination takes its scalar operands as
+    // they are, so that no v_readfirstlane ends up right in front of a load.)
+    const uint32_t pass_bytes = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(ROWS_PER_PASS) * static_cast<uint32_t>(K) * 2u);  // the launcher keeps BM * K * 2 below 2^31
     const int p_first = row0 + wave * ROWS_PER_LOAD, q_first = col0 + wave * ROWS_PER_LOAD;
     const long long p_left = static_cast<long long>(R - p_first) * K * 2, q_left = static_cast<long long>(Cn - q_first) * K * 2;
     const i32x4 p_rsrc = buffer_descriptor(EDGE && p_left <= 0 ? reinterpret_cast<const char*>(P) : p_wave, EDGE ? clamped_extent(p_left) : 0x7fffffffu);
@@ -1200,6 +1206,14 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     for (int t = 0; t < k_tiles; t += 2) {
+        // Fragment registers that the vector ALU has written (the zeros of set 2 above, and the copies the
+        // compiler makes of them in front of the loop) need wait states before a matrix instruction reads
+        // them. The compiler inserts those for its own matrix instructions, not for one in inline assembly:
+        // in a variant of this loop that began right at a matrix instruction, the first one read stale
+        // registers on some lanes (0 x NaN from whatever ran before = NaN in the first sub-tile, on the first
+        // call only). Here scalar instructions happen to sit in between; the five wait states make that
+        // independent of what the compiler puts at the head of the loop, and cost nothing measurable.
+        asm volatile("s_nop 4");
         const int next = t + 2 < k_tiles ? t + 2 : k_tiles - 2;
         phase(s0{}, static_cast<uint32_t>(next) * (BK * 2));
         phase(s1{}, static_cast<uint32_t>(next + 1) * (BK * 2));
