@@ -1,7 +1,7 @@
 """Checks on the machine code hipcc generates for the two GEMM sources (CPU only: cross-compiles to assembly).
 
-The direct-to-LDS loads are inline assembly, which the compiler does not look into. Three things it would
-otherwise take care of are therefore checked on the generated text:
+The direct-to-LDS loads and some matrix instructions are inline assembly, which the compiler does not look
+into. Four things it would otherwise take care of are therefore checked on the generated text:
 
 * M0 carries a load's LDS destination. Every `s_mov_b32 m0` in these files is one of ours, so the number of M0
   mentions must equal the number of direct loads, and walking back from every direct load the first M0 write
@@ -10,6 +10,10 @@ otherwise take care of are therefore checked on the generated text:
   a vector-memory instruction reads it. The compiler inserts them for instructions it knows; in front of an
   inline-assembly load nothing does. No direct load may read such a register within five instructions unless a
   scalar instruction has rewritten it in between.
+* A vector register written by the vector ALU needs wait states before a matrix instruction reads it as an
+  operand; for the matrix instructions issued from inline assembly nothing inserts them. No matrix instruction
+  may read a register that a vector ALU instruction wrote within the two instructions before it (`s_nop n`
+  counts as n + 1).
 * The kernels whose K loops keep all 256 accumulation registers pinned (`gemm_bf16_early_kernel` for whole
   tiles, `sgemm_wave_tile_dma_kernel`) must not spill: a spill there means the compiler has started to move
   accumulators, which with matrix instructions in inline assembly is also a correctness hazard.
@@ -97,6 +101,38 @@ def test_no_vector_written_scalar_is_read_by_a_direct_load_too_soon(assembly, so
             if p.startswith(("v_readfirstlane", "v_readlane")):
                 assert not (written & wanted), f"{p}  ...  {i}  ({back} instructions apart)"
             wanted -= written  # rewritten by a scalar instruction: the load reads that result instead
+
+
+def vector_registers(text):
+    regs = set()
+    for m in re.finditer(r"(?<![\w])v\[(\d+):(\d+)\]", text):
+        regs |= set(range(int(m.group(1)), int(m.group(2)) + 1))
+    for m in re.finditer(r"(?<![\w\[])v(\d+)\b", text):
+        regs.add(int(m.group(1)))
+    return regs
+
+
+def test_no_matrix_instruction_reads_a_register_the_vector_alu_has_just_written(assembly):
+    ins = [i for _, i in instructions(assembly["gemm_bf16.hip"])]
+    checked = 0
+    for n, i in enumerate(ins):
+        if not i.startswith("v_mfma_"):
+            continue
+        operands = i.split(None, 1)[1].split(",")
+        sources = vector_registers(operands[1]) | vector_registers(operands[2])
+        checked += 1
+        distance, back = 0, 1
+        while distance < 2 and n - back >= 0:
+            p = ins[n - back]
+            if p.startswith("s_nop"):
+                distance += int(p.split()[1]) + 1
+            else:
+                distance += 1
+                if p.startswith("v_") and not p.startswith(("v_mfma_", "v_cmp", "v_readfirstlane", "v_readlane")):
+                    written = vector_registers(p.split(None, 1)[1].split(",")[0])
+                    assert not (written & sources), f"{p}  ...  {i}"
+            back += 1
+    assert checked > 1000
 
 
 def test_pinned_accumulator_kernels_do_not_spill(assembly):
