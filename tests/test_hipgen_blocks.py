@@ -436,6 +436,51 @@ def one_bf16_mfma_per_wavefront(P: ptr(const(bf16)) @ grid[1], Q: ptr(const(bf16
                             D_tile[(4 * q + 3) * N + r] = c3
 
 
+@attr("__launch_bounds__(256)")
+@requires(grid[1], block[1], thread[64])
+@prism("global")
+def mfma_tile_sgemm(M: int @ grid[1], N: int @ grid[1], K: int @ grid[1], alpha: float @ grid[1],
+                    A: ptr(const(float)) @ grid[1], B: ptr(const(float)) @ grid[1], beta: float @ grid[1],
+                    C: ptr(float) @ grid[1], tiles_n: int @ grid[1]):
+    """C = alpha A B + beta C with 64 x 64 x 8 tiles staged in LDS and the product on fp32 MFMA: four wavefronts
+    per workgroup, each owning a 32 x 32 corner in sixteen accumulators, one 32x32x2 instruction per pair of k
+    values (the wave-level tiling of examples/sgemm_kernel_5.py with the matrix instruction in place of its
+    per-thread loops). A is stored k-major so that both operands are read along a row of LDS."""
+    tile_r: const(int) @ block[1] = id() / tiles_n
+    tile_c: const(int) @ block[1] = id() % tiles_n
+    with partition(A, p=block[1], offset=tile_r * 64 * K) as A_rows:
+        with partition(B, p=block[1], offset=tile_c * 64) as B_cols:
+            with partition(C, p=block[1], offset=tile_r * 64 * N + tile_c * 64) as C_tile:
+                with group(block[1]):
+                    a_lds: shared(float[512], static=True) @ block[1]
+                    b_lds: shared(float[512], static=True) @ block[1]
+                    t: const(int) @ thread[1] = id()
+                    wave: const(int) @ thread[64] = id()
+                    corner_r: const(int) @ thread[64] = (wave / 2) * 32
+                    corner_c: const(int) @ thread[64] = (wave % 2) * 32
+                    with group(thread[64]):
+                        lane: const(int) @ thread[1] = id()
+                        r: const(int) @ thread[1] = lane % 32
+                        q: const(int) @ thread[1] = lane / 32
+                        acc: float[16] @ thread[1] = {0}
+                        with group(thread[1]):
+                            for k0 in range(0, K, 8):
+                                for e in range(t, 512, 256):
+                                    a_lds[(e % 8) * 64 + e / 8] = A_rows[(e / 8) * K + k0 + e % 8]
+                                    b_lds[e] = B_cols[(k0 + e / 64) * N + e % 64]
+                                for kk in range(0, 8, 2):
+                                    intrinsic.mfma_f32_32x32x2_f32(
+                                        a_lds[(kk + q) * 64 + corner_r + r], b_lds[(kk + q) * 64 + corner_c + r],
+                                        acc[0], acc[1], acc[2], acc[3], acc[4], acc[5], acc[6], acc[7],
+                                        acc[8], acc[9], acc[10], acc[11], acc[12], acc[13], acc[14], acc[15],
+                                        out=[acc[0], acc[1], acc[2], acc[3], acc[4], acc[5], acc[6], acc[7],
+                                             acc[8], acc[9], acc[10], acc[11], acc[12], acc[13], acc[14], acc[15]])
+                            for v in range(16):
+                                with partition(C_tile, p=thread[1],
+                                               offset=(corner_r + 8 * (v / 4) + 4 * q + v % 4) * N + corner_c + r) as c:
+                                    c[0] = alpha * acc[v] + beta * c[0]
+
+
 def lines(text):
     return [ln.strip() for ln in text.splitlines()]
 
@@ -553,6 +598,13 @@ def test_matrix_instruction_statement():
     assert "const int w = (__thread_id_0 / 64);" in got
     with pytest.raises(HipgenError, match="intrinsic.mma is not an instruction of this target"):
         generate("foreign_instruction")
+    tiled = lines(generate("mfma_tile_sgemm"))
+    i = tiled.index("typedef float __acc_t __attribute__((ext_vector_type(16)));")
+    assert tiled[i + 2].startswith("__acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a_lds[((((kk + q) * 64) + corner_r) + r)], b_lds[")
+    assert tiled[i + 3] == "acc[0] = __acc[0];" and tiled[i + 18] == "acc[15] = __acc[15];"
+    # a barrier between the staging loop and the matrix instructions, one before the next K step
+    assert tiled.count("__syncthreads();") == 2
+    assert tiled[tiled.index("__syncthreads();") + 1] == "for (int kk = 0; kk < 8; kk += 2) {"
     half = lines(generate("one_bf16_mfma_per_wavefront"))
     assert half[0].startswith("__global__ void one_bf16_mfma_per_wavefront(const __bf16* P, const __bf16* Q, float* D,")
     assert "float4 a = reinterpret_cast<const float4 *>(&P_rows[(((r * K) + k0) + (8 * q))])[0];" in half
@@ -611,7 +663,7 @@ BUILDS = {"two_roles": (256, None), "row_scan32": (256, None), "add_m_blocks": (
           "thread_tile_sgemm": (256, [64, 64, 8, 4, 4]), "scaled_sum_all": (256, None),
           "vector_tile_sgemm": (256, [128, 128, 8, 8, 8]), "gather_columns": (256, None),
           "add_m_by_wavefronts": (256, None), "one_mfma_per_wavefront": (256, None),
-          "one_bf16_mfma_per_wavefront": (256, None)}
+          "one_bf16_mfma_per_wavefront": (256, None), "mfma_tile_sgemm": (256, None)}
 
 
 @pytest.fixture(scope="module")
@@ -812,3 +864,11 @@ def test_generated_one_bf16_mfma_per_wavefront(built, oracle, shape):
     assert np.all(out[:64] == 777.0) and np.all(out[64 + M * N:] == 777.0)
     ref = oracle.gemm_bf16_f64(P16, Q16)
     assert np.max(np.abs(out[64:64 + M * N].reshape(M, N) - ref)) <= 1e-3 * np.abs(ref).max()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(64, 64, 8), (128, 192, 72), (256, 128, 256)])
+def test_generated_lds_tiled_mfma_sgemm(built, oracle, shape):
+    """LDS staging with the emitter's barriers around wavefront-wide matrix instructions."""
+    M, N, K = shape
+    run_sgemm(built["mfma_tile_sgemm"], "mfma_tile_sgemm", oracle, M, N, K, N // 64, (M // 64) * (N // 64))
