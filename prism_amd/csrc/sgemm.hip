@@ -461,8 +461,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
     constexpr int ROWS_PER_PASS = ROWS_PER_LOAD * WAVES;
     static_assert(BM % ROWS_PER_PASS == 0 && BK % WAVES == 0, "whole load passes");
     constexpr int A_PER = BM / ROWS_PER_PASS, B_PER = BK / WAVES;  // loads per wave per tile
-    constexpr int LOAD_GAP = PRISM_SGEMM5_LOAD_GAP;                  // MFMAs between two direct loads
-    static_assert((A_PER + B_PER) * LOAD_GAP <= 4 * MI * 4, "the loads of a tile fit among the MFMAs of one group");
+    // MFMAs between two direct loads: the configured gap, or less when the first group is too short for it
+    constexpr int LOAD_GAP = (A_PER + B_PER) * PRISM_SGEMM5_LOAD_GAP <= 4 * MI * 4 ? PRISM_SGEMM5_LOAD_GAP : (4 * MI * 4) / (A_PER + B_PER);
+    static_assert(LOAD_GAP >= 1 && (A_PER + B_PER) * LOAD_GAP <= 4 * MI * 4, "the loads of a tile fit among the MFMAs of one group");
     static_assert(((ROWS_PER_PASS >> SWZ) % KP) == 0 && ((32 >> SWZ) % KP) == 0,
                   "the swizzle term must repeat with the load pass and the 32-row MFMA block");
 
@@ -1041,6 +1042,43 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
     return true;
 }
 
+// Between the one-wave tiles (up to one 64 x 64 tile per SIMD) and the 256 x 256 tiles (from three quarters of
+// the CUs up) lies a range in which neither fills the chip: there the same direct-to-LDS kernel runs on
+// 128 x 256 tiles (four waves of 64 x 128, K tiles of 16, 48 KiB of LDS, one workgroup per CU) when those give
+// every CU at most one tile, else on 64 x 256 tiles (four waves of 32 x 128, 40 KiB of LDS, 138 registers: three
+// workgroups per CU) when those give every CU at most three; in both cases at least half of the CUs get one.
+#ifndef PRISM_SGEMM5_HALF_TILES
+#define PRISM_SGEMM5_HALF_TILES 1
+#endif
+#ifndef PRISM_SGEMM5_QUARTER_TILES
+#define PRISM_SGEMM5_QUARTER_TILES 1
+#endif
+template <int BM, bool ALLOW_EDGES>
+bool try_half_tile_dma(int M, int N, int K, float alpha, const float* A, const float* B, float beta,
+                       float* C, hipStream_t s, int* rc) {
+    constexpr int BN = 256, BK = 16, WM = BM / 2, WN = 128;
+    if (!PRISM_SGEMM5_DMA || !PRISM_SGEMM5_HALF_TILES) return false;
+    if (K <= 0 || !aligned16(A) || !aligned16(B) || !aligned16(C)) return false;
+    const bool whole = M % BM == 0 && N % BN == 0 && K % BK == 0;
+    if (!whole && (!PRISM_SGEMM5_EDGES || !ALLOW_EDGES || N % 4 || K % 4 ||
+                   (static_cast<long long>(BM) + 64) * K * 4 >= (1ll << 31) ||
+                   (static_cast<long long>(K) + 64) * N * 4 >= (1ll << 31)))
+        return false;
+    const int tiles_m = ceil_div(M, BM), tiles_n = ceil_div(N, BN);
+    const long long tiles = static_cast<long long>(tiles_m) * tiles_n;
+    // 128 x 256: at most one tile per CU. 64 x 256 (three workgroups fit a CU): at most three.
+    if (tiles > (BM == 128 ? 1 : 3) * cu_count() || tiles * 2 < cu_count()) return false;
+    const dim3 grid(static_cast<unsigned>(tiles)), block((BM / WM) * (BN / WN) * kWave);
+    if (whole) {
+        sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, false><<<grid, block, 0, s>>>(M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n);
+    } else {
+        if constexpr (ALLOW_EDGES)
+            sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, true><<<grid, block, 0, s>>>(M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n);
+    }
+    *rc = check_launch("sgemm_wave_tile_dma_kernel (128 x 256)");
+    return true;
+}
+
 #ifndef PRISM_SGEMM5_SINGLE
 #define PRISM_SGEMM5_SINGLE 1
 #endif
@@ -1121,14 +1159,17 @@ int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, 
                 if (try_wave_tile_dma<256, 256, 32, 128, 128, true>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
                 if (try_wave_tile_dma<256, 256, 16, 128, 128, false>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
                 // Small problems (at most one 64 x 64 tile per SIMD): one wave per tile, 32 x 32 tiles when
-                // 64 x 64 ones would leave SIMDs without work. In between, the general kernel's 128 x 128
-                // tiles quantise best.
+                // 64 x 64 ones would leave SIMDs without work. In between, the direct-to-LDS kernel on
+                // 128 x 256 tiles (at most one per CU) or 64 x 256 tiles (at most three per CU); what is left
+                // (N or K not a multiple of 4, unaligned operands) goes to the general kernel.
                 const long long simds = 4ll * cu_count();
                 const long long tiles64 = static_cast<long long>(ceil_div(M, 64)) * ceil_div(N, 64);
                 if (tiles64 <= PRISM_SGEMM5_SINGLE_ROUNDS * simds) {
                     if (tiles64 < simds && try_single_wave<32>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
                     if (try_single_wave<64>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
                 }
+                if (try_half_tile_dma<128, true>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
+                if (PRISM_SGEMM5_QUARTER_TILES && try_half_tile_dma<64, true>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
             }
             return run_wave_tile<PRISM_SGEMM5_CFG>(M, N, K, alpha, A, B, beta, C, s);
     }

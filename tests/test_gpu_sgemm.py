@@ -256,6 +256,26 @@ def test_wave_tile_ragged_edges(prism, oracle, shape):
         assert np.max(np.abs(got - oracle.np_sgemm_f64(1.25, A, B, beta, Cm))) <= tol(oracle, K, A, B, beta, Cm)
 
 
+@pytest.mark.parametrize("shape", [(2304, 2304, 64), (2560, 2816, 48), (2300, 2564, 100), (2817, 2560, 36),
+                                   (3072, 3072, 64), (3328, 2944, 32), (3000, 3332, 68), (3329, 3072, 20), (1152, 6144, 16)])
+def test_wave_tile_mid_sizes(prism, oracle, shape):
+    """Between the one-wave tiles (up to 1024 tiles of 64 x 64) and the 256 x 256 tiles (from 192 of them): the
+    direct-to-LDS kernel on 128 x 256 tiles when those give every CU at most one (the first four shapes and the
+    last), on 64 x 256 tiles when they give it at most three (the others); whole and ragged shapes, K tile counts
+    from 1 up. Operands between NaNs, C fenced, every element checked, with and without reading C."""
+    M, N, K = shape
+    A, B, Cm = oracle.gen_sgemm(M, N, K, seed=M + 5 * K)
+    for beta in (0.5, 0.0):
+        buf = torch.full((M * N + 512,), 777.0, dtype=torch.float32, device=DEV)
+        c = buf[256:256 + M * N].view(M, N)
+        c.copy_(dev(Cm))
+        prism.sgemm(M, N, K, 1.25, nan_fenced(A), nan_fenced(B), beta, c, variant=5)
+        out = host(buf)
+        assert np.all(out[:256] == 777.0) and np.all(out[256 + M * N:] == 777.0)
+        got = out[256:256 + M * N].reshape(M, N)
+        assert np.max(np.abs(got - oracle.np_sgemm_f64(1.25, A, B, beta, Cm))) <= tol(oracle, K, A, B, beta, Cm)
+
+
 def test_wave_tile_ragged_tall_matrix(prism, oracle):
     """A ragged A of more than 4 GiB: the bytes from a tile's first row to the end of A do not fit the 32 bits
     of a buffer descriptor's extent and are cut to 2 GiB - 1 (a tile only reaches 256 rows ahead). Rows are
