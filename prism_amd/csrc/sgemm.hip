@@ -448,7 +448,7 @@ __attribute__((amdgpu_waves_per_eu(PRISM_SGEMM5_WAVES_PER_EU))) void sgemm_wave_
 template <int BM, int BN, int BK, int WM, int WN, bool EDGE>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile_dma_kernel(
     int M, int N, int K, float alpha, const float* __restrict__ A, const float* __restrict__ B,
-    float beta, float* C, int tiles_m, int tiles_n) {
+    float beta, float* C, int tiles_m, int tiles_n, int first_big) {
     constexpr int WAVES_N = BN / WN;
     constexpr int WAVES = (BM / WM) * WAVES_N;
     constexpr int MI = WM / 32, NI = 4;
@@ -472,9 +472,22 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
     __shared__ __attribute__((aligned(1024))) float Bs0[BK * BN];
     __shared__ __attribute__((aligned(1024))) float Bs1[BK * BN];
 
-    int tm, tn;
-    xcd_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
-    const int row0 = tm * BM, col0 = tn * BN;
+    // first_big < 0: the grid covers the tiles_m x tiles_n grid of BM x BN tiles. Otherwise this launch
+    // finishes what a launch on 256 x 256 tiles left over: tiles_m x tiles_n is that launch's grid, first_big
+    // the first tile number it did not take, and every leftover tile is cut into 256 / BM row slices.
+    int row0, col0;
+    if (first_big < 0) {
+        int tm, tn;
+        xcd_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+        row0 = tm * BM;
+        col0 = tn * BN;
+    } else {
+        constexpr int SUB = 256 / BM;
+        int tm, tn;
+        xcd_tile_coords(first_big + blockIdx.x / SUB, tiles_m, tiles_n, tm, tn);
+        row0 = tm * 256 + static_cast<int>(blockIdx.x % SUB) * BM;
+        col0 = tn * 256;
+    }
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -985,6 +998,9 @@ int run_wave_tile(int M, int N, int K, float alpha, const float* A, const float*
 #ifndef PRISM_SGEMM5_SINGLE_ROUNDS
 #define PRISM_SGEMM5_SINGLE_ROUNDS 1
 #endif
+#ifndef PRISM_SGEMM5_LEFTOVER_SLICES
+#define PRISM_SGEMM5_LEFTOVER_SLICES 1
+#endif
 template <int BM, int BN, int BK, int WM, int WN, bool ALLOW_EDGES>
 bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const float* B, float beta,
                        float* C, hipStream_t s, int* rc) {
@@ -1017,14 +1033,29 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
             main_tiles = tiles - left;
             leftover_wt = cost64 <= cost32 ? 64 : 32;
         }
+        // Or into 64 x 256 slices of this kernel (K tiles of 16, up to three workgroups to a CU). Measured
+        // cost of the last round in full rounds, slices against one-wave tiles: 16 tiles left over 0.27 / 0.15,
+        // 33 0.26 / 0.35, 64 0.28 / 0.53, 68 0.51 / 0.35, 132 0.75 / 1.05, 144 0.77 / 0.93, 164 0.76 / 1.06:
+        // slices cost about 0.27 per slice on the fullest CU, so they win when they give every CU exactly
+        // one, or three where one-wave tiles are no better than a full round.
+        const bool one_each = left * 4 <= cus && left * 8 >= cus, three_each = left * 4 > 2 * cus && left * 4 <= 3 * cus;
+        if (PRISM_SGEMM5_LEFTOVER_SLICES && (one_each || three_each)) {
+            main_tiles = tiles - left;
+            leftover_wt = 256;
+        }
     }
     // `edge` selects the zero-filling variants of both kernels (sub-tiles that lie wholly outside C exit at once).
     auto launch = [&](auto edge) {
         constexpr bool EDGE = decltype(edge)::value;
         sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, EDGE><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
-            M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n);
+            M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
         *rc = check_launch("sgemm_wave_tile_dma_kernel");
-        if (*rc == 0 && leftover_wt == 64) {
+        if (*rc == 0 && leftover_wt == 256) {
+            // 64 x 256 slices of the same kernel, three workgroups to a CU
+            sgemm_wave_tile_dma_kernel<64, 256, 16, 32, 128, EDGE><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 4), dim3(256), 0, s>>>(
+                M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, main_tiles);
+            *rc = check_launch("sgemm_wave_tile_dma_kernel (leftover slices)");
+        } else if (*rc == 0 && leftover_wt == 64) {
             sgemm_single_wave_kernel<64, 4, EDGE><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 16), dim3(kWave), 0, s>>>(
                 M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, main_tiles);
             *rc = check_launch("sgemm_single_wave_kernel");
@@ -1070,10 +1101,10 @@ bool try_half_tile_dma(int M, int N, int K, float alpha, const float* A, const f
     if (tiles > (BM == 128 ? 1 : 3) * cu_count() || tiles * 2 < cu_count()) return false;
     const dim3 grid(static_cast<unsigned>(tiles)), block((BM / WM) * (BN / WN) * kWave);
     if (whole) {
-        sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, false><<<grid, block, 0, s>>>(M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n);
+        sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, false><<<grid, block, 0, s>>>(M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
     } else {
         if constexpr (ALLOW_EDGES)
-            sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, true><<<grid, block, 0, s>>>(M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n);
+            sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, true><<<grid, block, 0, s>>>(M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
     }
     *rc = check_launch("sgemm_wave_tile_dma_kernel (128 x 256)");
     return true;
