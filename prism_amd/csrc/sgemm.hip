@@ -998,6 +998,9 @@ int run_wave_tile(int M, int N, int K, float alpha, const float* A, const float*
 #ifndef PRISM_SGEMM5_SINGLE_ROUNDS
 #define PRISM_SGEMM5_SINGLE_ROUNDS 1
 #endif
+#ifndef PRISM_SGEMM5_LEFTOVER_HALVES
+#define PRISM_SGEMM5_LEFTOVER_HALVES 1
+#endif
 #ifndef PRISM_SGEMM5_LEFTOVER_SLICES
 #define PRISM_SGEMM5_LEFTOVER_SLICES 1
 #endif
@@ -1043,6 +1046,12 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
             main_tiles = tiles - left;
             leftover_wt = 256;
         }
+        // In between, 128 x 256 halves (one workgroup to a CU) cost 0.55-0.6 of a round whatever their number;
+        // one-wave tiles cost 0.35 for 68 tiles left over, as much for 73, and 0.9 for 105.
+        if (PRISM_SGEMM5_LEFTOVER_HALVES && left * 16 >= 5 * cus && left * 2 <= cus) {
+            main_tiles = tiles - left;
+            leftover_wt = 128;
+        }
     }
     // `edge` selects the zero-filling variants of both kernels (sub-tiles that lie wholly outside C exit at once).
     auto launch = [&](auto edge) {
@@ -1050,7 +1059,12 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
         sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, EDGE><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
             M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
         *rc = check_launch("sgemm_wave_tile_dma_kernel");
-        if (*rc == 0 && leftover_wt == 256) {
+        if (*rc == 0 && leftover_wt == 128) {
+            // 128 x 256 halves of the same kernel, one workgroup to a CU
+            sgemm_wave_tile_dma_kernel<128, 256, 16, 64, 128, EDGE><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 2), dim3(256), 0, s>>>(
+                M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, main_tiles);
+            *rc = check_launch("sgemm_wave_tile_dma_kernel (leftover halves)");
+        } else if (*rc == 0 && leftover_wt == 256) {
             // 64 x 256 slices of the same kernel, three workgroups to a CU
             sgemm_wave_tile_dma_kernel<64, 256, 16, 32, 128, EDGE><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 4), dim3(256), 0, s>>>(
                 M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, main_tiles);

@@ -193,13 +193,14 @@ def test_wave_tile_one_wave_per_tile_path(prism, oracle, shape):
 
 
 @pytest.mark.parametrize("shape", [(4352, 4352, 64), (4096, 5120, 80), (5120, 5120, 80), (5120, 5120, 48), (4608, 4608, 64),
-                                   (4096, 4352, 96)])
+                                   (4096, 4352, 96), (4864, 4864, 64), (4736, 4740, 68)])
 def test_wave_tile_leftover_round(prism, oracle, shape):
     """Whole 256 x 256 tiles that do not fill whole rounds of the 256 CUs: the last, partial round is cut
     into smaller tiles by a second launch: 64 x 256 slices of the same kernel when that gives every CU one
     (289 tiles: 33 left over; 320: 64 left over) or three (400: 144 left over), else one-wave tiles (324: 68 left
-    over as 64 x 64 tiles; 272: 16 left over as 32 x 32). With K below 64 (fourth shape) the big kernel takes every
-    tile. Every element is checked."""
+    over as 64 x 64 tiles; 272: 16 left over as 32 x 32), and 128 x 256 halves for 80 to 128 tiles left over (361
+    tiles: 105 left over, whole and ragged). With K below 64 (fourth shape) the big kernel takes every tile. Every
+    element is checked."""
     M, N, K = shape
     A, B, Cm = oracle.gen_sgemm(M, N, K, seed=M + K)
     got = run(prism, 5, 1.25, A, B, 0.5, Cm)
