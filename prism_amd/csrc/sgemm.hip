@@ -17,10 +17,11 @@
 // sub-tiles with v_mfma_f32_32x32x2_f32 instead of per-thread outer products;
 // its summation order inside the matrix unit is not specified, so it is
 // checked against an fp64 product within a tolerance. It comes in three forms,
-// chosen by the launcher from the tile count: a 256 x 256 direct-to-LDS kernel
-// for problems with enough such tiles to fill the chip, a one-wave-per-tile
-// kernel for small problems and for the tiles of a partial last round of the
-// big kernel, and the general 128 x 128 block kernel for what lies in between.
+// chosen by the launcher from the tile count: a direct-to-LDS kernel on
+// 256 x 256 tiles for problems with enough such tiles to fill the chip (on
+// 128 x 256 or 64 x 256 tiles below that, and for a partial last round), a
+// one-wave-per-tile kernel for small problems and for some partial rounds, and
+// the general 128 x 128 block kernel for shapes and alignments the others refuse.
 // The two direct-to-LDS kernels have edge variants for ragged M, N, K with N and K
 // multiples of 4 (16 B-aligned rows): their loads go through buffer descriptors
 // whose range check zero-fills everything beyond the matrices. Other shapes and
