@@ -1275,6 +1275,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
 #ifndef PRISM_BF16_SMALL_MAX_QUARTERS
 #define PRISM_BF16_SMALL_MAX_QUARTERS 2
 #endif
+#ifndef PRISM_BF16_SMALL_DEEP_RING
+#define PRISM_BF16_SMALL_DEEP_RING 1
+#endif
 #ifndef PRISM_BF16_RING_BK
 #define PRISM_BF16_RING_BK 64
 #endif
@@ -1333,8 +1336,12 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
                 R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
         if (int rc = check_launch("gemm_bf16_staged_kernel")) return rc;
         if (cut) {
-            gemm_bf16_ring_kernel<128, 128, 64, 2, 64, 64, false, OutT><<<dim3(static_cast<unsigned>(left) * 4), dim3(256), 0, s>>>(
-                R, Cn, K, P, Q, OUT, tiles_m, tiles_n, main_tiles);
+            if (PRISM_BF16_SMALL_DEEP_RING && left * 4 <= cus)  // one per CU: the four-deep ring, as below
+                gemm_bf16_ring_kernel<128, 128, 64, 4, 64, 64, false, OutT><<<dim3(static_cast<unsigned>(left) * 4), dim3(256), 0, s>>>(
+                    R, Cn, K, P, Q, OUT, tiles_m, tiles_n, main_tiles);
+            else
+                gemm_bf16_ring_kernel<128, 128, 64, 2, 64, 64, false, OutT><<<dim3(static_cast<unsigned>(left) * 4), dim3(256), 0, s>>>(
+                    R, Cn, K, P, Q, OUT, tiles_m, tiles_n, main_tiles);
             return check_launch("gemm_bf16_ring_kernel (leftover)");
         }
         return 0;
@@ -1343,8 +1350,15 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
     if (few_tiles && aligned && K % 8 == 0 && K > 0 && panel_ok) {
         const int tm = ceil_div(R, 128), tn = ceil_div(Cn, 128);
         const dim3 grid128(static_cast<unsigned>(tm) * tn);
-        if (R % 128 == 0 && Cn % 128 == 0 && K % 64 == 0 && K >= 128)
+        const bool whole128 = R % 128 == 0 && Cn % 128 == 0 && K % 64 == 0;
+        // At most one workgroup per CU: nothing else hides the memory latency, so the ring is four K tiles
+        // deep (128 KB of LDS) instead of two.
+        if (PRISM_BF16_SMALL_DEEP_RING && whole128 && K >= 256 && tm * tn <= cu_count())
+            gemm_bf16_ring_kernel<128, 128, 64, 4, 64, 64, false, OutT><<<grid128, dim3(256), 0, s>>>(R, Cn, K, P, Q, OUT, tm, tn, -1);
+        else if (whole128 && K >= 128)
             gemm_bf16_ring_kernel<128, 128, 64, 2, 64, 64, false, OutT><<<grid128, dim3(256), 0, s>>>(R, Cn, K, P, Q, OUT, tm, tn, -1);
+        else if (PRISM_BF16_SMALL_DEEP_RING && K >= 256 && tm * tn <= cu_count())
+            gemm_bf16_ring_kernel<128, 128, 64, 4, 64, 64, true, OutT><<<grid128, dim3(256), 0, s>>>(R, Cn, K, P, Q, OUT, tm, tn, -1);
         else
             gemm_bf16_ring_kernel<128, 128, 64, 2, 64, 64, true, OutT><<<grid128, dim3(256), 0, s>>>(R, Cn, K, P, Q, OUT, tm, tn, -1);
         return check_launch("gemm_bf16_ring_kernel (128 x 128)");
