@@ -55,6 +55,11 @@
 #define PRISM_BF16_M16_LOAD_J 3   // ... and the global load, which must come after the write of the same packet
                                   // (2/3, 2/6, 1/5, 3/7 all within 0.5 % of each other; 6/7 is 5 % slower at 8192^3)
 #endif
+#ifndef PRISM_BF16_K_STAGGER
+#define PRISM_BF16_K_STAGGER 64  // gemm_bf16_early_kernel: K tiles (of 128 B) between the starting points of two XCDs; 0: all start at 0.
+// 8192 x 8192 x K, TFLOP/s without / with 64: K = 12288 1316 / 1427, 6144 1432 / 1495, 10240 1436 / 1502, 14336 1507 / 1522,
+// 8192 and 4096 level, 24576 1302 / 1273. Steps of 2 and 8 tiles (256 B, 1 KB) gain nothing, 16 half of it, 32 the same.
+#endif
 #ifndef PRISM_BF16_EARLY_BARRIER_AT
 #define PRISM_BF16_EARLY_BARRIER_AT 36  // gemm_bf16_early_kernel: instructions of a phase before the barrier that frees its stage
 #endif
@@ -1190,13 +1195,27 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     // Tile t lives in stage t % 2. Whole tiles: the launcher guarantees an even number of K tiles, at least 4;
     // EDGE: the count is padded to one (the padding tiles load zeros).
     const int k_tiles = EDGE ? (ceil_div(K, BK) < 4 ? 4 : (ceil_div(K, BK) + 1) / 2 * 2) : K / BK;
+    // Whole tiles: the workgroups of XCD x start their walk along K at tile k_first = x * stagger (even) and
+    // wrap around, so that at any time the eight XCDs fetch from eight different column windows of the
+    // operands instead of all 256 workgroups from the same 128 B of 8192 rows. (All workgroups of one XCD
+    // keep the same phase: they share panels through its L2.)
+    int k_first = 0;
+    if constexpr (!EDGE && PRISM_BF16_K_STAGGER != 0) {
+        const int step = PRISM_BF16_K_STAGGER > 0 ? PRISM_BF16_K_STAGGER : (k_tiles / kXcds) & ~1;
+        k_first = __builtin_amdgcn_readfirstlane((static_cast<int>(blockIdx.x % kXcds) * step) % k_tiles);
+    }
+    auto k_bytes_of = [&](int t) -> uint32_t {  // byte offset along K of the t-th tile of this workgroup's walk
+        const int at = t + k_first;
+        return static_cast<uint32_t>(at < k_tiles ? at : at - k_tiles) * (BK * 2);
+    };
     {
+        const i32x4 pd = advanced(p_rsrc, k_bytes_of(0)), qd = advanced(q_rsrc, k_bytes_of(0));
         const uint32_t off = lane_offset_at(0);
 #pragma unroll
-        for (int m = 0; m < LOADS; ++m) issue_load(0, p_rsrc, q_rsrc, off, m);
+        for (int m = 0; m < LOADS; ++m) issue_load(0, pd, qd, off, m);
     }
     {
-        const i32x4 pd = advanced(p_rsrc, BK * 2), qd = advanced(q_rsrc, BK * 2);
+        const i32x4 pd = advanced(p_rsrc, k_bytes_of(1)), qd = advanced(q_rsrc, k_bytes_of(1));
         const uint32_t off = lane_offset_at(BK);
 #pragma unroll
         for (int m = 0; m < LOADS; ++m) issue_load(1, pd, qd, off, m);
@@ -1215,8 +1234,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
         // independent of what the compiler puts at the head of the loop, and cost nothing measurable.
         asm volatile("s_nop 4");
         const int next = t + 2 < k_tiles ? t + 2 : k_tiles - 2;
-        phase(s0{}, static_cast<uint32_t>(next) * (BK * 2));
-        phase(s1{}, static_cast<uint32_t>(next + 1) * (BK * 2));
+        const uint32_t k_next_bytes = k_bytes_of(next);  // k_first and next are even: next + 1 does not wrap
+        phase(s0{}, k_next_bytes);
+        phase(s1{}, k_next_bytes + BK * 2);
     }
     // k-step 1 of the last tile (stage 1 -> set 2). Outside the loop the compiler is free to move accumulators
     // to other registers; it does so between these instructions, so here they are issued through the builtin,

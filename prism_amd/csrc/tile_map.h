@@ -21,7 +21,10 @@
 namespace prism {
 
 constexpr int kXcds = 8;
-constexpr int kGroupM = 8;
+#ifndef PRISM_TILE_GROUP_M
+#define PRISM_TILE_GROUP_M 8
+#endif
+constexpr int kGroupM = PRISM_TILE_GROUP_M;  // rows of tiles in one XCD's patch
 #ifndef PRISM_TILE_SUPER
 #define PRISM_TILE_SUPER 16
 #endif
