@@ -39,9 +39,9 @@ PEAK = {  # MI355X published peaks
 # counters read for a 1 GiB copy (`--workload calibrate`): FETCH_SIZE x 2.0, WRITE_SIZE x 1.0
 # (summaries under profiles/). None where not measured for that shape.
 TRAFFIC_BYTES = {
-    ("sgemm", 8192, 5): (4016897 + 262144) * 1024,
-    ("scan", 1 << 30): (4201770 + 4201210) * 1024,
-    ("gemm_bf16", 8192): (1584263 + 271766) * 1024,
+    ("sgemm", 8192, 5): (4074176 + 262144) * 1024,
+    ("scan", 1 << 30): (4201763 + 4201231) * 1024,
+    ("gemm_bf16", 8192): (1582365 + 273438) * 1024,
     ("add_m", 1 << 24): (65555 + 65536) * 1024,
 }
 
