@@ -272,6 +272,7 @@ def main() -> int:
     ap.add_argument("--workload", default="all", choices=["all", "sgemm", "scan", "gemm_bf16", "add_m", "calibrate"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--sweep", action="store_true", help="also time every BASELINE config (table on stderr)")
+    ap.add_argument("--sweep-out", default=None, help="with --sweep: also write the table to this JSON file")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no multi-GPU part); run with --gpus 1",
@@ -338,9 +339,10 @@ def main() -> int:
             sweep[f"gemm_bf16_{n}"] = r
             log(f"  gemm_bf16 {n}^3: {r['ms']:.3f} ms  {r['tflops']:.1f} TFLOP/s "
                 f"({100 * r['roofline']['frac']:.1f}% of bf16 MFMA peak)")
-        os.makedirs("gpurun_out", exist_ok=True)
-        with open("gpurun_out/sweep.json", "w") as f:
-            json.dump(sweep, f, indent=1)
+        if args.sweep_out:
+            os.makedirs(os.path.dirname(os.path.abspath(args.sweep_out)), exist_ok=True)
+            with open(args.sweep_out, "w") as f:
+                json.dump(sweep, f, indent=1)
 
     cpu = {}
     if not args.no_cpu_baseline:
