@@ -102,6 +102,16 @@ int prism_scan_exclusive_i32(const int32_t* in, int32_t* out, size_t n, void* wo
                              size_t workspace_bytes, void* stream);
 
 /*
+ * Running maximum of signed 32-bit integers, out[i] = max(in[0], ..., in[i]): the same single-pass kernel
+ * with the addition of scan_kernel's stages (examples/scan.py:106-173, the combination of aggregates in
+ * lookback_to_prev_blocks :34-85) replaced by a maximum and 0 by INT32_MIN. Arguments, workspace and
+ * aliasing rules as for prism_scan_i32; tiles are always numbered by workgroup id. The reference scans
+ * sums only; this is the operator form of the same decomposition.
+ */
+int prism_scan_max_i32(const int32_t* in, int32_t* out, size_t n, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
+/*
  * The reference launcher's own shape: in-place on x, default stream, returns
  * the device pointer that holds the result (x) or NULL on failure.
  * Replaces scan_gpu::launch_scan (evals/4090_scan/main.cu:68-86). Unlike the

@@ -41,6 +41,8 @@ def lib() -> C.CDLL:
         L.oracle_scan_cpu.restype = None
         L.oracle_scan_exclusive_cpu.argtypes = [sz, vp, vp]
         L.oracle_scan_exclusive_cpu.restype = None
+        L.oracle_scan_max_cpu.argtypes = [sz, vp, vp]
+        L.oracle_scan_max_cpu.restype = None
         L.oracle_scan_lookback.argtypes = [sz, vp, C.c_uint]
         L.oracle_scan_lookback.restype = sz
         L.oracle_sgemm_fma.argtypes = [C.c_int, C.c_int, C.c_int, f32, vp, vp, f32, vp]
@@ -102,6 +104,14 @@ def scan_exclusive_cpu(x: np.ndarray) -> np.ndarray:
     out = np.empty_like(xu)
     lib().oracle_scan_exclusive_cpu(xu.size, _p(xu), _p(out))
     return out.view(dt)
+
+
+def scan_max_cpu(x: np.ndarray) -> np.ndarray:
+    """Serial running maximum of int32: out[i] = max(x[0], ..., x[i])."""
+    xi = _c(x, np.int32)
+    out = np.empty_like(xi)
+    lib().oracle_scan_max_cpu(xi.size, _p(xi), _p(out))
+    return out
 
 
 def scan_lookback(x: np.ndarray, stall_every: int = 0) -> np.ndarray:

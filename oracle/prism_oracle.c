@@ -15,6 +15,8 @@
  *   oracle_scan_cpu         closed forms (all-ones -> i+1, wrap cases), numpy.cumsum(int32),
  *                           difference invariant out[i]-out[i-1] == x[i]
  *   oracle_scan_exclusive_cpu  closed forms (all-ones -> i, wrap), inclusive[i] - x[i], shifted numpy.cumsum
+ *   oracle_scan_max_cpu     closed forms (rising -> itself, falling -> first element, INT32_MIN / INT32_MAX),
+ *                           numpy.maximum.accumulate, monotone and out[i] >= x[i] with equality where out steps
  *   oracle_scan_lookback    equality with oracle_scan_cpu on the reference's own test sizes
  *                           and distribution; tail beyond the last full block left untouched
  *   oracle_sgemm_fma        brute-force exact rational/fp64 check on small integer-valued
@@ -60,6 +62,17 @@ void oracle_scan_exclusive_cpu(size_t n, const uint32_t* x, uint32_t* out) {
         const uint32_t element = x[i];  /* x may be out */
         out[i] = accumulator;
         accumulator = accumulator + element;
+    }
+}
+
+/* The same serial loop with a maximum of signed 32-bit integers in place of the sum: out[i] =
+ * max(x[0], ..., x[i]). No reference counterpart (the reference scans sums, scan_harness.cuh:30-36); it is
+ * the serial definition the running-maximum entry point of the library is checked against. */
+void oracle_scan_max_cpu(size_t n, const int32_t* x, int32_t* out) {
+    int32_t best = INT32_MIN;
+    for (size_t i = 0; i < n; i++) {
+        if (x[i] > best) best = x[i];
+        out[i] = best;
     }
 }
 

@@ -133,19 +133,69 @@ __device__ __forceinline__ uint32_t wave_last_lane(uint32_t x) {
     return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(x), 63));
 }
 
+// The operator of the scan: elements travel as 32-bit patterns; `identity` is what padding and "nothing
+// before this" contribute.
+struct SumOp {
+    static constexpr bool kIsSum = true;
+    static constexpr uint32_t identity = 0u;
+    static __device__ __forceinline__ uint32_t apply(uint32_t a, uint32_t b) { return a + b; }
+};
+struct MaxI32Op {  // running maximum of signed 32-bit integers
+    static constexpr bool kIsSum = false;
+    static constexpr uint32_t identity = 0x80000000u;  // INT32_MIN
+    static __device__ __forceinline__ uint32_t apply(uint32_t a, uint32_t b) {
+        const int x = static_cast<int>(a), y = static_cast<int>(b);
+        return static_cast<uint32_t>(x > y ? x : y);
+    }
+};
+
+// Inclusive scan across the wavefront for any operator: lanes without a source (the first lanes of a row
+// for the shifts, the rows a broadcast is masked off for) receive the identity, through the DPP `old`
+// operand instead of the zero fill.
+template <typename Op, int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_or_identity(uint32_t x) {
+    return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(static_cast<int>(Op::identity), static_cast<int>(x), CTRL,
+                                                             ROW_MASK, 0xf, false));
+}
+template <typename Op>
+__device__ __forceinline__ uint32_t wave_inclusive_scan_op(uint32_t x) {
+    if constexpr (Op::kIsSum) {
+        return wave_inclusive_scan(x);
+    } else {
+        x = Op::apply(x, dpp_or_identity<Op, 0x111, 0xf>(x));
+        x = Op::apply(x, dpp_or_identity<Op, 0x112, 0xf>(x));
+        x = Op::apply(x, dpp_or_identity<Op, 0x114, 0xf>(x));
+        x = Op::apply(x, dpp_or_identity<Op, 0x118, 0xf>(x));
+        x = Op::apply(x, dpp_or_identity<Op, 0x142, 0xa>(x));
+        x = Op::apply(x, dpp_or_identity<Op, 0x143, 0xc>(x));
+        return x;
+    }
+}
+// What the lanes before this one combine to (the identity in lane 0), from the inclusive result.
+template <typename Op>
+__device__ __forceinline__ uint32_t wave_exclusive_from_inclusive(uint32_t inclusive, uint32_t own, int lane) {
+    if constexpr (Op::kIsSum) {
+        return inclusive - own;
+    } else {
+        const uint32_t up = static_cast<uint32_t>(__shfl_up(static_cast<int>(inclusive), 1, kWave));
+        return lane == 0 ? Op::identity : up;
+    }
+}
+
 // Exclusive prefix of tile `tile` (> 0): the sum of all earlier tiles. Run by
 // one whole wavefront; lane l inspects tile (window_end - l). Every tile below
 // `tile` is running or finished (see "Tile order" above) and will publish without
 // waiting for anything later, so the loop terminates; the spin limit is a guard.
+template <typename Op>
 __device__ __forceinline__ uint32_t look_back(const u64* status, uint32_t tile, int lane, uint32_t spin_limit,
                                               uint32_t* timed_out) {
-    uint32_t sum = 0;
+    uint32_t sum = Op::identity;
     uint32_t spins = 0;
     long long window_end = static_cast<long long>(tile) - 1;
     while (true) {
         const long long t = window_end - lane;
-        // Tiles "before the first" count as a published prefix of 0.
-        const u64 w = (t >= 0) ? poll(&status[t]) : pack_status(kPrefix, 0);
+        // Tiles "before the first" count as a published prefix of nothing.
+        const u64 w = (t >= 0) ? poll(&status[t]) : pack_status(kPrefix, Op::identity);
         const uint32_t state = static_cast<uint32_t>(w);
         const uint32_t value = static_cast<uint32_t>(w >> 32);
         const u64 has_prefix = __ballot(state == kPrefix);
@@ -160,8 +210,8 @@ __device__ __forceinline__ uint32_t look_back(const u64* status, uint32_t tile, 
             __builtin_amdgcn_s_sleep(PRISM_SCAN_SLEEP);
             continue;
         }
-        const uint32_t contrib = ((needed >> lane) & 1ull) ? value : 0u;
-        sum += wave_last_lane(wave_inclusive_scan(contrib));
+        const uint32_t contrib = ((needed >> lane) & 1ull) ? value : Op::identity;
+        sum = Op::apply(sum, wave_last_lane(wave_inclusive_scan_op<Op>(contrib)));
         if (has_prefix) break;
         window_end -= kWave;
     }
@@ -172,7 +222,8 @@ __device__ __forceinline__ uint32_t look_back(const u64* status, uint32_t tile, 
 // TICKET: tiles are numbered by the ticket counter, else by workgroup id.
 // EXCLUSIVE: out[i] is the sum of the elements before i (out[0] = 0) instead of up to and including i;
 // only the write-back differs.
-template <typename Cfg, bool VEC, bool TICKET, bool EXCLUSIVE>
+// Op: the operator (sums by default; the other operators are inclusive only).
+template <typename Cfg, bool VEC, bool TICKET, bool EXCLUSIVE, typename Op = SumOp>
 __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_t* in, uint32_t* out,
                                                                    size_t n, uint32_t* header,
                                                                    u64* status, uint32_t spin_limit) {
@@ -182,6 +233,7 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
     constexpr int WAVE_ELEMS = kWave * VPT * 4;
     constexpr int ROW_ELEMS = kWave * 4;  // elements one wave instruction covers
     static_assert(BLOCK % kWave == 0 && BLOCK <= 1024, "block must be whole waves");
+    static_assert(Op::kIsSum || !EXCLUSIVE, "the exclusive write-back is written for sums");
 
     __shared__ uint32_t s_tile;
     __shared__ uint32_t s_wave_total[WAVES];
@@ -231,7 +283,7 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const size_t i = lane_base + j * ROW_ELEMS + c;
-                v[j][c] = (i < n) ? in[i] : 0u;
+                v[j][c] = (i < n) ? in[i] : Op::identity;
             }
         }
     }
@@ -239,58 +291,65 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
     // Lane-local inclusive sums of each packet, then the packet totals are
     // scanned across the wave; rows are chained by the wave-uniform carry.
     uint32_t offset[VPT];
-    uint32_t carry = 0;
+    uint32_t carry = Op::identity;
 #pragma unroll
     for (int j = 0; j < VPT; ++j) {
-        v[j].y += v[j].x;
-        v[j].z += v[j].y;
-        v[j].w += v[j].z;
-        const uint32_t inclusive = wave_inclusive_scan(v[j].w);
-        offset[j] = carry + (inclusive - v[j].w);
-        carry += wave_last_lane(inclusive);
+        v[j].y = Op::apply(v[j].y, v[j].x);
+        v[j].z = Op::apply(v[j].z, v[j].y);
+        v[j].w = Op::apply(v[j].w, v[j].z);
+        const uint32_t inclusive = wave_inclusive_scan_op<Op>(v[j].w);
+        offset[j] = Op::apply(carry, wave_exclusive_from_inclusive<Op>(inclusive, v[j].w, lane));
+        carry = Op::apply(carry, wave_last_lane(inclusive));
     }
     if (lane == 0) s_wave_total[wave] = carry;
     __syncthreads();
 
-    uint32_t wave_prefix = 0;
-    uint32_t aggregate = 0;
+    uint32_t wave_prefix = Op::identity;
+    uint32_t aggregate = Op::identity;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) {
         const uint32_t t = s_wave_total[w];
-        if (w < wave) wave_prefix += t;
-        aggregate += t;
+        if (w < wave) wave_prefix = Op::apply(wave_prefix, t);
+        aggregate = Op::apply(aggregate, t);
     }
 
     if (wave == 0) {
-        uint32_t prefix = 0;
+        uint32_t prefix = Op::identity;
         if (tile == 0) {
             if (lane == 0) publish(&status[0], kPrefix, aggregate);
         } else {
             if (lane == 0) publish(&status[tile], kAggregate, aggregate);
-            prefix = look_back(status, tile, lane, spin_limit, &header[2]);
-            if (lane == 0) publish(&status[tile], kPrefix, aggregate + prefix);
+            prefix = look_back<Op>(status, tile, lane, spin_limit, &header[2]);
+            if (lane == 0) publish(&status[tile], kPrefix, Op::apply(aggregate, prefix));
         }
         if (lane == 0) s_tile_prefix = prefix;
     }
     __syncthreads();
-    const uint32_t base_sum = s_tile_prefix + wave_prefix;
+    const uint32_t base_sum = Op::apply(s_tile_prefix, wave_prefix);
 
     if (full) {
 #pragma unroll
         for (int j = 0; j < VPT; ++j) {
             // v[j] holds the running sums inside the packet; shifted by one element they are the exclusive ones.
             const u32x4 sums = EXCLUSIVE ? u32x4{0u, v[j].x, v[j].y, v[j].z} : v[j];
-            const u32x4 r = sums + (offset[j] + base_sum);
+            const uint32_t before = Op::apply(offset[j], base_sum);
+            u32x4 r;
+            if constexpr (Op::kIsSum) {
+                r = sums + before;
+            } else {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) r[c] = Op::apply(sums[c], before);
+            }
             __builtin_nontemporal_store(r, reinterpret_cast<u32x4*>(out + lane_base + j * ROW_ELEMS));
         }
     } else {
 #pragma unroll
         for (int j = 0; j < VPT; ++j) {
-            const uint32_t add = offset[j] + base_sum;
+            const uint32_t add = Op::apply(offset[j], base_sum);
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const size_t i = lane_base + j * ROW_ELEMS + c;
-                if (i < n) out[i] = (EXCLUSIVE ? (c ? v[j][c - 1] : 0u) : v[j][c]) + add;
+                if (i < n) out[i] = Op::apply(EXCLUSIVE ? (c ? v[j][c - 1] : 0u) : v[j][c], add);
             }
         }
     }
@@ -331,9 +390,16 @@ void with_flag(bool flag, F&& f) {
 
 template <typename Cfg>
 int launch_cfg(const uint32_t* in, uint32_t* out, size_t n, uint32_t* header, u64* status, size_t tiles,
-               bool exclusive, hipStream_t s) {
+               bool exclusive, bool maximum, hipStream_t s) {
     const dim3 grid(static_cast<unsigned>(tiles)), block(Cfg::BLOCK);
     const uint32_t limit = spin_limit();
+    if (maximum) {  // tiles by workgroup id only
+        with_flag(aligned16(in) && aligned16(out), [&](auto vec) {
+            scan_lookback_kernel<Cfg, decltype(vec)::value, false, false, MaxI32Op>
+                <<<grid, block, 0, s>>>(in, out, n, header, status, limit);
+        });
+        return check_launch("scan_lookback_kernel (maximum)");
+    }
     with_flag(aligned16(in) && aligned16(out), [&](auto vec) {
         with_flag(ticket_order(), [&](auto ticket) {
             with_flag(exclusive, [&](auto excl) {
@@ -347,6 +413,9 @@ int launch_cfg(const uint32_t* in, uint32_t* out, size_t n, uint32_t* header, u6
 
 }  // namespace
 
+int launch_scan_op(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, bool exclusive,
+                   bool maximum, hipStream_t s);
+
 size_t scan_workspace_bytes(size_t n) {
     const size_t tiles = num_tiles_for(n);
     return kHeaderBytes + sizeof(u64) * (tiles > 0 ? tiles : 1);
@@ -354,6 +423,15 @@ size_t scan_workspace_bytes(size_t n) {
 
 int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, bool exclusive,
                 hipStream_t s) {
+    return launch_scan_op(in, out, n, ws, ws_bytes, exclusive, false, s);
+}
+
+int launch_scan_max(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, hipStream_t s) {
+    return launch_scan_op(in, out, n, ws, ws_bytes, false, true, s);
+}
+
+int launch_scan_op(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, bool exclusive,
+                   bool maximum, hipStream_t s) {
     if (n == 0) return 0;
     if (in == nullptr || out == nullptr || ws == nullptr)
         return fail(1, "prism_scan: null pointer with n=%zu", n);
@@ -382,8 +460,8 @@ int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws
         words, n_words);
     if (int rc = check_launch("scan_reset_kernel")) return rc;
 
-    if (use_small(n)) return launch_cfg<SmallCfg>(in, out, n, ticket, status, tiles, exclusive, s);
-    return launch_cfg<BigCfg>(in, out, n, ticket, status, tiles, exclusive, s);
+    if (use_small(n)) return launch_cfg<SmallCfg>(in, out, n, ticket, status, tiles, exclusive, maximum, s);
+    return launch_cfg<BigCfg>(in, out, n, ticket, status, tiles, exclusive, maximum, s);
 }
 
 }  // namespace prism

@@ -109,6 +109,31 @@ def test_exclusive_scan(prism, oracle, n):
         assert np.array_equal(host(y)[1:], want)
 
 
+@pytest.mark.parametrize("n", [1, 2, 255, 256, 257, 4096, 16385, 65536, 65537, 100_003, (1 << 24) - 1, (1 << 24) + 65536 * 3 + 5,
+                               1 << 26])
+def test_running_maximum(prism, oracle, n):
+    """The operator form of the scan, out[i] = max(in[0..i]) over int32, on both tile shapes: out of place with a
+    fenced output, in place, and from a view that is only 4 B aligned (the scalar path). Three inputs: uniform
+    over all of int32 (new maxima die out quickly), a slow random walk (new maxima throughout, so every stage
+    of the kernel carries a value that matters), and all INT32_MIN (the operator's identity as data)."""
+    lo, hi = np.iinfo(np.int32).min, np.iinfo(np.int32).max
+    rng = np.random.default_rng(n + 2)
+    walk = np.cumsum(rng.integers(-3, 4, n, dtype=np.int64)).clip(lo, hi).astype(np.int32)
+    for x in (rng.integers(lo, hi, n, dtype=np.int32, endpoint=True), walk, np.full(n, lo, dtype=np.int32)):
+        want = oracle.scan_max_cpu(x)
+        out = torch.full((n + 8,), -7, dtype=torch.int32, device=DEV)
+        xd = dev(x)
+        prism.scan(xd, out[:n], op="max")
+        got = host(out)
+        assert np.array_equal(got[:n], want) and np.all(got[n:] == -7)
+        prism.scan(xd, xd, op="max")
+        assert np.array_equal(host(xd), want)
+        if n >= 256:
+            y = torch.zeros(n + 1, dtype=torch.int32, device=DEV)
+            prism.scan(dev(np.concatenate([[0], x]).astype(np.int32))[1:], y[1:], op="max")
+            assert np.array_equal(host(y)[1:], want)
+
+
 @pytest.mark.parametrize("n", [16384, 32768, 1 << 20, 1 << 24, 1 << 26])
 def test_scan_reference_test_sizes_inplace(prism, oracle, n):
     """The reference's own correctness sizes and distribution (evals/4090_scan/main.cu:97-109),

@@ -70,6 +70,22 @@ def test_exclusive_scan_closed_forms_and_relation_to_inclusive(oracle):
         assert np.array_equal(ex.view(np.uint32) + x.view(np.uint32), inc.view(np.uint32))  # exclusive + element
 
 
+def test_running_maximum_closed_forms_library_routine_and_invariants(oracle):
+    rising = np.arange(-40_000, 40_000, dtype=np.int32)
+    assert np.array_equal(oracle.scan_max_cpu(rising), rising)
+    assert np.all(oracle.scan_max_cpu(rising[::-1].copy()) == 39_999)
+    lo, hi = np.iinfo(np.int32).min, np.iinfo(np.int32).max
+    assert oracle.scan_max_cpu(np.array([lo, lo, -7, lo, hi, 3], dtype=np.int32)).tolist() == [lo, lo, -7, -7, hi, hi]
+    assert oracle.scan_max_cpu(np.array([], dtype=np.int32)).size == 0
+    for n in (1, 2, 63, 64, 65, 4097, 100_003):
+        x = np.random.default_rng(n).integers(lo, hi, n, dtype=np.int32, endpoint=True)
+        got = oracle.scan_max_cpu(x)
+        assert np.array_equal(got, np.maximum.accumulate(x))
+        assert np.all(np.diff(got.astype(np.int64)) >= 0) and np.all(got >= x)
+        steps = np.flatnonzero(np.diff(got.astype(np.int64)) > 0) + 1
+        assert got[0] == x[0] and np.array_equal(got[steps], x[steps])  # a new maximum is the element itself
+
+
 def test_scan_vs_numpy_cumsum_and_difference_invariant(oracle):
     for n in (1, 63, 64, 65, 4095, 4096, 4097, 16384, 100_003):
         x = oracle.gen_scan(n, seed=n)
