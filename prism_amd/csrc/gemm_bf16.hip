@@ -1195,12 +1195,12 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     // Tile t lives in stage t % 2. Whole tiles: the launcher guarantees an even number of K tiles, at least 4;
     // EDGE: the count is padded to one (the padding tiles load zeros).
     const int k_tiles = EDGE ? (ceil_div(K, BK) < 4 ? 4 : (ceil_div(K, BK) + 1) / 2 * 2) : K / BK;
-    // Whole tiles: the workgroups of XCD x start their walk along K at tile k_first = x * stagger (even) and
+    // The workgroups of XCD x start their walk along K at tile k_first = x * stagger (even) and
     // wrap around, so that at any time the eight XCDs fetch from eight different column windows of the
     // operands instead of all 256 workgroups from the same 128 B of 8192 rows. (All workgroups of one XCD
     // keep the same phase: they share panels through its L2.)
     int k_first = 0;
-    if constexpr (!EDGE && PRISM_BF16_K_STAGGER != 0) {
+    if constexpr (PRISM_BF16_K_STAGGER != 0) {
         const int step = PRISM_BF16_K_STAGGER > 0 ? PRISM_BF16_K_STAGGER : (k_tiles / kXcds) & ~1;
         k_first = __builtin_amdgcn_readfirstlane((static_cast<int>(blockIdx.x % kXcds) * step) % k_tiles);
     }
@@ -1210,13 +1210,13 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     };
     {
         const i32x4 pd = advanced(p_rsrc, k_bytes_of(0)), qd = advanced(q_rsrc, k_bytes_of(0));
-        const uint32_t off = lane_offset_at(0);
+        const uint32_t off = lane_offset_at(static_cast<int>(k_bytes_of(0) / 2));
 #pragma unroll
         for (int m = 0; m < LOADS; ++m) issue_load(0, pd, qd, off, m);
     }
     {
         const i32x4 pd = advanced(p_rsrc, k_bytes_of(1)), qd = advanced(q_rsrc, k_bytes_of(1));
-        const uint32_t off = lane_offset_at(BK);
+        const uint32_t off = lane_offset_at(static_cast<int>(k_bytes_of(1) / 2));
 #pragma unroll
         for (int m = 0; m < LOADS; ++m) issue_load(1, pd, qd, off, m);
     }
