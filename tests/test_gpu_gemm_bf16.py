@@ -24,8 +24,9 @@ def host(t):
     return t.cpu().numpy()
 
 
-def check_f32(oracle, got, A16, B16):
-    ref = oracle.gemm_bf16_f64(A16, B16)
+def check_f32(oracle, got, A16, B16, ref=None):
+    if ref is None:
+        ref = oracle.gemm_bf16_f64(A16, B16)
     err = np.abs(got - ref)
     scale = float(np.abs(ref).max(initial=0.0))
     assert err.max(initial=0.0) <= REL * scale + 1e-30
@@ -49,27 +50,29 @@ def test_fp32_output_vs_fp64_oracle(prism, oracle, shape):
 @pytest.mark.parametrize("shape", [(256, 256, 128), (256, 512, 192), (512, 256, 256), (256, 256, 320), (512, 512, 1024), (256, 256, 384), (256, 256, 448),
                                    (256, 512, 6144), (512, 256, 6208), (128, 384, 6272),
                                    (3072, 3072, 384), (3072, 3072, 192), (2816, 3328, 448), (3072, 3328, 512),
-                                   (4352, 4352, 384), (4608, 4608, 384), (2560, 2304, 320), (2304, 2560, 448)])
+                                   (4352, 4352, 384), (4608, 4608, 384), (2560, 2304, 320), (2304, 2560, 448),
+                                   (3072, 3072, 1280)])
 def test_whole_tile_paths(prism, oracle, shape):
     """Problems made of whole tiles leave the general kernel. Fewer than 128 tiles of 256 x 256 (the first
     ten shapes and the last two): 128 x 128 tiles, direct-to-LDS ring, four K tiles deep where every CU gets at
     most one tile and K has four tiles (K tile counts of 4, 5, 6, 7, 16, 96, 97 and 98 here), two deep otherwise
-    (K of 128 and 192; the last two shapes with 360 tiles). From 128 tiles up: an even K tile count from 6 up
+    (K of 128 and 192; the two shapes before the last with 360 tiles). From 128 tiles up: an even K tile count from 6 up
     takes the direct-to-LDS pipeline with early fragment reads (6 and 8 K tiles here), the others the
     direct-to-LDS ring of 256 x 256 tiles (3 and 7 K tiles). Two shapes have 289 and 324 tiles for 256 CUs: the 33 or
     68 tiles of the partial second round are cut into 128 x 128 tiles by a second launch (the four-deep ring for
-    132 of them, the two-deep ring for 272). Every element is checked, for both
+    132 of them, the two-deep ring for 272). In that pipeline the workgroups of XCD x start at K tile 64 x modulo
+    the tile count and wrap around: with 6 K tiles at 0, 4, 2, with 20 (the last shape) at 0, 4, 8, 12, 16. Every element is checked, for both
     output types."""
     M, N, K = shape
     A16, B16 = oracle.gen_gemm_bf16(M, N, K, seed=K + M)
     D = prism.gemm_bf16(dev16(A16), dev16(B16))
-    check_f32(oracle, host(D), A16, B16)
+    ref = oracle.gemm_bf16_f64(A16, B16)
+    check_f32(oracle, host(D), A16, B16, ref)
     Cc = torch.full((N * M + 64,), -7.0, dtype=torch.bfloat16, device=DEV)
     prism.runmyh100(M, N, K, dev16(A16), dev16(B16), Cc[32:32 + N * M])
     got = host(Cc.view(torch.int16)).view(np.uint16)
     guard = np.float32(-7.0).view(np.uint32) >> 16
     assert np.all(got[:32] == guard) and np.all(got[32 + N * M:] == guard)
-    ref = oracle.gemm_bf16_f64(A16, B16)
     c = oracle.bf16_to_f32(got[32:32 + N * M]).reshape(N, M).T
     assert np.all(np.abs(c - ref) <= 2.0**-8 * np.abs(ref) + REL * np.abs(ref).max())
 
@@ -84,13 +87,14 @@ def nan_fenced(a16: np.ndarray) -> torch.Tensor:
 @pytest.mark.parametrize("shape", [(1, 1, 8), (257, 255, 8), (300, 520, 392), (255, 513, 456), (512, 512, 72), (1000, 1000, 1000),
                                    (256, 256, 64), (8, 8, 1032), (264, 24, 6152), (777, 300, 128),
                                    (3000, 3080, 392), (2900, 3100, 72), (3072, 3072, 8), (3000, 3072, 264), (2816, 3000, 328),
-                                   (2500, 2300, 264)])
+                                   (2500, 2300, 264), (3000, 3072, 1288)])
 def test_ragged_shapes_with_aligned_rows(prism, oracle, shape):
     """M, N not whole tiles or K not a multiple of 64, K a multiple of 8: the kernels' edge variants
     (rows beyond the matrix and K tiles beyond K read as zeros through the buffer descriptor's range
     check): the ring of 128 x 128 tiles for small problems (four deep up to 256 tiles with K from 256 up, two
-    deep for K below that and for the last shape's 360 tiles), the direct-to-LDS pipeline with early fragment
-    reads from 128 tiles of 256 x 256 up (the five shapes before the last: K tile counts of 7, 2, 1, 5 and 6 before
+    deep for K below that and for the 360 tiles of the shape before the last), the direct-to-LDS pipeline with early fragment
+    reads from 128 tiles of 256 x 256 up (the last shape, 21 K tiles padded to 22 and walked from staggered
+    starting points, and the five shapes before the last two: K tile counts of 7, 2, 1, 5 and 6 before
     padding to an even count of at least 4). The matrices sit between NaNs, so one element read from outside a
     matrix, or from the next row in the partial K tile, would poison the output; stores are fenced too."""
     M, N, K = shape
@@ -100,13 +104,13 @@ def test_ragged_shapes_with_aligned_rows(prism, oracle, shape):
     prism.gemm_bf16(nan_fenced(A16), nan_fenced(B16), D)
     out = host(buf)
     assert np.all(out[:256] == 777.0) and np.all(out[256 + M * N:] == 777.0)
-    check_f32(oracle, out[256:256 + M * N].reshape(M, N), A16, B16)
+    ref = oracle.gemm_bf16_f64(A16, B16)
+    check_f32(oracle, out[256:256 + M * N].reshape(M, N), A16, B16, ref)
     Cc = torch.full((N * M + 64,), -7.0, dtype=torch.bfloat16, device=DEV)
     prism.runmyh100(M, N, K, nan_fenced(A16), nan_fenced(B16), Cc[32:32 + N * M])
     got = host(Cc.view(torch.int16)).view(np.uint16)
     guard = np.float32(-7.0).view(np.uint32) >> 16
     assert np.all(got[:32] == guard) and np.all(got[32 + N * M:] == guard)
-    ref = oracle.gemm_bf16_f64(A16, B16)
     c = oracle.bf16_to_f32(got[32:32 + N * M]).reshape(N, M).T
     assert np.all(np.abs(c - ref) <= 2.0**-8 * np.abs(ref) + REL * np.abs(ref).max())
 
