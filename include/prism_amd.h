@@ -112,6 +112,13 @@ int prism_scan_max_i32(const int32_t* in, int32_t* out, size_t n, void* workspac
                        size_t workspace_bytes, void* stream);
 
 /*
+ * Running minimum, out[i] = min(in[0], ..., in[i]): prism_scan_max_i32 with the order reversed (the
+ * operator form of examples/scan.py:106-173 again, identity INT32_MAX).
+ */
+int prism_scan_min_i32(const int32_t* in, int32_t* out, size_t n, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
+/*
  * The reference launcher's own shape: in-place on x, default stream, returns
  * the device pointer that holds the result (x) or NULL on failure.
  * Replaces scan_gpu::launch_scan (evals/4090_scan/main.cu:68-86). Unlike the

@@ -75,6 +75,12 @@ int prism_scan_max_i32(const int32_t* in, int32_t* out, size_t n, void* workspac
                            workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
+int prism_scan_min_i32(const int32_t* in, int32_t* out, size_t n, void* workspace,
+                       size_t workspace_bytes, void* stream) {
+    return launch_scan_min(reinterpret_cast<const uint32_t*>(in), reinterpret_cast<uint32_t*>(out), n,
+                           workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
 uint32_t* prism_launch_scan(size_t n, uint32_t* x, void* workspace) {
     int rc = launch_scan(x, x, n, workspace, scan_workspace_bytes(n), false, nullptr);
     return rc == 0 ? x : nullptr;

@@ -61,6 +61,7 @@ size_t scan_workspace_bytes(size_t n);
 int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, bool exclusive,
                 hipStream_t s);
 int launch_scan_max(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, hipStream_t s);
+int launch_scan_min(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, hipStream_t s);
 int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, const float* B,
                  float beta, float* C, hipStream_t s);
 int launch_gemm_bf16(int M, int N, int K, const uint16_t* A, const uint16_t* B, float* D_f32,

@@ -133,6 +133,8 @@ __device__ __forceinline__ uint32_t wave_last_lane(uint32_t x) {
     return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(x), 63));
 }
 
+enum { kScanSum = 0, kScanMax = 1, kScanMin = 2 };
+
 // The operator of the scan: elements travel as 32-bit patterns; `identity` is what padding and "nothing
 // before this" contribute.
 struct SumOp {
@@ -146,6 +148,15 @@ struct MaxI32Op {  // running maximum of signed 32-bit integers
     static __device__ __forceinline__ uint32_t apply(uint32_t a, uint32_t b) {
         const int x = static_cast<int>(a), y = static_cast<int>(b);
         return static_cast<uint32_t>(x > y ? x : y);
+    }
+};
+
+struct MinI32Op {  // running minimum of signed 32-bit integers
+    static constexpr bool kIsSum = false;
+    static constexpr uint32_t identity = 0x7fffffffu;  // INT32_MAX
+    static __device__ __forceinline__ uint32_t apply(uint32_t a, uint32_t b) {
+        const int x = static_cast<int>(a), y = static_cast<int>(b);
+        return static_cast<uint32_t>(x < y ? x : y);
     }
 };
 
@@ -390,15 +401,19 @@ void with_flag(bool flag, F&& f) {
 
 template <typename Cfg>
 int launch_cfg(const uint32_t* in, uint32_t* out, size_t n, uint32_t* header, u64* status, size_t tiles,
-               bool exclusive, bool maximum, hipStream_t s) {
+               bool exclusive, int op, hipStream_t s) {
     const dim3 grid(static_cast<unsigned>(tiles)), block(Cfg::BLOCK);
     const uint32_t limit = spin_limit();
-    if (maximum) {  // tiles by workgroup id only
+    if (op != kScanSum) {  // inclusive, tiles by workgroup id only
         with_flag(aligned16(in) && aligned16(out), [&](auto vec) {
-            scan_lookback_kernel<Cfg, decltype(vec)::value, false, false, MaxI32Op>
-                <<<grid, block, 0, s>>>(in, out, n, header, status, limit);
+            if (op == kScanMax)
+                scan_lookback_kernel<Cfg, decltype(vec)::value, false, false, MaxI32Op>
+                    <<<grid, block, 0, s>>>(in, out, n, header, status, limit);
+            else
+                scan_lookback_kernel<Cfg, decltype(vec)::value, false, false, MinI32Op>
+                    <<<grid, block, 0, s>>>(in, out, n, header, status, limit);
         });
-        return check_launch("scan_lookback_kernel (maximum)");
+        return check_launch("scan_lookback_kernel (maximum / minimum)");
     }
     with_flag(aligned16(in) && aligned16(out), [&](auto vec) {
         with_flag(ticket_order(), [&](auto ticket) {
@@ -414,7 +429,7 @@ int launch_cfg(const uint32_t* in, uint32_t* out, size_t n, uint32_t* header, u6
 }  // namespace
 
 int launch_scan_op(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, bool exclusive,
-                   bool maximum, hipStream_t s);
+                   int op, hipStream_t s);
 
 size_t scan_workspace_bytes(size_t n) {
     const size_t tiles = num_tiles_for(n);
@@ -423,15 +438,19 @@ size_t scan_workspace_bytes(size_t n) {
 
 int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, bool exclusive,
                 hipStream_t s) {
-    return launch_scan_op(in, out, n, ws, ws_bytes, exclusive, false, s);
+    return launch_scan_op(in, out, n, ws, ws_bytes, exclusive, kScanSum, s);
 }
 
 int launch_scan_max(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, hipStream_t s) {
-    return launch_scan_op(in, out, n, ws, ws_bytes, false, true, s);
+    return launch_scan_op(in, out, n, ws, ws_bytes, false, kScanMax, s);
+}
+
+int launch_scan_min(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, hipStream_t s) {
+    return launch_scan_op(in, out, n, ws, ws_bytes, false, kScanMin, s);
 }
 
 int launch_scan_op(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, bool exclusive,
-                   bool maximum, hipStream_t s) {
+                   int op, hipStream_t s) {
     if (n == 0) return 0;
     if (in == nullptr || out == nullptr || ws == nullptr)
         return fail(1, "prism_scan: null pointer with n=%zu", n);
@@ -460,8 +479,8 @@ int launch_scan_op(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t
         words, n_words);
     if (int rc = check_launch("scan_reset_kernel")) return rc;
 
-    if (use_small(n)) return launch_cfg<SmallCfg>(in, out, n, ticket, status, tiles, exclusive, maximum, s);
-    return launch_cfg<BigCfg>(in, out, n, ticket, status, tiles, exclusive, maximum, s);
+    if (use_small(n)) return launch_cfg<SmallCfg>(in, out, n, ticket, status, tiles, exclusive, op, s);
+    return launch_cfg<BigCfg>(in, out, n, ticket, status, tiles, exclusive, op, s);
 }
 
 }  // namespace prism

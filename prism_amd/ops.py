@@ -108,13 +108,13 @@ def launch_scan(n: int, x: "torch.Tensor", workspace: "torch.Tensor") -> "torch.
 def scan(inp: "torch.Tensor", out: Optional["torch.Tensor"] = None,
          workspace: Optional["torch.Tensor"] = None, exclusive: bool = False, op: str = "sum") -> "torch.Tensor":
     """Prefix sum modulo 2^32 of a 1-D int32/uint32 tensor; out may be inp. Inclusive (out[i] includes
-    inp[i]) unless exclusive=True (out[0] = 0, out[i] = inp[0] + ... + inp[i-1]). op="max": the running
-    maximum of an int32 tensor instead (inclusive only)."""
-    if op not in ("sum", "max"):
-        raise ValueError("scan: op must be 'sum' or 'max'")
-    if op == "max" and exclusive:
-        raise ValueError("scan: the running maximum is inclusive only")
-    _need(inp, (torch.int32,) if op == "max" else (torch.int32, torch.uint32), 0, "inp")
+    inp[i]) unless exclusive=True (out[0] = 0, out[i] = inp[0] + ... + inp[i-1]). op="max" / op="min": the
+    running maximum / minimum of an int32 tensor instead (inclusive only)."""
+    if op not in ("sum", "max", "min"):
+        raise ValueError("scan: op must be 'sum', 'max' or 'min'")
+    if op != "sum" and exclusive:
+        raise ValueError("scan: the running maximum and minimum are inclusive only")
+    _need(inp, (torch.int32,) if op != "sum" else (torch.int32, torch.uint32), 0, "inp")
     n = inp.numel()
     if out is None:
         out = torch.empty_like(inp)
@@ -124,7 +124,8 @@ def scan(inp: "torch.Tensor", out: Optional["torch.Tensor"] = None,
         workspace = torch.empty(need, dtype=torch.uint8, device=inp.device)
     ws_bytes = workspace.numel() * workspace.element_size()
     lib = _lib.load()
-    fn = lib.prism_scan_max_i32 if op == "max" else (lib.prism_scan_exclusive_i32 if exclusive else lib.prism_scan_i32)
+    fn = {"max": lib.prism_scan_max_i32, "min": lib.prism_scan_min_i32}.get(
+        op, lib.prism_scan_exclusive_i32 if exclusive else lib.prism_scan_i32)
     _check(fn(_ptr(inp), _ptr(out), n, _ptr(workspace), ws_bytes, _stream()), "scan")
     return out
 

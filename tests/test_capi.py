@@ -42,7 +42,7 @@ def test_every_declaration_cites_the_reference():
     # each entry point's comment names the reference file it replaces
     for name, cite in [("prism_add_m", "add_m_thread.py"), ("prism_scan_workspace_bytes", "4090_scan/main.cu"),
                        ("prism_scan_i32", "scan.py"), ("prism_scan_exclusive_i32", "scan.py:174-193"),
-                       ("prism_scan_max_i32", "scan.py:106-173"),
+                       ("prism_scan_max_i32", "scan.py:106-173"), ("prism_scan_min_i32", "scan.py:106-173"),
                        ("prism_launch_scan", "4090_scan/main.cu"),
                        ("prism_sgemm", "runner.cu"), ("prism_run_my_kernel", "runner.cu"),
                        ("prism_gemm_bf16", "h100_matmul.py"), ("prism_runmyh100", "utils.cuh")]:

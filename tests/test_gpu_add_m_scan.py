@@ -132,6 +132,11 @@ def test_running_maximum(prism, oracle, n):
             y = torch.zeros(n + 1, dtype=torch.int32, device=DEV)
             prism.scan(dev(np.concatenate([[0], x]).astype(np.int32))[1:], y[1:], op="max")
             assert np.array_equal(host(y)[1:], want)
+        # the running minimum is the running maximum of the bitwise complements, complemented (~v = -v - 1
+        # reverses the order of int32 without overflow): checked against the same oracle
+        prism.scan(dev(~x), out[:n], op="min")
+        got = host(out)
+        assert np.array_equal(~got[:n], want) and np.all(got[n:] == -7)
 
 
 @pytest.mark.parametrize("n", [16384, 32768, 1 << 20, 1 << 24, 1 << 26])
