@@ -56,9 +56,10 @@
                                   // (2/3, 2/6, 1/5, 3/7 all within 0.5 % of each other; 6/7 is 5 % slower at 8192^3)
 #endif
 #ifndef PRISM_BF16_K_STAGGER
-#define PRISM_BF16_K_STAGGER 64  // gemm_bf16_early_kernel: K tiles (of 128 B) between the starting points of two XCDs; 0: all start at 0.
+#define PRISM_BF16_K_STAGGER 64  // gemm_bf16_early_kernel: K tiles (of 128 B) between the starting points of two XCDs; 0: all start at 0; -1: K tiles / 8; -2: K tiles / 2.
 // 8192 x 8192 x K, TFLOP/s without / with 64: K = 12288 1316 / 1427, 6144 1432 / 1495, 10240 1436 / 1502, 14336 1507 / 1522,
-// 8192 and 4096 level, 24576 1302 / 1273. Steps of 2 and 8 tiles (256 B, 1 KB) gain nothing, 16 half of it, 32 the same.
+// 8192 and 4096 level, 24576 1302 / 1273. Steps of 2 and 8 tiles (256 B, 1 KB) gain nothing, 16 half of it, 32 the same;
+// at K = 12288 steps of 48, 96, 128 tiles and of half the K tiles give 1395, 1366, 1420, 1345 against 1435 for 64.
 #endif
 #ifndef PRISM_BF16_EARLY_BARRIER_AT
 #define PRISM_BF16_EARLY_BARRIER_AT 36  // gemm_bf16_early_kernel: instructions of a phase before the barrier that frees its stage
@@ -1201,7 +1202,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     // keep the same phase: they share panels through its L2.)
     int k_first = 0;
     if constexpr (PRISM_BF16_K_STAGGER != 0) {
-        const int step = PRISM_BF16_K_STAGGER > 0 ? PRISM_BF16_K_STAGGER : (k_tiles / kXcds) & ~1;
+        const int step = PRISM_BF16_K_STAGGER > 0 ? PRISM_BF16_K_STAGGER : (PRISM_BF16_K_STAGGER == -2 ? (k_tiles / 2) & ~1 : (k_tiles / kXcds) & ~1);
         k_first = __builtin_amdgcn_readfirstlane((static_cast<int>(blockIdx.x % kXcds) * step) % k_tiles);
     }
     auto k_bytes_of = [&](int t) -> uint32_t {  // byte offset along K of the t-th tile of this workgroup's walk
