@@ -127,7 +127,7 @@ def bench_scan(prism, n, steps, warmup, gate=True):
     g.manual_seed(0)
     x = torch.randint(-1000, 1001, (n,), dtype=torch.int32, device="cuda", generator=g)
     out = torch.empty_like(x)
-    ws = torch.empty(prism.get_workspace_size(n), dtype=torch.uint8, device="cuda")
+    ws = prism.new_scan_workspace(n)
     if gate:
         prism.scan(x, out, ws)
         torch.cuda.synchronize()
@@ -142,11 +142,13 @@ def bench_scan(prism, n, steps, warmup, gate=True):
         ok = ok and int(out[-1]) == ((total + 2**31) % 2**32) - 2**31
         if not ok:
             raise RuntimeError(f"scan n={n} failed the parity gate")
-    # Out of place, so no restore is needed between steps; the workspace reset is part of the step,
-    # as the reference times its launcher's memsets (evals/4090_scan/main.cu:81-82).
+    # Out of place, so no restore is needed between steps. A step is the whole call: the kernel itself leaves
+    # the workspace ready for the next call (the reference times two memsets per launch for that,
+    # evals/4090_scan/main.cu:81-82).
     lib, st = _capi()
     xp, op, wp, wb = x.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel()
     ms = time_steps(lambda: lib.prism_scan_i32(xp, op, n, wp, wb, st), steps, warmup)
+    prism.scan_status(ws)  # raises if any timed call gave up in its look-back
     nbytes = 2.0 * 4 * n  # scan_harness.cuh:161
     gbps = nbytes / (ms * 1e-3) / 1e9
     return {"ms": ms, "GBps": gbps,

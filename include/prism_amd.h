@@ -11,8 +11,9 @@
  *   - Functions returning int return 0 on success, otherwise a non-zero
  *     hipError_t value (1 = invalid argument); prism_last_error_string() then
  *     describes the failure for the calling thread.
- *   - No entry point reads or keeps host-side state between calls, so all of
- *     them are re-entrant and may be used from several host threads.
+ *   - No entry point reads the environment or keeps options between calls
+ *     (every choice is an argument), so all of them are re-entrant and may be
+ *     used from several host threads.
  *
  * "Reference" citations below are paths in the manya-bansal/prism tree.
  */
@@ -65,31 +66,79 @@ int prism_add_m(const int32_t* x, int32_t* y, int32_t m, size_t n, void* stream)
 /* ------------------------------------------------------------------ scan -- */
 
 /*
- * Bytes of device workspace prism_scan_i32 / prism_launch_scan need for n
- * elements. Replaces scan_gpu::get_workspace_size
+ * Bytes of device workspace the scans need for n elements: a 256-byte header
+ * and 16 bytes per 16384 elements (the size the reference's launcher uses,
+ * n / 16384 * 16 + 4). Replaces scan_gpu::get_workspace_size
  * (evals/4090_scan/main.cu:63-66). Never 0, so a caller may always allocate it.
+ * A workspace sized for n serves every smaller n too.
  */
 size_t prism_scan_workspace_bytes(size_t n);
+
+/*
+ * Brings a workspace (16-byte aligned) into its initial state: all zeros. Call
+ * it once after allocating (a zero-filled allocation is initialised as well).
+ * The reference clears its workspace with two cudaMemset calls in front of
+ * every launch (evals/4090_scan/main.cu:81-82); here every scan leaves the
+ * workspace ready for the next one, so no clearing launch sits in front of a
+ * scan. Enqueues a fill kernel on `stream` (no memset node, so the call can be
+ * captured into a HIP graph).
+ */
+int prism_scan_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Inclusive prefix sum, out[i] = in[0] + ... + in[i] modulo 2^32 (identical
  * bit patterns for int32 and uint32). Single pass with decoupled look-back
  * between tiles. Any n >= 0; in == out is allowed (in-place, as the reference
- * runs); partial overlap is not. The workspace contents on entry do not
- * matter: the call resets it itself, as the reference launcher does
- * (evals/4090_scan/main.cu:81-82). Two calls that share a workspace must be
- * ordered on one stream.
- * Tiles are numbered by workgroup id; with PRISM_SCAN_ORDER=ticket in the
- * environment (read at every call) by the reference's ticket counter
- * (get_block_idx_from_global_counter, examples/scan.py:88-99). A tile's wait
- * for its predecessors is bounded: should it ever run out, the kernel still
- * finishes, ((uint32_t*)workspace)[2] holds the tile number + 1 and the output
- * is not valid; after every normal call that word is 0.
+ * runs); partial overlap is not. The workspace must be initialised (above) and
+ * hold prism_scan_workspace_bytes(n) bytes; calls that share a workspace must
+ * be ordered on one stream, and may differ in n and in kind.
+ * Tiles are numbered by workgroup id, which relies on workgroups starting in
+ * id order; prism_scan_i32_ex can select the reference's ticket counter
+ * instead. A tile's wait for its predecessors is bounded, so the kernel always
+ * finishes; should a wait ever run out, the output is invalid and
+ * prism_scan_status reports it. Callers that must not return a wrong scan call
+ * prism_scan_status before they use the output.
  * Replaces scan_kernel + its device helpers (examples/scan.py:23-227,
  * generated/scan_kernel.cu:1-29).
  */
 int prism_scan_i32(const int32_t* in, int32_t* out, size_t n, void* workspace,
                    size_t workspace_bytes, void* stream);
+
+/* Flags of prism_scan_i32_ex (one PRISM_SCAN_OP_* value, or-ed with the others). */
+enum {
+    PRISM_SCAN_EXCLUSIVE = 1,     /* prism_scan_exclusive_i32's result                                  */
+    PRISM_SCAN_TICKET_ORDER = 2,  /* tiles numbered by get_block_idx_from_global_counter's ticket        */
+                                  /* (examples/scan.py:88-99) instead of by workgroup id                 */
+    PRISM_SCAN_OP_SUM = 0x00,
+    PRISM_SCAN_OP_MAX = 0x10,     /* prism_scan_max_i32's result (inclusive, workgroup-id order only)    */
+    PRISM_SCAN_OP_MIN = 0x20      /* prism_scan_min_i32's result (inclusive, workgroup-id order only)    */
+};
+
+/* prism_scan_status: a tile gave up waiting for its predecessors. */
+#define PRISM_ERROR_SCAN_ORDER 10001
+
+/*
+ * prism_scan_i32 with every choice spelled out as an argument (the library
+ * reads no environment variables and keeps no options between calls).
+ * spin_limit bounds the polls of one look-back window: negative = the
+ * library's default (2^22, seconds), 0 = every look-back gives up at once,
+ * which exercises the kernel's way out from the host without a stuck
+ * predecessor. The reference's kernel waits without bound
+ * (generated/lookback_to_prev_blocks.cu:12-21).
+ */
+int prism_scan_i32_ex(const int32_t* in, int32_t* out, size_t n, void* workspace,
+                      size_t workspace_bytes, unsigned flags, long long spin_limit,
+                      void* stream);
+
+/*
+ * Waits for `stream`, then reports whether any scan on this workspace since
+ * the last report gave up waiting in its look-back: 0 = none did;
+ * PRISM_ERROR_SCAN_ORDER = one did, the output of that call is invalid, the
+ * error string names the tile, and the workspace has been re-initialised. The
+ * reference has no counterpart (its look-back cannot give up); this is what
+ * turns a broken tile-order assumption into an error instead of a wrong sum.
+ */
+int prism_scan_status(void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Exclusive prefix sum, out[i] = in[0] + ... + in[i-1] modulo 2^32, out[0] = 0: the same single-pass
@@ -121,9 +170,10 @@ int prism_scan_min_i32(const int32_t* in, int32_t* out, size_t n, void* workspac
 /*
  * The reference launcher's own shape: in-place on x, default stream, returns
  * the device pointer that holds the result (x) or NULL on failure.
- * Replaces scan_gpu::launch_scan (evals/4090_scan/main.cu:68-86). Unlike the
- * reference, n need not be a multiple of 16384. The workspace must hold at
- * least prism_scan_workspace_bytes(n) bytes.
+ * Replaces scan_gpu::launch_scan (evals/4090_scan/main.cu:68-86). Like the
+ * reference it accepts a workspace with any contents and clears it inside the
+ * call. Unlike the reference, n need not be a multiple of 16384. The workspace
+ * must hold at least prism_scan_workspace_bytes(n) bytes.
  */
 uint32_t* prism_launch_scan(size_t n, uint32_t* x, void* workspace);
 

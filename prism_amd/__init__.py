@@ -8,15 +8,19 @@ call loads (and, if the file is absent, builds) libprism_amd.so.
 """
 from .ops import (  # noqa: F401
     PrismError,
+    ScanOrderError,
     SGEMM_KERNELS,
     add_m,
     device_info,
     gemm_bf16,
     get_workspace_size,
     launch_scan,
+    new_scan_workspace,
     run_my_kernel,
     runmyh100,
     scan,
+    scan_status,
+    scan_workspace_init,
     sgemm,
     tile_coords,
 )

@@ -19,7 +19,11 @@ SIGNATURES = {
     "prism_tile_coords": (C.c_int, [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "prism_add_m": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_size_t, C.c_void_p]),
     "prism_scan_workspace_bytes": (C.c_size_t, [C.c_size_t]),
+    "prism_scan_workspace_init": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p]),
+    "prism_scan_status": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p]),
     "prism_scan_i32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "prism_scan_i32_ex": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_uint,
+                                    C.c_longlong, C.c_void_p]),
     "prism_scan_exclusive_i32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p]),
     "prism_scan_max_i32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p]),
     "prism_scan_min_i32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p]),

@@ -57,32 +57,57 @@ int prism_add_m(const int32_t* x, int32_t* y, int32_t m, size_t n, void* stream)
 
 size_t prism_scan_workspace_bytes(size_t n) { return scan_workspace_bytes(n); }
 
+static_assert(PRISM_SCAN_EXCLUSIVE == kFlagExclusive && PRISM_SCAN_TICKET_ORDER == kFlagTicket &&
+                  PRISM_SCAN_OP_MAX == kFlagOpMax && PRISM_SCAN_OP_MIN == kFlagOpMin &&
+                  PRISM_ERROR_SCAN_ORDER == kScanOrderError,
+              "include/prism_amd.h and common.h disagree");
+
+static const uint32_t* u32(const int32_t* p) { return reinterpret_cast<const uint32_t*>(p); }
+static uint32_t* u32(int32_t* p) { return reinterpret_cast<uint32_t*>(p); }
+
+int prism_scan_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {
+    return scan_workspace_init(workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int prism_scan_status(void* workspace, size_t workspace_bytes, void* stream) {
+    return scan_status(workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
 int prism_scan_i32(const int32_t* in, int32_t* out, size_t n, void* workspace,
                    size_t workspace_bytes, void* stream) {
-    return launch_scan(reinterpret_cast<const uint32_t*>(in), reinterpret_cast<uint32_t*>(out), n,
-                       workspace, workspace_bytes, false, static_cast<hipStream_t>(stream));
+    return launch_scan(u32(in), u32(out), n, workspace, workspace_bytes, 0u, -1, static_cast<hipStream_t>(stream));
+}
+
+int prism_scan_i32_ex(const int32_t* in, int32_t* out, size_t n, void* workspace, size_t workspace_bytes,
+                      unsigned flags, long long spin_limit, void* stream) {
+    return launch_scan(u32(in), u32(out), n, workspace, workspace_bytes, flags, spin_limit,
+                       static_cast<hipStream_t>(stream));
 }
 
 int prism_scan_exclusive_i32(const int32_t* in, int32_t* out, size_t n, void* workspace,
                              size_t workspace_bytes, void* stream) {
-    return launch_scan(reinterpret_cast<const uint32_t*>(in), reinterpret_cast<uint32_t*>(out), n,
-                       workspace, workspace_bytes, true, static_cast<hipStream_t>(stream));
+    return launch_scan(u32(in), u32(out), n, workspace, workspace_bytes, kFlagExclusive, -1,
+                       static_cast<hipStream_t>(stream));
 }
 
 int prism_scan_max_i32(const int32_t* in, int32_t* out, size_t n, void* workspace,
                        size_t workspace_bytes, void* stream) {
-    return launch_scan_max(reinterpret_cast<const uint32_t*>(in), reinterpret_cast<uint32_t*>(out), n,
-                           workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+    return launch_scan(u32(in), u32(out), n, workspace, workspace_bytes, kFlagOpMax, -1,
+                       static_cast<hipStream_t>(stream));
 }
 
 int prism_scan_min_i32(const int32_t* in, int32_t* out, size_t n, void* workspace,
                        size_t workspace_bytes, void* stream) {
-    return launch_scan_min(reinterpret_cast<const uint32_t*>(in), reinterpret_cast<uint32_t*>(out), n,
-                           workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+    return launch_scan(u32(in), u32(out), n, workspace, workspace_bytes, kFlagOpMin, -1,
+                       static_cast<hipStream_t>(stream));
 }
 
 uint32_t* prism_launch_scan(size_t n, uint32_t* x, void* workspace) {
-    int rc = launch_scan(x, x, n, workspace, scan_workspace_bytes(n), false, nullptr);
+    // The reference's launcher accepts any workspace contents (it clears them itself,
+    // evals/4090_scan/main.cu:81-82), so this one initialises before every scan.
+    if (n == 0) return x;
+    if (scan_workspace_init(workspace, scan_workspace_bytes(n), nullptr) != 0) return nullptr;
+    int rc = launch_scan(x, x, n, workspace, scan_workspace_bytes(n), 0u, -1, nullptr);
     return rc == 0 ? x : nullptr;
 }
 

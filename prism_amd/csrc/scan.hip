@@ -42,12 +42,26 @@
 // workgroups of one XCD, see the kernel), which is deadlock-free as long as the
 // dispatcher starts the workgroups of a 1-D grid in id order on every XCD (then
 // the lowest unfinished tile is always running; this is the same assumption
-// CUB's look-back scan makes on NVIDIA hardware). PRISM_SCAN_ORDER=ticket in the environment selects the
+// CUB's look-back scan makes on NVIDIA hardware). The flag kFlagTicket selects the
 // reference's ticket order instead. In both modes the look-back wait is bounded
 // (kSpinLimit polls, several seconds): a wave that runs out stores the tile number
-// plus one into the workspace header (word 2) and carries on with a wrong prefix,
-// so that a broken ordering assumption shows up as a wrong result, not as a hung
-// GPU.
+// plus one into the workspace header (kHdrReport) and carries on with a wrong
+// prefix, so that the GPU never hangs; scan_status() reads that word after the
+// stream has drained and turns it into an error, so that a broken ordering
+// assumption is reported, not returned as a wrong result.
+//
+// Workspace protocol (no reset launch per call). Every tile owns TWO status words,
+// one per parity of the workspace's call counter. A call with parity p publishes
+// and polls the p words and stores zeros into the other ones, which the previous
+// call on this workspace used (calls that share a workspace are ordered on one
+// stream, so that call has finished). The header records up to which tile each
+// parity may hold non-zero words, so a short call after a long one clears the
+// long one's words as well. The last tile, once its look-back is complete,
+// advances the call counter: by then every tile has published and therefore has
+// read the header (a tile's status address depends on the parity it read). The
+// reference clears its workspace with two memsets in front of every launch
+// (evals/4090_scan/main.cu:81-82); here a workspace is cleared once, by
+// scan_workspace_init(), and each call leaves it ready for the next.
 //
 // Status words use RELAXED agent-scope atomics: the value travels inside the
 // atomic word, no other memory is communicated between tiles, so no fence is
@@ -56,8 +70,6 @@
 //
 // HBM-bound: 8 algorithmic bytes per element (4 B read + 4 B write); status
 // traffic is 8 B per tile plus the polls.
-#include <cstdlib>
-#include <cstring>
 #include <type_traits>
 
 #include "common.h"
@@ -68,30 +80,28 @@ namespace {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned long long u64;
 
-constexpr size_t kHeaderBytes = 256;  // word 0: ticket counter, word 2: look-back time-out report
+// Workspace: a 256-byte header, then two 64-bit status words per tile (word 2 t + p for parity p).
+constexpr size_t kHeaderBytes = 256;
+enum : int {                // header fields, as indices of 32-bit words
+    kHdrTicket = 0,         // ticket counter (ticket order only); 0 between calls
+    kHdrReport = 2,         // look-back time-out report: tile number + 1, sticky until scan_status() reads it
+    kHdrCalls = 4,          // calls completed on this workspace; its low bit is the parity of the next call
+    kHdrDirty0 = 5,         // tiles whose parity-0 words may be non-zero
+    kHdrDirty1 = 6,         // same for parity 1
+};
 constexpr uint32_t kSpinLimit = 1u << 22;  // polls of one look-back window before giving up
 
 // Tile shapes: {threads, 16 B packets per lane}.
 struct SmallCfg { static constexpr int BLOCK = 1024, VPT = 4; };
-#ifndef PRISM_SCAN_BIG_BLOCK
-#define PRISM_SCAN_BIG_BLOCK 1024
-#endif
-#ifndef PRISM_SCAN_BIG_VPT
-#define PRISM_SCAN_BIG_VPT 16
-#endif
-#ifndef PRISM_SCAN_CHUNK
-#define PRISM_SCAN_CHUNK 4  // consecutive tiles per XCD in workgroup-id order; 4-5 measured best, 1 and 32 worst
-#endif
-#ifndef PRISM_SCAN_SLEEP
-#define PRISM_SCAN_SLEEP 1
-#endif
-struct BigCfg { static constexpr int BLOCK = PRISM_SCAN_BIG_BLOCK, VPT = PRISM_SCAN_BIG_VPT; };
+struct BigCfg { static constexpr int BLOCK = 1024, VPT = 16; };
 template <typename Cfg> constexpr int tile_elems() { return Cfg::BLOCK * Cfg::VPT * 4; }
-// Inputs up to this many elements use the small tile.
-#ifndef PRISM_SCAN_SMALL_MAX
-#define PRISM_SCAN_SMALL_MAX ((size_t{1} << 24) - 1)
-#endif
-constexpr size_t kSmallMax = PRISM_SCAN_SMALL_MAX;
+constexpr int kChunk = 4;  // consecutive tiles per XCD in workgroup-id order; 4-5 measured best, 1 and 32 worst
+// Inputs up to this many elements use the small tile; so do inputs that are not 16-byte aligned (their
+// element-wise loads would need more registers than the big tile leaves).
+constexpr size_t kSmallMax = (size_t{1} << 24) - 1;
+// Status words are sized for the small tile whatever tile a call ends up using.
+constexpr size_t kWorkspaceTileElems = 16384;
+static_assert(tile_elems<SmallCfg>() == kWorkspaceTileElems && tile_elems<BigCfg>() >= kWorkspaceTileElems, "");
 
 // Tile states, the three-valued form of the reference's two ready flags
 // (BlockInfo::prefix.ready / aggregate.ready, evals/4090_scan/main.cu:21-37).
@@ -133,7 +143,6 @@ __device__ __forceinline__ uint32_t wave_last_lane(uint32_t x) {
     return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(x), 63));
 }
 
-enum { kScanSum = 0, kScanMax = 1, kScanMin = 2 };
 
 // The operator of the scan: elements travel as 32-bit patterns; `identity` is what padding and "nothing
 // before this" contribute.
@@ -194,19 +203,26 @@ __device__ __forceinline__ uint32_t wave_exclusive_from_inclusive(uint32_t inclu
 }
 
 // Exclusive prefix of tile `tile` (> 0): the sum of all earlier tiles. Run by
-// one whole wavefront; lane l inspects tile (window_end - l). Every tile below
-// `tile` is running or finished (see "Tile order" above) and will publish without
-// waiting for anything later, so the loop terminates; the spin limit is a guard.
+// one whole wavefront; lane l inspects tile (window_end - l), whose status word
+// of this call's parity is status[2 * tile + parity]. Every tile below `tile` is
+// running or finished (see "Tile order" above) and will publish without waiting
+// for anything later, so the loop terminates; the spin limit is a guard, and
+// spin_limit == 0 gives up before the first poll (a host-side way to exercise the
+// way out).
 template <typename Op>
-__device__ __forceinline__ uint32_t look_back(const u64* status, uint32_t tile, int lane, uint32_t spin_limit,
-                                              uint32_t* timed_out) {
+__device__ __forceinline__ uint32_t look_back(const u64* status, uint32_t parity, uint32_t tile, int lane,
+                                              uint32_t spin_limit, uint32_t* report) {
     uint32_t sum = Op::identity;
     uint32_t spins = 0;
     long long window_end = static_cast<long long>(tile) - 1;
     while (true) {
+        if (spins >= spin_limit) {
+            if (lane == 0) __hip_atomic_store(report, tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+        }
         const long long t = window_end - lane;
         // Tiles "before the first" count as a published prefix of nothing.
-        const u64 w = (t >= 0) ? poll(&status[t]) : pack_status(kPrefix, Op::identity);
+        const u64 w = (t >= 0) ? poll(&status[2 * t + parity]) : pack_status(kPrefix, Op::identity);
         const uint32_t state = static_cast<uint32_t>(w);
         const uint32_t value = static_cast<uint32_t>(w >> 32);
         const u64 has_prefix = __ballot(state == kPrefix);
@@ -214,11 +230,8 @@ __device__ __forceinline__ uint32_t look_back(const u64* status, uint32_t tile, 
         // Lanes 0..first-prefix-lane are needed; all 64 when no prefix is in the window.
         const u64 needed = has_prefix ? ((2ull << __builtin_ctzll(has_prefix)) - 1ull) : ~0ull;
         if (is_invalid & needed) {
-            if (++spins > spin_limit) {
-                if (lane == 0) __hip_atomic_store(timed_out, tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                break;
-            }
-            __builtin_amdgcn_s_sleep(PRISM_SCAN_SLEEP);
+            ++spins;
+            __builtin_amdgcn_s_sleep(1);
             continue;
         }
         const uint32_t contrib = ((needed >> lane) & 1ull) ? value : Op::identity;
@@ -227,6 +240,15 @@ __device__ __forceinline__ uint32_t look_back(const u64* status, uint32_t tile, 
         window_end -= kWave;
     }
     return sum;
+}
+
+// 16-byte streaming store. `sc1 nt` writes through towards memory and marks the line for early
+// eviction: measured on 4 GiB streams, stores with sc1 run 2-5 % faster than plain or nt-only ones
+// (every line of the output is written exactly once and never read again by this kernel). The
+// two wait states keep the next instruction from overwriting the data registers while the store
+// still reads them (the compiler does not see a store inside the assembly).
+__device__ __forceinline__ void stream_store(u32x4* p, u32x4 v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
 }
 
 // VEC: in and out are 16 B aligned, full tiles use 16 B accesses.
@@ -253,28 +275,27 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
+    const uint32_t tiles = gridDim.x;
 
     uint32_t tile = blockIdx.x;
-#if PRISM_SCAN_CHUNK > 1
     {
         // Consecutive workgroup ids go to the 8 XCDs in turn, and the XCDs drift apart, so in plain id
         // order half of all tiles start before their predecessor and wait longer for it. Chunks of
-        // PRISM_SCAN_CHUNK consecutive tiles are given to workgroups of one XCD instead (every 8th id),
-        // which start in order; only chunk boundaries cross XCDs. A tile's predecessors then have ids at
-        // most 8 * PRISM_SCAN_CHUNK above its own, far fewer than the workgroups resident at once, so
-        // the lowest unfinished tile is still always running.
-        constexpr uint32_t G = PRISM_SCAN_CHUNK, SPAN = 8 * G;
-        const uint32_t whole = (gridDim.x / SPAN) * SPAN;
+        // kChunk consecutive tiles are given to workgroups of one XCD instead (every 8th id), which
+        // start in order; only chunk boundaries cross XCDs. A tile's predecessors then have ids at
+        // most 8 * kChunk above its own, far fewer than the workgroups resident at once, so the lowest
+        // unfinished tile is still always running.
+        constexpr uint32_t G = kChunk, SPAN = 8 * G;
+        const uint32_t whole = (tiles / SPAN) * SPAN;
         if (tile < whole) {
             const uint32_t xcd = tile % 8, j = tile / 8;
             tile = (j / G) * SPAN + xcd * G + (j % G);
         }
     }
-#endif
     if constexpr (TICKET) {
         // Dynamic tile id: tiles are numbered in the order blocks start running (examples/scan.py:88-99).
         if (tid == 0)
-            s_tile = __hip_atomic_fetch_add(&header[0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_tile = __hip_atomic_fetch_add(&header[kHdrTicket], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         tile = s_tile;
     }
@@ -298,6 +319,11 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
             }
         }
     }
+    // {calls, dirty0, dirty1, -} in one load: the status addresses below depend on it, so it has
+    // completed before this tile publishes anything. Only the last tile of a call writes these words,
+    // and only after every tile has published.
+    u32x4 hdr = {0u, 0u, 0u, 0u};
+    if (wave == 0) hdr = *reinterpret_cast<const u32x4*>(header + kHdrCalls);
 
     // Lane-local inclusive sums of each packet, then the packet totals are
     // scanned across the wave; rows are chained by the wave-uniform carry.
@@ -325,15 +351,30 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
     }
 
     if (wave == 0) {
+        const uint32_t calls = hdr.x;
+        const uint32_t parity = calls & 1u;
+        u64* const mine = &status[2 * static_cast<size_t>(tile) + parity];
         uint32_t prefix = Op::identity;
         if (tile == 0) {
-            if (lane == 0) publish(&status[0], kPrefix, aggregate);
+            if (lane == 0) publish(mine, kPrefix, aggregate);
         } else {
-            if (lane == 0) publish(&status[tile], kAggregate, aggregate);
-            prefix = look_back<Op>(status, tile, lane, spin_limit, &header[2]);
-            if (lane == 0) publish(&status[tile], kPrefix, Op::apply(aggregate, prefix));
+            if (lane == 0) publish(mine, kAggregate, aggregate);
+            prefix = look_back<Op>(status, parity, tile, lane, spin_limit, &header[kHdrReport]);
+            if (lane == 0) publish(mine, kPrefix, Op::apply(aggregate, prefix));
         }
         if (lane == 0) s_tile_prefix = prefix;
+        // Zero the other parity's words: tile t clears words t, t + tiles, ... below that parity's mark.
+        const uint32_t dirty_other = parity ? hdr.y : hdr.z;
+        for (size_t w = tile + static_cast<size_t>(lane) * tiles; w < dirty_other; w += static_cast<size_t>(kWave) * tiles)
+            __hip_atomic_store(&status[2 * w + (parity ^ 1u)], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // The last tile closes the call: every earlier tile has published by now (its look-back saw
+        // them all), so every tile has read the header.
+        if (tile == tiles - 1 && lane == 0) {
+            __hip_atomic_store(&header[kHdrTicket], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&header[kHdrDirty0 + parity], tiles, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&header[kHdrDirty0 + (parity ^ 1u)], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&header[kHdrCalls], calls + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
     __syncthreads();
     const uint32_t base_sum = Op::apply(s_tile_prefix, wave_prefix);
@@ -351,7 +392,7 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
 #pragma unroll
                 for (int c = 0; c < 4; ++c) r[c] = Op::apply(sums[c], before);
             }
-            __builtin_nontemporal_store(r, reinterpret_cast<u32x4*>(out + lane_base + j * ROW_ELEMS));
+            stream_store(reinterpret_cast<u32x4*>(out + lane_base + j * ROW_ELEMS), r);
         }
     } else {
 #pragma unroll
@@ -366,31 +407,13 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
     }
 }
 
-// Clears the ticket counter and every status word (the two memsets of the
-// reference launcher, evals/4090_scan/main.cu:81-82, as one fill kernel).
-__global__ __launch_bounds__(256) void scan_reset_kernel(u64* words, size_t n_words) {
+// Zero fill of a workspace (a kernel, not hipMemsetAsync, so that it can be captured into a graph).
+__global__ __launch_bounds__(256) void scan_fill_zero_kernel(u64* words, size_t n_words) {
     const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
     if (i < n_words) words[i] = 0ull;
 }
 
-inline bool use_small(size_t n) { return n <= kSmallMax; }
-
-inline size_t num_tiles_for(size_t n) {
-    const size_t tile = use_small(n) ? tile_elems<SmallCfg>() : tile_elems<BigCfg>();
-    return ceil_div(n, tile);
-}
-
-// PRISM_SCAN_ORDER=ticket selects the reference's ticket order (read at every call, so a process can
-// switch); PRISM_SCAN_SPIN_LIMIT overrides the look-back bound (0 makes every wait time out at once:
-// the kernel's way out can then be exercised without a stuck predecessor).
-inline bool ticket_order() {
-    const char* v = getenv("PRISM_SCAN_ORDER");
-    return v != nullptr && strcmp(v, "ticket") == 0;
-}
-inline uint32_t spin_limit() {
-    const char* v = getenv("PRISM_SCAN_SPIN_LIMIT");
-    return v != nullptr ? static_cast<uint32_t>(strtoul(v, nullptr, 10)) : kSpinLimit;
-}
+inline bool use_small(size_t n, bool vec) { return n <= kSmallMax || !vec; }
 
 // Calls f with std::true_type or std::false_type for a run-time flag.
 template <typename F>
@@ -399,64 +422,57 @@ void with_flag(bool flag, F&& f) {
     else f(std::false_type{});
 }
 
-template <typename Cfg>
-int launch_cfg(const uint32_t* in, uint32_t* out, size_t n, uint32_t* header, u64* status, size_t tiles,
-               bool exclusive, int op, hipStream_t s) {
+template <typename Cfg, bool VEC>
+int launch_cfg(const uint32_t* in, uint32_t* out, size_t n, uint32_t* header, u64* status, unsigned flags,
+               uint32_t limit, hipStream_t s) {
+    const size_t tiles = ceil_div(n, static_cast<size_t>(tile_elems<Cfg>()));
     const dim3 grid(static_cast<unsigned>(tiles)), block(Cfg::BLOCK);
-    const uint32_t limit = spin_limit();
-    if (op != kScanSum) {  // inclusive, tiles by workgroup id only
-        with_flag(aligned16(in) && aligned16(out), [&](auto vec) {
-            if (op == kScanMax)
-                scan_lookback_kernel<Cfg, decltype(vec)::value, false, false, MaxI32Op>
-                    <<<grid, block, 0, s>>>(in, out, n, header, status, limit);
-            else
-                scan_lookback_kernel<Cfg, decltype(vec)::value, false, false, MinI32Op>
-                    <<<grid, block, 0, s>>>(in, out, n, header, status, limit);
-        });
-        return check_launch("scan_lookback_kernel (maximum / minimum)");
-    }
-    with_flag(aligned16(in) && aligned16(out), [&](auto vec) {
-        with_flag(ticket_order(), [&](auto ticket) {
-            with_flag(exclusive, [&](auto excl) {
-                scan_lookback_kernel<Cfg, decltype(vec)::value, decltype(ticket)::value, decltype(excl)::value>
+    const int op = static_cast<int>(flags & kFlagOpMask);
+    if (op == kFlagOpMax)
+        scan_lookback_kernel<Cfg, VEC, false, false, MaxI32Op><<<grid, block, 0, s>>>(in, out, n, header, status, limit);
+    else if (op == kFlagOpMin)
+        scan_lookback_kernel<Cfg, VEC, false, false, MinI32Op><<<grid, block, 0, s>>>(in, out, n, header, status, limit);
+    else
+        with_flag((flags & kFlagTicket) != 0, [&](auto ticket) {
+            with_flag((flags & kFlagExclusive) != 0, [&](auto excl) {
+                scan_lookback_kernel<Cfg, VEC, decltype(ticket)::value, decltype(excl)::value>
                     <<<grid, block, 0, s>>>(in, out, n, header, status, limit);
             });
         });
-    });
     return check_launch("scan_lookback_kernel");
 }
 
 }  // namespace
 
-int launch_scan_op(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, bool exclusive,
-                   int op, hipStream_t s);
-
 size_t scan_workspace_bytes(size_t n) {
-    const size_t tiles = num_tiles_for(n);
-    return kHeaderBytes + sizeof(u64) * (tiles > 0 ? tiles : 1);
+    const size_t tiles = ceil_div(n, kWorkspaceTileElems);
+    return kHeaderBytes + 16 * (tiles > 0 ? tiles : 1);
 }
 
-int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, bool exclusive,
-                hipStream_t s) {
-    return launch_scan_op(in, out, n, ws, ws_bytes, exclusive, kScanSum, s);
+int scan_workspace_init(void* ws, size_t ws_bytes, hipStream_t s) {
+    if (ws == nullptr || ws_bytes < kHeaderBytes + 16)
+        return fail(1, "prism_scan_workspace_init: workspace of %zu bytes is too small", ws_bytes);
+    if ((reinterpret_cast<uintptr_t>(ws) & 15u) != 0)
+        return fail(1, "prism_scan_workspace_init: workspace must be 16-byte aligned");
+    const size_t n_words = ws_bytes / sizeof(u64);
+    scan_fill_zero_kernel<<<dim3(static_cast<unsigned>(ceil_div(n_words, size_t{256}))), dim3(256), 0, s>>>(
+        reinterpret_cast<u64*>(ws), n_words);
+    return check_launch("scan_fill_zero_kernel");
 }
 
-int launch_scan_max(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, hipStream_t s) {
-    return launch_scan_op(in, out, n, ws, ws_bytes, false, kScanMax, s);
-}
-
-int launch_scan_min(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, hipStream_t s) {
-    return launch_scan_op(in, out, n, ws, ws_bytes, false, kScanMin, s);
-}
-
-int launch_scan_op(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, bool exclusive,
-                   int op, hipStream_t s) {
+int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, unsigned flags,
+                long long spin_limit, hipStream_t s) {
     if (n == 0) return 0;
     if (in == nullptr || out == nullptr || ws == nullptr)
         return fail(1, "prism_scan: null pointer with n=%zu", n);
     if (!aligned4(in) || !aligned4(out)) return fail(1, "prism_scan: data pointers must be 4-byte aligned");
-    if ((reinterpret_cast<uintptr_t>(ws) & 7u) != 0)
-        return fail(1, "prism_scan: workspace must be 8-byte aligned");
+    if ((reinterpret_cast<uintptr_t>(ws) & 15u) != 0)
+        return fail(1, "prism_scan: workspace must be 16-byte aligned");
+    const int op = static_cast<int>(flags & kFlagOpMask);
+    if ((flags & ~(kFlagExclusive | kFlagTicket | kFlagOpMask)) != 0 || op > kFlagOpMin)
+        return fail(1, "prism_scan: unknown flag bits 0x%x", flags);
+    if (op != kFlagOpSum && (flags & (kFlagExclusive | kFlagTicket)) != 0)
+        return fail(1, "prism_scan: the running maximum / minimum is inclusive and numbers tiles by workgroup id");
     const size_t need = scan_workspace_bytes(n);
     if (ws_bytes < need)
         return fail(1, "prism_scan: workspace of %zu bytes is smaller than the %zu needed for n=%zu",
@@ -467,20 +483,35 @@ int launch_scan_op(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t
         if (a < b + bytes && b < a + bytes)
             return fail(1, "prism_scan: in and out overlap without being equal");
     }
-    const size_t tiles = num_tiles_for(n);
-    if (tiles > 0x7fffffffull) return fail(1, "prism_scan: n=%zu too large", n);
+    if (ceil_div(n, kWorkspaceTileElems) > 0x7fffffffull) return fail(1, "prism_scan: n=%zu too large", n);
+    const uint32_t limit = spin_limit < 0 ? kSpinLimit
+                                          : static_cast<uint32_t>(spin_limit > 0xffffffffll ? 0xffffffffll : spin_limit);
 
-    u64* words = reinterpret_cast<u64*>(ws);
-    const size_t n_words = need / sizeof(u64);
-    uint32_t* ticket = reinterpret_cast<uint32_t*>(ws);
+    uint32_t* header = reinterpret_cast<uint32_t*>(ws);
     u64* status = reinterpret_cast<u64*>(static_cast<char*>(ws) + kHeaderBytes);
+    const bool vec = aligned16(in) && aligned16(out);
+    if (!vec) return launch_cfg<SmallCfg, false>(in, out, n, header, status, flags, limit, s);
+    if (use_small(n, vec)) return launch_cfg<SmallCfg, true>(in, out, n, header, status, flags, limit, s);
+    return launch_cfg<BigCfg, true>(in, out, n, header, status, flags, limit, s);
+}
 
-    scan_reset_kernel<<<dim3(static_cast<unsigned>(ceil_div(n_words, size_t{256}))), dim3(256), 0, s>>>(
-        words, n_words);
-    if (int rc = check_launch("scan_reset_kernel")) return rc;
-
-    if (use_small(n)) return launch_cfg<SmallCfg>(in, out, n, ticket, status, tiles, exclusive, op, s);
-    return launch_cfg<BigCfg>(in, out, n, ticket, status, tiles, exclusive, op, s);
+int scan_status(void* ws, size_t ws_bytes, hipStream_t s) {
+    if (ws == nullptr || ws_bytes < kHeaderBytes + 16) return fail(1, "prism_scan_status: workspace of %zu bytes is too small", ws_bytes);
+    hipError_t e = hipStreamSynchronize(s);
+    if (e != hipSuccess) return hip_fail(e, "prism_scan_status: hipStreamSynchronize");
+    uint32_t report = 0;
+    e = hipMemcpy(&report, static_cast<const uint32_t*>(ws) + kHdrReport, sizeof(report), hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return hip_fail(e, "prism_scan_status: hipMemcpy");
+    if (report == 0) return 0;
+    // A tile gave up waiting: its call's output is invalid, and the tile that closes a call may have done
+    // so before every tile had started. Bring the workspace back to its initial state.
+    if (int rc = scan_workspace_init(ws, ws_bytes, s)) return rc;
+    e = hipStreamSynchronize(s);
+    if (e != hipSuccess) return hip_fail(e, "prism_scan_status: hipStreamSynchronize");
+    return fail(kScanOrderError,
+                "prism_scan: tile %u gave up waiting for its predecessors (workgroups did not start in the assumed "
+                "order, or the spin limit was set too low); the output of that call is invalid",
+                report - 1u);
 }
 
 }  // namespace prism

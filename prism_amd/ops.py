@@ -83,6 +83,16 @@ def add_m(x: "torch.Tensor", y: "torch.Tensor", m: int) -> "torch.Tensor":
 
 # -------------------------------------------------------------------- scan --
 
+SCAN_EXCLUSIVE = 1       # flag values of include/prism_amd.h
+SCAN_TICKET_ORDER = 2
+SCAN_OP = {"sum": 0x00, "max": 0x10, "min": 0x20}
+ERROR_SCAN_ORDER = 10001
+
+
+class ScanOrderError(PrismError):
+    """A tile of a scan gave up waiting for its predecessors; that call's output is invalid."""
+
+
 def get_workspace_size(n: int) -> int:
     """Workspace bytes for an n-element scan (scan_gpu::get_workspace_size)."""
     if n < 0:
@@ -90,43 +100,80 @@ def get_workspace_size(n: int) -> int:
     return int(_lib.load().prism_scan_workspace_bytes(n))
 
 
-def launch_scan(n: int, x: "torch.Tensor", workspace: "torch.Tensor") -> "torch.Tensor":
+def _ws_bytes(workspace: "torch.Tensor") -> int:
+    return workspace.numel() * workspace.element_size()
+
+
+def new_scan_workspace(n: int, device="cuda") -> "torch.Tensor":
+    """An initialised (zero-filled) workspace for scans of up to n elements."""
+    return torch.zeros(get_workspace_size(n), dtype=torch.uint8, device=device)
+
+
+def scan_workspace_init(workspace: "torch.Tensor") -> "torch.Tensor":
+    """Bring a workspace into its initial state (needed once; every scan leaves it ready for the next)."""
+    _check(_lib.load().prism_scan_workspace_init(_ptr(workspace), _ws_bytes(workspace), _stream()),
+           "scan_workspace_init")
+    return workspace
+
+
+def scan_status(workspace: "torch.Tensor", stream: Optional[int] = None) -> None:
+    """Wait for the stream and raise ScanOrderError if a scan on this workspace gave up in its look-back."""
+    rc = _lib.load().prism_scan_status(_ptr(workspace), _ws_bytes(workspace), _stream() if stream is None else stream)
+    if rc == ERROR_SCAN_ORDER:
+        raise ScanOrderError(_lib.last_error())
+    _check(rc, "scan_status")
+
+
+def launch_scan(n: int, x: "torch.Tensor", workspace: "torch.Tensor", check: bool = True) -> "torch.Tensor":
     """In-place inclusive scan of the first n elements of x (scan_gpu::launch_scan).
 
     Returns the tensor that holds the result (x itself), as the reference
-    returns its device pointer. Runs on the default stream like the reference.
+    returns its device pointer. Runs on the default stream like the reference,
+    and like the reference accepts a workspace with any contents. With
+    check=True (default) it then waits for the result and raises ScanOrderError
+    if the look-back gave up; check=False leaves the call asynchronous and the
+    check (scan_status) to the caller.
     """
     _need(x, (torch.int32, torch.uint32), n, "x")
-    if workspace.numel() * workspace.element_size() < get_workspace_size(n):
+    if _ws_bytes(workspace) < get_workspace_size(n):
         raise ValueError("workspace smaller than get_workspace_size(n)")
-    out =_lib.load().prism_launch_scan(n, _ptr(x), _ptr(workspace))
+    out = _lib.load().prism_launch_scan(n, _ptr(x), _ptr(workspace))
     if n > 0 and not out:
         raise PrismError(f"launch_scan: {_lib.last_error()}")
+    if check and n > 0:
+        scan_status(workspace, stream=0)
     return x
 
 
 def scan(inp: "torch.Tensor", out: Optional["torch.Tensor"] = None,
-         workspace: Optional["torch.Tensor"] = None, exclusive: bool = False, op: str = "sum") -> "torch.Tensor":
+         workspace: Optional["torch.Tensor"] = None, exclusive: bool = False, op: str = "sum",
+         ticket_order: bool = False, spin_limit: int = -1, check: bool = True) -> "torch.Tensor":
     """Prefix sum modulo 2^32 of a 1-D int32/uint32 tensor; out may be inp. Inclusive (out[i] includes
     inp[i]) unless exclusive=True (out[0] = 0, out[i] = inp[0] + ... + inp[i-1]). op="max" / op="min": the
-    running maximum / minimum of an int32 tensor instead (inclusive only)."""
-    if op not in ("sum", "max", "min"):
+    running maximum / minimum of an int32 tensor instead (inclusive only).
+
+    workspace: an initialised workspace (new_scan_workspace / scan_workspace_init) that calls on one stream
+    may share; None allocates one. ticket_order numbers tiles by the reference's ticket counter instead of
+    by workgroup id; spin_limit bounds the look-back polls (-1: library default, 0: give up at once).
+    check=True (default) waits for the result and raises ScanOrderError if the look-back gave up;
+    check=False leaves the call asynchronous and the check (scan_status) to the caller.
+    """
+    if op not in SCAN_OP:
         raise ValueError("scan: op must be 'sum', 'max' or 'min'")
-    if op != "sum" and exclusive:
-        raise ValueError("scan: the running maximum and minimum are inclusive only")
+    if op != "sum" and (exclusive or ticket_order):
+        raise ValueError("scan: the running maximum and minimum are inclusive and use workgroup-id order")
     _need(inp, (torch.int32,) if op != "sum" else (torch.int32, torch.uint32), 0, "inp")
     n = inp.numel()
     if out is None:
         out = torch.empty_like(inp)
     _need(out, (inp.dtype,), n, "out")
-    need = get_workspace_size(n)
     if workspace is None:
-        workspace = torch.empty(need, dtype=torch.uint8, device=inp.device)
-    ws_bytes = workspace.numel() * workspace.element_size()
-    lib = _lib.load()
-    fn = {"max": lib.prism_scan_max_i32, "min": lib.prism_scan_min_i32}.get(
-        op, lib.prism_scan_exclusive_i32 if exclusive else lib.prism_scan_i32)
-    _check(fn(_ptr(inp), _ptr(out), n, _ptr(workspace), ws_bytes, _stream()), "scan")
+        workspace = new_scan_workspace(n, inp.device)
+    flags = SCAN_OP[op] | (SCAN_EXCLUSIVE if exclusive else 0) | (SCAN_TICKET_ORDER if ticket_order else 0)
+    _check(_lib.load().prism_scan_i32_ex(_ptr(inp), _ptr(out), n, _ptr(workspace), _ws_bytes(workspace), flags,
+                                         int(spin_limit), _stream()), "scan")
+    if check and n > 0:
+        scan_status(workspace)
     return out
 
 

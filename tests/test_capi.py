@@ -24,7 +24,8 @@ def lib():
 
 def test_header_lists_the_expected_entry_points():
     names = declared_functions()
-    for must in ("prism_add_m", "prism_scan_i32", "prism_scan_workspace_bytes", "prism_launch_scan",
+    for must in ("prism_add_m", "prism_scan_i32", "prism_scan_i32_ex", "prism_scan_workspace_bytes",
+                 "prism_scan_workspace_init", "prism_scan_status", "prism_launch_scan",
                  "prism_sgemm", "prism_run_my_kernel", "prism_gemm_bf16", "prism_runmyh100"):
         assert must in names
 
@@ -41,7 +42,8 @@ def test_every_declaration_cites_the_reference():
     text = HEADER.read_text()
     # each entry point's comment names the reference file it replaces
     for name, cite in [("prism_add_m", "add_m_thread.py"), ("prism_scan_workspace_bytes", "4090_scan/main.cu"),
-                       ("prism_scan_i32", "scan.py"), ("prism_scan_exclusive_i32", "scan.py:174-193"),
+                       ("prism_scan_i32", "scan.py"), ("prism_scan_i32_ex", "lookback_to_prev_blocks.cu"),
+                       ("prism_scan_workspace_init", "4090_scan/main.cu:81-82"), ("prism_scan_exclusive_i32", "scan.py:174-193"),
                        ("prism_scan_max_i32", "scan.py:106-173"), ("prism_scan_min_i32", "scan.py:106-173"),
                        ("prism_launch_scan", "4090_scan/main.cu"),
                        ("prism_sgemm", "runner.cu"), ("prism_run_my_kernel", "runner.cu"),
@@ -79,14 +81,24 @@ def test_argument_checks_run_before_any_gpu_work(lib):
     need = lib.prism_scan_workspace_bytes(1 << 20)
     assert lib.prism_scan_i32(0x100000, 0x100000, 1 << 20, 0x9000, need - 1, None) == 1
     assert b"workspace" in lib.prism_last_error_string()
+    # the explicit form: unknown flag bits, flag combinations that do not exist, workspace alignment
+    assert lib.prism_scan_i32_ex(0x100000, 0x100000, 1 << 20, 0x9000, need, 0x40, -1, None) == 1
+    assert b"flag" in lib.prism_last_error_string()
+    assert lib.prism_scan_i32_ex(0x100000, 0x100000, 1 << 20, 0x9000, need, 0x30, -1, None) == 1
+    assert lib.prism_scan_i32_ex(0x100000, 0x100000, 1 << 20, 0x9000, need, 0x10 | 1, -1, None) == 1
+    assert lib.prism_scan_i32_ex(0x100000, 0x100000, 1 << 20, 0x9008, need, 0, -1, None) == 1
+    assert lib.prism_scan_i32_ex(None, None, 0, None, 0, 3, 0, None) == 0
+    assert lib.prism_scan_workspace_init(None, 4096, None) == 1
+    assert lib.prism_scan_workspace_init(0x9000, 8, None) == 1
+    assert lib.prism_scan_workspace_init(0x9004, 4096, None) == 1
 
 
 def test_scan_workspace_size(lib):
     sizes = [lib.prism_scan_workspace_bytes(n) for n in (0, 1, 4096, 4097, 1 << 20, 1 << 30)]
-    assert all(s > 0 and s % 8 == 0 for s in sizes)
+    assert all(s > 0 and s % 16 == 0 for s in sizes)
     assert sizes == sorted(sizes)
-    # 8 bytes of status per tile; the reference uses 16 per 16384 elements (main.cu:63-66)
-    assert sizes[-1] < (1 << 30) // 16384 * 16 * 8
+    # a header plus the reference's 16 bytes per 16384 elements (main.cu:63-66)
+    assert sizes[-1] == 256 + (1 << 30) // 16384 * 16
 
 
 @pytest.mark.parametrize("tiles", [(1, 1), (1, 9), (7, 1), (8, 8), (64, 64), (3, 5), (33, 17), (64, 33), (5, 129)])

@@ -146,7 +146,7 @@ def test_scan_reference_test_sizes_inplace(prism, oracle, n):
     x = oracle.gen_scan_reference_style(n)
     xd = dev(x.view(np.int32))
     ws = torch.empty(prism.get_workspace_size(n), dtype=torch.uint8, device=DEV)
-    ws.fill_(0xAB)  # garbage: the launcher resets the workspace itself
+    ws.fill_(0xAB)  # garbage: this launcher clears the workspace itself, like the reference's
     ret = prism.launch_scan(n, xd, ws)
     assert ret.data_ptr() == xd.data_ptr()
     assert np.array_equal(host(xd).view(np.uint32), oracle.scan_cpu(x))
@@ -159,54 +159,74 @@ def test_scan_baseline_sizes(prism, oracle, n):
     assert np.array_equal(host(out), oracle.scan_cpu(x))
 
 
-@pytest.fixture
-def scan_env(monkeypatch):
-    """The library reads PRISM_SCAN_ORDER / PRISM_SCAN_SPIN_LIMIT at every call."""
-    def set_(order=None, spin_limit=None):
-        for key, val in (("PRISM_SCAN_ORDER", order), ("PRISM_SCAN_SPIN_LIMIT", spin_limit)):
-            if val is None:
-                monkeypatch.delenv(key, raising=False)
-            else:
-                monkeypatch.setenv(key, str(val))
-    yield set_
-    set_()
-
-
 @pytest.mark.parametrize("n", [1, 4097, 65536 * 3 + 5, (1 << 24) + 1, 1 << 26, (1 << 28) + 12345])
-def test_scan_ticket_order_matches_dispatch_order(prism, oracle, scan_env, n):
+def test_scan_ticket_order_matches_dispatch_order(prism, oracle, n):
     """Tiles numbered by the ticket counter (the reference's get_block_idx_from_global_counter,
-    examples/scan.py:88-99) and tiles numbered by workgroup id give the same bits."""
+    examples/scan.py:88-99) and tiles numbered by workgroup id give the same bits, also when the two
+    orders alternate on one workspace (the ticket counter is back at zero after every call)."""
     x = oracle.gen_scan(n, seed=n % 1000)
     want = oracle.scan_cpu(x)
     xd = dev(x)
-    for order in ("ticket", None):
-        scan_env(order=order)
-        out = prism.scan(xd)
-        assert np.array_equal(host(out), want), order
+    ws = prism.new_scan_workspace(n)
+    for ticket in (True, False, True, True, False):
+        out = prism.scan(xd, workspace=ws, ticket_order=ticket)
+        assert np.array_equal(host(out), want), ticket
 
 
-def test_scan_look_back_wait_is_bounded(prism, oracle, scan_env):
-    """With the spin limit forced to 0 a look-back that has to wait even once gives up: the kernel
-    must still finish, and a wave that gave up reports its tile + 1 in word 2 of the workspace.
-    With the default limit the same workspace reports nothing and the result is exact."""
+def test_scan_that_gives_up_is_an_error(prism, oracle):
+    """With the spin limit forced to 0 every look-back gives up before its first poll: the kernel must
+    still finish (the point of the bound), and the failure must be loud: scan() raises, and so does
+    scan_status() after an unchecked call. Afterwards the same workspace serves exact scans again and
+    reports nothing."""
     n = 1 << 26
     x = oracle.gen_scan(n, seed=3)
+    want = oracle.scan_cpu(x)
     xd = dev(x)
     out = torch.empty_like(xd)
-    ws = torch.empty(prism.get_workspace_size(n), dtype=torch.uint8, device=DEV)
-    for order in ("ticket", None):
-        scan_env(order=order, spin_limit=0)
-        prism.scan(xd, out, ws)
-        torch.cuda.synchronize()  # the point of the test: this returns
-        report = int(ws[8:12].view(torch.int32).item())
-        tiles = -(-n // 16384)
-        assert 0 <= report <= tiles
-        if report == 0:  # nobody had to wait: then the result must be right
-            assert np.array_equal(host(out), oracle.scan_cpu(x))
-        scan_env(order=order)
-        prism.scan(xd, out, ws)
-        assert int(ws[8:12].view(torch.int32).item()) == 0
-        assert np.array_equal(host(out), oracle.scan_cpu(x))
+    ws = prism.new_scan_workspace(n)
+    for ticket in (True, False):
+        with pytest.raises(prism.ScanOrderError, match="gave up waiting"):
+            prism.scan(xd, out, ws, ticket_order=ticket, spin_limit=0)
+        prism.scan(xd, out, ws, ticket_order=ticket, spin_limit=0, check=False)  # asynchronous, unchecked
+        with pytest.raises(prism.ScanOrderError):
+            prism.scan_status(ws)
+        prism.scan_status(ws)  # the report was consumed and the workspace re-initialised
+        for _ in range(2):
+            prism.scan(xd, out, ws, ticket_order=ticket)
+            assert np.array_equal(host(out), want)
+    # the reference-shaped launcher checks as well (through the library: no spin limit to force here)
+    prism.launch_scan(n, xd, ws)
+    assert np.array_equal(host(xd), want)
+
+
+def test_scan_workspace_shared_by_calls_of_any_length_and_kind(prism, oracle):
+    """One workspace, initialised once, then calls of very different tile counts and kinds back to back
+    and unsynchronised: every call clears the status words the call before it used (also those of a longer
+    call), so no call may see a stale word. Long, short and long again is the case that needs the
+    high-water mark in the header."""
+    big, mid, small = (1 << 26) + 77, (1 << 22) + 5, 70_001
+    ws = prism.new_scan_workspace(big)
+    xs = {n: oracle.gen_scan(n, seed=n % 97) for n in (big, mid, small)}
+    xd = {n: dev(x) for n, x in xs.items()}
+    inc = {n: oracle.scan_cpu(x) for n, x in xs.items()}
+    plan = [(big, {}), (small, {}), (big, {}), (small, {}), (small, {}), (big, {"ticket_order": True}),
+            (mid, {"exclusive": True}), (small, {"op": "max"}), (mid, {}), (big, {"exclusive": True}),
+            (small, {"ticket_order": True}), (small, {}), (small, {}), (big, {}), (mid, {"op": "min"}), (big, {})]
+    outs = []
+    for n, kw in plan:  # all enqueued before anything is checked
+        outs.append(prism.scan(xd[n], workspace=ws, check=False, **kw))
+    prism.scan_status(ws)
+    for (n, kw), out in zip(plan, outs):
+        x = xs[n]
+        if kw.get("exclusive"):
+            want = oracle.scan_exclusive_cpu(x)
+        elif kw.get("op") == "max":
+            want = oracle.scan_max_cpu(x)
+        elif kw.get("op") == "min":
+            want = ~oracle.scan_max_cpu(~x)
+        else:
+            want = inc[n]
+        assert np.array_equal(host(out), want), (n, kw)
 
 
 def test_scan_2pow30_properties(prism):
@@ -248,7 +268,7 @@ def test_scan_wraparound_and_all_ones(prism, oracle):
 
 def test_scan_workspace_reuse_and_unaligned(prism, oracle):
     n = 70_001
-    ws = torch.empty(prism.get_workspace_size(1 << 20), dtype=torch.uint8, device=DEV)
+    ws = prism.new_scan_workspace(1 << 20)
     for seed in range(4):  # same workspace, different data and lengths, back to back
         m = n - 1000 * seed
         x = oracle.gen_scan(m, seed=seed)
