@@ -131,11 +131,28 @@ int prism_scan_i32_ex(const int32_t* in, int32_t* out, size_t n, void* workspace
                       void* stream);
 
 /*
+ * prism_scan_i32 without a workspace argument and without any allocation: the
+ * status words live in a device array that is part of the library (2 MiB + 256
+ * bytes per GPU, held until the process ends), so n is limited to 2^31
+ * elements; a larger n returns 1 with an error string. No counterpart in the
+ * reference (its launcher takes a workspace the caller allocated,
+ * evals/4090_scan/main.cu:68-86). It is for callers that cannot allocate:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc. The call makes no hipMalloc / hipFree and uses no allocating
+ * library routine. All calls on one GPU share that GPU's array: they must be
+ * ordered on one stream, calls that overlap on one GPU race. Same kernels,
+ * same result and same bounded look-back as prism_scan_i32;
+ * prism_scan_status(NULL, 0, stream) reports for the library's array.
+ */
+int prism_scan_i32_static(const int32_t* in, int32_t* out, size_t n, void* stream);
+
+/*
  * Waits for `stream`, then reports whether any scan on this workspace since
  * the last report gave up waiting in its look-back: 0 = none did;
  * PRISM_ERROR_SCAN_ORDER = one did, the output of that call is invalid, the
- * error string names the tile, and the workspace has been re-initialised. The
- * reference has no counterpart (its look-back cannot give up); this is what
+ * error string names the tile, and the workspace has been re-initialised.
+ * workspace == NULL stands for the array prism_scan_i32_static uses on the
+ * current device. The reference has no counterpart (its look-back cannot give up); this is what
  * turns a broken tile-order assumption into an error instead of a wrong sum.
  */
 int prism_scan_status(void* workspace, size_t workspace_bytes, void* stream);

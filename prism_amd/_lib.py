@@ -22,6 +22,7 @@ SIGNATURES = {
     "prism_scan_workspace_init": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p]),
     "prism_scan_status": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p]),
     "prism_scan_i32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "prism_scan_i32_static": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "prism_scan_i32_ex": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_uint,
                                     C.c_longlong, C.c_void_p]),
     "prism_scan_exclusive_i32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p]),

@@ -84,6 +84,10 @@ int prism_scan_i32_ex(const int32_t* in, int32_t* out, size_t n, void* workspace
                        static_cast<hipStream_t>(stream));
 }
 
+int prism_scan_i32_static(const int32_t* in, int32_t* out, size_t n, void* stream) {
+    return launch_scan_static(u32(in), u32(out), n, static_cast<hipStream_t>(stream));
+}
+
 int prism_scan_exclusive_i32(const int32_t* in, int32_t* out, size_t n, void* workspace,
                              size_t workspace_bytes, void* stream) {
     return launch_scan(u32(in), u32(out), n, workspace, workspace_bytes, kFlagExclusive, -1,

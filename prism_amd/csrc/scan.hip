@@ -70,6 +70,7 @@
 //
 // HBM-bound: 8 algorithmic bytes per element (4 B read + 4 B write); status
 // traffic is 8 B per tile plus the polls.
+#include <mutex>
 #include <type_traits>
 
 #include "common.h"
@@ -442,6 +443,41 @@ int launch_cfg(const uint32_t* in, uint32_t* out, size_t n, uint32_t* header, u6
     return check_launch("scan_lookback_kernel");
 }
 
+// ------------------------------------------------------------- library-owned scratch --
+//
+// Workspace for callers that cannot allocate (prism_scan_i32_static): a device array that lives as
+// long as the module. Every GPU holds its own copy at its own address; host code must use the
+// address hipGetSymbolAddress returns, never the array's name.
+constexpr size_t kStaticMaxElems = size_t{1} << 31;
+constexpr size_t kStaticBytes = kHeaderBytes + 16 * (kStaticMaxElems / kWorkspaceTileElems);
+static __device__ __align__(256) unsigned char scratch[kStaticBytes];  // zero at load = initialised
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+int scan_workspace_init_impl(void* ws, size_t ws_bytes, hipStream_t s);
+
+// Device address of `scratch` on the current device. Looked up once per device; that first call also
+// enqueues a zero fill on `s`, so that nothing rests on what the array held before.
+int static_scratch(void** ptr, hipStream_t s) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    if (dev < 0 || dev >= kMaxDevices) return fail(1, "prism_scan: device %d outside the supported range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+        if (p == nullptr) return fail(1, "hipGetSymbolAddress(scratch) returned no address");
+        if (int rc = scan_workspace_init_impl(p, kStaticBytes, s)) return rc;
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return 0;
+}
+
 }  // namespace
 
 size_t scan_workspace_bytes(size_t n) {
@@ -449,7 +485,10 @@ size_t scan_workspace_bytes(size_t n) {
     return kHeaderBytes + 16 * (tiles > 0 ? tiles : 1);
 }
 
-int scan_workspace_init(void* ws, size_t ws_bytes, hipStream_t s) {
+int scan_workspace_init(void* ws, size_t ws_bytes, hipStream_t s) { return scan_workspace_init_impl(ws, ws_bytes, s); }
+
+namespace {
+int scan_workspace_init_impl(void* ws, size_t ws_bytes, hipStream_t s) {
     if (ws == nullptr || ws_bytes < kHeaderBytes + 16)
         return fail(1, "prism_scan_workspace_init: workspace of %zu bytes is too small", ws_bytes);
     if ((reinterpret_cast<uintptr_t>(ws) & 15u) != 0)
@@ -459,6 +498,7 @@ int scan_workspace_init(void* ws, size_t ws_bytes, hipStream_t s) {
         reinterpret_cast<u64*>(ws), n_words);
     return check_launch("scan_fill_zero_kernel");
 }
+}  // namespace
 
 int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, unsigned flags,
                 long long spin_limit, hipStream_t s) {
@@ -495,8 +535,22 @@ int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws
     return launch_cfg<BigCfg, true>(in, out, n, header, status, flags, limit, s);
 }
 
+int launch_scan_static(const uint32_t* in, uint32_t* out, size_t n, hipStream_t s) {
+    if (n > kStaticMaxElems)
+        return fail(1, "prism_scan_i32_static: n=%zu exceeds the %zu elements the library's scratch array covers",
+                    n, kStaticMaxElems);
+    if (n == 0) return 0;
+    void* ws = nullptr;
+    if (int rc = static_scratch(&ws, s)) return rc;
+    return launch_scan(in, out, n, ws, kStaticBytes, 0u, -1, s);
+}
+
 int scan_status(void* ws, size_t ws_bytes, hipStream_t s) {
-    if (ws == nullptr || ws_bytes < kHeaderBytes + 16) return fail(1, "prism_scan_status: workspace of %zu bytes is too small", ws_bytes);
+    if (ws == nullptr) {  // the library's own scratch array on the current device
+        if (int rc = static_scratch(&ws, s)) return rc;
+        ws_bytes = kStaticBytes;
+    }
+    if (ws_bytes < kHeaderBytes + 16) return fail(1, "prism_scan_status: workspace of %zu bytes is too small", ws_bytes);
     hipError_t e = hipStreamSynchronize(s);
     if (e != hipSuccess) return hip_fail(e, "prism_scan_status: hipStreamSynchronize");
     uint32_t report = 0;
