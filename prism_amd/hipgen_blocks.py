@@ -271,12 +271,18 @@ class _SyncPlan:
                     self._mark(s, may_sync)
                     pr, pw = set(), set()
                 pr |= self._reads(s.iter if isinstance(s, ast.For) else s.test)
+                before_loop = (set(pr), set(pw))
                 pr, pw = self._walk(s.body, (pr, pw), may_sync)
                 if self._probe(s.body, (pr, pw)) == "hazard":
                     if not may_sync:
                         raise HipgenError(f"{_line(s)}: a loop inside an `if` needs a barrier between its iterations")
                     self.at_end.add(id(s))
                     pr, pw = set(), set()
+                if not self._runs_at_least_once(s):
+                    # With zero trips none of the body's barriers is executed: what was pending in front
+                    # of the loop is still pending behind it.
+                    pr |= before_loop[0]
+                    pw |= before_loop[1]
             elif isinstance(s, (ast.If, ast.Match)):
                 r, w = self._whole([s])
                 if self._hazard(r, w, (pr, pw)):
@@ -300,6 +306,20 @@ class _SyncPlan:
                 pw |= w
         return pr, pw
 
+    @staticmethod
+    def _runs_at_least_once(s: ast.stmt) -> bool:
+        """True only for `for ... in range(...)` whose bounds are integer literals with at least one trip."""
+        if not (isinstance(s, ast.For) and _is_call(s.iter, "range") and not s.iter.keywords):
+            return False
+        args = s.iter.args
+        if not (1 <= len(args) <= 3) or not all(isinstance(a, ast.Constant) and isinstance(a.value, int)
+                                                and not isinstance(a.value, bool) for a in args):
+            return False
+        try:
+            return len(range(*(a.value for a in args))) >= 1
+        except ValueError:
+            return False
+
     def _mark(self, s: ast.stmt, may_sync: bool) -> None:
         if not may_sync:
             raise HipgenError(f"{_line(s)}: LDS is written and read inside one `if`; the barrier between "
@@ -319,7 +339,9 @@ class _SyncPlan:
                 got = self._probe(s.body, pending)
             elif isinstance(s, (ast.For, ast.While)):
                 r, w = self._whole([s])
-                got = "hazard" if self._hazard(r, w, pending) else ("barrier" if id(s) in self.at_end else "none")
+                # the barrier at the end of an inner loop's body only counts if that loop is sure to run
+                got = "hazard" if self._hazard(r, w, pending) else (
+                    "barrier" if id(s) in self.at_end and self._runs_at_least_once(s) else "none")
             elif isinstance(s, (ast.If, ast.Match)):
                 r, w = self._whole([s])
                 got = "hazard" if self._hazard(r, w, pending) else "none"

@@ -529,6 +529,50 @@ def test_barriers_of_the_lds_tiled_kernel():
     assert "__syncthreads();" not in lines(generate("tiled_sgemm", auto_sync=False))
 
 
+@requires(grid[1], block[1], thread[1])
+@prism("global")
+def maybe_no_trips(x: ptr(const(int)) @ grid[1], y: ptr(int) @ grid[1], trips: int @ grid[1]):
+    a: shared(int[64], static=True) @ block[1]
+    b: shared(int[64], static=True) @ block[1]
+    with group(block[1]):
+        t: int @ thread[1] = id()
+        with group(thread[1]):
+            a[t] = x[t]
+            for i in range(trips):
+                b[t] = i
+                y[t] = b[63 - t]
+            y[t] = a[63 - t]
+
+
+@requires(grid[1], block[1], thread[1])
+@prism("global")
+def surely_some_trips(x: ptr(const(int)) @ grid[1], y: ptr(int) @ grid[1]):
+    a: shared(int[64], static=True) @ block[1]
+    b: shared(int[64], static=True) @ block[1]
+    with group(block[1]):
+        t: int @ thread[1] = id()
+        with group(thread[1]):
+            a[t] = x[t]
+            for i in range(3):
+                b[t] = i
+                y[t] = b[63 - t]
+            y[t] = a[63 - t]
+
+
+def test_a_loop_that_may_not_run_keeps_what_was_pending_in_front_of_it():
+    """A write of `a`, a loop with a run-time trip count whose body only touches `b` (and gets its own two
+    barriers), then a cross-thread read of `a`. With zero trips none of the loop's barriers runs, so the
+    read needs a barrier of its own behind the loop. With a literal trip count of at least one the
+    barriers inside the loop are sure to run and order the write of `a` as well: no third barrier."""
+    got = lines(generate("maybe_no_trips"))
+    read = got.index("y[t] = a[(63 - t)];")
+    assert got[read - 1] == "__syncthreads();" and got[read - 2] == "}"
+    assert got.count("__syncthreads();") == 3
+    got = lines(generate("surely_some_trips"))
+    read = got.index("y[t] = a[(63 - t)];")
+    assert got[read - 1] == "}" and got.count("__syncthreads();") == 2
+
+
 def test_dynamic_lds_windows_private_arrays_and_attr():
     text = generate("thread_tile_sgemm")
     got = lines(text)
