@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--sweep]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-configs]
 
 Headline (BASELINE.json `metric`): fp32 SGEMM TFLOP/s at 8192^3 (alpha 1, beta 0.5,
 kernel 5 = wave tile on fp32 MFMA); the same JSON line carries the int32 scan at 2^30,
@@ -10,20 +10,29 @@ object. A "step" is one launch of the workload's entry point through the C ABI w
 inputs already resident in HBM. Timing: W untimed steps, then exactly K steps between
 two HIP events on the launch stream, device-synchronised on both sides.
 
-Every timed workload first passes a parity gate against a CPU check on the same data;
-a workload that fails the gate raises and reports nothing.
+"also" further holds every other BASELINE configuration ("configs": kernels 1..6 at 1024..8192, the
+tail shapes, the scan and bf16 sizes), timed with fewer steps, and add_m at 2^28 (2^24 fits the
+memory-side cache).
 
-cpu_baseline: the CPU oracle (oracle/prism_oracle.c, a scalar port, 1 core) timed on a
-bounded sample of the same workload, plus numpy/OpenBLAS and numpy.cumsum lines as
-additional baselines. Baselines, not targets.
+Every timed workload first passes a parity gate on the same data: the GEMMs against an fp64 product
+of the whole matrix formed on the device, the scan through its difference invariant over the whole
+array, add_m element for element; a workload that fails the gate raises and reports nothing. Every
+timed call's return code is checked.
+
+cpu_baseline: numpy/OpenBLAS sgemm on all host cores at the headline size; the scalar CPU oracle
+(oracle/prism_oracle.c, 1 core) on a bounded sample and numpy.cumsum are listed beside it.
+Baselines, not targets.
 """
 from __future__ import annotations
 
 import argparse
+import hashlib
 import json
 import os
+import re
 import sys
 import time
+from pathlib import Path
 
 import numpy as np
 
@@ -34,16 +43,29 @@ PEAK = {  # MI355X published peaks
 }
 
 
-# HBM-side bytes per launch (L2 misses: TCC fetches + write-backs), measured with
-# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over this script and scaled by what the same
-# counters read for a 1 GiB copy (`--workload calibrate`): FETCH_SIZE x 2.0, WRITE_SIZE x 1.0
-# (summaries under profiles/). None where not measured for that shape.
-TRAFFIC_BYTES = {
-    ("sgemm", 8192, 5): (4074176 + 262144) * 1024,
-    ("scan", 1 << 30): (4201763 + 4201231) * 1024,
-    ("gemm_bf16", 8192): (1582365 + 273438) * 1024,
-    ("add_m", 1 << 24): (65555 + 65536) * 1024,
-}
+ROOT = Path(__file__).resolve().parent
+TRAFFIC_FILE = ROOT / "profiles" / "hbm_traffic.md"
+KERNEL_SOURCE = {"sgemm": "sgemm.hip", "scan": "scan.hip", "gemm_bf16": "gemm_bf16.hip", "add_m": "add_m.hip"}
+
+
+def source_hash(workload: str) -> str:
+    """First 16 hex digits of the SHA-256 of the kernel source a workload runs."""
+    return hashlib.sha256((ROOT / "prism_amd" / "csrc" / KERNEL_SOURCE[workload]).read_bytes()).hexdigest()[:16]
+
+
+def measured_traffic(workload: str, size: int):
+    """HBM-side bytes per launch (L2 misses: TCC fetches + write-backs) from profiles/hbm_traffic.md, the
+    summary of two `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE, scaled by what the same
+    counters read for a copy of known size). Each row records the hash of the kernel source it was measured
+    on; a row whose hash differs from the source now in the tree is stale and gives None."""
+    try:
+        text = TRAFFIC_FILE.read_text()
+    except OSError:
+        return None
+    for m in re.finditer(r"^\|\s*(\w+)\s*\|\s*(\d+)\s*\|\s*(\d+)\s*\|\s*(\d+)\s*\|\s*([0-9a-f]{16})\s*\|", text, re.M):
+        if m.group(1) == workload and int(m.group(2)) == size:
+            return int(m.group(3)) + int(m.group(4)) if m.group(5) == source_hash(workload) else None
+    return None
 
 
 def log(*a):
@@ -62,28 +84,61 @@ SETTLE_MS = 150.0  # untimed run of the workload before the warm-up steps, see t
 
 
 def time_steps(fn, steps: int, warmup: int):
-    """Returns mean milliseconds per step, measured with HIP events on the current stream.
+    """Returns mean milliseconds per step, measured with HIP events on the current stream. `fn` is one
+    call of a C-ABI entry point and returns its code (0 = ok); any other code raises after the loop.
 
     Before the W warm-up steps the workload runs untimed for SETTLE_MS: the chip's clock and power
     management take tens of milliseconds to settle under a new load (the first launches of the bf16
     GEMM after an idle or memory-bound phase measured up to 15 % off the sustained rate), and three
     sub-millisecond warm-up steps do not cover that."""
     import torch
+    bad = 0
     t0 = time.perf_counter()
     while (time.perf_counter() - t0) * 1e3 < SETTLE_MS:
-        fn()
+        bad |= fn() or 0
         torch.cuda.synchronize()
     for _ in range(warmup):
-        fn()
+        bad |= fn() or 0
     torch.cuda.synchronize()
     beg = torch.cuda.Event(enable_timing=True)
     end = torch.cuda.Event(enable_timing=True)
     beg.record()
     for _ in range(steps):
-        fn()
+        bad |= fn() or 0
     end.record()
     torch.cuda.synchronize()
+    if bad:
+        from prism_amd import _lib
+        raise RuntimeError(f"a timed call returned an error code ({bad}): {_lib.last_error()}")
     return beg.elapsed_time(end) / steps
+
+
+# -------------------------------------------------- full-matrix parity checks --
+
+def sgemm_max_err_fp64(alpha, A, B, beta, C0, C, rows: int = 1024) -> float:
+    """max |C - (alpha A @ B + beta C0)| over EVERY element; the reference product is formed in fp64 on the
+    device (torch's fp64 GEMM), `rows` rows of C at a time."""
+    import torch
+    Bd = B.double()
+    worst = 0.0
+    for s in range(0, A.shape[0], rows):
+        ref = torch.matmul(A[s:s + rows].double(), Bd).mul_(alpha)
+        if beta != 0:
+            ref.add_(C0[s:s + rows].double(), alpha=beta)
+        worst = max(worst, float((C[s:s + rows].double() - ref).abs().max()))
+    return worst
+
+
+def gemm_bf16_max_err_fp64(A, B, D, rows: int = 1024):
+    """(max |D - A @ B^T| over every element, max |A @ B^T|); the product of the bf16 inputs in fp64 on the device."""
+    import torch
+    Bt = B.double().T.contiguous()
+    worst, ref_max = 0.0, 0.0
+    for s in range(0, A.shape[0], rows):
+        ref = torch.matmul(A[s:s + rows].double(), Bt)
+        worst = max(worst, float((D[s:s + rows].double() - ref).abs().max()))
+        ref_max = max(ref_max, float(ref.abs().max()))
+    return worst, ref_max
 
 
 # ------------------------------------------------------------------ sgemm --
@@ -98,10 +153,7 @@ def bench_sgemm(prism, M, N, K, alpha, beta, variant, steps, warmup, gate=True):
     C = C0.clone()
     if gate:
         prism.sgemm(M, N, K, alpha, A, B, beta, C, variant=variant)
-        torch.cuda.synchronize()
-        rows = torch.tensor(sorted({0, M // 3, M // 2, M - 1}), device="cuda")
-        ref = alpha * (A[rows].double() @ B.double()) + (beta * C0[rows].double() if beta != 0 else 0)
-        err = float((C[rows].double() - ref).abs().max())
+        err = sgemm_max_err_fp64(alpha, A, B, beta, C0, C)
         bound = 1e-5 * np.sqrt(K) + abs(beta) * 2**-22
         if not err <= bound:
             raise RuntimeError(f"sgemm kernel {variant} {M}x{N}x{K} failed the parity gate: err {err} > {bound}")
@@ -116,7 +168,7 @@ def bench_sgemm(prism, M, N, K, alpha, beta, variant, steps, warmup, gate=True):
     return {"ms": ms, "tflops": tflops,
             "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK["fp32_mfma_TFLOPs"], "unit": "TFLOP/s",
                          "frac": tflops / PEAK["fp32_mfma_TFLOPs"],
-                         "traffic": TRAFFIC_BYTES.get(("sgemm", M, variant)) if M == N == K else None}}
+                         "traffic": measured_traffic("sgemm", M) if M == N == K and variant == 5 else None}}
 
 
 # ------------------------------------------------------------------- scan --
@@ -153,7 +205,7 @@ def bench_scan(prism, n, steps, warmup, gate=True):
     gbps = nbytes / (ms * 1e-3) / 1e9
     return {"ms": ms, "GBps": gbps,
             "roofline": {"bound": "hbm", "achieved": gbps, "peak": PEAK["hbm_GBps"], "unit": "GB/s",
-                         "frac": gbps / PEAK["hbm_GBps"], "traffic": TRAFFIC_BYTES.get(("scan", n))}}
+                         "frac": gbps / PEAK["hbm_GBps"], "traffic": measured_traffic("scan", n)}}
 
 
 # ------------------------------------------------------------------ add_m --
@@ -175,7 +227,7 @@ def bench_add_m(prism, n, steps, warmup, gate=True):
     gbps = 8.0 * n / (ms * 1e-3) / 1e9
     return {"ms": ms, "GBps": gbps,
             "roofline": {"bound": "hbm", "achieved": gbps, "peak": PEAK["hbm_GBps"], "unit": "GB/s",
-                         "frac": gbps / PEAK["hbm_GBps"], "traffic": TRAFFIC_BYTES.get(("add_m", n))}}
+                         "frac": gbps / PEAK["hbm_GBps"], "traffic": measured_traffic("add_m", n)}}
 
 
 # -------------------------------------------------------------- bf16 gemm --
@@ -189,11 +241,8 @@ def bench_gemm_bf16(prism, n, steps, warmup, gate=True):
     D = torch.empty((n, n), dtype=torch.float32, device="cuda")
     if gate:
         prism.gemm_bf16(A, B, D)
-        torch.cuda.synchronize()
-        rows = torch.tensor(sorted({0, n // 3, n // 2, n - 1}), device="cuda")
-        ref = A[rows].double() @ B.double().T
-        err = float((D[rows].double() - ref).abs().max())
-        if not err <= 1e-3 * float(ref.abs().max()):
+        err, ref_max = gemm_bf16_max_err_fp64(A, B, D)
+        if not err <= 1e-3 * ref_max:
             raise RuntimeError(f"gemm_bf16 n={n} failed the parity gate: err {err}")
     lib, st = _capi()
     a, b, d = A.data_ptr(), B.data_ptr(), D.data_ptr()
@@ -201,13 +250,13 @@ def bench_gemm_bf16(prism, n, steps, warmup, gate=True):
     tflops = 2.0 * n * n * n / (ms * 1e-3) / 1e12
     return {"ms": ms, "tflops": tflops,
             "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK["bf16_mfma_TFLOPs"], "unit": "TFLOP/s",
-                         "frac": tflops / PEAK["bf16_mfma_TFLOPs"], "traffic": TRAFFIC_BYTES.get(("gemm_bf16", n))}}
+                         "frac": tflops / PEAK["bf16_mfma_TFLOPs"], "traffic": measured_traffic("gemm_bf16", n)}}
 
 
 # ----------------------------------------------------------- CPU baselines --
 
-def cpu_baseline_sgemm(n=8192, rows=32):
-    """Oracle (scalar fmaf port, 1 core) on the first `rows` rows of the n^3 problem."""
+def cpu_baseline_sgemm(n=8192, rows=4):
+    """Oracle (scalar fmaf port, 1 core) on the first `rows` rows of the n^3 problem (about 2 s)."""
     import oracle
     A, B, Cm = oracle.gen_sgemm(rows, n, n, seed=0)
     t0 = time.perf_counter()
@@ -217,12 +266,13 @@ def cpu_baseline_sgemm(n=8192, rows=32):
             "sample": f"oracle_sgemm_fma on the first {rows} rows of C ({rows}x{n}x{n}), {dt:.1f} s"}
 
 
-def cpu_blas_sgemm(n=4096):
+def cpu_blas_sgemm(n=8192):
+    """numpy/OpenBLAS sgemm on all host cores at the headline size (one untimed product first)."""
     rng = np.random.default_rng(0)
     A = rng.random((n, n), dtype=np.float32)
     B = rng.random((n, n), dtype=np.float32)
     Cm = rng.random((n, n), dtype=np.float32)
-    A @ B  # warm
+    A[:1024] @ B  # warm: thread pool and pages
     t0 = time.perf_counter()
     np.float32(1.0) * (A @ B) + np.float32(0.5) * Cm
     dt = time.perf_counter() - t0
@@ -233,8 +283,8 @@ def cpu_blas_sgemm(n=4096):
     except Exception:
         pass
     return {"value": 2.0 * n**3 / dt / 1e12, "unit": "TFLOP/s", "cores": threads or os.cpu_count(),
-            "kind": "numpy/OpenBLAS sgemm", "sample": f"{n}^3, alpha*(A@B)+beta*C, {dt:.2f} s",
-            "os_cpu_count": os.cpu_count()}
+            "kind": "port", "library": "numpy/OpenBLAS sgemm (the reference holds no CPU GEMM)",
+            "sample": f"the whole {n}^3 problem once, alpha*(A@B)+beta*C, {dt:.2f} s", "os_cpu_count": os.cpu_count()}
 
 
 def cpu_baseline_scan(n=1 << 28):
@@ -273,8 +323,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="all", choices=["all", "sgemm", "scan", "gemm_bf16", "add_m", "calibrate"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--sweep", action="store_true", help="also time every BASELINE config (table on stderr)")
-    ap.add_argument("--sweep-out", default=None, help="with --sweep: also write the table to this JSON file")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the table of the other BASELINE configurations (also.configs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no multi-GPU part); run with --gpus 1",
@@ -316,41 +366,44 @@ def main() -> int:
         res["add_m"] = bench_add_m(prism, 1 << 24, max(K, 50), W)
         log("add_m 2^24:", res["add_m"])
 
-    if args.sweep:
-        sweep = {}
+    if want("add_m"):
+        res["add_m_2p28"] = bench_add_m(prism, 1 << 28, K, W)
+        res["add_m_2p28"]["note"] = "x and y are 2 GiB together: beyond the 256 MiB memory-side cache"
+        res["add_m"]["note"] = "x and y are 128 MiB together and fit the 256 MiB memory-side cache: not an HBM-bound figure"
+        log("add_m 2^28:", res["add_m_2p28"])
+
+    # Every other BASELINE configuration, with fewer steps (kernel 1 at 8192^3 takes 0.35 s a step): a table
+    # under "also.configs" of the JSON line, each entry parity-gated like the headline workloads.
+    configs = {}
+    if args.workload == "all" and not args.no_configs:
         for n in (1024, 2048, 4096, 8192):
             for v in (1, 2, 3, 6, 4, 5):
-                if n == 8192 and v in (1, 2, 3):
-                    k, w = 2, 1
-                else:
-                    k, w = (5, 1) if n >= 4096 else (10, 2)
-                r = bench_sgemm(prism, n, n, n, 1.0, 0.5, v, k, w, gate=(v == 5))
-                sweep[f"sgemm_k{v}_{n}"] = r
+                if n == 8192 and v == 5:
+                    continue  # the headline
+                k, w = (2, 1) if (n >= 4096 and v in (1, 2, 3)) else (5, 1) if n >= 4096 else (10, 2)
+                r = bench_sgemm(prism, n, n, n, 1.0, 0.5, v, k, w)
+                configs[f"sgemm_k{v}_{n}"] = {"ms": r["ms"], "tflops": r["tflops"], "frac": r["roofline"]["frac"], "steps": k}
                 log(f"  sgemm kernel {v} {n}^3: {r['ms']:.3f} ms  {r['tflops']:.2f} TFLOP/s  "
                     f"({100 * r['roofline']['frac']:.1f}% of fp32 MFMA peak)")
         for (M, N, Kd) in ((4096, 4096, 128), (128, 4096, 4096), (8191, 4097, 1023), (16384, 16384, 512)):
             r = bench_sgemm(prism, M, N, Kd, 1.0, 0.0, 5, 10, 2)
-            sweep[f"sgemm_k5_{M}x{N}x{Kd}"] = r
+            configs[f"sgemm_k5_{M}x{N}x{Kd}"] = {"ms": r["ms"], "tflops": r["tflops"], "frac": r["roofline"]["frac"], "steps": 10}
             log(f"  sgemm kernel 5 {M}x{N}x{Kd}: {r['ms']:.3f} ms  {r['tflops']:.2f} TFLOP/s")
-        for p in (20, 24, 28, 30):
+        for p in (20, 24, 28):
             r = bench_scan(prism, 1 << p, 20, 3)
-            sweep[f"scan_2p{p}"] = r
+            configs[f"scan_2p{p}"] = {"ms": r["ms"], "GBps": r["GBps"], "frac": r["roofline"]["frac"], "steps": 20}
             log(f"  scan 2^{p}: {r['ms']:.4f} ms  {r['GBps']:.1f} GB/s ({100 * r['roofline']['frac']:.1f}% of HBM peak)")
-        for n in (4096, 8192, 16384):
+        for n in (4096, 16384):
             r = bench_gemm_bf16(prism, n, 8, 2)
-            sweep[f"gemm_bf16_{n}"] = r
+            configs[f"gemm_bf16_{n}"] = {"ms": r["ms"], "tflops": r["tflops"], "frac": r["roofline"]["frac"], "steps": 8}
             log(f"  gemm_bf16 {n}^3: {r['ms']:.3f} ms  {r['tflops']:.1f} TFLOP/s "
                 f"({100 * r['roofline']['frac']:.1f}% of bf16 MFMA peak)")
-        if args.sweep_out:
-            os.makedirs(os.path.dirname(os.path.abspath(args.sweep_out)), exist_ok=True)
-            with open(args.sweep_out, "w") as f:
-                json.dump(sweep, f, indent=1)
 
     cpu = {}
     if not args.no_cpu_baseline:
         if want("sgemm"):
-            cpu["sgemm"] = cpu_baseline_sgemm()
-            cpu["sgemm_blas"] = cpu_blas_sgemm()
+            cpu["sgemm"] = cpu_blas_sgemm()
+            cpu["sgemm_scalar_oracle"] = cpu_baseline_sgemm()
         if want("scan"):
             cpu["scan"] = cpu_baseline_scan()
         if want("add_m"):
@@ -378,7 +431,7 @@ def main() -> int:
         "config": {"workload": workload, "device": info["name"], "cu_count": info["cu_count"]},
         "roofline": head["roofline"],
         "cpu_baseline": cpu.get(head_name),
-        "also": {k: {kk: vv for kk, vv in v.items()} for k, v in res.items() if k != head_name},
+        "also": {**{k: v for k, v in res.items() if k != head_name}, **({"configs": configs} if configs else {})},
         "cpu_baselines_also": {k: v for k, v in cpu.items() if k != head_name},
     }
     print(json.dumps(line), flush=True)

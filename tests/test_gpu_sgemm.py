@@ -303,41 +303,58 @@ def test_wave_tile_ragged_tall_matrix(prism, oracle):
     assert np.max(np.abs(got - want)) <= 1e-5 * np.sqrt(K)
 
 
-def _sampled_check(prism, oracle, M, N, K, alpha, beta, variant, rows=48):
-    """Full-size run, checked on `rows` random rows against an fp64 product."""
+def _device_inputs(M, N, K):
     g = torch.Generator(device=DEV)
     g.manual_seed(0)
     A = torch.rand((M, K), dtype=torch.float32, device=DEV, generator=g) * 2 - 1
     B = torch.rand((K, N), dtype=torch.float32, device=DEV, generator=g) * 2 - 1
     C0 = torch.rand((M, N), dtype=torch.float32, device=DEV, generator=g) * 2 - 1
+    return A, B, C0
+
+
+def _bound(K, beta):
+    # entries are uniform in [-1, 1): max|A| max|B| <= 1; the beta * C term adds its own rounding
+    return 1e-5 * np.sqrt(K) + (abs(beta) * 2**-22 if beta else 0.0)
+
+
+def _full_check(prism, M, N, K, alpha, beta, variant, linearity=True):
+    """Full-size run; EVERY element is compared with an fp64 product formed on the device
+    (bench.sgemm_max_err_fp64: torch's fp64 GEMM on row blocks), bound 1e-5 * sqrt(K) * max|A| * max|B|."""
+    import bench
+    A, B, C0 = _device_inputs(M, N, K)
     c = C0.clone()
     prism.sgemm(M, N, K, alpha, A, B, beta, c, variant=variant)
-    torch.cuda.synchronize()
-    idx = np.sort(np.random.default_rng(0).choice(M, rows, replace=False))
-    idx[0], idx[-1] = 0, M - 1
-    it = torch.from_numpy(idx).to(DEV)
-    a_rows = A[it].cpu().numpy()
-    b_host = B.cpu().numpy()
-    want = oracle.np_sgemm_f64(alpha, a_rows, b_host, beta, C0[it].cpu().numpy())
-    got = c[it].cpu().numpy()
-    bound = 1e-5 * np.sqrt(K) * 1.0 * 1.0 + (abs(beta) * 2**-22 if beta else 0.0)
-    assert np.max(np.abs(got - want)) <= bound
-    # linearity in alpha: doubling alpha with beta = 0 doubles every element exactly
-    c1 = torch.empty_like(c)
-    c2 = torch.empty_like(c)
-    prism.sgemm(M, N, K, 1.0, A, B, 0.0, c1, variant=variant)
-    prism.sgemm(M, N, K, 2.0, A, B, 0.0, c2, variant=variant)
-    assert torch.equal(c2, 2.0 * c1)
+    err = bench.sgemm_max_err_fp64(alpha, A, B, beta, C0, c)
+    assert err <= _bound(K, beta), f"kernel {variant} {M}x{N}x{K}: max error {err:.3e}"
+    if linearity:  # doubling alpha with beta = 0 doubles every element exactly
+        c1 = torch.empty_like(c)
+        c2 = torch.empty_like(c)
+        prism.sgemm(M, N, K, 1.0, A, B, 0.0, c1, variant=variant)
+        prism.sgemm(M, N, K, 2.0, A, B, 0.0, c2, variant=variant)
+        assert torch.equal(c2, 2.0 * c1)
+    return c
 
 
-def test_wave_tile_4096_and_8192(prism, oracle):
-    _sampled_check(prism, oracle, 4096, 4096, 4096, 1.0, 0.5, 5)
-    _sampled_check(prism, oracle, 8192, 8192, 8192, 1.0, 0.5, 5)
+@pytest.mark.parametrize("n", [4096, 8192])
+def test_baseline_square_all_kernels_full_size(prism, n):
+    """BASELINE's square sizes 4096 and 8192 (alpha 1, beta 0.5) for every kernel of the progression: every
+    element against the fp64 product, and kernels 1, 2, 3, 4, 6 (one fused multiply-add per k, in order)
+    bit-identical to each other."""
+    first = None
+    for v in ALL:
+        c = _full_check(prism, n, n, n, 1.0, 0.5, v, linearity=(v == 5))
+        if v in EXACT:
+            first = c if first is None else first
+            assert torch.equal(c, first), f"kernel {v} differs from kernel 1 bitwise at n = {n}"
 
 
-def test_wave_tile_16384x16384x512(prism, oracle):
-    _sampled_check(prism, oracle, 16384, 16384, 512, 1.0, 0.0, 5)
+def test_wave_tile_16384x16384x512(prism):
+    _full_check(prism, 16384, 16384, 512, 1.0, 0.0, 5)
 
 
-def test_thread_tile_4096(prism, oracle):
-    _sampled_check(prism, oracle, 4096, 4096, 4096, 1.0, 0.5, 4, rows=16)
+@pytest.mark.parametrize("shape", [(4096, 4096, 128), (128, 4096, 4096), (8191, 4097, 1023), (16384, 16384, 512)])
+def test_baseline_tail_shapes_all_kernels_full(prism, shape):
+    """BASELINE's non-square and tail shapes (beta = 0) through every kernel, every element against fp64."""
+    M, N, K = shape
+    for v in ALL:
+        _full_check(prism, M, N, K, 1.0, 0.0, v, linearity=False)
