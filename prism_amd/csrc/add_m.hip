@@ -10,62 +10,45 @@
 namespace prism {
 namespace {
 
-#ifndef PRISM_ADDM_BLOCK
-#define PRISM_ADDM_BLOCK 256
-#endif
-#ifndef PRISM_ADDM_UNROLL
-#define PRISM_ADDM_UNROLL 1
-#endif
-constexpr int kAddBlock = PRISM_ADDM_BLOCK;
-// 16 B accesses per lane. One is best: measured at 2^30 elements, 1 / 2 / 4 / 8 packets per lane give
-// 6.50 / 5.96 / 5.84 / 4.05 TB/s (many small workgroups keep more independent streams in flight).
-constexpr int kAddUnroll = PRISM_ADDM_UNROLL;
-// Streams larger than this bypass the caches with non-temporal accesses (6.50 against 6.20 TB/s at
-// 2^30); smaller ones use ordinary accesses so that repeated passes over the same buffers are served
-// by the 256 MiB memory-side cache (6.8 against 6.4 TB/s at 2^24, the size the reference quotes).
+constexpr int kAddBlock = 256;
+// One 16 B packet per lane, so a workgroup is 4 KiB and a wavefront lives for one load and one store.
+// Measured at 2^30 elements, 1 / 2 / 4 / 8 packets per lane give 6.50 / 5.96 / 5.84 / 4.05 TB/s: with
+// one packet the workgroups sweep memory in dispatch order as one compact front (about 8 MiB in
+// flight on the whole chip), which is what the write side of HBM wants: a write-only kernel of this
+// shape reaches 7.0 TB/s, the same kernel writing its 4 KiB chunks in a scattered order 5.4.
+// Streams larger than this use non-temporal loads and `sc1 nt` stores (write through towards memory,
+// evict early: 6.68 against 6.51 TB/s for nt-only stores and 6.44 for plain ones at 2^30); smaller ones
+// use ordinary accesses so that repeated passes over the same buffers are served by the 256 MiB
+// memory-side cache (6.8 against 6.4 TB/s at 2^24, the size the reference quotes).
 constexpr size_t kAddStreamingBytes = size_t{192} << 20;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-// Each block owns kAddBlock * kAddUnroll consecutive 16 B packets; within the
-// block, access u of lane t is packet (u * kAddBlock + t), so a wavefront always
-// touches 1 KiB of contiguous memory per instruction.
+// The two wait states keep the next instruction from overwriting the data registers while the store
+// still reads them (the compiler does not see a store inside the assembly).
+__device__ __forceinline__ void stream_store(u32x4* p, u32x4 v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
+}
+
+// Lane t of block b handles packet (b * kAddBlock + t): a wavefront touches 1 KiB of contiguous
+// memory per instruction.
 template <bool STREAMING>
 __global__ __launch_bounds__(kAddBlock) void add_m_vec4_kernel(const u32x4* __restrict__ x,
                                                                u32x4* __restrict__ y, uint32_t m,
                                                                size_t n_vec) {
-    const size_t base = static_cast<size_t>(blockIdx.x) * (kAddBlock * kAddUnroll) + threadIdx.x;
-    u32x4 v[kAddUnroll];
-#pragma unroll
-    for (int u = 0; u < kAddUnroll; ++u) {
-        const size_t i = base + static_cast<size_t>(u) * kAddBlock;
-        if (i < n_vec) v[u] = STREAMING ? __builtin_nontemporal_load(&x[i]) : x[i];
-    }
-#pragma unroll
-    for (int u = 0; u < kAddUnroll; ++u) {
-        const size_t i = base + static_cast<size_t>(u) * kAddBlock;
-        if (i < n_vec) {
-            if (STREAMING) __builtin_nontemporal_store(v[u] + m, &y[i]);
-            else y[i] = v[u] + m;
-        }
-    }
+    const size_t i = static_cast<size_t>(blockIdx.x) * kAddBlock + threadIdx.x;
+    if (i >= n_vec) return;
+    if (STREAMING) stream_store(&y[i], __builtin_nontemporal_load(&x[i]) + m);
+    else y[i] = x[i] + m;
 }
 
 // Same as above when x and y are the same buffer (no __restrict__ promise).
-__global__ __launch_bounds__(kAddBlock) void add_m_vec4_inplace_kernel(u32x4* xy, uint32_t m,
-                                                                       size_t n_vec) {
-    const size_t base = static_cast<size_t>(blockIdx.x) * (kAddBlock * kAddUnroll) + threadIdx.x;
-    u32x4 v[kAddUnroll];
-#pragma unroll
-    for (int u = 0; u < kAddUnroll; ++u) {
-        const size_t i = base + static_cast<size_t>(u) * kAddBlock;
-        if (i < n_vec) v[u] = xy[i];
-    }
-#pragma unroll
-    for (int u = 0; u < kAddUnroll; ++u) {
-        const size_t i = base + static_cast<size_t>(u) * kAddBlock;
-        if (i < n_vec) xy[i] = v[u] + m;
-    }
+template <bool STREAMING>
+__global__ __launch_bounds__(kAddBlock) void add_m_vec4_inplace_kernel(u32x4* xy, uint32_t m, size_t n_vec) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * kAddBlock + threadIdx.x;
+    if (i >= n_vec) return;
+    if (STREAMING) stream_store(&xy[i], __builtin_nontemporal_load(&xy[i]) + m);
+    else xy[i] = xy[i] + m;
 }
 
 // One element per thread: the tail of a vector launch, or the whole array when
@@ -98,13 +81,16 @@ int launch_add_m(const int32_t* x_, int32_t* y_, int32_t m_, size_t n, hipStream
     size_t n_vec = 0;
     if (aligned16(x) && aligned16(y)) n_vec = n / 4;
     if (n_vec > 0) {
-        const size_t per_block = static_cast<size_t>(kAddBlock) * kAddUnroll;
-        const size_t blocks = ceil_div(n_vec, per_block);
+        const size_t blocks = ceil_div(n_vec, static_cast<size_t>(kAddBlock));
         if (blocks > 0x7fffffffull) return fail(1, "prism_add_m: n=%zu too large", n);
-        if (x == y)
-            add_m_vec4_inplace_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(kAddBlock), 0, s>>>(
+        const bool streaming = (x == y ? 1 : 2) * n * sizeof(uint32_t) > kAddStreamingBytes;
+        if (x == y && streaming)
+            add_m_vec4_inplace_kernel<true><<<dim3(static_cast<unsigned>(blocks)), dim3(kAddBlock), 0, s>>>(
                 reinterpret_cast<u32x4*>(y), m, n_vec);
-        else if (2 * n * sizeof(uint32_t) > kAddStreamingBytes)
+        else if (x == y)
+            add_m_vec4_inplace_kernel<false><<<dim3(static_cast<unsigned>(blocks)), dim3(kAddBlock), 0, s>>>(
+                reinterpret_cast<u32x4*>(y), m, n_vec);
+        else if (streaming)
             add_m_vec4_kernel<true><<<dim3(static_cast<unsigned>(blocks)), dim3(kAddBlock), 0, s>>>(
                 reinterpret_cast<const u32x4*>(x), reinterpret_cast<u32x4*>(y), m, n_vec);
         else

@@ -10,9 +10,7 @@
 //                                               a stage freed in mid-phase once its fragments are in
 //                                               registers (gemm_bf16_early_kernel); odd or small K tile
 //                                               counts: direct-to-LDS ring of two stages
-//                                               (gemm_bf16_ring_kernel); selectable: buffer loads into two
-//                                               register sets two K tiles ahead, written to LDS by the
-//                                               waves (gemm_bf16_staged16_kernel, _staged_kernel)
+//                                               (gemm_bf16_ring_kernel)
 //   1 producer + 2 consumer warpgroups      ->  every wave loads and multiplies
 //   persistent CTAs + 16x8 super-tiles      ->  one workgroup per tile, 16x16 super-blocks with an
 //                                               8x4 patch per XCD (tile_map.h)
@@ -36,48 +34,24 @@
 //
 // In gemm_bf16_kernel LDS rows are BK + 8 elements (144 B for BK = 64): eight lanes
 // reading 16 B from eight consecutive rows then cover all banks exactly once.
-#include <cstdlib>
-#include <cstring>
 #include <type_traits>
 
 #include "common.h"
 #include "direct_load.h"
 #include "tile_map.h"
 
-// Block tile BM x BN x BK and wave tile WM x WN.
-#ifndef PRISM_BF16_SCHED
-#define PRISM_BF16_SCHED 1
-#endif
-#ifndef PRISM_BF16_M16_WRITE_J
-#define PRISM_BF16_M16_WRITE_J 2  // in the 16x16x32 kernel: the instruction of a row behind which the LDS write goes
-#endif
-#ifndef PRISM_BF16_M16_LOAD_J
-#define PRISM_BF16_M16_LOAD_J 3   // ... and the global load, which must come after the write of the same packet
-                                  // (2/3, 2/6, 1/5, 3/7 all within 0.5 % of each other; 6/7 is 5 % slower at 8192^3)
-#endif
-#ifndef PRISM_BF16_K_STAGGER
-#define PRISM_BF16_K_STAGGER 64  // gemm_bf16_early_kernel: K tiles (of 128 B) between the starting points of two XCDs; 0: all start at 0; -1: K tiles / 8; -2: K tiles / 2.
-// 8192 x 8192 x K, TFLOP/s without / with 64: K = 12288 1316 / 1427, 6144 1432 / 1495, 10240 1436 / 1502, 14336 1507 / 1522,
-// 8192 and 4096 level, 24576 1302 / 1273. Steps of 2 and 8 tiles (256 B, 1 KB) gain nothing, 16 half of it, 32 the same;
-// at K = 12288 steps of 48, 96, 128 tiles and of half the K tiles give 1395, 1366, 1420, 1345 against 1435 for 64.
-#endif
-#ifndef PRISM_BF16_EARLY_BARRIER_AT
-#define PRISM_BF16_EARLY_BARRIER_AT 36  // gemm_bf16_early_kernel: instructions of a phase before the barrier that frees its stage
-#endif
-#ifndef PRISM_BF16_EARLY_LOAD_GAP
-#define PRISM_BF16_EARLY_LOAD_GAP 6  // matrix instructions between two direct loads in gemm_bf16_early_kernel.
-// Barrier position / gap, PFLOP/s at 8192^3 and 16384^3: 64/2 1.33-1.37, 1.32; 64/4 1.41-1.42, 1.42; 48/5 1.43-1.44,
-// 1.47; 40/5 1.44-1.45, 1.47; 36/6 1.44, 1.49 (the staged kernel in the same run: 1.38-1.42, 1.45). A wave-wide
-// 16 B load keeps the CU's vector memory path busy for 16 clocks, and the 64 loads of a K tile are half of a
-// phase's clocks: the more evenly they are spread, the less they hold up the matrix instructions behind them.
-#endif
-#ifndef PRISM_BF16_MFMA_ORDER
-#define PRISM_BF16_MFMA_ORDER 2  // issue order of a group's MFMAs in the staged kernel (see mfma_group there);
-                                 // 8192^3: 1431-1437 / 1434 / 1438-1442 TFLOP/s for 0 / 1 / 2
-#endif
-#ifndef PRISM_BF16_CFG
-#define PRISM_BF16_CFG 256, 256, 64, 128, 128
-#endif
+// gemm_bf16_early_kernel: K tiles (of 128 B) between the starting points of two XCDs' walks along K.
+// 8192 x 8192 x K, TFLOP/s all starting at 0 / with 64: K = 12288 1316 / 1427, 6144 1432 / 1495, 10240 1436 / 1502,
+// 14336 1507 / 1522, 8192 and 4096 level, 24576 1302 / 1273. Steps of 2 and 8 tiles (256 B, 1 KB) gain nothing,
+// 16 half of it, 32 the same; at K = 12288 steps of 48, 96, 128 tiles and of half the K tiles give 1395, 1366,
+// 1420, 1345 against 1435 for 64.
+constexpr int kEarlyKStagger = 64;
+// gemm_bf16_early_kernel: matrix instructions of a phase before the barrier that frees its stage, and between two
+// direct loads. Barrier position / gap, PFLOP/s at 8192^3 and 16384^3: 64/2 1.33-1.37, 1.32; 64/4 1.41-1.42, 1.42;
+// 48/5 1.43-1.44, 1.47; 40/5 1.44-1.45, 1.47; 36/6 1.44, 1.49. A wave-wide 16 B load keeps the CU's vector memory
+// path busy for 16 clocks, and the 64 loads of a K tile are half of a phase's clocks: the more evenly they are
+// spread, the less they hold up the matrix instructions behind them.
+constexpr int kEarlyBarrierAt = 36, kEarlyLoadGap = 6;
 
 namespace prism {
 namespace {
@@ -246,7 +220,6 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_kerne
                 for (int j = 0; j < NI; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[kk & 1][i], fb[kk & 1][j], acc[i][j], 0, 0, 0);
         }
-#if PRISM_BF16_SCHED
         // Issue order for the whole step: LDS reads of the next k-substep ride
         // under the first MFMAs of each substep, LDS writes and global loads of
         // the following tiles under the rest, so the matrix pipe never waits for
@@ -261,7 +234,6 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_kerne
             else
                 sched_substep<0, W_PER, L_PER, MI * NI>();
         }
-#endif
         __syncthreads();
         if constexpr (store_next) read_frags(buf ^ 1, 0, 0);
     };
@@ -316,11 +288,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_kerne
 // of the group before it; loads use a scalar base and a fixed lane offset (no
 // vector ALU work in the loop).
 //
-// 64 x 2 stages is the shape used, for the K tile counts the register-staged kernel
-// below does not take: a direct load cannot be issued before its stage is free, so
-// it has less than one tile time to land, which the staged kernel avoids. 32 x 4
-// stages (also supported by the template) gives loads three tile times but reads
-// half cache lines (64 B per row and tile) and measured slower than both.
+// 64 x 2 stages is the shape used, for the K tile counts gemm_bf16_early_kernel below
+// does not take: a direct load cannot be issued before its stage is free, so it has
+// less than one tile time to land, which the early-read kernel avoids. 32 x 4 stages
+// (also supported by the template) gives loads three tile times but reads half cache
+// lines (64 B per row and tile) and measured slower than both.
 //
 // EDGE: M, N, K need not be whole tiles (K a multiple of 8, so that rows stay 16 B aligned and a
 // 16 B chunk is whole or absent). The direct loads then go through buffer descriptors whose extents
@@ -547,261 +519,24 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_
     }
 }
 
-// ------------------------------------------- register-staged pipeline kernel --
-// Whole tiles, K a multiple of 128 (an even number of K tiles, at least 6). Two LDS stages of one
-// 256 x 256 x 64 tile pair each (128 KiB), plus two register sets that each hold
-// a wave's share of one more tile pair (16 x 16 B per lane). Tile t+3 is loaded
-// from global memory into registers while tile t is multiplied, and is written
-// to LDS two tiles later, so a load has two tile times (about 4000 clocks) to
-// land. A direct-to-LDS load cannot be issued before its LDS stage is free,
-// which with two stages leaves it less than one tile time; measured with
-// all-zero operands (no power throttling), waiting for those loads cost 35 % of
-// the run time. This is the depth the reference gets from its four-stage
-// mbarrier ring (QSIZE = 4, generated/cutlass_my_h100_match_no_tail.cu:117);
-// 160 KiB of LDS cannot hold four such stages, registers can hold two.
+// ------------------------------------------- the 16x16x32 matrix instruction in place --
+// v_mfma_f32_16x16x32_bf16: OUT (16 x 16) += P fragment (16 rows x 32 k) * Q fragment (16 rows x 32 k)^T;
+// lane l supplies 8 consecutive k of row l % 16, starting at k = 8 (l / 16); result register v of lane l is
+// OUT[4 (l / 16) + v][l % 16]. A wave's 128 x 128 tile is 8 x 8 such sub-tiles (64 accumulators of 4
+// registers). Against v_mfma_f32_32x32x16_bf16 the instruction has the same peak rate and draws about
+// 12 % less power per flop (register-only loops on random operands: 2.04 against 1.82 PFLOP/s).
 //
-// Every barrier orders LDS traffic only (lds_barrier), so global loads stay in
-// flight across it. The K loop is laid out by hand and pinned with scheduling
-// barriers: between two barriers a wave issues 64 MFMAs; behind the first 8 of
-// every group of 16 go the LDS reads of the next group's operands, behind the
-// other 8 alternately one LDS write of a staged 16 B packet (tile t+1) and the
-// global load that refills its registers (tile t+3).
-//
-// LDS rows are 128 B (8 chunks of 16 B); chunk c of row r sits in slot
-// c ^ ((r >> 1) & 7): a wave writes 1 KiB of contiguous LDS per instruction, and
-// the 16 rows a quarter-wave reads with ds_read_b128 cover all 64 banks.
-template <int BM, int BN, int WM, int WN, bool EDGE, typename OutT>
-__global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_staged_kernel(
-    int R, int Cn, int K, const uint16_t* __restrict__ P, const uint16_t* __restrict__ Q,
-    OutT* __restrict__ OUT, int tiles_m, int tiles_n) {
-    constexpr int BK = 64, KP = 8, SWZ = 1, KS = 4;
-    constexpr int WAVES_N = BN / WN;
-    constexpr int WAVES = (BM / WM) * WAVES_N;
-    constexpr int MI = WM / 32, NI = WN / 32;
-    constexpr int ROWS_PER_LOAD = kWave / KP;         // 8 rows of 128 B per wave-wide access
-    constexpr int ROWS_PER_PASS = ROWS_PER_LOAD * WAVES;
-    static_assert(BM % ROWS_PER_PASS == 0 && BN % ROWS_PER_PASS == 0, "whole load passes");
-    constexpr int P_PER = BM / ROWS_PER_PASS, Q_PER = BN / ROWS_PER_PASS;
-    constexpr int PACKETS = P_PER + Q_PER;            // 16 B packets per lane per tile pair
-    constexpr int READS = MI + NI, GROUP = MI * NI;
-    static_assert(2 * PACKETS == (GROUP - READS) * KS, "one write and one load behind every free MFMA of a phase");
-
-    __shared__ __attribute__((aligned(1024))) uint16_t Ps[2][BM * BK];
-    __shared__ __attribute__((aligned(1024))) uint16_t Qs[2][BN * BK];
-
-    int tm, tn;
-    xcd_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
-    const int row0 = tm * BM, col0 = tn * BN;
-
-    const int tid = threadIdx.x;
-    const int lane = tid & (kWave - 1);
-    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
-    const int l32 = lane & 31, lhi = lane >> 5;
-
-    f32x16 acc[MI][NI];
-#pragma unroll
-    for (int i = 0; i < MI; ++i)
-#pragma unroll
-        for (int j = 0; j < NI; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-
-    // Global side: packet m of a tile pair is rows [(m * WAVES + wave) * 8, + 8) of P (m < P_PER) or Q;
-    // lane l owns row l / 8 of those and the chunk that belongs in slot l % 8. Addresses are a
-    // wave-uniform base plus a loop-invariant 32-bit lane offset.
-    const int ld_row = wave * ROWS_PER_LOAD + lane / KP;
-    const int ld_chunk = (lane % KP) ^ ((ld_row >> SWZ) & (KP - 1));
-    const uint32_t lane_off = (static_cast<uint32_t>(lane / KP) * static_cast<uint32_t>(K) + ld_chunk * 8) * 2u;  // bytes
-    // Buffer loads: the address is (descriptor base) + (vector offset) + (scalar offset), so a load
-    // needs no vector ALU work; offsets stay inside this workgroup's 256-row panel (the launcher
-    // checks that a panel is below 2 GiB).
-    //
-    // EDGE: the matrices need not be whole tiles. A buffer load returns zero for every dword at or
-    // beyond the descriptor's extent (vector + scalar offset are both checked), so with the extent set
-    // to the end of the matrix the rows below it read as zeros. Columns k >= K of a row are the
-    // next row's data and in range, so there the lane offset is replaced by one beyond any extent
-    // (kBeyond); K is a multiple of 8, so a 16 B chunk is either whole or absent. The K loop runs
-    // over an even number (at least 6) of K tiles, the ones past K reading zeros.
-    constexpr uint32_t kBeyond = 0x80000000u;
-    auto extent = [&](int first_row, int rows) -> int {  // bytes from a wave's first row to the end of the matrix
-        if (!EDGE) return 0x7fffffff;
-        const long long left = static_cast<long long>(rows - first_row) * K * 2;
-        return static_cast<int>(left < 0 ? 0 : (left > 0x7fffffff ? 0x7fffffff : left));
-    };
-    const int p_first = row0 + wave * ROWS_PER_LOAD, q_first = col0 + wave * ROWS_PER_LOAD;
-    // A wave whose first row is already outside the matrix gets extent 0 on a valid base address.
-    const auto p_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t*>(P + (EDGE && p_first >= R ? size_t{0} : static_cast<size_t>(p_first) * K)), 0,
-        extent(p_first, R), 0x00020000);
-    const auto q_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t*>(Q + (EDGE && q_first >= Cn ? size_t{0} : static_cast<size_t>(q_first) * K)), 0,
-        extent(q_first, Cn), 0x00020000);
-    const int pass_bytes = ROWS_PER_PASS * K * 2;
-    const int k_full = K - K % BK;                                   // tiles that start below it are whole
-    const int k_end = EDGE ? ((K + 2 * BK - 1) / (2 * BK) < 3 ? 6 * BK : (K + 2 * BK - 1) / (2 * BK) * 2 * BK) : K;
-    const uint32_t tail_off = (EDGE && k_full + ld_chunk * 8 < K) ? lane_off : kBeyond;  // lane offset in the partial tile
-    u32x4 staged[2][PACKETS];
-    // Lane offset for the loads of the tile that starts at k0: two selects on scalar conditions.
-    auto offset_for = [&](int k0) -> uint32_t {
-        if (!EDGE) return lane_off;
-        return k0 < k_full ? lane_off : (k0 < K ? tail_off : kBeyond);
-    };
-    auto load_packet = [&](int set, int k0, int m, uint32_t off) {
-        if (m < P_PER)
-            staged[set][m] = __builtin_amdgcn_raw_buffer_load_b128(p_rsrc, off, m * pass_bytes + k0 * 2, 0);
-        else
-            staged[set][m] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, off, (m - P_PER) * pass_bytes + k0 * 2, 0);
-    };
-    // LDS side: the same packet lands at (its first row) * 128 B + 16 B * lane.
-    auto write_packet = [&](int set, int m) {
-        uint16_t* dst = (m < P_PER) ? &Ps[set][(m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]
-                                    : &Qs[set][((m - P_PER) * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK];
-        *reinterpret_cast<u32x4*>(dst + lane * 8) = staged[set][m];
-    };
-
-    // Operand side: row (wave tile origin + 32 i + l32), chunk 2 kk + lhi of the row.
-    const int sw = (l32 >> SWZ) & (KP - 1);
-    int p_off[KS], q_off[KS];
-#pragma unroll
-    for (int kk = 0; kk < KS; ++kk) {
-        const int slot = (2 * kk + lhi) ^ sw;
-        p_off[kk] = (wave_m * WM + l32) * BK + slot * 8;
-        q_off[kk] = (wave_n * WN + l32) * BK + slot * 8;
-    }
-    bf16x8 fa[2][MI], fb[2][NI];
-    auto read_one = [&](int stage, int kk, int r) {
-        if (r < MI)
-            fa[kk & 1][r] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&Ps[stage][p_off[kk] + r * 32 * BK]));
-        else
-            fb[kk & 1][r - MI] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&Qs[stage][q_off[kk] + (r - MI) * 32 * BK]));
-    };
-    auto mfma_group = [&](int slot, auto after) {
-#pragma unroll
-        for (int m = 0; m < MI * NI; ++m) {
-#if PRISM_BF16_MFMA_ORDER == 1   // column-major: B operand fixed for MI instructions
-            const int j = m / MI, i = m % MI;
-#elif PRISM_BF16_MFMA_ORDER == 2  // serpentine: consecutive instructions always share one operand
-            const int i = m / NI, j = (i & 1) ? NI - 1 - m % NI : m % NI;
-#else                             // row-major: A operand fixed for NI instructions
-            const int i = m / NI, j = m % NI;
-#endif
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[slot][i], fb[slot][j], acc[i][j], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            after(m);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    };
-
-    // One phase = everything between two barriers, for the tile in stage S (tile t). Entered
-    // right after the barrier that says "tile t is complete in stage S and nobody reads stage
-    // S^1 any more", while operand slot 1 holds the last k-group of tile t-1. Register set S^1
-    // holds tile t+1 (loaded two phases ago): it is written to stage S^1 (`write`) and refilled
-    // with tile t+3, which starts at k_load (`load`).
-    auto phase = [&](auto stage_c, auto write, auto load, int k_load) {
-        constexpr int S = decltype(stage_c)::value;
-        const uint32_t off = offset_for(k_load);
-#pragma unroll
-        for (int g = 0; g < KS; ++g) {
-            mfma_group((g + 1) & 1, [&](int m) {
-                if (m < READS) {
-                    read_one(S, g, m);
-                } else {
-                    const int packet = (g * (GROUP - READS) + (m - READS)) / 2;
-                    if ((m - READS) % 2 == 0) {
-                        if constexpr (write) write_packet(S ^ 1, packet);
-                    } else {
-                        if constexpr (load) load_packet(S ^ 1, k_load, packet, off);
-                    }
-                }
-            });
-        }
-        lds_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    using yes = std::integral_constant<bool, true>;
-    using no = std::integral_constant<bool, false>;
-    using s0 = std::integral_constant<int, 0>;
-    using s1 = std::integral_constant<int, 1>;
-
-    // Slot 1 starts as zeros, so the "previous tile" MFMAs of the first phase add nothing.
-#pragma unroll
-    for (int i = 0; i < MI; ++i) fa[1][i] = bf16x8{};
-#pragma unroll
-    for (int j = 0; j < NI; ++j) fb[1][j] = bf16x8{};
-
-    // The launcher guarantees an even number of K tiles, at least 6: tiles alternate between the
-    // two stages (and register sets), the first in stage 0 and the last in stage 1.
-#pragma unroll
-    for (int m = 0; m < PACKETS; ++m) load_packet(0, 0, m, offset_for(0));
-#pragma unroll
-    for (int m = 0; m < PACKETS; ++m) load_packet(1, BK, m, offset_for(BK));
-#pragma unroll
-    for (int m = 0; m < PACKETS; ++m) write_packet(0, m);
-    __builtin_amdgcn_sched_barrier(0);  // the set is reloaded only after it has been written out
-#pragma unroll
-    for (int m = 0; m < PACKETS; ++m) load_packet(0, 2 * BK, m, offset_for(2 * BK));
-    lds_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-    int k_load = 3 * BK;  // first k of the tile the next phase loads
-    // All but the last four tiles run in pairs of phases that write and load; the last four wind
-    // the pipeline down.
-    do {  // runs at least once: 4 tiles are loaded by now and at least 6 exist
-        phase(s0{}, yes{}, yes{}, k_load);
-        phase(s1{}, yes{}, yes{}, k_load + BK);
-        k_load += 2 * BK;
-    } while (k_load + BK < k_end);
-    phase(s0{}, yes{}, yes{}, k_load);
-    phase(s1{}, yes{}, no{}, 0);
-    phase(s0{}, yes{}, no{}, 0);
-    phase(s1{}, no{}, no{}, 0);
-    mfma_group(1, [](int) {});  // last k-group of the last tile
-
-#pragma unroll
-    for (int i = 0; i < MI; ++i) {
-#pragma unroll
-        for (int j = 0; j < NI; ++j) {
-            const int col = col0 + wave_n * WN + j * 32 + l32;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int row = row0 + wave_m * WM + i * 32 + 8 * (v / 4) + 4 * lhi + (v % 4);
-                if (!EDGE || (row < R && col < Cn))
-                    store_out(&OUT[static_cast<size_t>(row) * Cn + col], acc[i][j][v]);
-            }
-        }
-    }
-}
-
-// ------------------------------ register-staged pipeline, 16x16x32 matrix instructions --
-// The same pipeline (two LDS stages, two register sets, tile t+3 loaded while tile t is multiplied,
-// LDS-only barriers, the edge handling) around v_mfma_f32_16x16x32_bf16 instead of 32x32x16. Both forms
-// have the same peak rate; on random operands, where the chip is power-limited, a register-only loop
-// of the 16x16x32 form sustains 2.04 PFLOP/s against 1.82 for 32x32x16 (2.47 / 2.50 on all-zero
-// operands), so the same schedule runs at a higher clock.
-//
-// Operand layout of the instruction: lane l supplies P[row l % 16][k = 8 (l / 16) .. + 7] and
-// Q[col l % 16][same k] (one 16 B chunk each, 32 k values per instruction over the four lane
-// groups); result register v of lane l is OUT[4 (l / 16) + v][l % 16]. A wave's 128 x 128 tile is
-// 8 x 8 such sub-tiles (64 accumulators of 4 registers). A K tile of 64 is two k-steps of 32; a k-step
-// is eight "rows" of eight instructions (one P fragment against the eight Q fragments).
-//
-// Fragments: the eight Q fragments of a k-step are double-buffered by k-step parity; the eight P
-// fragments of a k-step have one register slot per row, and the fragment of row i of the next k-step
-// is read four rows after row i of the current one has been issued. The last four rows of a tile
-// are issued after the barrier that ends its phase, from fragments read before it; behind them go the
-// first reads of the next tile (four P fragments, all eight Q fragments of its first k-step), so that
-// no read is needed sooner than about 200 clocks after it is issued: with 48 LDS instructions of
-// 1 KiB per wave and K tile the LDS pipeline of a CU is busy three quarters of the time, and a design
-// with 128 clocks of slack was no faster. Behind the instructions of every row: one P read (j = 0),
-// one LDS write of a staged packet (j = 2) and the global load that refills its registers (j = 3), one
-// Q read for the next k-step (j = 4; after a barrier three per row, j odd).
-//
-// The matrix instruction is issued from inline assembly with the accumulator as a read-write operand:
-// written with the builtin, the compiler gave result and addend different registers, and with all 256
-// accumulation registers taken by the 64 accumulators that meant moving them around in every
-// iteration (hundreds of copies and spills). The compiler does not know the instruction's result
-// latency then; the only place a result is read soon after it is produced is the write-back, which
-// therefore waits first (mfma_results_settle).
+// It is issued from inline assembly with the accumulator as a read-write operand: written with the
+// builtin, the compiler gave result and addend different registers, and with all 256 accumulation
+// registers taken by the 64 accumulators that meant moving them around in every iteration (hundreds of
+// copies and spills). The compiler does not know the instruction's result latency then. What every site
+// that uses it has to guarantee: (1) no instruction other than another in-place matrix instruction on the
+// same accumulator reads or copies an accumulator within 64 idle cycles of the last instruction that wrote
+// it: the only such place is the write-back, which calls mfma_results_settle() first; (2) a fragment
+// register written by a vector instruction (not by an LDS read, whose wait the compiler inserts) is not
+// used by the next five instructions: loops that start with a matrix instruction begin with five wait
+// states; (3) all phases of a K loop are the same straight-line code inside one loop, so that the compiler
+// has no reason to move accumulators between registers behind an instruction whose latency it cannot see.
 __device__ __forceinline__ void mfma_16x16x32_in_place(f32x4& c, bf16x8 a, bf16x8 b) {
     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
@@ -809,206 +544,11 @@ __device__ __forceinline__ void mfma_results_settle() {
     asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 }
 
-template <int BM, int BN, int WM, int WN, bool EDGE, typename OutT>
-__global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_staged16_kernel(
-    int R, int Cn, int K, const uint16_t* __restrict__ P, const uint16_t* __restrict__ Q,
-    OutT* __restrict__ OUT, int tiles_m, int tiles_n) {
-    constexpr int BK = 64, KP = 8, SWZ = 1;
-    constexpr int WAVES_N = BN / WN;
-    constexpr int WAVES = (BM / WM) * WAVES_N;
-    constexpr int MI = WM / 16, NI = WN / 16;
-    static_assert(MI == 8 && NI == 8, "the row schedule below is written for 128 x 128 wave tiles");
-    constexpr int ROWS_PER_LOAD = kWave / KP;
-    constexpr int ROWS_PER_PASS = ROWS_PER_LOAD * WAVES;
-    static_assert(BM % ROWS_PER_PASS == 0 && BN % ROWS_PER_PASS == 0, "whole load passes");
-    constexpr int P_PER = BM / ROWS_PER_PASS, Q_PER = BN / ROWS_PER_PASS;
-    constexpr int PACKETS = P_PER + Q_PER;
-    static_assert(PACKETS == 16, "one LDS write and one global load per row of a phase");
-    static_assert(PRISM_BF16_M16_WRITE_J < PRISM_BF16_M16_LOAD_J && PRISM_BF16_M16_LOAD_J < 8, "a packet is written out before its registers are reloaded");
-
-    __shared__ __attribute__((aligned(1024))) uint16_t Ps[2][BM * BK];
-    __shared__ __attribute__((aligned(1024))) uint16_t Qs[2][BN * BK];
-
-    int tm, tn;
-    xcd_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
-    const int row0 = tm * BM, col0 = tn * BN;
-
-    const int tid = threadIdx.x;
-    const int lane = tid & (kWave - 1);
-    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
-    const int l16 = lane & 15, lq = lane >> 4;
-
-    f32x4 acc[MI][NI];
-#pragma unroll
-    for (int i = 0; i < MI; ++i)
-#pragma unroll
-        for (int j = 0; j < NI; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-
-    // Global and LDS-write side: as in gemm_bf16_staged_kernel.
-    const int ld_row = wave * ROWS_PER_LOAD + lane / KP;
-    const int ld_chunk = (lane % KP) ^ ((ld_row >> SWZ) & (KP - 1));
-    const uint32_t lane_off = (static_cast<uint32_t>(lane / KP) * static_cast<uint32_t>(K) + ld_chunk * 8) * 2u;
-    constexpr uint32_t kBeyond = 0x80000000u;
-    auto extent = [&](int first_row, int rows) -> int {
-        if (!EDGE) return 0x7fffffff;
-        return static_cast<int>(clamped_extent(static_cast<long long>(rows - first_row) * K * 2));
-    };
-    const int p_first = row0 + wave * ROWS_PER_LOAD, q_first = col0 + wave * ROWS_PER_LOAD;
-    const auto p_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t*>(P + (EDGE && p_first >= R ? size_t{0} : static_cast<size_t>(p_first) * K)), 0,
-        extent(p_first, R), 0x00020000);
-    const auto q_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t*>(Q + (EDGE && q_first >= Cn ? size_t{0} : static_cast<size_t>(q_first) * K)), 0,
-        extent(q_first, Cn), 0x00020000);
-    const int pass_bytes = ROWS_PER_PASS * K * 2;
-    const int k_full = K - K % BK;
-    const int k_end = EDGE ? ((K + 2 * BK - 1) / (2 * BK) < 3 ? 6 * BK : (K + 2 * BK - 1) / (2 * BK) * 2 * BK) : K;
-    const uint32_t tail_off = (EDGE && k_full + ld_chunk * 8 < K) ? lane_off : kBeyond;
-    u32x4 staged[2][PACKETS];
-    auto offset_for = [&](int k0) -> uint32_t {
-        if (!EDGE) return lane_off;
-        return k0 < k_full ? lane_off : (k0 < K ? tail_off : kBeyond);
-    };
-    auto load_packet = [&](int set, int k0, int m, uint32_t off) {
-        if (m < P_PER)
-            staged[set][m] = __builtin_amdgcn_raw_buffer_load_b128(p_rsrc, off, m * pass_bytes + k0 * 2, 0);
-        else
-            staged[set][m] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, off, (m - P_PER) * pass_bytes + k0 * 2, 0);
-    };
-    auto write_packet = [&](int set, int m) {
-        uint16_t* dst = (m < P_PER) ? &Ps[set][(m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]
-                                    : &Qs[set][((m - P_PER) * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK];
-        *reinterpret_cast<u32x4*>(dst + lane * 8) = staged[set][m];
-    };
-
-    // Operand side: row (wave tile origin + 16 i + l16), chunk 4 kk + lq of the row, kept in slot
-    // chunk ^ ((row >> 1) & 7) (the row term is that of l16: 16 i is a multiple of 16).
-    const int sw = (l16 >> SWZ) & (KP - 1);
-    int p_off[2], q_off[2];
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-        const int slot = (4 * kk + lq) ^ sw;
-        p_off[kk] = (wave_m * WM + l16) * BK + slot * 8;
-        q_off[kk] = (wave_n * WN + l16) * BK + slot * 8;
-    }
-    bf16x8 fp[MI], fq[2][NI];  // P fragments: one slot per row; Q fragments: by k-step parity
-    auto read_p = [&](int stage, int kk, int i) {
-        fp[i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&Ps[stage][p_off[kk] + i * 16 * BK]));
-    };
-    auto read_q = [&](int stage, int kk, int j) {
-        fq[kk][j] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&Qs[stage][q_off[kk] + j * 16 * BK]));
-    };
-    // Row i of k-step kk: eight instructions; `after(j)` is issued right behind the j-th.
-    auto mfma_row = [&](int kk, int i, auto after) {
-#pragma unroll
-        for (int j = 0; j < NI; ++j) {
-            mfma_16x16x32_in_place(acc[i][j], fp[i], fq[kk][j]);
-            __builtin_amdgcn_sched_barrier(0);
-            after(j);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    };
-
-    // One phase = everything between two barriers, for the tile in stage S (tile t). Entered right after
-    // the barrier that says "tile t is complete in stage S and nobody reads stage S^1 any more", with
-    // rows 4..7 of tile t-1's second k-step still to do (their fragments are in registers). Register set
-    // S^1 holds tile t+1: packet n is written to stage S^1 behind row n of the phase (`write`) and
-    // refilled with tile t+3, which starts at k_load (`load`).
-    auto phase = [&](auto stage_c, auto write, auto load, int k_load) {
-        constexpr int S = decltype(stage_c)::value;
-        const uint32_t off = offset_for(k_load);
-        auto staging = [&](int n, int j) {  // the LDS write and the global load of row n of the phase
-            if (j == PRISM_BF16_M16_WRITE_J) { if constexpr (write) write_packet(S ^ 1, n); }
-            if (j == PRISM_BF16_M16_LOAD_J) { if constexpr (load) load_packet(S ^ 1, k_load, n, off); }
-        };
-        // rows 4..7 of the previous tile; behind them the first reads of this tile
-#pragma unroll
-        for (int i = 4; i < 8; ++i)
-            mfma_row(1, i, [&](int j) {
-                if (j == 0) read_p(S, 0, i - 4);
-                if (j % 2 == 1 && j < 6 && 3 * (i - 4) + j / 2 < NI) read_q(S, 0, 3 * (i - 4) + j / 2);
-                staging(i - 4, j);
-            });
-        // k-step 0: rows 0..7
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-            mfma_row(0, i, [&](int j) {
-                if (j == 0) { if (i < 4) read_p(S, 0, i + 4); else read_p(S, 1, i - 4); }
-                if (j == 4) read_q(S, 1, i);
-                staging(4 + i, j);
-            });
-        // k-step 1: rows 0..3 (4..7 follow the barrier)
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            mfma_row(1, i, [&](int j) {
-                if (j == 0) read_p(S, 1, i + 4);
-                staging(12 + i, j);
-            });
-        lds_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    using yes = std::integral_constant<bool, true>;
-    using no = std::integral_constant<bool, false>;
-    using s0 = std::integral_constant<int, 0>;
-    using s1 = std::integral_constant<int, 1>;
-
-    // "Rows 4..7 of the tile before the first" multiply zeros.
-#pragma unroll
-    for (int i = 4; i < 8; ++i) fp[i] = bf16x8{};
-#pragma unroll
-    for (int j = 0; j < NI; ++j) fq[1][j] = bf16x8{};
-
-    // Even number of K tiles, at least 6; the first in stage 0 and the last in stage 1 (as above).
-#pragma unroll
-    for (int m = 0; m < PACKETS; ++m) load_packet(0, 0, m, offset_for(0));
-#pragma unroll
-    for (int m = 0; m < PACKETS; ++m) load_packet(1, BK, m, offset_for(BK));
-#pragma unroll
-    for (int m = 0; m < PACKETS; ++m) write_packet(0, m);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int m = 0; m < PACKETS; ++m) load_packet(0, 2 * BK, m, offset_for(2 * BK));
-    lds_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-    int k_load = 3 * BK;
-    do {
-        // Wait states between vector-ALU writes of fragment registers (the zeros above, the compiler's
-        // copies of them in front of the loop) and the inline-assembly matrix instructions that read
-        // them; see the note at the head of gemm_bf16_early_kernel's loop.
-        asm volatile("s_nop 4");
-        phase(s0{}, yes{}, yes{}, k_load);
-        phase(s1{}, yes{}, yes{}, k_load + BK);
-        k_load += 2 * BK;
-    } while (k_load + BK < k_end);
-    phase(s0{}, yes{}, yes{}, k_load);
-    phase(s1{}, yes{}, no{}, 0);
-    phase(s0{}, yes{}, no{}, 0);
-    phase(s1{}, no{}, no{}, 0);
-#pragma unroll
-    for (int i = 4; i < 8; ++i) mfma_row(1, i, [](int) {});  // the last four rows of the last tile
-    mfma_results_settle();
-
-#pragma unroll
-    for (int i = 0; i < MI; ++i) {
-#pragma unroll
-        for (int j = 0; j < NI; ++j) {
-            const int col = col0 + wave_n * WN + j * 16 + l16;
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int row = row0 + wave_m * WM + i * 16 + 4 * lq + v;
-                if (!EDGE || (row < R && col < Cn))
-                    store_out(&OUT[static_cast<size_t>(row) * Cn + col], acc[i][j][v]);
-            }
-        }
-    }
-}
-
 // ------------------------------ direct-to-LDS loads with early fragment reads, 16x16x32 --
-// Whole tiles, an even number (at least 4) of K tiles. The staged kernels above pay for their lead time
-// with 16 LDS write instructions per wave and K tile; this one has none: global data goes straight into
-// LDS (direct_load.h) as in the ring kernel, whose problem was that a stage had to be free before the
-// load into it could be issued, which left a load less than one tile time. Here all 32 fragments of a K
+// Whole tiles, an even number (at least 4) of K tiles. Global data goes straight into LDS (direct_load.h) as
+// in the ring kernel, whose problem is that a stage has to be free before the load into it can be issued,
+// which leaves a load less than one tile time (a pipeline that staged tiles through registers instead bought
+// its lead time with 16 LDS write instructions per wave and K tile and was 2-3 % slower). Here all 32 fragments of a K
 // tile are read into registers behind the first 32 matrix instructions of its phase (three sets of
 // 8 + 8 fragments: k-step 0 of this tile, k-step 1 of this tile, k-step 1 of the previous tile, which is
 // what those instructions multiply), a barrier in mid-phase then says that nobody reads the stage any
@@ -1110,7 +650,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
                                  &Qs[stage][((m - P_PER) * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK]);
     };
 
-    // Operand side, as in gemm_bf16_staged16_kernel.
+    // Operand side.
     const int sw = (l16 >> SWZ) & (KP - 1);
     int p_off[2], q_off[2];
 #pragma unroll
@@ -1158,7 +698,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
         constexpr int MINE = 1 + S, OTHER = 2 - S;  // fragment sets of k-step 1: this stage's, the other stage's
         // Load number n goes behind instruction BARRIER_AT + n * GAP of the phase's 128 (counted from the
         // start of the first block); the barrier that frees the stage sits behind instruction BARRIER_AT - 1.
-        constexpr int BARRIER_AT = PRISM_BF16_EARLY_BARRIER_AT, GAP = PRISM_BF16_EARLY_LOAD_GAP;
+        constexpr int BARRIER_AT = kEarlyBarrierAt, GAP = kEarlyLoadGap;
         static_assert(BARRIER_AT >= 33 && BARRIER_AT <= 64 && BARRIER_AT + (LOADS - 1) * GAP < 128, "loads fit the phase");
         const i32x4 pd = advanced(p_rsrc, k_next_bytes), qd = advanced(q_rsrc, k_next_bytes);
         const uint32_t off = lane_offset_at(static_cast<int>(k_next_bytes / 2));
@@ -1201,8 +741,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     // operands instead of all 256 workgroups from the same 128 B of 8192 rows. (All workgroups of one XCD
     // keep the same phase: they share panels through its L2.)
     int k_first = 0;
-    if constexpr (PRISM_BF16_K_STAGGER != 0) {
-        const int step = PRISM_BF16_K_STAGGER > 0 ? PRISM_BF16_K_STAGGER : (PRISM_BF16_K_STAGGER == -2 ? (k_tiles / 2) & ~1 : (k_tiles / kXcds) & ~1);
+    if constexpr (kEarlyKStagger != 0) {
+        const int step = kEarlyKStagger;
         k_first = __builtin_amdgcn_readfirstlane((static_cast<int>(blockIdx.x % kXcds) * step) % k_tiles);
     }
     auto k_bytes_of = [&](int t) -> uint32_t {  // byte offset along K of the t-th tile of this workgroup's walk
@@ -1270,58 +810,10 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));
 }
 
-// Kernel choice. Whole 256 x 256 x 64 tiles: the early-read pipeline (or, on request, a register-staged
-// one) whenever the K tile count is even and at least 6, else the direct-to-LDS ring (any count from 2).
-// Ragged M, N or K with K a multiple of 8 and 16 B-aligned operands: the same pipeline's edge variant
-// (K tiles padded with zeros to an even count). Fewer than 128 tiles: 128 x 128 tiles of the ring.
-// Everything else: the general kernel.
-#ifndef PRISM_BF16_STAGED_MIN_K
-#define PRISM_BF16_STAGED_MIN_K 384
-#endif
-#ifndef PRISM_BF16_STAGED_EDGES
-#define PRISM_BF16_STAGED_EDGES 1
-#endif
-#ifndef PRISM_BF16_LEFTOVER
-#define PRISM_BF16_LEFTOVER 1
-#endif
-#ifndef PRISM_BF16_EARLY
-#define PRISM_BF16_EARLY 1  // 1: whole-tile problems take gemm_bf16_early_kernel, 0: the staged pipeline
-#endif
-#ifndef PRISM_BF16_MFMA16
-#define PRISM_BF16_MFMA16 1  // the staged pipeline on 16x16x32 instructions (0: on 32x32x16)
-#endif
-#ifndef PRISM_BF16_SMALL_TILES
-#define PRISM_BF16_SMALL_TILES 1
-#endif
-#ifndef PRISM_BF16_SMALL_MAX_QUARTERS
-#define PRISM_BF16_SMALL_MAX_QUARTERS 2
-#endif
-#ifndef PRISM_BF16_SMALL_DEEP_RING
-#define PRISM_BF16_SMALL_DEEP_RING 1
-#endif
-#ifndef PRISM_BF16_RING_BK
-#define PRISM_BF16_RING_BK 64
-#endif
-#ifndef PRISM_BF16_RING_STAGES
-#define PRISM_BF16_RING_STAGES 2
-#endif
-
-// Which of the three pipelines takes problems made of whole 256 x 256 x 64 tiles: PRISM_BF16_KERNEL in the
-// environment, read at every call.
-//   early (default)  direct-to-LDS with early fragment reads, 16x16x32 instructions
-//   staged16         register-staged, 16x16x32 instructions (also the kernel for ragged problems)
-//   staged32         register-staged, 32x32x16 instructions (then also for ragged problems)
-// Under bench.py at 8192^3, alternating on one box: early 1.43 PFLOP/s, staged16 1.39-1.41; early is also
-// 2-3 % ahead at 16384^3 and level at 4096^3.
-inline int whole_tile_kernel() {
-    const char* v = getenv("PRISM_BF16_KERNEL");
-    if (v == nullptr) return PRISM_BF16_EARLY ? 2 : (PRISM_BF16_MFMA16 ? 1 : 0);
-    if (strcmp(v, "staged32") == 0) return 0;
-    if (strcmp(v, "staged16") == 0) return 1;
-    if (strcmp(v, "early") == 0) return 2;
-    return PRISM_BF16_EARLY ? 2 : (PRISM_BF16_MFMA16 ? 1 : 0);
-}
-
+// Kernel choice. Whole 256 x 256 x 64 tiles: the early-read pipeline whenever the K tile count is even and
+// at least 6, else the direct-to-LDS ring (any count from 2). Ragged M, N or K with K a multiple of 8 and
+// 16 B-aligned operands: the early-read pipeline's edge variant (K tiles padded with zeros to an even count).
+// Fewer than 128 tiles: 128 x 128 tiles of the ring. Everything else: the general kernel.
 template <int BM, int BN, int BK, int WM, int WN, typename OutT>
 int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, OutT* OUT,
                   hipStream_t s) {
@@ -1331,33 +823,24 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
     const dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n), block((BM / WM) * (BN / WN) * kWave);
     const bool aligned = aligned16(P) && aligned16(Q);
     const bool whole = (R % BM == 0) && (Cn % BN == 0) && aligned;
-    // The staged kernel addresses a 256-row panel (plus up to six K tiles of padding) with 32-bit offsets.
+    // A 256-row panel (plus up to six K tiles of padding) is addressed with 32-bit offsets.
     const bool panel_ok = static_cast<long long>(BM > BN ? BM : BN) * (static_cast<long long>(K) + 6 * 64) * 2 < (1ll << 31);
-    const bool few_tiles = PRISM_BF16_SMALL_TILES && static_cast<long long>(tiles_m) * tiles_n * 4 <
-                                                         static_cast<long long>(PRISM_BF16_SMALL_MAX_QUARTERS) * cu_count();
-    if (whole && !few_tiles && K % 128 == 0 && K >= 6 * 64 && K >= PRISM_BF16_STAGED_MIN_K && panel_ok) {
-        // Tile counts that do not fill whole rounds of CUs: the staged kernel takes the whole rounds and
+    const bool few_tiles = static_cast<long long>(tiles_m) * tiles_n * 2 < cu_count();
+    const bool lane_offsets_ok = static_cast<long long>(K) * 2 * 64 < (1ll << 32);  // 32-bit lane offsets inside a load's rows
+    if (whole && !few_tiles && K % 128 == 0 && K >= 6 * 64 && panel_ok && lane_offsets_ok) {
+        // Tile counts that do not fill whole rounds of CUs: the 256 x 256 kernel takes the whole rounds and
         // the tiles of the last, partial round are cut into 128 x 128 tiles (two workgroups per CU), when
         // that gives every CU at most two of them (6144^3: 2 rounds + 64 tiles instead of 3 rounds).
         static_assert(BM == 256 && BN == 256, "the leftover launch cuts 256 x 256 tiles");
         const int tiles = tiles_m * tiles_n, cus = cu_count();
         const int left = tiles % cus;
-        const bool cut = PRISM_BF16_LEFTOVER && tiles > cus && left != 0 && left * 4 <= 2 * cus &&
-                         static_cast<long long>(K) * 2 * 64 < (1ll << 32);
+        const bool cut = tiles > cus && left != 0 && left * 4 <= 2 * cus;
         const int main_tiles = cut ? tiles - left : tiles;
-        const int which = whole_tile_kernel();
-        if (which == 2 && static_cast<long long>(K) * 2 * 64 < (1ll << 32))
-            gemm_bf16_early_kernel<BM, BN, WM, WN, false, OutT><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
-                R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
-        else if (which != 0)
-            gemm_bf16_staged16_kernel<BM, BN, WM, WN, false, OutT><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
-                R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
-        else
-            gemm_bf16_staged_kernel<BM, BN, WM, WN, false, OutT><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
-                R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
-        if (int rc = check_launch("gemm_bf16_staged_kernel")) return rc;
+        gemm_bf16_early_kernel<BM, BN, WM, WN, false, OutT><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
+            R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
+        if (int rc = check_launch("gemm_bf16_early_kernel")) return rc;
         if (cut) {
-            if (PRISM_BF16_SMALL_DEEP_RING && left * 4 <= cus)  // one per CU: the four-deep ring, as below
+            if (left * 4 <= cus)  // one per CU: the four-deep ring, as below
                 gemm_bf16_ring_kernel<128, 128, 64, 4, 64, 64, false, OutT><<<dim3(static_cast<unsigned>(left) * 4), dim3(256), 0, s>>>(
                     R, Cn, K, P, Q, OUT, tiles_m, tiles_n, main_tiles);
             else
@@ -1374,31 +857,25 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
         const bool whole128 = R % 128 == 0 && Cn % 128 == 0 && K % 64 == 0;
         // At most one workgroup per CU: nothing else hides the memory latency, so the ring is four K tiles
         // deep (128 KB of LDS) instead of two.
-        if (PRISM_BF16_SMALL_DEEP_RING && whole128 && K >= 256 && tm * tn <= cu_count())
+        if (whole128 && K >= 256 && tm * tn <= cu_count())
             gemm_bf16_ring_kernel<128, 128, 64, 4, 64, 64, false, OutT><<<grid128, dim3(256), 0, s>>>(R, Cn, K, P, Q, OUT, tm, tn, -1);
         else if (whole128 && K >= 128)
             gemm_bf16_ring_kernel<128, 128, 64, 2, 64, 64, false, OutT><<<grid128, dim3(256), 0, s>>>(R, Cn, K, P, Q, OUT, tm, tn, -1);
-        else if (PRISM_BF16_SMALL_DEEP_RING && K >= 256 && tm * tn <= cu_count())
+        else if (K >= 256 && tm * tn <= cu_count())
             gemm_bf16_ring_kernel<128, 128, 64, 4, 64, 64, true, OutT><<<grid128, dim3(256), 0, s>>>(R, Cn, K, P, Q, OUT, tm, tn, -1);
         else
             gemm_bf16_ring_kernel<128, 128, 64, 2, 64, 64, true, OutT><<<grid128, dim3(256), 0, s>>>(R, Cn, K, P, Q, OUT, tm, tn, -1);
         return check_launch("gemm_bf16_ring_kernel (128 x 128)");
     }
-    if (whole && K % PRISM_BF16_RING_BK == 0 && K >= PRISM_BF16_RING_BK * PRISM_BF16_RING_STAGES &&
-        static_cast<long long>(K) * 2 * 64 < (1ll << 32)) {  // 32-bit lane offsets inside a load's rows
-        gemm_bf16_ring_kernel<BM, BN, PRISM_BF16_RING_BK, PRISM_BF16_RING_STAGES, WM, WN, false, OutT>
+    if (whole && K % 64 == 0 && K >= 64 * 2 && lane_offsets_ok) {
+        gemm_bf16_ring_kernel<BM, BN, 64, 2, WM, WN, false, OutT>
             <<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n, -1);
         return check_launch("gemm_bf16_ring_kernel");
     }
-    // Ragged M, N or K with 16 B-aligned rows: the staged kernel with zero-filled edges.
-    if (PRISM_BF16_STAGED_EDGES && aligned && K % 8 == 0 && K > 0 && panel_ok) {
-        if (whole_tile_kernel() == 2 && static_cast<long long>(K) * 2 * 64 < (1ll << 32))
-            gemm_bf16_early_kernel<BM, BN, WM, WN, true, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
-        else if (whole_tile_kernel() != 0)
-            gemm_bf16_staged16_kernel<BM, BN, WM, WN, true, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
-        else
-            gemm_bf16_staged_kernel<BM, BN, WM, WN, true, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
-        return check_launch("gemm_bf16_staged_kernel (edges)");
+    // Ragged M, N or K with 16 B-aligned rows: the early-read kernel with zero-filled edges.
+    if (aligned && K % 8 == 0 && K > 0 && panel_ok && lane_offsets_ok) {
+        gemm_bf16_early_kernel<BM, BN, WM, WN, true, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
+        return check_launch("gemm_bf16_early_kernel (edges)");
     }
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<BM, BN, BK, WM, WN, true, OutT>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
@@ -1418,9 +895,9 @@ int launch_gemm_bf16(int M, int N, int K, const uint16_t* A, const uint16_t* B, 
     if (K > 0 && (A == nullptr || B == nullptr)) return fail(1, "prism_gemm_bf16: null matrix pointer");
     if (!aligned2(A) || !aligned2(B) || !aligned4(D_f32) || !aligned2(C_bf16_colmajor))
         return fail(1, "prism_gemm_bf16: misaligned pointer");
-    if (D_f32) return run_gemm_bf16<PRISM_BF16_CFG, float>(M, N, K, A, B, D_f32, s);
+    if (D_f32) return run_gemm_bf16<256, 256, 64, 128, 128, float>(M, N, K, A, B, D_f32, s);
     // Column-major M x N == row-major N x M of B @ A^T.
-    return run_gemm_bf16<PRISM_BF16_CFG, uint16_t>(N, M, K, B, A, C_bf16_colmajor, s);
+    return run_gemm_bf16<256, 256, 64, 128, 128, uint16_t>(N, M, K, B, A, C_bf16_colmajor, s);
 }
 
 }  // namespace prism

@@ -231,8 +231,7 @@ __device__ __forceinline__ uint32_t look_back(const u64* status, uint32_t parity
         // Lanes 0..first-prefix-lane are needed; all 64 when no prefix is in the window.
         const u64 needed = has_prefix ? ((2ull << __builtin_ctzll(has_prefix)) - 1ull) : ~0ull;
         if (is_invalid & needed) {
-            ++spins;
-            __builtin_amdgcn_s_sleep(1);
+            ++spins;  // no s_sleep: the wait for the poll's answer paces the loop (sleeping measured 1 % slower)
             continue;
         }
         const uint32_t contrib = ((needed >> lane) & 1ull) ? value : Op::identity;

@@ -34,11 +34,6 @@
 #include "direct_load.h"
 #include "tile_map.h"
 
-// General kernel 5 tile shape: BM, BN, BK, WM, WN.
-#ifndef PRISM_SGEMM5_CFG
-#define PRISM_SGEMM5_CFG 128, 128, 16, 64, 64
-#endif
-
 namespace prism {
 namespace {
 
@@ -258,12 +253,9 @@ __global__ __launch_bounds__((BM * BN) / (TM * TN)) void sgemm_thread_tile_kerne
 // Workgroups are dealt to the 8 XCDs round-robin by id; the id is remapped so
 // that every XCD walks its own contiguous band of C tiles in columns of 8, and
 // the tiles resident on one XCD share A and B panels in that XCD's L2.
-#ifndef PRISM_SGEMM5_WAVES_PER_EU
-#define PRISM_SGEMM5_WAVES_PER_EU 4
-#endif
 template <int BM, int BN, int BK, int WM, int WN, bool EDGE>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave)
-__attribute__((amdgpu_waves_per_eu(PRISM_SGEMM5_WAVES_PER_EU))) void sgemm_wave_tile_kernel(
+__attribute__((amdgpu_waves_per_eu(4))) void sgemm_wave_tile_kernel(
     int M, int N, int K, float alpha, const float* __restrict__ A, const float* __restrict__ B,
     float beta, float* C, int tiles_m, int tiles_n) {
     constexpr int WAVES_N = BN / WN;
@@ -420,7 +412,7 @@ __attribute__((amdgpu_waves_per_eu(PRISM_SGEMM5_WAVES_PER_EU))) void sgemm_wave_
 // clocks (measured with one wave per SIMD; LDS reads cost about 5, scalar
 // instructions and barriers nothing), so the loop contains none: the direct
 // loads take a scalar base and a fixed lane offset (direct_load.h), one load
-// behind every PRISM_SGEMM5_LOAD_GAP-th MFMA of the first group, pinned there
+// behind every fourth MFMA of the first group, pinned there
 // with scheduling barriers (bunched loads hold the wave at the memory pipeline).
 //
 // LDS layout of one K tile (two stages):
@@ -437,15 +429,6 @@ __attribute__((amdgpu_waves_per_eu(PRISM_SGEMM5_WAVES_PER_EU))) void sgemm_wave_
 // chunk into sub-tile j: the two k values of a 32x32x2 instruction are
 // k8 + jj and k8 + 4 + jj, and lane l32 of sub-tile j holds column 4 l32 + j,
 // so a lane owns 4 consecutive columns of C and stores them as one 16 B packet.
-#ifndef PRISM_SGEMM5_SCHED
-#define PRISM_SGEMM5_SCHED 1
-#endif
-#ifndef PRISM_SGEMM5_LATE_BARRIER
-#define PRISM_SGEMM5_LATE_BARRIER 1
-#endif
-#ifndef PRISM_SGEMM5_LOAD_GAP
-#define PRISM_SGEMM5_LOAD_GAP 4
-#endif
 template <int BM, int BN, int BK, int WM, int WN, bool EDGE>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile_dma_kernel(
     int M, int N, int K, float alpha, const float* __restrict__ A, const float* __restrict__ B,
@@ -463,7 +446,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
     static_assert(BM % ROWS_PER_PASS == 0 && BK % WAVES == 0, "whole load passes");
     constexpr int A_PER = BM / ROWS_PER_PASS, B_PER = BK / WAVES;  // loads per wave per tile
     // MFMAs between two direct loads: the configured gap, or less when the first group is too short for it
-    constexpr int LOAD_GAP = (A_PER + B_PER) * PRISM_SGEMM5_LOAD_GAP <= 4 * MI * 4 ? PRISM_SGEMM5_LOAD_GAP : (4 * MI * 4) / (A_PER + B_PER);
+    constexpr int WANTED_GAP = 4;
+    constexpr int LOAD_GAP = (A_PER + B_PER) * WANTED_GAP <= 4 * MI * 4 ? WANTED_GAP : (4 * MI * 4) / (A_PER + B_PER);
     static_assert(LOAD_GAP >= 1 && (A_PER + B_PER) * LOAD_GAP <= 4 * MI * 4, "the loads of a tile fit among the MFMAs of one group");
     static_assert(((ROWS_PER_PASS >> SWZ) % KP) == 0 && ((32 >> SWZ) % KP) == 0,
                   "the swizzle term must repeat with the load pass and the 32-row MFMA block");
@@ -609,7 +593,6 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
             read_frags(as, bs, s + 1, (s + 1) & 1);
             mfma_all(s & 1, nothing);
         }
-#if PRISM_SGEMM5_SCHED
         constexpr int G = 4 * MI * NI;  // MFMAs per group
         constexpr int PLACED = prefetch ? (LOADS - 1) * LOAD_GAP + 1 : 0;  // MFMAs above the last sched_barrier
         if constexpr (!prefetch) __builtin_amdgcn_sched_group_barrier(0x100, MI + 4, 0);
@@ -620,10 +603,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
             __builtin_amdgcn_sched_group_barrier(0x100, MI + 4, 0);
             __builtin_amdgcn_sched_group_barrier(0x008, G - 4, 0);
         }
-#endif
-#if PRISM_SGEMM5_LATE_BARRIER
         __builtin_amdgcn_sched_barrier(0);  // keep the MFMAs above the barrier: the direct loads get a whole tile to land
-#endif
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));  // the direct loads are invisible to the compiler's wait counts
         __syncthreads();
     };
@@ -713,8 +693,14 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
 // EDGE: M, N, K need not be whole tiles (N and K multiples of 4); edges are zero-filled as in the
 // whole-tile kernel above (buffer descriptors that end with the matrices, an out-of-range lane
 // offset past a row's end), and the K loop runs over at least STAGES tiles, those beyond K all zeros.
-template <int WT, int STAGES, bool EDGE>
-__global__ __launch_bounds__(kWave) void sgemm_single_wave_kernel(
+//
+// KSPLIT > 1 (whole tiles only): with fewer tiles than SIMDs a tile's K range is cut into KSPLIT equal
+// parts, one per wave of a workgroup of KSPLIT waves, each with its own ring; the partial tiles meet in
+// LDS and wave 0 adds them in the fixed order 0, 1, ..., KSPLIT - 1 (the same bits on every run) and
+// writes C. A K split across workgroups would need a workspace the entry points do not have; this one
+// needs none. (128 x 4096 x 4096: 512 tiles of 32 x 32 on 1024 SIMDs, 72 TFLOP/s unsplit.)
+template <int WT, int STAGES, bool EDGE, int KSPLIT = 1>
+__global__ __launch_bounds__(kWave * KSPLIT) void sgemm_single_wave_kernel(
     int M, int N, int K, float alpha, const float* __restrict__ A, const float* __restrict__ B,
     float beta, float* C, int tiles_m, int tiles_n, int first_big) {
     constexpr int BK = 16, KP = 4, SWZ = 2, KS = 2;
@@ -728,8 +714,12 @@ __global__ __launch_bounds__(kWave) void sgemm_single_wave_kernel(
     static_assert(LOADS <= GROUP, "the loads of a tile fit among the MFMAs of one group");
     static_assert((STAGES - 1) * LOADS < 64, "outstanding loads fit the vmcnt counter");
 
-    __shared__ __attribute__((aligned(1024))) float As[STAGES][WT * BK];
-    __shared__ __attribute__((aligned(1024))) float Bs[STAGES][BK * WT];
+    static_assert(KSPLIT == 1 || !EDGE, "the K split is written for whole tiles");
+    __shared__ __attribute__((aligned(1024))) float As_all[KSPLIT][STAGES][WT * BK];
+    __shared__ __attribute__((aligned(1024))) float Bs_all[KSPLIT][STAGES][BK * WT];
+    const int wave = KSPLIT == 1 ? 0 : __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / kWave);
+    float (&As)[STAGES][WT * BK] = As_all[wave];
+    float (&Bs)[STAGES][BK * WT] = Bs_all[wave];
 
     // first_big < 0: the grid covers the whole tiles_m x tiles_n grid of WT x WT tiles. Otherwise this
     // launch finishes what a launch of the 256 x 256 kernel left over: tiles_m x tiles_n is that kernel's
@@ -750,8 +740,10 @@ __global__ __launch_bounds__(kWave) void sgemm_single_wave_kernel(
         col0 = tn * 256 + (sub % SUB) * WT;
     }
     if (EDGE && (row0 >= M || col0 >= N)) return;  // a piece of an edge tile that lies wholly outside C
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x % kWave;
     const int l32 = lane & 31, lhi = lane >> 5;
+    // This wave's part of K: k_len values starting at k_begin (the launcher makes K / KSPLIT whole K tiles).
+    const int k_len = K / KSPLIT, k_begin = wave * k_len;
 
     f32x16 acc[MI][NI];
 #pragma unroll
@@ -769,8 +761,8 @@ __global__ __launch_bounds__(kWave) void sgemm_single_wave_kernel(
     const int b_krow = WT == 64 ? lane / 16 : (lane / 16) + 4 * ((lane / 8) & 1);
     const int b_col = WT == 64 ? 4 * (lane % 16) : 4 * (lane % 8);
     const uint32_t b_lane = (static_cast<uint32_t>(b_krow) * static_cast<uint32_t>(N) + b_col) * 4u;
-    const char* a_base = reinterpret_cast<const char*>(A + static_cast<size_t>(row0) * K);
-    const char* b_base = reinterpret_cast<const char*>(B + col0);
+    const char* a_base = reinterpret_cast<const char*>(A + static_cast<size_t>(row0) * K + k_begin);
+    const char* b_base = reinterpret_cast<const char*>(B + static_cast<size_t>(k_begin) * N + col0);
     const i32x4 a_rsrc = buffer_descriptor(a_base, EDGE ? clamped_extent(static_cast<long long>(M - row0) * K * 4) : 0u);
     const i32x4 b_rsrc = buffer_descriptor(b_base, EDGE ? clamped_extent((static_cast<long long>(K) * N - col0) * 4) : 0u);
     const int k_full = K - K % BK;
@@ -873,7 +865,7 @@ __global__ __launch_bounds__(kWave) void sgemm_single_wave_kernel(
 
     // Unless EDGE, the launcher guarantees K % 16 == 0 and at least STAGES tiles. Tile t lives in stage
     // (first + t) % STAGES with `first` chosen such that the last tile sits in the last stage.
-    const int k_tiles = EDGE ? ((K + BK - 1) / BK < STAGES ? STAGES : (K + BK - 1) / BK) : K / BK;
+    const int k_tiles = EDGE ? ((K + BK - 1) / BK < STAGES ? STAGES : (K + BK - 1) / BK) : k_len / BK;
     const int ragged = k_tiles % STAGES;
     const int first = (STAGES - ragged) % STAGES;
 #pragma unroll
@@ -905,6 +897,30 @@ __global__ __launch_bounds__(kWave) void sgemm_single_wave_kernel(
     phase(s2{}, no{}, 0);
     phase(s3{}, no{}, 0);
     mfma_group(1, nothing);  // last group of the last tile
+
+    if constexpr (KSPLIT > 1) {
+        // Partial tiles of waves 1 .. KSPLIT - 1 go through LDS (register v of lane l at [v][l]: no bank
+        // conflicts); wave 0 adds them in order and carries on alone.
+        __shared__ float partial[KSPLIT - 1][MI * NI * 16][kWave];
+        if (wave > 0) {
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) partial[wave - 1][(i * NI + j) * 16 + v][lane] = acc[i][j][v];
+        }
+        __syncthreads();
+        if (wave > 0) return;
+#pragma unroll
+        for (int w = 1; w < KSPLIT; ++w)
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) acc[i][j][v] += partial[w - 1][(i * NI + j) * 16 + v][lane];
+    }
 
     // Epilogue: a lane holds columns NI l32 .. NI l32 + NI - 1 of 16 rows per 32-row block.
     float* c_lane = C + static_cast<size_t>(row0 + 4 * lhi) * N + col0 + NI * l32;
@@ -984,41 +1000,19 @@ int run_wave_tile(int M, int N, int K, float alpha, const float* A, const float*
 
 // Whole-tile kernel when the problem is made of 256 x 256 tiles and there are
 // enough of them for three quarters of the CUs.
-#ifndef PRISM_SGEMM5_DMA
-#define PRISM_SGEMM5_DMA 1
-#endif
-#ifndef PRISM_SGEMM5_LEFTOVER
-#define PRISM_SGEMM5_LEFTOVER 1
-#endif
-#ifndef PRISM_SGEMM5_EDGES
-#define PRISM_SGEMM5_EDGES 1
-#endif
-#ifndef PRISM_SGEMM5_DMA_MIN_QUARTERS
-#define PRISM_SGEMM5_DMA_MIN_QUARTERS 3
-#endif
-#ifndef PRISM_SGEMM5_SINGLE_ROUNDS
-#define PRISM_SGEMM5_SINGLE_ROUNDS 1
-#endif
-#ifndef PRISM_SGEMM5_LEFTOVER_HALVES
-#define PRISM_SGEMM5_LEFTOVER_HALVES 1
-#endif
-#ifndef PRISM_SGEMM5_LEFTOVER_SLICES
-#define PRISM_SGEMM5_LEFTOVER_SLICES 1
-#endif
 template <int BM, int BN, int BK, int WM, int WN, bool ALLOW_EDGES>
 bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const float* B, float beta,
                        float* C, hipStream_t s, int* rc) {
-    if (!PRISM_SGEMM5_DMA) return false;
     if (K <= 0 || !aligned16(A) || !aligned16(B) || !aligned16(C)) return false;
     const bool whole = M % BM == 0 && N % BN == 0 && K % BK == 0;
     // Ragged edges: rows must stay 16 B aligned, and the kernel's buffer offsets are 32 bits wide
     // (a 256-row panel of A plus one K tile; all of B plus one K tile).
-    if (!whole && (!PRISM_SGEMM5_EDGES || !ALLOW_EDGES || N % 4 || K % 4 ||
+    if (!whole && (!ALLOW_EDGES || N % 4 || K % 4 ||
                    (static_cast<long long>(BM) + 64) * K * 4 >= (1ll << 31) ||
                    (static_cast<long long>(K) + 64) * N * 4 >= (1ll << 31)))
         return false;
     const int tiles_m = ceil_div(M, BM), tiles_n = ceil_div(N, BN);
-    if (static_cast<long long>(tiles_m) * tiles_n * 4 < static_cast<long long>(PRISM_SGEMM5_DMA_MIN_QUARTERS) * cu_count()) return false;
+    if (static_cast<long long>(tiles_m) * tiles_n * 4 < 3ll * cu_count()) return false;
     const dim3 block((BM / WM) * (BN / WN) * kWave);
     // Tile counts that do not fill whole rounds of CUs: the 256 x 256 kernel takes the whole rounds, and
     // the tiles of the last, partial round are cut into 64 x 64 wave tiles that spread over all SIMDs
@@ -1027,7 +1021,7 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
     const int tiles = tiles_m * tiles_n, cus = cu_count();
     int main_tiles = tiles, leftover_wt = 0;
     const bool lane_offsets_fit = static_cast<long long>(K) * 64 < (1ll << 30) && static_cast<long long>(N) * 64 < (1ll << 30);
-    if (PRISM_SGEMM5_LEFTOVER && lane_offsets_fit && tiles > cus && tiles % cus != 0 && K >= 64) {
+    if (lane_offsets_fit && tiles > cus && tiles % cus != 0 && K >= 64) {
         // Cost of the last round in units of one full round of 256 x 256 tiles: a wave tile of 64 (32)
         // is 1/4 (1/16) of a SIMD's share of a big tile and runs at about 0.87 (0.72) of its rate.
         const int left = tiles % cus, simds = 4 * cus;
@@ -1043,13 +1037,13 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
         // slices cost about 0.27 per slice on the fullest CU, so they win when they give every CU exactly
         // one, or three where one-wave tiles are no better than a full round.
         const bool one_each = left * 4 <= cus && left * 8 >= cus, three_each = left * 4 > 2 * cus && left * 4 <= 3 * cus;
-        if (PRISM_SGEMM5_LEFTOVER_SLICES && (one_each || three_each)) {
+        if (one_each || three_each) {
             main_tiles = tiles - left;
             leftover_wt = 256;
         }
         // In between, 128 x 256 halves (one workgroup to a CU) cost 0.55-0.6 of a round whatever their number;
         // one-wave tiles cost 0.35 for 68 tiles left over, as much for 73, and 0.9 for 105.
-        if (PRISM_SGEMM5_LEFTOVER_HALVES && left * 16 >= 5 * cus && left * 2 <= cus) {
+        if (left * 16 >= 5 * cus && left * 2 <= cus) {
             main_tiles = tiles - left;
             leftover_wt = 128;
         }
@@ -1093,20 +1087,13 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
 // 128 x 256 tiles (four waves of 64 x 128, K tiles of 16, 48 KiB of LDS, one workgroup per CU) when those give
 // every CU at most one tile, else on 64 x 256 tiles (four waves of 32 x 128, 40 KiB of LDS, 138 registers: three
 // workgroups per CU) when those give every CU at most three; in both cases at least half of the CUs get one.
-#ifndef PRISM_SGEMM5_HALF_TILES
-#define PRISM_SGEMM5_HALF_TILES 1
-#endif
-#ifndef PRISM_SGEMM5_QUARTER_TILES
-#define PRISM_SGEMM5_QUARTER_TILES 1
-#endif
 template <int BM, bool ALLOW_EDGES>
 bool try_half_tile_dma(int M, int N, int K, float alpha, const float* A, const float* B, float beta,
                        float* C, hipStream_t s, int* rc) {
     constexpr int BN = 256, BK = 16, WM = BM / 2, WN = 128;
-    if (!PRISM_SGEMM5_DMA || !PRISM_SGEMM5_HALF_TILES) return false;
     if (K <= 0 || !aligned16(A) || !aligned16(B) || !aligned16(C)) return false;
     const bool whole = M % BM == 0 && N % BN == 0 && K % BK == 0;
-    if (!whole && (!PRISM_SGEMM5_EDGES || !ALLOW_EDGES || N % 4 || K % 4 ||
+    if (!whole && (!ALLOW_EDGES || N % 4 || K % 4 ||
                    (static_cast<long long>(BM) + 64) * K * 4 >= (1ll << 31) ||
                    (static_cast<long long>(K) + 64) * N * 4 >= (1ll << 31)))
         return false;
@@ -1125,27 +1112,34 @@ bool try_half_tile_dma(int M, int N, int K, float alpha, const float* A, const f
     return true;
 }
 
-#ifndef PRISM_SGEMM5_SINGLE
-#define PRISM_SGEMM5_SINGLE 1
-#endif
+// ksplit: waves per tile, each with 1 / ksplit of K (1, 2, or 4 for 32 x 32 tiles); more than 1 only for whole tiles.
 template <int WT>
 bool try_single_wave(int M, int N, int K, float alpha, const float* A, const float* B, float beta, float* C,
-                     hipStream_t s, int* rc) {
+                     hipStream_t s, int* rc, int ksplit = 1) {
     constexpr int STAGES = 4;
-    if (!PRISM_SGEMM5_SINGLE) return false;
     if (K <= 0 || !aligned16(A) || !aligned16(B) || !aligned16(C)) return false;
     if (static_cast<long long>(K) * 64 >= (1ll << 30) || static_cast<long long>(N) * 64 >= (1ll << 30)) return false;
     const int tiles_m = ceil_div(M, WT), tiles_n = ceil_div(N, WT);
     const dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n);
-    if (M % WT == 0 && N % WT == 0 && K % 16 == 0 && K >= 16 * STAGES) {
-        sgemm_single_wave_kernel<WT, STAGES, false><<<grid, dim3(kWave), 0, s>>>(
-            M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
+    if (M % WT == 0 && N % WT == 0 && K % (16 * ksplit) == 0 && K >= 16 * STAGES * ksplit) {
+        if (ksplit == 4 && WT == 32)
+            sgemm_single_wave_kernel<32, STAGES, false, 4><<<grid, dim3(4 * kWave), 0, s>>>(
+                M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
+        else if (ksplit == 2)
+            sgemm_single_wave_kernel<WT, STAGES, false, 2><<<grid, dim3(2 * kWave), 0, s>>>(
+                M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
+        else if (ksplit == 1)
+            sgemm_single_wave_kernel<WT, STAGES, false><<<grid, dim3(kWave), 0, s>>>(
+                M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
+        else
+            return false;
         *rc = check_launch("sgemm_single_wave_kernel");
         return true;
     }
+    if (ksplit != 1) return false;
     // Ragged edges: rows must stay 16 B aligned; all of B plus the padding K tiles is addressed with
     // 32-bit byte offsets.
-    if (!PRISM_SGEMM5_EDGES || N % 4 || K % 4 || (static_cast<long long>(K) + 16 * STAGES) * N * 4 >= (1ll << 31)) return false;
+    if (N % 4 || K % 4 || (static_cast<long long>(K) + 16 * STAGES) * N * 4 >= (1ll << 31)) return false;
     sgemm_single_wave_kernel<WT, STAGES, true><<<grid, dim3(kWave), 0, s>>>(
         M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
     *rc = check_launch("sgemm_single_wave_kernel (edges)");
@@ -1210,14 +1204,22 @@ int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, 
                 // (N or K not a multiple of 4, unaligned operands) goes to the general kernel.
                 const long long simds = 4ll * cu_count();
                 const long long tiles64 = static_cast<long long>(ceil_div(M, 64)) * ceil_div(N, 64);
-                if (tiles64 <= PRISM_SGEMM5_SINGLE_ROUNDS * simds) {
+                if (tiles64 <= simds) {
+                    // Far fewer 32 x 32 tiles than SIMDs: cut K inside the workgroup (2 or 4 waves per tile) as
+                    // long as every wave keeps at least 256 of K and at most half of the SIMDs end up with a
+                    // wave: 32 x 32 wave tiles move 1 B from L2 per 8 flop, and with a wave on every SIMD that
+                    // traffic, not the matrix pipe, is the limit (128 x 4096 x 4096: 72 TFLOP/s with 512 waves,
+                    // 65 with 1024). 512^3: 24 -> 35 TFLOP/s, 256 x 256 x 4096: 29 (rocBLAS 13 and 23).
+                    const long long tiles32 = static_cast<long long>(ceil_div(M, 32)) * ceil_div(N, 32);
+                    if (tiles32 * 8 <= simds && K >= 4 * 256 && try_single_wave<32>(M, N, K, alpha, A, B, beta, C, s, &rc, 4)) return rc;
+                    if (tiles32 * 4 <= simds && K >= 2 * 256 && try_single_wave<32>(M, N, K, alpha, A, B, beta, C, s, &rc, 2)) return rc;
                     if (tiles64 < simds && try_single_wave<32>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
                     if (try_single_wave<64>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
                 }
                 if (try_half_tile_dma<128, true>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
-                if (PRISM_SGEMM5_QUARTER_TILES && try_half_tile_dma<64, true>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
+                if (try_half_tile_dma<64, true>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
             }
-            return run_wave_tile<PRISM_SGEMM5_CFG>(M, N, K, alpha, A, B, beta, C, s);
+            return run_wave_tile<128, 128, 16, 64, 64>(M, N, K, alpha, A, B, beta, C, s);  // BM, BN, BK, WM, WN
     }
     return fail(1, "prism_sgemm: unknown kernel number %d", variant);
 }

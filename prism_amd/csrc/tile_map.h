@@ -21,14 +21,8 @@
 namespace prism {
 
 constexpr int kXcds = 8;
-#ifndef PRISM_TILE_GROUP_M
-#define PRISM_TILE_GROUP_M 8
-#endif
-constexpr int kGroupM = PRISM_TILE_GROUP_M;  // rows of tiles in one XCD's patch
-#ifndef PRISM_TILE_SUPER
-#define PRISM_TILE_SUPER 16
-#endif
-constexpr int kSuper = PRISM_TILE_SUPER;  // super-block edge, in tiles
+constexpr int kGroupM = 8;  // rows of tiles in one XCD's patch
+constexpr int kSuper = 16;  // super-block edge, in tiles
 
 __host__ __device__ __forceinline__ void xcd_tile_coords(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
     // Which super-block: rows of super-blocks hold kSuper * tiles_n tiles each (the last one fewer).

@@ -1,7 +1,7 @@
 """Checks on the machine code hipcc generates for the two GEMM sources (CPU only: cross-compiles to assembly).
 
 The direct-to-LDS loads and some matrix instructions are inline assembly, which the compiler does not look
-into. Four things it would otherwise take care of are therefore checked on the generated text:
+into. Five things it would otherwise take care of are therefore checked on the generated text:
 
 * M0 carries a load's LDS destination. Every `s_mov_b32 m0` in these files is one of ours, so the number of M0
   mentions must equal the number of direct loads, and walking back from every direct load the first M0 write
@@ -14,6 +14,10 @@ into. Four things it would otherwise take care of are therefore checked on the g
   operand; for the matrix instructions issued from inline assembly nothing inserts them. No matrix instruction
   may read a register that a vector ALU instruction wrote within the two instructions before it (`s_nop n`
   counts as n + 1).
+* The result of a matrix instruction issued from inline assembly is not tracked by the compiler either. No
+  instruction other than a matrix instruction may read an accumulation register (`a`) within 64 clocks of the
+  in-place matrix instruction that last wrote it, counting 16 clocks per matrix instruction in between,
+  n + 1 per `s_nop n` and 1 per other instruction (the write-back waits with four `s_nop 15`).
 * The kernels whose K loops keep all 256 accumulation registers pinned (`gemm_bf16_early_kernel` for whole
   tiles, `sgemm_wave_tile_dma_kernel`) must not spill: a spill there means the compiler has started to move
   accumulators, which with matrix instructions in inline assembly is also a correctness hazard.
@@ -146,3 +150,52 @@ def test_pinned_accumulator_kernels_do_not_spill(assembly):
                 size = re.search(r"\.amdhsa_private_segment_fixed_size\s+(\d+)", m.group(2))
                 assert size and int(size.group(1)) == 0, f"{m.group(1)} uses {size.group(1) if size else '?'} bytes of scratch"
         assert found >= 2, f"no kernel matching {pattern} in {source}"
+
+
+def accumulation_registers(text):
+    regs = set()
+    for m in re.finditer(r"\ba\[(\d+):(\d+)\]", text):
+        regs |= set(range(int(m.group(1)), int(m.group(2)) + 1))
+    for m in re.finditer(r"(?<![\w\[])a(\d+)\b", text):
+        regs.add(int(m.group(1)))
+    return regs
+
+
+def test_no_accumulator_is_read_too_soon_after_an_in_place_matrix_instruction(assembly):
+    """In gemm_bf16_early_kernel the accumulating v_mfma_f32_16x16x32_bf16 comes from inline assembly (between
+    the compiler's ASMSTART / ASMEND marks) with its destination as addend. Reads and copies of its result by
+    anything but another matrix instruction (the write-back's stores, a compiler-made copy) must keep their
+    distance; results of matrix instructions the compiler issued itself are its own business."""
+    reads, from_asm = 0, 0
+    last_write = {}  # accumulation register -> clock of the inline-assembly matrix instruction that wrote it
+    clock, kernel, in_asm = 0, None, False
+    for raw in assembly["gemm_bf16.hip"].splitlines():
+        if "#ASMSTART" in raw:
+            in_asm = True
+        elif "#ASMEND" in raw:
+            in_asm = False
+        i = raw.split(";")[0].strip()
+        if not i or i.startswith((".", "#")):
+            continue
+        if i.endswith(":"):
+            if i.startswith("_Z"):
+                kernel, clock, last_write = i[:-1], 0, {}
+            continue
+        if kernel is None or "gemm_bf16_early_kernel" not in kernel:
+            continue
+        if i.startswith("v_mfma_"):
+            clock += 16
+            dest = i.split(None, 1)[1].split(",")[0]
+            for r in accumulation_registers(dest):
+                if in_asm:
+                    last_write[r] = clock
+                    from_asm += 1
+                else:
+                    last_write.pop(r, None)
+            continue
+        clock += int(i.split()[1]) + 1 if i.startswith("s_nop") else 1
+        used = accumulation_registers(i.split(None, 1)[1]) if " " in i else set()
+        for r in used:
+            reads += 1
+            assert clock - last_write.get(r, -10**9) >= 64, f"{kernel}: `{i}` reads a{r} {clock - last_write[r]} clocks after its matrix instruction"
+    assert reads >= 512 and from_asm >= 512  # two instances, 256 accumulation registers each, at least

@@ -115,20 +115,6 @@ def test_ragged_shapes_with_aligned_rows(prism, oracle, shape):
     assert np.all(np.abs(c - ref) <= 2.0**-8 * np.abs(ref) + REL * np.abs(ref).max())
 
 
-@pytest.mark.parametrize("kernel", ["staged32", "staged16"])
-@pytest.mark.parametrize("shape", [(3072, 3072, 384), (3072, 3328, 512), (4352, 4352, 640), (3000, 3080, 392)])
-def test_alternative_whole_tile_pipelines(prism, oracle, shape, kernel, monkeypatch):
-    """PRISM_BF16_KERNEL selects the pipeline for problems of whole 256 x 256 x 64 tiles: one of the two
-    register-staged ones (32x32x16 or 16x16x32 instructions) instead of the default, the direct-to-LDS pipeline
-    with early fragment reads, which every other test runs. Every element is checked; the third shape also has
-    a partial last round, the fourth is ragged (the staged kernels' edge variants)."""
-    monkeypatch.setenv("PRISM_BF16_KERNEL", kernel)
-    M, N, K = shape
-    A16, B16 = oracle.gen_gemm_bf16(M, N, K, seed=K + 2 * M)
-    D = prism.gemm_bf16(dev16(A16), dev16(B16))
-    check_f32(oracle, host(D), A16, B16)
-
-
 def test_fixture(prism, golden, oracle):
     A16, B16 = golden["bf16_A"], golden["bf16_B"]
     D = host(prism.gemm_bf16(dev16(A16), dev16(B16)))

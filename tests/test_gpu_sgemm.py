@@ -178,11 +178,15 @@ def test_wave_tile_whole_tile_path(prism, oracle, shape):
 
 
 @pytest.mark.parametrize("shape", [(512, 512, 64), (1024, 1024, 80), (1024, 1024, 96), (1024, 1024, 112), (1024, 512, 256),
-                                   (2048, 2048, 128), (128, 4096, 256), (64, 64, 2048), (96, 160, 64)])
+                                   (2048, 2048, 128), (128, 4096, 256), (64, 64, 2048), (96, 160, 64),
+                                   (128, 2048, 512), (128, 2048, 544), (64, 1024, 1024), (128, 128, 4096), (512, 512, 1088),
+                                   (64, 4096, 2048), (32, 32, 1024), (32, 64, 1216)])
 def test_wave_tile_one_wave_per_tile_path(prism, oracle, shape):
     """Problems with at most one 64 x 64 tile per SIMD take kernel 5's one-wave-per-tile path (32 x 32
-    tiles below that, 64 x 64 at exactly that); K covers every residue of the 4-stage ring. Every element is
-    checked, with and without reading C."""
+    tiles below that, 64 x 64 at exactly that); K covers every residue of the 4-stage ring. The second row
+    of shapes has at most a quarter as many 32 x 32 tiles as there are SIMDs and a long K: two or four waves share a tile, each with a
+    part of K (every residue of the ring again), and add up in LDS. Every element is checked, with and
+    without reading C, and a second run gives the same bits."""
     M, N, K = shape
     A, B, Cm = oracle.gen_sgemm(M, N, K, seed=K + N)
     got = run(prism, 5, -0.75, A, B, 2.0, Cm)
@@ -190,6 +194,7 @@ def test_wave_tile_one_wave_per_tile_path(prism, oracle, shape):
     poison = np.full((M, N), np.nan, dtype=np.float32)
     got0 = run(prism, 5, 1.0, A, B, 0.0, poison)
     assert np.max(np.abs(got0 - oracle.np_sgemm_f64(1.0, A, B, 0.0))) <= oracle.sgemm_tolerance(K, A, B)
+    assert np.array_equal(run(prism, 5, -0.75, A, B, 2.0, Cm), got)
 
 
 @pytest.mark.parametrize("shape", [(4352, 4352, 64), (4096, 5120, 80), (5120, 5120, 80), (5120, 5120, 48), (4608, 4608, 64),
