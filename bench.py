@@ -230,6 +230,34 @@ def bench_add_m(prism, n, steps, warmup, gate=True):
                          "frac": gbps / PEAK["hbm_GBps"], "traffic": measured_traffic("add_m", n)}}
 
 
+# ------------------------------------------------------------ calibration --
+
+CALIBRATION_KINDS = {0: "copy_packet_per_lane", 1: "copy_scan_tile_shape", 2: "read_only", 3: "write_only"}
+
+
+def bench_calibration(steps, warmup):
+    """What the memory system gives kernels that only move bytes (prism_calibrate_stream): a 1 GiB copy in
+    add_m's shape (the counter calibration) and, at the scan's size of 4 GiB per buffer, the copy in add_m's
+    shape, the copy in the scan's tile shape, a read-only and a write-only stream."""
+    import torch
+    lib, st = _capi()
+    n = 1 << 30
+    x = torch.randint(-1000, 1001, (n,), dtype=torch.int32, device="cuda")
+    y = torch.empty_like(x)
+    out = {}
+    one_gib = 1 << 30
+    ms = time_steps(lambda: lib.prism_calibrate_stream(0, x.data_ptr(), y.data_ptr(), one_gib, st), steps, warmup)
+    if not torch.equal(x[: one_gib // 4], y[: one_gib // 4]):
+        raise RuntimeError("calibration copy is wrong")
+    out["copy_1GiB"] = {"kernel": "calibrate_copy_packet_kernel", "bytes_read": one_gib, "bytes_written": one_gib,
+                        "ms": ms, "GBps": 2.0 * one_gib / ms / 1e6}
+    for kind, name in CALIBRATION_KINDS.items():
+        ms = time_steps(lambda: lib.prism_calibrate_stream(kind, x.data_ptr(), y.data_ptr(), 4 * n, st), steps, warmup)
+        moved = (2 if kind < 2 else 1) * 4.0 * n
+        out[name] = {"ms": ms, "GBps": moved / ms / 1e6, "frac_of_peak": moved / ms / 1e6 / PEAK["hbm_GBps"]}
+    return out
+
+
 # -------------------------------------------------------------- bf16 gemm --
 
 def bench_gemm_bf16(prism, n, steps, warmup, gate=True):
@@ -314,6 +342,73 @@ def cpu_baseline_add_m(n=1 << 24):
             "sample": f"oracle_add_m on n=2^24, {dt * 1e3:.1f} ms", "numpy_GBps": 8.0 * n / dt_np / 1e9}
 
 
+# ------------------------------------------------- HBM-side traffic table --
+
+TRAFFIC_KERNELS = [  # (workload, size, substring of the kernel name, threads in the grid)
+    ("sgemm", 8192, "sgemm_wave_tile_dma_kernel", 1024 * 256),
+    ("scan", 1 << 30, "scan_lookback_kernel", (1 << 30) // 65536 * 1024),
+    ("gemm_bf16", 8192, "gemm_bf16_early_kernel", 1024 * 256),
+    ("add_m", 1 << 24, "add_m_vec4_kernel", (1 << 24) // 4),
+    ("add_m", 1 << 28, "add_m_vec4_kernel", (1 << 28) // 4),
+]
+
+
+def write_traffic_table(pmc_dir: str) -> int:
+    """Summarises four `rocprofv3 --pmc` runs of this script into profiles/hbm_traffic.md, the table
+    measured_traffic() reads. Expected in pmc_dir (rocprofv3 -d pmc_dir -o NAME --output-format csv):
+    bench_FETCH_SIZE, bench_WRITE_SIZE (`bench.py --no-configs --no-cpu-baseline --steps 3 --warmup 1`) and
+    calib_FETCH_SIZE, calib_WRITE_SIZE (`bench.py --workload calibrate --steps 3 --warmup 1`)."""
+    import csv
+
+    def readings(name, counter, match, grid=None):
+        vals = []
+        with open(os.path.join(pmc_dir, f"{name}_{counter}_counter_collection.csv"), newline="") as f:
+            for r in csv.DictReader(f):
+                if r["Counter_Name"] == counter and match in r["Kernel_Name"] and (grid is None or int(r["Grid_Size"]) == grid):
+                    vals.append(float(r["Counter_Value"]))
+        return vals
+
+    scale = {}
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        v = readings("calib", counter, "calibrate_copy_packet_kernel", (1 << 30) // 16)
+        if not v:
+            print(f"no copy kernel in calib_{counter}", file=sys.stderr)
+            return 1
+        scale[counter] = (1 << 20) / (sum(v) / len(v))  # the copy moves 1 GiB = 2^20 KiB each way
+    lines = ["# HBM-side traffic per launch (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)", "",
+             "Written by `python bench.py --traffic-summary $R/gpurun_out/pmc_traffic` from four counter runs (from /tmp with",
+             "TMPDIR=/tmp on the GPU box, R = repo root, C = FETCH_SIZE, then WRITE_SIZE; each run its own process):", "",
+             "    rocprofv3 --pmc $C --kernel-trace -d $R/gpurun_out/pmc_traffic -o bench_$C --output-format csv -- \\",
+             "        python3 $R/bench.py --steps 3 --warmup 1 --no-configs --no-cpu-baseline",
+             "    rocprofv3 --pmc $C --kernel-trace -d $R/gpurun_out/pmc_traffic -o calib_$C --output-format csv -- \\",
+             "        python3 $R/bench.py --workload calibrate --steps 3 --warmup 1", "",
+             "`bench.py` reads the table back for `roofline.traffic`. A row counts only while the hash of its kernel source",
+             "(first 16 hex digits of the SHA-256 of `prism_amd/csrc/<file>`) is the one in the tree; otherwise the bench line",
+             "says `null`. The counters sit at the L2's memory side, so they include what the 256 MiB memory-side cache serves.",
+             "", f"Scale factors from the 1 GiB copy (calibrate_copy_packet_kernel): FETCH_SIZE x {scale['FETCH_SIZE']:.3f}, WRITE_SIZE x {scale['WRITE_SIZE']:.3f}"
+             " (KiB per dispatch -> KiB moved).", "",
+             "| workload | size | bytes read | bytes written | source hash | launches averaged | algorithmic bytes | ratio |",
+             "|---|---:|---:|---:|---|---:|---:|---:|"]
+    algorithmic = {("sgemm", 8192): 4 * 4 * 8192 ** 2, ("scan", 1 << 30): 8 << 30, ("gemm_bf16", 8192): (2 * 2 + 4) * 8192 ** 2,
+                   ("add_m", 1 << 24): 8 << 24, ("add_m", 1 << 28): 8 << 28}
+    for workload, size, match, grid in TRAFFIC_KERNELS:
+        f, w = readings("bench", "FETCH_SIZE", match, grid), readings("bench", "WRITE_SIZE", match, grid)
+        if not f or not w:
+            print(f"no readings for {workload} {size}", file=sys.stderr)
+            continue
+        rd = int(sum(f) / len(f) * scale["FETCH_SIZE"] * 1024)
+        wr = int(sum(w) / len(w) * scale["WRITE_SIZE"] * 1024)
+        alg = algorithmic[(workload, size)]
+        lines.append(f"| {workload} | {size} | {rd} | {wr} | {source_hash(workload)} | {min(len(f), len(w))} | {alg} | {(rd + wr) / alg:.3f} |")
+    lines += ["", "The streaming kernels move their algorithmic bytes and nothing else (the scan's status words and polls are",
+              "0.1 %). The GEMMs are compute-bound; their HBM-side reads are L2 misses of re-used A / B panels: with 256 x 256",
+              "tiles and an 8 x 4 tile patch per XCD, 12 of the 64 panel reads of a patch miss, which is what an XCD's 32 CUs",
+              "working in step can reach at best with that patch shape."]
+    TRAFFIC_FILE.write_text("\n".join(lines) + "\n")
+    print("\n".join(lines))
+    return 0
+
+
 # ------------------------------------------------------------------- main --
 
 def main() -> int:
@@ -325,7 +420,11 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-configs", action="store_true",
                     help="skip the table of the other BASELINE configurations (also.configs)")
+    ap.add_argument("--traffic-summary", metavar="DIR", default=None,
+                    help="no GPU work: summarise the rocprofv3 --pmc outputs in DIR into profiles/hbm_traffic.md")
     args = ap.parse_args()
+    if args.traffic_summary:
+        return write_traffic_table(args.traffic_summary)
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no multi-GPU part); run with --gpus 1",
               file=sys.stderr)
@@ -342,14 +441,10 @@ def main() -> int:
     want = lambda w: args.workload in ("all", w)
 
     if args.workload == "calibrate":
-        # A plain copy of known size (1 GiB read + 1 GiB written per launch) for scaling the
-        # FETCH_SIZE / WRITE_SIZE counters of a `rocprofv3 --pmc` run of this same script.
-        n = 1 << 28
-        x = torch.randint(-1000, 1001, (n,), dtype=torch.int32, device="cuda")
-        y = torch.empty_like(x)
-        ms = time_steps(lambda: y.copy_(x), K, W)
-        print(json.dumps({"workload": "calibrate", "kernel": "torch copy_ int32", "bytes_read": 4 * n,
-                          "bytes_written": 4 * n, "ms_per_step": ms, "GBps": 8.0 * n / ms / 1e6}), flush=True)
+        # Plain streaming kernels of known size (prism_calibrate_stream): the copy of 1 GiB (kind 0) is what the
+        # FETCH_SIZE / WRITE_SIZE counters of a `rocprofv3 --pmc` run of this script are scaled by; all four kinds
+        # at 4 GiB are the ceiling the streaming workloads are compared with.
+        print(json.dumps({"workload": "calibrate", **bench_calibration(K, W)}), flush=True)
         return 0
 
     res = {}
@@ -366,6 +461,9 @@ def main() -> int:
         res["add_m"] = bench_add_m(prism, 1 << 24, max(K, 50), W)
         log("add_m 2^24:", res["add_m"])
 
+    if args.workload == "all" or args.workload in ("scan", "add_m"):
+        res["hbm_calibration"] = bench_calibration(K, W)
+        log("streaming calibration:", res["hbm_calibration"])
     if want("add_m"):
         res["add_m_2p28"] = bench_add_m(prism, 1 << 28, K, W)
         res["add_m_2p28"]["note"] = "x and y are 2 GiB together: beyond the 256 MiB memory-side cache"

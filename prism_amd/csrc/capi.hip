@@ -51,6 +51,10 @@ int prism_tile_coords(int workgroup_id, int tiles_m, int tiles_n, int* tile_m, i
     return 0;
 }
 
+int prism_calibrate_stream(int kind, const void* in, void* out, size_t bytes, void* stream) {
+    return launch_calibrate_stream(kind, in, out, bytes, static_cast<hipStream_t>(stream));
+}
+
 int prism_add_m(const int32_t* x, int32_t* y, int32_t m, size_t n, void* stream) {
     return launch_add_m(x, y, m, n, static_cast<hipStream_t>(stream));
 }

@@ -68,6 +68,7 @@ int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws
                 long long spin_limit, hipStream_t s);
 int scan_status(void* ws, size_t ws_bytes, hipStream_t s);
 int launch_scan_static(const uint32_t* in, uint32_t* out, size_t n, hipStream_t s);
+int launch_calibrate_stream(int kind, const void* in, void* out, size_t bytes, hipStream_t s);
 int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, const float* B,
                  float beta, float* C, hipStream_t s);
 int launch_gemm_bf16(int M, int N, int K, const uint16_t* A, const uint16_t* B, float* D_f32,
