@@ -274,7 +274,7 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
-    const int wave = tid / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // uniform: what only wave 0 does stays in scalar registers
     const uint32_t tiles = gridDim.x;
 
     uint32_t tile = blockIdx.x;
@@ -325,9 +325,9 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
     u32x4 hdr = {0u, 0u, 0u, 0u};
     if (wave == 0) hdr = *reinterpret_cast<const u32x4*>(header + kHdrCalls);
 
-    // Lane-local inclusive sums of each packet, then the packet totals are
-    // scanned across the wave; rows are chained by the wave-uniform carry.
-    uint32_t offset[VPT];
+    // Lane-local inclusive sums of each packet, then the packet totals are scanned across the wave; rows
+    // are chained by the wave-uniform carry. Afterwards v[j] holds the running sums within this wave's
+    // 4 * VPT * 64 elements (what comes before the wave is added at the write-back).
     uint32_t carry = Op::identity;
 #pragma unroll
     for (int j = 0; j < VPT; ++j) {
@@ -335,7 +335,9 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
         v[j].z = Op::apply(v[j].z, v[j].y);
         v[j].w = Op::apply(v[j].w, v[j].z);
         const uint32_t inclusive = wave_inclusive_scan_op<Op>(v[j].w);
-        offset[j] = Op::apply(carry, wave_exclusive_from_inclusive<Op>(inclusive, v[j].w, lane));
+        const uint32_t before = Op::apply(carry, wave_exclusive_from_inclusive<Op>(inclusive, v[j].w, lane));
+#pragma unroll
+        for (int c = 0; c < 4; ++c) v[j][c] = Op::apply(v[j][c], before);
         carry = Op::apply(carry, wave_last_lane(inclusive));
     }
     if (lane == 0) s_wave_total[wave] = carry;
@@ -379,29 +381,39 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
     __syncthreads();
     const uint32_t base_sum = Op::apply(s_tile_prefix, wave_prefix);
 
+    // Exclusive sums: element c of a packet gets the running sum of element c - 1; element 0 that of the
+    // previous lane's last element (wave_shr:1), lane 0 that of the row before (0 for the first row).
+    uint32_t row_before = 0u;
+    auto shifted = [&](int j) {
+        const uint32_t from_lane_below = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(
+            static_cast<int>(row_before), static_cast<int>(v[j].w), 0x138 /* wave_shr:1 */, 0xf, 0xf, false));
+        row_before = wave_last_lane(v[j].w);
+        return u32x4{from_lane_below, v[j].x, v[j].y, v[j].z};
+    };
     if (full) {
 #pragma unroll
         for (int j = 0; j < VPT; ++j) {
-            // v[j] holds the running sums inside the packet; shifted by one element they are the exclusive ones.
-            const u32x4 sums = EXCLUSIVE ? u32x4{0u, v[j].x, v[j].y, v[j].z} : v[j];
-            const uint32_t before = Op::apply(offset[j], base_sum);
             u32x4 r;
-            if constexpr (Op::kIsSum) {
-                r = sums + before;
+            if constexpr (EXCLUSIVE) {
+                r = shifted(j) + base_sum;
+            } else if constexpr (Op::kIsSum) {
+                r = v[j] + base_sum;
             } else {
 #pragma unroll
-                for (int c = 0; c < 4; ++c) r[c] = Op::apply(sums[c], before);
+                for (int c = 0; c < 4; ++c) r[c] = Op::apply(v[j][c], base_sum);
             }
             stream_store(reinterpret_cast<u32x4*>(out + lane_base + j * ROW_ELEMS), r);
         }
     } else {
 #pragma unroll
         for (int j = 0; j < VPT; ++j) {
-            const uint32_t add = Op::apply(offset[j], base_sum);
+            u32x4 r;
+            if constexpr (EXCLUSIVE) r = shifted(j);
+            else r = v[j];
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const size_t i = lane_base + j * ROW_ELEMS + c;
-                if (i < n) out[i] = Op::apply(EXCLUSIVE ? (c ? v[j][c - 1] : 0u) : v[j][c], add);
+                if (i < n) out[i] = Op::apply(r[c], base_sum);
             }
         }
     }
