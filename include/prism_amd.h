@@ -197,6 +197,20 @@ int prism_scan_min_i32(const int32_t* in, int32_t* out, size_t n, void* workspac
                        size_t workspace_bytes, void* stream);
 
 /*
+ * Segmented inclusive prefix sum: out[i] = the sum of in[j] over j from the last
+ * element at or before i whose byte in `heads` is non-zero (element 0 always
+ * starts a segment) up to i, modulo 2^32. The same single pass with the sum of
+ * scan_kernel's stages (examples/scan.py:106-227; the combination of records in
+ * lookback_to_prev_blocks :60-85) replaced by the associative, non-commutative
+ * operator on (head seen, sum) pairs; a tile's walk back ends at the nearest
+ * tile that holds a head. Workspace, aliasing of in and out, ordering and the
+ * status check as for prism_scan_i32; heads must not overlap out. The reference
+ * scans one segment only.
+ */
+int prism_segmented_scan_i32(const int32_t* in, const uint8_t* heads, int32_t* out, size_t n,
+                             void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * The reference launcher's own shape: in-place on x, default stream, returns
  * the device pointer that holds the result (x) or NULL on failure.
  * Replaces scan_gpu::launch_scan (evals/4090_scan/main.cu:68-86). Like the

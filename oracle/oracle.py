@@ -41,6 +41,10 @@ def lib() -> C.CDLL:
         L.oracle_scan_cpu.restype = None
         L.oracle_scan_exclusive_cpu.argtypes = [sz, vp, vp]
         L.oracle_scan_exclusive_cpu.restype = None
+        L.oracle_segmented_scan_cpu.argtypes = [sz, vp, vp, vp]
+        L.oracle_segmented_scan_cpu.restype = None
+        L.oracle_scan_i64_cpu.argtypes = [sz, vp, vp]
+        L.oracle_scan_i64_cpu.restype = None
         L.oracle_scan_max_cpu.argtypes = [sz, vp, vp]
         L.oracle_scan_max_cpu.restype = None
         L.oracle_scan_lookback.argtypes = [sz, vp, C.c_uint]
@@ -112,6 +116,49 @@ def scan_max_cpu(x: np.ndarray) -> np.ndarray:
     out = np.empty_like(xi)
     lib().oracle_scan_max_cpu(xi.size, _p(xi), _p(out))
     return out
+
+
+def segmented_scan_cpu(x: np.ndarray, heads: np.ndarray) -> np.ndarray:
+    """Serial uint32 inclusive scan that starts again at every element whose head flag is non-zero."""
+    dt = x.dtype
+    xu = _c(x, dt).view(np.uint32)
+    h = _c(heads, np.uint8)
+    assert h.size == xu.size
+    out = np.empty_like(xu)
+    lib().oracle_segmented_scan_cpu(xu.size, _p(xu), _p(h), _p(out))
+    return out.view(dt)
+
+
+def np_segmented_scan(x: np.ndarray, heads: np.ndarray) -> np.ndarray:
+    """The same through one global cumulative sum: out[i] = S[i] - S[start(i) - 1] modulo 2^32, where start(i)
+    is the last head at or before i."""
+    xu = x.view(np.uint32).astype(np.uint64)
+    S = np.cumsum(xu)  # exact in 64 bits for fewer than 2^32 elements
+    idx = np.arange(x.size)
+    h = np.asarray(heads) != 0
+    if x.size:
+        h = h.copy()
+        h[0] = True
+    start = np.maximum.accumulate(np.where(h, idx, 0))
+    before = np.where(start > 0, S[np.maximum(start - 1, 0)], 0)
+    return ((S - before) % np.uint64(2**32)).astype(np.uint32).view(x.dtype)
+
+
+def scan_i64_cpu(x: np.ndarray) -> np.ndarray:
+    """Serial inclusive scan of 64-bit elements modulo 2^64."""
+    dt = x.dtype
+    xu = _c(x, dt).view(np.uint64)
+    out = np.empty_like(xu)
+    lib().oracle_scan_i64_cpu(xu.size, _p(xu), _p(out))
+    return out.view(dt)
+
+
+def gen_heads(n: int, mean_segment: float, seed: int = 0) -> np.ndarray:
+    """Head flags (uint8, values 0 / 1 / 255) with segments of the given mean length."""
+    rng = np.random.default_rng(seed)
+    h = (rng.random(n) < 1.0 / mean_segment).astype(np.uint8)
+    h[rng.random(n) < 0.5] *= np.uint8(255)  # any non-zero byte is a head
+    return h
 
 
 def scan_lookback(x: np.ndarray, stall_every: int = 0) -> np.ndarray:

@@ -17,6 +17,9 @@
  *   oracle_scan_exclusive_cpu  closed forms (all-ones -> i, wrap), inclusive[i] - x[i], shifted numpy.cumsum
  *   oracle_scan_max_cpu     closed forms (rising -> itself, falling -> first element, INT32_MIN / INT32_MAX),
  *                           numpy.maximum.accumulate, monotone and out[i] >= x[i] with equality where out steps
+ *   oracle_segmented_scan_cpu  no heads -> oracle_scan_cpu; every element a head -> the input; hand-computed
+ *                           case with wrap; per-segment numpy.cumsum; the closed form through one global cumsum
+ *   oracle_scan_i64_cpu     closed forms (all-ones -> i+1, wrap at 2^63), numpy.cumsum(int64)
  *   oracle_scan_lookback    equality with oracle_scan_cpu on the reference's own test sizes
  *                           and distribution; tail beyond the last full block left untouched
  *   oracle_sgemm_fma        brute-force exact rational/fp64 check on small integer-valued
@@ -47,6 +50,27 @@ void oracle_add_m(const int32_t* x, int32_t* y, int32_t m, size_t n) {
  * (evals/4090_scan/scan_harness.cuh:30-36): serial uint32 accumulator. */
 void oracle_scan_cpu(size_t n, const uint32_t* x, uint32_t* out) {
     uint32_t accumulator = 0;
+    for (size_t i = 0; i < n; i++) {
+        accumulator = accumulator + x[i];
+        out[i] = accumulator;
+    }
+}
+
+/* Segmented form of the loop above: the accumulator starts again at every element whose head flag is
+ * non-zero (and at element 0). No reference counterpart (examples/scan.py scans one segment); it is the
+ * serial definition the segmented entry point of the library is checked against. */
+void oracle_segmented_scan_cpu(size_t n, const uint32_t* x, const uint8_t* heads, uint32_t* out) {
+    uint32_t accumulator = 0;
+    for (size_t i = 0; i < n; i++) {
+        if (heads[i]) accumulator = 0;
+        accumulator = accumulator + x[i];
+        out[i] = accumulator;
+    }
+}
+
+/* The loop of scan_cpu (evals/4090_scan/scan_harness.cuh:30-36) on 64-bit elements, modulo 2^64. */
+void oracle_scan_i64_cpu(size_t n, const uint64_t* x, uint64_t* out) {
+    uint64_t accumulator = 0;
     for (size_t i = 0; i < n; i++) {
         accumulator = accumulator + x[i];
         out[i] = accumulator;

@@ -21,6 +21,7 @@ from .ops import (  # noqa: F401
     scan,
     scan_status,
     scan_workspace_init,
+    segmented_scan,
     sgemm,
     tile_coords,
 )

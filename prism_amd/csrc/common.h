@@ -67,6 +67,8 @@ int scan_workspace_init(void* ws, size_t ws_bytes, hipStream_t s);
 int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, unsigned flags,
                 long long spin_limit, hipStream_t s);
 int scan_status(void* ws, size_t ws_bytes, hipStream_t s);
+int launch_segmented_scan(const uint32_t* in, const uint8_t* heads, uint32_t* out, size_t n, void* ws, size_t ws_bytes,
+                          hipStream_t s);
 int launch_scan_static(const uint32_t* in, uint32_t* out, size_t n, hipStream_t s);
 int launch_calibrate_stream(int kind, const void* in, void* out, size_t bytes, hipStream_t s);
 int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, const float* B,

@@ -32,6 +32,20 @@ __device__ __forceinline__ void direct_load16(const char* base, uint32_t lane_of
 #pragma clang diagnostic pop
 }
 
+// The 4-byte form: lane l reads base + lane_offset(l) and lands at lds_dst + 4 l (256 B of contiguous LDS
+// per instruction).
+__device__ __forceinline__ void direct_load4(const char* base, uint32_t lane_offset, const void* lds_dst) {
+    const uint32_t lds_addr = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+        (const __attribute__((address_space(3))) void*)lds_dst));
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+                 :
+                 : "v"(lane_offset), "s"(base), "s"(lds_addr)
+                 : "memory", "m0");
+#pragma clang diagnostic pop
+}
+
 // The same load through a buffer descriptor: lane l reads descriptor base + lane_offset(l) +
 // scalar_offset. Every dword whose offset (lane + scalar part) is at or beyond the descriptor's
 // extent arrives as zero, which is how ragged matrix edges are filled: the extent ends with the

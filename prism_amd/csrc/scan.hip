@@ -74,6 +74,7 @@
 #include <type_traits>
 
 #include "common.h"
+#include "direct_load.h"
 
 namespace prism {
 namespace {
@@ -86,6 +87,7 @@ constexpr size_t kHeaderBytes = 256;
 enum : int {                // header fields, as indices of 32-bit words
     kHdrTicket = 0,         // ticket counter (ticket order only); 0 between calls
     kHdrReport = 2,         // look-back time-out report: tile number + 1, sticky until scan_status() reads it
+    kHdrDone = 3,           // tiles that have finished (segmented scan only); 0 between calls
     kHdrCalls = 4,          // calls completed on this workspace; its low bit is the parity of the next call
     kHdrDirty0 = 5,         // tiles whose parity-0 words may be non-zero
     kHdrDirty1 = 6,         // same for parity 1
@@ -203,6 +205,48 @@ __device__ __forceinline__ uint32_t wave_exclusive_from_inclusive(uint32_t inclu
     }
 }
 
+// Tile number of a workgroup in workgroup-id order. Consecutive workgroup ids go to the 8 XCDs in turn, and
+// the XCDs drift apart, so in plain id order half of all tiles start before their predecessor and wait
+// longer for it. Chunks of kChunk consecutive tiles are given to workgroups of one XCD instead (every 8th
+// id), which start in order; only chunk boundaries cross XCDs. A tile's predecessors then have ids at most
+// 8 * kChunk above its own, far fewer than the workgroups resident at once, so the lowest unfinished tile
+// is still always running.
+__device__ __forceinline__ uint32_t tile_of_workgroup(uint32_t workgroup, uint32_t tiles) {
+    constexpr uint32_t G = kChunk, SPAN = 8 * G;
+    const uint32_t whole = (tiles / SPAN) * SPAN;
+    if (workgroup >= whole) return workgroup;
+    const uint32_t xcd = workgroup % 8, j = workgroup / 8;
+    return (j / G) * SPAN + xcd * G + (j % G);
+}
+
+// What wave 0 of every tile does for the workspace once its own status word is final. hdr = the header
+// words {calls, dirty0, dirty1, -} as read at the start of the kernel.
+__device__ __forceinline__ void clear_other_parity(u64* status, u32x4 hdr, uint32_t tile, uint32_t tiles, int lane) {
+    // Tile t clears words t, t + tiles, ... below the other parity's mark.
+    const uint32_t parity = hdr.x & 1u, dirty_other = parity ? hdr.y : hdr.z;
+    for (size_t w = tile + static_cast<size_t>(lane) * tiles; w < dirty_other; w += static_cast<size_t>(kWave) * tiles)
+        __hip_atomic_store(&status[2 * w + (parity ^ 1u)], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Closes a call (one lane of one tile): counters back to zero, marks set, call counter advanced. Only when
+// every tile of the call has read the header.
+__device__ __forceinline__ void close_call(uint32_t* header, u32x4 hdr, uint32_t tiles) {
+    const uint32_t calls = hdr.x, parity = calls & 1u;
+    __hip_atomic_store(&header[kHdrTicket], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&header[kHdrDone], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&header[kHdrDirty0 + parity], tiles, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&header[kHdrDirty0 + (parity ^ 1u)], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&header[kHdrCalls], calls + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ void finish_status_protocol(uint32_t* header, u64* status, u32x4 hdr, uint32_t tile,
+                                                       uint32_t tiles, int lane) {
+    clear_other_parity(status, hdr, tile, tiles, lane);
+    // The last tile closes the call: every earlier tile has published by now (its look-back saw them
+    // all), so every tile has read the header.
+    if (tile == tiles - 1 && lane == 0) close_call(header, hdr, tiles);
+}
+
 // Exclusive prefix of tile `tile` (> 0): the sum of all earlier tiles. Run by
 // one whole wavefront; lane l inspects tile (window_end - l), whose status word
 // of this call's parity is status[2 * tile + parity]. Every tile below `tile` is
@@ -277,21 +321,7 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // uniform: what only wave 0 does stays in scalar registers
     const uint32_t tiles = gridDim.x;
 
-    uint32_t tile = blockIdx.x;
-    {
-        // Consecutive workgroup ids go to the 8 XCDs in turn, and the XCDs drift apart, so in plain id
-        // order half of all tiles start before their predecessor and wait longer for it. Chunks of
-        // kChunk consecutive tiles are given to workgroups of one XCD instead (every 8th id), which
-        // start in order; only chunk boundaries cross XCDs. A tile's predecessors then have ids at
-        // most 8 * kChunk above its own, far fewer than the workgroups resident at once, so the lowest
-        // unfinished tile is still always running.
-        constexpr uint32_t G = kChunk, SPAN = 8 * G;
-        const uint32_t whole = (tiles / SPAN) * SPAN;
-        if (tile < whole) {
-            const uint32_t xcd = tile % 8, j = tile / 8;
-            tile = (j / G) * SPAN + xcd * G + (j % G);
-        }
-    }
+    uint32_t tile = tile_of_workgroup(blockIdx.x, tiles);
     if constexpr (TICKET) {
         // Dynamic tile id: tiles are numbered in the order blocks start running (examples/scan.py:88-99).
         if (tid == 0)
@@ -365,18 +395,7 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
             if (lane == 0) publish(mine, kPrefix, Op::apply(aggregate, prefix));
         }
         if (lane == 0) s_tile_prefix = prefix;
-        // Zero the other parity's words: tile t clears words t, t + tiles, ... below that parity's mark.
-        const uint32_t dirty_other = parity ? hdr.y : hdr.z;
-        for (size_t w = tile + static_cast<size_t>(lane) * tiles; w < dirty_other; w += static_cast<size_t>(kWave) * tiles)
-            __hip_atomic_store(&status[2 * w + (parity ^ 1u)], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        // The last tile closes the call: every earlier tile has published by now (its look-back saw
-        // them all), so every tile has read the header.
-        if (tile == tiles - 1 && lane == 0) {
-            __hip_atomic_store(&header[kHdrTicket], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(&header[kHdrDirty0 + parity], tiles, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(&header[kHdrDirty0 + (parity ^ 1u)], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(&header[kHdrCalls], calls + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
+        finish_status_protocol(header, status, hdr, tile, tiles, lane);
     }
     __syncthreads();
     const uint32_t base_sum = Op::apply(s_tile_prefix, wave_prefix);
@@ -416,6 +435,231 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
                 if (i < n) out[i] = Op::apply(r[c], base_sum);
             }
         }
+    }
+}
+
+// ------------------------------------------------------------------ segmented scan --
+//
+// Inclusive sums that start again at every element whose head flag is set: the same single pass over
+// (flag, value) pairs, flag = "a head lies in the range the value covers", combined as
+// (fa, va) (+) (fb, vb) = (fa | fb, fb ? vb : va + vb), a earlier than b. The operator is associative but not
+// commutative, so every combination below keeps the order of the elements. The reference scans one segment
+// (examples/scan.py:200-227); this is the decomposition of that kernel with the pair in place of the sum.
+// A status word carries the pair: state in bits 0-7, flag in bit 8, value in the upper half.
+struct Seg {
+    uint32_t f, v;
+};
+__device__ __forceinline__ Seg seg_combine(Seg a, Seg b) { return Seg{a.f | b.f, b.f ? b.v : a.v + b.v}; }
+
+template <int CTRL, int ROW_MASK, bool ZERO_FILL>
+__device__ __forceinline__ Seg seg_dpp(Seg x) {  // lanes without a source receive (0, 0), the identity
+    return Seg{dpp<CTRL, ROW_MASK, ZERO_FILL>(x.f), dpp<CTRL, ROW_MASK, ZERO_FILL>(x.v)};
+}
+__device__ __forceinline__ Seg wave_inclusive_scan_seg(Seg x) {
+    x = seg_combine(seg_dpp<0x111, 0xf, true>(x), x);
+    x = seg_combine(seg_dpp<0x112, 0xf, true>(x), x);
+    x = seg_combine(seg_dpp<0x114, 0xf, true>(x), x);
+    x = seg_combine(seg_dpp<0x118, 0xf, true>(x), x);
+    x = seg_combine(seg_dpp<0x142, 0xa, false>(x), x);
+    x = seg_combine(seg_dpp<0x143, 0xc, false>(x), x);
+    return x;
+}
+__device__ __forceinline__ u64 pack_seg_status(uint32_t state, Seg p) {
+    return static_cast<u64>(state | (p.f << 8)) | (static_cast<u64>(p.v) << 32);
+}
+
+// The pair that everything before tile `tile` (> 0) contributes to it. The walk back ends at the nearest
+// tile that has published a prefix or whose own range holds a head: what lies before a head does not matter.
+__device__ __forceinline__ Seg look_back_seg(const u64* status, uint32_t parity, uint32_t tile, int lane,
+                                             uint32_t spin_limit, uint32_t* report) {
+    Seg sum{0u, 0u};
+    uint32_t spins = 0;
+    long long window_end = static_cast<long long>(tile) - 1;
+    while (true) {
+        if (spins >= spin_limit) {
+            if (lane == 0) __hip_atomic_store(report, tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+        }
+        const long long t = window_end - lane;
+        const u64 w = (t >= 0) ? poll(&status[2 * t + parity]) : pack_status(kPrefix, 0u);
+        const uint32_t state = static_cast<uint32_t>(w) & 0xffu;
+        const uint32_t flag = (static_cast<uint32_t>(w) >> 8) & 1u;
+        const uint32_t value = static_cast<uint32_t>(w >> 32);
+        const u64 is_invalid = __ballot(state == kInvalid);
+        const u64 ends_walk = __ballot(state == kPrefix || flag != 0u);
+        const int first_invalid = is_invalid ? __builtin_ctzll(is_invalid) : kWave;
+        const int first_end = ends_walk ? __builtin_ctzll(ends_walk) : kWave;
+        if (first_end >= first_invalid) {  // no end of the walk among the lanes known so far
+            if (first_invalid < kWave) {
+                ++spins;
+                continue;
+            }
+        }
+        // Lanes 0 .. last are valid; none before `last` holds a head, so their values simply add up
+        // (lane 0 is the nearest tile; the order does not matter for flagless pairs).
+        const int last = first_end < kWave ? first_end : kWave - 1;
+        const uint32_t contrib = lane <= last ? value : 0u;
+        sum.v += wave_last_lane(wave_inclusive_scan(contrib));
+        if (first_end < kWave) {
+            sum.f = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(flag), first_end));
+            break;
+        }
+        window_end -= kWave;
+    }
+    return sum;
+}
+
+// heads: one byte per element, non-zero = the element starts a segment. VEC: in and out 16 B aligned and
+// heads 4 B aligned.
+template <typename Cfg, bool VEC>
+__global__ __launch_bounds__(Cfg::BLOCK) void segmented_scan_lookback_kernel(const uint32_t* in, const uint8_t* heads,
+                                                                             uint32_t* out, size_t n, uint32_t* header,
+                                                                             u64* status, uint32_t spin_limit) {
+    constexpr int BLOCK = Cfg::BLOCK, VPT = Cfg::VPT;
+    constexpr int WAVES = BLOCK / kWave;
+    constexpr int TILE = BLOCK * VPT * 4;
+    constexpr int WAVE_ELEMS = kWave * VPT * 4;
+    constexpr int ROW_ELEMS = kWave * 4;
+    static_assert(VPT <= 16, "four `head seen` bits per packet are kept in two 32-bit masks");
+
+    __shared__ uint32_t s_wave_f[WAVES], s_wave_v[WAVES];
+    __shared__ uint32_t s_tile_prefix_v;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const uint32_t tiles = gridDim.x;
+    const uint32_t tile = tile_of_workgroup(blockIdx.x, tiles);
+
+    const size_t tile_base = static_cast<size_t>(tile) * TILE;
+    const size_t lane_base = tile_base + static_cast<size_t>(wave) * WAVE_ELEMS + lane * 4;
+    const bool full = VEC && (tile_base + TILE <= n);
+
+    // The head bytes of the tile wait in LDS (a dword per packet, row j of a wave at my_heads + 64 j) until
+    // the packet is scanned: sixteen more registers per lane would not fit beside the tile itself. Whole
+    // tiles fetch them with direct-to-LDS loads, issued in front of the value loads.
+    __shared__ uint32_t s_heads[BLOCK * VPT];
+    uint32_t* const my_heads = &s_heads[wave * VPT * kWave];
+    u32x4 v[VPT];
+    if (full) {
+        const char* wave_heads = reinterpret_cast<const char*>(heads + tile_base + static_cast<size_t>(wave) * WAVE_ELEMS);
+#pragma unroll
+        for (int j = 0; j < VPT; ++j) direct_load4(wave_heads + j * ROW_ELEMS, lane * 4u, my_heads + j * kWave);
+#pragma unroll
+        for (int j = 0; j < VPT; ++j)
+            v[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(in + lane_base + j * ROW_ELEMS));
+    } else {
+#pragma unroll
+        for (int j = 0; j < VPT; ++j) {
+            uint32_t hb = 0u;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const size_t i = lane_base + j * ROW_ELEMS + c;
+                v[j][c] = (i < n) ? in[i] : 0u;
+                if (i < n && heads[i] != 0) hb |= 1u << (8 * c);
+            }
+            my_heads[j * kWave + lane] = hb;
+        }
+    }
+    u32x4 hdr = {0u, 0u, 0u, 0u};
+    if (wave == 0) hdr = *reinterpret_cast<const u32x4*>(header + kHdrCalls);
+    // The direct loads are invisible to the compiler's wait counts; a wave reads only what it loaded itself.
+    __builtin_amdgcn_s_waitcnt(0);
+    asm volatile("" ::: "memory");
+
+    // seen[j / 8], bit 4 (j % 8) + c: a head lies between the start of this wave's part and element c of packet j.
+    uint32_t seen[2] = {0u, 0u};
+    Seg carry{0u, 0u};
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const uint32_t hb = my_heads[j * kWave + lane];
+        const bool h0 = (hb & 0x000000ffu) != 0, h1 = (hb & 0x0000ff00u) != 0, h2 = (hb & 0x00ff0000u) != 0,
+                   h3 = (hb & 0xff000000u) != 0;
+        v[j].y = h1 ? v[j].y : v[j].x + v[j].y;
+        v[j].z = h2 ? v[j].z : v[j].y + v[j].z;
+        v[j].w = h3 ? v[j].w : v[j].z + v[j].w;
+        const uint32_t s0 = h0, s1 = s0 | h1, s2 = s1 | h2, s3 = s2 | h3;  // head seen up to element c of the packet
+        const Seg inclusive = wave_inclusive_scan_seg(Seg{s3, v[j].w});
+        // what the lanes below contribute (identity in lane 0), then what the rows before do
+        Seg below{static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(inclusive.f), 0x138, 0xf, 0xf, false)),
+                  static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(inclusive.v), 0x138, 0xf, 0xf, false))};
+        const Seg before = seg_combine(carry, below);
+        v[j].x += s0 ? 0u : before.v;
+        v[j].y += s1 ? 0u : before.v;
+        v[j].z += s2 ? 0u : before.v;
+        v[j].w += s3 ? 0u : before.v;
+        const uint32_t bf = before.f;
+        seen[j / 8] |= ((s0 | bf) | ((s1 | bf) << 1) | ((s2 | bf) << 2) | ((s3 | bf) << 3)) << (4 * (j % 8));
+        carry = seg_combine(carry, Seg{wave_last_lane(inclusive.f), wave_last_lane(inclusive.v)});
+        // The packet's sums are final here: said explicitly, because the compiler otherwise postpones the
+        // additions above to the write-back and keeps their operands and conditions alive until then.
+        asm volatile("" : "+v"(v[j]));
+    }
+    // From here on the masks are all the compiler knows about the heads (it would otherwise keep three
+    // conditions per packet alive until the write-back: 48 spilled registers in the big tile).
+    asm volatile("" : "+v"(seen[0]), "+v"(seen[1]));
+    if (lane == 0) {
+        s_wave_f[wave] = carry.f;
+        s_wave_v[wave] = carry.v;
+    }
+    __syncthreads();
+
+    Seg wave_prefix{0u, 0u}, aggregate{0u, 0u};
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+        const Seg t{s_wave_f[w], s_wave_v[w]};
+        if (w < wave) wave_prefix = seg_combine(wave_prefix, t);
+        aggregate = seg_combine(aggregate, t);
+    }
+
+    if (wave == 0) {
+        const uint32_t parity = hdr.x & 1u;
+        u64* const mine = &status[2 * static_cast<size_t>(tile) + parity];
+        Seg prefix{0u, 0u};
+        if (tile == 0) {
+            if (lane == 0) __hip_atomic_store(mine, pack_seg_status(kPrefix, aggregate), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+            if (lane == 0) __hip_atomic_store(mine, pack_seg_status(kAggregate, aggregate), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            prefix = look_back_seg(status, parity, tile, lane, spin_limit, &header[kHdrReport]);
+            if (lane == 0)
+                __hip_atomic_store(mine, pack_seg_status(kPrefix, seg_combine(prefix, aggregate)), __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (lane == 0) s_tile_prefix_v = prefix.v;
+        clear_other_parity(status, hdr, tile, tiles, lane);
+    }
+    __syncthreads();
+    // What comes before this wave: the tile's prefix, unless a head in an earlier wave of the tile cuts it off.
+    const uint32_t base = seg_combine(Seg{0u, s_tile_prefix_v}, wave_prefix).v;
+
+    if (full) {
+#pragma unroll
+        for (int j = 0; j < VPT; ++j) {
+            const uint32_t bits = seen[j / 8] >> (4 * (j % 8));
+            u32x4 r = v[j];
+            r.x += (bits & 1u) ? 0u : base;
+            r.y += (bits & 2u) ? 0u : base;
+            r.z += (bits & 4u) ? 0u : base;
+            r.w += (bits & 8u) ? 0u : base;
+            stream_store(reinterpret_cast<u32x4*>(out + lane_base + j * ROW_ELEMS), r);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < VPT; ++j) {
+            const uint32_t bits = seen[j / 8] >> (4 * (j % 8));
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const size_t i = lane_base + j * ROW_ELEMS + c;
+                if (i < n) out[i] = v[j][c] + (((bits >> c) & 1u) ? 0u : base);
+            }
+        }
+    }
+    // A look-back that ended at a head says nothing about the tiles before that head, so the last tile's
+    // look-back cannot tell that every tile has read the header. Tiles count themselves off instead, and
+    // the one that counts last closes the call.
+    if (tid == 0) {
+        const uint32_t done = __hip_atomic_fetch_add(&header[kHdrDone], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (done == tiles - 1) close_call(header, hdr, tiles);
     }
 }
 
@@ -544,6 +788,39 @@ int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws
     if (!vec) return launch_cfg<SmallCfg, false>(in, out, n, header, status, flags, limit, s);
     if (use_small(n, vec)) return launch_cfg<SmallCfg, true>(in, out, n, header, status, flags, limit, s);
     return launch_cfg<BigCfg, true>(in, out, n, header, status, flags, limit, s);
+}
+
+int launch_segmented_scan(const uint32_t* in, const uint8_t* heads, uint32_t* out, size_t n, void* ws, size_t ws_bytes,
+                          hipStream_t s) {
+    if (n == 0) return 0;
+    if (in == nullptr || out == nullptr || heads == nullptr || ws == nullptr)
+        return fail(1, "prism_segmented_scan: null pointer with n=%zu", n);
+    if (!aligned4(in) || !aligned4(out)) return fail(1, "prism_segmented_scan: data pointers must be 4-byte aligned");
+    if ((reinterpret_cast<uintptr_t>(ws) & 15u) != 0)
+        return fail(1, "prism_segmented_scan: workspace must be 16-byte aligned");
+    const size_t need = scan_workspace_bytes(n);
+    if (ws_bytes < need)
+        return fail(1, "prism_segmented_scan: workspace of %zu bytes is smaller than the %zu needed for n=%zu",
+                    ws_bytes, need, n);
+    const uintptr_t a = reinterpret_cast<uintptr_t>(in), b = reinterpret_cast<uintptr_t>(out),
+                    h = reinterpret_cast<uintptr_t>(heads), bytes = n * sizeof(uint32_t);
+    if (in != out && a < b + bytes && b < a + bytes)
+        return fail(1, "prism_segmented_scan: in and out overlap without being equal");
+    if (h < b + bytes && b < h + n) return fail(1, "prism_segmented_scan: heads and out overlap");
+    if (ceil_div(n, kWorkspaceTileElems) > 0x7fffffffull) return fail(1, "prism_segmented_scan: n=%zu too large", n);
+    uint32_t* header = reinterpret_cast<uint32_t*>(ws);
+    u64* status = reinterpret_cast<u64*>(static_cast<char*>(ws) + kHeaderBytes);
+    const bool vec = aligned16(in) && aligned16(out) && aligned4(heads);
+    const bool small = use_small(n, vec);
+    const size_t tiles = ceil_div(n, static_cast<size_t>(small ? tile_elems<SmallCfg>() : tile_elems<BigCfg>()));
+    const dim3 grid(static_cast<unsigned>(tiles));
+    if (!vec)
+        segmented_scan_lookback_kernel<SmallCfg, false><<<grid, dim3(SmallCfg::BLOCK), 0, s>>>(in, heads, out, n, header, status, kSpinLimit);
+    else if (small)
+        segmented_scan_lookback_kernel<SmallCfg, true><<<grid, dim3(SmallCfg::BLOCK), 0, s>>>(in, heads, out, n, header, status, kSpinLimit);
+    else
+        segmented_scan_lookback_kernel<BigCfg, true><<<grid, dim3(BigCfg::BLOCK), 0, s>>>(in, heads, out, n, header, status, kSpinLimit);
+    return check_launch("segmented_scan_lookback_kernel");
 }
 
 int launch_scan_static(const uint32_t* in, uint32_t* out, size_t n, hipStream_t s) {

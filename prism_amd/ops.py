@@ -177,6 +177,25 @@ def scan(inp: "torch.Tensor", out: Optional["torch.Tensor"] = None,
     return out
 
 
+def segmented_scan(inp: "torch.Tensor", heads: "torch.Tensor", out: Optional["torch.Tensor"] = None,
+                   workspace: Optional["torch.Tensor"] = None, check: bool = True) -> "torch.Tensor":
+    """Inclusive sums modulo 2^32 that start again at every element whose byte in `heads` (uint8 / bool, one per
+    element) is non-zero; element 0 always starts a segment. out may be inp. workspace and check as for scan()."""
+    _need(inp, (torch.int32, torch.uint32), 0, "inp")
+    n = inp.numel()
+    _need(heads, (torch.uint8, torch.bool), n, "heads")
+    if out is None:
+        out = torch.empty_like(inp)
+    _need(out, (inp.dtype,), n, "out")
+    if workspace is None:
+        workspace = new_scan_workspace(n, inp.device)
+    _check(_lib.load().prism_segmented_scan_i32(_ptr(inp), _ptr(heads), _ptr(out), n, _ptr(workspace),
+                                                _ws_bytes(workspace), _stream()), "segmented_scan")
+    if check and n > 0:
+        scan_status(workspace)
+    return out
+
+
 # ------------------------------------------------------------------- sgemm --
 
 def run_my_kernel(my_kernel_num: int, M: int, N: int, K: int, alpha: float, A: Ptr, B: Ptr,

@@ -251,6 +251,71 @@ def test_scan_workspace_shared_by_calls_of_any_length_and_kind(prism, oracle):
         assert np.array_equal(host(out), want), (n, kw)
 
 
+SEG_SIZES = [1, 2, 63, 64, 65, 255, 256, 257, 1023, 1025, 4096, 16383, 16384, 16385, 65535, 65536, 65537, 100_003,
+             262_145, (1 << 24) - 1, (1 << 24) + 65536 * 3 + 5, 1 << 26]
+
+
+@pytest.mark.parametrize("n", SEG_SIZES)
+def test_segmented_scan(prism, oracle, n):
+    """Sums that start again at every head, on both tile shapes, for segments that are much shorter than a
+    packet, about a wave's row, about a tile and many tiles long, with no head at all and with every element a
+    head; out of place with a fenced output, in place, from views that are only 4-byte (values) / 1-byte
+    (heads) aligned, and through one workspace shared with plain scans. Bit for bit against the serial loop."""
+    x = oracle.gen_scan(n, seed=n % 101)
+    xd = dev(x)
+    ws = prism.new_scan_workspace(n)
+    for mean in (1.3, 6, 300, 20_000, 3_000_000):
+        h = oracle.gen_heads(n, mean, seed=int(mean) + n % 7)
+        want = oracle.segmented_scan_cpu(x, h)
+        out = torch.full((n + 8,), -7, dtype=torch.int32, device=DEV)
+        prism.segmented_scan(xd, dev(h), out[:n], workspace=ws)
+        got = host(out)
+        assert np.array_equal(got[:n], want), mean
+        assert np.all(got[n:] == -7)
+        assert np.array_equal(host(prism.scan(xd, workspace=ws)), oracle.scan_cpu(x))  # same workspace, other kind
+    none, every = np.zeros(n, np.uint8), np.ones(n, np.uint8)
+    assert np.array_equal(host(prism.segmented_scan(xd, dev(none), workspace=ws)), oracle.scan_cpu(x))
+    assert np.array_equal(host(prism.segmented_scan(xd, dev(every), workspace=ws)), x)
+    h = oracle.gen_heads(n, 50, seed=3)
+    want = oracle.segmented_scan_cpu(x, h)
+    buf = xd.clone()
+    prism.segmented_scan(buf, dev(h).bool(), buf, workspace=ws)  # in place, bool flags
+    assert np.array_equal(host(buf), want)
+    if n >= 256:
+        x1 = dev(np.concatenate([[0], x]).astype(np.int32))[1:]
+        h1 = dev(np.concatenate([[9], h]).astype(np.uint8))[1:]
+        y = torch.zeros(n + 1, dtype=torch.int32, device=DEV)
+        prism.segmented_scan(x1, h1, y[1:], workspace=ws)
+        assert np.array_equal(host(y)[1:], want)
+        prism.segmented_scan(xd, h1, buf, workspace=ws)  # aligned values, unaligned heads
+        assert np.array_equal(host(buf), want)
+
+
+def test_segmented_scan_2pow30_properties(prism):
+    """Full size: out[i] == in[i] at every head, out[i] - out[i-1] == in[i] everywhere else, over the whole
+    array, for segments of about 1000 elements and for one head in the middle of every 2^20."""
+    n = 1 << 30
+    g = torch.Generator(device=DEV)
+    g.manual_seed(1)
+    x = torch.randint(-1000, 1001, (n,), dtype=torch.int32, device=DEV, generator=g)
+    for kind in ("dense", "sparse"):
+        if kind == "dense":
+            heads = (torch.rand((n,), device=DEV, generator=g) < 1e-3).to(torch.uint8)
+        else:
+            heads = torch.zeros(n, dtype=torch.uint8, device=DEV)
+            heads[(1 << 19)::(1 << 20)] = 1
+        out = prism.segmented_scan(x, heads)
+        chunk = 1 << 26
+        assert int(out[0]) == int(x[0])
+        for s in range(0, n, chunk):
+            e = s + chunk
+            lo = max(s, 1)
+            is_head = heads[lo:e] != 0
+            want = torch.where(is_head, x[lo:e], out[lo - 1:e - 1] + x[lo:e])
+            assert torch.equal(out[lo:e], want), (kind, s)
+        del out
+
+
 def test_scan_2pow30_properties(prism):
     """Full BASELINE size (4 GiB in, 4 GiB out): checked on the device through
     size-independent properties - first element, the difference invariant

@@ -86,6 +86,46 @@ def test_running_maximum_closed_forms_library_routine_and_invariants(oracle):
         assert got[0] == x[0] and np.array_equal(got[steps], x[steps])  # a new maximum is the element itself
 
 
+def test_segmented_scan_special_cases_hand_case_and_two_library_routes(oracle):
+    """Pins oracle_segmented_scan_cpu: without heads it is the plain scan; with every element a head it is the
+    input; a hand-computed case with a wrap; against numpy.cumsum run segment by segment; and against the
+    closed form through ONE global cumulative sum (out[i] = S[i] - S[start(i) - 1])."""
+    rng = np.random.default_rng(5)
+    x = rng.integers(-1000, 1001, 10_000, dtype=np.int32)
+    none = np.zeros(x.size, np.uint8)
+    assert np.array_equal(oracle.segmented_scan_cpu(x, none), oracle.scan_cpu(x))
+    assert np.array_equal(oracle.segmented_scan_cpu(x, np.ones(x.size, np.uint8)), x)
+    hx = np.array([5, 7, 2**31 - 1, 1, 4, -3, 10], dtype=np.int32)
+    hh = np.array([0, 0, 1, 0, 0, 255, 0], dtype=np.uint8)  # element 0 starts a segment whatever its flag says
+    assert oracle.segmented_scan_cpu(hx, hh).tolist() == [5, 12, 2**31 - 1, -2**31, -2**31 + 4, -3, 7]
+    for mean in (1.5, 7, 300, 5000):
+        h = oracle.gen_heads(x.size, mean, seed=int(mean))
+        got = oracle.segmented_scan_cpu(x, h)
+        want = np.empty_like(x)
+        starts = np.flatnonzero(np.concatenate([[True], h[1:] != 0]))
+        for a, b in zip(starts, np.concatenate([starts[1:], [x.size]])):
+            want[a:b] = np.cumsum(x[a:b], dtype=np.int32)
+        assert np.array_equal(got, want)
+        assert np.array_equal(got, oracle.np_segmented_scan(x, h))
+    big = np.full(100, 2**31 - 1, dtype=np.int32)
+    bh = np.zeros(100, np.uint8)
+    bh[50] = 1
+    assert np.array_equal(oracle.segmented_scan_cpu(big, bh), oracle.np_segmented_scan(big, bh))
+    assert oracle.segmented_scan_cpu(np.zeros(0, np.int32), np.zeros(0, np.uint8)).size == 0
+
+
+def test_scan_i64_closed_forms_and_numpy(oracle):
+    n = 5000
+    assert np.array_equal(oracle.scan_i64_cpu(np.ones(n, np.int64)), np.arange(1, n + 1, dtype=np.int64))
+    wrap = np.array([2**63 - 1, 1, 2**63 - 1, 2], dtype=np.int64)
+    assert oracle.scan_i64_cpu(wrap).tolist() == [2**63 - 1, -2**63, -1, 1]
+    x = np.random.default_rng(6).integers(-2**62, 2**62, 20_000, dtype=np.int64)
+    with np.errstate(over="ignore"):
+        assert np.array_equal(oracle.scan_i64_cpu(x), np.cumsum(x, dtype=np.int64))
+    u = x.view(np.uint64)
+    assert np.array_equal(oracle.scan_i64_cpu(u), np.cumsum(u, dtype=np.uint64))
+
+
 def test_scan_vs_numpy_cumsum_and_difference_invariant(oracle):
     for n in (1, 63, 64, 65, 4095, 4096, 4097, 16384, 100_003):
         x = oracle.gen_scan(n, seed=n)
