@@ -79,8 +79,8 @@ int prism_add_m(const int32_t* x, int32_t* y, int32_t m, size_t n, void* stream)
 
 /*
  * Bytes of device workspace the scans need for n elements: a 256-byte header
- * and 16 bytes per 16384 elements (the size the reference's launcher uses,
- * n / 16384 * 16 + 4). Replaces scan_gpu::get_workspace_size
+ * and 16 bytes per 16384 elements plus 16 (the size the reference's launcher
+ * uses, n / 16384 * 16 + 4, rounded up). Replaces scan_gpu::get_workspace_size
  * (evals/4090_scan/main.cu:63-66). Never 0, so a caller may always allocate it.
  * A workspace sized for n serves every smaller n too.
  */
@@ -209,6 +209,20 @@ int prism_scan_min_i32(const int32_t* in, int32_t* out, size_t n, void* workspac
  */
 int prism_segmented_scan_i32(const int32_t* in, const uint8_t* heads, int32_t* out, size_t n,
                              void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Inclusive prefix sum of 64-bit elements, out[i] = in[0] + ... + in[i] modulo
+ * 2^64 (identical bit patterns for int64 and uint64): scan_kernel's
+ * decomposition (examples/scan.py:106-227) on wider elements. A tile publishes
+ * its 64-bit aggregate and prefix as two status words (state + half each) and
+ * a reader accepts them only as a pair of the same state. Pointers 8-byte
+ * aligned (16-byte aligned ones take the fast path); workspace
+ * (prism_scan_workspace_bytes(n) for the same n), aliasing, ordering and the
+ * status check as for prism_scan_i32. The reference scans uint32 only
+ * (evals/4090_scan/scan_harness.cuh:30-36).
+ */
+int prism_scan_i64(const int64_t* in, int64_t* out, size_t n, void* workspace,
+                   size_t workspace_bytes, void* stream);
 
 /*
  * The reference launcher's own shape: in-place on x, default stream, returns

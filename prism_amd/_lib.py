@@ -31,6 +31,7 @@ SIGNATURES = {
     "prism_scan_min_i32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p]),
     "prism_segmented_scan_i32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t,
                                            C.c_void_p]),
+    "prism_scan_i64": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p]),
     "prism_launch_scan": (C.c_void_p, [C.c_size_t, C.c_void_p, C.c_void_p]),
     "prism_sgemm": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_void_p,
                               C.c_float, C.c_void_p, C.c_void_p]),

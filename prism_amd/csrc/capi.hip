@@ -115,6 +115,11 @@ int prism_segmented_scan_i32(const int32_t* in, const uint8_t* heads, int32_t* o
     return launch_segmented_scan(u32(in), heads, u32(out), n, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
+int prism_scan_i64(const int64_t* in, int64_t* out, size_t n, void* workspace, size_t workspace_bytes, void* stream) {
+    return launch_scan64(reinterpret_cast<const unsigned long long*>(in), reinterpret_cast<unsigned long long*>(out), n,
+                         workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
 uint32_t* prism_launch_scan(size_t n, uint32_t* x, void* workspace) {
     // The reference's launcher accepts any workspace contents (it clears them itself,
     // evals/4090_scan/main.cu:81-82), so this one initialises before every scan.

@@ -69,6 +69,7 @@ int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws
 int scan_status(void* ws, size_t ws_bytes, hipStream_t s);
 int launch_segmented_scan(const uint32_t* in, const uint8_t* heads, uint32_t* out, size_t n, void* ws, size_t ws_bytes,
                           hipStream_t s);
+int launch_scan64(const unsigned long long* in, unsigned long long* out, size_t n, void* ws, size_t ws_bytes, hipStream_t s);
 int launch_scan_static(const uint32_t* in, uint32_t* out, size_t n, hipStream_t s);
 int launch_calibrate_stream(int kind, const void* in, void* out, size_t bytes, hipStream_t s);
 int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, const float* B,

@@ -663,6 +663,173 @@ __global__ __launch_bounds__(Cfg::BLOCK) void segmented_scan_lookback_kernel(con
     }
 }
 
+// ------------------------------------------------------------------ 64-bit elements --
+//
+// Inclusive sums of 64-bit elements modulo 2^64 (int64 and uint64 share the bits): the same single pass with
+// two elements per 16 B packet. A 64-bit value does not fit a 64-bit status word beside its state, so a tile
+// owns two status slots, {state, low half} and {state, high half}; a reader accepts the pair only when both
+// carry the same state (a tile rewrites both on its way from aggregate to prefix, low half first) and polls
+// again otherwise. The reference scans uint32 (evals/4090_scan/scan_harness.cuh:30-36); this is its
+// decomposition (examples/scan.py:106-227) on wider elements.
+typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
+
+template <int CTRL, int ROW_MASK, bool ZERO_FILL>
+__device__ __forceinline__ u64 dpp64(u64 x) {
+    return static_cast<u64>(dpp<CTRL, ROW_MASK, ZERO_FILL>(static_cast<uint32_t>(x))) |
+           (static_cast<u64>(dpp<CTRL, ROW_MASK, ZERO_FILL>(static_cast<uint32_t>(x >> 32))) << 32);
+}
+__device__ __forceinline__ u64 wave_inclusive_scan64(u64 x) {
+    x += dpp64<0x111, 0xf, true>(x);
+    x += dpp64<0x112, 0xf, true>(x);
+    x += dpp64<0x114, 0xf, true>(x);
+    x += dpp64<0x118, 0xf, true>(x);
+    x += dpp64<0x142, 0xa, false>(x);
+    x += dpp64<0x143, 0xc, false>(x);
+    return x;
+}
+__device__ __forceinline__ u64 wave_last_lane64(u64 x) {
+    return static_cast<u64>(wave_last_lane(static_cast<uint32_t>(x))) | (static_cast<u64>(wave_last_lane(static_cast<uint32_t>(x >> 32))) << 32);
+}
+__device__ __forceinline__ void publish64(u64* lo_word, uint32_t state, u64 value) {  // the high half sits one slot on
+    publish(lo_word, state, static_cast<uint32_t>(value));
+    publish(lo_word + 2, state, static_cast<uint32_t>(value >> 32));
+}
+
+// Sum of all tiles before `tile` (> 0). Lane l inspects tile window_end - l: slots 2 t and 2 t + 1.
+__device__ __forceinline__ u64 look_back64(const u64* status, uint32_t parity, uint32_t tile, int lane, uint32_t spin_limit,
+                                           uint32_t* report) {
+    u64 sum = 0;
+    uint32_t spins = 0;
+    long long window_end = static_cast<long long>(tile) - 1;
+    while (true) {
+        if (spins >= spin_limit) {
+            if (lane == 0) __hip_atomic_store(report, tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+        }
+        const long long t = window_end - lane;
+        const u64 lo = (t >= 0) ? poll(&status[4 * t + parity]) : pack_status(kPrefix, 0u);
+        const u64 hi = (t >= 0) ? poll(&status[4 * t + 2 + parity]) : pack_status(kPrefix, 0u);
+        const uint32_t state_lo = static_cast<uint32_t>(lo), state_hi = static_cast<uint32_t>(hi);
+        // halves of two different publications (or one still missing) count as "nothing yet"
+        const uint32_t state = state_lo == state_hi ? state_lo : kInvalid;
+        const u64 value = (lo >> 32) | (hi & 0xffffffff00000000ull);
+        const u64 has_prefix = __ballot(state == kPrefix);
+        const u64 is_invalid = __ballot(state == kInvalid);
+        const u64 needed = has_prefix ? ((2ull << __builtin_ctzll(has_prefix)) - 1ull) : ~0ull;
+        if (is_invalid & needed) {
+            ++spins;
+            continue;
+        }
+        const u64 contrib = ((needed >> lane) & 1ull) ? value : 0ull;
+        sum += wave_last_lane64(wave_inclusive_scan64(contrib));
+        if (has_prefix) break;
+        window_end -= kWave;
+    }
+    return sum;
+}
+
+// VEC: in and out are 16 B aligned. One tile shape: a tile of 2 * BLOCK * VPT elements owns two status slots,
+// which is what the workspace holds per 32768 elements.
+template <typename Cfg, bool VEC>
+__global__ __launch_bounds__(Cfg::BLOCK) void scan64_lookback_kernel(const u64* in, u64* out, size_t n, uint32_t* header,
+                                                                     u64* status, uint32_t spin_limit) {
+    constexpr int BLOCK = Cfg::BLOCK, VPT = Cfg::VPT;
+    constexpr int WAVES = BLOCK / kWave;
+    constexpr int TILE = BLOCK * VPT * 2;
+    constexpr int WAVE_ELEMS = kWave * VPT * 2;
+    constexpr int ROW_ELEMS = kWave * 2;
+    static_assert(TILE >= 2 * static_cast<int>(kWorkspaceTileElems), "two status slots per tile");
+
+    __shared__ u64 s_wave_total[WAVES];
+    __shared__ u64 s_tile_prefix;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const uint32_t tiles = gridDim.x;
+    const uint32_t tile = tile_of_workgroup(blockIdx.x, tiles);
+
+    const size_t tile_base = static_cast<size_t>(tile) * TILE;
+    const size_t lane_base = tile_base + static_cast<size_t>(wave) * WAVE_ELEMS + lane * 2;
+    const bool full = VEC && (tile_base + TILE <= n);
+
+    u64x2 v[VPT];
+    if (full) {
+#pragma unroll
+        for (int j = 0; j < VPT; ++j)
+            v[j] = __builtin_nontemporal_load(reinterpret_cast<const u64x2*>(in + lane_base + j * ROW_ELEMS));
+    } else {
+#pragma unroll
+        for (int j = 0; j < VPT; ++j)
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const size_t i = lane_base + j * ROW_ELEMS + c;
+                v[j][c] = (i < n) ? in[i] : 0ull;
+            }
+    }
+    u32x4 hdr = {0u, 0u, 0u, 0u};
+    if (wave == 0) hdr = *reinterpret_cast<const u32x4*>(header + kHdrCalls);
+
+    u64 carry = 0;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        v[j].y += v[j].x;
+        const u64 inclusive = wave_inclusive_scan64(v[j].y);
+        const u64 before = carry + (inclusive - v[j].y);
+        v[j].x += before;
+        v[j].y += before;
+        carry += wave_last_lane64(inclusive);
+    }
+    if (lane == 0) s_wave_total[wave] = carry;
+    __syncthreads();
+
+    u64 wave_prefix = 0, aggregate = 0;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+        const u64 t = s_wave_total[w];
+        if (w < wave) wave_prefix += t;
+        aggregate += t;
+    }
+
+    if (wave == 0) {
+        const uint32_t parity = hdr.x & 1u;
+        u64* const mine = &status[4 * static_cast<size_t>(tile) + parity];
+        u64 prefix = 0;
+        if (tile == 0) {
+            if (lane == 0) publish64(mine, kPrefix, aggregate);
+        } else {
+            if (lane == 0) publish64(mine, kAggregate, aggregate);
+            prefix = look_back64(status, parity, tile, lane, spin_limit, &header[kHdrReport]);
+            if (lane == 0) publish64(mine, kPrefix, aggregate + prefix);
+        }
+        if (lane == 0) s_tile_prefix = prefix;
+        // The workspace protocol counts status slots: this tile's are 2 t and 2 t + 1 of 2 * tiles.
+        clear_other_parity(status, hdr, 2 * tile, 2 * tiles, lane);
+        clear_other_parity(status, hdr, 2 * tile + 1, 2 * tiles, lane);
+        if (tile == tiles - 1 && lane == 0) close_call(header, hdr, 2 * tiles);
+    }
+    __syncthreads();
+    const u64 base = s_tile_prefix + wave_prefix;
+
+    if (full) {
+#pragma unroll
+        for (int j = 0; j < VPT; ++j) {
+            const u64x2 r = v[j] + base;
+            u32x4 bits;
+            __builtin_memcpy(&bits, &r, 16);
+            stream_store(reinterpret_cast<u32x4*>(out + lane_base + j * ROW_ELEMS), bits);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < VPT; ++j)
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const size_t i = lane_base + j * ROW_ELEMS + c;
+                if (i < n) out[i] = v[j][c] + base;
+            }
+    }
+}
+
 // Zero fill of a workspace (a kernel, not hipMemsetAsync, so that it can be captured into a graph).
 __global__ __launch_bounds__(256) void scan_fill_zero_kernel(u64* words, size_t n_words) {
     const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
@@ -704,7 +871,7 @@ int launch_cfg(const uint32_t* in, uint32_t* out, size_t n, uint32_t* header, u6
 // long as the module. Every GPU holds its own copy at its own address; host code must use the
 // address hipGetSymbolAddress returns, never the array's name.
 constexpr size_t kStaticMaxElems = size_t{1} << 31;
-constexpr size_t kStaticBytes = kHeaderBytes + 16 * (kStaticMaxElems / kWorkspaceTileElems);
+constexpr size_t kStaticBytes = kHeaderBytes + 16 * (kStaticMaxElems / kWorkspaceTileElems + 1);
 static __device__ __align__(256) unsigned char scratch[kStaticBytes];  // zero at load = initialised
 
 constexpr int kMaxDevices = 64;
@@ -736,8 +903,8 @@ int static_scratch(void** ptr, hipStream_t s) {
 }  // namespace
 
 size_t scan_workspace_bytes(size_t n) {
-    const size_t tiles = ceil_div(n, kWorkspaceTileElems);
-    return kHeaderBytes + 16 * (tiles > 0 ? tiles : 1);
+    // One 16-byte slot per 16384 elements and one to spare: a tile of 64-bit elements (32768 of them) owns two.
+    return kHeaderBytes + 16 * (ceil_div(n, kWorkspaceTileElems) + 1);
 }
 
 int scan_workspace_init(void* ws, size_t ws_bytes, hipStream_t s) { return scan_workspace_init_impl(ws, ws_bytes, s); }
@@ -821,6 +988,32 @@ int launch_segmented_scan(const uint32_t* in, const uint8_t* heads, uint32_t* ou
     else
         segmented_scan_lookback_kernel<BigCfg, true><<<grid, dim3(BigCfg::BLOCK), 0, s>>>(in, heads, out, n, header, status, kSpinLimit);
     return check_launch("segmented_scan_lookback_kernel");
+}
+
+int launch_scan64(const unsigned long long* in, unsigned long long* out, size_t n, void* ws, size_t ws_bytes, hipStream_t s) {
+    if (n == 0) return 0;
+    if (in == nullptr || out == nullptr || ws == nullptr) return fail(1, "prism_scan_i64: null pointer with n=%zu", n);
+    if ((reinterpret_cast<uintptr_t>(in) & 7u) != 0 || (reinterpret_cast<uintptr_t>(out) & 7u) != 0)
+        return fail(1, "prism_scan_i64: data pointers must be 8-byte aligned");
+    if ((reinterpret_cast<uintptr_t>(ws) & 15u) != 0) return fail(1, "prism_scan_i64: workspace must be 16-byte aligned");
+    const size_t need = scan_workspace_bytes(n);
+    if (ws_bytes < need)
+        return fail(1, "prism_scan_i64: workspace of %zu bytes is smaller than the %zu needed for n=%zu", ws_bytes, need, n);
+    if (in != out) {
+        const uintptr_t a = reinterpret_cast<uintptr_t>(in), b = reinterpret_cast<uintptr_t>(out), bytes = n * sizeof(u64);
+        if (a < b + bytes && b < a + bytes) return fail(1, "prism_scan_i64: in and out overlap without being equal");
+    }
+    constexpr size_t tile = 2 * static_cast<size_t>(BigCfg::BLOCK) * BigCfg::VPT;
+    const size_t tiles = ceil_div(n, tile);
+    if (tiles > 0x3fffffffull) return fail(1, "prism_scan_i64: n=%zu too large", n);
+    uint32_t* header = reinterpret_cast<uint32_t*>(ws);
+    u64* status = reinterpret_cast<u64*>(static_cast<char*>(ws) + kHeaderBytes);
+    const dim3 grid(static_cast<unsigned>(tiles)), block(BigCfg::BLOCK);
+    if (aligned16(in) && aligned16(out))
+        scan64_lookback_kernel<BigCfg, true><<<grid, block, 0, s>>>(in, out, n, header, status, kSpinLimit);
+    else
+        scan64_lookback_kernel<BigCfg, false><<<grid, block, 0, s>>>(in, out, n, header, status, kSpinLimit);
+    return check_launch("scan64_lookback_kernel");
 }
 
 int launch_scan_static(const uint32_t* in, uint32_t* out, size_t n, hipStream_t s) {

@@ -148,7 +148,7 @@ def launch_scan(n: int, x: "torch.Tensor", workspace: "torch.Tensor", check: boo
 def scan(inp: "torch.Tensor", out: Optional["torch.Tensor"] = None,
          workspace: Optional["torch.Tensor"] = None, exclusive: bool = False, op: str = "sum",
          ticket_order: bool = False, spin_limit: int = -1, check: bool = True) -> "torch.Tensor":
-    """Prefix sum modulo 2^32 of a 1-D int32/uint32 tensor; out may be inp. Inclusive (out[i] includes
+    """Prefix sum modulo 2^32 of a 1-D int32/uint32 tensor (modulo 2^64 of an int64/uint64 one); out may be inp. Inclusive (out[i] includes
     inp[i]) unless exclusive=True (out[0] = 0, out[i] = inp[0] + ... + inp[i-1]). op="max" / op="min": the
     running maximum / minimum of an int32 tensor instead (inclusive only).
 
@@ -160,6 +160,19 @@ def scan(inp: "torch.Tensor", out: Optional["torch.Tensor"] = None,
     """
     if op not in SCAN_OP:
         raise ValueError("scan: op must be 'sum', 'max' or 'min'")
+    if inp.dtype in (torch.int64, torch.uint64):  # 64-bit elements: inclusive sums modulo 2^64 only
+        if op != "sum" or exclusive or ticket_order or spin_limit != -1:
+            raise ValueError("scan: 64-bit elements support the inclusive sum in workgroup-id order only")
+        n = inp.numel()
+        if out is None:
+            out = torch.empty_like(inp)
+        _need(out, (inp.dtype,), n, "out")
+        if workspace is None:
+            workspace = new_scan_workspace(n, inp.device)
+        _check(_lib.load().prism_scan_i64(_ptr(inp), _ptr(out), n, _ptr(workspace), _ws_bytes(workspace), _stream()), "scan")
+        if check and n > 0:
+            scan_status(workspace)
+        return out
     if op != "sum" and (exclusive or ticket_order):
         raise ValueError("scan: the running maximum and minimum are inclusive and use workgroup-id order")
     _need(inp, (torch.int32,) if op != "sum" else (torch.int32, torch.uint32), 0, "inp")

@@ -43,7 +43,8 @@ def test_every_declaration_cites_the_reference():
     # each entry point's comment names the reference file it replaces
     for name, cite in [("prism_add_m", "add_m_thread.py"), ("prism_scan_workspace_bytes", "4090_scan/main.cu"),
                        ("prism_scan_i32", "scan.py"), ("prism_scan_i32_ex", "lookback_to_prev_blocks.cu"),
-                       ("prism_scan_workspace_init", "4090_scan/main.cu:81-82"), ("prism_scan_exclusive_i32", "scan.py:174-193"),
+                       ("prism_scan_workspace_init", "4090_scan/main.cu:81-82"), ("prism_scan_i64", "scan_harness.cuh:30-36"),
+                       ("prism_segmented_scan_i32", "scan.py:106-227"), ("prism_scan_exclusive_i32", "scan.py:174-193"),
                        ("prism_scan_max_i32", "scan.py:106-173"), ("prism_scan_min_i32", "scan.py:106-173"),
                        ("prism_launch_scan", "4090_scan/main.cu"),
                        ("prism_sgemm", "runner.cu"), ("prism_run_my_kernel", "runner.cu"),
@@ -98,7 +99,7 @@ def test_scan_workspace_size(lib):
     assert all(s > 0 and s % 16 == 0 for s in sizes)
     assert sizes == sorted(sizes)
     # a header plus the reference's 16 bytes per 16384 elements (main.cu:63-66)
-    assert sizes[-1] == 256 + (1 << 30) // 16384 * 16
+    assert sizes[-1] == 256 + ((1 << 30) // 16384 + 1) * 16 and sizes[0] == 256 + 16
 
 
 @pytest.mark.parametrize("tiles", [(1, 1), (1, 9), (7, 1), (8, 8), (64, 64), (3, 5), (33, 17), (64, 33), (5, 129)])

@@ -316,6 +316,55 @@ def test_segmented_scan_2pow30_properties(prism):
         del out
 
 
+@pytest.mark.parametrize("n", [1, 2, 127, 128, 129, 4095, 32767, 32768, 32769, 65536, 100_003, 1 << 20, (1 << 22) + 32768 * 3 + 5, 1 << 26])
+def test_scan_of_64_bit_elements(prism, oracle, n):
+    """Inclusive sums modulo 2^64: values that use all 64 bits (so both status halves matter and carries cross
+    them), out of place with a fenced output, in place, as uint64, from a view that is only 8-byte aligned, and on
+    a workspace shared with 32-bit scans. Bit for bit against the serial loop."""
+    rng = np.random.default_rng(n % 211)
+    x = rng.integers(-2**62, 2**62, n, dtype=np.int64)
+    want = oracle.scan_i64_cpu(x)
+    ws = prism.new_scan_workspace(n)
+    xd = dev(x)
+    out = torch.full((n + 8,), -7, dtype=torch.int64, device=DEV)
+    prism.scan(xd, out[:n], workspace=ws)
+    got = host(out)
+    assert np.array_equal(got[:n], want) and np.all(got[n:] == -7)
+    small = oracle.gen_scan(min(n, 70_001), seed=1)
+    assert np.array_equal(host(prism.scan(dev(small), workspace=ws)), oracle.scan_cpu(small))  # a 32-bit scan in between
+    buf = xd.clone()
+    prism.scan(buf, buf, workspace=ws)
+    assert np.array_equal(host(buf), want)
+    carries = np.full(n, 0xffffffff, dtype=np.uint64)  # every addition carries into the high half
+    got_u = host(prism.scan(dev(carries.view(np.int64)), workspace=ws)).view(np.uint64)
+    assert np.array_equal(got_u, oracle.scan_i64_cpu(carries))
+    if n >= 128:
+        x1 = dev(np.concatenate([[0], x]).astype(np.int64))[1:]
+        y = torch.zeros(n + 1, dtype=torch.int64, device=DEV)
+        prism.scan(x1, y[1:], workspace=ws)
+        assert np.array_equal(host(y)[1:], want)
+    with pytest.raises(ValueError):
+        prism.scan(xd, exclusive=True)
+
+
+def test_scan_of_64_bit_elements_2pow29_properties(prism):
+    """4 GiB in, 4 GiB out: difference invariant over the whole array and the last element against block sums."""
+    n = 1 << 29
+    g = torch.Generator(device=DEV)
+    g.manual_seed(2)
+    x = torch.randint(-2**40, 2**40, (n,), dtype=torch.int64, device=DEV, generator=g)
+    out = prism.scan(x)
+    assert int(out[0]) == int(x[0])
+    chunk = 1 << 25
+    total = 0
+    for s in range(0, n, chunk):
+        e = s + chunk
+        lo = max(s, 1)
+        assert torch.equal(out[lo:e] - out[lo - 1:e - 1], x[lo:e])
+        total += int(x[s:e].sum())
+    assert int(out[-1]) == ((total + 2**63) % 2**64) - 2**63
+
+
 def test_scan_2pow30_properties(prism):
     """Full BASELINE size (4 GiB in, 4 GiB out): checked on the device through
     size-independent properties - first element, the difference invariant
