@@ -75,6 +75,24 @@ int prism_calibrate_stream(int kind, const void* in, void* out, size_t bytes, vo
  */
 int prism_add_m(const int32_t* x, int32_t* y, int32_t m, size_t n, void* stream);
 
+/*
+ * The reference's warp_load / warp_store (examples/warp_load.py:13-22,
+ * warp_store.py:13-22, with thread_load.py / thread_store.py) as an operator on
+ * 64-lane wavefronts: every chunk of 64 * items_per_lane ints is moved between
+ * the arrangement those functions give a warp (lane l holds items
+ * [l * items_per_lane, (l + 1) * items_per_lane), "blocked") and the one in
+ * which every instruction of the wavefront touches 64 consecutive ints
+ * ("striped": item j of lane l is element 64 j + l).
+ *   direction 0: out[c][64 j + l] = in[c][items_per_lane * l + j]
+ *   direction 1: the inverse
+ * for chunk c. items_per_lane is 1, 2, 4, 8 or 16; any n (a last, partial
+ * chunk counts as one padded with zeros: positions at or beyond n are neither
+ * read nor written, every position below n is written); in and out must not
+ * overlap.
+ */
+int prism_wave_regroup_i32(const int32_t* in, int32_t* out, size_t n, int items_per_lane,
+                           int direction, void* stream);
+
 /* ------------------------------------------------------------------ scan -- */
 
 /*

@@ -24,6 +24,7 @@ from .ops import (  # noqa: F401
     segmented_scan,
     sgemm,
     tile_coords,
+    wave_regroup,
 )
 
 __version__ = "0.1.0"

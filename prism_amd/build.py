@@ -16,7 +16,7 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "libprism_amd.so"
-SOURCES = ["capi.hip", "add_m.hip", "scan.hip", "sgemm.hip", "gemm_bf16.hip", "calibrate.hip"]
+SOURCES = ["capi.hip", "add_m.hip", "scan.hip", "sgemm.hip", "gemm_bf16.hip", "calibrate.hip", "regroup.hip"]
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_*_f32 out of scalar
 # float code; the kernels here get their fp32 throughput from MFMA instead.

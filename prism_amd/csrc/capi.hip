@@ -55,6 +55,10 @@ int prism_calibrate_stream(int kind, const void* in, void* out, size_t bytes, vo
     return launch_calibrate_stream(kind, in, out, bytes, static_cast<hipStream_t>(stream));
 }
 
+int prism_wave_regroup_i32(const int32_t* in, int32_t* out, size_t n, int items_per_lane, int direction, void* stream) {
+    return launch_wave_regroup(in, out, n, items_per_lane, direction, static_cast<hipStream_t>(stream));
+}
+
 int prism_add_m(const int32_t* x, int32_t* y, int32_t m, size_t n, void* stream) {
     return launch_add_m(x, y, m, n, static_cast<hipStream_t>(stream));
 }

@@ -75,6 +75,7 @@
 
 #include "common.h"
 #include "direct_load.h"
+#include "wave_io.h"
 
 namespace prism {
 namespace {
@@ -336,9 +337,7 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
 
     u32x4 v[VPT];
     if (full) {
-#pragma unroll
-        for (int j = 0; j < VPT; ++j)
-            v[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(in + lane_base + j * ROW_ELEMS));
+        wave_load_striped_streaming(reinterpret_cast<const u32x4*>(in + tile_base + static_cast<size_t>(wave) * WAVE_ELEMS), lane, v);
     } else {
 #pragma unroll
         for (int j = 0; j < VPT; ++j) {

@@ -81,6 +81,19 @@ def add_m(x: "torch.Tensor", y: "torch.Tensor", m: int) -> "torch.Tensor":
     return y
 
 
+def wave_regroup(inp: "torch.Tensor", items_per_lane: int, to_striped: bool = True,
+                 out: Optional["torch.Tensor"] = None) -> "torch.Tensor":
+    """Moves every chunk of 64 * items_per_lane int32 between the blocked arrangement of the reference's warp_load
+    (lane l holds items_per_lane consecutive items) and the striped one (item j of lane l is element 64 j + l)."""
+    _need(inp, (torch.int32,), 0, "inp")
+    if out is None:
+        out = torch.empty_like(inp)
+    _need(out, (torch.int32,), inp.numel(), "out")
+    _check(_lib.load().prism_wave_regroup_i32(_ptr(inp), _ptr(out), inp.numel(), int(items_per_lane),
+                                              0 if to_striped else 1, _stream()), "wave_regroup")
+    return out
+
+
 # -------------------------------------------------------------------- scan --
 
 SCAN_EXCLUSIVE = 1       # flag values of include/prism_amd.h

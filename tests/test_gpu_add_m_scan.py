@@ -62,6 +62,34 @@ def test_add_m_unaligned_views_and_wrap(prism, oracle):
     assert host(out)[:3].tolist() == [0, 0, 0]
 
 
+@pytest.mark.parametrize("items", [1, 2, 4, 8, 16])
+def test_wave_regroup_blocked_and_striped(prism, items):
+    """The wave64 warp_load / warp_store primitives through prism_wave_regroup_i32: blocked -> striped is the
+    transpose of every chunk seen as a 64 x items matrix, striped -> blocked its inverse; a partial last chunk
+    counts as one padded with zeros; nothing is read or written beyond n."""
+    for n in (64 * items * 5, 64 * items * 1000 + 64 * items // 2 + 3, 7, 1 << 20):
+        x = np.random.default_rng(n).integers(-2**31, 2**31 - 1, n, dtype=np.int32)
+        chunk = 64 * items
+        whole = n // chunk * chunk
+        want = x.copy()
+        want[:whole] = x[:whole].reshape(-1, 64, items).transpose(0, 2, 1).reshape(-1)
+        tail = n - whole
+        if tail:  # the partial chunk counts as one padded with zeros: position N l + j goes to 64 j + l if that exists
+            src = np.arange(tail)
+            dst = 64 * (src % items) + src // items
+            ok = dst < tail
+            want[whole:] = 0
+            want[whole + dst[ok]] = x[whole + src[ok]]
+        out = torch.full((n + 8,), -7, dtype=torch.int32, device=DEV)
+        prism.wave_regroup(dev(x), items, True, out[:n])
+        got = host(out)
+        assert np.array_equal(got[:n], want) and np.all(got[n:] == -7), (n, items)
+        back = prism.wave_regroup(dev(want[:whole]), items, False)
+        assert np.array_equal(host(back), x[:whole])
+    with pytest.raises(ValueError):
+        prism.wave_regroup(torch.zeros(64, dtype=torch.int32, device=DEV), 3)
+
+
 def test_calibration_streams(prism):
     """prism_calibrate_stream: both copy shapes copy exactly `bytes` bytes and nothing more; the one-way
     kinds run; bad arguments are refused."""
