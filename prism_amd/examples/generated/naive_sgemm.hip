@@ -1,0 +1,30 @@
+__global__ void naive_sgemm(int M, int N, int K, float alpha, const float* A, const float* B, float beta, float* C, int per_block) {
+    extern __shared__ __align__(128) char __smem[];
+    int __block_id_0 = blockIdx.x;
+    int __thread_id_0 = __block_id_0 * blockDim.x + threadIdx.x;
+    int blk = __block_id_0;
+    {
+        float* C_of_block = C + (0);
+        {
+            int __block_id_1 = __block_id_0 % 1;
+            int __thread_id_1 = __block_id_1 * blockDim.x + threadIdx.x;
+            int e = ((blk * per_block) + __thread_id_1);
+            const int row = (e / N);
+            const int col = (e % N);
+            {
+                float* C_mine = C_of_block + (0);
+                {
+                    int __block_id_2 = __block_id_1;
+                    int __thread_id_2 = __thread_id_1 % 1;
+                    if ((e < (M * N))) {
+                        float acc = 0;
+                        for (int k = 0; k < K; k++) {
+                            acc += (A[((row * K) + k)] * B[((k * N) + col)]);
+                        }
+                        C_mine[((row * N) + col)] = ((alpha * acc) + (beta * C_mine[((row * N) + col)]));
+                    }
+                }
+            }
+        }
+    }
+}

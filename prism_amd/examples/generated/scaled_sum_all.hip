@@ -1,0 +1,20 @@
+__global__ void scaled_sum_all(const float* x, float* y, float s, int n) {
+    extern __shared__ __align__(128) char __smem[];
+    int __block_id_0 = blockIdx.x;
+    int __thread_id_0 = __block_id_0 * blockDim.x + threadIdx.x;
+    int i = __thread_id_0;
+    {
+        float* y_one = y + (i);
+        {
+            int __block_id_1 = __block_id_0 % 1;
+            int __thread_id_1 = __block_id_1 * blockDim.x + threadIdx.x;
+            {
+                int __block_id_2 = __block_id_1;
+                int __thread_id_2 = __thread_id_1 % 1;
+                if ((i < n)) {
+                    y_one[0] = scaled_sum(__block_id_2, __thread_id_2, __smem, x[i], y_one[0], s);
+                }
+            }
+        }
+    }
+}

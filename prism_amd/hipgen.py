@@ -97,6 +97,8 @@ def _ctype_text(t) -> str:
     name = getattr(t, "__name__", str(t))
     if name in _SCALARS:
         return _SCALARS[name]
+    if isinstance(t, _TypeName):  # shared(T) inside ptr(...): kernels are compiled from their source text,
+        return name               # these objects only have to let the annotations evaluate
     raise HipgenError(f"unsupported element type {t!r}")
 
 
@@ -401,6 +403,13 @@ def _structured(k: Kernel) -> bool:
     return k.kind == "device" or any(p.level == "block" for p in k.requires)
 
 
+def _check_perspectives(name: str) -> None:
+    """Nothing is printed for a program that moves data against the perspective order
+    (the reference type-checks before it generates, prism/codegen.py:1000-1014)."""
+    from .hipgen_check import check
+    check(name)
+
+
 def generate(name: str, bounded: bool = False, auto_sync: bool = True) -> str:
     """HIP text of kernel `name`.
 
@@ -410,6 +419,7 @@ def generate(name: str, bounded: bool = False, auto_sync: bool = True) -> str:
     covering n is legal. Kernels with a block perspective are printed by hipgen_blocks.generate_blocks
     (auto_sync places the barriers); they carry their own guards, so bounded does not apply."""
     k = _kernel(name)
+    _check_perspectives(name)
     if _structured(k):
         if bounded:
             raise HipgenError("bounded=True applies to thread-level kernels only")
@@ -429,6 +439,7 @@ def generate_launcher(name: str, block_size: int = 256, template: Optional[List[
     if block_size % 64 or not 64 <= block_size <= 1024:
         raise HipgenError("block_size must be a multiple of 64 between 64 and 1024")
     k = _kernel(name)
+    _check_perspectives(name)
     head = "#include <hip/hip_runtime.h>\n#include <cstddef>\n#include <cstdint>\n\n"
     if _structured(k):
         from .hipgen_blocks import BlockEmitter, device_functions_used, generate_blocks

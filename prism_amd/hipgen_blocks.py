@@ -124,7 +124,10 @@ class _Scalar:
         if isinstance(node, ast.Call) and isinstance(node.func, ast.Name) and node.args:
             inner = _Scalar.text(node.args[0])
             if node.func.id == "ptr":
-                return inner if inner.endswith("*") and _is_call(node.args[0], "shared") else inner + "*"
+                # ptr(shared(T)) and ptr(const(shared(T))): shared() already made the pointer
+                a = node.args[0]
+                into_lds = _is_call(a, "shared") or (_is_call(a, "const") and a.args and _is_call(a.args[0], "shared"))
+                return inner if into_lds else inner + "*"
             if node.func.id == "shared":  # ptr(shared(T)): a pointer into LDS is a plain pointer in the text
                 return inner + "*"
             if node.func.id == "const":
@@ -143,6 +146,17 @@ def _annotation(node: ast.AST) -> Tuple[ast.AST, Optional[Tuple[str, int]]]:
     return node, None
 
 
+def _const_pointer_params(name: str) -> Set[int]:
+    """Positions of the parameters of Prism function `name` that are declared `ptr(const(T))`."""
+    fn = ast.parse(_REGISTRY[name].source).body[0]
+    out: Set[int] = set()
+    for i, a in enumerate(x for x in fn.args.args if x.arg != "template"):
+        t = _annotation(a.annotation)[0] if a.annotation is not None else None
+        if _is_call(t, "ptr") and t.args and _is_call(t.args[0], "const"):
+            out.add(i)
+    return out
+
+
 # --------------------------------------------------------------- barrier plan --
 
 class _SyncPlan:
@@ -152,6 +166,10 @@ class _SyncPlan:
         self.before: Set[int] = set()     # id(stmt)
         self.at_end: Set[int] = set()     # id(loop stmt)
         self.root: Dict[str, str] = {}    # LDS array or view of one -> the array
+        for a in fn.args.args:            # a parameter declared ptr(shared(T)) points into LDS (prism/sync_analysis.py:151-158)
+            if a.arg != "template" and a.annotation is not None and any(
+                    _is_call(n, "shared") for n in ast.walk(_annotation(a.annotation)[0])):
+                self.root[a.arg] = a.arg
         self._collect(fn.body)
         self._walk(fn.body, (set(), set()), True)
 
@@ -184,6 +202,21 @@ class _SyncPlan:
                 out.add(self.root[n.id])  # an element read, or the array handed to a function
         return out
 
+    def _handed_over(self, node: Optional[ast.AST]) -> Set[str]:
+        """LDS arrays named as a whole among the arguments of a call of a Prism function: the callee may write
+        them, unless it declares the parameter a pointer to const (the way the reference's consumer takes its
+        tiles, examples/sgemm_kernel_5.py:16-17). An element read (`f(a[i])`) passes a value and is not meant."""
+        out: Set[str] = set()
+        if node is None:
+            return out
+        for n in ast.walk(node):
+            if isinstance(n, ast.Call) and isinstance(n.func, ast.Name) and n.func.id in _REGISTRY:
+                read_only = _const_pointer_params(n.func.id)
+                for i, a in enumerate(n.args):
+                    if isinstance(a, ast.Name) and a.id in self.root and i not in read_only:
+                        out.add(self.root[a.id])
+        return out
+
     def _with_reads(self, s: ast.With) -> Set[str]:
         """A view is pointer arithmetic; only its offset expression can read memory."""
         out: Set[str] = set()
@@ -198,7 +231,7 @@ class _SyncPlan:
     def _access(self, s: ast.stmt) -> Tuple[Set[str], Set[str]]:
         """(reads, writes) of a statement that holds no other statements."""
         if isinstance(s, ast.Assign):
-            r, w = self._reads(s.value), set()
+            r, w = self._reads(s.value), self._handed_over(s.value)
             for t in s.targets:
                 if (isinstance(t, ast.Subscript) and isinstance(t.value, ast.Name) and t.value.id == "float4_cast"
                         and isinstance(t.slice, ast.Subscript)):
@@ -211,16 +244,15 @@ class _SyncPlan:
             return r, w
         if isinstance(s, ast.AugAssign):
             r = self._reads(s.value) | self._reads(s.target)
-            w = set()
+            w = self._handed_over(s.value)
             if isinstance(s.target, ast.Subscript) and isinstance(s.target.value, ast.Name) and s.target.value.id in self.root:
                 w.add(self.root[s.target.value.id])
             return r, w
         if isinstance(s, ast.AnnAssign):
-            return self._reads(s.value), set()
-        if isinstance(s, ast.Expr):
             r = self._reads(s.value)
-            # A call that is handed an LDS array may write it as well.
-            return r, (set(r) if isinstance(s.value, ast.Call) else set())
+            return r, self._handed_over(s.value)
+        if isinstance(s, ast.Expr):
+            return self._reads(s.value), self._handed_over(s.value)
         if isinstance(s, ast.Return):
             return self._reads(s.value), set()
         return set(), set()

@@ -1,9 +1,8 @@
 """The HIP emitter for Prism kernels with block-level structure (prism_amd/hipgen_blocks.py).
 
-The kernels below are written in the reference's surface syntax (block and thread perspectives, views,
-LDS arrays without hand-placed barriers, templates, private arrays, a device function) in the manner of
-its examples (examples/sgemm_kernel_1.py, examples/sgemm_shared_mem_block.py, examples/sgemm_kernel_3.py,
-examples/add_m_block_thread.py, examples/function_call.py; 16-byte accesses as in examples/sgemm_kernel_4.py).
+The programs are the example set under prism_amd/examples (add_m, the SGEMM steps, matrix-instruction kernels,
+the row scan, small one-construct programs), written in the reference's surface syntax; the few kernels defined
+here exist to be refused or to probe one rule of the barrier plan.
 CPU: structure of the printed text (id chain, scopes, LDS declarations, where the barriers land), refusals
 by name, and that every launcher cross-compiles for gfx950.
 GPU: the compiled kernels run through their C launchers; add_m bit for bit against numpy, the SGEMMs
@@ -15,170 +14,39 @@ import numpy as np
 import pytest
 
 from prism_amd import hipgen
-from prism_amd.hipgen import (HipgenError, attr, bf16, block, const, float4, float4_cast, generate, generate_launcher, grid,
-                              group, intrinsic, partition, prism, ptr, requires, shared, split, thread, uint32_t, unsafe)
+from prism_amd.examples import add_m, basics, mfma, scan, sgemm  # noqa: F401  (define the kernels)
+from prism_amd.hipgen import (HipgenError, block, const, generate, generate_launcher, grid, group, intrinsic, partition, prism,
+                              ptr, requires, shared, split, thread)
 from prism_amd.hipgen_blocks import dynamic_lds_bytes
 
 
 @requires(grid[1], block[1], thread[1])
 @prism("global")
-def add_m_blocks(x: ptr(const(int)) @ grid[1], y: ptr(int) @ grid[1], m: int @ grid[1],
-                 per_block: int @ grid[1], n: int @ grid[1]):
-    first: int @ block[1] = id() * per_block
-    with partition(x, p=block[1], offset=first) as x_blk:
-        with partition(y, p=block[1], offset=first) as y_blk:
-            with group(block[1]):
-                lane: int @ thread[1] = id()
-                with partition(x_blk, p=thread[1], offset=lane) as x_one:
-                    with partition(y_blk, p=thread[1], offset=lane) as y_one:
-                        with group(thread[1]):
-                            if first + lane < n:
-                                y_one[0] = x_one[0] + m
-
-
-@requires(grid[1], block[1], thread[1])
-@prism("global")
-def naive_sgemm(M: int @ grid[1], N: int @ grid[1], K: int @ grid[1], alpha: float @ grid[1],
-                A: ptr(const(float)) @ grid[1], B: ptr(const(float)) @ grid[1], beta: float @ grid[1],
-                C: ptr(float) @ grid[1], per_block: int @ grid[1]):
-    blk: int @ block[1] = id()
-    with partition(C, p=block[1], offset=0) as C_of_block:
-        with group(block[1]):
-            e: int @ thread[1] = blk * per_block + id()
-            row: const(int) @ thread[1] = e / N
-            col: const(int) @ thread[1] = e % N
-            with partition(C_of_block, p=thread[1], offset=0) as C_mine:
-                with group(thread[1]):
-                    if e < M * N:
-                        acc: float @ thread[1] = 0
-                        for k in range(K):
-                            acc += A[row * K + k] * B[k * N + col]
-                        C_mine[row * N + col] = alpha * acc + beta * C_mine[row * N + col]
-
-
-@requires(grid[1], block[1], thread[1])
-@prism("global")
-def tiled_sgemm(M: int @ grid[1], N: int @ grid[1], K: int @ grid[1], alpha: float @ grid[1],
-                A: ptr(const(float)) @ grid[1], B: ptr(const(float)) @ grid[1], beta: float @ grid[1],
-                C: ptr(float) @ grid[1], tiles_n: int @ grid[1], template=[("TILE", int)]):
-    tile_r: const(int) @ block[1] = id() / tiles_n
-    tile_c: const(int) @ block[1] = id() % tiles_n
-    with partition(A, p=block[1], offset=tile_r * TILE * K) as A_rows:
-        with partition(B, p=block[1], offset=tile_c * TILE) as B_cols:
-            with partition(C, p=block[1], offset=tile_r * TILE * N + tile_c * TILE) as C_tile:
-                with group(block[1]):
-                    a_lds: shared(float[TILE * TILE], static=True) @ block[1]
-                    b_lds: shared(float[TILE * TILE], static=True) @ block[1]
-                    r: const(int) @ thread[1] = id() / TILE
-                    c: const(int) @ thread[1] = id() % TILE
-                    acc: float @ thread[1] = 0
-                    with group(thread[1]):
-                        for k0 in range(0, K, TILE):
-                            a_lds[r * TILE + c] = A_rows[r * K + k0 + c]
-                            b_lds[r * TILE + c] = B_cols[(k0 + r) * N + c]
-                            for d in range(TILE):
-                                acc += a_lds[r * TILE + d] * b_lds[d * TILE + c]
-                        C_tile[r * N + c] = alpha * acc + beta * C_tile[r * N + c]
-
-
-@attr("__launch_bounds__((BM * BN) / (TM * TN))")
-@requires(grid[1], block[1], thread[1], smem=8192)
-@prism("global")
-def thread_tile_sgemm(M: int @ grid[1], N: int @ grid[1], K: int @ grid[1], alpha: float @ grid[1],
-                      A: ptr(const(float)) @ grid[1], B: ptr(const(float)) @ grid[1], beta: float @ grid[1],
-                      C: ptr(float) @ grid[1], tiles_n: int @ grid[1],
-                      template=[("BM", int), ("BN", int), ("BK", int), ("TM", int), ("TN", int)]):
-    tile_r: const(int) @ block[1] = id() / tiles_n
-    tile_c: const(int) @ block[1] = id() % tiles_n
-    with partition(A, p=block[1], offset=tile_r * BM * K) as A_rows:
-        with partition(B, p=block[1], offset=tile_c * BN) as B_cols:
-            with partition(C, p=block[1], offset=tile_r * BM * N + tile_c * BN) as C_tile:
-                with group(block[1]):
-                    a_lds: shared(float[1024]) @ block[1]
-                    b_lds: shared(float[1024]) @ block[1]
-                    t: const(int) @ thread[1] = id()
-                    threads: const(int) @ thread[1] = (BM * BN) / (TM * TN)
-                    out_r: const(int) @ thread[1] = t / (BN / TN)
-                    out_c: const(int) @ thread[1] = t % (BN / TN)
-                    acc: float[16] @ thread[1] = {0}
-                    a_reg: float[4] @ thread[1] = {0}
-                    b_reg: float[4] @ thread[1] = {0}
-                    for k0 in range(0, K, BK):
-                        with group(thread[1]):
-                            for e in range(t, BM * BK, threads):
-                                a_lds[e] = A_rows[(e / BK) * K + k0 + e % BK]
-                            for e in range(t, BK * BN, threads):
-                                b_lds[e] = B_cols[(k0 + e / BN) * N + e % BN]
-                            for kk in range(BK):
-                                for i in range(TM):
-                                    a_reg[i] = a_lds[(out_r * TM + i) * BK + kk]
-                                for j in range(TN):
-                                    b_reg[j] = b_lds[kk * BN + out_c * TN + j]
-                                for i in range(TM):
-                                    for j in range(TN):
-                                        acc[i * TN + j] += a_reg[i] * b_reg[j]
-                    with group(thread[1]):
-                        for i in range(TM):
-                            for j in range(TN):
-                                C_tile[(out_r * TM + i) * N + out_c * TN + j] = \
-                                    alpha * acc[i * TN + j] + beta * C_tile[(out_r * TM + i) * N + out_c * TN + j]
-
-
-@requires(thread[1])
-@prism("device")
-def scaled_sum(a: float @ thread[1], b: float @ thread[1], s: float @ thread[1]) -> float @ thread[1]:
-    return s * (a + b)
-
-
-@requires(grid[1], block[1], thread[1])
-@prism("global")
-def scaled_sum_all(x: ptr(const(float)) @ grid[1], y: ptr(float) @ grid[1], s: float @ grid[1], n: int @ grid[1]):
-    i: int @ thread[1] = id()  # outside every group: the thread's number in the whole grid
-    with group(block[1]):
-        with group(thread[1]):
-            if i < n:
-                y[i] = scaled_sum(x[i], y[i], s)
-
-
-@requires(grid[1], block[1], thread[1])
-@prism("global")
 def hazard_in_branch(x: ptr(float) @ grid[1]):
-    with group(block[1]):
-        buf: shared(float[64], static=True) @ block[1]
-        t: int @ thread[1] = id()
-        if t < 32:
-            buf[t] = x[t]
-            x[t] = buf[31 - t]
+    with partition(x, p=thread[1], offset=0) as x_mine:
+        with group(block[1]):
+            buf: shared(float[64], static=True) @ block[1]
+            t: int @ thread[1] = id()
+            with partition(buf, p=thread[1], offset=t) as slot:
+                with group(thread[1]):
+                    if t < 32:
+                        slot[0] = x_mine[t]
+                        x_mine[t] = buf[31 - t]
 
 
-@requires(grid[1], block[1], thread[1])
-@prism("global")
-def two_roles(x: ptr(const(int)) @ grid[1], y: ptr(int) @ grid[1], n: int @ grid[1]):
-    """The first 128 threads of a block double their element, the next 128 add one to theirs (the shape of
-    the reference's producer / consumer split, examples/h100_matmul.py:203-206)."""
-    base: int @ block[1] = id() * 256
-    with group(block[1]):
-        match split(thread):
-            case 128:
-                t: int @ thread[1] = id()
-                if base + t < n:
-                    y[base + t] = x[base + t] * 2
-            case 128:
-                t: int @ thread[1] = id()
-                if base + 128 + t < n:
-                    y[base + 128 + t] = x[base + 128 + t] + 1
-
-
-@requires(grid[1], block[1], thread[1])
+@requires(grid[1], block[1], thread[128])
 @prism("global")
 def split_with_hazard(x: ptr(float) @ grid[1]):
-    with group(block[1]):
-        buf: shared(float[256], static=True) @ block[1]
-        match split(thread):
-            case 128:
-                t: int @ thread[1] = id()
-                buf[t] = x[t]
-                x[t] = buf[127 - t]
+    with partition(x, p=thread[1], offset=0) as x_mine:
+        with group(block[1]):
+            buf: shared(float[256], static=True) @ block[1]
+            with partition(buf, p=thread[1], offset=0) as buf_mine:
+                match split(thread):
+                    case 128:
+                        t: int @ thread[1] = id()
+                        with group(thread[1]):
+                            buf_mine[t] = x_mine[t]
+                            x_mine[t] = buf[127 - t]
 
 
 @requires(grid[1], block[1], thread[48])
@@ -189,210 +57,14 @@ def straddling_groups(x: ptr(float) @ grid[1]):
             w: int @ thread[48] = id()
 
 
-@requires(thread[1])
-@prism("device")
-def lane_shift_up(val: uint32_t @ thread[1], delta: uint32_t @ thread[1]) -> uint32_t @ thread[1]:
-    with group(thread[1]):
-        unsafe("return __shfl_up(val, delta, 32);")
-    return
-
-
-@requires(grid[1], block[1], thread[32])
-@prism("global")
-def row_scan32(x: ptr(const(uint32_t)) @ grid[1], y: ptr(uint32_t) @ grid[1], rows: int @ grid[1]):
-    """Inclusive scan of every row of 32 elements by a group of 32 threads (half a wavefront), the
-    building block of the reference's scan (scan_warps, examples/scan.py:106-128)."""
-    first_row: int @ block[1] = id() * 8
-    with partition(x, p=block[1], offset=first_row * 32) as x_blk:
-        with partition(y, p=block[1], offset=first_row * 32) as y_blk:
-            with group(block[1]):
-                g: int @ thread[32] = id()
-                with partition(x_blk, p=thread[32], offset=g * 32) as x_row:
-                    with partition(y_blk, p=thread[32], offset=g * 32) as y_row:
-                        with group(thread[32]):
-                            lane: uint32_t @ thread[1] = id()
-                            with group(thread[1]):
-                                v: uint32_t @ thread[1] = 0
-                                if first_row + g < rows:
-                                    v = x_row[lane]
-                                step: uint32_t @ thread[1] = 1
-                                while step < 32:
-                                    got: uint32_t @ thread[1] = lane_shift_up(v, step)
-                                    if lane >= step:
-                                        v = got + v
-                                    step *= 2
-                                if first_row + g < rows:
-                                    y_row[lane] = v
-
-
-@attr("__launch_bounds__((BM * BN) / (TM * TN))")
-@requires(grid[1], block[1], thread[1], smem=8192)
-@prism("global")
-def vector_tile_sgemm(M: int @ grid[1], N: int @ grid[1], K: int @ grid[1], alpha: float @ grid[1],
-                      A: ptr(float) @ grid[1], B: ptr(float) @ grid[1], beta: float @ grid[1],
-                      C: ptr(float) @ grid[1], tiles_n: int @ grid[1],
-                      template=[("BM", int), ("BN", int), ("BK", int), ("TM", int), ("TN", int)]):
-    """Thread-tile SGEMM with 16-byte global loads and stores; the A tile is stored transposed (BK x BM)
-    through an index-mapped view, so that a K slice of it is contiguous. One packet of A and one of B per
-    thread: BM * BK = BK * BN = 4 * threads."""
-    tile_r: const(int) @ block[1] = id() / tiles_n
-    tile_c: const(int) @ block[1] = id() % tiles_n
-    with partition(A, p=block[1], offset=tile_r * BM * K) as A_rows:
-        with partition(B, p=block[1], offset=tile_c * BN) as B_cols:
-            with partition(C, p=block[1], offset=tile_r * BM * N + tile_c * BN) as C_tile:
-                with group(block[1]):
-                    a_lds: shared(float[1024]) @ block[1]
-                    b_lds: shared(float[1024]) @ block[1]
-                    t: const(int) @ thread[1] = id()
-                    out_r: const(int) @ thread[1] = t / (BN / TN)
-                    out_c: const(int) @ thread[1] = t % (BN / TN)
-                    a_row: const(int) @ thread[1] = t / (BK / 4)
-                    a_quad: const(int) @ thread[1] = t % (BK / 4)
-                    b_row: const(int) @ thread[1] = t / (BN / 4)
-                    b_quad: const(int) @ thread[1] = t % (BN / 4)
-                    acc: float[64] @ thread[1] = {0}
-                    a_reg: float[8] @ thread[1] = {0}
-                    b_reg: float[8] @ thread[1] = {0}
-                    for k0 in range(0, K, BK):
-                        with partition(a_lds, p=thread[1], f=lambda e: (e % BK) * BM + e / BK) as a_by_row:
-                            with group(thread[1]):
-                                quad: float4 @ thread[1] = float4_cast(A_rows[a_row * K + k0 + a_quad * 4])
-                                a_by_row[a_row * BK + a_quad * 4] = quad.x
-                                a_by_row[a_row * BK + a_quad * 4 + 1] = quad.y
-                                a_by_row[a_row * BK + a_quad * 4 + 2] = quad.z
-                                a_by_row[a_row * BK + a_quad * 4 + 3] = quad.w
-                                float4_cast[b_lds[b_row * BN + b_quad * 4]] = \
-                                    float4_cast(B_cols[(k0 + b_row) * N + b_quad * 4])
-                                for kk in range(BK):
-                                    for i in range(TM):
-                                        a_reg[i] = a_lds[kk * BM + out_r * TM + i]
-                                    for j in range(TN):
-                                        b_reg[j] = b_lds[kk * BN + out_c * TN + j]
-                                    for i in range(TM):
-                                        for j in range(TN):
-                                            acc[i * TN + j] += a_reg[i] * b_reg[j]
-                    with group(thread[1]):
-                        for i in range(TM):
-                            for j in range(0, TN, 4):
-                                with partition(C_tile, p=thread[1], offset=(out_r * TM + i) * N + out_c * TN + j) as c4:
-                                    was: float4 @ thread[1] = float4_cast(c4[0])
-                                    was.x = alpha * acc[i * TN + j] + beta * was.x
-                                    was.y = alpha * acc[i * TN + j + 1] + beta * was.y
-                                    was.z = alpha * acc[i * TN + j + 2] + beta * was.z
-                                    was.w = alpha * acc[i * TN + j + 3] + beta * was.w
-                                    float4_cast[c4[0]] = was
-
-
-@requires(grid[1], block[1], thread[1])
-@prism("global")
-def gather_columns(x: ptr(const(int)) @ grid[1], y: ptr(int) @ grid[1], rows: int @ grid[1], cols: int @ grid[1]):
-    """y = x transposed, written through two stacked index-mapped views: `column` picks every cols-th element
-    starting at the thread's column, `shifted` skips its first element; thread c writes column c."""
-    c: int @ thread[1] = id()
-    with partition(x, p=thread[1], f=lambda r: r * cols + c) as column:
-        with partition(column, p=thread[1], f=lambda r: r + 1) as shifted:
-            with partition(y, p=thread[1], offset=c * rows) as mine:
-                with group(block[1]):
-                    with group(thread[1]):
-                        if c < cols:
-                            mine[0] = column[0]
-                            for r in range(rows - 1):
-                                mine[r + 1] = shifted[r]
-
-
 @requires(grid[1], block[1], thread[1])
 @prism("global")
 def view_without_address(x: ptr(int) @ grid[1]):
     with partition(x, p=thread[1], f=lambda i: 2 * i) as evens:
-        with partition(evens, p=thread[1], offset=4) as later:
-            later[0] = 1
-
-
-@requires(thread[1])
-@prism("device")
-def lane_load(src: ptr(const(int)) @ thread[1], dst: ptr(int) @ thread[1], items: int @ thread[1]):
-    with group(thread[1]):
-        for i in range(items):
-            dst[i] = src[i]
-
-
-@requires(thread[1])
-@prism("device")
-def lane_store(src: ptr(const(int)) @ thread[1], dst: ptr(int) @ thread[1], items: int @ thread[1]):
-    with group(thread[1]):
-        for i in range(items):
-            dst[i] = src[i]
-
-
-@requires(thread[64])
-@prism("device")
-def wave_load(src: ptr(const(int)) @ thread[64], dst: ptr(int) @ thread[1], items: int @ thread[64]):
-    """Blocked arrangement: lane l of the wavefront takes items l * items .. l * items + items - 1 of the
-    wavefront's range (the reference's warp_load, examples/warp_load.py:13-22, on 64 lanes)."""
-    with group(thread[64]):
-        lane: int @ thread[1] = id()
-        with partition(src, p=thread[1], offset=lane * items) as mine:
+        with group(block[1]):
             with group(thread[1]):
-                lane_load(mine, dst, items)
-
-
-@requires(thread[64])
-@prism("device")
-def wave_store(src: ptr(const(int)) @ thread[1], dst: ptr(int) @ thread[64], items: int @ thread[64]):
-    with group(thread[64]):
-        lane: int @ thread[1] = id()
-        with partition(dst, p=thread[1], offset=lane * items) as mine:
-            with group(thread[1]):
-                lane_store(src, mine, items)
-
-
-@requires(grid[1], block[1], thread[64])
-@prism("global")
-def add_m_by_wavefronts(x: ptr(const(int)) @ grid[1], y: ptr(int) @ grid[1], m: int @ grid[1], wavefronts: int @ grid[1]):
-    """Every wavefront loads 64 x 4 consecutive elements into registers, adds m and stores them."""
-    w: int @ thread[64] = id()
-    with partition(x, p=thread[64], offset=w * 256) as x_wave:
-        with partition(y, p=thread[64], offset=w * 256) as y_wave:
-            with group(block[1]):
-                with group(thread[64]):
-                    held: int[4] @ thread[1]
-                    if w < wavefronts:
-                        wave_load(x_wave, held, 4)
-                        for i in range(4):
-                            held[i] += m
-                        wave_store(held, y_wave, 4)
-
-
-@requires(grid[1], block[1], thread[64])
-@prism("global")
-def one_mfma_per_wavefront(A: ptr(const(float)) @ grid[1], B: ptr(const(float)) @ grid[1], C: ptr(float) @ grid[1],
-                           M: int @ grid[1], N: int @ grid[1], K: int @ grid[1]):
-    """C = A B with one wavefront per 16 x 16 tile of C and one 16x16x4 fp32 MFMA per K step of 4, operands
-    straight from global memory (the teaching kernel of examples/mmaTF32NaiveKernel.py:14-85, for whole tiles)."""
-    tiles_n: const(int) @ grid[1] = N / 16
-    w: const(int) @ thread[64] = id()
-    tile_r: const(int) @ thread[64] = w / tiles_n
-    tile_c: const(int) @ thread[64] = w % tiles_n
-    with partition(A, p=thread[64], offset=tile_r * 16 * K) as A_rows:
-        with partition(B, p=thread[64], offset=tile_c * 16) as B_cols:
-            with partition(C, p=thread[64], offset=tile_r * 16 * N + tile_c * 16) as C_tile:
-                with group(block[1]):
-                    with group(thread[64]):
-                        lane: const(int) @ thread[1] = id()
-                        r: const(int) @ thread[1] = lane % 16
-                        q: const(int) @ thread[1] = lane / 16
-                        c0: float @ thread[1] = 0
-                        c1: float @ thread[1] = 0
-                        c2: float @ thread[1] = 0
-                        c3: float @ thread[1] = 0
-                        if w < (M / 16) * tiles_n:
-                            for k0 in range(0, K, 4):
-                                intrinsic.mfma_f32_16x16x4_f32(A_rows[r * K + k0 + q], B_cols[(k0 + q) * N + r],
-                                                               c0, c1, c2, c3, out=[c0, c1, c2, c3])
-                            C_tile[(4 * q + 0) * N + r] = c0
-                            C_tile[(4 * q + 1) * N + r] = c1
-                            C_tile[(4 * q + 2) * N + r] = c2
-                            C_tile[(4 * q + 3) * N + r] = c3
+                with partition(evens, p=thread[1], offset=4) as later:
+                    later[0] = 1
 
 
 @requires(grid[1], block[1], thread[64])
@@ -402,83 +74,19 @@ def foreign_instruction(x: ptr(float) @ grid[1]):
     intrinsic.mma(a, a, a, a, a, a, a, a, a, a, out=[a, a, a, a])
 
 
-@requires(grid[1], block[1], thread[64])
+@requires(grid[1], block[1], thread[1])
 @prism("global")
-def one_bf16_mfma_per_wavefront(P: ptr(const(bf16)) @ grid[1], Q: ptr(const(bf16)) @ grid[1], D: ptr(float) @ grid[1],
-                                M: int @ grid[1], N: int @ grid[1], K: int @ grid[1]):
-    """D = P Q^T (P is M x K, Q is N x K, both bf16 with K contiguous: the operand layout of
-    examples/h100_matmul.py) with one wavefront per 16 x 16 tile of D and one 16x16x32 bf16 MFMA per K step of
-    32; every lane fetches 16-byte packets of eight bf16 straight from global memory."""
-    tiles_n: const(int) @ grid[1] = N / 16
-    w: const(int) @ thread[64] = id()
-    tile_r: const(int) @ thread[64] = w / tiles_n
-    tile_c: const(int) @ thread[64] = w % tiles_n
-    with partition(P, p=thread[64], offset=tile_r * 16 * K) as P_rows:
-        with partition(Q, p=thread[64], offset=tile_c * 16 * K) as Q_rows:
-            with partition(D, p=thread[64], offset=tile_r * 16 * N + tile_c * 16) as D_tile:
-                with group(block[1]):
-                    with group(thread[64]):
-                        lane: const(int) @ thread[1] = id()
-                        r: const(int) @ thread[1] = lane % 16
-                        q: const(int) @ thread[1] = lane / 16
-                        c0: float @ thread[1] = 0
-                        c1: float @ thread[1] = 0
-                        c2: float @ thread[1] = 0
-                        c3: float @ thread[1] = 0
-                        if w < (M / 16) * tiles_n:
-                            for k0 in range(0, K, 32):
-                                a: float4 @ thread[1] = float4_cast(P_rows[r * K + k0 + 8 * q])
-                                b: float4 @ thread[1] = float4_cast(Q_rows[r * K + k0 + 8 * q])
-                                intrinsic.mfma_f32_16x16x32_bf16(a, b, c0, c1, c2, c3, out=[c0, c1, c2, c3])
-                            D_tile[(4 * q + 0) * N + r] = c0
-                            D_tile[(4 * q + 1) * N + r] = c1
-                            D_tile[(4 * q + 2) * N + r] = c2
-                            D_tile[(4 * q + 3) * N + r] = c3
-
-
-@attr("__launch_bounds__(256)")
-@requires(grid[1], block[1], thread[64])
-@prism("global")
-def mfma_tile_sgemm(M: int @ grid[1], N: int @ grid[1], K: int @ grid[1], alpha: float @ grid[1],
-                    A: ptr(const(float)) @ grid[1], B: ptr(const(float)) @ grid[1], beta: float @ grid[1],
-                    C: ptr(float) @ grid[1], tiles_n: int @ grid[1]):
-    """C = alpha A B + beta C with 64 x 64 x 8 tiles staged in LDS and the product on fp32 MFMA: four wavefronts
-    per workgroup, each owning a 32 x 32 corner in sixteen accumulators, one 32x32x2 instruction per pair of k
-    values (the wave-level tiling of examples/sgemm_kernel_5.py with the matrix instruction in place of its
-    per-thread loops). A is stored k-major so that both operands are read along a row of LDS."""
-    tile_r: const(int) @ block[1] = id() / tiles_n
-    tile_c: const(int) @ block[1] = id() % tiles_n
-    with partition(A, p=block[1], offset=tile_r * 64 * K) as A_rows:
-        with partition(B, p=block[1], offset=tile_c * 64) as B_cols:
-            with partition(C, p=block[1], offset=tile_r * 64 * N + tile_c * 64) as C_tile:
-                with group(block[1]):
-                    a_lds: shared(float[512], static=True) @ block[1]
-                    b_lds: shared(float[512], static=True) @ block[1]
-                    t: const(int) @ thread[1] = id()
-                    wave: const(int) @ thread[64] = id()
-                    corner_r: const(int) @ thread[64] = (wave / 2) * 32
-                    corner_c: const(int) @ thread[64] = (wave % 2) * 32
-                    with group(thread[64]):
-                        lane: const(int) @ thread[1] = id()
-                        r: const(int) @ thread[1] = lane % 32
-                        q: const(int) @ thread[1] = lane / 32
-                        acc: float[16] @ thread[1] = {0}
-                        with group(thread[1]):
-                            for k0 in range(0, K, 8):
-                                for e in range(t, 512, 256):
-                                    a_lds[(e % 8) * 64 + e / 8] = A_rows[(e / 8) * K + k0 + e % 8]
-                                    b_lds[e] = B_cols[(k0 + e / 64) * N + e % 64]
-                                for kk in range(0, 8, 2):
-                                    intrinsic.mfma_f32_32x32x2_f32(
-                                        a_lds[(kk + q) * 64 + corner_r + r], b_lds[(kk + q) * 64 + corner_c + r],
-                                        acc[0], acc[1], acc[2], acc[3], acc[4], acc[5], acc[6], acc[7],
-                                        acc[8], acc[9], acc[10], acc[11], acc[12], acc[13], acc[14], acc[15],
-                                        out=[acc[0], acc[1], acc[2], acc[3], acc[4], acc[5], acc[6], acc[7],
-                                             acc[8], acc[9], acc[10], acc[11], acc[12], acc[13], acc[14], acc[15]])
-                            for v in range(16):
-                                with partition(C_tile, p=thread[1],
-                                               offset=(corner_r + 8 * (v / 4) + 4 * q + v % 4) * N + corner_c + r) as c:
-                                    c[0] = alpha * acc[v] + beta * c[0]
+def two_readers(x: ptr(const(float)) @ grid[1], y: ptr(float) @ grid[1], template=[("BM", int), ("BN", int), ("BK", int)]):
+    """One fill, then two calls that take the tiles as pointers to const: a barrier in front of the first only."""
+    with partition(x, p=block[1], offset=0) as x_blk:
+        with group(block[1]):
+            a_lds: shared(float[1024], static=True) @ block[1]
+            b_lds: shared(float[1024], static=True) @ block[1]
+            acc: float[16] @ thread[1] = {0}
+            stage_tiles(BN, BK, x_blk, x_blk, a_lds, b_lds, template=[BM, BN, BK, 256])
+            multiply_tiles(acc, a_lds, b_lds, 0, 0, template=[BM, BN, BK, 4, 4])
+            multiply_tiles(acc, b_lds, a_lds, 0, 0, template=[BM, BN, BK, 4, 4])
+            stage_tiles(BN, BK, x_blk, x_blk, a_lds, b_lds, template=[BM, BN, BK, 256])
 
 
 def lines(text):
@@ -521,10 +129,11 @@ def test_barriers_of_the_lds_tiled_kernel():
     assert "__shared__ float a_lds[(TILE * TILE)];" in got and "__shared__ float b_lds[(TILE * TILE)];" in got
     assert got.count("__syncthreads();") == 2
     first = got.index("__syncthreads();")
-    assert got[first - 1].startswith("b_lds[") and got[first + 1] == "for (int d = 0; d < TILE; d++) {"
+    assert got[first - 1].startswith("b_mine[") and got[first + 1] == "for (int d = 0; d < TILE; d++) {"
     second = got.index("__syncthreads();", first + 1)
-    assert got[second - 1] == "}" and got[second + 1] == "}"          # closes the d loop, then the k0 loop
-    assert got[second + 2].startswith("C_tile[")
+    # the d loop, the thread group and the two views close; the barrier is the last statement of the k0 loop
+    assert got[second - 4:second] == ["}"] * 4 and got[second + 1] == "}"
+    assert got[second + 3].startswith("float* C_mine = C_tile + ")
     assert "for (int k0 = 0; k0 < K; k0 += TILE) {" in got
     assert "__syncthreads();" not in lines(generate("tiled_sgemm", auto_sync=False))
 
@@ -534,14 +143,17 @@ def test_barriers_of_the_lds_tiled_kernel():
 def maybe_no_trips(x: ptr(const(int)) @ grid[1], y: ptr(int) @ grid[1], trips: int @ grid[1]):
     a: shared(int[64], static=True) @ block[1]
     b: shared(int[64], static=True) @ block[1]
-    with group(block[1]):
-        t: int @ thread[1] = id()
-        with group(thread[1]):
-            a[t] = x[t]
-            for i in range(trips):
-                b[t] = i
-                y[t] = b[63 - t]
-            y[t] = a[63 - t]
+    with partition(y, p=thread[1], offset=0) as y_mine:
+        with group(block[1]):
+            t: int @ thread[1] = id()
+            with partition(a, p=thread[1], offset=t) as a_one:
+                with partition(b, p=thread[1], offset=t) as b_one:
+                    with group(thread[1]):
+                        a_one[0] = x[t]
+                        for i in range(trips):
+                            b_one[0] = i
+                            y_mine[t] = b[63 - t]
+                        y_mine[t] = a[63 - t]
 
 
 @requires(grid[1], block[1], thread[1])
@@ -549,14 +161,17 @@ def maybe_no_trips(x: ptr(const(int)) @ grid[1], y: ptr(int) @ grid[1], trips: i
 def surely_some_trips(x: ptr(const(int)) @ grid[1], y: ptr(int) @ grid[1]):
     a: shared(int[64], static=True) @ block[1]
     b: shared(int[64], static=True) @ block[1]
-    with group(block[1]):
-        t: int @ thread[1] = id()
-        with group(thread[1]):
-            a[t] = x[t]
-            for i in range(3):
-                b[t] = i
-                y[t] = b[63 - t]
-            y[t] = a[63 - t]
+    with partition(y, p=thread[1], offset=0) as y_mine:
+        with group(block[1]):
+            t: int @ thread[1] = id()
+            with partition(a, p=thread[1], offset=t) as a_one:
+                with partition(b, p=thread[1], offset=t) as b_one:
+                    with group(thread[1]):
+                        a_one[0] = x[t]
+                        for i in range(3):
+                            b_one[0] = i
+                            y_mine[t] = b[63 - t]
+                        y_mine[t] = a[63 - t]
 
 
 def test_a_loop_that_may_not_run_keeps_what_was_pending_in_front_of_it():
@@ -565,12 +180,38 @@ def test_a_loop_that_may_not_run_keeps_what_was_pending_in_front_of_it():
     read needs a barrier of its own behind the loop. With a literal trip count of at least one the
     barriers inside the loop are sure to run and order the write of `a` as well: no third barrier."""
     got = lines(generate("maybe_no_trips"))
-    read = got.index("y[t] = a[(63 - t)];")
+    read = got.index("y_mine[t] = a[(63 - t)];")
     assert got[read - 1] == "__syncthreads();" and got[read - 2] == "}"
     assert got.count("__syncthreads();") == 3
     got = lines(generate("surely_some_trips"))
-    read = got.index("y[t] = a[(63 - t)];")
+    read = got.index("y_mine[t] = a[(63 - t)];")
     assert got[read - 1] == "}" and got.count("__syncthreads();") == 2
+
+
+def test_barriers_between_device_functions_that_are_handed_the_tiles():
+    """Filling call, barrier, reading call, and a barrier as the last statement of the K loop's body: where the
+    reference prints them for its kernel 5 (generated/my_sgemm_kernel_5.cu:40-46). What a call does to an LDS
+    array it is handed is read off the callee's signature: a pointer to const is only read, any other pointer
+    may be written (prism/sync_analysis.py:871-877)."""
+    got = lines(generate("staged_sgemm"))
+    assert got[0] == "template<int BM, int BN, int BK, int TM, int TN, int THREADS>"
+    fill = got.index("stage_tiles<BM, BN, BK, THREADS>(__block_id_1, __thread_id_1, __smem, N, K, A_now, B_now, a_lds, b_lds);")
+    assert got[fill + 1] == "__syncthreads();"
+    assert got[fill + 2] == ("multiply_tiles<BM, BN, BK, TM, TN>(__block_id_1, __thread_id_1, __smem, acc, a_lds, b_lds, "
+                             "out_r, out_c);")
+    assert got[fill + 3:fill + 7] == ["}", "}", "__syncthreads();", "}"]   # the two views close, barrier, the loop closes
+    assert got.count("__syncthreads();") == 2
+    # the callees' own text: stores through thread[1] views of the pointer parameters, no barrier of their own
+    filler = lines(generate("stage_tiles"))
+    assert filler[0] == "template<int BM, int BN, int BK, int THREADS>"
+    assert filler[1] == ("__device__ void stage_tiles(int __block_id, int __thread_id, char* __smem, int N, int K, "
+                         "const float* A_from, const float* B_from, float* a_tile, float* b_tile) {")
+    assert "float* a_mine = a_tile + (0);" in filler and "__syncthreads();" not in filler
+    # two readers in a row need nothing between them; the fill behind them does
+    got = lines(generate("two_readers"))
+    calls = [n for n, ln in enumerate(got) if ln.startswith(("stage_tiles<", "multiply_tiles<"))]
+    sync = [n for n, ln in enumerate(got) if ln == "__syncthreads();"]
+    assert len(calls) == 4 and sync == [calls[0] + 1, calls[3] - 1] and calls[2] == calls[1] + 1
 
 
 def test_dynamic_lds_windows_private_arrays_and_attr():
@@ -663,7 +304,7 @@ def test_device_function_gets_the_callers_ids():
     assert helper[1:3] == ["int __block_id_0 = __block_id;", "int __thread_id_0 = __thread_id;"]
     assert "return (s * (a + b));" in helper
     caller = generate("scaled_sum_all")
-    assert "y[i] = scaled_sum(__block_id_2, __thread_id_2, __smem, x[i], y[i], s);" in caller
+    assert "y_one[0] = scaled_sum(__block_id_2, __thread_id_2, __smem, x[i], y_one[0], s);" in caller
     launcher = generate_launcher("scaled_sum_all")
     assert launcher.index("__device__ float scaled_sum(") < launcher.index("__global__ void scaled_sum_all(")
 
@@ -675,7 +316,7 @@ def test_split_restarts_ids_in_every_case():
     assert got[i + 1] == "if (__thread_id_2 >= 0 && __thread_id_2 < 128) {" and got[i + 2] == "int t = __thread_id_2;"
     k = got.index("int __thread_id_2 = __thread_id_1 - 128;")
     assert got[k + 1] == "if (__thread_id_2 >= 0 && __thread_id_2 < 128) {" and k > i
-    assert "y[((base + 128) + t)] = (x[((base + 128) + t)] + 1);" in got
+    assert "y_mine[(128 + t)] = (x[((base + 128) + t)] + 1);" in got
     with pytest.raises(HipgenError, match="inside one `if`"):
         generate("split_with_hazard")  # a barrier inside a case would not be reached by the other threads
 
@@ -707,7 +348,8 @@ BUILDS = {"two_roles": (256, None), "row_scan32": (256, None), "add_m_blocks": (
           "thread_tile_sgemm": (256, [64, 64, 8, 4, 4]), "scaled_sum_all": (256, None),
           "vector_tile_sgemm": (256, [128, 128, 8, 8, 8]), "gather_columns": (256, None),
           "add_m_by_wavefronts": (256, None), "one_mfma_per_wavefront": (256, None),
-          "one_bf16_mfma_per_wavefront": (256, None), "mfma_tile_sgemm": (256, None)}
+          "one_bf16_mfma_per_wavefront": (256, None), "mfma_tile_sgemm": (256, None),
+          "staged_sgemm": (256, [64, 64, 8, 4, 4, 256])}
 
 
 @pytest.fixture(scope="module")
@@ -780,6 +422,14 @@ def test_generated_lds_tiled_sgemm(built, oracle, shape):
 def test_generated_thread_tile_sgemm(built, oracle, shape):
     M, N, K = shape
     run_sgemm(built["thread_tile_sgemm"], "thread_tile_sgemm", oracle, M, N, K, N // 64, (M // 64) * (N // 64))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(64, 64, 8), (128, 192, 72), (256, 64, 256)])
+def test_generated_sgemm_staged_by_device_functions(built, oracle, shape):
+    """The tiles are filled and read by device functions; the barriers around the calls make it right."""
+    M, N, K = shape
+    run_sgemm(built["staged_sgemm"], "staged_sgemm", oracle, M, N, K, N // 64, (M // 64) * (N // 64))
 
 
 @pytest.mark.gpu
