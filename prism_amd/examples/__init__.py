@@ -31,6 +31,7 @@ KERNELS: Dict[str, Tuple[str, int, Optional[List[int]]]] = {
     "scaled_sum_all": ("basics", 256, None),
     "two_roles": ("basics", 256, None),
     "gather_columns": ("basics", 256, None),
+    "handed_over_gemm": ("handover", 320, None),
 }
 # device functions, printed on their own as well (the reference prints its scan's helpers one file each)
 DEVICE_FUNCTIONS: Dict[str, str] = {

@@ -146,6 +146,11 @@ def _annotation(node: ast.AST) -> Tuple[ast.AST, Optional[Tuple[str, int]]]:
     return node, None
 
 
+def _is_intrinsic(node: ast.AST, name: str) -> bool:
+    return (isinstance(node, ast.Call) and isinstance(node.func, ast.Attribute) and node.func.attr == name
+            and isinstance(node.func.value, ast.Name) and node.func.value.id == "intrinsic")
+
+
 def _const_pointer_params(name: str) -> Set[int]:
     """Positions of the parameters of Prism function `name` that are declared `ptr(const(T))`."""
     fn = ast.parse(_REGISTRY[name].source).body[0]
@@ -166,11 +171,18 @@ class _SyncPlan:
         self.before: Set[int] = set()     # id(stmt)
         self.at_end: Set[int] = set()     # id(loop stmt)
         self.root: Dict[str, str] = {}    # LDS array or view of one -> the array
+        # hand-over of LDS arrays between the cases of a split (see _plan_handovers)
+        self.declared_here: Set[str] = set()                       # LDS arrays declared in this function's body
+        self.handed: Dict[str, Tuple[int, int]] = {}               # array -> (writing wavefronts, reading wavefronts)
+        self.covered: Dict[int, Set[str]] = {}                     # id(match) -> arrays handed over inside it
+        self.wait_before: Dict[int, List[Tuple[str, str]]] = {}    # id(stmt) -> [(array, "full" | "empty")]
+        self.signal_after: Dict[int, List[Tuple[str, str]]] = {}
         for a in fn.args.args:            # a parameter declared ptr(shared(T)) points into LDS (prism/sync_analysis.py:151-158)
             if a.arg != "template" and a.annotation is not None and any(
                     _is_call(n, "shared") for n in ast.walk(_annotation(a.annotation)[0])):
                 self.root[a.arg] = a.arg
         self._collect(fn.body)
+        self._plan_handovers(fn.body)
         self._walk(fn.body, (set(), set()), True)
 
     def _collect(self, stmts: List[ast.stmt]) -> None:
@@ -179,6 +191,7 @@ class _SyncPlan:
                 t, _ = _annotation(s.annotation)
                 if _is_call(t, "shared"):
                     self.root[s.target.id] = s.target.id
+                    self.declared_here.add(s.target.id)
             elif isinstance(s, ast.With):
                 call = s.items[0].context_expr
                 target = s.items[0].optional_vars
@@ -252,6 +265,11 @@ class _SyncPlan:
             r = self._reads(s.value)
             return r, self._handed_over(s.value)
         if isinstance(s, ast.Expr):
+            if _is_intrinsic(s.value, "load_to_lds") and len(s.value.args) == 2:
+                dst, src = s.value.args   # the destination element is written, its index and the source are read
+                w = {self.root[dst.value.id]} if (isinstance(dst, ast.Subscript) and isinstance(dst.value, ast.Name)
+                                                  and dst.value.id in self.root) else set()
+                return self._reads(src) | self._reads(getattr(dst, "slice", None)), w
             return self._reads(s.value), self._handed_over(s.value)
         if isinstance(s, ast.Return):
             return self._reads(s.value), set()
@@ -277,6 +295,57 @@ class _SyncPlan:
             r |= a
             w |= b
         return r, w
+
+    def _plan_handovers(self, stmts: List[ast.stmt]) -> None:
+        """An LDS array that one case of `match split(thread)` writes and other cases read is handed from case
+        to case: the writing wavefronts wait until the array is empty, fill it and signal that it is full; the
+        reading wavefronts wait until it is full, read it and signal that it is empty (the reference's split
+        barriers, prism/sync_analysis.py:500-570, which it lowers to mbarrier arrive / wait; here the two
+        sides count rounds in two LDS words per array). In each case the wait goes in front of the first
+        statement that touches the array and the signal behind the last one, in the innermost statement list
+        that `with` scopes alone lead to. No workgroup
+        barrier is involved, so a writer may run as many arrays ahead of the readers as there are arrays."""
+        for s in stmts:
+            if isinstance(s, ast.Match) and _is_call(s.subject, "split") and s.subject.args \
+                    and isinstance(s.subject.args[0], ast.Name) and s.subject.args[0].id == "thread":
+                access = [self._whole(c.body) for c in s.cases]
+                counts = [c.pattern.value.value if isinstance(c.pattern, ast.MatchValue)
+                          and isinstance(c.pattern.value, ast.Constant) else 0 for c in s.cases]
+                for array in sorted(set().union(*(r | w for r, w in access))):
+                    writers = [i for i, (_, w) in enumerate(access) if array in w]
+                    readers = [i for i, (r, w) in enumerate(access) if array in r and array not in w]
+                    if len(writers) > 1 and any(array in r for r, _ in access):
+                        raise HipgenError(f"{_line(s)}: {array} is written by more than one case of the split and read "
+                                          "in it: a hand-over has one writing case")
+                    if not writers or not readers:
+                        continue
+                    if array in self.handed:
+                        raise HipgenError(f"{_line(s)}: {array} is already handed over in another split")
+                    if array not in self.declared_here:
+                        raise HipgenError(f"{_line(s)}: {array} is handed from case to case but declared elsewhere; its "
+                                          "round counters live beside its declaration")
+                    involved = writers + readers
+                    if any(counts[i] <= 0 or counts[i] % 64 for i in involved):
+                        raise HipgenError(f"{_line(s)}: {array} is handed from case to case; those cases must be whole "
+                                          "wavefronts (multiples of 64 threads)")
+                    self.handed[array] = (counts[writers[0]] // 64, sum(counts[i] for i in readers) // 64)
+                    self.covered.setdefault(id(s), set()).add(array)
+                    for i in involved:
+                        body = s.cases[i].body
+                        while True:   # through `with` scopes (every thread of the case runs them), not into loops or branches
+                            touching = [t for t in body if array in set().union(*self._whole([t]))]
+                            if len(touching) == 1 and isinstance(touching[0], ast.With):
+                                body = touching[0].body
+                            else:
+                                break
+                        wait, signal = ("empty", "full") if i in writers else ("full", "empty")
+                        self.wait_before.setdefault(id(touching[0]), []).append((array, wait))
+                        self.signal_after.setdefault(id(touching[-1]), []).append((array, signal))
+            for field in ("body", "orelse"):
+                self._plan_handovers(getattr(s, field, []) or [])
+            if isinstance(s, ast.Match):
+                for case in s.cases:
+                    self._plan_handovers(case.body)
 
     @staticmethod
     def _hazard(r: Set[str], w: Set[str], pending: Tuple[Set[str], Set[str]]) -> bool:
@@ -376,7 +445,8 @@ class _SyncPlan:
                     "barrier" if id(s) in self.at_end and self._runs_at_least_once(s) else "none")
             elif isinstance(s, (ast.If, ast.Match)):
                 r, w = self._whole([s])
-                got = "hazard" if self._hazard(r, w, pending) else "none"
+                flagged = self.covered.get(id(s), set())  # ordered from round to round by their full / empty words
+                got = "hazard" if self._hazard(r - flagged, w - flagged, pending) else "none"
             else:
                 r, w = self._access(s)
                 got = "hazard" if self._hazard(r, w, pending) else "none"
@@ -511,7 +581,11 @@ class BlockEmitter:
         for s in stmts:
             if self.plan is not None and id(s) in self.plan.before:
                 self.emit("__syncthreads();")
+            for array, what in (self.plan.wait_before.get(id(s), []) if self.plan is not None else []):
+                self.wait_for(array, what)
             self.stmt(s)
+            for array, what in (self.plan.signal_after.get(id(s), []) if self.plan is not None else []):
+                self.signal(array, what)
 
     def stmt(self, s: ast.stmt) -> None:
         if isinstance(s, ast.AnnAssign) and isinstance(s.target, ast.Name):
@@ -570,8 +644,41 @@ class BlockEmitter:
             return self.emit(f"{self.expr(s.value)};")
         raise HipgenError(f"{_line(s)}: unsupported statement {type(s).__name__}")
 
+    # -- hand-over of an LDS array between the cases of a split: two words per array count the rounds
+    HANDOVER_SPINS = 1 << 16   # a wait gives up after this many polls (milliseconds; a real wait takes microseconds), so that a broken protocol cannot hang the GPU
+
+    def wait_for(self, array: str, what: str) -> None:
+        writers, readers = self.plan.handed[array]
+        need = f"(__round_{array} + 1) * {writers}" if what == "full" else f"__round_{array} * {readers}"
+        self.emit(f"for (int __spin = 0; __spin < {self.HANDOVER_SPINS} && __hip_atomic_load(&__{what}_{array}, "
+                  f"__ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>({need}); ++__spin) "
+                  "__builtin_amdgcn_s_sleep(1);")
+        self.emit('__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");')
+
+    def signal(self, array: str, what: str) -> None:
+        # every memory operation of the wavefront is complete (direct-to-LDS loads count as vector memory
+        # operations), then one lane counts the wavefront in
+        self.emit("__builtin_amdgcn_s_waitcnt(0);")
+        self.emit('__builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");')
+        self.emit(f"if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__{what}_{array}, 1u, __ATOMIC_RELAXED, "
+                  "__HIP_MEMORY_SCOPE_WORKGROUP);")
+        self.emit(f"__round_{array} += 1;")
+
+    def load_to_lds(self, n: ast.Call) -> None:
+        """`intrinsic.load_to_lds(dst[i], src[j])`: the wavefront copies 64 x 16 bytes from global memory into LDS
+        without staging registers: lane l's 16 bytes at &src[j] (j is the lane's own) land at &dst[i] + 16 l
+        (i is the same for the whole wavefront). The counterpart of the reference's asynchronous tile load
+        (load_tma, examples/h100_helpers.py); completion is what the hand-over's signal waits for."""
+        if len(n.args) != 2 or n.keywords or not all(isinstance(a, ast.Subscript) for a in n.args):
+            raise HipgenError(f"{_line(n)}: intrinsic.load_to_lds(dst[i], src[j])")
+        dst, src = self.expr(n.args[0]), self.expr(n.args[1])
+        self.emit(f"__builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&{src}), "
+                  f"(__attribute__((address_space(3))) void*)(&{dst}), 16, 0, 0);")
+
     def matrix_instruction(self, n: ast.Call) -> None:
         name = n.func.attr
+        if name == "load_to_lds":
+            return self.load_to_lds(n)
         if name not in _MFMA:
             raise HipgenError(f"{_line(n)}: intrinsic.{name} is not an instruction of this target "
                               f"(available: {', '.join(sorted(_MFMA))})")
@@ -719,13 +826,20 @@ class BlockEmitter:
                 raise HipgenError(f"{_line(t)}: shared() takes align= and static=")
         self.pointer_type[name] = ctype + "*"
         if static:
-            return self.emit(f"__shared__ {f'__align__({align}) ' if align else ''}{ctype} {name}[{size}];")
-        count = self.constant(arg.slice)
-        if align:
-            self.smem_offset = (self.smem_offset + align - 1) // align * align
-        self.emit(f"{f'__align__({align}) ' if align else ''}{ctype} (&{name})[{size}] = "
-                  f"*(({ctype} (*)[{size}])(__smem + {self.smem_offset}));")
-        self.smem_offset += count * nbytes
+            self.emit(f"__shared__ {f'__align__({align}) ' if align else ''}{ctype} {name}[{size}];")
+        else:
+            count = self.constant(arg.slice)
+            if align:
+                self.smem_offset = (self.smem_offset + align - 1) // align * align
+            self.emit(f"{f'__align__({align}) ' if align else ''}{ctype} (&{name})[{size}] = "
+                      f"*(({ctype} (*)[{size}])(__smem + {self.smem_offset}));")
+            self.smem_offset += count * nbytes
+        if self.plan is not None and name in self.plan.handed:
+            # the array is handed between the cases of a split: its two round counters, cleared before anyone waits
+            self.emit(f"__shared__ unsigned int __full_{name}, __empty_{name};")
+            self.emit(f"int __round_{name} = 0;")
+            self.emit(f"if (threadIdx.x == 0) {{ __full_{name} = 0; __empty_{name} = 0; }}")
+            self.emit("__syncthreads();")
 
     def constant(self, n: ast.AST) -> int:
         """Element count of a dynamic LDS window: it fixes the next window's offset, so it must be a number."""

@@ -1,0 +1,150 @@
+"""LDS arrays handed between the cases of `match split(thread)` (prism_amd/hipgen_blocks.py, _plan_handovers) and the
+producer / consumer GEMM built on it (prism_amd/examples/handover.py).
+
+CPU: where the waits and signals land in each case, the round arithmetic, that the K loop carries no workgroup
+barrier, and what is refused. GPU: the kernel against the fp64 oracle of the bf16 GEMM (1e-3 of the largest
+|element|, the tolerance of the library's own bf16 kernel; sums are fp32).
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+from prism_amd import hipgen
+from prism_amd.examples import handover  # noqa: F401  (defines the kernel)
+from prism_amd.hipgen import HipgenError, block, claim, generate, grid, group, intrinsic, partition, prism, ptr, requires, shared, split, thread
+
+
+def lines(text):
+    return [ln.strip() for ln in text.splitlines()]
+
+
+def test_waits_and_signals_of_the_producer_consumer_gemm():
+    got = lines(generate("handed_over_gemm"))
+    # two round counters per slot beside its declaration, cleared before anyone can wait
+    at = got.index("__shared__ __bf16 p_first[2048];")
+    assert got[at + 1:at + 5] == ["__shared__ unsigned int __full_p_first, __empty_p_first;", "int __round_p_first = 0;",
+                                  "if (threadIdx.x == 0) { __full_p_first = 0; __empty_p_first = 0; }", "__syncthreads();"]
+    # the only workgroup barriers are those four: none in the K loop, whose iterations are ordered by the counters
+    loop = got.index("for (int k0 = 0; k0 < K; k0 += 64) {")
+    assert got.count("__syncthreads();") == 4 and all(n < loop for n, ln in enumerate(got) if ln == "__syncthreads();")
+
+    def events(start, stop):
+        out = []
+        for ln in got[start:stop]:
+            if ln.startswith("for (int __spin"):
+                word = ln.split("__hip_atomic_load(&__")[1].split(",")[0]
+                need = ln.split("static_cast<unsigned int>(")[1].split("); ++__spin")[0]
+                out.append(("wait", word, need))
+            elif "__hip_atomic_fetch_add(&__" in ln:
+                out.append(("signal", ln.split("__hip_atomic_fetch_add(&__")[1].split(",")[0]))
+            elif ln.startswith(("for (int part", "for (int n", "float4 a")):
+                out.append(("work", ln.split(" = ")[0] if ln.startswith("float4") else ln.split(";")[0]))
+        return out
+
+    producer = got.index("if (__thread_id_2 >= 0 && __thread_id_2 < 64) {")
+    consumer = got.index("if (__thread_id_2 >= 0 && __thread_id_2 < 256) {")
+    end = got.index("float* D_mine = D_tile + (0);")
+    # the producer (one wavefront) waits for the four reading wavefronts of the round before, fills, and counts itself in;
+    # it goes on to the second pair of slots while the consumers may still be reading the first
+    assert events(producer, consumer) == [
+        ("wait", "empty_p_first", "__round_p_first * 4"), ("wait", "empty_q_first", "__round_q_first * 4"),
+        ("work", "for (int part = 0"), ("signal", "full_p_first"), ("signal", "full_q_first"),
+        ("wait", "empty_p_second", "__round_p_second * 4"), ("wait", "empty_q_second", "__round_q_second * 4"),
+        ("work", "for (int part = 0"), ("signal", "full_p_second"), ("signal", "full_q_second")]
+    # a consumer gives a slot back as soon as its last read of it is behind it
+    assert events(consumer, end) == [
+        ("wait", "full_p_first", "(__round_p_first + 1) * 1"), ("work", "float4 a"), ("signal", "empty_p_first"),
+        ("wait", "full_q_first", "(__round_q_first + 1) * 1"), ("work", "for (int n = 0"), ("signal", "empty_q_first"),
+        ("wait", "full_p_second", "(__round_p_second + 1) * 1"), ("work", "float4 a2"), ("signal", "empty_p_second"),
+        ("wait", "full_q_second", "(__round_q_second + 1) * 1"), ("work", "for (int n = 0"), ("signal", "empty_q_second")]
+    # a signal follows the completion of everything the wavefront has in flight, direct-to-LDS loads included
+    first_signal = next(n for n, ln in enumerate(got) if "__hip_atomic_fetch_add(&__full_p_first" in ln)
+    assert got[first_signal - 2:first_signal] == ["__builtin_amdgcn_s_waitcnt(0);", '__builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");']
+    assert got[first_signal + 1] == "__round_p_first += 1;"
+    assert ("__builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&P_rows[(((((16 * part) + row) * K) "
+            "+ k0) + k8)]), (__attribute__((address_space(3))) void*)(&p_first_fill[(512 * part)]), 16, 0, 0);") in got
+    # every wait is bounded
+    assert all("__spin < 65536 &&" in ln for ln in got if ln.startswith("for (int __spin"))
+
+
+@requires(grid[1], block[1], thread[128])
+@prism("global")
+def two_writers(x: ptr(int) @ grid[1]):
+    with group(block[1]):
+        buf: shared(int[128], static=True) @ block[1]
+        with partition(buf, p=thread[64], offset=0) as mine:
+            match split(thread):
+                case 64:
+                    with partition(mine, p=thread[1], offset=0) as one:
+                        one[0] = 1
+                    t: int @ thread[1] = buf[1]
+                case 64:
+                    with partition(mine, p=thread[1], offset=1) as other:
+                        other[0] = buf[0]
+
+
+@requires(grid[1], block[1], thread[96])
+@prism("global")
+def half_a_wavefront_reads(x: ptr(int) @ grid[1]):
+    with group(block[1]):
+        buf: shared(int[128], static=True) @ block[1]
+        with partition(buf, p=thread[64], offset=0) as mine:
+            match split(thread):
+                case 64:
+                    with partition(mine, p=thread[1], offset=0) as one:
+                        one[0] = 1
+                case 32:
+                    t: int @ thread[1] = buf[0]
+
+
+@requires(grid[1], block[1], thread[128])
+@prism("global")
+def one_side_only(x: ptr(int) @ grid[1]):
+    with group(block[1]):
+        buf: shared(int[128], static=True) @ block[1]
+        match split(thread):
+            case 64:
+                t: int @ thread[1] = buf[0]
+            case 64:
+                u: int @ thread[1] = buf[1]
+
+
+def test_what_is_refused_and_what_needs_no_handover():
+    with pytest.raises(HipgenError, match="buf is written by more than one case"):
+        generate("two_writers")
+    with pytest.raises(HipgenError, match="whole wavefronts"):
+        generate("half_a_wavefront_reads")
+    assert "__full_buf" not in generate("one_side_only")      # read by both cases, written by none
+
+
+@pytest.fixture(scope="module")
+def built(tmp_path_factory):
+    return hipgen.build("handed_over_gemm", out_dir=str(tmp_path_factory.mktemp("hipgen_handover")), block_size=320)
+
+
+def test_launcher_compiles_for_gfx950(built):
+    assert hasattr(built, "handed_over_gemm_launch")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(64, 64, 64), (128, 192, 256), (256, 128, 1024), (512, 512, 4096)])
+def test_producer_consumer_gemm_against_the_oracle(built, oracle, shape):
+    """Up to 64 rounds of hand-over per workgroup; a lost or early signal shows as a wrong tile."""
+    import torch
+    M, N, K = shape
+    fn = built.handed_over_gemm_launch
+    fn.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int] * 3 + [ctypes.c_uint, ctypes.c_void_p]
+    p16, q16 = oracle.gen_gemm_bf16(M, N, K, seed=M + N + K)
+    P = torch.from_numpy(p16.view(np.int16)).to("cuda:0")
+    Q = torch.from_numpy(q16.view(np.int16)).to("cuda:0")
+    buf = torch.full((M * N + 128,), 777.0, dtype=torch.float32, device="cuda:0")
+    D = buf[64:64 + M * N]
+    torch.cuda.synchronize()
+    print(f"handed_over_gemm M={M} N={N} K={K}", flush=True)
+    assert fn(P.data_ptr(), Q.data_ptr(), D.data_ptr(), N, K, N // 64, (M // 64) * (N // 64), None) == 0
+    torch.cuda.synchronize()
+    out = buf.cpu().numpy()
+    assert np.all(out[:64] == 777.0) and np.all(out[64 + M * N:] == 777.0)
+    ref = oracle.gemm_bf16_f64(p16, q16)
+    assert np.max(np.abs(out[64:64 + M * N].reshape(M, N) - ref)) <= 1e-3 * np.abs(ref).max()
