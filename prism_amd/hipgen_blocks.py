@@ -18,16 +18,20 @@ per-thread kernel into a flat body; this one keeps the reference's structure:
     `__global__` and the return type; `@prism("device")` functions take the caller's ids and `__smem`
     as three leading arguments, which calls to them pass along.
 
-Barriers. The reference derives `__syncthreads()` placement from an analysis of which threads touch
-which elements (prism/sync_analysis.py, prism/sync_transform.py). Here placement is conservative and
-array-granular: walking a block's statements in program order, a barrier goes in front of the first
-statement that reads an LDS array written since the last barrier (by any thread), or writes one read
-since then (in front of the whole loop when that statement sits in one); a loop whose body would meet
-such a hazard with its own previous iteration gets a barrier at the end of the body. A barrier is never placed inside an `if` (threads may disagree on the branch):
-the hazard is resolved in front of the `if`, and one that lies wholly inside an `if` is an error.
-Two writes to one array without a read in between are taken to hit different elements. For the
-reference's LDS-tiled SGEMM example this gives the two barriers the reference prints
-(generated/sgemm_shared_mem_block.cu:38,42).
+Barriers. The reference places `__syncthreads()` from a phase analysis per LDS array (prism/sync_analysis.py:
+each array is in a READ or WRITE phase since the last barrier; a read after a write or a write after a read
+conflicts, two writes do not). The plan here is that analysis at the same granularity: walking a block's
+statements in program order, a barrier goes in front of the first statement that reads an LDS array written
+since the last barrier (by any thread), or writes one read since then (in front of the whole loop when that
+statement sits in one); a loop whose body would meet such a hazard with its own previous iteration gets a
+barrier at the end of the body. What a call does to an array it is handed is read off the callee's signature
+(a pointer to const is only read, :871-940), and a `ptr(shared(T))` parameter is an LDS array of its own
+(:151-158); a pointer that a call returns is not followed. A barrier is never placed inside an `if` (threads
+may disagree on the branch): the hazard is resolved in front of the `if`, and one that lies wholly inside an
+`if` is an error; the reference walks into branches (:424-447). For programs in the shapes of the reference's
+LDS-tiled SGEMMs, its kernel 5 and its scan this gives the barriers the reference prints
+(generated/sgemm_shared_mem_block.cu:38,42, my_sgemm_kernel_4.cu:48,65, my_sgemm_kernel_5.cu:41,46,
+scan_kernel.cu:17,19).
 
 Thread groups (`group(thread[n])`, the reference's warps for n = 32) are index arithmetic only
 (`__thread_id_d = outer % n`), so they carry over to 64-lane wavefronts unchanged as long as a group
@@ -40,8 +44,10 @@ does not look into unsafe() text.
 
 `match split(level): case n: ...` hands the first n members of a level one body and the next ones
 another (ids restart in every case; the reference's producer / consumer split,
-examples/h100_matmul.py:203-206); `claim(...)` prints like `partition(...)`. A split's cases are treated
-like the branches of an `if` by the barrier plan.
+examples/h100_matmul.py:203-206); `claim(...)` prints like `partition(...)`. No workgroup barrier is placed
+inside a case. An LDS array that one case of `match split(thread)` writes and other cases read is handed
+from case to case through two round counters in LDS (_SyncPlan._plan_handovers), the counterpart of the
+mbarrier waits and arrives the reference inserts (prism/sync_analysis.py:500-570, prism/codegen.py:886-934).
 
 Vector accesses (prism/codegen.py:239-242,544-549; examples/sgemm_kernel_4.py:53-60,78-84):
 `float4_cast(a[i])` reads and `float4_cast[a[i]] = v` writes the 16 bytes at `&a[i]`
@@ -65,8 +71,9 @@ forms, `intrinsic.mfma_f32_16x16x32_bf16(a, b, c0..c3, out=[...])` and `intrinsi
 c0..c15, out=[...])`, take `float4` operands that carry eight consecutive bf16 of a row, the way
 `float4_cast(P[i])` reads them from a `ptr(bf16)`: a = P[l % 16][8 (l / 16) .. + 7], b = Q[l % 16][same k] for
 C = P Q^T (32-row form: l % 32 and 8 (l / 32)); accumulators as in the fp32 forms. All 64
-lanes of the wavefront must reach the statement together. Inline PTX itself (`intrinsic.mma`,
-`intrinsic.wgmma256`) has no meaning on this target and is refused by name, like asynchronous copies.
+lanes of the wavefront must reach the statement together. `intrinsic.load_to_lds(dst[i], src[j])` is the
+asynchronous copy of this target (BlockEmitter.load_to_lds). Inline PTX itself (`intrinsic.mma`,
+`intrinsic.wgmma256`) has no meaning here and is refused by name.
 """
 from __future__ import annotations
 
