@@ -403,10 +403,10 @@ __attribute__((amdgpu_waves_per_eu(4))) void sgemm_wave_tile_kernel(
 // ------------------------------------------------- kernel 5, whole tiles --
 // The same product for problems made of whole 256 x 256 tiles: global data goes
 // straight into LDS (global_load_lds_dwordx4: no staging registers, no LDS
-// write instructions), four waves each own a 128 x 128 corner held in 256
-// accumulator registers, and one workgroup occupies a CU. With a single wave
-// per SIMD nothing else hides a stall, so the K loop is written as phases that
-// run from barrier to barrier with the matrix pipe fed throughout.
+// write instructions), every wave owns a WM x 128 strip of the tile in
+// accumulator registers, and one workgroup occupies a CU. The K loop is written
+// as phases that run from barrier to barrier with the matrix pipe fed
+// throughout.
 //
 // A vector ALU instruction between two MFMAs delays the second one by about 12
 // clocks (measured with one wave per SIMD; LDS reads cost about 5, scalar
@@ -414,6 +414,18 @@ __attribute__((amdgpu_waves_per_eu(4))) void sgemm_wave_tile_kernel(
 // loads take a scalar base and a fixed lane offset (direct_load.h), one load
 // behind every fourth MFMA of the first group, pinned there
 // with scheduling barriers (bunched loads hold the wave at the memory pipeline).
+//
+// Wave tile. What is left of those delays (LDS reads, direct loads, the wait at
+// the barrier, prologue and write-back of a tile) shows when a SIMD has a single
+// wave: 8192^3 ran at 0.952 of the fp32 peak with four waves of 128 x 128 (256
+// accumulators each), 0.965 with eight of 64 x 128 and 0.973 with sixteen of
+// 32 x 128 (64 accumulators, 124 registers, four waves per SIMD: while one wave
+// issues its reads or stores its strip, the others keep the matrix pipe busy);
+// 8192 x 8192 x 1024, where the write-back weighs more, 125 -> 134 -> 139.5
+// TFLOP/s. The narrow strips read the B operand four times as often from LDS
+// (5 reads per 16 MFMAs instead of 8 per 64), which fp32 MFMAs, 64 clocks for
+// two registers of operands, leave ample room for. The whole-tile launches use
+// 32 x 128.
 //
 // LDS layout of one K tile (two stages):
 //   As[m][k]  as in global memory, BK floats per row. A wave-wide direct load
@@ -1056,7 +1068,7 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
         *rc = check_launch("sgemm_wave_tile_dma_kernel");
         if (*rc == 0 && leftover_wt == 128) {
             // 128 x 256 halves of the same kernel, one workgroup to a CU
-            sgemm_wave_tile_dma_kernel<128, 256, 16, 64, 128, EDGE><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 2), dim3(256), 0, s>>>(
+            sgemm_wave_tile_dma_kernel<128, 256, 16, 32, 128, EDGE><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 2), dim3(512), 0, s>>>(
                 M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, main_tiles);
             *rc = check_launch("sgemm_wave_tile_dma_kernel (leftover halves)");
         } else if (*rc == 0 && leftover_wt == 256) {
@@ -1084,13 +1096,13 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
 
 // Between the one-wave tiles (up to one 64 x 64 tile per SIMD) and the 256 x 256 tiles (from three quarters of
 // the CUs up) lies a range in which neither fills the chip: there the same direct-to-LDS kernel runs on
-// 128 x 256 tiles (four waves of 64 x 128, K tiles of 16, 48 KiB of LDS, one workgroup per CU) when those give
+// 128 x 256 tiles (eight waves of 32 x 128, K tiles of 16, 48 KiB of LDS, one workgroup per CU) when those give
 // every CU at most one tile, else on 64 x 256 tiles (four waves of 32 x 128, 40 KiB of LDS, 138 registers: three
 // workgroups per CU) when those give every CU at most three; in both cases at least half of the CUs get one.
 template <int BM, bool ALLOW_EDGES>
 bool try_half_tile_dma(int M, int N, int K, float alpha, const float* A, const float* B, float beta,
                        float* C, hipStream_t s, int* rc) {
-    constexpr int BN = 256, BK = 16, WM = BM / 2, WN = 128;
+    constexpr int BN = 256, BK = 16, WM = 32, WN = 128;
     if (K <= 0 || !aligned16(A) || !aligned16(B) || !aligned16(C)) return false;
     const bool whole = M % BM == 0 && N % BN == 0 && K % BK == 0;
     if (!whole && (!ALLOW_EDGES || N % 4 || K % 4 ||
@@ -1196,8 +1208,8 @@ int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, 
                 // K tiles of 32 (128 KiB of LDS) when K allows, else of 16.
                 int rc = 0;
                 // Ragged M, N, K (N and K multiples of 4) take the K-tile-of-32 kernel with zero-filled edges.
-                if (try_wave_tile_dma<256, 256, 32, 128, 128, true>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
-                if (try_wave_tile_dma<256, 256, 16, 128, 128, false>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
+                if (try_wave_tile_dma<256, 256, 32, 32, 128, true>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
+                if (try_wave_tile_dma<256, 256, 16, 32, 128, false>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
                 // Small problems (at most one 64 x 64 tile per SIMD): one wave per tile, 32 x 32 tiles when
                 // 64 x 64 ones would leave SIMDs without work. In between, the direct-to-LDS kernel on
                 // 128 x 256 tiles (at most one per CU) or 64 x 256 tiles (at most three per CU); what is left
