@@ -345,7 +345,7 @@ def cpu_baseline_add_m(n=1 << 24):
 # ------------------------------------------------- HBM-side traffic table --
 
 TRAFFIC_KERNELS = [  # (workload, size, substring of the kernel name, threads in the grid)
-    ("sgemm", 8192, "sgemm_wave_tile_dma_kernel", 1024 * 256),
+    ("sgemm", 8192, "sgemm_wave_tile_dma_kernel", 1024 * 1024),
     ("scan", 1 << 30, "scan_lookback_kernel", (1 << 30) // 65536 * 1024),
     ("gemm_bf16", 8192, "gemm_bf16_early_kernel", 1024 * 256),
     ("add_m", 1 << 24, "add_m_vec4_kernel", (1 << 24) // 4),

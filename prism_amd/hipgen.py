@@ -47,7 +47,7 @@ from dataclasses import dataclass, field
 from pathlib import Path
 from typing import Callable, Dict, List, Optional
 
-__all__ = ["prism", "requires", "attr", "grid", "block", "warp", "thread", "ptr", "const", "restrict", "constexpr",
+__all__ = ["prism", "requires", "attr", "grid", "block", "thread", "ptr", "const", "restrict", "constexpr",
            "shared", "uint", "double", "uint32_t", "uint64_t", "group", "partition", "claim", "split", "unsafe",
            "generate", "generate_launcher", "build", "HipgenError"]
 
@@ -84,7 +84,8 @@ class CType:
         return Located(self, where)
 
 
-grid, block, warp, thread = (Perspective(n) for n in ("grid", "block", "warp", "thread"))
+# The levels of the reference (prism/perspective.py:10-14); its "warps" are thread[32] groups, here thread[64].
+grid, block, thread = (Perspective(n) for n in ("grid", "block", "thread"))
 
 _SCALARS = {"int": "int", "float": "float", "unsigned": "unsigned int", "uint": "unsigned int", "bool": "bool",
             "double": "double", "uint32_t": "uint32_t", "uint64_t": "uint64_t", "bf16": "__bf16", "float4": "float4",
@@ -218,7 +219,7 @@ _UNOPS = {ast.USub: "-", ast.Invert: "~", ast.Not: "!"}
 def _perspective_of(node: ast.AST) -> Perspective:
     """`thread[1]` / `grid[1]` as written in the source."""
     if isinstance(node, ast.Subscript) and isinstance(node.value, ast.Name) and node.value.id in (
-            "grid", "block", "warp", "thread"):
+            "grid", "block", "thread"):
         size = node.slice
         if isinstance(size, ast.Constant) and isinstance(size.value, int):
             return Perspective(node.value.id, size.value)

@@ -110,8 +110,6 @@ def _level(node: ast.AST) -> Tuple[str, int]:
     if (isinstance(node, ast.Subscript) and isinstance(node.value, ast.Name) and node.value.id in _LEVELS
             and isinstance(node.slice, ast.Constant) and isinstance(node.slice.value, int)):
         return node.value.id, node.slice.value
-    if isinstance(node, ast.Subscript) and isinstance(node.value, ast.Name) and node.value.id == "warp":
-        raise HipgenError(f"{_line(node)}: warp-level perspectives are not part of this slice")
     raise HipgenError(f"{_line(node)}: expected a perspective such as block[1]")
 
 
