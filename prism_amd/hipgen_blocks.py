@@ -177,7 +177,7 @@ class _SyncPlan:
         self.at_end: Set[int] = set()     # id(loop stmt)
         self.root: Dict[str, str] = {}    # LDS array or view of one -> the array
         # hand-over of LDS arrays between the cases of a split (see _plan_handovers)
-        self.declared_here: Set[str] = set()                       # LDS arrays declared in this function's body
+        self.declared_here: Set[str] = set()                       # LDS arrays declared in this function's body, outside loops
         self.handed: Dict[str, Tuple[int, int]] = {}               # array -> (writing wavefronts, reading wavefronts)
         self.covered: Dict[int, Set[str]] = {}                     # id(match) -> arrays handed over inside it
         self.wait_before: Dict[int, List[Tuple[str, str]]] = {}    # id(stmt) -> [(array, "full" | "empty")]
@@ -190,13 +190,14 @@ class _SyncPlan:
         self._plan_handovers(fn.body)
         self._walk(fn.body, (set(), set()), True)
 
-    def _collect(self, stmts: List[ast.stmt]) -> None:
+    def _collect(self, stmts: List[ast.stmt], in_loop: bool = False) -> None:
         for s in stmts:
             if isinstance(s, ast.AnnAssign) and isinstance(s.target, ast.Name):
                 t, _ = _annotation(s.annotation)
                 if _is_call(t, "shared"):
                     self.root[s.target.id] = s.target.id
-                    self.declared_here.add(s.target.id)
+                    if not in_loop:   # a declaration inside a loop would start its round counters afresh in every trip
+                        self.declared_here.add(s.target.id)
             elif isinstance(s, ast.With):
                 call = s.items[0].context_expr
                 target = s.items[0].optional_vars
@@ -205,10 +206,10 @@ class _SyncPlan:
                         and call.args[0].id in self.root):
                     self.root[target.id] = self.root[call.args[0].id]
             for field in ("body", "orelse"):
-                self._collect(getattr(s, field, []) or [])
+                self._collect(getattr(s, field, []) or [], in_loop or isinstance(s, (ast.For, ast.While)))
             if isinstance(s, ast.Match):
                 for case in s.cases:
-                    self._collect(case.body)
+                    self._collect(case.body, in_loop)
 
     # read / write sets of LDS arrays
     def _reads(self, node: Optional[ast.AST]) -> Set[str]:
@@ -327,8 +328,8 @@ class _SyncPlan:
                     if array in self.handed:
                         raise HipgenError(f"{_line(s)}: {array} is already handed over in another split")
                     if array not in self.declared_here:
-                        raise HipgenError(f"{_line(s)}: {array} is handed from case to case but declared elsewhere; its "
-                                          "round counters live beside its declaration")
+                        raise HipgenError(f"{_line(s)}: {array} is handed from case to case; it must be declared in this function, "
+                                          "outside any loop: its round counters live beside its declaration")
                     involved = writers + readers
                     if any(counts[i] <= 0 or counts[i] % 64 for i in involved):
                         raise HipgenError(f"{_line(s)}: {array} is handed from case to case; those cases must be whole "

@@ -148,3 +148,23 @@ def test_producer_consumer_gemm_against_the_oracle(built, oracle, shape):
     assert np.all(out[:64] == 777.0) and np.all(out[64 + M * N:] == 777.0)
     ref = oracle.gemm_bf16_f64(p16, q16)
     assert np.max(np.abs(out[64:64 + M * N].reshape(M, N) - ref)) <= 1e-3 * np.abs(ref).max()
+
+
+@requires(grid[1], block[1], thread[128])
+@prism("global")
+def slot_declared_in_the_loop(x: ptr(int) @ grid[1], trips: int @ grid[1]):
+    with group(block[1]):
+        for i in range(trips):
+            buf: shared(int[128], static=True) @ block[1]
+            with partition(buf, p=thread[64], offset=0) as mine:
+                match split(thread):
+                    case 64:
+                        with partition(mine, p=thread[1], offset=0) as one:
+                            one[0] = i
+                    case 64:
+                        t: int @ thread[1] = buf[0]
+
+
+def test_a_handed_over_array_is_declared_outside_loops():
+    with pytest.raises(HipgenError, match="outside any loop"):
+        generate("slot_declared_in_the_loop")
