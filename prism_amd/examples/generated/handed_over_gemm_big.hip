@@ -1,0 +1,113 @@
+__global__ __launch_bounds__(768) void handed_over_gemm_big(const __bf16* P, const __bf16* Q, float* D, int N, int K, int tiles_m, int tiles_n) {
+    extern __shared__ __align__(128) char __smem[];
+    int __block_id_0 = blockIdx.x;
+    int __thread_id_0 = __block_id_0 * blockDim.x + threadIdx.x;
+    const int per_xcd = ((tiles_m * tiles_n) / 8);
+    const int t = (((__block_id_0 % 8) * per_xcd) + (__block_id_0 / 8));
+    const int tile_r = ((8 * (t / (8 * tiles_n))) + (t % 8));
+    const int tile_c = ((t % (8 * tiles_n)) / 8);
+    {
+        const __bf16* P_rows = P + (((tile_r * 128) * K));
+        {
+            const __bf16* Q_rows = Q + (((tile_c * 256) * K));
+            {
+                float* D_tile = D + ((((tile_r * 128) * N) + (tile_c * 256)));
+                {
+                    int __block_id_1 = __block_id_0 % 1;
+                    int __thread_id_1 = __block_id_1 * blockDim.x + threadIdx.x;
+                    __shared__ __bf16 first[24576];
+                    __shared__ unsigned int __full_first, __empty_first;
+                    int __round_first = 0;
+                    if (threadIdx.x == 0) { __full_first = 0; __empty_first = 0; }
+                    __syncthreads();
+                    __shared__ __bf16 second[24576];
+                    __shared__ unsigned int __full_second, __empty_second;
+                    int __round_second = 0;
+                    if (threadIdx.x == 0) { __full_second = 0; __empty_second = 0; }
+                    __syncthreads();
+                    float acc[64] = {0};
+                    for (int k0 = 0; k0 < K; k0 += 128) {
+                        {
+                            __bf16* first_fill = first + (0);
+                            {
+                                __bf16* second_fill = second + (0);
+                                {
+                                    int __block_id_2 = __block_id_1;
+                                    int __thread_id_2 = __thread_id_1;
+                                    if (__thread_id_2 >= 0 && __thread_id_2 < 256) {
+                                        for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__empty_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_first * 8); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                                        fill_slot(__block_id_2, __thread_id_2, __smem, first_fill, P_rows, Q_rows, K, k0);
+                                        __builtin_amdgcn_s_waitcnt(0);
+                                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                                        if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__full_first, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                                        __round_first += 1;
+                                        for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__empty_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_second * 8); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                                        fill_slot(__block_id_2, __thread_id_2, __smem, second_fill, P_rows, Q_rows, K, (k0 + 64));
+                                        __builtin_amdgcn_s_waitcnt(0);
+                                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                                        if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__full_second, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                                        __round_second += 1;
+                                    }
+                                }
+                                {
+                                    int __block_id_2 = __block_id_1;
+                                    int __thread_id_2 = __thread_id_1 - 256;
+                                    if (__thread_id_2 >= 0 && __thread_id_2 < 512) {
+                                        for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__full_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_first + 1) * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                                        multiply_slot(__block_id_2, __thread_id_2, __smem, acc, first);
+                                        __builtin_amdgcn_s_waitcnt(0);
+                                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                                        if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__empty_first, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                                        __round_first += 1;
+                                        for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__full_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_second + 1) * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                                        multiply_slot(__block_id_2, __thread_id_2, __smem, acc, second);
+                                        __builtin_amdgcn_s_waitcnt(0);
+                                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                                        if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__empty_second, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                                        __round_second += 1;
+                                    }
+                                }
+                            }
+                        }
+                    }
+                    {
+                        float* D_mine = D_tile + (0);
+                        {
+                            int __block_id_2 = __block_id_1;
+                            int __thread_id_2 = __thread_id_1;
+                            if (__thread_id_2 >= 0 && __thread_id_2 < 256) {
+                            }
+                        }
+                        {
+                            int __block_id_2 = __block_id_1;
+                            int __thread_id_2 = __thread_id_1 - 256;
+                            if (__thread_id_2 >= 0 && __thread_id_2 < 512) {
+                                int wave = (__thread_id_2 / 64);
+                                {
+                                    int __block_id_3 = __block_id_2;
+                                    int __thread_id_3 = __thread_id_2 % 64;
+                                    int lane = __thread_id_3;
+                                    {
+                                        int __block_id_4 = __block_id_3;
+                                        int __thread_id_4 = __thread_id_3 % 1;
+                                        for (int i = 0; i < 4; i++) {
+                                            for (int j = 0; j < 4; j++) {
+                                                for (int v = 0; v < 4; v++) {
+                                                    D_mine[((((((((64 * (wave / 4)) + (16 * i)) + (4 * (lane / 16))) + v) * N) + (64 * (wave % 4))) + (16 * j)) + (lane % 16))] = acc[((((4 * i) + j) * 4) + v)];
+                                                }
+                                            }
+                                        }
+                                    }
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    }
+}

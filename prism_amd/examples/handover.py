@@ -13,7 +13,7 @@ producer fills two pairs of slots (32 k each) and each consumer wavefront multip
 the four 16-row groups of the Q slot. While the consumers work on one pair of slots the producer fills the other.
 M and N are multiples of 64, K of 64.
 """
-from prism_amd.hipgen import bf16, block, claim, const, float4, float4_cast, grid, group, intrinsic, partition, prism, ptr, requires, shared, split, thread
+from prism_amd.hipgen import attr, bf16, block, claim, const, float4, float4_cast, grid, group, intrinsic, partition, prism, ptr, requires, shared, split, thread
 
 
 @requires(grid[1], block[1], thread[320])
@@ -82,3 +82,101 @@ def handed_over_gemm(P: ptr(const(bf16)) @ grid[1], Q: ptr(const(bf16)) @ grid[1
                                         for n in range(4):
                                             for v in range(4):
                                                 D_mine[(16 * wave + 4 * (lane / 16) + v) * N + 16 * n + lane % 16] = acc[4 * n + v]
+
+
+# The same hand-over at full size: a 128 x 256 tile per workgroup, four producer and eight consumer wavefronts,
+# two slots of 64 k (48 KiB each: 128 rows of P, then 256 rows of Q, 128-byte rows).
+
+@requires(thread[256])
+@prism("device")
+def fill_slot(slot: ptr(bf16) @ thread[256], P_from: ptr(const(bf16)) @ block[1], Q_from: ptr(const(bf16)) @ block[1],
+              K: int @ grid[1], k_at: int @ block[1]):
+    """Four wavefronts copy 128 rows x 64 k of P and 256 rows x 64 k of Q, starting at column k_at, into a slot.
+    One direct load covers 8 rows. The 16-byte chunk c of row r is kept at position c ^ ((r / 2) % 8) of the row,
+    so that the sixteen rows a quarter of a wavefront reads later fall into different LDS banks: a lane fetches
+    the chunk that belongs where its 16 bytes land."""
+    with group(thread[256]):
+        w: int @ thread[64] = id()
+        with group(thread[64]):
+            lane: int @ thread[1] = id()
+            for part in range(4):
+                prow: int @ thread[1] = 8 * (4 * part + w) + lane / 8
+                intrinsic.load_to_lds(slot[512 * (4 * part + w)],
+                                      P_from[prow * K + k_at + 8 * ((lane % 8) ^ ((prow / 2) % 8))])
+            for part in range(8):
+                qrow: int @ thread[1] = 8 * (4 * part + w) + lane / 8
+                intrinsic.load_to_lds(slot[8192 + 512 * (4 * part + w)],
+                                      Q_from[qrow * K + k_at + 8 * ((lane % 8) ^ ((qrow / 2) % 8))])
+    return
+
+
+@requires(thread[512])
+@prism("device")
+def multiply_slot(acc: ptr(float) @ thread[1], slot: ptr(const(bf16)) @ block[1]):
+    """Eight wavefronts, two down and four across, each adding its 64 x 64 part of (P part)(Q part)^T to acc: two
+    k-steps of 4 x 4 matrix instructions of 16 x 16 x 32, acc[(4 i + j) * 4 + v] = D[16 i + 4 (lane / 16) + v][16 j + lane % 16]."""
+    with group(thread[512]):
+        wave: int @ thread[64] = id()
+        row0: int @ thread[64] = 64 * (wave / 4)
+        col0: int @ thread[64] = 64 * (wave % 4)
+        with group(thread[64]):
+            lane: int @ thread[1] = id()
+            r: int @ thread[1] = lane % 16
+            a: float4[4] @ thread[1]
+            for kk in range(2):
+                k8: int @ thread[1] = 8 * ((4 * kk + lane / 16) ^ ((r / 2) % 8))
+                for i in range(4):
+                    a[i] = float4_cast(slot[(row0 + 16 * i + r) * 64 + k8])
+                for j in range(4):
+                    b: float4 @ thread[1] = float4_cast(slot[8192 + (col0 + 16 * j + r) * 64 + k8])
+                    for i in range(4):
+                        intrinsic.mfma_f32_16x16x32_bf16(
+                            a[i], b, acc[(4 * i + j) * 4], acc[(4 * i + j) * 4 + 1], acc[(4 * i + j) * 4 + 2], acc[(4 * i + j) * 4 + 3],
+                            out=[acc[(4 * i + j) * 4], acc[(4 * i + j) * 4 + 1], acc[(4 * i + j) * 4 + 2], acc[(4 * i + j) * 4 + 3]])
+    return
+
+
+@attr("__launch_bounds__(768)")
+@requires(grid[1], block[1], thread[768])
+@prism("global")
+def handed_over_gemm_big(P: ptr(const(bf16)) @ grid[1], Q: ptr(const(bf16)) @ grid[1], D: ptr(float) @ grid[1],
+                         N: int @ grid[1], K: int @ grid[1], tiles_m: int @ grid[1], tiles_n: int @ grid[1]):
+    """D = P Q^T on 128 x 256 tiles: 256 producer threads keep two slots filled, 512 consumer threads multiply
+    them. K is a multiple of 128, M of 1024 and N of 256 (tiles_m = M / 128 a multiple of 8, tiles_n = N / 256).
+    Workgroups are dealt to the eight XCDs in turn; the tile order gives the workgroups that run on one XCD at the
+    same time a patch of eight tile rows by four tile columns, so that they share their panels in its L2."""
+    per_xcd: const(int) @ block[1] = (tiles_m * tiles_n) / 8
+    t: const(int) @ block[1] = (id() % 8) * per_xcd + id() / 8
+    tile_r: const(int) @ block[1] = 8 * (t / (8 * tiles_n)) + t % 8
+    tile_c: const(int) @ block[1] = (t % (8 * tiles_n)) / 8
+    with partition(P, p=block[1], offset=tile_r * 128 * K) as P_rows:
+        with partition(Q, p=block[1], offset=tile_c * 256 * K) as Q_rows:
+            with partition(D, p=block[1], offset=tile_r * 128 * N + tile_c * 256) as D_tile:
+                with group(block[1]):
+                    first: shared(bf16[24576], static=True) @ block[1]
+                    second: shared(bf16[24576], static=True) @ block[1]
+                    acc: float[64] @ thread[1] = {0}
+                    for k0 in range(0, K, 128):
+                        with claim(first, p=thread[256], offset=0) as first_fill:
+                            with claim(second, p=thread[256], offset=0) as second_fill:
+                                match split(thread):
+                                    case 256:
+                                        fill_slot(first_fill, P_rows, Q_rows, K, k0)
+                                        fill_slot(second_fill, P_rows, Q_rows, K, k0 + 64)
+                                    case 512:
+                                        multiply_slot(acc, first)
+                                        multiply_slot(acc, second)
+                    with partition(D_tile, p=thread[1], offset=0) as D_mine:
+                        match split(thread):
+                            case 256:
+                                pass
+                            case 512:
+                                wave: int @ thread[64] = id()
+                                with group(thread[64]):
+                                    lane: int @ thread[1] = id()
+                                    with group(thread[1]):
+                                        for i in range(4):
+                                            for j in range(4):
+                                                for v in range(4):
+                                                    D_mine[(64 * (wave / 4) + 16 * i + 4 * (lane / 16) + v) * N
+                                                           + 64 * (wave % 4) + 16 * j + lane % 16] = acc[(4 * i + j) * 4 + v]

@@ -35,8 +35,8 @@ scan_kernel.cu:17,19).
 
 Thread groups (`group(thread[n])`, the reference's warps for n = 32) are index arithmetic only
 (`__thread_id_d = outer % n`), so they carry over to 64-lane wavefronts unchanged as long as a group
-does not straddle two wavefronts: n is a power of two up to 64, and a 32-wide group is one half of a
-wavefront. Cross-lane traffic inside a group comes from `unsafe("...")` statements, whose text is
+does not share a wavefront with another: n is a power of two up to 64 (a 32-wide group is one half of a
+wavefront) or a multiple of 64 (the reference's 128-thread warp groups are two wavefronts). Cross-lane traffic inside a group comes from `unsafe("...")` statements, whose text is
 printed as it stands and must therefore be HIP: the counterpart of the reference's
 `__shfl_up_sync(static_cast<uint32_t>(-1), val, delta)` (examples/scan.py:23-29) is
 `__shfl_up(val, delta, 32)`, which shifts within each aligned group of 32 lanes. The barrier plan
@@ -869,9 +869,9 @@ class BlockEmitter:
         level, size = _level(call.args[0])
         if size < 1:
             raise HipgenError(f"{_line(s)}: a group has at least one member")
-        if level == "thread" and size > 1 and (size & (size - 1) or size > 64):
-            raise HipgenError(f"{_line(s)}: group(thread[{size}]): thread groups are powers of two up to the 64-lane "
-                              "wavefront, so that a group never straddles two wavefronts")
+        if level == "thread" and size > 1 and size % 64 and (size & (size - 1) or size > 64):
+            raise HipgenError(f"{_line(s)}: group(thread[{size}]): a thread group is a power of two up to the 64-lane "
+                              "wavefront or a whole number of wavefronts, so that no wavefront is shared between groups")
         outer = self.ids
         inner = _Ids(f"__block_id_{outer.depth + 1}", f"__thread_id_{outer.depth + 1}", outer.depth + 1)
         self.open()

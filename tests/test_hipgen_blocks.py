@@ -324,7 +324,7 @@ def test_split_restarts_ids_in_every_case():
 def test_refusals_name_the_construct():
     with pytest.raises(HipgenError, match="inside one `if`"):
         generate("hazard_in_branch")
-    with pytest.raises(HipgenError, match="powers of two"):
+    with pytest.raises(HipgenError, match="a power of two up to the 64-lane wavefront or a whole number of wavefronts"):
         generate("straddling_groups")
     with pytest.raises(HipgenError, match="thread-level kernels only"):
         generate("naive_sgemm", bounded=True)

@@ -123,8 +123,34 @@ def built(tmp_path_factory):
     return hipgen.build("handed_over_gemm", out_dir=str(tmp_path_factory.mktemp("hipgen_handover")), block_size=320)
 
 
-def test_launcher_compiles_for_gfx950(built):
-    assert hasattr(built, "handed_over_gemm_launch")
+@pytest.fixture(scope="module")
+def built_big(tmp_path_factory):
+    return hipgen.build("handed_over_gemm_big", out_dir=str(tmp_path_factory.mktemp("hipgen_handover_big")), block_size=768)
+
+
+def test_launcher_compiles_for_gfx950(built, built_big):
+    assert hasattr(built, "handed_over_gemm_launch") and hasattr(built_big, "handed_over_gemm_big_launch")
+
+
+def test_hand_over_through_device_functions():
+    """The full-size kernel fills and multiplies its slots in device functions: what a call does to a slot is read
+    off the callee's signature (a pointer to const is read, another pointer written), as for the barriers."""
+    got = lines(generate("handed_over_gemm_big"))
+    fills = [n for n, ln in enumerate(got) if ln.startswith("fill_slot(")]
+    mults = [n for n, ln in enumerate(got) if ln.startswith("multiply_slot(")]
+    assert len(fills) == 2 and len(mults) == 2
+    for name, n in zip(("first", "second"), fills):   # wait until the eight readers are done, fill, count in
+        assert got[n - 2].startswith(f"for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__empty_{name},")
+        assert f"__round_{name} * 8" in got[n - 2]
+        assert f"__hip_atomic_fetch_add(&__full_{name}, 1u" in got[n + 3] and got[n + 4] == f"__round_{name} += 1;"
+    for name, n in zip(("first", "second"), mults):   # wait until the four writers are done, multiply, give back
+        assert f"__hip_atomic_load(&__full_{name}," in got[n - 2] and f"(__round_{name} + 1) * 4" in got[n - 2]
+        assert f"__hip_atomic_fetch_add(&__empty_{name}, 1u" in got[n + 3]
+    loop = got.index("for (int k0 = 0; k0 < K; k0 += 128) {")
+    assert got.count("__syncthreads();") == 2 and all(n < loop for n, ln in enumerate(got) if ln == "__syncthreads();")
+    assert "__launch_bounds__(768)" in got[0]
+    # a thread group may be a whole number of wavefronts (the callee's group of 256 producer threads)
+    assert "int __thread_id_1 = __thread_id_0 % 256;" in lines(generate("fill_slot"))
 
 
 @pytest.mark.gpu
@@ -168,3 +194,27 @@ def slot_declared_in_the_loop(x: ptr(int) @ grid[1], trips: int @ grid[1]):
 def test_a_handed_over_array_is_declared_outside_loops():
     with pytest.raises(HipgenError, match="outside any loop"):
         generate("slot_declared_in_the_loop")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(1024, 256, 128), (1024, 512, 1024), (2048, 1024, 4096), (2048, 2048, 512)])
+def test_full_size_producer_consumer_gemm_against_the_oracle(built_big, oracle, shape):
+    """128 x 256 tiles, four producer and eight consumer wavefronts, two slots of 64 k in flight, tiles dealt to
+    the XCDs in patches."""
+    import torch
+    M, N, K = shape
+    fn = built_big.handed_over_gemm_big_launch
+    fn.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int] * 4 + [ctypes.c_uint, ctypes.c_void_p]
+    p16, q16 = oracle.gen_gemm_bf16(M, N, K, seed=M + N + K + 1)
+    P = torch.from_numpy(p16.view(np.int16)).to("cuda:0")
+    Q = torch.from_numpy(q16.view(np.int16)).to("cuda:0")
+    buf = torch.full((M * N + 128,), 777.0, dtype=torch.float32, device="cuda:0")
+    D = buf[64:64 + M * N]
+    torch.cuda.synchronize()
+    print(f"handed_over_gemm_big M={M} N={N} K={K}", flush=True)
+    assert fn(P.data_ptr(), Q.data_ptr(), D.data_ptr(), N, K, M // 128, N // 256, (M // 128) * (N // 256), None) == 0
+    torch.cuda.synchronize()
+    out = buf.cpu().numpy()
+    assert np.all(out[:64] == 777.0) and np.all(out[64 + M * N:] == 777.0)
+    ref = oracle.gemm_bf16_f64(p16, q16)
+    assert np.max(np.abs(out[64:64 + M * N].reshape(M, N) - ref)) <= 1e-3 * np.abs(ref).max()
