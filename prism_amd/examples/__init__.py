@@ -33,6 +33,7 @@ KERNELS: Dict[str, Tuple[str, int, Optional[List[int]]]] = {
     "gather_columns": ("basics", 256, None),
     "handed_over_gemm": ("handover", 320, None),
     "handed_over_gemm_big": ("handover", 768, None),
+    "handed_over_sgemm": ("handover", 768, None),
 }
 # device functions, printed on their own as well (the reference prints its scan's helpers one file each)
 DEVICE_FUNCTIONS: Dict[str, str] = {
@@ -40,7 +41,7 @@ DEVICE_FUNCTIONS: Dict[str, str] = {
     "stage_tiles": "sgemm", "multiply_tiles": "sgemm", "scaled_sum": "basics",
     "lane_shift_up": "scan", "shift_up_in_wavefront": "scan", "take_ticket": "scan", "publish": "scan",
     "look_back": "scan", "scan_rows": "scan", "collect_row_ends": "scan", "scan_row_ends": "scan", "write_back": "scan",
-    "fill_slot": "handover", "multiply_slot": "handover",
+    "fill_slot": "handover", "multiply_slot": "handover", "fill_slot_f32": "handover", "multiply_slot_f32": "handover",
 }
 GENERATED = Path(__file__).resolve().parent / "generated"
 

@@ -1,0 +1,114 @@
+__global__ __launch_bounds__(768) void handed_over_sgemm(int M, int N, int K, float alpha, const float* A, const float* B, float beta, float* C, int tiles_n) {
+    extern __shared__ __align__(128) char __smem[];
+    int __block_id_0 = blockIdx.x;
+    int __thread_id_0 = __block_id_0 * blockDim.x + threadIdx.x;
+    const int per_xcd = (((M / 128) * tiles_n) / 8);
+    const int t = (((__block_id_0 % 8) * per_xcd) + (__block_id_0 / 8));
+    const int tile_r = ((8 * (t / (8 * tiles_n))) + (t % 8));
+    const int tile_c = ((t % (8 * tiles_n)) / 8);
+    {
+        const float* A_rows = A + (((tile_r * 128) * K));
+        {
+            const float* B_cols = B + ((tile_c * 256));
+            {
+                float* C_tile = C + ((((tile_r * 128) * N) + (tile_c * 256)));
+                {
+                    int __block_id_1 = __block_id_0 % 1;
+                    int __thread_id_1 = __block_id_1 * blockDim.x + threadIdx.x;
+                    __shared__ float first[12288];
+                    __shared__ unsigned int __full_first, __empty_first;
+                    int __round_first = 0;
+                    if (threadIdx.x == 0) { __full_first = 0; __empty_first = 0; }
+                    __syncthreads();
+                    __shared__ float second[12288];
+                    __shared__ unsigned int __full_second, __empty_second;
+                    int __round_second = 0;
+                    if (threadIdx.x == 0) { __full_second = 0; __empty_second = 0; }
+                    __syncthreads();
+                    float acc[64] = {0};
+                    for (int k0 = 0; k0 < K; k0 += 64) {
+                        {
+                            float* first_fill = first + (0);
+                            {
+                                float* second_fill = second + (0);
+                                {
+                                    int __block_id_2 = __block_id_1;
+                                    int __thread_id_2 = __thread_id_1;
+                                    if (__thread_id_2 >= 0 && __thread_id_2 < 256) {
+                                        for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__empty_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_first * 8); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                                        fill_slot_f32(__block_id_2, __thread_id_2, __smem, first_fill, A_rows, B_cols, N, K, k0);
+                                        __builtin_amdgcn_s_waitcnt(0);
+                                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                                        if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__full_first, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                                        __round_first += 1;
+                                        for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__empty_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_second * 8); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                                        fill_slot_f32(__block_id_2, __thread_id_2, __smem, second_fill, A_rows, B_cols, N, K, (k0 + 32));
+                                        __builtin_amdgcn_s_waitcnt(0);
+                                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                                        if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__full_second, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                                        __round_second += 1;
+                                    }
+                                }
+                                {
+                                    int __block_id_2 = __block_id_1;
+                                    int __thread_id_2 = __thread_id_1 - 256;
+                                    if (__thread_id_2 >= 0 && __thread_id_2 < 512) {
+                                        for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__full_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_first + 1) * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                                        multiply_slot_f32(__block_id_2, __thread_id_2, __smem, acc, first);
+                                        __builtin_amdgcn_s_waitcnt(0);
+                                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                                        if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__empty_first, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                                        __round_first += 1;
+                                        for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__full_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_second + 1) * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                                        multiply_slot_f32(__block_id_2, __thread_id_2, __smem, acc, second);
+                                        __builtin_amdgcn_s_waitcnt(0);
+                                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                                        if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__empty_second, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                                        __round_second += 1;
+                                    }
+                                }
+                            }
+                        }
+                    }
+                    {
+                        float* C_mine = C_tile + (0);
+                        {
+                            int __block_id_2 = __block_id_1;
+                            int __thread_id_2 = __thread_id_1;
+                            if (__thread_id_2 >= 0 && __thread_id_2 < 256) {
+                            }
+                        }
+                        {
+                            int __block_id_2 = __block_id_1;
+                            int __thread_id_2 = __thread_id_1 - 256;
+                            if (__thread_id_2 >= 0 && __thread_id_2 < 512) {
+                                int wave = (__thread_id_2 / 64);
+                                {
+                                    int __block_id_3 = __block_id_2;
+                                    int __thread_id_3 = __thread_id_2 % 64;
+                                    int lane = __thread_id_3;
+                                    {
+                                        int __block_id_4 = __block_id_3;
+                                        int __thread_id_4 = __thread_id_3 % 1;
+                                        for (int i = 0; i < 2; i++) {
+                                            for (int j = 0; j < 2; j++) {
+                                                for (int v = 0; v < 16; v++) {
+                                                    int at = (((((((((64 * (wave / 4)) + (32 * i)) + (8 * (v / 4))) + (4 * (lane / 32))) + (v % 4)) * N) + (64 * (wave % 4))) + (32 * j)) + (lane % 32));
+                                                    C_mine[at] = ((alpha * acc[((((2 * i) + j) * 16) + v)]) + (beta * C_mine[at]));
+                                                }
+                                            }
+                                        }
+                                    }
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    }
+}

@@ -180,3 +180,98 @@ def handed_over_gemm_big(P: ptr(const(bf16)) @ grid[1], Q: ptr(const(bf16)) @ gr
                                                 for v in range(4):
                                                     D_mine[(64 * (wave / 4) + 16 * i + 4 * (lane / 16) + v) * N
                                                            + 64 * (wave % 4) + 16 * j + lane % 16] = acc[(4 * i + j) * 4 + v]
+
+
+# SGEMM the same way: C = alpha A B + beta C (row-major fp32) on the fp32 matrix instruction, 128 x 256 tiles,
+# two slots of 32 k (48 KiB each: 128 rows of A with 128-byte rows, then 32 rows of B with 1 KiB rows).
+
+@requires(thread[256])
+@prism("device")
+def fill_slot_f32(slot: ptr(float) @ thread[256], A_from: ptr(const(float)) @ block[1], B_from: ptr(const(float)) @ block[1],
+                  N: int @ grid[1], K: int @ grid[1], k_at: int @ block[1]):
+    """Four wavefronts copy 128 rows x 32 k of A (8 rows per direct load, 16-byte chunks placed at
+    c ^ ((row / 2) % 8) as in fill_slot) and 32 k-rows x 256 columns of B (one k-row per direct load)."""
+    with group(thread[256]):
+        w: int @ thread[64] = id()
+        with group(thread[64]):
+            lane: int @ thread[1] = id()
+            for part in range(4):
+                arow: int @ thread[1] = 8 * (4 * part + w) + lane / 8
+                intrinsic.load_to_lds(slot[256 * (4 * part + w)],
+                                      A_from[arow * K + k_at + 4 * ((lane % 8) ^ ((arow / 2) % 8))])
+            for part in range(8):
+                intrinsic.load_to_lds(slot[4096 + 256 * (4 * part + w)], B_from[(k_at + 4 * part + w) * N + 4 * lane])
+    return
+
+
+@requires(thread[512])
+@prism("device")
+def multiply_slot_f32(acc: ptr(float) @ thread[1], slot: ptr(const(float)) @ block[1]):
+    """Eight wavefronts, two down and four across, each adding its 64 x 64 part of (A part)(B part) to acc: sixteen
+    pairs of k values, 2 x 2 instructions of 32 x 32 x 2 per pair;
+    acc[(2 i + j) * 16 + v] = C[32 i + 8 (v / 4) + 4 (lane / 32) + v % 4][32 j + lane % 32]."""
+    with group(thread[512]):
+        wave: int @ thread[64] = id()
+        row0: int @ thread[64] = 64 * (wave / 4)
+        col0: int @ thread[64] = 64 * (wave % 4)
+        with group(thread[64]):
+            lane: int @ thread[1] = id()
+            l32: int @ thread[1] = lane % 32
+            a: float[2] @ thread[1]
+            b: float[2] @ thread[1]
+            for kk in range(0, 32, 2):
+                k: int @ thread[1] = kk + lane / 32
+                for i in range(2):
+                    a[i] = slot[(row0 + 32 * i + l32) * 32 + 4 * ((k / 4) ^ ((l32 / 2) % 8)) + k % 4]
+                for j in range(2):
+                    b[j] = slot[4096 + k * 256 + col0 + 32 * j + l32]
+                for i in range(2):
+                    for j in range(2):
+                        intrinsic.mfma_f32_32x32x2_f32(a[i], b[j], acc[(2 * i + j) * 16 + 0], acc[(2 * i + j) * 16 + 1], acc[(2 * i + j) * 16 + 2], acc[(2 * i + j) * 16 + 3], acc[(2 * i + j) * 16 + 4], acc[(2 * i + j) * 16 + 5], acc[(2 * i + j) * 16 + 6], acc[(2 * i + j) * 16 + 7], acc[(2 * i + j) * 16 + 8], acc[(2 * i + j) * 16 + 9], acc[(2 * i + j) * 16 + 10], acc[(2 * i + j) * 16 + 11], acc[(2 * i + j) * 16 + 12], acc[(2 * i + j) * 16 + 13], acc[(2 * i + j) * 16 + 14], acc[(2 * i + j) * 16 + 15],
+                                                       out=[acc[(2 * i + j) * 16 + 0], acc[(2 * i + j) * 16 + 1], acc[(2 * i + j) * 16 + 2], acc[(2 * i + j) * 16 + 3], acc[(2 * i + j) * 16 + 4], acc[(2 * i + j) * 16 + 5], acc[(2 * i + j) * 16 + 6], acc[(2 * i + j) * 16 + 7], acc[(2 * i + j) * 16 + 8], acc[(2 * i + j) * 16 + 9], acc[(2 * i + j) * 16 + 10], acc[(2 * i + j) * 16 + 11], acc[(2 * i + j) * 16 + 12], acc[(2 * i + j) * 16 + 13], acc[(2 * i + j) * 16 + 14], acc[(2 * i + j) * 16 + 15]])
+    return
+
+
+@attr("__launch_bounds__(768)")
+@requires(grid[1], block[1], thread[768])
+@prism("global")
+def handed_over_sgemm(M: int @ grid[1], N: int @ grid[1], K: int @ grid[1], alpha: float @ grid[1],
+                      A: ptr(const(float)) @ grid[1], B: ptr(const(float)) @ grid[1], beta: float @ grid[1],
+                      C: ptr(float) @ grid[1], tiles_n: int @ grid[1]):
+    """M a multiple of 1024, N of 256, K of 64; tiles_n = N / 256. Tile order as in handed_over_gemm_big."""
+    per_xcd: const(int) @ block[1] = ((M / 128) * tiles_n) / 8
+    t: const(int) @ block[1] = (id() % 8) * per_xcd + id() / 8
+    tile_r: const(int) @ block[1] = 8 * (t / (8 * tiles_n)) + t % 8
+    tile_c: const(int) @ block[1] = (t % (8 * tiles_n)) / 8
+    with partition(A, p=block[1], offset=tile_r * 128 * K) as A_rows:
+        with partition(B, p=block[1], offset=tile_c * 256) as B_cols:
+            with partition(C, p=block[1], offset=tile_r * 128 * N + tile_c * 256) as C_tile:
+                with group(block[1]):
+                    first: shared(float[12288], static=True) @ block[1]
+                    second: shared(float[12288], static=True) @ block[1]
+                    acc: float[64] @ thread[1] = {0}
+                    for k0 in range(0, K, 64):
+                        with claim(first, p=thread[256], offset=0) as first_fill:
+                            with claim(second, p=thread[256], offset=0) as second_fill:
+                                match split(thread):
+                                    case 256:
+                                        fill_slot_f32(first_fill, A_rows, B_cols, N, K, k0)
+                                        fill_slot_f32(second_fill, A_rows, B_cols, N, K, k0 + 32)
+                                    case 512:
+                                        multiply_slot_f32(acc, first)
+                                        multiply_slot_f32(acc, second)
+                    with partition(C_tile, p=thread[1], offset=0) as C_mine:
+                        match split(thread):
+                            case 256:
+                                pass
+                            case 512:
+                                wave: int @ thread[64] = id()
+                                with group(thread[64]):
+                                    lane: int @ thread[1] = id()
+                                    with group(thread[1]):
+                                        for i in range(2):
+                                            for j in range(2):
+                                                for v in range(16):
+                                                    at: int @ thread[1] = (64 * (wave / 4) + 32 * i + 8 * (v / 4) + 4 * (lane / 32) + v % 4) * N \
+                                                        + 64 * (wave % 4) + 32 * j + lane % 32
+                                                    C_mine[at] = alpha * acc[(2 * i + j) * 16 + v] + beta * C_mine[at]

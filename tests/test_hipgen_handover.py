@@ -218,3 +218,40 @@ def test_full_size_producer_consumer_gemm_against_the_oracle(built_big, oracle, 
     assert np.all(out[:64] == 777.0) and np.all(out[64 + M * N:] == 777.0)
     ref = oracle.gemm_bf16_f64(p16, q16)
     assert np.max(np.abs(out[64:64 + M * N].reshape(M, N) - ref)) <= 1e-3 * np.abs(ref).max()
+
+
+@pytest.fixture(scope="module")
+def built_sgemm(tmp_path_factory):
+    return hipgen.build("handed_over_sgemm", out_dir=str(tmp_path_factory.mktemp("hipgen_handover_sgemm")), block_size=768)
+
+
+def test_sgemm_launcher_compiles_for_gfx950(built_sgemm):
+    assert hasattr(built_sgemm, "handed_over_sgemm_launch")
+    got = lines(generate("handed_over_sgemm"))
+    loop = got.index("for (int k0 = 0; k0 < K; k0 += 64) {")
+    assert got.count("__syncthreads();") == 2 and all(n < loop for n, ln in enumerate(got) if ln == "__syncthreads();")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(1024, 256, 64), (1024, 768, 1000 // 64 * 64), (2048, 1024, 2048)])
+def test_producer_consumer_sgemm_against_the_oracle(built_sgemm, oracle, shape):
+    """fp32 matrix instructions fed through handed-over slots; the kernel-5 tolerance against fp64."""
+    import torch
+    M, N, K = shape
+    fn = built_sgemm.handed_over_sgemm_launch
+    fn.argtypes = [ctypes.c_int] * 3 + [ctypes.c_float, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p,
+                                       ctypes.c_int, ctypes.c_uint, ctypes.c_void_p]
+    A, B, Cm = oracle.gen_sgemm(M, N, K, seed=M + N + K)
+    a, b = torch.from_numpy(A).to("cuda:0"), torch.from_numpy(B).to("cuda:0")
+    buf = torch.full((M * N + 128,), 777.0, dtype=torch.float32, device="cuda:0")
+    c = buf[64:64 + M * N].view(M, N)
+    c.copy_(torch.from_numpy(Cm))
+    torch.cuda.synchronize()
+    print(f"handed_over_sgemm M={M} N={N} K={K}", flush=True)
+    assert fn(M, N, K, 0.5, a.data_ptr(), b.data_ptr(), 3.0, c.data_ptr(), N // 256, (M // 128) * (N // 256), None) == 0
+    torch.cuda.synchronize()
+    out = buf.cpu().numpy()
+    assert np.all(out[:64] == 777.0) and np.all(out[64 + M * N:] == 777.0)
+    want = oracle.np_sgemm_f64(0.5, A, B, 3.0, Cm)
+    tol = oracle.sgemm_tolerance(K, A, B) + 3.0 * float(np.abs(Cm).max()) * 2**-22
+    assert np.max(np.abs(out[64:64 + M * N].reshape(M, N) - want)) <= tol
