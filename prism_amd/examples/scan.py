@@ -274,3 +274,97 @@ def lookback_scan_by_parts(x: ptr(const(uint32_t)) @ grid[1], y: ptr(uint32_t) @
                     before: uint32_t @ block[1] = look_back(status_blk, tile, spin_limit)
                     publish(status_blk, tile, 2, before + total)
                     write_back(y_tile, scanned, upto, before)
+
+
+# The look-back scan with sixteen elements per thread and a look-back that reads 64 status words at a time.
+
+@requires(block[1], thread[1])
+@prism("device")
+def look_back_wide(status: ptr(uint64_t) @ block[1], tile: uint32_t @ block[1], spin_limit: int @ block[1]) -> uint32_t @ block[1]:
+    """Sum of all tiles before `tile`. The first wavefront reads the status words of the 64 tiles before it at once
+    (lane 0 the nearest), waits until every word between this tile and the nearest inclusive prefix is there, adds
+    them up, and moves on by 64 tiles if the window held no prefix. Tiles before the first count as a prefix of 0.
+    The wait is bounded: a broken ordering shows as a wrong result, never as a hang."""
+    with group(block[1]):
+        unsafe("""
+__shared__ uint32_t before;
+if (threadIdx.x < 64) {
+    uint32_t sum = 0;
+    int nearest = static_cast<int>(tile) - 1, spins = 0;
+    bool done = false;
+    while (!done) {
+        const int id = nearest - static_cast<int>(threadIdx.x);
+        for (;;) {
+            const uint64_t word = id >= 0 ? __hip_atomic_load(&status[id], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                          : (static_cast<uint64_t>(2) << 32);
+            const uint64_t prefixes = __ballot((word >> 32) == 2), missing = __ballot((word >> 32) == 0);
+            const int first = prefixes ? __ffsll(static_cast<unsigned long long>(prefixes)) - 1 : 64;
+            const uint64_t wanted = first >= 63 ? ~0ull : ((1ull << (first + 1)) - 1);
+            if ((missing & wanted) == 0 || ++spins > spin_limit) {
+                uint32_t part = static_cast<int>(threadIdx.x) <= first ? static_cast<uint32_t>(word) : 0u;
+                for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o, 64);
+                sum += part;
+                done = first < 64 || spins > spin_limit;
+                nearest -= 64;
+                break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
+    }
+    if (threadIdx.x == 0) before = sum;
+}
+__syncthreads();
+return before;
+""")
+    return
+
+
+@requires(grid[1], block[1], thread[64])
+@prism("global")
+def lookback_scan_wide(x: ptr(const(uint32_t)) @ grid[1], y: ptr(uint32_t) @ grid[1], counter: ptr(uint32_t) @ grid[1],
+                       status: ptr(uint64_t) @ grid[1], spin_limit: int @ grid[1]):
+    """Tiles of 4096 elements, 256 threads with 16 consecutive elements each in a private array: a serial scan per
+    thread, one scan by lane shifts over the thread totals of a wavefront, the four wavefront totals through LDS."""
+    tile: uint32_t @ grid[1] = take_ticket(counter)
+    with partition(x, p=block[1], offset=tile * 4096) as x_tile:
+        with partition(y, p=block[1], offset=tile * 4096) as y_tile:
+            with partition(status, p=block[1], offset=0) as status_blk:
+                with group(block[1]):
+                    wave_sums: shared(uint32_t[4], static=True) @ block[1]
+                    t: int @ thread[1] = id()
+                    wave: int @ thread[64] = id()
+                    v: uint32_t[16] @ thread[1]
+                    with partition(x_tile, p=thread[1], offset=16 * t) as x_mine:
+                        with group(thread[1]):
+                            for i in range(16):
+                                v[i] = x_mine[i]
+                            for i in range(1, 16):
+                                v[i] += v[i - 1]
+                    upto_me: uint32_t @ thread[1] = v[15]
+                    with partition(wave_sums, p=thread[64], offset=wave) as my_wave_sum:
+                        with group(thread[64]):
+                            lane: uint32_t @ thread[1] = id()
+                            with partition(my_wave_sum, p=thread[1], offset=0) as sum_one:
+                                with group(thread[1]):
+                                    stride: uint32_t @ thread[1] = 1
+                                    while stride < 64:
+                                        got: uint32_t @ thread[1] = shift_up_in_wavefront(upto_me, stride)
+                                        if lane >= stride:
+                                            upto_me = got + upto_me
+                                        stride *= 2
+                                    if lane == 63:
+                                        sum_one[0] = upto_me
+                    total: uint32_t @ block[1] = wave_sums[0] + wave_sums[1] + wave_sums[2] + wave_sums[3]
+                    publish(status_blk, tile, 1, total)
+                    before: uint32_t @ block[1] = look_back_wide(status_blk, tile, spin_limit)
+                    publish(status_blk, tile, 2, before + total)
+                    with partition(y_tile, p=thread[1], offset=16 * t) as y_mine:
+                        with group(thread[64]):
+                            earlier_waves: uint32_t @ thread[64] = 0
+                            for w in range(4):
+                                if w < wave:
+                                    earlier_waves += wave_sums[w]
+                            with group(thread[1]):
+                                base: uint32_t @ thread[1] = before + earlier_waves + (upto_me - v[15])
+                                for i in range(16):
+                                    y_mine[i] = base + v[i]

@@ -12,9 +12,6 @@ from prism_amd import hipgen
 from prism_amd.examples import scan as _programs  # noqa: F401  (defines the kernels)
 from prism_amd.hipgen import generate, generate_launcher
 
-TILE = 1024
-
-
 def lines(text):
     return [ln.strip() for ln in text.splitlines()]
 
@@ -62,7 +59,19 @@ def test_barriers_of_the_scan_made_of_device_functions():
     assert "const uint32_t* scanned" in generate("collect_row_ends").splitlines()[0]
 
 
-KERNELS = ("lookback_scan", "lookback_scan_by_parts")
+def test_structure_of_the_wide_scan():
+    """Sixteen elements per thread in a private array; one barrier between the wavefront totals going into LDS and
+    the sum that reads them; the look-back reads 64 status words per step."""
+    got = lines(generate("lookback_scan_wide"))
+    assert "uint32_t v[16];" in got and "v[i] += v[(i - 1)];" in got
+    sync = [n for n, ln in enumerate(got) if ln == "__syncthreads();"]
+    assert len(sync) == 1 and got[sync[0] + 1].startswith("uint32_t total = (((wave_sums[0] + wave_sums[1])")
+    assert "uint32_t base = ((before + earlier_waves) + (upto_me - v[15]));" in got
+    text = generate("look_back_wide")
+    assert "__ballot((word >> 32) == 2)" in text and "spin_limit" in text
+
+
+KERNELS = {"lookback_scan": 1024, "lookback_scan_by_parts": 1024, "lookback_scan_wide": 4096}   # kernel -> elements per tile
 
 
 @pytest.fixture(scope="module")
@@ -83,7 +92,7 @@ def test_generated_lookback_scan_is_bit_exact(built, tiles, name):
     import torch
     fn = getattr(built[name], f"{name}_launch")
     fn.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int, ctypes.c_uint, ctypes.c_void_p]
-    n = tiles * TILE
+    n = tiles * KERNELS[name]
     x = np.random.default_rng(tiles).integers(0, 2**32, n, dtype=np.uint32)
     xd = torch.from_numpy(x.view(np.int32)).to("cuda:0")
     yd = torch.full((n + 8,), -5, dtype=torch.int32, device="cuda:0")
