@@ -1,6 +1,7 @@
 """Evaluation sweeps in the reference harnesses' own methodology and text format.
 
     python -m prism_amd.eval_report [sgemm] [scan] [h100]      (default: all three)
+    python -m prism_amd.eval_report generated                  (the same three sweeps over kernels generated from the DSL)
 
 The counterpart of the reference's three benchmark mains, so that the text it
 prints can be fed to the reference's plotting script unchanged:
@@ -17,6 +18,13 @@ prints can be fed to the reference's plotting script unchanged:
 The vendor-library slots ("cuBLAS", "CUB") are filled with what the ROCm stack
 offers through PyTorch: rocBLAS/hipBLASLt `torch.matmul` and rocPRIM
 `torch.cumsum`. They are comparison lines, like the reference's.
+
+`generated` runs the same protocols over the kernels that prism_amd.hipgen prints from the example programs
+(prism_amd/examples), which is what the reference's figures show for its own back-end: "My Kernel" 1..5 are
+naive_sgemm, remapped_sgemm, tiled_sgemm<32>, vector_tile_sgemm<128,128,8,8,8> and handed_over_sgemm (the
+producer / consumer kernel on the fp32 matrix instruction; sizes it does not take, below 1024, are left out),
+the scan is lookback_scan_wide, and "Kernel:" in the bf16 sweep is handed_over_gemm_big (fp32 row-major output,
+where the reference's kernel writes bf16 column-major). The kernels are compiled for gfx950 on the spot.
 """
 from __future__ import annotations
 
@@ -167,6 +175,111 @@ def sweep_h100(out=sys.stdout, sizes=H100_SIZES, repeats: int = 8) -> None:
         del A, B, Cc
 
 
+def sweep_generated(out=sys.stdout, sgemm_sizes=SGEMM_SIZES, scan_log2_sizes=SCAN_LOG2_SIZES, h100_sizes=H100_SIZES,
+                    repeats: int = 10, target_ms: float = 500.0) -> None:
+    """The three sweeps over kernels generated from the example programs."""
+    import ctypes
+    import tempfile
+
+    import torch
+
+    from . import examples, hipgen
+    examples.load()
+    built = {}
+
+    def kernel(name):
+        if name not in built:
+            _, block_size, template = examples.KERNELS[name]
+            lib = hipgen.build(name, out_dir=tempfile.mkdtemp(prefix="prism_eval_"), block_size=block_size, template=template)
+            built[name] = getattr(lib, f"{name}_launch")
+        return built[name]
+
+    sgemm_args = [ctypes.c_int] * 3 + [ctypes.c_float, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p,
+                                       ctypes.c_int, ctypes.c_uint, ctypes.c_void_p]
+    # "My Kernel" k -> (program, smallest size it takes, last integer argument, number of workgroups)
+    steps = {1: ("naive_sgemm", 1, lambda n: 256, lambda n: (n * n + 255) // 256),
+             2: ("remapped_sgemm", 1, lambda n: (n + 31) // 32, lambda n: ((n + 31) // 32) ** 2),
+             3: ("tiled_sgemm", 32, lambda n: n // 32, lambda n: (n // 32) ** 2),
+             4: ("vector_tile_sgemm", 128, lambda n: n // 128, lambda n: (n // 128) ** 2),
+             5: ("handed_over_sgemm", 1024, lambda n: n // 256, lambda n: (n // 128) * (n // 256))}
+    alpha, beta = 0.5, 3.0
+    top = max(sgemm_sizes)
+    A = torch.rand((top, top), device="cuda") * 2 - 1
+    B = torch.rand((top, top), device="cuda") * 2 - 1
+    C = torch.rand((top, top), device="cuda") * 2 - 1
+    print("\n====================================\nStarting Performance Sweep\n====================================", file=out)
+    for n in sgemm_sizes:
+        a, b = A.flatten()[: n * n].view(n, n), B.flatten()[: n * n].view(n, n)
+        c = C.flatten()[: n * n].view(n, n).clone()
+        flops = 2.0 * n * n * n
+        print(f"\n====================================\nSize: {n}x{n}x{n}\n====================================", file=out)
+        print("\n[cuBLAS FP32]", file=out)
+        ref = c.clone()
+        torch.addmm(ref, a, b, beta=beta, alpha=alpha, out=ref)
+        ms = _events_ms(lambda: torch.addmm(ref, a, b, beta=beta, alpha=alpha, out=ref), repeats)
+        print(sgemm_line(ms / 1e3 / repeats, repeats * flops * 1e-9 / (ms / 1e3), n), file=out)
+        for k, (name, smallest, last, blocks) in steps.items():
+            if n < smallest:
+                continue
+            launch = kernel(name)
+            launch.argtypes = sgemm_args
+            print(f"\n[My Kernel {k}]", file=out)
+            c.copy_(C.flatten()[: n * n].view(n, n))
+            fn = lambda: launch(n, n, n, alpha, a.data_ptr(), b.data_ptr(), beta, c.data_ptr(), last(n), blocks(n), None)
+            if fn() != 0:
+                raise RuntimeError(f"{name} failed to launch at {n}")
+            ms = _events_ms(fn, repeats)
+            print(sgemm_line(ms / 1e3 / repeats, repeats * flops * 1e-9 / (ms / 1e3), n), file=out)
+        out.flush()
+    del A, B, C
+
+    scan = kernel("lookback_scan_wide")
+    scan.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int, ctypes.c_uint, ctypes.c_void_p]
+    top = 1 << max(scan_log2_sizes)
+    x = torch.randint(0, 101, (top,), dtype=torch.int32, device="cuda")
+    work = torch.empty_like(x)
+    counter = torch.zeros(1, dtype=torch.int32, device="cuda")
+    status = torch.zeros(top // 4096, dtype=torch.int64, device="cuda")
+    print("\n" + scan_header(), file=out)
+    for p in scan_log2_sizes:
+        n = 1 << p
+        xin, buf = x[:n], work[:n]
+
+        def ours():  # the two clearing fills are timed, as the reference's two memsets are
+            counter.zero_()
+            status[: n // 4096].zero_()
+            if scan(xin.data_ptr(), buf.data_ptr(), counter.data_ptr(), status.data_ptr(), 1 << 22, n // 4096, None) != 0:
+                raise RuntimeError("lookback_scan_wide failed to launch")
+
+        def vendor():
+            torch.cumsum(xin, 0, dtype=torch.int32, out=buf)
+        results = [_best_wall_ms(fn, target_ms) for fn in (vendor, ours)]
+        bytes_ = n * 4 * 2
+        print(scan_row(n, results[0], bytes_ / results[0] / 1e6, results[1], bytes_ / results[1] / 1e6), file=out)
+        out.flush()
+    print("", file=out)
+    del x, work
+
+    gemm = kernel("handed_over_gemm_big")
+    gemm.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int] * 4 + [ctypes.c_uint, ctypes.c_void_p]
+    for n in h100_sizes:
+        P = torch.randn((n, n), device="cuda").to(torch.bfloat16)
+        Q = torch.randn((n, n), device="cuda").to(torch.bfloat16)
+        D = torch.empty((n, n), dtype=torch.float32, device="cuda")
+        flops = 2.0 * n * n * n
+        fn = lambda: gemm(P.data_ptr(), Q.data_ptr(), D.data_ptr(), n, n, n // 128, n // 256, (n // 128) * (n // 256), None)
+        if fn() != 0:
+            raise RuntimeError(f"handed_over_gemm_big failed to launch at {n}")
+        ms = _events_ms(fn, 8)
+        print(h100_line("Kernel:", ms / 1e3 / 8, 8 * flops * 1e-9 / ms, n), file=out)
+        vend = lambda: torch.matmul(P, Q.T)
+        vend()
+        ms = _events_ms(vend, 8)
+        print(h100_line("cuBLAS:", ms / 1e3 / 8, 8 * flops * 1e-9 / ms, n) + "\n", file=out)
+        out.flush()
+        del P, Q, D
+
+
 def main(argv=None) -> int:
     which = [a for a in (argv if argv is not None else sys.argv[1:])] or ["sgemm", "scan", "h100"]
     for w in which:
@@ -176,8 +289,10 @@ def main(argv=None) -> int:
             sweep_scan()
         elif w == "h100":
             sweep_h100()
+        elif w == "generated":
+            sweep_generated()
         else:
-            print(f"unknown sweep {w!r}; expected sgemm, scan or h100", file=sys.stderr)
+            print(f"unknown sweep {w!r}; expected sgemm, scan, h100 or generated", file=sys.stderr)
             return 2
     return 0
 

@@ -18,6 +18,7 @@ KERNELS: Dict[str, Tuple[str, int, Optional[List[int]]]] = {
     "add_m_blocks": ("add_m", 256, None),
     "add_m_by_wavefronts": ("add_m", 256, None),
     "naive_sgemm": ("sgemm", 256, None),
+    "remapped_sgemm": ("sgemm", 1024, None),
     "tiled_sgemm": ("sgemm", 1024, [32]),
     "thread_tile_sgemm": ("sgemm", 256, [64, 64, 8, 4, 4]),
     "vector_tile_sgemm": ("sgemm", 256, [128, 128, 8, 8, 8]),

@@ -1,0 +1,31 @@
+__global__ void remapped_sgemm(int M, int N, int K, float alpha, const float* A, const float* B, float beta, float* C, int tiles_n) {
+    extern __shared__ __align__(128) char __smem[];
+    int __block_id_0 = blockIdx.x;
+    int __thread_id_0 = __block_id_0 * blockDim.x + threadIdx.x;
+    const int tile_r = (__block_id_0 / tiles_n);
+    const int tile_c = (__block_id_0 % tiles_n);
+    {
+        float* C_of_block = C + (0);
+        {
+            int __block_id_1 = __block_id_0 % 1;
+            int __thread_id_1 = __block_id_1 * blockDim.x + threadIdx.x;
+            int t = __thread_id_1;
+            const int row = ((tile_r * 32) + (t / 32));
+            const int col = ((tile_c * 32) + (t % 32));
+            {
+                float* C_mine = C_of_block + (0);
+                {
+                    int __block_id_2 = __block_id_1;
+                    int __thread_id_2 = __thread_id_1 % 1;
+                    if (((row < M) && (col < N))) {
+                        float acc = 0;
+                        for (int k = 0; k < K; k++) {
+                            acc += (A[((row * K) + k)] * B[((k * N) + col)]);
+                        }
+                        C_mine[((row * N) + col)] = ((alpha * acc) + (beta * C_mine[((row * N) + col)]));
+                    }
+                }
+            }
+        }
+    }
+}

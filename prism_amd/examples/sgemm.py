@@ -1,6 +1,7 @@
 """SGEMM, C = alpha A B + beta C (row-major), in the steps of the reference's example set.
 
 naive_sgemm        one thread per element of C (examples/sgemm_kernel_1.py)
+remapped_sgemm     the same with a workgroup's threads laid over a 32 x 32 tile (examples/sgemm_kernel_2.py)
 tiled_sgemm        TILE x TILE tiles of A and B staged in LDS (examples/sgemm_shared_mem_block.py)
 thread_tile_sgemm  a TM x TN block of C per thread, operands in private arrays (examples/sgemm_kernel_3.py)
 vector_tile_sgemm  16-byte global accesses, the A tile stored k-major (examples/sgemm_kernel_4.py)
@@ -27,6 +28,29 @@ def naive_sgemm(M: int @ grid[1], N: int @ grid[1], K: int @ grid[1], alpha: flo
             with partition(C_of_block, p=thread[1], offset=0) as C_mine:
                 with group(thread[1]):
                     if e < M * N:
+                        acc: float @ thread[1] = 0
+                        for k in range(K):
+                            acc += A[row * K + k] * B[k * N + col]
+                        C_mine[row * N + col] = alpha * acc + beta * C_mine[row * N + col]
+
+
+@requires(grid[1], block[1], thread[1])
+@prism("global")
+def remapped_sgemm(M: int @ grid[1], N: int @ grid[1], K: int @ grid[1], alpha: float @ grid[1],
+                   A: ptr(const(float)) @ grid[1], B: ptr(const(float)) @ grid[1], beta: float @ grid[1],
+                   C: ptr(float) @ grid[1], tiles_n: int @ grid[1]):
+    """One thread per element with the 1024 threads of a workgroup laid over a 32 x 32 tile of C, consecutive
+    threads along a row (examples/sgemm_kernel_2.py); guarded, so that M and N need not be multiples of 32."""
+    tile_r: const(int) @ block[1] = id() / tiles_n
+    tile_c: const(int) @ block[1] = id() % tiles_n
+    with partition(C, p=block[1], offset=0) as C_of_block:
+        with group(block[1]):
+            t: int @ thread[1] = id()
+            row: const(int) @ thread[1] = tile_r * 32 + t / 32
+            col: const(int) @ thread[1] = tile_c * 32 + t % 32
+            with partition(C_of_block, p=thread[1], offset=0) as C_mine:
+                with group(thread[1]):
+                    if row < M and col < N:
                         acc: float @ thread[1] = 0
                         for k in range(K):
                             acc += A[row * K + k] * B[k * N + col]

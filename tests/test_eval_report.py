@@ -79,3 +79,18 @@ def test_sweeps_produce_parseable_reports():
     er.sweep_h100(buf, sizes=(2048,), repeats=3)
     text = buf.getvalue()
     assert re.search(H100_KERNEL, text) and re.search(H100_VENDOR, text)
+
+
+@pytest.mark.gpu
+def test_sweeps_over_generated_kernels_produce_parseable_reports():
+    """The same three formats from kernels generated out of the example programs (compiled on the spot)."""
+    buf = io.StringIO()
+    er.sweep_generated(buf, sgemm_sizes=(256, 1024), scan_log2_sizes=(20, 22), h100_sizes=(1024,), repeats=2, target_ms=20.0)
+    text = buf.getvalue()
+    parsed = parse_sgemm(text)
+    assert sorted(parsed, key=str) == [1, 2, 3, 4, 5, 'vendor']
+    assert [r[0] for r in parsed[1]] == [256, 1024] and [r[0] for r in parsed[5]] == [1024]   # the last step starts at 1024
+    assert all(r[1] > 0 for rows in parsed.values() for r in rows)
+    rows = parse_scan_table(text)
+    assert [r[0] for r in rows] == [1 << 20, 1 << 22] and all(r[1] > 0 and r[2] > 0 for r in rows)
+    assert re.search(H100_KERNEL, text) and re.search(H100_VENDOR, text)
