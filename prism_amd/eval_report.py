@@ -23,7 +23,7 @@ offers through PyTorch: rocBLAS/hipBLASLt `torch.matmul` and rocPRIM
 (prism_amd/examples), which is what the reference's figures show for its own back-end: "My Kernel" 1..5 are
 naive_sgemm, remapped_sgemm, tiled_sgemm<32>, vector_tile_sgemm<128,128,8,8,8> and handed_over_sgemm (the
 producer / consumer kernel on the fp32 matrix instruction; sizes it does not take, below 1024, are left out),
-the scan is lookback_scan_wide, and "Kernel:" in the bf16 sweep is handed_over_gemm_big (fp32 row-major output,
+the scan is lookback_scan_striped, and "Kernel:" in the bf16 sweep is handed_over_gemm_big (fp32 row-major output,
 where the reference's kernel writes bf16 column-major). The kernels are compiled for gfx950 on the spot.
 """
 from __future__ import annotations
@@ -233,13 +233,13 @@ def sweep_generated(out=sys.stdout, sgemm_sizes=SGEMM_SIZES, scan_log2_sizes=SCA
         out.flush()
     del A, B, C
 
-    scan = kernel("lookback_scan_wide")
+    scan = kernel("lookback_scan_striped")
     scan.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int, ctypes.c_uint, ctypes.c_void_p]
     top = 1 << max(scan_log2_sizes)
     x = torch.randint(0, 101, (top,), dtype=torch.int32, device="cuda")
     work = torch.empty_like(x)
     counter = torch.zeros(1, dtype=torch.int32, device="cuda")
-    status = torch.zeros(top // 4096, dtype=torch.int64, device="cuda")
+    status = torch.zeros(top // 16384, dtype=torch.int64, device="cuda")
     print("\n" + scan_header(), file=out)
     for p in scan_log2_sizes:
         n = 1 << p
@@ -247,9 +247,9 @@ def sweep_generated(out=sys.stdout, sgemm_sizes=SGEMM_SIZES, scan_log2_sizes=SCA
 
         def ours():  # the two clearing fills are timed, as the reference's two memsets are
             counter.zero_()
-            status[: n // 4096].zero_()
-            if scan(xin.data_ptr(), buf.data_ptr(), counter.data_ptr(), status.data_ptr(), 1 << 22, n // 4096, None) != 0:
-                raise RuntimeError("lookback_scan_wide failed to launch")
+            status[: n // 16384].zero_()
+            if scan(xin.data_ptr(), buf.data_ptr(), counter.data_ptr(), status.data_ptr(), 1 << 22, n // 16384, None) != 0:
+                raise RuntimeError("lookback_scan_striped failed to launch")
 
         def vendor():
             torch.cumsum(xin, 0, dtype=torch.int32, out=buf)

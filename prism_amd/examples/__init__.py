@@ -30,6 +30,7 @@ KERNELS: Dict[str, Tuple[str, int, Optional[List[int]]]] = {
     "lookback_scan": ("scan", 256, None),
     "lookback_scan_by_parts": ("scan", 256, None),
     "lookback_scan_wide": ("scan", 256, None),
+    "lookback_scan_striped": ("scan", 1024, None),
     "scaled_sum_all": ("basics", 256, None),
     "two_roles": ("basics", 256, None),
     "gather_columns": ("basics", 256, None),
@@ -44,7 +45,7 @@ DEVICE_FUNCTIONS: Dict[str, str] = {
     "lane_shift_up": "scan", "shift_up_in_wavefront": "scan", "take_ticket": "scan", "publish": "scan",
     "look_back": "scan", "scan_rows": "scan", "collect_row_ends": "scan", "scan_row_ends": "scan", "write_back": "scan",
     "fill_slot": "handover", "multiply_slot": "handover", "fill_slot_f32": "handover", "multiply_slot_f32": "handover",
-    "look_back_wide": "scan",
+    "look_back_wide": "scan", "value_of_last_lane": "scan",
 }
 GENERATED = Path(__file__).resolve().parent / "generated"
 

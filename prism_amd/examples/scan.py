@@ -368,3 +368,76 @@ def lookback_scan_wide(x: ptr(const(uint32_t)) @ grid[1], y: ptr(uint32_t) @ gri
                                 base: uint32_t @ thread[1] = before + earlier_waves + (upto_me - v[15])
                                 for i in range(16):
                                     y_mine[i] = base + v[i]
+
+
+# The same scan with the tile read the way the memory system likes it: a lane's 16 bytes next to its neighbour's.
+
+@requires(thread[1])
+@prism("device")
+def value_of_last_lane(val: uint32_t @ thread[1]) -> uint32_t @ thread[1]:
+    with group(thread[1]):
+        unsafe("return __shfl(val, 63, 64);")
+    return
+
+
+@requires(grid[1], block[1], thread[64])
+@prism("global")
+def lookback_scan_striped(x: ptr(const(uint32_t)) @ grid[1], y: ptr(uint32_t) @ grid[1], counter: ptr(uint32_t) @ grid[1],
+                          status: ptr(uint64_t) @ grid[1], spin_limit: int @ grid[1]):
+    """Tiles of 16384 elements as 64 rows of 256 (1024 threads); a wavefront owns four consecutive rows and a lane four consecutive
+    elements of each (one 16-byte access per row, the 64 lanes of an access side by side). Per row: the lane's
+    four elements serially, the lane totals by lane shifts, and what the wavefront's earlier rows hold added on."""
+    tile: uint32_t @ grid[1] = take_ticket(counter)
+    with partition(x, p=block[1], offset=tile * 16384) as x_tile:
+        with partition(y, p=block[1], offset=tile * 16384) as y_tile:
+            with partition(status, p=block[1], offset=0) as status_blk:
+                with group(block[1]):
+                    wave_sums: shared(uint32_t[16], static=True) @ block[1]
+                    wave: int @ thread[64] = id()
+                    v: uint32_t[16] @ thread[1]
+                    with partition(x_tile, p=thread[64], offset=1024 * wave) as x_wave:
+                        with partition(wave_sums, p=thread[64], offset=wave) as my_wave_sum:
+                            with group(thread[64]):
+                                lane: uint32_t @ thread[1] = id()
+                                with partition(x_wave, p=thread[1], offset=4 * lane) as x_mine:
+                                    with partition(my_wave_sum, p=thread[1], offset=0) as sum_one:
+                                        with group(thread[1]):
+                                            for j in range(4):
+                                                for e in range(4):
+                                                    v[4 * j + e] = x_mine[256 * j + e]
+                                            carry: uint32_t @ thread[1] = 0
+                                            for j in range(4):
+                                                v[4 * j + 1] += v[4 * j]
+                                                v[4 * j + 2] += v[4 * j + 1]
+                                                v[4 * j + 3] += v[4 * j + 2]
+                                                upto_me: uint32_t @ thread[1] = v[4 * j + 3]
+                                                stride: uint32_t @ thread[1] = 1
+                                                while stride < 64:
+                                                    got: uint32_t @ thread[1] = shift_up_in_wavefront(upto_me, stride)
+                                                    if lane >= stride:
+                                                        upto_me = got + upto_me
+                                                    stride *= 2
+                                                ahead: uint32_t @ thread[1] = carry + (upto_me - v[4 * j + 3])
+                                                for e in range(4):
+                                                    v[4 * j + e] += ahead
+                                                carry += value_of_last_lane(upto_me)
+                                            if lane == 63:
+                                                sum_one[0] = carry
+                    total: uint32_t @ block[1] = 0
+                    for w in range(16):
+                        total += wave_sums[w]
+                    publish(status_blk, tile, 1, total)
+                    before: uint32_t @ block[1] = look_back_wide(status_blk, tile, spin_limit)
+                    publish(status_blk, tile, 2, before + total)
+                    with partition(y_tile, p=thread[64], offset=1024 * wave) as y_wave:
+                        with group(thread[64]):
+                            lane_out: uint32_t @ thread[1] = id()
+                            earlier_waves: uint32_t @ thread[64] = 0
+                            for w in range(16):
+                                if w < wave:
+                                    earlier_waves += wave_sums[w]
+                            with partition(y_wave, p=thread[1], offset=4 * lane_out) as y_mine:
+                                with group(thread[1]):
+                                    for j in range(4):
+                                        for e in range(4):
+                                            y_mine[256 * j + e] = before + earlier_waves + v[4 * j + e]

@@ -71,13 +71,14 @@ def test_structure_of_the_wide_scan():
     assert "__ballot((word >> 32) == 2)" in text and "spin_limit" in text
 
 
-KERNELS = {"lookback_scan": 1024, "lookback_scan_by_parts": 1024, "lookback_scan_wide": 4096}   # kernel -> elements per tile
+KERNELS = {"lookback_scan": 1024, "lookback_scan_by_parts": 1024, "lookback_scan_wide": 4096, "lookback_scan_striped": 16384}   # kernel -> elements per tile
 
 
 @pytest.fixture(scope="module")
 def built(tmp_path_factory):
     d = tmp_path_factory.mktemp("hipgen_scan")
-    return {name: hipgen.build(name, out_dir=str(d), block_size=256) for name in KERNELS}
+    from prism_amd import examples
+    return {name: hipgen.build(name, out_dir=str(d), block_size=examples.KERNELS[name][1]) for name in KERNELS}
 
 
 def test_launcher_compiles_for_gfx950(built):
