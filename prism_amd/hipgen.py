@@ -411,21 +411,22 @@ def _check_perspectives(name: str) -> None:
     check(name)
 
 
-def generate(name: str, bounded: bool = False, auto_sync: bool = True) -> str:
+def generate(name: str, bounded: bool = False, auto_sync: bool = True, annotate: bool = False) -> str:
     """HIP text of kernel `name`.
 
     Thread-level kernels (@requires without a block perspective) are printed flat. bounded=False prints
     what the reference prints for the same source (one thread per element, no guard); bounded=True
     appends a `size_t prism_n` parameter and returns early for thread ids beyond it, so that any grid
     covering n is legal. Kernels with a block perspective are printed by hipgen_blocks.generate_blocks
-    (auto_sync places the barriers); they carry their own guards, so bounded does not apply."""
+    (auto_sync places the barriers, annotate=True says in a comment what each is for); they carry their own
+    guards, so bounded does not apply."""
     k = _kernel(name)
     _check_perspectives(name)
     if _structured(k):
         if bounded:
             raise HipgenError("bounded=True applies to thread-level kernels only")
         from .hipgen_blocks import generate_blocks
-        return generate_blocks(name, auto_sync)
+        return generate_blocks(name, auto_sync, annotate)
     return _Emitter(k, bounded).emit()
 
 

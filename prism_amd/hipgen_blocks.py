@@ -175,6 +175,7 @@ class _SyncPlan:
     def __init__(self, fn: ast.FunctionDef):
         self.before: Set[int] = set()     # id(stmt)
         self.at_end: Set[int] = set()     # id(loop stmt)
+        self.why: Dict[int, str] = {}     # id(stmt) -> what the barrier there is for (see explain_barriers)
         self.root: Dict[str, str] = {}    # LDS array or view of one -> the array
         # hand-over of LDS arrays between the cases of a split (see _plan_handovers)
         self.declared_here: Set[str] = set()                       # LDS arrays declared in this function's body, outside loops
@@ -366,7 +367,7 @@ class _SyncPlan:
             if isinstance(s, ast.With):
                 r = self._with_reads(s)
                 if self._hazard(r, set(), (pr, pw)):
-                    self._mark(s, may_sync)
+                    self._mark(s, may_sync, self._reason(r, set(), (pr, pw)))
                     pr, pw = set(), set()
                 pr |= r
                 pr, pw = self._walk(s.body, (pr, pw), may_sync)
@@ -375,7 +376,7 @@ class _SyncPlan:
                 # of the loop, not in every iteration.
                 r, w = self._whole([s])
                 if self._hazard(r, w, (pr, pw)):
-                    self._mark(s, may_sync)
+                    self._mark(s, may_sync, self._reason(r, w, (pr, pw)))
                     pr, pw = set(), set()
                 pr |= self._reads(s.iter if isinstance(s, ast.For) else s.test)
                 before_loop = (set(pr), set(pw))
@@ -384,6 +385,7 @@ class _SyncPlan:
                     if not may_sync:
                         raise HipgenError(f"{_line(s)}: a loop inside an `if` needs a barrier between its iterations")
                     self.at_end.add(id(s))
+                    self.why[id(s)] = "the next trip of the loop " + self._reason(*self._whole(s.body), (pr, pw))
                     pr, pw = set(), set()
                 if not self._runs_at_least_once(s):
                     # With zero trips none of the body's barriers is executed: what was pending in front
@@ -393,7 +395,7 @@ class _SyncPlan:
             elif isinstance(s, (ast.If, ast.Match)):
                 r, w = self._whole([s])
                 if self._hazard(r, w, (pr, pw)):
-                    self._mark(s, may_sync)
+                    self._mark(s, may_sync, self._reason(r, w, (pr, pw)))
                     pr, pw = set(), set()
                 # Inside the branches (or the cases of a split) no barrier may be placed: not every thread
                 # gets there. Hazards inside are errors.
@@ -407,7 +409,7 @@ class _SyncPlan:
             else:
                 r, w = self._access(s)
                 if self._hazard(r, w, (pr, pw)):
-                    self._mark(s, may_sync)
+                    self._mark(s, may_sync, self._reason(r, w, (pr, pw)))
                     pr, pw = set(), set()
                 pr |= r
                 pw |= w
@@ -427,11 +429,22 @@ class _SyncPlan:
         except ValueError:
             return False
 
-    def _mark(self, s: ast.stmt, may_sync: bool) -> None:
+    @staticmethod
+    def _reason(r: Set[str], w: Set[str], pending: Tuple[Set[str], Set[str]]) -> str:
+        pr, pw = pending
+        parts = []
+        if r & pw:
+            parts.append("reads " + ", ".join(sorted(r & pw)) + " (written since the last barrier)")
+        if w & pr:
+            parts.append("writes " + ", ".join(sorted(w & pr)) + " (read since the last barrier)")
+        return " and ".join(parts)
+
+    def _mark(self, s: ast.stmt, may_sync: bool, why: str = "") -> None:
         if not may_sync:
             raise HipgenError(f"{_line(s)}: LDS is written and read inside one `if`; the barrier between "
                               "them cannot be placed in divergent code")
         self.before.add(id(s))
+        self.why[id(s)] = why
 
     def _probe(self, stmts: List[ast.stmt], pending: Tuple[Set[str], Set[str]]) -> str:
         """Runs the next iteration's statements against what the previous one left pending:
@@ -464,8 +477,9 @@ class _SyncPlan:
 # -------------------------------------------------------------------- emitter --
 
 class BlockEmitter:
-    def __init__(self, kernel: Kernel, auto_sync: bool = True):
+    def __init__(self, kernel: Kernel, auto_sync: bool = True, annotate: bool = False):
         self.k = kernel
+        self.annotate = annotate          # a comment in front of every barrier says what it is for
         self.auto_sync = auto_sync
         self.out: List[str] = []
         self.indent = 0
@@ -586,6 +600,8 @@ class BlockEmitter:
     def block(self, stmts: List[ast.stmt]) -> None:
         for s in stmts:
             if self.plan is not None and id(s) in self.plan.before:
+                if self.annotate:
+                    self.emit(f"// {_line(s)} {self.plan.why.get(id(s), '')}")
                 self.emit("__syncthreads();")
             for array, what in (self.plan.wait_before.get(id(s), []) if self.plan is not None else []):
                 self.wait_for(array, what)
@@ -710,6 +726,8 @@ class BlockEmitter:
         self.indent += 1
         self.block(s.body)
         if self.plan is not None and id(s) in self.plan.at_end:
+            if self.annotate:
+                self.emit(f"// {self.plan.why.get(id(s), '')}")
             self.emit("__syncthreads();")
         self.indent -= 1
         self.emit("}")
@@ -981,11 +999,19 @@ class BlockEmitter:
         return "\n".join(self.out) + "\n"
 
 
-def generate_blocks(name: str, auto_sync: bool = True) -> str:
-    """HIP text of kernel or device function `name` in the structured form described above."""
+def generate_blocks(name: str, auto_sync: bool = True, annotate: bool = False) -> str:
+    """HIP text of kernel or device function `name` in the structured form described above. annotate=True puts a
+    comment in front of every barrier that names the statement's source line and the arrays the barrier is for
+    (the reference keeps such a record per barrier as well, SyncReason, prism/sync_analysis.py:40-73)."""
     if name not in _REGISTRY:
         raise HipgenError(f"no kernel named {name!r} has been defined with @prism")
-    return BlockEmitter(_REGISTRY[name], auto_sync).emit_function()
+    return BlockEmitter(_REGISTRY[name], auto_sync, annotate).emit_function()
+
+
+def explain_barriers(name: str) -> List[str]:
+    """One line per barrier of `name`, in program order: where it stands and which arrays it orders."""
+    text = generate_blocks(name, True, annotate=True).splitlines()
+    return [text[n - 1].strip()[3:] for n, ln in enumerate(text) if ln.strip() == "__syncthreads();" and text[n - 1].strip().startswith("// ")]
 
 
 def dynamic_lds_bytes(name: str) -> int:

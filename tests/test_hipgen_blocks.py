@@ -214,6 +214,17 @@ def test_barriers_between_device_functions_that_are_handed_the_tiles():
     assert len(calls) == 4 and sync == [calls[0] + 1, calls[3] - 1] and calls[2] == calls[1] + 1
 
 
+def test_every_barrier_can_say_what_it_is_for():
+    from prism_amd.hipgen_blocks import explain_barriers
+    assert explain_barriers("staged_sgemm") == [
+        "line 27 reads a_lds, b_lds (written since the last barrier)",
+        "the next trip of the loop writes a_lds, b_lds (read since the last barrier)"]
+    got = lines(generate("tiled_sgemm", annotate=True))
+    first = got.index("__syncthreads();")
+    assert got[first - 1] == "// line 23 reads a_lds, b_lds (written since the last barrier)"
+    assert not any(ln.startswith("//") for ln in lines(generate("tiled_sgemm")))   # only on request
+
+
 def test_dynamic_lds_windows_private_arrays_and_attr():
     text = generate("thread_tile_sgemm")
     got = lines(text)
