@@ -239,7 +239,7 @@ def sweep_generated(out=sys.stdout, sgemm_sizes=SGEMM_SIZES, scan_log2_sizes=SCA
     x = torch.randint(0, 101, (top,), dtype=torch.int32, device="cuda")
     work = torch.empty_like(x)
     counter = torch.zeros(1, dtype=torch.int32, device="cuda")
-    status = torch.zeros(top // 16384, dtype=torch.int64, device="cuda")
+    status = torch.zeros(top // 65536, dtype=torch.int64, device="cuda")
     print("\n" + scan_header(), file=out)
     for p in scan_log2_sizes:
         n = 1 << p
@@ -247,8 +247,8 @@ def sweep_generated(out=sys.stdout, sgemm_sizes=SGEMM_SIZES, scan_log2_sizes=SCA
 
         def ours():  # the two clearing fills are timed, as the reference's two memsets are
             counter.zero_()
-            status[: n // 16384].zero_()
-            if scan(xin.data_ptr(), buf.data_ptr(), counter.data_ptr(), status.data_ptr(), 1 << 22, n // 16384, None) != 0:
+            status[: n // 65536].zero_()
+            if scan(xin.data_ptr(), buf.data_ptr(), counter.data_ptr(), status.data_ptr(), 1 << 22, n // 65536, None) != 0:
                 raise RuntimeError("lookback_scan_striped failed to launch")
 
         def vendor():

@@ -86,9 +86,9 @@ __global__ void lookback_scan_striped(const uint32_t* x, uint32_t* y, uint32_t* 
     int __thread_id_0 = __block_id_0 * blockDim.x + threadIdx.x;
     uint32_t tile = take_ticket(__block_id_0, __thread_id_0, __smem, counter);
     {
-        const uint32_t* x_tile = x + ((tile * 16384));
+        const uint32_t* x_tile = x + ((tile * 65536));
         {
-            uint32_t* y_tile = y + ((tile * 16384));
+            uint32_t* y_tile = y + ((tile * 65536));
             {
                 uint64_t* status_blk = status + (0);
                 {
@@ -96,9 +96,9 @@ __global__ void lookback_scan_striped(const uint32_t* x, uint32_t* y, uint32_t* 
                     int __thread_id_1 = __block_id_1 * blockDim.x + threadIdx.x;
                     __shared__ uint32_t wave_sums[16];
                     int wave = (__thread_id_1 / 64);
-                    uint32_t v[16];
+                    uint32_t v[64];
                     {
-                        const uint32_t* x_wave = x_tile + ((1024 * wave));
+                        const uint32_t* x_wave = x_tile + ((4096 * wave));
                         {
                             uint32_t* my_wave_sum = wave_sums + (wave);
                             {
@@ -112,13 +112,13 @@ __global__ void lookback_scan_striped(const uint32_t* x, uint32_t* y, uint32_t* 
                                         {
                                             int __block_id_3 = __block_id_2;
                                             int __thread_id_3 = __thread_id_2 % 1;
-                                            for (int j = 0; j < 4; j++) {
+                                            for (int j = 0; j < 16; j++) {
                                                 for (int e = 0; e < 4; e++) {
                                                     v[((4 * j) + e)] = x_mine[((256 * j) + e)];
                                                 }
                                             }
                                             uint32_t carry = 0;
-                                            for (int j = 0; j < 4; j++) {
+                                            for (int j = 0; j < 16; j++) {
                                                 v[((4 * j) + 1)] += v[(4 * j)];
                                                 v[((4 * j) + 2)] += v[((4 * j) + 1)];
                                                 v[((4 * j) + 3)] += v[((4 * j) + 2)];
@@ -155,7 +155,7 @@ __global__ void lookback_scan_striped(const uint32_t* x, uint32_t* y, uint32_t* 
                     uint32_t before = look_back_wide(__block_id_1, __thread_id_1, __smem, status_blk, tile, spin_limit);
                     publish(__block_id_1, __thread_id_1, __smem, status_blk, tile, 2, (before + total));
                     {
-                        uint32_t* y_wave = y_tile + ((1024 * wave));
+                        uint32_t* y_wave = y_tile + ((4096 * wave));
                         {
                             int __block_id_2 = __block_id_1;
                             int __thread_id_2 = __thread_id_1 % 64;
@@ -171,7 +171,7 @@ __global__ void lookback_scan_striped(const uint32_t* x, uint32_t* y, uint32_t* 
                                 {
                                     int __block_id_3 = __block_id_2;
                                     int __thread_id_3 = __thread_id_2 % 1;
-                                    for (int j = 0; j < 4; j++) {
+                                    for (int j = 0; j < 16; j++) {
                                         for (int e = 0; e < 4; e++) {
                                             y_mine[((256 * j) + e)] = ((before + earlier_waves) + v[((4 * j) + e)]);
                                         }

@@ -384,29 +384,29 @@ def value_of_last_lane(val: uint32_t @ thread[1]) -> uint32_t @ thread[1]:
 @prism("global")
 def lookback_scan_striped(x: ptr(const(uint32_t)) @ grid[1], y: ptr(uint32_t) @ grid[1], counter: ptr(uint32_t) @ grid[1],
                           status: ptr(uint64_t) @ grid[1], spin_limit: int @ grid[1]):
-    """Tiles of 16384 elements as 64 rows of 256 (1024 threads); a wavefront owns four consecutive rows and a lane four consecutive
-    elements of each (one 16-byte access per row, the 64 lanes of an access side by side). Per row: the lane's
+    """Tiles of 65536 elements as 256 rows of 256 (1024 threads); a wavefront owns sixteen consecutive rows and a lane
+    four consecutive elements of each (one 16-byte access per row, the 64 lanes of an access side by side). Per row: the lane's
     four elements serially, the lane totals by lane shifts, and what the wavefront's earlier rows hold added on."""
     tile: uint32_t @ grid[1] = take_ticket(counter)
-    with partition(x, p=block[1], offset=tile * 16384) as x_tile:
-        with partition(y, p=block[1], offset=tile * 16384) as y_tile:
+    with partition(x, p=block[1], offset=tile * 65536) as x_tile:
+        with partition(y, p=block[1], offset=tile * 65536) as y_tile:
             with partition(status, p=block[1], offset=0) as status_blk:
                 with group(block[1]):
                     wave_sums: shared(uint32_t[16], static=True) @ block[1]
                     wave: int @ thread[64] = id()
-                    v: uint32_t[16] @ thread[1]
-                    with partition(x_tile, p=thread[64], offset=1024 * wave) as x_wave:
+                    v: uint32_t[64] @ thread[1]
+                    with partition(x_tile, p=thread[64], offset=4096 * wave) as x_wave:
                         with partition(wave_sums, p=thread[64], offset=wave) as my_wave_sum:
                             with group(thread[64]):
                                 lane: uint32_t @ thread[1] = id()
                                 with partition(x_wave, p=thread[1], offset=4 * lane) as x_mine:
                                     with partition(my_wave_sum, p=thread[1], offset=0) as sum_one:
                                         with group(thread[1]):
-                                            for j in range(4):
+                                            for j in range(16):
                                                 for e in range(4):
                                                     v[4 * j + e] = x_mine[256 * j + e]
                                             carry: uint32_t @ thread[1] = 0
-                                            for j in range(4):
+                                            for j in range(16):
                                                 v[4 * j + 1] += v[4 * j]
                                                 v[4 * j + 2] += v[4 * j + 1]
                                                 v[4 * j + 3] += v[4 * j + 2]
@@ -429,7 +429,7 @@ def lookback_scan_striped(x: ptr(const(uint32_t)) @ grid[1], y: ptr(uint32_t) @ 
                     publish(status_blk, tile, 1, total)
                     before: uint32_t @ block[1] = look_back_wide(status_blk, tile, spin_limit)
                     publish(status_blk, tile, 2, before + total)
-                    with partition(y_tile, p=thread[64], offset=1024 * wave) as y_wave:
+                    with partition(y_tile, p=thread[64], offset=4096 * wave) as y_wave:
                         with group(thread[64]):
                             lane_out: uint32_t @ thread[1] = id()
                             earlier_waves: uint32_t @ thread[64] = 0
@@ -438,6 +438,6 @@ def lookback_scan_striped(x: ptr(const(uint32_t)) @ grid[1], y: ptr(uint32_t) @ 
                                     earlier_waves += wave_sums[w]
                             with partition(y_wave, p=thread[1], offset=4 * lane_out) as y_mine:
                                 with group(thread[1]):
-                                    for j in range(4):
+                                    for j in range(16):
                                         for e in range(4):
                                             y_mine[256 * j + e] = before + earlier_waves + v[4 * j + e]
