@@ -186,7 +186,8 @@ def handed_over_gemm_big(P: ptr(const(bf16)) @ grid[1], Q: ptr(const(bf16)) @ gr
 # two slots of 32 k (48 KiB each: 128 rows of A with 128-byte rows, then 32 rows of B with 1 KiB rows).
 # Measured at 8192^3: 129 TFLOP/s; 150 with the loads taken out (hand-over still running, results invalid), so the
 # protocol and the consumers' schedule cost 5 % and the loads 13 %; four slots of 16 k, which let the producers
-# run further ahead, gave 124, and 256 x 256 tiles (42 registers spilled) 129: it is not the lead.
+# run further ahead, gave 124, three slots of 32 k 129, 256 x 256 tiles (42 registers spilled) 129: it is not the
+# lead. One, two, four, eight producer wavefronts: 107, 126, 129, 128; fills staged through registers: 104.
 
 @requires(thread[256])
 @prism("device")
