@@ -376,11 +376,11 @@ def write_traffic_table(pmc_dir: str) -> int:
             return 1
         scale[counter] = (1 << 20) / (sum(v) / len(v))  # the copy moves 1 GiB = 2^20 KiB each way
     lines = ["# HBM-side traffic per launch (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)", "",
-             "Written by `python bench.py --traffic-summary $R/gpurun_out/pmc_traffic` from four counter runs (from /tmp with",
-             "TMPDIR=/tmp on the GPU box, R = repo root, C = FETCH_SIZE, then WRITE_SIZE; each run its own process):", "",
-             "    rocprofv3 --pmc $C --kernel-trace -d $R/gpurun_out/pmc_traffic -o bench_$C --output-format csv -- \\",
+             "Written by `python bench.py --traffic-summary $OUT/pmc_traffic` from four counter runs (from /tmp with TMPDIR=/tmp on",
+             "the GPU box, R = repo root, OUT = a scratch directory, C = FETCH_SIZE, then WRITE_SIZE; each run its own process):", "",
+             "    rocprofv3 --pmc $C --kernel-trace -d $OUT/pmc_traffic -o bench_$C --output-format csv -- \\",
              "        python3 $R/bench.py --steps 3 --warmup 1 --no-configs --no-cpu-baseline",
-             "    rocprofv3 --pmc $C --kernel-trace -d $R/gpurun_out/pmc_traffic -o calib_$C --output-format csv -- \\",
+             "    rocprofv3 --pmc $C --kernel-trace -d $OUT/pmc_traffic -o calib_$C --output-format csv -- \\",
              "        python3 $R/bench.py --workload calibrate --steps 3 --warmup 1", "",
              "`bench.py` reads the table back for `roofline.traffic`. A row counts only while the hash of its kernel source",
              "(first 16 hex digits of the SHA-256 of `prism_amd/csrc/<file>`) is the one in the tree; otherwise the bench line",

@@ -1,7 +1,7 @@
 // A stand-in for the three harness mains of the reference (evals/4090_scan/main.cu + scan_harness.cuh:112-168,
 // evals/4090_sgemm/main.cu:84-147, evals/h100_bench/main.cu:112-141), reduced to their correctness runs, around
-// the launcher replacements that INTEGRATION.md shows. The test that builds this file extracts those code blocks
-// from INTEGRATION.md into integration_snippets.inc, so the text a maintainer would paste is the text compiled,
+// the launcher replacements that the integration guide shows. The test that builds this file extracts those code
+// blocks from the guide into integration_snippets.inc, so the text a maintainer would paste is the text compiled,
 // linked against libprism_amd.so and run here. Host code only: device memory comes from the HIP runtime API.
 #include <hip/hip_runtime_api.h>
 

@@ -1,9 +1,9 @@
-"""The launcher replacements that INTEGRATION.md shows to a maintainer of the reference's harnesses, compiled
+"""The launcher replacements that the integration guide shows to a maintainer of the reference's harnesses, compiled
 as C++ against include/prism_amd.h, linked with libprism_amd.so and run.
 
 tests/native/harness_main.cpp is this repository's own stand-in for the three harness mains (their
 correctness runs in outline: scan_harness.cuh:112-168, 4090_sgemm/main.cu:84-147, h100_bench/main.cu:123-141);
-the C++ code blocks of INTEGRATION.md sections 1-3 are extracted verbatim into the file it includes, so the
+the C++ code blocks of the guide's sections 1-3 are extracted verbatim into the file it includes, so the
 documentation's snippets are what is compiled and executed. Host code only (g++ against the HIP runtime API).
 """
 import re
@@ -23,7 +23,7 @@ def build_harness(out_dir: Path) -> Path:
     text = (ROOT / "INTEGRATION.md").read_text()
     head = text[text.index("## 1. Scan harness"):text.index("## 4. add_m")]
     blocks = re.findall(r"```cpp\n(.*?)```", head, flags=re.S)
-    assert len(blocks) == 3, "INTEGRATION.md sections 1-3 should hold one C++ block each"
+    assert len(blocks) == 3, "sections 1-3 of the integration guide should hold one C++ block each"
     out_dir.mkdir(parents=True, exist_ok=True)
     (out_dir / "integration_snippets.inc").write_text("\n".join(blocks))
     exe = out_dir / "native_harness"
