@@ -24,9 +24,11 @@
 // the general 128 x 128 block kernel for shapes and alignments the others refuse.
 // The two direct-to-LDS kernels have edge variants for ragged M, N, K with N and K
 // multiples of 4 (16 B-aligned rows): their loads go through buffer descriptors
-// whose range check zero-fills everything beyond the matrices. Other shapes and
-// alignments take the general kernel, whose edge variant uses range-checked
-// 16 B buffer loads plus masks.
+// whose range check zero-fills everything beyond the matrices. The workgroup
+// kernel also has a form for rows that are only 4 B aligned (any N and K,
+// matrices at any element). What is left (small problems with such rows, K < 4,
+// offsets beyond 32 bits) takes the general kernel, whose edge variant uses
+// range-checked 16 B buffer loads plus masks.
 //
 // Unlike the reference kernels (no guards in kernels 1, 3, 4, 5), every kernel
 // here accepts any M, N, K. When beta == 0, C is not read.
@@ -441,10 +443,22 @@ __attribute__((amdgpu_waves_per_eu(4))) void sgemm_wave_tile_kernel(
 // chunk into sub-tile j: the two k values of a 32x32x2 instruction are
 // k8 + jj and k8 + 4 + jj, and lane l32 of sub-tile j holds column 4 l32 + j,
 // so a lane owns 4 consecutive columns of C and stores them as one 16 B packet.
-template <int BM, int BN, int BK, int WM, int WN, bool EDGE>
+//
+// RAGGED (with EDGE): N and K need not be multiples of 4 and the matrices need only be 4 B aligned. The 16 B
+// loads then start at 4 B-aligned addresses, which the memory path accepts, and a descriptor's range check
+// is made dword by dword, so that a chunk that straddles an extent's end arrives with its outer dwords
+// zeroed (both measured on gfx950). The K loop covers K rounded down to a multiple of 4, where every A
+// chunk lies inside its row; a B chunk that straddles the end of a row brings the head of the next row
+// into columns >= N, which are never stored. The last K % 4 values of k are added in front of the
+// write-back from ordinary loads, and C is written element by element where a chunk straddles N.
+template <int BM, int BN, int BK, int WM, int WN, bool EDGE, bool RAGGED = false>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile_dma_kernel(
-    int M, int N, int K, float alpha, const float* __restrict__ A, const float* __restrict__ B,
+    int M, int N, int K_all, float alpha, const float* __restrict__ A, const float* __restrict__ B,
     float beta, float* C, int tiles_m, int tiles_n, int first_big) {
+    static_assert(EDGE || !RAGGED, "the ragged form is an edge form");
+    // lda: elements between A rows. K: the part of the k range the loop covers.
+    const int lda = K_all;
+    const int K = RAGGED ? K_all - K_all % 4 : K_all;
     constexpr int WAVES_N = BN / WN;
     constexpr int WAVES = (BM / WM) * WAVES_N;
     constexpr int MI = WM / 32, NI = 4;
@@ -508,11 +522,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
     // a vector ALU instruction between two MFMAs delays the second one.
     const int ld_row = wave * ROWS_PER_LOAD + lane / KP;
     const int ld_chunk = (lane % KP) ^ ((ld_row >> SWZ) & (KP - 1));
-    const uint32_t a_lane = (static_cast<uint32_t>(lane / KP) * static_cast<uint32_t>(K) + ld_chunk * 4) * 4u;  // bytes
+    const uint32_t a_lane = (static_cast<uint32_t>(lane / KP) * static_cast<uint32_t>(lda) + ld_chunk * 4) * 4u;  // bytes
     const uint32_t b_lane = static_cast<uint32_t>(lane) * 16u;
-    const char* a_wave = reinterpret_cast<const char*>(A + static_cast<size_t>(row0 + wave * ROWS_PER_LOAD) * K);
+    const char* a_wave = reinterpret_cast<const char*>(A + static_cast<size_t>(row0 + wave * ROWS_PER_LOAD) * lda);
     const char* b_wave = reinterpret_cast<const char*>(B + static_cast<size_t>(wave) * N + col0);
-    const size_t a_pass = static_cast<size_t>(ROWS_PER_PASS) * K * 4;
+    const size_t a_pass = static_cast<size_t>(ROWS_PER_PASS) * lda * 4;
     const size_t b_pass = static_cast<size_t>(WAVES) * N * 4;
 
     // EDGE: M, N, K need not be whole tiles (N and K multiples of 4, so that rows stay 16 B aligned and
@@ -521,7 +535,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
     // the end of a row is the next row, so there the lane offset is replaced by one beyond any extent:
     // B columns >= N (fixed per lane) and, in the partial K tile, A chunks with k >= K.
     const int a_first = row0 + wave * ROWS_PER_LOAD;              // this wave's first A row
-    const long long a_left = static_cast<long long>(M - a_first) * K * 4;
+    const long long a_left = static_cast<long long>(M - a_first) * lda * 4;
     const long long b_left = (static_cast<long long>(K - wave) * N - col0) * 4;
     const i32x4 a_rsrc = buffer_descriptor(EDGE && a_left > 0 ? static_cast<const void*>(a_wave) : static_cast<const void*>(A),
                                            EDGE ? clamped_extent(a_left) : 0u);
@@ -681,7 +695,65 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
             __builtin_amdgcn_sched_barrier(0);  // at most one 32-row block of C reads in flight (64 registers)
         }
     };
-    if (beta == 0.0f) write_back(no{}); else write_back(yes{});
+    if constexpr (!RAGGED) {
+        if (beta == 0.0f) write_back(no{}); else write_back(yes{});
+    } else {
+        // The k values the loop left out (K_all % 4 of them): a lane adds them to its 16 rows x 4 columns
+        // per 32-row block from ordinary loads.
+        const int k_tail = K_all - K;
+        if (k_tail > 0 && c_col < N) {
+            float bt[3][NI];
+#pragma unroll
+            for (int t = 0; t < 3; ++t)
+#pragma unroll
+                for (int j = 0; j < NI; ++j)
+                    bt[t][j] = (t < k_tail && c_col + j < N) ? B[static_cast<size_t>(K + t) * N + c_col + j] : 0.0f;
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int row = c_row + i * 32 + 8 * (v / 4) + (v % 4);
+                    if (row >= M) continue;
+                    const float* a_row = A + static_cast<size_t>(row) * lda + K;
+#pragma unroll
+                    for (int t = 0; t < 3; ++t)
+                        if (t < k_tail) {
+                            const float a = a_row[t];
+#pragma unroll
+                            for (int j = 0; j < NI; ++j) acc[i][j][v] = __builtin_fmaf(a, bt[t][j], acc[i][j][v]);
+                        }
+                }
+        }
+        // C rows are 4 B aligned only: whole chunks as 16 B accesses at that alignment, the chunk that
+        // straddles N element by element.
+        typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+        const bool read_c = beta != 0.0f;
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int r_in = i * 32 + 8 * (v / 4) + (v % 4);
+                if (c_row + r_in >= M || c_col >= N) continue;
+                float* c = c_lane + static_cast<size_t>(r_in) * N;
+                if (c_col + NI <= N) {
+                    f32x4_a4* c4 = reinterpret_cast<f32x4_a4*>(c);
+                    f32x4 old = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                    if (read_c) old = *c4;
+                    f32x4 r;
+#pragma unroll
+                    for (int j = 0; j < NI; ++j)
+                        r[j] = read_c ? __builtin_fmaf(alpha, acc[i][j][v], beta * old[j]) : alpha * acc[i][j][v];
+                    *c4 = r;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < NI; ++j)
+                        if (c_col + j < N)
+                            c[j] = read_c ? __builtin_fmaf(alpha, acc[i][j][v], beta * c[j]) : alpha * acc[i][j][v];
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
 }
 
 // -------------------------------------------- kernel 5, one wave per tile --
@@ -1015,11 +1087,14 @@ int run_wave_tile(int M, int N, int K, float alpha, const float* A, const float*
 template <int BM, int BN, int BK, int WM, int WN, bool ALLOW_EDGES>
 bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const float* B, float beta,
                        float* C, hipStream_t s, int* rc) {
-    if (K <= 0 || !aligned16(A) || !aligned16(B) || !aligned16(C)) return false;
-    const bool whole = M % BM == 0 && N % BN == 0 && K % BK == 0;
-    // Ragged edges: rows must stay 16 B aligned, and the kernel's buffer offsets are 32 bits wide
-    // (a 256-row panel of A plus one K tile; all of B plus one K tile).
-    if (!whole && (!ALLOW_EDGES || N % 4 || K % 4 ||
+    if (K <= 0) return false;
+    const bool aligned = aligned16(A) && aligned16(B) && aligned16(C);
+    const bool whole = aligned && M % BM == 0 && N % BN == 0 && K % BK == 0;
+    // Edges: the kernel's buffer offsets are 32 bits wide (a 256-row panel of A plus one K tile; all of B
+    // plus one K tile). Rows that do not stay 16 B aligned (N or K not a multiple of 4, or matrices that
+    // are only 4 B aligned) take the ragged form, whose K loop needs at least one group of 4.
+    const bool ragged = !whole && (!aligned || N % 4 || K % 4);
+    if (!whole && (!ALLOW_EDGES || (ragged && K < 4) ||
                    (static_cast<long long>(BM) + 64) * K * 4 >= (1ll << 31) ||
                    (static_cast<long long>(K) + 64) * N * 4 >= (1ll << 31)))
         return false;
@@ -1033,7 +1108,16 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
     const int tiles = tiles_m * tiles_n, cus = cu_count();
     int main_tiles = tiles, leftover_wt = 0;
     const bool lane_offsets_fit = static_cast<long long>(K) * 64 < (1ll << 30) && static_cast<long long>(N) * 64 < (1ll << 30);
-    if (lane_offsets_fit && tiles > cus && tiles % cus != 0 && K >= 64) {
+    if (ragged && lane_offsets_fit && tiles > cus && tiles % cus != 0 && K >= 64) {
+        // The one-wave kernels have no ragged form: 64 x 256 slices, which cost about 0.27 of a round per
+        // slice on the fullest CU (128 x 256 halves cost 0.58 per half, never less), when three to a CU do.
+        const int left = tiles % cus;
+        if (left * 4 <= 3 * cus) {
+            main_tiles = tiles - left;
+            leftover_wt = 256;
+        }
+    }
+    if (!ragged && lane_offsets_fit && tiles > cus && tiles % cus != 0 && K >= 64) {
         // Cost of the last round in units of one full round of 256 x 256 tiles: a wave tile of 64 (32)
         // is 1/4 (1/16) of a SIMD's share of a big tile and runs at about 0.87 (0.72) of its rate.
         const int left = tiles % cus, simds = 4 * cus;
@@ -1061,21 +1145,23 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
         }
     }
     // `edge` selects the zero-filling variants of both kernels (sub-tiles that lie wholly outside C exit at once).
-    auto launch = [&](auto edge) {
-        constexpr bool EDGE = decltype(edge)::value;
-        sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, EDGE><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
+    auto launch = [&](auto edge, auto ragged_rows) {
+        constexpr bool EDGE = decltype(edge)::value, RAGGED = decltype(ragged_rows)::value;
+        sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, EDGE, RAGGED><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
             M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
         *rc = check_launch("sgemm_wave_tile_dma_kernel");
         if (*rc == 0 && leftover_wt == 128) {
             // 128 x 256 halves of the same kernel, one workgroup to a CU
-            sgemm_wave_tile_dma_kernel<128, 256, 16, 32, 128, EDGE><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 2), dim3(512), 0, s>>>(
+            sgemm_wave_tile_dma_kernel<128, 256, 16, 32, 128, EDGE, RAGGED><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 2), dim3(512), 0, s>>>(
                 M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, main_tiles);
             *rc = check_launch("sgemm_wave_tile_dma_kernel (leftover halves)");
         } else if (*rc == 0 && leftover_wt == 256) {
             // 64 x 256 slices of the same kernel, three workgroups to a CU
-            sgemm_wave_tile_dma_kernel<64, 256, 16, 32, 128, EDGE><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 4), dim3(256), 0, s>>>(
+            sgemm_wave_tile_dma_kernel<64, 256, 16, 32, 128, EDGE, RAGGED><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 4), dim3(256), 0, s>>>(
                 M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, main_tiles);
             *rc = check_launch("sgemm_wave_tile_dma_kernel (leftover slices)");
+        } else if constexpr (RAGGED) {
+            // no one-wave form for rows that are not 16 B aligned
         } else if (*rc == 0 && leftover_wt == 64) {
             sgemm_single_wave_kernel<64, 4, EDGE><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 16), dim3(kWave), 0, s>>>(
                 M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, main_tiles);
@@ -1087,9 +1173,11 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
         }
     };
     if (whole) {
-        launch(std::false_type{});
+        launch(std::false_type{}, std::false_type{});
+    } else if (!ragged) {
+        if constexpr (ALLOW_EDGES) launch(std::true_type{}, std::false_type{});
     } else {
-        if constexpr (ALLOW_EDGES) launch(std::true_type{});
+        if constexpr (ALLOW_EDGES) launch(std::true_type{}, std::true_type{});
     }
     return true;
 }
@@ -1103,9 +1191,11 @@ template <int BM, bool ALLOW_EDGES>
 bool try_half_tile_dma(int M, int N, int K, float alpha, const float* A, const float* B, float beta,
                        float* C, hipStream_t s, int* rc) {
     constexpr int BN = 256, BK = 16, WM = 32, WN = 128;
-    if (K <= 0 || !aligned16(A) || !aligned16(B) || !aligned16(C)) return false;
-    const bool whole = M % BM == 0 && N % BN == 0 && K % BK == 0;
-    if (!whole && (!ALLOW_EDGES || N % 4 || K % 4 ||
+    if (K <= 0) return false;
+    const bool aligned = aligned16(A) && aligned16(B) && aligned16(C);
+    const bool whole = aligned && M % BM == 0 && N % BN == 0 && K % BK == 0;
+    const bool ragged = !whole && (!aligned || N % 4 || K % 4);
+    if (!whole && (!ALLOW_EDGES || (ragged && K < 4) ||
                    (static_cast<long long>(BM) + 64) * K * 4 >= (1ll << 31) ||
                    (static_cast<long long>(K) + 64) * N * 4 >= (1ll << 31)))
         return false;
@@ -1116,9 +1206,12 @@ bool try_half_tile_dma(int M, int N, int K, float alpha, const float* A, const f
     const dim3 grid(static_cast<unsigned>(tiles)), block((BM / WM) * (BN / WN) * kWave);
     if (whole) {
         sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, false><<<grid, block, 0, s>>>(M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
-    } else {
+    } else if (!ragged) {
         if constexpr (ALLOW_EDGES)
             sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, true><<<grid, block, 0, s>>>(M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
+    } else {
+        if constexpr (ALLOW_EDGES)
+            sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, true, true><<<grid, block, 0, s>>>(M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
     }
     *rc = check_launch("sgemm_wave_tile_dma_kernel (128 x 256)");
     return true;
@@ -1207,13 +1300,14 @@ int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, 
                 // Whole 256 x 256 tiles for at least three quarters of the CUs: the direct-to-LDS kernel,
                 // K tiles of 32 (128 KiB of LDS) when K allows, else of 16.
                 int rc = 0;
-                // Ragged M, N, K (N and K multiples of 4) take the K-tile-of-32 kernel with zero-filled edges.
+                // Ragged M, N, K take the K-tile-of-32 kernel with zero-filled edges (its ragged form when
+                // rows are not 16 B aligned).
                 if (try_wave_tile_dma<256, 256, 32, 32, 128, true>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
                 if (try_wave_tile_dma<256, 256, 16, 32, 128, false>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
                 // Small problems (at most one 64 x 64 tile per SIMD): one wave per tile, 32 x 32 tiles when
                 // 64 x 64 ones would leave SIMDs without work. In between, the direct-to-LDS kernel on
                 // 128 x 256 tiles (at most one per CU) or 64 x 256 tiles (at most three per CU); what is left
-                // (N or K not a multiple of 4, unaligned operands) goes to the general kernel.
+                // (small problems whose rows are not 16 B aligned) goes to the general kernel.
                 const long long simds = 4ll * cu_count();
                 const long long tiles64 = static_cast<long long>(ceil_div(M, 64)) * ceil_div(N, 64);
                 if (tiles64 <= simds) {

@@ -284,6 +284,52 @@ def test_wave_tile_mid_sizes(prism, oracle, shape):
         assert np.max(np.abs(got - oracle.np_sgemm_f64(1.25, A, B, beta, Cm))) <= tol(oracle, K, A, B, beta, Cm)
 
 
+@pytest.mark.parametrize("shape", [(3581, 3582, 101), (3584, 3585, 67), (3585, 3587, 38), (3500, 3601, 5), (3841, 3333, 233),
+                                   (3584, 3584, 7), (3584, 3584, 64), (2300, 2566, 101), (3001, 3333, 69), (2304, 2305, 4),
+                                   (4300, 4349, 101), (4090, 5117, 70), (5377, 5375, 66)])
+def test_wave_tile_rows_not_16_byte_aligned(prism, oracle, shape):
+    """N or K not a multiple of 4, or matrices that start at an odd element: rows are then only 4 B aligned and
+    the direct-to-LDS kernel runs in its ragged form (256 x 256 tiles for the first seven shapes, 128 x 256 and
+    64 x 256 tiles for the next three; the last three have 289, 320 and 462 tiles for 256 CUs, so the 33, 64 and
+    206 tiles of their partial last round are cut into 64 x 256 slices, or not at all): 16 B loads from 4 B-aligned addresses, a K loop over K rounded down to a
+    multiple of 4 with the last K % 4 values added in front of the write-back, and C written element by element
+    where a chunk straddles N. A and B sit between NaNs and C is fenced; every element is checked, with and
+    without reading C, with the matrices at an even and at an odd element."""
+    M, N, K = shape
+    A, B, Cm = oracle.gen_sgemm(M, N, K, seed=M + 7 * K)
+    for beta, start, c_at in ((0.5, 1024, 256), (0.0, 1021, 255), (0.5, 1022, 257)):
+        buf = torch.full((M * N + 512,), 777.0, dtype=torch.float32, device=DEV)
+        c = buf[c_at:c_at + M * N].view(M, N)
+        c.copy_(dev(Cm))
+        prism.sgemm(M, N, K, 1.25, nan_fenced(A, start), nan_fenced(B, start), beta, c, variant=5)
+        out = host(buf)
+        assert np.all(out[:c_at] == 777.0) and np.all(out[c_at + M * N:] == 777.0)
+        got = out[c_at:c_at + M * N].reshape(M, N)
+        assert np.max(np.abs(got - oracle.np_sgemm_f64(1.25, A, B, beta, Cm))) <= tol(oracle, K, A, B, beta, Cm)
+
+
+def test_wave_tile_ragged_rows_keep_infinities_in_their_row(prism, oracle):
+    """An infinite element of A belongs to one row of C only. With K % 4 != 0 the 16 B chunk that holds the
+    end of row r of A also holds the head of row r + 1; the ragged form must not let that reach row r
+    (0 x inf would turn it into NaN). Likewise an infinite element in the first column of B stays in column 0."""
+    M, N, K = 3584, 3585, 67
+    A, B, Cm = oracle.gen_sgemm(M, N, K, seed=11)
+    A[1000, 0] = np.inf
+    B[5, 0] = np.inf
+    c = dev(Cm).clone()
+    prism.sgemm(M, N, K, 1.0, dev(A), dev(B), 0.0, c, variant=5)
+    got = host(c)
+    clean = np.ones((M, N), dtype=bool)
+    clean[1000, :] = False
+    clean[:, 0] = False
+    assert np.all(np.isfinite(got[clean]))
+    assert not np.any(np.isfinite(got[1000, :])) and not np.any(np.isfinite(got[:, 0]))
+    A[1000, 0] = 0.0
+    B[5, 0] = 0.0
+    want = oracle.np_sgemm_f64(1.0, A, B, 0.0, Cm)
+    assert np.max(np.abs(got[clean] - want[clean])) <= tol(oracle, K, A, B, 0.0, Cm)
+
+
 def test_wave_tile_ragged_tall_matrix(prism, oracle):
     """A ragged A of more than 4 GiB: the bytes from a tile's first row to the end of A do not fit the 32 bits
     of a buffer descriptor's extent and are cut to 2 GiB - 1 (a tile only reaches 256 rows ahead). Rows are
