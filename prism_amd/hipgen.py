@@ -48,6 +48,7 @@ from pathlib import Path
 from typing import Callable, Dict, List, Optional
 
 __all__ = ["prism", "requires", "attr", "grid", "block", "thread", "ptr", "const", "restrict", "constexpr",
+           "GLOBAL", "SHARED", "LOCAL",
            "shared", "uint", "double", "uint32_t", "uint64_t", "group", "partition", "claim", "split", "unsafe",
            "generate", "generate_launcher", "build", "HipgenError"]
 
@@ -139,8 +140,27 @@ float4 = _TypeName("float4")
 float4_cast = _TypeName("float4_cast")  # float4_cast(x[i]) reads, float4_cast[x[i]] = v writes 16 bytes at &x[i]
 
 
-def ptr(t) -> CType:
+def ptr(t, space=None) -> CType:
+    """`ptr(T)` or `ptr(T, GLOBAL | SHARED | LOCAL)` (prism/type_checker.py:656-667); the address space does not
+    show in the C text: HIP's generic pointers cover global memory, LDS and private arrays alike."""
     return CType(_ctype_text(t) + "*")
+
+
+# The address spaces a pointer type may name. `ptr(T, SHARED)` is what `shared(T)` is as a parameter type: a
+# pointer into LDS, which the barrier analysis follows; `ptr(T, LOCAL)` points at a thread's private array
+# and may be stored through at any perspective.
+GLOBAL, SHARED, LOCAL = (_TypeName(n) for n in ("GLOBAL", "SHARED", "LOCAL"))
+ADDRESS_SPACES = ("GLOBAL", "SHARED", "LOCAL")
+
+
+def address_space_of(node: ast.AST) -> str:
+    """The address space a `ptr(T[, SPACE])` call node names (GLOBAL when it names none)."""
+    if len(node.args) < 2:
+        return "GLOBAL"
+    space = node.args[1]
+    if not isinstance(space, ast.Name) or space.id not in ADDRESS_SPACES:
+        raise HipgenError(f"line {getattr(node, 'lineno', '?')}: the address space of a pointer is GLOBAL, SHARED or LOCAL")
+    return space.id
 
 
 def group(_where):  # only ever appears inside kernel bodies, which are parsed, not run
@@ -232,6 +252,9 @@ def _type_of(node: ast.AST) -> str:
         if node.id in _SCALARS:
             return _SCALARS[node.id]
         raise HipgenError(f"line {node.lineno}: unsupported type {node.id}")
+    if isinstance(node, ast.Call) and isinstance(node.func, ast.Name) and node.func.id == "ptr" and len(node.args) == 2:
+        address_space_of(node)
+        return _type_of(node.args[0]) + "*"
     if isinstance(node, ast.Call) and isinstance(node.func, ast.Name) and len(node.args) == 1:
         inner = _type_of(node.args[0])
         if node.func.id == "ptr":

@@ -81,7 +81,7 @@ import ast
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Set, Tuple
 
-from .hipgen import HipgenError, Kernel, _BINOPS, _CMPOPS, _REGISTRY, _UNOPS
+from .hipgen import HipgenError, Kernel, _BINOPS, _CMPOPS, _REGISTRY, _UNOPS, address_space_of
 
 _TYPES = {"int": ("int", 4), "float": ("float", 4), "double": ("double", 8), "bool": ("bool", 1),
           "uint": ("unsigned int", 4), "unsigned": ("unsigned int", 4), "uint32_t": ("uint32_t", 4),
@@ -129,6 +129,7 @@ class _Scalar:
         if isinstance(node, ast.Call) and isinstance(node.func, ast.Name) and node.args:
             inner = _Scalar.text(node.args[0])
             if node.func.id == "ptr":
+                address_space_of(node)   # ptr(T, GLOBAL | SHARED | LOCAL): checked here, the same `T*` in the text
                 # ptr(shared(T)) and ptr(const(shared(T))): shared() already made the pointer
                 a = node.args[0]
                 into_lds = _is_call(a, "shared") or (_is_call(a, "const") and a.args and _is_call(a.args[0], "shared"))
@@ -183,9 +184,10 @@ class _SyncPlan:
         self.covered: Dict[int, Set[str]] = {}                     # id(match) -> arrays handed over inside it
         self.wait_before: Dict[int, List[Tuple[str, str]]] = {}    # id(stmt) -> [(array, "full" | "empty")]
         self.signal_after: Dict[int, List[Tuple[str, str]]] = {}
-        for a in fn.args.args:            # a parameter declared ptr(shared(T)) points into LDS (prism/sync_analysis.py:151-158)
-            if a.arg != "template" and a.annotation is not None and any(
-                    _is_call(n, "shared") for n in ast.walk(_annotation(a.annotation)[0])):
+        for a in fn.args.args:            # a parameter declared ptr(shared(T)) or ptr(T, SHARED) points into LDS
+            if a.arg != "template" and a.annotation is not None and any(   # (prism/sync_analysis.py:151-158)
+                    _is_call(n, "shared") or (_is_call(n, "ptr") and address_space_of(n) == "SHARED")
+                    for n in ast.walk(_annotation(a.annotation)[0])):
                 self.root[a.arg] = a.arg
         self._collect(fn.body)
         self._plan_handovers(fn.body)
@@ -491,7 +493,8 @@ class BlockEmitter:
         self.id_level: Optional[Tuple[str, int]] = None  # perspective `id()` resolves against
         self.returns_value = False
         self.plan: Optional[_SyncPlan] = None
-        self.views: Dict[str, Tuple[str, ast.Lambda]] = {}  # f=lambda view -> (array it indexes, the lambda)
+        # f=lambda view -> (array it indexes, the lambda, the level p= names: what id() means inside the lambda)
+        self.views: Dict[str, Tuple[str, ast.Lambda, Optional[Tuple[str, int]]]] = {}
         self.bound: Dict[str, str] = {}                     # lambda parameter -> text of the index in hand
 
     # -- text helpers
@@ -544,11 +547,13 @@ class BlockEmitter:
 
     def view_element(self, view: str, index: str) -> str:
         """`view[index]` for a view declared with f=lambda: the element of the underlying array."""
-        parent, fn = self.views[view]
+        parent, fn, level = self.views[view]
         param = fn.args.args[0].arg
         saved = self.bound.get(param)
         self.bound[param] = index
+        saved_level, self.id_level = self.id_level, (level or self.id_level)
         mapped = self.expr(fn.body)
+        self.id_level = saved_level
         if saved is None:
             del self.bound[param]
         else:
@@ -928,7 +933,7 @@ class BlockEmitter:
             if target.id in self.views or target.id in self.pointer_type:
                 raise HipgenError(f"{_line(s)}: {target.id} is already the name of an array or view")
             # No pointer is declared: every element access goes through the index map.
-            self.views[target.id] = (parent, fn)
+            self.views[target.id] = (parent, fn, _level(kw["p"]) if "p" in kw else None)
             self.pointer_type[target.id] = ctype
             self.block(s.body)
             del self.views[target.id]
@@ -962,7 +967,10 @@ class BlockEmitter:
                 for item in d.elts:
                     if not (isinstance(item, ast.Tuple) and len(item.elts) == 2 and isinstance(item.elts[0], ast.Constant)):
                         raise HipgenError("template= takes a list of (name, type) pairs")
-                    self.template.append((_Scalar.text(item.elts[1]), str(item.elts[0].value)))
+                    ttype = item.elts[1]
+                    if _is_call(ttype, "constexpr") and ttype.args:   # every template parameter is a constant already
+                        ttype = ttype.args[0]
+                    self.template.append((_Scalar.text(ttype), str(item.elts[0].value)))
                 continue
             if a.annotation is None:
                 raise HipgenError(f"parameter {a.arg} needs a `type @ perspective` annotation")

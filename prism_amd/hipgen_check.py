@@ -44,7 +44,7 @@ import ast
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Set, Tuple
 
-from .hipgen import HipgenError, _REGISTRY
+from .hipgen import HipgenError, _REGISTRY, address_space_of
 
 _ORDER = {"grid": 0, "block": 1, "thread": 2}
 _SKIPPED_CALLS = {"id", "range", "group", "split", "requires", "prism", "shared", "ptr", "const", "restrict",
@@ -140,6 +140,12 @@ def _kind_of_type(t: ast.AST) -> str:
         if name == "shared":
             return "pointer"
         if name == "ptr":
+            try:
+                space = address_space_of(t)
+            except HipgenError as e:
+                raise PerspectiveError(str(e)) from None
+            if space == "LOCAL":    # a thread's private array: indexed and stored through like one
+                return "array"      # (prism/type_checker.py:399-403, 436-441)
             inner = t.args[0] if t.args else None
             if isinstance(inner, ast.Call) and isinstance(inner.func, ast.Name) and inner.func.id == "const":
                 return "const pointer"
@@ -153,6 +159,9 @@ def _kind_of_type(t: ast.AST) -> str:
 def _shared_bytes(t: ast.Call, constants: Dict[str, int]) -> int:
     sizes = {"int": 4, "float": 4, "double": 8, "bool": 1, "uint": 4, "unsigned": 4, "uint32_t": 4, "uint64_t": 8,
              "float4": 16, "bf16": 2}
+    # static=True arrays are sized by the compiler and do not draw on the budget (prism/type_checker.py:466-473)
+    if any(kw.arg == "static" and isinstance(kw.value, ast.Constant) and kw.value.value is True for kw in t.keywords):
+        return 0
     arg = t.args[0] if t.args else None
     if not isinstance(arg, ast.Subscript) or not isinstance(arg.value, ast.Name):
         return 0
@@ -202,7 +211,7 @@ class _Checker:
         if grid is not None or block is not None:
             thread = thread or P("thread", 1)
         self.bound = Bound(grid, block, thread)
-        self.smem_left = k.smem if k.smem is not None else None
+        self.smem_left = k.smem if k.smem is not None else 0   # no smem=: no budget (prism/type_checker.py:288-292)
         self.scopes: List[Dict[str, Symbol]] = [{}]
         self.partitioned: List[Set[str]] = [set()]
         self.claimed: List[Set[str]] = []
