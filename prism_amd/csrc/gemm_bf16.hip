@@ -16,8 +16,11 @@
 //                                               8x4 patch per XCD (tile_map.h)
 //   K tail dropped, M/N multiples required  ->  any M, N, K. Ragged M, N, K with K a multiple of 8
 //                                               (16 B-aligned rows): the same kernels, edges zero-filled
-//                                               by the buffer loads' range check. Anything else (K not a
-//                                               multiple of 8, operands not 16 B aligned):
+//                                               by the buffer loads' range check. K not a multiple of 8
+//                                               or operands not 16 B aligned, from 128 tiles up: the
+//                                               early-read kernel's ragged form (16 B loads from 2 B-
+//                                               aligned addresses, the last K % 8 values of k added on
+//                                               the way out). Smaller problems of that kind:
 //                                               gemm_bf16_kernel (guarded loads, 16 B where a packet
 //                                               lies inside its row; staged in registers one K step
 //                                               ahead, padded LDS rows)
@@ -554,10 +557,19 @@ __device__ __forceinline__ void mfma_results_settle() {
 // what those instructions multiply), a barrier in mid-phase then says that nobody reads the stage any
 // more, and the loads of the tile after next are issued into it right away: about one and a half tile
 // times before they are needed.
-template <int BM, int BN, int WM, int WN, bool EDGE, typename OutT>
+//
+// RAGGED (with EDGE): K need not be a multiple of 8 and P, Q need only be 2 B aligned. The 16 B loads then
+// start at 2 B-aligned addresses, which the memory path accepts (measured on gfx950, for the lane offset and
+// for the descriptor's base). The K loop covers K rounded down to a multiple of 8, where every chunk lies
+// inside its row, and the last K % 8 values of k are added in front of the write-back from ordinary loads.
+template <int BM, int BN, int WM, int WN, bool EDGE, typename OutT, bool RAGGED = false>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early_kernel(
-    int R, int Cn, int K, const uint16_t* __restrict__ P, const uint16_t* __restrict__ Q,
+    int R, int Cn, int K_all, const uint16_t* __restrict__ P, const uint16_t* __restrict__ Q,
     OutT* __restrict__ OUT, int tiles_m, int tiles_n) {
+    static_assert(EDGE || !RAGGED, "the ragged form is an edge form");
+    // ld: elements between rows of P and of Q. K: the part of the k range the loop covers.
+    const int ld = K_all;
+    const int K = RAGGED ? K_all - K_all % 8 : K_all;
     constexpr int BK = 64, KP = 8, SWZ = 1;
     constexpr int WAVES_N = BN / WN;
     constexpr int WAVES = (BM / WM) * WAVES_N;
@@ -590,9 +602,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     // Load side, as in gemm_bf16_ring_kernel.
     const int ld_row = wave * ROWS_PER_LOAD + lane / KP;
     const int ld_chunk = (lane % KP) ^ ((ld_row >> SWZ) & (KP - 1));
-    const uint32_t lane_off = (static_cast<uint32_t>(lane / KP) * static_cast<uint32_t>(K) + ld_chunk * 8) * 2u;
-    const char* p_wave = reinterpret_cast<const char*>(P + static_cast<size_t>(row0 + wave * ROWS_PER_LOAD) * K);
-    const char* q_wave = reinterpret_cast<const char*>(Q + static_cast<size_t>(col0 + wave * ROWS_PER_LOAD) * K);
+    const uint32_t lane_off = (static_cast<uint32_t>(lane / KP) * static_cast<uint32_t>(ld) + ld_chunk * 8) * 2u;
+    const char* p_wave = reinterpret_cast<const char*>(P + static_cast<size_t>(row0 + wave * ROWS_PER_LOAD) * ld);
+    const char* q_wave = reinterpret_cast<const char*>(Q + static_cast<size_t>(col0 + wave * ROWS_PER_LOAD) * ld);
     // The loads go through two buffer descriptors (this wave's first P row, its first Q row) for their
     // addressing mode, not for range checks: descriptor base + scalar offset + lane offset, where the scalar
     // offset (load number x rows per pass) and the lane offset are loop-invariant and only the two bases
@@ -607,9 +619,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     // extent, and in the K tiles that pad the count to an even number of at least 4 all lanes do.
     // (Forced into a scalar register here: direct_load16_buffer_to_destination takes its scalar operands as
     // they are, so that no v_readfirstlane ends up right in front of a load.)
-    const uint32_t pass_bytes = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(ROWS_PER_PASS) * static_cast<uint32_t>(K) * 2u);  // the launcher keeps BM * K * 2 below 2^31
+    const uint32_t pass_bytes = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(ROWS_PER_PASS) * static_cast<uint32_t>(ld) * 2u);  // the launcher keeps BM * K * 2 below 2^31
     const int p_first = row0 + wave * ROWS_PER_LOAD, q_first = col0 + wave * ROWS_PER_LOAD;
-    const long long p_left = static_cast<long long>(R - p_first) * K * 2, q_left = static_cast<long long>(Cn - q_first) * K * 2;
+    const long long p_left = static_cast<long long>(R - p_first) * ld * 2, q_left = static_cast<long long>(Cn - q_first) * ld * 2;
     const i32x4 p_rsrc = buffer_descriptor(EDGE && p_left <= 0 ? reinterpret_cast<const char*>(P) : p_wave, EDGE ? clamped_extent(p_left) : 0x7fffffffu);
     const i32x4 q_rsrc = buffer_descriptor(EDGE && q_left <= 0 ? reinterpret_cast<const char*>(Q) : q_wave, EDGE ? clamped_extent(q_left) : 0x7fffffffu);
     auto advanced = [](i32x4 d, uint32_t bytes) {  // the descriptor with its base moved up
@@ -803,8 +815,58 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
             }
         }
     };
-    if (!EDGE || (row0 + BM <= R && col0 + BN <= Cn)) write_back(std::false_type{});
-    else write_back(std::true_type{});
+    if constexpr (RAGGED) {
+        // The k values the loop left out (K_all % 8 of them, at most 7) are added on the way out. A lane holds
+        // 32 rows x 8 columns; the tail of a row is one 16 B chunk (k = K .. K + 7, the last of them the head of
+        // the next row), fetched with a range-checked buffer load so that nothing past a matrix is touched;
+        // slots beyond the tail and rows beyond the matrix become zeros. The range check works on dwords: with
+        // an odd tail the very last element of a matrix shares its dword with what lies beyond and arrives as
+        // zero; it is fetched again on its own. The product of two bf16 values is exact in fp32.
+        auto as_float = [](uint32_t bits16) { return __builtin_bit_cast(float, bits16 << 16); };
+        const int tail = K_all - K;  // wave-uniform, 0 .. 7
+        auto tails_of = [&](const uint16_t* base, int first, int rows, int row, float (&out)[7]) {
+            // `base`: the matrix; `first`: this tile's first row of it; `rows`: its row count; `row`: the lane's row
+            const long long left = static_cast<long long>(rows - first) * ld * 2;
+            const auto rsrc = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<uint16_t*>(base + (left > 0 ? static_cast<size_t>(first) * ld : size_t{0})), 0,
+                static_cast<int>(clamped_extent(left)), 0x00020000);
+            const u32x4 c = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                rsrc, (static_cast<uint32_t>(row - first) * static_cast<uint32_t>(ld) + static_cast<uint32_t>(K)) * 2u, 0, 0));
+            const bool last_of_matrix = (tail & 1) && row == rows - 1;
+            const float last = last_of_matrix ? as_float(base[static_cast<size_t>(row) * ld + K_all - 1]) : 0.0f;
+#pragma unroll
+            for (int t = 0; t < 7; ++t) {
+                const uint32_t bits = (t & 1) ? (c[t / 2] >> 16) : (c[t / 2] & 0xffffu);
+                out[t] = (t < tail && row < rows) ? as_float(bits) : 0.0f;
+                if (last_of_matrix && t == tail - 1) out[t] = last;
+            }
+        };
+        float qt[NI][7];
+#pragma unroll
+        for (int j = 0; j < NI; ++j) tails_of(Q, col0, Cn, col0 + wave_n * WN + j * 16 + l16, qt[j]);
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+            float pt[4][7];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) tails_of(P, row0, R, row0 + wave_m * WM + i * 16 + 4 * lq + v, pt[v]);
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+                const int col = col0 + wave_n * WN + j * 16 + l16;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int row = row0 + wave_m * WM + i * 16 + 4 * lq + v;
+                    float r = acc[i][j][v];
+#pragma unroll
+                    for (int t = 0; t < 7; ++t) r = __builtin_fmaf(pt[v][t], qt[j][t], r);
+                    if (row < R && col < Cn) store_out(&OUT[static_cast<size_t>(row) * Cn + col], r);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);  // one row block at a time: its 28 P values and no more
+        }
+    } else {
+        if (!EDGE || (row0 + BM <= R && col0 + BN <= Cn)) write_back(std::false_type{});
+        else write_back(std::true_type{});
+    }
     // The last, redundant loads write LDS: they must have landed before the wave ends and its LDS goes to
     // the next workgroup. Behind the write-back the wait is covered by the stores.
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));
@@ -813,7 +875,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
 // Kernel choice. Whole 256 x 256 x 64 tiles: the early-read pipeline whenever the K tile count is even and
 // at least 6, else the direct-to-LDS ring (any count from 2). Ragged M, N or K with K a multiple of 8 and
 // 16 B-aligned operands: the early-read pipeline's edge variant (K tiles padded with zeros to an even count).
-// Fewer than 128 tiles: 128 x 128 tiles of the ring. Everything else: the general kernel.
+// Rows that are not 16 B aligned, from 128 tiles up: its ragged form. Fewer than 128 tiles: 128 x 128 tiles of
+// the ring. Everything else: the general kernel.
 template <int BM, int BN, int BK, int WM, int WN, typename OutT>
 int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, OutT* OUT,
                   hipStream_t s) {
@@ -876,6 +939,12 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
     if (aligned && K % 8 == 0 && K > 0 && panel_ok && lane_offsets_ok) {
         gemm_bf16_early_kernel<BM, BN, WM, WN, true, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
         return check_launch("gemm_bf16_early_kernel (edges)");
+    }
+    // Rows that are not 16 B aligned (K not a multiple of 8, or operands at an odd element): its ragged form,
+    // when there are enough tiles for the CUs and at least one group of 8 along K.
+    if (!few_tiles && K >= 8 && panel_ok && lane_offsets_ok) {
+        gemm_bf16_early_kernel<BM, BN, WM, WN, true, OutT, true><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
+        return check_launch("gemm_bf16_early_kernel (ragged rows)");
     }
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<BM, BN, BK, WM, WN, true, OutT>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));

@@ -77,11 +77,12 @@ def test_whole_tile_paths(prism, oracle, shape):
     assert np.all(np.abs(c - ref) <= 2.0**-8 * np.abs(ref) + REL * np.abs(ref).max())
 
 
-def nan_fenced(a16: np.ndarray) -> torch.Tensor:
-    """The matrix as a view into a device buffer whose other elements are bf16 NaN patterns (16 B-aligned start)."""
+def nan_fenced(a16: np.ndarray, start: int = 1024) -> torch.Tensor:
+    """The matrix as a view into a device buffer whose other elements are bf16 NaN patterns; `start` is its
+    first element's index (a multiple of 8 keeps it 16 B aligned)."""
     buf = torch.full((a16.size + 2048,), 0x7FC0, dtype=torch.int16, device=DEV)
-    buf[1024:1024 + a16.size] = torch.from_numpy(np.ascontiguousarray(a16).view(np.int16).ravel()).to(DEV)
-    return buf[1024:1024 + a16.size].view(torch.bfloat16).view(a16.shape)
+    buf[start:start + a16.size] = torch.from_numpy(np.ascontiguousarray(a16).view(np.int16).ravel()).to(DEV)
+    return buf[start:start + a16.size].view(torch.bfloat16).view(a16.shape)
 
 
 @pytest.mark.parametrize("shape", [(1, 1, 8), (257, 255, 8), (300, 520, 392), (255, 513, 456), (512, 512, 72), (1000, 1000, 1000),
@@ -112,6 +113,33 @@ def test_ragged_shapes_with_aligned_rows(prism, oracle, shape):
     guard = np.float32(-7.0).view(np.uint32) >> 16
     assert np.all(got[:32] == guard) and np.all(got[32 + N * M:] == guard)
     c = oracle.bf16_to_f32(got[32:32 + N * M]).reshape(N, M).T
+    assert np.all(np.abs(c - ref) <= 2.0**-8 * np.abs(ref) + REL * np.abs(ref).max())
+
+
+@pytest.mark.parametrize("shape", [(3000, 3080, 393), (2900, 3100, 75), (3072, 3072, 9), (3000, 3072, 647), (3072, 3072, 15),
+                                   (3072, 3072, 264), (2817, 3001, 406)])
+def test_rows_not_16_byte_aligned(prism, oracle, shape):
+    """K not a multiple of 8, or operands that start at an odd element: rows are then only 2 B or 4 B aligned
+    and, from 128 tiles of 256 x 256 up, the early-read kernel runs in its ragged form: 16 B direct loads from
+    2 B-aligned addresses, a K loop over K rounded down to a multiple of 8 (1 to 11 tiles here, padded to an
+    even count of at least 4), and the last K % 8 values of k added on the way out. The matrices sit between
+    NaNs at an even and at an odd element; stores are fenced; fp32 and bf16 outputs."""
+    M, N, K = shape
+    A16, B16 = oracle.gen_gemm_bf16(M, N, K, seed=5 * M + N + K)
+    ref = oracle.gemm_bf16_f64(A16, B16)
+    for start in ((1025, 1030) if K % 8 == 0 else (1024, 1025)):  # K % 8 == 0 at a multiple of 8: the aligned edge variant
+        buf = torch.full((M * N + 512,), 777.0, dtype=torch.float32, device=DEV)
+        D = buf[255:255 + M * N].view(M, N)
+        prism.gemm_bf16(nan_fenced(A16, start), nan_fenced(B16, start), D)
+        out = host(buf)
+        assert np.all(out[:255] == 777.0) and np.all(out[255 + M * N:] == 777.0)
+        check_f32(oracle, out[255:255 + M * N].reshape(M, N), A16, B16, ref)
+    Cc = torch.full((N * M + 64,), -7.0, dtype=torch.bfloat16, device=DEV)
+    prism.runmyh100(M, N, K, nan_fenced(A16, 1027), nan_fenced(B16, 1029), Cc[31:31 + N * M])
+    got = host(Cc.view(torch.int16)).view(np.uint16)
+    guard = np.float32(-7.0).view(np.uint32) >> 16
+    assert np.all(got[:31] == guard) and np.all(got[31 + N * M:] == guard)
+    c = oracle.bf16_to_f32(got[31:31 + N * M]).reshape(N, M).T
     assert np.all(np.abs(c - ref) <= 2.0**-8 * np.abs(ref) + REL * np.abs(ref).max())
 
 
