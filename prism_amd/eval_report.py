@@ -21,10 +21,11 @@ offers through PyTorch: rocBLAS/hipBLASLt `torch.matmul` and rocPRIM
 
 `generated` runs the same protocols over the kernels that prism_amd.hipgen prints from the example programs
 (prism_amd/examples), which is what the reference's figures show for its own back-end: "My Kernel" 1..5 are
-naive_sgemm, remapped_sgemm, tiled_sgemm<32>, vector_tile_sgemm<128,128,8,8,8> and handed_over_sgemm (the
-producer / consumer kernel on the fp32 matrix instruction; sizes it does not take, below 1024, are left out),
-the scan is lookback_scan_striped, and "Kernel:" in the bf16 sweep is handed_over_gemm_big (fp32 row-major output,
-where the reference's kernel writes bf16 column-major). The kernels are compiled for gfx950 on the spot.
+naive_sgemm, remapped_sgemm, tiled_sgemm<32>, vector_tile_sgemm<128,128,8,8,8> and, on the fp32 matrix
+instruction, pipelined_sgemm from 4096 up and handed_over_sgemm (the producer / consumer kernel) at 1024 and 2048
+(smaller sizes, which neither takes, are left out), the scan is lookback_scan_striped, and "Kernel:" in the bf16
+sweep is pipelined_gemm_bf16 from 4096 up and handed_over_gemm_big below (fp32 row-major output, where the
+reference's kernel writes bf16 column-major). The kernels are compiled for gfx950 on the spot.
 """
 from __future__ import annotations
 
@@ -202,6 +203,8 @@ def sweep_generated(out=sys.stdout, sgemm_sizes=SGEMM_SIZES, scan_log2_sizes=SCA
              3: ("tiled_sgemm", 32, lambda n: n // 32, lambda n: (n // 32) ** 2),
              4: ("vector_tile_sgemm", 128, lambda n: n // 128, lambda n: (n // 128) ** 2),
              5: ("handed_over_sgemm", 1024, lambda n: n // 256, lambda n: (n // 128) * (n // 256))}
+    # from 4096 up kernel 5 is the program in which every wavefront loads and multiplies (256 x 256 tiles)
+    big5 = ("pipelined_sgemm", 4096, lambda n: n // 256, lambda n: (n // 256) ** 2)
     alpha, beta = 0.5, 3.0
     top = max(sgemm_sizes)
     A = torch.rand((top, top), device="cuda") * 2 - 1
@@ -219,6 +222,8 @@ def sweep_generated(out=sys.stdout, sgemm_sizes=SGEMM_SIZES, scan_log2_sizes=SCA
         ms = _events_ms(lambda: torch.addmm(ref, a, b, beta=beta, alpha=alpha, out=ref), repeats)
         print(sgemm_line(ms / 1e3 / repeats, repeats * flops * 1e-9 / (ms / 1e3), n), file=out)
         for k, (name, smallest, last, blocks) in steps.items():
+            if k == 5 and n >= big5[1] and n % 2048 == 0:
+                name, smallest, last, blocks = big5
             if n < smallest:
                 continue
             launch = kernel(name)
@@ -260,16 +265,19 @@ def sweep_generated(out=sys.stdout, sgemm_sizes=SGEMM_SIZES, scan_log2_sizes=SCA
     print("", file=out)
     del x, work
 
-    gemm = kernel("handed_over_gemm_big")
-    gemm.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int] * 4 + [ctypes.c_uint, ctypes.c_void_p]
     for n in h100_sizes:
+        # 256 x 256 tiles with every wavefront loading and multiplying from 4096 up, the producer / consumer
+        # kernel on 128 x 256 tiles below (twice the workgroups)
+        name, rows = ("pipelined_gemm_bf16", 256) if n >= 4096 and n % 2048 == 0 else ("handed_over_gemm_big", 128)
+        gemm = kernel(name)
+        gemm.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int] * 4 + [ctypes.c_uint, ctypes.c_void_p]
         P = torch.randn((n, n), device="cuda").to(torch.bfloat16)
         Q = torch.randn((n, n), device="cuda").to(torch.bfloat16)
         D = torch.empty((n, n), dtype=torch.float32, device="cuda")
         flops = 2.0 * n * n * n
-        fn = lambda: gemm(P.data_ptr(), Q.data_ptr(), D.data_ptr(), n, n, n // 128, n // 256, (n // 128) * (n // 256), None)
+        fn = lambda: gemm(P.data_ptr(), Q.data_ptr(), D.data_ptr(), n, n, n // rows, n // 256, (n // rows) * (n // 256), None)
         if fn() != 0:
-            raise RuntimeError(f"handed_over_gemm_big failed to launch at {n}")
+            raise RuntimeError(f"{name} failed to launch at {n}")
         ms = _events_ms(fn, 8)
         print(h100_line("Kernel:", ms / 1e3 / 8, 8 * flops * 1e-9 / ms, n), file=out)
         vend = lambda: torch.matmul(P, Q.T)

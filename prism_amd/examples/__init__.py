@@ -37,6 +37,8 @@ KERNELS: Dict[str, Tuple[str, int, Optional[List[int]]]] = {
     "handed_over_gemm": ("handover", 320, None),
     "handed_over_gemm_big": ("handover", 768, None),
     "handed_over_sgemm": ("handover", 768, None),
+    "pipelined_sgemm": ("pipelined", 1024, None),
+    "pipelined_gemm_bf16": ("pipelined", 512, None),
 }
 # device functions, printed on their own as well (the reference prints its scan's helpers one file each)
 DEVICE_FUNCTIONS: Dict[str, str] = {
@@ -46,6 +48,8 @@ DEVICE_FUNCTIONS: Dict[str, str] = {
     "look_back": "scan", "scan_rows": "scan", "collect_row_ends": "scan", "scan_row_ends": "scan", "write_back": "scan",
     "fill_slot": "handover", "multiply_slot": "handover", "fill_slot_f32": "handover", "multiply_slot_f32": "handover",
     "look_back_wide": "scan", "value_of_last_lane": "scan",
+    "fill_stage_f32": "pipelined", "multiply_stage_f32": "pipelined",
+    "fill_stage_bf16": "pipelined", "multiply_stage_bf16": "pipelined",
 }
 GENERATED = Path(__file__).resolve().parent / "generated"
 
