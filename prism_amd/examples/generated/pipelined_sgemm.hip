@@ -40,9 +40,9 @@ __global__ __launch_bounds__(1024) void pipelined_sgemm(int M, int N, int K, flo
                             {
                                 int __block_id_3 = __block_id_2;
                                 int __thread_id_3 = __thread_id_2 % 1;
-                                for (int j = 0; j < 4; j++) {
-                                    for (int v = 0; v < 16; v++) {
-                                        int at = ((((((((32 * (wave / 2)) + (8 * (v / 4))) + (4 * (lane / 32))) + (v % 4)) * N) + (128 * (wave % 2))) + (32 * j)) + (lane % 32));
+                                for (int v = 0; v < 16; v++) {
+                                    for (int j = 0; j < 4; j++) {
+                                        int at = ((((((((32 * (wave / 2)) + (8 * (v / 4))) + (4 * (lane / 32))) + (v % 4)) * N) + (128 * (wave % 2))) + (4 * (lane % 32))) + j);
                                         C_mine[at] = ((alpha * acc[((j * 16) + v)]) + (beta * C_mine[at]));
                                     }
                                 }

@@ -37,9 +37,12 @@ def fill_stage_f32(stage: ptr(float) @ block[1], A_from: ptr(const(float)) @ blo
 @requires(thread[1024])
 @prism("device")
 def multiply_stage_f32(acc: ptr(float) @ thread[1], stage: ptr(const(float)) @ block[1]):
-    """Sixteen wavefronts, eight down and two across, each adding its 32 x 128 strip of (A part)(B part) to acc:
-    sixteen pairs of k values, four instructions of 32 x 32 x 2 per pair;
-    acc[j * 16 + v] = C[8 (v / 4) + 4 (lane / 32) + v % 4][32 j + lane % 32] of the strip."""
+    """Sixteen wavefronts, eight down and two across, each adding its 32 x 128 strip of (A part)(B part) to acc.
+    Operands come in 16-byte LDS reads: per group of 8 k a lane (l32, half) takes the chunk of 4 k values
+    8 s + 4 half .. + 3 of its A row and, for each of those k, 4 consecutive B columns 4 l32 .. 4 l32 + 3.
+    Instruction (jj, j) multiplies k = 8 s + jj (lower half-wavefront) and 8 s + 4 + jj (upper half) into
+    sub-tile j, whose lane l32 thereby holds column 4 l32 + j:
+    acc[j * 16 + v] = C[8 (v / 4) + 4 half + v % 4][4 l32 + j] of the strip."""
     with group(thread[1024]):
         wave: int @ thread[64] = id()
         row0: int @ thread[64] = 32 * (wave / 2)
@@ -47,16 +50,17 @@ def multiply_stage_f32(acc: ptr(float) @ thread[1], stage: ptr(const(float)) @ b
         with group(thread[64]):
             lane: int @ thread[1] = id()
             l32: int @ thread[1] = lane % 32
-            a: float @ thread[1]
-            b: float[4] @ thread[1]
-            for kk in range(0, 32, 2):
-                k: int @ thread[1] = kk + lane / 32
-                a = stage[(row0 + l32) * 32 + 4 * ((k / 4) ^ ((l32 / 2) % 8)) + k % 4]
-                for j in range(4):
-                    b[j] = stage[8192 + k * 256 + col0 + 32 * j + l32]
-                for j in range(4):
-                    intrinsic.mfma_f32_32x32x2_f32(a, b[j], acc[j * 16 + 0], acc[j * 16 + 1], acc[j * 16 + 2], acc[j * 16 + 3], acc[j * 16 + 4], acc[j * 16 + 5], acc[j * 16 + 6], acc[j * 16 + 7], acc[j * 16 + 8], acc[j * 16 + 9], acc[j * 16 + 10], acc[j * 16 + 11], acc[j * 16 + 12], acc[j * 16 + 13], acc[j * 16 + 14], acc[j * 16 + 15],
-                                                   out=[acc[j * 16 + 0], acc[j * 16 + 1], acc[j * 16 + 2], acc[j * 16 + 3], acc[j * 16 + 4], acc[j * 16 + 5], acc[j * 16 + 6], acc[j * 16 + 7], acc[j * 16 + 8], acc[j * 16 + 9], acc[j * 16 + 10], acc[j * 16 + 11], acc[j * 16 + 12], acc[j * 16 + 13], acc[j * 16 + 14], acc[j * 16 + 15]])
+            half: int @ thread[1] = lane / 32
+            a: float[4] @ thread[1]
+            b: float[16] @ thread[1]
+            for s in range(4):
+                float4_cast[a[0]] = float4_cast(stage[(row0 + l32) * 32 + 4 * ((2 * s + half) ^ ((l32 / 2) % 8))])
+                for jj in range(4):
+                    float4_cast[b[4 * jj]] = float4_cast(stage[8192 + (8 * s + 4 * half + jj) * 256 + col0 + 4 * l32])
+                for jj in range(4):
+                    for j in range(4):
+                        intrinsic.mfma_f32_32x32x2_f32(a[jj], b[4 * jj + j], acc[j * 16 + 0], acc[j * 16 + 1], acc[j * 16 + 2], acc[j * 16 + 3], acc[j * 16 + 4], acc[j * 16 + 5], acc[j * 16 + 6], acc[j * 16 + 7], acc[j * 16 + 8], acc[j * 16 + 9], acc[j * 16 + 10], acc[j * 16 + 11], acc[j * 16 + 12], acc[j * 16 + 13], acc[j * 16 + 14], acc[j * 16 + 15],
+                                                       out=[acc[j * 16 + 0], acc[j * 16 + 1], acc[j * 16 + 2], acc[j * 16 + 3], acc[j * 16 + 4], acc[j * 16 + 5], acc[j * 16 + 6], acc[j * 16 + 7], acc[j * 16 + 8], acc[j * 16 + 9], acc[j * 16 + 10], acc[j * 16 + 11], acc[j * 16 + 12], acc[j * 16 + 13], acc[j * 16 + 14], acc[j * 16 + 15]])
     return
 
 
@@ -91,10 +95,10 @@ def pipelined_sgemm(M: int @ grid[1], N: int @ grid[1], K: int @ grid[1], alpha:
                         with group(thread[64]):
                             lane: int @ thread[1] = id()
                             with group(thread[1]):
-                                for j in range(4):
-                                    for v in range(16):
+                                for v in range(16):
+                                    for j in range(4):
                                         at: int @ thread[1] = (32 * (wave / 2) + 8 * (v / 4) + 4 * (lane / 32) + v % 4) * N \
-                                            + 128 * (wave % 2) + 32 * j + lane % 32
+                                            + 128 * (wave % 2) + 4 * (lane % 32) + j
                                         C_mine[at] = alpha * acc[j * 16 + v] + beta * C_mine[at]
 
 
