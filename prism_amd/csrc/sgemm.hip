@@ -24,11 +24,10 @@
 // the general 128 x 128 block kernel for shapes and alignments the others refuse.
 // The two direct-to-LDS kernels have edge variants for ragged M, N, K with N and K
 // multiples of 4 (16 B-aligned rows): their loads go through buffer descriptors
-// whose range check zero-fills everything beyond the matrices. The workgroup
-// kernel also has a form for rows that are only 4 B aligned (any N and K,
-// matrices at any element). What is left (small problems with such rows, K < 4,
-// offsets beyond 32 bits) takes the general kernel, whose edge variant uses
-// range-checked 16 B buffer loads plus masks.
+// whose range check zero-fills everything beyond the matrices. Both also have a
+// form for rows that are only 4 B aligned (any N and K, matrices at any
+// element). What is left (K < 4, offsets beyond 32 bits) takes the general
+// kernel, whose edge variant uses range-checked 16 B buffer loads plus masks.
 //
 // Unlike the reference kernels (no guards in kernels 1, 3, 4, 5), every kernel
 // here accepts any M, N, K. When beta == 0, C is not read.
@@ -783,10 +782,17 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
 // LDS and wave 0 adds them in the fixed order 0, 1, ..., KSPLIT - 1 (the same bits on every run) and
 // writes C. A K split across workgroups would need a workspace the entry points do not have; this one
 // needs none. (128 x 4096 x 4096: 512 tiles of 32 x 32 on 1024 SIMDs, 72 TFLOP/s unsplit.)
-template <int WT, int STAGES, bool EDGE, int KSPLIT = 1>
+//
+// RAGGED (with EDGE): rows that are only 4 B aligned (any N and K, matrices at any element), handled as in the
+// whole-tile kernel: 16 B loads from 4 B-aligned addresses, a K loop over K rounded down to a multiple of 4, the
+// last K % 4 values of k added in front of the write-back, C written element by element.
+template <int WT, int STAGES, bool EDGE, int KSPLIT = 1, bool RAGGED = false>
 __global__ __launch_bounds__(kWave * KSPLIT) void sgemm_single_wave_kernel(
-    int M, int N, int K, float alpha, const float* __restrict__ A, const float* __restrict__ B,
+    int M, int N, int K_all, float alpha, const float* __restrict__ A, const float* __restrict__ B,
     float beta, float* C, int tiles_m, int tiles_n, int first_big) {
+    static_assert(EDGE || !RAGGED, "the ragged form is an edge form");
+    const int lda = K_all;                                       // elements between A rows
+    const int K = RAGGED ? K_all - K_all % 4 : K_all;            // the part of the k range the loop covers
     constexpr int BK = 16, KP = 4, SWZ = 2, KS = 2;
     constexpr int MI = WT / 32, NI = WT / 32;
     static_assert(WT == 32 || WT == 64, "wave tile");
@@ -839,15 +845,15 @@ __global__ __launch_bounds__(kWave * KSPLIT) void sgemm_single_wave_kernel(
 
     // Load side (lane offsets in bytes, loop-invariant).
     const int a_chunk = (lane % KP) ^ (((lane / KP) >> SWZ) & (KP - 1));
-    const uint32_t a_lane = (static_cast<uint32_t>(lane / KP) * static_cast<uint32_t>(K) + a_chunk * 4) * 4u;
+    const uint32_t a_lane = (static_cast<uint32_t>(lane / KP) * static_cast<uint32_t>(lda) + a_chunk * 4) * 4u;
     // B: WT = 64: lane l fetches k-row l / 16, columns 4 (l % 16) ..; WT = 32: LDS position l holds
     // k-row (l / 16) + 4 ((l / 8) & 1), columns 4 (l % 8) .. (see the layout note above).
     const int b_krow = WT == 64 ? lane / 16 : (lane / 16) + 4 * ((lane / 8) & 1);
     const int b_col = WT == 64 ? 4 * (lane % 16) : 4 * (lane % 8);
     const uint32_t b_lane = (static_cast<uint32_t>(b_krow) * static_cast<uint32_t>(N) + b_col) * 4u;
-    const char* a_base = reinterpret_cast<const char*>(A + static_cast<size_t>(row0) * K + k_begin);
+    const char* a_base = reinterpret_cast<const char*>(A + static_cast<size_t>(row0) * lda + k_begin);
     const char* b_base = reinterpret_cast<const char*>(B + static_cast<size_t>(k_begin) * N + col0);
-    const i32x4 a_rsrc = buffer_descriptor(a_base, EDGE ? clamped_extent(static_cast<long long>(M - row0) * K * 4) : 0u);
+    const i32x4 a_rsrc = buffer_descriptor(a_base, EDGE ? clamped_extent(static_cast<long long>(M - row0) * lda * 4) : 0u);
     const i32x4 b_rsrc = buffer_descriptor(b_base, EDGE ? clamped_extent((static_cast<long long>(K) * N - col0) * 4) : 0u);
     const int k_full = K - K % BK;
     const uint32_t a_tail = (k_full + a_chunk * 4 < K) ? a_lane : kBeyondExtent;
@@ -856,7 +862,7 @@ __global__ __launch_bounds__(kWave * KSPLIT) void sgemm_single_wave_kernel(
         if constexpr (EDGE) {
             if (m < A_LOADS)
                 direct_load16_buffer(a_rsrc, k0 < k_full ? a_lane : (k0 < K ? a_tail : kBeyondExtent),
-                                     (static_cast<uint32_t>(m) * 16u * static_cast<uint32_t>(K) + k0) * 4u,
+                                     (static_cast<uint32_t>(m) * 16u * static_cast<uint32_t>(lda) + k0) * 4u,
                                      &As[stage][m * 16 * BK]);
             else
                 direct_load16_buffer(b_rsrc, b_edge,
@@ -864,7 +870,7 @@ __global__ __launch_bounds__(kWave * KSPLIT) void sgemm_single_wave_kernel(
                                      &Bs[stage][(m - A_LOADS) * B_ROWS_PER_LOAD * WT]);
         } else {
             if (m < A_LOADS)
-                direct_load16(a_base + (static_cast<size_t>(m) * 16 * K + k0) * 4, a_lane, &As[stage][m * 16 * BK]);
+                direct_load16(a_base + (static_cast<size_t>(m) * 16 * lda + k0) * 4, a_lane, &As[stage][m * 16 * BK]);
             else
                 direct_load16(b_base + static_cast<size_t>(k0 + (m - A_LOADS) * B_ROWS_PER_LOAD) * N * 4, b_lane,
                               &Bs[stage][(m - A_LOADS) * B_ROWS_PER_LOAD * WT]);
@@ -1042,7 +1048,48 @@ __global__ __launch_bounds__(kWave * KSPLIT) void sgemm_single_wave_kernel(
                 }
             }
     };
-    if (beta == 0.0f) write_back(no{}); else write_back(yes{});
+    if constexpr (!RAGGED) {
+        if (beta == 0.0f) write_back(no{}); else write_back(yes{});
+    } else {
+        const int c_row = row0 + 4 * lhi, c_col = col0 + NI * l32;
+        const int k_tail = K_all - K;
+        if (k_tail > 0 && c_col < N) {
+            float bt[3][NI];
+#pragma unroll
+            for (int t = 0; t < 3; ++t)
+#pragma unroll
+                for (int j = 0; j < NI; ++j)
+                    bt[t][j] = (t < k_tail && c_col + j < N) ? B[static_cast<size_t>(K + t) * N + c_col + j] : 0.0f;
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int row = c_row + i * 32 + 8 * (v / 4) + (v % 4);
+                    if (row >= M) continue;
+                    const float* a_row = A + static_cast<size_t>(row) * lda + K;
+#pragma unroll
+                    for (int t = 0; t < 3; ++t)
+                        if (t < k_tail) {
+                            const float a = a_row[t];
+#pragma unroll
+                            for (int j = 0; j < NI; ++j) acc[i][j][v] = __builtin_fmaf(a, bt[t][j], acc[i][j][v]);
+                        }
+                }
+        }
+        const bool read_c = beta != 0.0f;
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int r_in = i * 32 + 8 * (v / 4) + (v % 4);
+                if (c_row + r_in >= M) continue;
+                float* c = c_lane + static_cast<size_t>(r_in) * N;
+#pragma unroll
+                for (int j = 0; j < NI; ++j)
+                    if (c_col + j < N)
+                        c[j] = read_c ? __builtin_fmaf(alpha, acc[i][j][v], beta * c[j]) : alpha * acc[i][j][v];
+            }
+    }
 }
 
 // --------------------------------------------------------------- launchers --
@@ -1222,11 +1269,12 @@ template <int WT>
 bool try_single_wave(int M, int N, int K, float alpha, const float* A, const float* B, float beta, float* C,
                      hipStream_t s, int* rc, int ksplit = 1) {
     constexpr int STAGES = 4;
-    if (K <= 0 || !aligned16(A) || !aligned16(B) || !aligned16(C)) return false;
+    if (K <= 0) return false;
+    const bool aligned = aligned16(A) && aligned16(B) && aligned16(C);
     if (static_cast<long long>(K) * 64 >= (1ll << 30) || static_cast<long long>(N) * 64 >= (1ll << 30)) return false;
     const int tiles_m = ceil_div(M, WT), tiles_n = ceil_div(N, WT);
     const dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n);
-    if (M % WT == 0 && N % WT == 0 && K % (16 * ksplit) == 0 && K >= 16 * STAGES * ksplit) {
+    if (aligned && M % WT == 0 && N % WT == 0 && K % (16 * ksplit) == 0 && K >= 16 * STAGES * ksplit) {
         if (ksplit == 4 && WT == 32)
             sgemm_single_wave_kernel<32, STAGES, false, 4><<<grid, dim3(4 * kWave), 0, s>>>(
                 M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
@@ -1242,9 +1290,16 @@ bool try_single_wave(int M, int N, int K, float alpha, const float* A, const flo
         return true;
     }
     if (ksplit != 1) return false;
-    // Ragged edges: rows must stay 16 B aligned; all of B plus the padding K tiles is addressed with
-    // 32-bit byte offsets.
-    if (N % 4 || K % 4 || (static_cast<long long>(K) + 16 * STAGES) * N * 4 >= (1ll << 31)) return false;
+    // Ragged edges: all of B plus the padding K tiles is addressed with 32-bit byte offsets. Rows that do not
+    // stay 16 B aligned take the ragged form, whose K loop needs at least one group of 4.
+    if ((static_cast<long long>(K) + 16 * STAGES) * N * 4 >= (1ll << 31)) return false;
+    if (!aligned || N % 4 || K % 4) {
+        if (K < 4) return false;
+        sgemm_single_wave_kernel<WT, STAGES, true, 1, true><<<grid, dim3(kWave), 0, s>>>(
+            M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
+        *rc = check_launch("sgemm_single_wave_kernel (ragged rows)");
+        return true;
+    }
     sgemm_single_wave_kernel<WT, STAGES, true><<<grid, dim3(kWave), 0, s>>>(
         M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
     *rc = check_launch("sgemm_single_wave_kernel (edges)");
@@ -1307,7 +1362,7 @@ int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, 
                 // Small problems (at most one 64 x 64 tile per SIMD): one wave per tile, 32 x 32 tiles when
                 // 64 x 64 ones would leave SIMDs without work. In between, the direct-to-LDS kernel on
                 // 128 x 256 tiles (at most one per CU) or 64 x 256 tiles (at most three per CU); what is left
-                // (small problems whose rows are not 16 B aligned) goes to the general kernel.
+                // (K < 4, offsets that do not fit 32 bits) goes to the general kernel.
                 const long long simds = 4ll * cu_count();
                 const long long tiles64 = static_cast<long long>(ceil_div(M, 64)) * ceil_div(N, 64);
                 if (tiles64 <= simds) {

@@ -286,12 +286,14 @@ def test_wave_tile_mid_sizes(prism, oracle, shape):
 
 @pytest.mark.parametrize("shape", [(3581, 3582, 101), (3584, 3585, 67), (3585, 3587, 38), (3500, 3601, 5), (3841, 3333, 233),
                                    (3584, 3584, 7), (3584, 3584, 64), (2300, 2566, 101), (3001, 3333, 69), (2304, 2305, 4),
-                                   (4300, 4349, 101), (4090, 5117, 70), (5377, 5375, 66)])
+                                   (4300, 4349, 101), (4090, 5117, 70), (5377, 5375, 66),
+                                   (1001, 1001, 1001), (2001, 1999, 130), (64, 65, 6), (33, 31, 4), (700, 130, 77)])
 def test_wave_tile_rows_not_16_byte_aligned(prism, oracle, shape):
     """N or K not a multiple of 4, or matrices that start at an odd element: rows are then only 4 B aligned and
     the direct-to-LDS kernel runs in its ragged form (256 x 256 tiles for the first seven shapes, 128 x 256 and
     64 x 256 tiles for the next three; the last three have 289, 320 and 462 tiles for 256 CUs, so the 33, 64 and
-    206 tiles of their partial last round are cut into 64 x 256 slices, or not at all): 16 B loads from 4 B-aligned addresses, a K loop over K rounded down to a
+    206 tiles of their partial last round are cut into 64 x 256 slices, or not at all; the last five are small
+    problems for the one-wave-per-tile kernel's ragged form, 64 x 64 and 32 x 32 tiles, K tile counts from 1 up): 16 B loads from 4 B-aligned addresses, a K loop over K rounded down to a
     multiple of 4 with the last K % 4 values added in front of the write-back, and C written element by element
     where a chunk straddles N. A and B sit between NaNs and C is fenced; every element is checked, with and
     without reading C, with the matrices at an even and at an odd element."""
