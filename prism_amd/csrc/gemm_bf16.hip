@@ -17,13 +17,12 @@
 //   K tail dropped, M/N multiples required  ->  any M, N, K. Ragged M, N, K with K a multiple of 8
 //                                               (16 B-aligned rows): the same kernels, edges zero-filled
 //                                               by the buffer loads' range check. K not a multiple of 8
-//                                               or operands not 16 B aligned, from 128 tiles up: the
-//                                               early-read kernel's ragged form (16 B loads from 2 B-
-//                                               aligned addresses, the last K % 8 values of k added on
-//                                               the way out). Smaller problems of that kind:
-//                                               gemm_bf16_kernel (guarded loads, 16 B where a packet
-//                                               lies inside its row; staged in registers one K step
-//                                               ahead, padded LDS rows)
+//                                               or operands not 16 B aligned: the same kernels' ragged
+//                                               forms (16 B loads from 2 B-aligned addresses, the last
+//                                               K % 8 values of k added on the way out). K < 8 and
+//                                               offsets beyond 32 bits: gemm_bf16_kernel (guarded
+//                                               loads, 16 B where a packet lies inside its row; staged
+//                                               in registers one K step ahead, padded LDS rows)
 //
 // prism_gemm_bf16 calls it with (P, Q) = (A, B) and an fp32 OUT = D[M][N].
 // prism_runmyh100 needs the reference's column-major bf16 C (C[n * M + m],
@@ -270,6 +269,32 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_kerne
     }
 }
 
+// The last K_all - K (< 8) values of k of one row, for the kernels' ragged forms, whose K loops stop at K, a
+// multiple of 8: the row's tail is one 16 B chunk (k = K .. K + 7, its end the head of the next row), fetched
+// with a range-checked buffer load so that nothing past the matrix is touched; slots beyond the tail and rows
+// beyond the matrix become zeros. The range check works on dwords: with an odd tail the very last element of
+// the matrix shares its dword with what lies beyond and arrives as zero, so it is fetched again on its own.
+// `first`: the tile's first row (the descriptor starts there: offsets stay small), `rows`: the matrix's row count.
+__device__ __forceinline__ void load_k_tail(const uint16_t* base, int ld, int first, int rows, int row, int K, int K_all,
+                                            float (&out)[7]) {
+    auto as_float = [](uint32_t bits16) { return __builtin_bit_cast(float, bits16 << 16); };
+    const int tail = K_all - K;
+    const long long left = static_cast<long long>(rows - first) * ld * 2;
+    const auto rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(base + (left > 0 ? static_cast<size_t>(first) * ld : size_t{0})), 0,
+        static_cast<int>(clamped_extent(left)), 0x00020000);
+    const u32x4 c = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(
+        rsrc, (static_cast<uint32_t>(row - first) * static_cast<uint32_t>(ld) + static_cast<uint32_t>(K)) * 2u, 0, 0));
+    const bool last_of_matrix = (tail & 1) && row == rows - 1;
+    const float last = last_of_matrix ? as_float(base[static_cast<size_t>(row) * ld + K_all - 1]) : 0.0f;
+#pragma unroll
+    for (int t = 0; t < 7; ++t) {
+        const uint32_t bits = (t & 1) ? (c[t / 2] >> 16) : (c[t / 2] & 0xffffu);
+        out[t] = (t < tail && row < rows) ? as_float(bits) : 0.0f;
+        if (last_of_matrix && t == tail - 1) out[t] = last;
+    }
+}
+
 // ------------------------------------------------- direct-to-LDS ring kernel --
 // Whole tiles, K a multiple of BK and at least STAGES K tiles. Global data goes
 // straight into LDS (global_load_lds_dwordx4: no staging registers, no LDS write
@@ -302,10 +327,16 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_kerne
 // end with the matrices: rows beyond them arrive as zeros. Columns k >= K of a row are the next
 // row's data, so in the partial K tile those lanes use an offset beyond any extent; the K loop
 // runs over at least STAGES tiles, those beyond K all zeros.
-template <int BM, int BN, int BK, int STAGES, int WM, int WN, bool EDGE, typename OutT>
+//
+// RAGGED (with EDGE): K need not be a multiple of 8 and P, Q need only be 2 B aligned (16 B loads from 2 B-
+// aligned addresses); the K loop covers K rounded down to a multiple of 8 and the rest is added on the way out.
+template <int BM, int BN, int BK, int STAGES, int WM, int WN, bool EDGE, typename OutT, bool RAGGED = false>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_kernel(
-    int R, int Cn, int K, const uint16_t* __restrict__ P, const uint16_t* __restrict__ Q,
+    int R, int Cn, int K_all, const uint16_t* __restrict__ P, const uint16_t* __restrict__ Q,
     OutT* __restrict__ OUT, int tiles_m, int tiles_n, int first_big) {
+    static_assert(EDGE || !RAGGED, "the ragged form is an edge form");
+    const int ld = K_all;                                        // elements between rows of P and of Q
+    const int K = RAGGED ? K_all - K_all % 8 : K_all;            // the part of the k range the loop covers
     static_assert((BK == 32 || BK == 64) && (STAGES == 2 || STAGES == 4), "ring shape");
     constexpr int KP = BK / 8;                        // 16 B chunks per row
     constexpr int SWZ = KP == 4 ? 2 : 1;
@@ -362,13 +393,13 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_
     // Load side: lane l of a wave-wide load owns row l / KP of its rows and slot l % KP.
     const int ld_row = wave * ROWS_PER_LOAD + lane / KP;
     const int ld_chunk = (lane % KP) ^ ((ld_row >> SWZ) & (KP - 1));
-    const uint32_t lane_off = (static_cast<uint32_t>(lane / KP) * static_cast<uint32_t>(K) + ld_chunk * 8) * 2u;  // bytes
-    const char* p_wave = reinterpret_cast<const char*>(P + static_cast<size_t>(row0 + wave * ROWS_PER_LOAD) * K);
-    const char* q_wave = reinterpret_cast<const char*>(Q + static_cast<size_t>(col0 + wave * ROWS_PER_LOAD) * K);
-    const size_t pass_bytes = static_cast<size_t>(ROWS_PER_PASS) * K * 2;
+    const uint32_t lane_off = (static_cast<uint32_t>(lane / KP) * static_cast<uint32_t>(ld) + ld_chunk * 8) * 2u;  // bytes
+    const char* p_wave = reinterpret_cast<const char*>(P + static_cast<size_t>(row0 + wave * ROWS_PER_LOAD) * ld);
+    const char* q_wave = reinterpret_cast<const char*>(Q + static_cast<size_t>(col0 + wave * ROWS_PER_LOAD) * ld);
+    const size_t pass_bytes = static_cast<size_t>(ROWS_PER_PASS) * ld * 2;
     // Load number m (0 .. LOADS - 1) of the tile that starts at k0, into stage `stage`.
     const int p_first = row0 + wave * ROWS_PER_LOAD, q_first = col0 + wave * ROWS_PER_LOAD;
-    const long long p_left = static_cast<long long>(R - p_first) * K * 2, q_left = static_cast<long long>(Cn - q_first) * K * 2;
+    const long long p_left = static_cast<long long>(R - p_first) * ld * 2, q_left = static_cast<long long>(Cn - q_first) * ld * 2;
     const i32x4 p_rsrc = buffer_descriptor(EDGE && p_left > 0 ? static_cast<const void*>(p_wave) : static_cast<const void*>(P), EDGE ? clamped_extent(p_left) : 0u);
     const i32x4 q_rsrc = buffer_descriptor(EDGE && q_left > 0 ? static_cast<const void*>(q_wave) : static_cast<const void*>(Q), EDGE ? clamped_extent(q_left) : 0u);
     const int k_full = K - K % BK;
@@ -507,6 +538,31 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_
     }
     mfma_group(1, [](int) {});  // last k-group of the last tile
 
+    if constexpr (RAGGED) {
+        // The k values the loop left out are added on the way out (the product of two bf16 values is exact in
+        // fp32): a lane holds 16 rows per 32-row block and one column per 32-column block.
+        float qt[NI][7];
+#pragma unroll
+        for (int j = 0; j < NI; ++j) load_k_tail(Q, ld, col0, Cn, col0 + wave_n * WN + j * 32 + l32, K, K_all, qt[j]);
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = row0 + wave_m * WM + i * 32 + 8 * (v / 4) + 4 * lhi + (v % 4);
+                float pt[7];
+                load_k_tail(P, ld, row0, R, row, K, K_all, pt);
+#pragma unroll
+                for (int j = 0; j < NI; ++j) {
+                    const int col = col0 + wave_n * WN + j * 32 + l32;
+                    float r = acc[i][j][v];
+#pragma unroll
+                    for (int t = 0; t < 7; ++t) r = __builtin_fmaf(pt[t], qt[j][t], r);
+                    if (row < R && col < Cn) store_out(&OUT[static_cast<size_t>(row) * Cn + col], r);
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
 #pragma unroll
@@ -816,39 +872,16 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
         }
     };
     if constexpr (RAGGED) {
-        // The k values the loop left out (K_all % 8 of them, at most 7) are added on the way out. A lane holds
-        // 32 rows x 8 columns; the tail of a row is one 16 B chunk (k = K .. K + 7, the last of them the head of
-        // the next row), fetched with a range-checked buffer load so that nothing past a matrix is touched;
-        // slots beyond the tail and rows beyond the matrix become zeros. The range check works on dwords: with
-        // an odd tail the very last element of a matrix shares its dword with what lies beyond and arrives as
-        // zero; it is fetched again on its own. The product of two bf16 values is exact in fp32.
-        auto as_float = [](uint32_t bits16) { return __builtin_bit_cast(float, bits16 << 16); };
-        const int tail = K_all - K;  // wave-uniform, 0 .. 7
-        auto tails_of = [&](const uint16_t* base, int first, int rows, int row, float (&out)[7]) {
-            // `base`: the matrix; `first`: this tile's first row of it; `rows`: its row count; `row`: the lane's row
-            const long long left = static_cast<long long>(rows - first) * ld * 2;
-            const auto rsrc = __builtin_amdgcn_make_buffer_rsrc(
-                const_cast<uint16_t*>(base + (left > 0 ? static_cast<size_t>(first) * ld : size_t{0})), 0,
-                static_cast<int>(clamped_extent(left)), 0x00020000);
-            const u32x4 c = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(
-                rsrc, (static_cast<uint32_t>(row - first) * static_cast<uint32_t>(ld) + static_cast<uint32_t>(K)) * 2u, 0, 0));
-            const bool last_of_matrix = (tail & 1) && row == rows - 1;
-            const float last = last_of_matrix ? as_float(base[static_cast<size_t>(row) * ld + K_all - 1]) : 0.0f;
-#pragma unroll
-            for (int t = 0; t < 7; ++t) {
-                const uint32_t bits = (t & 1) ? (c[t / 2] >> 16) : (c[t / 2] & 0xffffu);
-                out[t] = (t < tail && row < rows) ? as_float(bits) : 0.0f;
-                if (last_of_matrix && t == tail - 1) out[t] = last;
-            }
-        };
+        // The k values the loop left out (K_all % 8 of them, at most 7) are added on the way out (load_k_tail
+        // above): a lane holds 32 rows x 8 columns. The product of two bf16 values is exact in fp32.
         float qt[NI][7];
 #pragma unroll
-        for (int j = 0; j < NI; ++j) tails_of(Q, col0, Cn, col0 + wave_n * WN + j * 16 + l16, qt[j]);
+        for (int j = 0; j < NI; ++j) load_k_tail(Q, ld, col0, Cn, col0 + wave_n * WN + j * 16 + l16, K, K_all, qt[j]);
 #pragma unroll
         for (int i = 0; i < MI; ++i) {
             float pt[4][7];
 #pragma unroll
-            for (int v = 0; v < 4; ++v) tails_of(P, row0, R, row0 + wave_m * WM + i * 16 + 4 * lq + v, pt[v]);
+            for (int v = 0; v < 4; ++v) load_k_tail(P, ld, row0, R, row0 + wave_m * WM + i * 16 + 4 * lq + v, K, K_all, pt[v]);
 #pragma unroll
             for (int j = 0; j < NI; ++j) {
                 const int col = col0 + wave_n * WN + j * 16 + l16;
@@ -875,8 +908,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
 // Kernel choice. Whole 256 x 256 x 64 tiles: the early-read pipeline whenever the K tile count is even and
 // at least 6, else the direct-to-LDS ring (any count from 2). Ragged M, N or K with K a multiple of 8 and
 // 16 B-aligned operands: the early-read pipeline's edge variant (K tiles padded with zeros to an even count).
-// Rows that are not 16 B aligned, from 128 tiles up: its ragged form. Fewer than 128 tiles: 128 x 128 tiles of
-// the ring. Everything else: the general kernel.
+// Rows that are not 16 B aligned: its ragged form. Fewer than 128 tiles: 128 x 128 tiles of the ring, with the
+// same edge and ragged forms. Everything else: the general kernel.
 template <int BM, int BN, int BK, int WM, int WN, typename OutT>
 int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, OutT* OUT,
                   hipStream_t s) {
@@ -912,6 +945,16 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
             return check_launch("gemm_bf16_ring_kernel (leftover)");
         }
         return 0;
+    }
+    // The same for rows that are not 16 B aligned (K not a multiple of 8, operands at an odd element).
+    if (few_tiles && !(aligned && K % 8 == 0) && K >= 8 && panel_ok) {
+        const int tm = ceil_div(R, 128), tn = ceil_div(Cn, 128);
+        const dim3 grid128(static_cast<unsigned>(tm) * tn);
+        if (K >= 256 && tm * tn <= cu_count())
+            gemm_bf16_ring_kernel<128, 128, 64, 4, 64, 64, true, OutT, true><<<grid128, dim3(256), 0, s>>>(R, Cn, K, P, Q, OUT, tm, tn, -1);
+        else
+            gemm_bf16_ring_kernel<128, 128, 64, 2, 64, 64, true, OutT, true><<<grid128, dim3(256), 0, s>>>(R, Cn, K, P, Q, OUT, tm, tn, -1);
+        return check_launch("gemm_bf16_ring_kernel (128 x 128, ragged rows)");
     }
     // Too few 256 x 256 tiles for the CUs: 128 x 128 tiles (four waves of 64 x 64), two workgroups per CU.
     if (few_tiles && aligned && K % 8 == 0 && K > 0 && panel_ok) {

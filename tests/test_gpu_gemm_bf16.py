@@ -117,12 +117,14 @@ def test_ragged_shapes_with_aligned_rows(prism, oracle, shape):
 
 
 @pytest.mark.parametrize("shape", [(3000, 3080, 393), (2900, 3100, 75), (3072, 3072, 9), (3000, 3072, 647), (3072, 3072, 15),
-                                   (3072, 3072, 264), (2817, 3001, 406)])
+                                   (3072, 3072, 264), (2817, 3001, 406),
+                                   (1001, 1001, 1001), (300, 520, 395), (257, 255, 9), (64, 64, 8), (2001, 1999, 130), (1000, 1000, 264)])
 def test_rows_not_16_byte_aligned(prism, oracle, shape):
     """K not a multiple of 8, or operands that start at an odd element: rows are then only 2 B or 4 B aligned
     and, from 128 tiles of 256 x 256 up, the early-read kernel runs in its ragged form: 16 B direct loads from
     2 B-aligned addresses, a K loop over K rounded down to a multiple of 8 (1 to 11 tiles here, padded to an
-    even count of at least 4), and the last K % 8 values of k added on the way out. The matrices sit between
+    even count of at least 4), and the last K % 8 values of k added on the way out; the last six shapes are small
+    problems for the ragged form of the ring of 128 x 128 tiles (two and four deep). The matrices sit between
     NaNs at an even and at an odd element; stores are fenced; fp32 and bf16 outputs."""
     M, N, K = shape
     A16, B16 = oracle.gen_gemm_bf16(M, N, K, seed=5 * M + N + K)
