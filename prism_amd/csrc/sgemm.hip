@@ -789,7 +789,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
 template <int WT, int STAGES, bool EDGE, int KSPLIT = 1, bool RAGGED = false>
 __global__ __launch_bounds__(kWave * KSPLIT) void sgemm_single_wave_kernel(
     int M, int N, int K_all, float alpha, const float* __restrict__ A, const float* __restrict__ B,
-    float beta, float* C, int tiles_m, int tiles_n, int first_big) {
+    float beta, float* C, int tiles_m, int tiles_n, int first_big, int big_rows = 256) {
     static_assert(EDGE || !RAGGED, "the ragged form is an edge form");
     const int lda = K_all;                                       // elements between A rows
     const int K = RAGGED ? K_all - K_all % 4 : K_all;            // the part of the k range the loop covers
@@ -812,9 +812,9 @@ __global__ __launch_bounds__(kWave * KSPLIT) void sgemm_single_wave_kernel(
     float (&Bs)[STAGES][BK * WT] = Bs_all[wave];
 
     // first_big < 0: the grid covers the whole tiles_m x tiles_n grid of WT x WT tiles. Otherwise this
-    // launch finishes what a launch of the 256 x 256 kernel left over: tiles_m x tiles_n is that kernel's
-    // grid, first_big the first tile number it did not take, and every leftover tile is cut into
-    // (256 / WT)^2 wave tiles.
+    // launch finishes what a launch of the workgroup kernel on big_rows x 256 tiles (big_rows = 256 or 64)
+    // left over: tiles_m x tiles_n is that kernel's grid, first_big the first tile number it did not take,
+    // and every leftover tile is cut into (big_rows / WT) x (256 / WT) wave tiles.
     int row0, col0;
     if (first_big < 0) {
         int tm, tn;
@@ -822,12 +822,13 @@ __global__ __launch_bounds__(kWave * KSPLIT) void sgemm_single_wave_kernel(
         row0 = tm * WT;
         col0 = tn * WT;
     } else {
-        constexpr int SUB = 256 / WT;
+        constexpr int SUB_N = 256 / WT;
+        const int per_big = (big_rows / WT) * SUB_N;
         int tm, tn;
-        xcd_tile_coords(first_big + blockIdx.x / (SUB * SUB), tiles_m, tiles_n, tm, tn);
-        const int sub = blockIdx.x % (SUB * SUB);
-        row0 = tm * 256 + (sub / SUB) * WT;
-        col0 = tn * 256 + (sub % SUB) * WT;
+        xcd_tile_coords(first_big + static_cast<int>(blockIdx.x) / per_big, tiles_m, tiles_n, tm, tn);
+        const int sub = static_cast<int>(blockIdx.x) % per_big;
+        row0 = tm * big_rows + (sub / SUB_N) * WT;
+        col0 = tn * 256 + (sub % SUB_N) * WT;
     }
     if (EDGE && (row0 >= M || col0 >= N)) return;  // a piece of an edge tile that lies wholly outside C
     const int lane = threadIdx.x % kWave;
@@ -1248,19 +1249,48 @@ bool try_half_tile_dma(int M, int N, int K, float alpha, const float* A, const f
         return false;
     const int tiles_m = ceil_div(M, BM), tiles_n = ceil_div(N, BN);
     const long long tiles = static_cast<long long>(tiles_m) * tiles_n;
-    // 128 x 256: at most one tile per CU. 64 x 256 (three workgroups fit a CU): at most three.
-    if (tiles > (BM == 128 ? 1 : 3) * cu_count() || tiles * 2 < cu_count()) return false;
-    const dim3 grid(static_cast<unsigned>(tiles)), block((BM / WM) * (BN / WN) * kWave);
-    if (whole) {
-        sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, false><<<grid, block, 0, s>>>(M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
-    } else if (!ragged) {
-        if constexpr (ALLOW_EDGES)
-            sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, true><<<grid, block, 0, s>>>(M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
-    } else {
-        if constexpr (ALLOW_EDGES)
-            sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, true, true><<<grid, block, 0, s>>>(M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
+    const int cus = cu_count(), simds = 4 * cus;
+    // 128 x 256 (two strips per SIMD): when nearly every CU gets a tile. 64 x 256 (one strip per SIMD, three
+    // workgroups fit a CU): at most three per CU, at least half of the CUs busy.
+    if (BM == 128 ? (tiles > cus || tiles * 8 < 7 * cus) : (tiles > 3 * cus || tiles * 2 < cus)) return false;
+    // The unit of work is a wavefront's 32 x 128 strip, and a round of 64 x 256 tiles gives every SIMD one.
+    // Tile counts that do not fill whole rounds leave most SIMDs waiting for the few that run one strip more
+    // (2304^3: 324 tiles, 0.63 at best), so the tiles of the partial last round are cut into one-wave tiles of
+    // 64 or 32 that spread over all SIMDs, as for the 256 x 256 tiles above; a 64 x 64 (32 x 32) wave tile is
+    // one strip's (a quarter of one strip's) work at about 0.87 (0.72) of its rate.
+    int main_tiles = static_cast<int>(tiles), leftover_wt = 0;
+    if (BM == 64 && tiles > cus && tiles % cus != 0 && K >= 64 &&
+        static_cast<long long>(K) * 64 < (1ll << 30) && static_cast<long long>(N) * 64 < (1ll << 30)) {
+        const int left = static_cast<int>(tiles % cus);
+        const double cost64 = ceil_div(left * 4, simds) / 0.87, cost32 = ceil_div(left * 16, simds) * 0.25 / 0.72;
+        if (cost64 < 0.9 || cost32 < 0.9) {
+            main_tiles = static_cast<int>(tiles) - left;
+            leftover_wt = cost64 <= cost32 ? 64 : 32;
+        }
     }
-    *rc = check_launch("sgemm_wave_tile_dma_kernel (128 x 256)");
+    const dim3 grid(static_cast<unsigned>(main_tiles)), block((BM / WM) * (BN / WN) * kWave);
+    auto launch = [&](auto edge, auto ragged_rows) {
+        constexpr bool EDGE = decltype(edge)::value, RAGGED = decltype(ragged_rows)::value;
+        sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, EDGE, RAGGED><<<grid, block, 0, s>>>(M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
+        *rc = check_launch("sgemm_wave_tile_dma_kernel (128 x 256 or 64 x 256)");
+        const unsigned left = static_cast<unsigned>(tiles - main_tiles);
+        if (*rc == 0 && leftover_wt == 64) {
+            sgemm_single_wave_kernel<64, 4, EDGE, 1, RAGGED><<<dim3(left * 4), dim3(kWave), 0, s>>>(
+                M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, main_tiles, BM);
+            *rc = check_launch("sgemm_single_wave_kernel (leftover of 64 x 256 tiles)");
+        } else if (*rc == 0 && leftover_wt == 32) {
+            sgemm_single_wave_kernel<32, 4, EDGE, 1, RAGGED><<<dim3(left * 16), dim3(kWave), 0, s>>>(
+                M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, main_tiles, BM);
+            *rc = check_launch("sgemm_single_wave_kernel (leftover of 64 x 256 tiles)");
+        }
+    };
+    if (whole) {
+        launch(std::false_type{}, std::false_type{});
+    } else if (!ragged) {
+        if constexpr (ALLOW_EDGES) launch(std::true_type{}, std::false_type{});
+    } else {
+        if constexpr (ALLOW_EDGES) launch(std::true_type{}, std::true_type{});
+    }
     return true;
 }
 

@@ -265,12 +265,14 @@ def test_wave_tile_ragged_edges(prism, oracle, shape):
 
 
 @pytest.mark.parametrize("shape", [(2304, 2304, 64), (2560, 2816, 48), (2300, 2564, 100), (2817, 2560, 36),
-                                   (3072, 3072, 64), (3328, 2944, 32), (3000, 3332, 68), (3329, 3072, 20), (1152, 6144, 16)])
+                                   (3072, 3072, 64), (3328, 2944, 32), (3000, 3332, 68), (3329, 3072, 20), (1152, 6144, 16),
+                                   (2080, 2048, 128), (2270, 2500, 200)])
 def test_wave_tile_mid_sizes(prism, oracle, shape):
     """Between the one-wave tiles (up to 1024 tiles of 64 x 64) and the 256 x 256 tiles (from 192 of them): the
-    direct-to-LDS kernel on 128 x 256 tiles when those give every CU at most one (the first four shapes and the
-    last), on 64 x 256 tiles when they give it at most three (the others); whole and ragged shapes, K tile counts
-    from 1 up. Operands between NaNs, C fenced, every element checked, with and without reading C."""
+    direct-to-LDS kernel on 128 x 256 tiles when those give nearly every CU one (2817 x 2560: 230 tiles), else
+    on 64 x 256 tiles, whose partial last round is cut into one-wave tiles of 32 x 32 when K is at least 64 and
+    that is cheaper (2304^2: 68 of 324 tiles, 3072^2: 64 of 576, 2080 x 2048: 8 of 264, 2270 x 2500: 104 of 360,
+    the last with zero-filled edges); whole and ragged shapes, K tile counts from 1 up. Operands between NaNs, C fenced, every element checked, with and without reading C."""
     M, N, K = shape
     A, B, Cm = oracle.gen_sgemm(M, N, K, seed=M + 5 * K)
     for beta in (0.5, 0.0):
@@ -287,13 +289,15 @@ def test_wave_tile_mid_sizes(prism, oracle, shape):
 @pytest.mark.parametrize("shape", [(3581, 3582, 101), (3584, 3585, 67), (3585, 3587, 38), (3500, 3601, 5), (3841, 3333, 233),
                                    (3584, 3584, 7), (3584, 3584, 64), (2300, 2566, 101), (3001, 3333, 69), (2304, 2305, 4),
                                    (4300, 4349, 101), (4090, 5117, 70), (5377, 5375, 66),
-                                   (1001, 1001, 1001), (2001, 1999, 130), (64, 65, 6), (33, 31, 4), (700, 130, 77)])
+                                   (1001, 1001, 1001), (2001, 1999, 130), (64, 65, 6), (33, 31, 4), (700, 130, 77),
+                                   (2305, 2303, 70)])
 def test_wave_tile_rows_not_16_byte_aligned(prism, oracle, shape):
     """N or K not a multiple of 4, or matrices that start at an odd element: rows are then only 4 B aligned and
     the direct-to-LDS kernel runs in its ragged form (256 x 256 tiles for the first seven shapes, 128 x 256 and
     64 x 256 tiles for the next three; the last three have 289, 320 and 462 tiles for 256 CUs, so the 33, 64 and
     206 tiles of their partial last round are cut into 64 x 256 slices, or not at all; the last five are small
-    problems for the one-wave-per-tile kernel's ragged form, 64 x 64 and 32 x 32 tiles, K tile counts from 1 up): 16 B loads from 4 B-aligned addresses, a K loop over K rounded down to a
+    problems for the one-wave-per-tile kernel's ragged form, 64 x 64 and 32 x 32 tiles, K tile counts from 1 up, and the
+    last has 333 tiles of 64 x 256 for 256 CUs, whose last 77 are cut into ragged one-wave tiles of 32 x 32): 16 B loads from 4 B-aligned addresses, a K loop over K rounded down to a
     multiple of 4 with the last K % 4 values added in front of the write-back, and C written element by element
     where a chunk straddles N. A and B sit between NaNs and C is fenced; every element is checked, with and
     without reading C, with the matrices at an even and at an odd element."""
