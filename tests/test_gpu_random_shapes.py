@@ -1,0 +1,94 @@
+"""Seeded random shapes and alignments through the two MFMA GEMMs, every element against an fp64 product.
+
+The hand-picked shapes of test_gpu_sgemm.py and test_gpu_gemm_bf16.py sit on the boundaries the launchers
+know about; these draws land between them: any M, N, K from 1 up, operands that start at any element of their
+buffers (so rows are 4 B, 8 B or 16 B aligned for fp32 and 2 B to 16 B aligned for bf16), beta zero or not.
+The operands sit between NaNs and the output between guard values, so a read outside a matrix or a store
+outside the output shows. The fp64 product is formed on the device (torch), which keeps the test short; the
+bounds are the ones of the hand-picked tests (1e-5 sqrt(K) max|A| max|B| for fp32, 1e-3 of the largest
+|element| for bf16).
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _draw_shapes(seed, count, big):
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(count):
+        kind = i % 4
+        if kind == 0:      # small: one-wave tiles, K from 1 up
+            M, N, K = rng.integers(1, 200), rng.integers(1, 200), rng.integers(1, 100)
+        elif kind == 1:    # a few hundred: rings, one-wave tiles with K split off
+            M, N, K = rng.integers(100, 900), rng.integers(100, 900), rng.integers(4, 600)
+        elif kind == 2:    # one long side
+            M, N, K = rng.integers(1, 64), rng.integers(500, 3000), rng.integers(8, 300)
+            if rng.integers(0, 2):
+                M, N = N, M
+        else:              # mid sizes: workgroup tiles, partial rounds
+            M, N, K = rng.integers(1500, big), rng.integers(1500, big), rng.integers(16, 200)
+        out.append((int(M), int(N), int(K), int(rng.integers(0, 8)), int(rng.integers(0, 8)), int(rng.integers(0, 4))))
+    return out
+
+
+def _fenced(values: torch.Tensor, start: int, fill) -> torch.Tensor:
+    """`values` as a view that starts at element `start` of a buffer otherwise filled with `fill`."""
+    buf = torch.full((values.numel() + 64,), fill, dtype=values.dtype, device=DEV)
+    view = buf[start:start + values.numel()].view(values.shape)
+    view.copy_(values)
+    return view
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_sgemm_kernel_5_random_shapes(prism, seed):
+    g = torch.Generator(device=DEV)
+    g.manual_seed(seed)
+    for (M, N, K, sa, sb, sc) in _draw_shapes(seed, 60, 4700):
+        A = torch.rand((M, K), device=DEV, generator=g) * 2 - 1
+        B = torch.rand((K, N), device=DEV, generator=g) * 2 - 1
+        C0 = torch.rand((M, N), device=DEV, generator=g) * 2 - 1
+        beta = 0.5 if (M + N + K) % 2 else 0.0
+        a, b = _fenced(A, sa % 4, float("nan")), _fenced(B, sb % 4, float("nan"))
+        cbuf = torch.full((M * N + 64,), 777.0, device=DEV)
+        c = cbuf[8 + sc:8 + sc + M * N].view(M, N)
+        c.copy_(C0)
+        print(f"sgemm M={M} N={N} K={K} starts {sa % 4} {sb % 4} {8 + sc} beta={beta}", flush=True)
+        prism.sgemm(M, N, K, 1.25, a, b, beta, c, variant=5)
+        torch.cuda.synchronize()
+        assert bool((cbuf[:8 + sc] == 777.0).all()) and bool((cbuf[8 + sc + M * N:] == 777.0).all())
+        want = 1.25 * (A.double() @ B.double()) + beta * C0.double()
+        err = float((c.double() - want).abs().max())
+        assert err <= 1e-5 * np.sqrt(K) + abs(beta) * 2**-22, f"{M}x{N}x{K}: max error {err:.3e}"
+
+
+@pytest.mark.parametrize("seed", [4, 5, 6])
+def test_gemm_bf16_random_shapes(prism, seed):
+    g = torch.Generator(device=DEV)
+    g.manual_seed(seed)
+    nan16 = torch.tensor(float("nan"), dtype=torch.bfloat16)
+    for (M, N, K, sa, sb, sc) in _draw_shapes(seed, 60, 4700):
+        A = torch.randn((M, K), device=DEV, generator=g).to(torch.bfloat16)
+        B = torch.randn((N, K), device=DEV, generator=g).to(torch.bfloat16)
+        a, b = _fenced(A, sa, nan16.item()), _fenced(B, sb, nan16.item())
+        dbuf = torch.full((M * N + 64,), 777.0, device=DEV)
+        d = dbuf[8 + sc:8 + sc + M * N].view(M, N)
+        print(f"gemm_bf16 M={M} N={N} K={K} starts {sa} {sb} {8 + sc}", flush=True)
+        prism.gemm_bf16(a, b, d)
+        torch.cuda.synchronize()
+        assert bool((dbuf[:8 + sc] == 777.0).all()) and bool((dbuf[8 + sc + M * N:] == 777.0).all())
+        want = A.double() @ B.double().t()
+        err = float((d.double() - want).abs().max())
+        assert err <= 1e-3 * float(want.abs().max()), f"{M}x{N}x{K}: max error {err:.3e}"
+        if K % 2 == 0:   # the bf16 column-major form on every other draw
+            cbuf = torch.full((N * M + 64,), -7.0, dtype=torch.bfloat16, device=DEV)
+            cc = cbuf[8 + sc:8 + sc + N * M]
+            prism.runmyh100(M, N, K, a, b, cc)
+            torch.cuda.synchronize()
+            assert bool((cbuf[:8 + sc] == -7.0).all()) and bool((cbuf[8 + sc + N * M:] == -7.0).all())
+            got = cc.view(N, M).t().double()
+            assert bool(((got - want).abs() <= 2.0**-8 * want.abs() + 1e-3 * float(want.abs().max())).all())
