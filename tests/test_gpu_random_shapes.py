@@ -92,3 +92,36 @@ def test_gemm_bf16_random_shapes(prism, seed):
             assert bool((cbuf[:8 + sc] == -7.0).all()) and bool((cbuf[8 + sc + N * M:] == -7.0).all())
             got = cc.view(N, M).t().double()
             assert bool(((got - want).abs() <= 2.0**-8 * want.abs() + 1e-3 * float(want.abs().max())).all())
+
+
+@pytest.mark.parametrize("seed", [7, 8])
+def test_scans_random_lengths_and_alignments(prism, seed):
+    """Random lengths (1 to 2^25, both tile shapes and their edges), first elements at any index (4 B to 16 B
+    aligned), in place or not, one workspace for all calls and kinds; against torch's scans on the device,
+    bit for bit."""
+    rng = np.random.default_rng(seed)
+    g = torch.Generator(device=DEV)
+    g.manual_seed(seed)
+    ws = prism.new_scan_workspace(1 << 25)
+    for i in range(40):
+        n = int(rng.integers(1, 1 << int(rng.integers(1, 26))))
+        start, kind, in_place = int(rng.integers(0, 4)), int(rng.integers(0, 4)), bool(rng.integers(0, 2))
+        buf = torch.randint(-1000, 1001, (n + 8,), dtype=torch.int32, device=DEV, generator=g)
+        if kind == 0:
+            buf[start] += 2**31 - 1000      # the sums wrap around
+        x = buf[start:start + n]
+        keep = x.clone()
+        out = x if in_place else torch.full((n + 8,), 12345, dtype=torch.int32, device=DEV)[4 - start:4 - start + n]
+        print(f"scan n={n} start={start} kind={kind} in_place={in_place}", flush=True)
+        if kind in (0, 1):
+            got = prism.scan(x, out=out, workspace=ws)
+            want = torch.cumsum(keep, 0, dtype=torch.int32)
+        elif kind == 2:
+            got = prism.scan(x, out=out, workspace=ws, exclusive=True)
+            want = torch.cumsum(keep, 0, dtype=torch.int32) - keep
+        else:
+            got = prism.scan(x, out=out, workspace=ws, op="max")
+            want = torch.cummax(keep, 0).values
+        assert torch.equal(got, want), f"n={n} start={start} kind={kind}"
+        if not in_place:
+            assert torch.equal(x, keep)
