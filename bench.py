@@ -143,7 +143,9 @@ def gemm_bf16_max_err_fp64(A, B, D, rows: int = 1024):
 
 # ------------------------------------------------------------------ sgemm --
 
-def bench_sgemm(prism, M, N, K, alpha, beta, variant, steps, warmup, gate=True):
+def bench_sgemm(prism, M, N, K, alpha, beta, variant, steps, warmup, gate=True, with_workspace=False):
+    """with_workspace: through prism_sgemm_ws with the workspace prism_sgemm_workspace_bytes asks for (kernel 5
+    then cuts K across workgroups on skinny shapes); otherwise the reference-shaped prism_sgemm."""
     import torch
     g = torch.Generator(device="cuda")
     g.manual_seed(0)
@@ -151,8 +153,9 @@ def bench_sgemm(prism, M, N, K, alpha, beta, variant, steps, warmup, gate=True):
     B = torch.rand((K, N), dtype=torch.float32, device="cuda", generator=g) * 2 - 1
     C0 = torch.rand((M, N), dtype=torch.float32, device="cuda", generator=g) * 2 - 1
     C = C0.clone()
+    ws = torch.empty(max(prism.sgemm_workspace_size(M, N, K), 16), dtype=torch.uint8, device="cuda") if with_workspace else None
     if gate:
-        prism.sgemm(M, N, K, alpha, A, B, beta, C, variant=variant)
+        prism.sgemm(M, N, K, alpha, A, B, beta, C, variant=variant, workspace=ws)
         err = sgemm_max_err_fp64(alpha, A, B, beta, C0, C)
         bound = 1e-5 * np.sqrt(K) + abs(beta) * 2**-22
         if not err <= bound:
@@ -162,7 +165,11 @@ def bench_sgemm(prism, M, N, K, alpha, beta, variant, steps, warmup, gate=True):
     # with |beta| < 1 it stays bounded.
     lib, st = _capi()
     a, b, c = A.data_ptr(), B.data_ptr(), C.data_ptr()
-    ms = time_steps(lambda: lib.prism_sgemm(variant, M, N, K, alpha, a, b, beta, c, st), steps, warmup)
+    if ws is None:
+        ms = time_steps(lambda: lib.prism_sgemm(variant, M, N, K, alpha, a, b, beta, c, st), steps, warmup)
+    else:
+        w, wn = ws.data_ptr(), ws.numel()
+        ms = time_steps(lambda: lib.prism_sgemm_ws(variant, M, N, K, alpha, a, b, beta, c, w, wn, st), steps, warmup)
     flops = 2.0 * M * N * K
     tflops = flops / (ms * 1e-3) / 1e12
     return {"ms": ms, "tflops": tflops,
@@ -487,6 +494,11 @@ def main() -> int:
             r = bench_sgemm(prism, M, N, Kd, 1.0, 0.0, 5, 10, 2)
             configs[f"sgemm_k5_{M}x{N}x{Kd}"] = {"ms": r["ms"], "tflops": r["tflops"], "frac": r["roofline"]["frac"], "steps": 10}
             log(f"  sgemm kernel 5 {M}x{N}x{Kd}: {r['ms']:.3f} ms  {r['tflops']:.2f} TFLOP/s")
+        # the skinny tail shape once more through the workspace form (K cut across workgroups)
+        r = bench_sgemm(prism, 128, 4096, 4096, 1.0, 0.0, 5, 10, 2, with_workspace=True)
+        configs["sgemm_k5_128x4096x4096_with_workspace"] = {"ms": r["ms"], "tflops": r["tflops"], "frac": r["roofline"]["frac"],
+                                                            "steps": 10, "entry": "prism_sgemm_ws"}
+        log(f"  sgemm kernel 5 128x4096x4096 with workspace: {r['ms']:.3f} ms  {r['tflops']:.2f} TFLOP/s")
         for p in (20, 24, 28):
             r = bench_scan(prism, 1 << p, 20, 3)
             configs[f"scan_2p{p}"] = {"ms": r["ms"], "GBps": r["GBps"], "frac": r["roofline"]["frac"], "steps": 20}

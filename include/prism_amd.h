@@ -277,6 +277,24 @@ int prism_sgemm(int variant, int M, int N, int K, float alpha, const float* A,
                 const float* B, float beta, float* C, void* stream);
 
 /*
+ * prism_sgemm with a workspace, for shapes that have too few tiles for the GPU
+ * and a long K (skinny products such as 128 x 4096 x 4096): kernel 5 then cuts K
+ * across workgroups, every part writes its M x N partial product into the
+ * workspace, and a second kernel adds the parts in a fixed order (the same bits
+ * on every run) and applies alpha and beta. prism_sgemm_workspace_bytes says
+ * how much a shape can use (0: it would not be cut); with a smaller or NULL
+ * workspace (16-byte aligned otherwise), or any other kernel number, the call is
+ * prism_sgemm. Calls that share a workspace must be ordered on one stream.
+ * No counterpart in the reference, whose launchers (evals/4090_sgemm/runner.cu:
+ * 191-243) take no workspace; a harness that wants the split holds one buffer
+ * and passes it here.
+ */
+size_t prism_sgemm_workspace_bytes(int M, int N, int K);
+int prism_sgemm_ws(int variant, int M, int N, int K, float alpha, const float* A,
+                   const float* B, float beta, float* C, void* workspace,
+                   size_t workspace_bytes, void* stream);
+
+/*
  * The reference dispatcher's own shape: default stream, kernel numbers 1..5.
  * Replaces run_my_kernel (evals/4090_sgemm/runner.cuh:28-29,
  * runner.cu:245-267). The reference throws std::invalid_argument for an

@@ -138,6 +138,14 @@ int prism_sgemm(int variant, int M, int N, int K, float alpha, const float* A, c
     return launch_sgemm(variant, M, N, K, alpha, A, B, beta, C, static_cast<hipStream_t>(stream));
 }
 
+size_t prism_sgemm_workspace_bytes(int M, int N, int K) { return sgemm_workspace_bytes(M, N, K); }
+
+int prism_sgemm_ws(int variant, int M, int N, int K, float alpha, const float* A, const float* B, float beta,
+                   float* C, void* workspace, size_t workspace_bytes, void* stream) {
+    return launch_sgemm_ws(variant, M, N, K, alpha, A, B, beta, C, workspace, workspace_bytes,
+                           static_cast<hipStream_t>(stream));
+}
+
 int prism_run_my_kernel(int my_kernel_num, int M, int N, int K, float alpha, float* A, float* B,
                         float beta, float* C) {
     if (my_kernel_num < 1 || my_kernel_num > 5)

@@ -75,6 +75,9 @@ int launch_wave_regroup(const int32_t* in, int32_t* out, size_t n, int items_per
 int launch_calibrate_stream(int kind, const void* in, void* out, size_t bytes, hipStream_t s);
 int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, const float* B,
                  float beta, float* C, hipStream_t s);
+size_t sgemm_workspace_bytes(int M, int N, int K);
+int launch_sgemm_ws(int variant, int M, int N, int K, float alpha, const float* A, const float* B, float beta,
+                    float* C, void* ws, size_t ws_bytes, hipStream_t s);
 int launch_gemm_bf16(int M, int N, int K, const uint16_t* A, const uint16_t* B, float* D_f32,
                      uint16_t* C_bf16_colmajor, hipStream_t s);
 

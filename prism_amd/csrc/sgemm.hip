@@ -31,6 +31,8 @@
 //
 // Unlike the reference kernels (no guards in kernels 1, 3, 4, 5), every kernel
 // here accepts any M, N, K. When beta == 0, C is not read.
+#include <algorithm>
+
 #include "common.h"
 #include "direct_load.h"
 #include "tile_map.h"
@@ -450,14 +452,27 @@ __attribute__((amdgpu_waves_per_eu(4))) void sgemm_wave_tile_kernel(
 // chunk lies inside its row; a B chunk that straddles the end of a row brings the head of the next row
 // into columns >= N, which are never stored. The last K % 4 values of k are added in front of the
 // write-back from ordinary loads, and C is written element by element where a chunk straddles N.
-template <int BM, int BN, int BK, int WM, int WN, bool EDGE, bool RAGGED = false>
+//
+// SPLIT (whole tiles only): the K range is cut into `first_big` equal parts and the grid holds one workgroup
+// per tile and part; part s multiplies k in [s K / parts, (s + 1) K / parts) and writes its M x N partial
+// product (alpha and beta are not applied) into slice s of the buffer passed as C, for sgemm_add_parts_kernel.
+template <int BM, int BN, int BK, int WM, int WN, bool EDGE, bool RAGGED = false, bool SPLIT = false>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile_dma_kernel(
     int M, int N, int K_all, float alpha, const float* __restrict__ A, const float* __restrict__ B,
     float beta, float* C, int tiles_m, int tiles_n, int first_big) {
     static_assert(EDGE || !RAGGED, "the ragged form is an edge form");
+    static_assert(!SPLIT || !EDGE, "the K split is written for whole tiles");
     // lda: elements between A rows. K: the part of the k range the loop covers.
     const int lda = K_all;
-    const int K = RAGGED ? K_all - K_all % 4 : K_all;
+    const int K = RAGGED ? K_all - K_all % 4 : (SPLIT ? K_all / first_big : K_all);
+    unsigned tile_id = blockIdx.x;
+    if constexpr (SPLIT) {
+        const unsigned tiles = static_cast<unsigned>(tiles_m) * tiles_n, part = blockIdx.x / tiles;
+        tile_id = blockIdx.x % tiles;
+        A += static_cast<size_t>(part) * K;
+        B += static_cast<size_t>(part) * K * N;
+        C += static_cast<size_t>(part) * M * N;
+    }
     constexpr int WAVES_N = BN / WN;
     constexpr int WAVES = (BM / WM) * WAVES_N;
     constexpr int MI = WM / 32, NI = 4;
@@ -486,9 +501,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
     // finishes what a launch on 256 x 256 tiles left over: tiles_m x tiles_n is that launch's grid, first_big
     // the first tile number it did not take, and every leftover tile is cut into 256 / BM row slices.
     int row0, col0;
-    if (first_big < 0) {
+    if (SPLIT || first_big < 0) {
         int tm, tn;
-        xcd_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+        xcd_tile_coords(static_cast<int>(tile_id), tiles_m, tiles_n, tm, tn);
         row0 = tm * BM;
         col0 = tn * BN;
     } else {
@@ -1093,6 +1108,27 @@ __global__ __launch_bounds__(kWave * KSPLIT) void sgemm_single_wave_kernel(
     }
 }
 
+// ------------------------------------------------ kernel 5, K split: adding up --
+// C = alpha * (part 0 + part 1 + ... in this order: the same bits on every run) + beta * C, four elements per
+// thread; the parts are the M x N slices the SPLIT form of the workgroup kernel wrote.
+__global__ __launch_bounds__(256) void sgemm_add_parts_kernel(size_t quads, int parts, const f32x4* __restrict__ ws,
+                                                              float alpha, float beta, f32x4* C) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= quads) return;
+    f32x4 sum = ws[i];
+    for (int p = 1; p < parts; ++p) sum += ws[static_cast<size_t>(p) * quads + i];
+    f32x4 r;
+    if (beta == 0.0f) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) r[j] = alpha * sum[j];
+    } else {
+        const f32x4 old = C[i];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) r[j] = __builtin_fmaf(alpha, sum[j], beta * old[j]);
+    }
+    C[i] = r;
+}
+
 // --------------------------------------------------------------- launchers --
 
 template <int BM, int BN, int BK, int TM, int TN, bool VEC>
@@ -1336,7 +1372,69 @@ bool try_single_wave(int M, int N, int K, float alpha, const float* A, const flo
     return true;
 }
 
+// K split across workgroups, for problems with too few 64 x 256 tiles for the CUs and a long K (skinny
+// problems: 128 x 4096 x 4096 has 32 such tiles for 256 CUs). Needs M x N x parts floats of workspace, which the
+// reference-shaped entry points do not have; prism_sgemm_ws takes one. Returns the number of parts (0: no split).
+int split_parts(int M, int N, int K, const float* A, const float* B, const float* C) {
+    if (M <= 0 || N <= 0 || K < 1024 || M % 64 || N % 256 || K % 16) return 0;
+    if (A != nullptr && !(aligned16(A) && aligned16(B) && aligned16(C))) return 0;
+    const long long tiles = static_cast<long long>(M / 64) * (N / 256);
+    const int cus = cu_count();
+    if (tiles * 5 > cus) return 0;                       // from about a fifth of the CUs up the unsplit kernels are level
+    if (static_cast<long long>(K) * 64 >= (1ll << 30) || static_cast<long long>(N) * 64 >= (1ll << 30)) return 0;
+    // The number of parts that a small model of the two kernels prefers: rounds of workgroups, each as long as
+    // its part of K plus a fixed cost worth about 128 k (53 ns per k for a wavefront's strip at the fp32 MFMA
+    // rate), and the adding-up, which moves parts + 2 times the output at about 5 TB/s behind a second launch.
+    // Measured against it on 128 x 4096 x 4096: 4 / 8 / 16 parts 65 / 100 / 93 TFLOP/s (model 65 / 105 / 84).
+    int parts = 0;
+    double best = 0.0;
+    for (int p = 2; p <= 64; p *= 2) {
+        if (K % (16 * p) != 0 || K / p < 128) break;
+        const double rounds = static_cast<double>((tiles * p + cus - 1) / cus);
+        const double us = rounds * (K / p + 128) * 0.053 + (p + 2) * (static_cast<double>(M) * N * 4.0) / 5.0e6 + 3.0;
+        if (parts == 0 || us < best) {
+            best = us;
+            parts = p;
+        }
+    }
+    // Against the unsplit one-wave tiles of 32 x 32, which such shapes take: bound by their L2 traffic (1 B per
+    // 8 flop at about 9 TB/s) or by the instructions a wavefront issues one after the other (13.3 ns per k and
+    // tile, K cut four or two ways inside the workgroup where launch_sgemm does that), plus about 6 us.
+    // Measured: 128 x 4096 x 4096 68 us (model 60), 64 x 512 x 2048 12 (13), 64 x 256 x 16384 65 (60).
+    const double flop = 2.0 * M * N * static_cast<double>(K);
+    const long long tiles32 = static_cast<long long>(M / 32) * (N / 32), simds = 4ll * cus;
+    const int inner = (tiles32 * 8 <= simds && K >= 1024) ? 4 : (tiles32 * 4 <= simds && K >= 512) ? 2 : 1;
+    const double chain_us = static_cast<double>((tiles32 * inner + simds - 1) / simds) * (K / inner) * 0.0133;
+    const double unsplit_us = std::max(flop / 8.0 / 9.0e6, chain_us) + 6.0;
+    return (parts >= 2 && best < 0.85 * unsplit_us) ? parts : 0;
+}
+
 }  // namespace
+
+size_t sgemm_workspace_bytes(int M, int N, int K) {
+    const int parts = split_parts(M, N, K, nullptr, nullptr, nullptr);
+    return static_cast<size_t>(parts) * static_cast<size_t>(M > 0 ? M : 0) * static_cast<size_t>(N > 0 ? N : 0) * sizeof(float);
+}
+
+int launch_sgemm_ws(int variant, int M, int N, int K, float alpha, const float* A, const float* B, float beta,
+                    float* C, void* ws, size_t ws_bytes, hipStream_t s) {
+    if (variant == 0 || variant == 5) {
+        const int parts = (C != nullptr && A != nullptr && B != nullptr && M > 0 && N > 0) ? split_parts(M, N, K, A, B, C) : 0;
+        const size_t need = static_cast<size_t>(parts) * static_cast<size_t>(M) * N * sizeof(float);
+        if (parts >= 2 && ws != nullptr && ws_bytes >= need && (reinterpret_cast<uintptr_t>(ws) & 15u) == 0) {
+            const int tiles_m = M / 64, tiles_n = N / 256;
+            const dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n * parts);
+            sgemm_wave_tile_dma_kernel<64, 256, 16, 32, 128, false, false, true><<<grid, dim3(256), 0, s>>>(
+                M, N, K, 1.0f, A, B, 0.0f, static_cast<float*>(ws), tiles_m, tiles_n, parts);
+            if (int rc = check_launch("sgemm_wave_tile_dma_kernel (K split)")) return rc;
+            const size_t quads = static_cast<size_t>(M) * N / 4;
+            sgemm_add_parts_kernel<<<dim3(static_cast<unsigned>(ceil_div(quads, size_t{256}))), dim3(256), 0, s>>>(
+                quads, parts, static_cast<const f32x4*>(ws), alpha, beta, reinterpret_cast<f32x4*>(C));
+            return check_launch("sgemm_add_parts_kernel");
+        }
+    }
+    return launch_sgemm(variant, M, N, K, alpha, A, B, beta, C, s);
+}
 
 int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, const float* B,
                  float beta, float* C, hipStream_t s) {

@@ -237,15 +237,29 @@ def run_my_kernel(my_kernel_num: int, M: int, N: int, K: int, alpha: float, A: P
            "run_my_kernel")
 
 
+def sgemm_workspace_size(M: int, N: int, K: int) -> int:
+    """Workspace bytes with which kernel 5 cuts K across workgroups for this shape (0: it would not)."""
+    return int(_lib.load().prism_sgemm_workspace_bytes(M, N, K))
+
+
 def sgemm(M: int, N: int, K: int, alpha: float, A: "torch.Tensor", B: "torch.Tensor", beta: float,
-          C: "torch.Tensor", variant: int = 5) -> "torch.Tensor":
-    """sgemm(M,N,K,alpha,A,B,beta,C): the kernel signature of generated/my_sgemm_kernel_*.cu."""
+          C: "torch.Tensor", variant: int = 5, workspace: Optional["torch.Tensor"] = None) -> "torch.Tensor":
+    """sgemm(M,N,K,alpha,A,B,beta,C): the kernel signature of generated/my_sgemm_kernel_*.cu.
+
+    workspace: a device buffer of at least sgemm_workspace_size(M, N, K) bytes lets kernel 5 cut K across
+    workgroups on skinny shapes (deterministic: the parts are added in a fixed order); calls that share one
+    must be ordered on one stream. Without it the call is the reference-shaped one.
+    """
     if variant not in (0, 1, 2, 3, 4, 5, 6):
         raise ValueError("Unknown my_kernel number")
     _need(A, (torch.float32,), M * K, "A")
     _need(B, (torch.float32,), K * N, "B")
     _need(C, (torch.float32,), M * N, "C")
-    _check(_lib.load().prism_sgemm(variant, M, N, K, alpha, _ptr(A), _ptr(B), beta, _ptr(C), _stream()), "sgemm")
+    if workspace is None:
+        _check(_lib.load().prism_sgemm(variant, M, N, K, alpha, _ptr(A), _ptr(B), beta, _ptr(C), _stream()), "sgemm")
+    else:
+        _check(_lib.load().prism_sgemm_ws(variant, M, N, K, alpha, _ptr(A), _ptr(B), beta, _ptr(C), _ptr(workspace),
+                                          _ws_bytes(workspace), _stream()), "sgemm")
     return C
 
 

@@ -118,6 +118,52 @@ static int check_sgemm(int n) {
     return 0;
 }
 
+// The workspace form on a skinny product (K cut across workgroups): against a host product, relative to the sums'
+// size, and twice with the same bits.
+static int check_sgemm_with_workspace(int M, int N, int K) {
+    std::vector<float> A(static_cast<size_t>(M) * K), B(static_cast<size_t>(K) * N), C(static_cast<size_t>(M) * N);
+    uint32_t seed = 5;
+    for (auto* m : {&A, &B, &C})
+        for (auto& v : *m) v = static_cast<float>(lcg(seed) % 5u) - 2.0f + 0.01f * static_cast<float>(lcg(seed) % 5u);
+    const float alpha = 0.5f, beta = 3.0f;
+    if (prism_sgemm_workspace_bytes(M, N, K) == 0) { fprintf(stderr, "sgemm: %dx%dx%d would not be cut\n", M, N, K); return 1; }
+    float *dA, *dB, *dC;
+    HIP_OK(hipMalloc(reinterpret_cast<void**>(&dA), sizeof(float) * A.size()));
+    HIP_OK(hipMalloc(reinterpret_cast<void**>(&dB), sizeof(float) * B.size()));
+    HIP_OK(hipMalloc(reinterpret_cast<void**>(&dC), sizeof(float) * C.size()));
+    HIP_OK(hipMemcpy(dA, A.data(), sizeof(float) * A.size(), hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(dB, B.data(), sizeof(float) * B.size(), hipMemcpyHostToDevice));
+    std::vector<float> got(C.size()), again(C.size());
+    for (auto* out : {&got, &again}) {
+        HIP_OK(hipMemcpy(dC, C.data(), sizeof(float) * C.size(), hipMemcpyHostToDevice));
+        run_my_sgemm_5_with_workspace(M, N, K, alpha, dA, dB, beta, dC);
+        HIP_OK(hipDeviceSynchronize());
+        HIP_OK(hipGetLastError());
+        HIP_OK(hipMemcpy(out->data(), dC, sizeof(float) * C.size(), hipMemcpyDeviceToHost));
+    }
+    for (int i = 0; i < M; ++i)
+        for (int j = 0; j < N; ++j) {
+            double s = 0, mag = 0;
+            for (int k = 0; k < K; ++k) {
+                const double p = static_cast<double>(A[static_cast<size_t>(i) * K + k]) * B[static_cast<size_t>(k) * N + j];
+                s += p;
+                mag += std::fabs(p);
+            }
+            const double want = alpha * s + beta * C[static_cast<size_t>(i) * N + j];
+            const float g = got[static_cast<size_t>(i) * N + j];
+            if (!(std::fabs(g - want) <= 1e-5 * mag + 1e-4) || g != again[static_cast<size_t>(i) * N + j]) {
+                fprintf(stderr, "sgemm with workspace: element (%d,%d) is %f / %f, expected %f\n", i, j, g,
+                        again[static_cast<size_t>(i) * N + j], want);
+                return 1;
+            }
+        }
+    HIP_OK(hipFree(dA));
+    HIP_OK(hipFree(dB));
+    HIP_OK(hipFree(dC));
+    printf("sgemm with workspace %dx%dx%d ok\n", M, N, K);
+    return 0;
+}
+
 // evals/h100_bench/main.cu:123-141 in outline: bf16 C, column-major, |d| <= 0.1 (main.cu:48).
 static int check_h100(int M, int N, int K) {
     std::vector<uint16_t> A(static_cast<size_t>(M) * K), B(static_cast<size_t>(N) * K);
@@ -157,6 +203,7 @@ int main() {
     for (size_t n : {size_t{16384}, size_t{32768}, size_t{1} << 20, (size_t{1} << 20) + 17, size_t{1} << 24})
         if (check_scan(n)) return 1;
     if (check_sgemm(256)) return 1;
+    if (check_sgemm_with_workspace(64, 256, 16384)) return 1;
     if (check_h100(256, 512, 192)) return 1;
     printf("OK\n");
     return 0;

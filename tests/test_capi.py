@@ -48,6 +48,7 @@ def test_every_declaration_cites_the_reference():
                        ("prism_scan_max_i32", "scan.py:106-173"), ("prism_scan_min_i32", "scan.py:106-173"),
                        ("prism_launch_scan", "4090_scan/main.cu"),
                        ("prism_sgemm", "runner.cu"), ("prism_run_my_kernel", "runner.cu"),
+                       ("prism_sgemm_ws", "runner.cu:\n * 191-243"),
                        ("prism_gemm_bf16", "h100_matmul.py"), ("prism_runmyh100", "utils.cuh")]:
         decl = text.index(name + "(")
         comment = text.rfind("/*", 0, decl)
@@ -67,6 +68,14 @@ def test_argument_checks_run_before_any_gpu_work(lib):
     assert lib.prism_sgemm(7, 4, 4, 4, 1.0, None, None, 0.0, None, None) == 1
     assert lib.prism_sgemm(5, -1, 4, 4, 1.0, None, None, 0.0, None, None) == 1
     assert lib.prism_sgemm(5, 4, 4, 4, 1.0, None, None, 0.0, None, None) == 1  # null matrices
+    # the workspace form checks like prism_sgemm; the size query needs no device (256 CUs assumed without one)
+    assert lib.prism_sgemm_ws(7, 4, 4, 4, 1.0, None, None, 0.0, None, None, 0, None) == 1
+    assert lib.prism_sgemm_ws(5, 4, 4, 4, 1.0, None, None, 0.0, None, None, 0, None) == 1
+    assert lib.prism_sgemm_ws(5, 0, 4, 4, 1.0, None, None, 0.0, None, None, 0, None) == 0
+    assert lib.prism_sgemm_workspace_bytes(128, 4096, 4096) % (128 * 4096 * 4) == 0
+    assert lib.prism_sgemm_workspace_bytes(128, 4096, 4096) >= 2 * 128 * 4096 * 4      # a skinny product is cut
+    for whole_chip in ((8192, 8192, 8192), (4096, 4096, 128), (128, 4096, 100), (100, 4096, 4096), (0, 4096, 4096), (-1, 4, 4)):
+        assert lib.prism_sgemm_workspace_bytes(*whole_chip) == 0
     # empty problems succeed without touching a device
     assert lib.prism_sgemm(5, 0, 4, 4, 1.0, None, None, 0.0, None, None) == 0
     assert lib.prism_add_m(None, None, 7, 0, None) == 0

@@ -212,6 +212,53 @@ def test_wave_tile_leftover_round(prism, oracle, shape):
     assert np.max(np.abs(got - oracle.np_sgemm_f64(1.25, A, B, 0.5, Cm))) <= tol(oracle, K, A, B, 0.5, Cm)
 
 
+@pytest.mark.parametrize("shape", [(128, 4096, 4096), (64, 2048, 8192), (256, 256, 16384), (192, 768, 8192), (64, 4096, 4096)])
+def test_wave_tile_k_split_with_workspace(prism, oracle, shape):
+    """Skinny products through prism_sgemm_ws: kernel 5 cuts K across workgroups (8, 32, 64, 16 and 16 parts
+    here), every part writes its partial product into the workspace and a second kernel adds the parts in a fixed
+    order. Every element against fp64, with and without reading C (C full of NaN when it is not read), the same
+    bits on a second run, nothing written beyond the bytes prism_sgemm_workspace_bytes names, and with a
+    workspace one byte short the call is the unsplit one, bit for bit."""
+    M, N, K = shape
+    need = prism.sgemm_workspace_size(M, N, K)
+    assert need >= 2 * M * N * 4 and need % (M * N * 4) == 0
+    A, B, Cm = oracle.gen_sgemm(M, N, K, seed=M + N + K)
+    a, b = dev(A), dev(B)
+    wsbuf = torch.full((need + 512,), 0x5A, dtype=torch.uint8, device=DEV)
+    ws = wsbuf[256:256 + need]
+    outs = []
+    for beta, c0 in ((0.5, Cm), (0.0, np.full((M, N), np.nan, dtype=np.float32))):
+        c = dev(c0).clone()
+        prism.sgemm(M, N, K, 1.25, a, b, beta, c, variant=5, workspace=ws)
+        got = host(c)
+        assert np.max(np.abs(got - oracle.np_sgemm_f64(1.25, A, B, beta, Cm))) <= tol(oracle, K, A, B, beta, Cm)
+        c2 = dev(c0).clone()
+        prism.sgemm(M, N, K, 1.25, a, b, beta, c2, variant=5, workspace=ws)
+        assert np.array_equal(host(c2), got)
+        outs.append(got)
+    guard = host(wsbuf)
+    assert np.all(guard[:256] == 0x5A) and np.all(guard[256 + need:] == 0x5A)
+    short = torch.empty(need - 1, dtype=torch.uint8, device=DEV)
+    c3, c4 = dev(Cm).clone(), dev(Cm).clone()
+    prism.sgemm(M, N, K, 1.25, a, b, 0.5, c3, variant=5, workspace=short)
+    prism.sgemm(M, N, K, 1.25, a, b, 0.5, c4, variant=5)
+    assert np.array_equal(host(c3), host(c4))
+    assert np.max(np.abs(host(c3) - outs[0])) <= 2 * tol(oracle, K, A, B, 0.5, Cm)
+
+
+def test_workspace_form_leaves_other_shapes_and_kernels_alone(prism, oracle):
+    """Shapes the split is not for, and the kernels other than 5, run as in prism_sgemm: same bits with and
+    without a workspace."""
+    ws = torch.empty(64 << 20, dtype=torch.uint8, device=DEV)
+    for (M, N, K, variant) in ((1024, 1024, 1024, 5), (128, 4096, 1000, 5), (100, 4096, 4096, 5), (128, 4096, 4096, 4), (128, 4096, 4096, 1)):
+        assert variant != 5 or prism.sgemm_workspace_size(M, N, K) == 0
+        A, B, Cm = oracle.gen_sgemm(M, N, K, seed=K)
+        c1, c2 = dev(Cm).clone(), dev(Cm).clone()
+        prism.sgemm(M, N, K, 1.0, dev(A), dev(B), 0.5, c1, variant=variant, workspace=ws)
+        prism.sgemm(M, N, K, 1.0, dev(A), dev(B), 0.5, c2, variant=variant)
+        assert np.array_equal(host(c1), host(c2))
+
+
 def nan_fenced(a: np.ndarray, start: int = 1024) -> torch.Tensor:
     """The matrix as a view into a device buffer whose other elements are NaN; `start` is its first
     element's index (a multiple of 4 keeps it 16 B aligned)."""

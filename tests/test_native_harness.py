@@ -23,7 +23,7 @@ def build_harness(out_dir: Path) -> Path:
     text = (ROOT / "INTEGRATION.md").read_text()
     head = text[text.index("## 1. Scan harness"):text.index("## 4. add_m")]
     blocks = re.findall(r"```cpp\n(.*?)```", head, flags=re.S)
-    assert len(blocks) == 3, "sections 1-3 of the integration guide should hold one C++ block each"
+    assert len(blocks) == 4, "sections 1-3 of the integration guide hold four C++ blocks (section 2 has two)"
     out_dir.mkdir(parents=True, exist_ok=True)
     (out_dir / "integration_snippets.inc").write_text("\n".join(blocks))
     exe = out_dir / "native_harness"
@@ -48,5 +48,6 @@ def test_integration_snippets_run(tmp_path):
     proc = subprocess.run([str(exe)], capture_output=True, text=True, timeout=110)
     assert proc.returncode == 0, proc.stdout + proc.stderr
     assert proc.stdout.strip().endswith("OK")
-    for must in ("scan n=16384 ok", "scan n=1048593 ok", "sgemm kernel 5 n=256 ok", "h100 256x512x192 ok"):
+    for must in ("scan n=16384 ok", "scan n=1048593 ok", "sgemm kernel 5 n=256 ok", "sgemm with workspace 64x256x16384 ok",
+                 "h100 256x512x192 ok"):
         assert must in proc.stdout
