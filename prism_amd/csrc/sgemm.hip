@@ -1184,6 +1184,15 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
         return false;
     const int tiles_m = ceil_div(M, BM), tiles_n = ceil_div(N, BN);
     if (static_cast<long long>(tiles_m) * tiles_n * 4 < 3ll * cu_count()) return false;
+    if (static_cast<long long>(tiles_m) * tiles_n < cu_count()) {
+        // A single, partial round of big tiles costs a full one: four strips per SIMD on the CUs that have a
+        // tile. The same output as 64 x 256 tiles is whole rounds of one strip per SIMD (about 8 % dearer per
+        // strip: less reuse of operands) plus a partial round that try_half_tile_dma cuts into one-wave tiles.
+        // 3584^3: 196 big tiles, or 784 = 3 x 256 + 16 small ones, 3.6 strips against 4 (116 -> 131 TFLOP/s).
+        const long long t64 = static_cast<long long>(ceil_div(M, 64)) * tiles_n, cus = cu_count(), left = t64 % cus;
+        const double last = left == 0 ? 0.0 : (left * 16 <= 8 * cus && K >= 64) ? ceil_div(left * 16, 4 * cus) * 0.35 : 1.08;
+        if ((t64 / cus) * 1.08 + last < 3.7) return false;
+    }
     const dim3 block((BM / WM) * (BN / WN) * kWave);
     // Tile counts that do not fill whole rounds of CUs: the 256 x 256 kernel takes the whole rounds, and
     // the tiles of the last, partial round are cut into 64 x 64 wave tiles that spread over all SIMDs
@@ -1287,8 +1296,8 @@ bool try_half_tile_dma(int M, int N, int K, float alpha, const float* A, const f
     const long long tiles = static_cast<long long>(tiles_m) * tiles_n;
     const int cus = cu_count(), simds = 4 * cus;
     // 128 x 256 (two strips per SIMD): when nearly every CU gets a tile. 64 x 256 (one strip per SIMD, three
-    // workgroups fit a CU): at most three per CU, at least half of the CUs busy.
-    if (BM == 128 ? (tiles > cus || tiles * 8 < 7 * cus) : (tiles > 3 * cus || tiles * 2 < cus)) return false;
+    // workgroups fit a CU): at most four rounds, at least half of the CUs busy.
+    if (BM == 128 ? (tiles > cus || tiles * 8 < 7 * cus) : (tiles > 4 * cus || tiles * 2 < cus)) return false;
     // The unit of work is a wavefront's 32 x 128 strip, and a round of 64 x 256 tiles gives every SIMD one.
     // Tile counts that do not fill whole rounds leave most SIMDs waiting for the few that run one strip more
     // (2304^3: 324 tiles, 0.63 at best), so the tiles of the partial last round are cut into one-wave tiles of
@@ -1493,6 +1502,15 @@ int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, 
                 // (K < 4, offsets that do not fit 32 bits) goes to the general kernel.
                 const long long simds = 4ll * cu_count();
                 const long long tiles64 = static_cast<long long>(ceil_div(M, 64)) * ceil_div(N, 64);
+                // A single round of 64 x 256 workgroup tiles that fills at least three quarters of the CUs (one
+                // strip per SIMD, operands shared through LDS) is ahead of one-wave tiles over the same output:
+                // 2048^3 119 -> 132, 1920 x 2048 x 2048 100 -> 133, 1664 x 2048 x 1024 86 -> 109 TFLOP/s on one box;
+                // with fewer tiles it is not (1536^3, 144 tiles: 100 -> 79).
+                {
+                    const long long t64x256 = static_cast<long long>(ceil_div(M, 64)) * ceil_div(N, 256);
+                    if (t64x256 <= cu_count() && t64x256 * 4 >= 3ll * cu_count() &&
+                        try_half_tile_dma<64, true>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;
+                }
                 if (tiles64 <= simds) {
                     // Far fewer 32 x 32 tiles than SIMDs: cut K inside the workgroup (2 or 4 waves per tile) as
                     // long as every wave keeps at least 256 of K and at most half of the SIMDs end up with a

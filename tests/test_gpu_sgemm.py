@@ -313,13 +313,15 @@ def test_wave_tile_ragged_edges(prism, oracle, shape):
 
 @pytest.mark.parametrize("shape", [(2304, 2304, 64), (2560, 2816, 48), (2300, 2564, 100), (2817, 2560, 36),
                                    (3072, 3072, 64), (3328, 2944, 32), (3000, 3332, 68), (3329, 3072, 20), (1152, 6144, 16),
-                                   (2080, 2048, 128), (2270, 2500, 200)])
+                                   (2080, 2048, 128), (2270, 2500, 200), (2048, 2048, 96), (1920, 2040, 100), (1664, 2048, 33)])
 def test_wave_tile_mid_sizes(prism, oracle, shape):
     """Between the one-wave tiles (up to 1024 tiles of 64 x 64) and the 256 x 256 tiles (from 192 of them): the
     direct-to-LDS kernel on 128 x 256 tiles when those give nearly every CU one (2817 x 2560: 230 tiles), else
     on 64 x 256 tiles, whose partial last round is cut into one-wave tiles of 32 x 32 when K is at least 64 and
     that is cheaper (2304^2: 68 of 324 tiles, 3072^2: 64 of 576, 2080 x 2048: 8 of 264, 2270 x 2500: 104 of 360,
-    the last with zero-filled edges); whole and ragged shapes, K tile counts from 1 up. Operands between NaNs, C fenced, every element checked, with and without reading C."""
+    the last with zero-filled edges); the last three shapes have 192 to 256 tiles of 64 x 256, a single round,
+    which is taken in place of one-wave tiles (whole, with edges, with rows that are not 16 B aligned); whole and
+    ragged shapes, K tile counts from 1 up. Operands between NaNs, C fenced, every element checked, with and without reading C."""
     M, N, K = shape
     A, B, Cm = oracle.gen_sgemm(M, N, K, seed=M + 5 * K)
     for beta in (0.5, 0.0):
