@@ -1,8 +1,10 @@
 """Seeded random shapes and alignments through the two MFMA GEMMs, every element against an fp64 product.
 
 The hand-picked shapes of test_gpu_sgemm.py and test_gpu_gemm_bf16.py sit on the boundaries the launchers
-know about; these draws land between them: any M, N, K from 1 up, operands that start at any element of their
-buffers (so rows are 4 B, 8 B or 16 B aligned for fp32 and 2 B to 16 B aligned for bf16), beta zero or not.
+know about; these draws land between them: any M, N, K from 1 up (K up to 4000: beyond about 8000 the rounding of
+a single fp32 sum chain, rocBLAS's included, reaches the sqrt(K) bound used here), operands that start at any
+element of their buffers (so rows are 4 B, 8 B or 16 B aligned for fp32 and 2 B to 16 B aligned for bf16), beta
+zero or not, and where the workspace form of the SGEMM would cut K, that form as well.
 The operands sit between NaNs and the output between guard values, so a read outside a matrix or a store
 outside the output shows. The fp64 product is formed on the device (torch), which keeps the test short; the
 bounds are the ones of the hand-picked tests (1e-5 sqrt(K) max|A| max|B| for fp32, 1e-3 of the largest
@@ -21,7 +23,7 @@ def _draw_shapes(seed, count, big):
     rng = np.random.default_rng(seed)
     out = []
     for i in range(count):
-        kind = i % 4
+        kind = i % 6
         if kind == 0:      # small: one-wave tiles, K from 1 up
             M, N, K = rng.integers(1, 200), rng.integers(1, 200), rng.integers(1, 100)
         elif kind == 1:    # a few hundred: rings, one-wave tiles with K split off
@@ -30,9 +32,16 @@ def _draw_shapes(seed, count, big):
             M, N, K = rng.integers(1, 64), rng.integers(500, 3000), rng.integers(8, 300)
             if rng.integers(0, 2):
                 M, N = N, M
-        else:              # mid sizes: workgroup tiles, partial rounds
+        elif kind == 3:    # mid sizes: workgroup tiles, partial rounds
             M, N, K = rng.integers(1500, big), rng.integers(1500, big), rng.integers(16, 200)
-        out.append((int(M), int(N), int(K), int(rng.integers(0, 8)), int(rng.integers(0, 8)), int(rng.integers(0, 4))))
+        elif kind == 4:    # few tiles and a long K: K cut inside the workgroup, long rings
+            M, N, K = rng.integers(1, 300), rng.integers(1, 1100), rng.integers(1000, 4000)
+        else:              # whole multiples of the tiles: the forms without range checks, when the starts allow
+            M, N, K = 64 * rng.integers(1, 12), 256 * rng.integers(1, 10), 16 * rng.integers(8, 250)
+        starts = [int(rng.integers(0, 8)), int(rng.integers(0, 8)), int(rng.integers(0, 4))]
+        if kind == 5 and rng.integers(0, 2):
+            starts = [0, 0, 0]
+        out.append((int(M), int(N), int(K), *starts))
     return out
 
 
@@ -48,7 +57,7 @@ def _fenced(values: torch.Tensor, start: int, fill) -> torch.Tensor:
 def test_sgemm_kernel_5_random_shapes(prism, seed):
     g = torch.Generator(device=DEV)
     g.manual_seed(seed)
-    for (M, N, K, sa, sb, sc) in _draw_shapes(seed, 60, 4700):
+    for (M, N, K, sa, sb, sc) in _draw_shapes(seed, 72, 4700):
         A = torch.rand((M, K), device=DEV, generator=g) * 2 - 1
         B = torch.rand((K, N), device=DEV, generator=g) * 2 - 1
         C0 = torch.rand((M, N), device=DEV, generator=g) * 2 - 1
@@ -64,6 +73,15 @@ def test_sgemm_kernel_5_random_shapes(prism, seed):
         want = 1.25 * (A.double() @ B.double()) + beta * C0.double()
         err = float((c.double() - want).abs().max())
         assert err <= 1e-5 * np.sqrt(K) + abs(beta) * 2**-22, f"{M}x{N}x{K}: max error {err:.3e}"
+        ws_bytes = prism.sgemm_workspace_size(M, N, K)
+        if ws_bytes:     # the same product through the entry point that may cut K across workgroups
+            ws = torch.full((ws_bytes // 4,), float("nan"), device=DEV)
+            c.copy_(C0)
+            prism.sgemm(M, N, K, 1.25, a, b, beta, c, variant=5, workspace=ws)
+            torch.cuda.synchronize()
+            assert bool((cbuf[:8 + sc] == 777.0).all()) and bool((cbuf[8 + sc + M * N:] == 777.0).all())
+            err = float((c.double() - want).abs().max())
+            assert err <= 1e-5 * np.sqrt(K) + abs(beta) * 2**-22, f"{M}x{N}x{K} with a workspace: max error {err:.3e}"
 
 
 @pytest.mark.parametrize("seed", [4, 5, 6])
@@ -71,7 +89,7 @@ def test_gemm_bf16_random_shapes(prism, seed):
     g = torch.Generator(device=DEV)
     g.manual_seed(seed)
     nan16 = torch.tensor(float("nan"), dtype=torch.bfloat16)
-    for (M, N, K, sa, sb, sc) in _draw_shapes(seed, 60, 4700):
+    for (M, N, K, sa, sb, sc) in _draw_shapes(seed, 72, 4700):
         A = torch.randn((M, K), device=DEV, generator=g).to(torch.bfloat16)
         B = torch.randn((N, K), device=DEV, generator=g).to(torch.bfloat16)
         a, b = _fenced(A, sa, nan16.item()), _fenced(B, sb, nan16.item())
