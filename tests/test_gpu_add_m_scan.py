@@ -124,7 +124,7 @@ def test_scan_fixtures(prism, golden):
 
 TILE_EDGES = [1, 2, 63, 64, 65, 255, 256, 257, 1023, 1024, 1025, 4095, 4096, 4097, 8191, 8192, 8193,
               16383, 16384, 16385, 32768, 65535, 65536, 65537, 100_003, 262_145,
-              (1 << 24) - 1, (1 << 24) + 1, (1 << 24) + 65536 * 3 + 5,
+              1 << 23, (1 << 23) + 1, (1 << 24) - 1, (1 << 24) + 1, (1 << 24) + 65536 * 3 + 5,
               65536 * 300 - 1, 65536 * 300, 65536 * 300 + 1]
 
 
@@ -138,7 +138,7 @@ def test_scan_tile_boundaries(prism, oracle, n):
     assert np.all(got[n:] == -7)
 
 
-@pytest.mark.parametrize("n", [1, 2, 255, 256, 257, 4096, 16385, 65536, 65537, 100_003, (1 << 24) - 1, (1 << 24) + 65536 * 3 + 5,
+@pytest.mark.parametrize("n", [1, 2, 255, 256, 257, 4096, 16385, 65536, 65537, 100_003, 1 << 23, (1 << 23) + 1, (1 << 24) - 1, (1 << 24) + 65536 * 3 + 5,
                                1 << 26])
 def test_exclusive_scan(prism, oracle, n):
     """The exclusive form (out[0] = 0, out[i] = in[0] + ... + in[i-1]) on both tile shapes, out of place with a
@@ -159,7 +159,7 @@ def test_exclusive_scan(prism, oracle, n):
         assert np.array_equal(host(y)[1:], want)
 
 
-@pytest.mark.parametrize("n", [1, 2, 255, 256, 257, 4096, 16385, 65536, 65537, 100_003, (1 << 24) - 1, (1 << 24) + 65536 * 3 + 5,
+@pytest.mark.parametrize("n", [1, 2, 255, 256, 257, 4096, 16385, 65536, 65537, 100_003, 1 << 23, (1 << 23) + 1, (1 << 24) - 1, (1 << 24) + 65536 * 3 + 5,
                                1 << 26])
 def test_running_maximum(prism, oracle, n):
     """The operator form of the scan, out[i] = max(in[0..i]) over int32, on both tile shapes: out of place with a
@@ -280,7 +280,7 @@ def test_scan_workspace_shared_by_calls_of_any_length_and_kind(prism, oracle):
 
 
 SEG_SIZES = [1, 2, 63, 64, 65, 255, 256, 257, 1023, 1025, 4096, 16383, 16384, 16385, 65535, 65536, 65537, 100_003,
-             262_145, (1 << 24) - 1, (1 << 24) + 65536 * 3 + 5, 1 << 26]
+             262_145, 1 << 23, (1 << 23) + 1, (1 << 24) - 1, (1 << 24) + 65536 * 3 + 5, 1 << 26]
 
 
 @pytest.mark.parametrize("n", SEG_SIZES)

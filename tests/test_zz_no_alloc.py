@@ -40,7 +40,7 @@ def test_static_scratch_scan_matches_the_workspace_scan(prism, oracle):
     assert np.array_equal(both(small), oracle.scan_cpu(small))
     # back to a long one (the short call must have cleared the long call's status words), then more shapes
     assert np.array_equal(both(big), oracle.scan_cpu(big))
-    for n in (1, 255, 16384, 16385, 65537, 1 << 20, (1 << 24) - 1, 1 << 26):
+    for n in (1, 255, 16384, 16385, 65537, 1 << 20, 1 << 23, (1 << 23) + 1, (1 << 24) - 1, 1 << 26):
         x = oracle.gen_scan(n, seed=n % 89)
         assert np.array_equal(both(x), oracle.scan_cpu(x)), n
 
