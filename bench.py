@@ -26,10 +26,8 @@ Baselines, not targets.
 from __future__ import annotations
 
 import argparse
-import hashlib
 import json
 import os
-import re
 import sys
 import time
 from pathlib import Path
@@ -44,28 +42,10 @@ PEAK = {  # MI355X published peaks
 
 
 ROOT = Path(__file__).resolve().parent
-TRAFFIC_FILE = ROOT / "profiles" / "hbm_traffic.md"
-KERNEL_SOURCE = {"sgemm": "sgemm.hip", "scan": "scan.hip", "gemm_bf16": "gemm_bf16.hip", "add_m": "add_m.hip"}
-
-
-def source_hash(workload: str) -> str:
-    """First 16 hex digits of the SHA-256 of the kernel source a workload runs."""
-    return hashlib.sha256((ROOT / "prism_amd" / "csrc" / KERNEL_SOURCE[workload]).read_bytes()).hexdigest()[:16]
-
-
-def measured_traffic(workload: str, size: int):
-    """HBM-side bytes per launch (L2 misses: TCC fetches + write-backs) from profiles/hbm_traffic.md, the
-    summary of two `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE, scaled by what the same
-    counters read for a copy of known size). Each row records the hash of the kernel source it was measured
-    on; a row whose hash differs from the source now in the tree is stale and gives None."""
-    try:
-        text = TRAFFIC_FILE.read_text()
-    except OSError:
-        return None
-    for m in re.finditer(r"^\|\s*(\w+)\s*\|\s*(\d+)\s*\|\s*(\d+)\s*\|\s*(\d+)\s*\|\s*([0-9a-f]{16})\s*\|", text, re.M):
-        if m.group(1) == workload and int(m.group(2)) == size:
-            return int(m.group(3)) + int(m.group(4)) if m.group(5) == source_hash(workload) else None
-    return None
+# Helpers shared with the tests live in tests/: the parity gate (fp64_referee), the tables under profiles/
+# (profile_tables) and the streaming calibration kernels (calibrate_stream).
+sys.path.insert(0, str(ROOT / "tests"))
+from profile_tables import measured_traffic, write_kernel_trace_table, write_traffic_table  # noqa: E402
 
 
 def log(*a):
@@ -114,31 +94,9 @@ def time_steps(fn, steps: int, warmup: int):
 
 
 # -------------------------------------------------- full-matrix parity checks --
-
-def sgemm_max_err_fp64(alpha, A, B, beta, C0, C, rows: int = 1024) -> float:
-    """max |C - (alpha A @ B + beta C0)| over EVERY element; the reference product is formed in fp64 on the
-    device (torch's fp64 GEMM), `rows` rows of C at a time."""
-    import torch
-    Bd = B.double()
-    worst = 0.0
-    for s in range(0, A.shape[0], rows):
-        ref = torch.matmul(A[s:s + rows].double(), Bd).mul_(alpha)
-        if beta != 0:
-            ref.add_(C0[s:s + rows].double(), alpha=beta)
-        worst = max(worst, float((C[s:s + rows].double() - ref).abs().max()))
-    return worst
-
-
-def gemm_bf16_max_err_fp64(A, B, D, rows: int = 1024):
-    """(max |D - A @ B^T| over every element, max |A @ B^T|); the product of the bf16 inputs in fp64 on the device."""
-    import torch
-    Bt = B.double().T.contiguous()
-    worst, ref_max = 0.0, 0.0
-    for s in range(0, A.shape[0], rows):
-        ref = torch.matmul(A[s:s + rows].double(), Bt)
-        worst = max(worst, float((D[s:s + rows].double() - ref).abs().max()))
-        ref_max = max(ref_max, float(ref.abs().max()))
-    return worst, ref_max
+# The parity gate is the tests' own full-size check (tests/fp64_referee.py): every element against an fp64
+# product formed on the device, which the GPU tests pin to the CPU oracle on sampled rows.
+from fp64_referee import gemm_bf16_max_err_fp64, sgemm_max_err_fp64  # noqa: E402
 
 
 # ------------------------------------------------------------------ sgemm --
@@ -243,23 +201,24 @@ CALIBRATION_KINDS = {0: "copy_packet_per_lane", 1: "copy_scan_tile_shape", 2: "r
 
 
 def bench_calibration(steps, warmup):
-    """What the memory system gives kernels that only move bytes (prism_calibrate_stream): a 1 GiB copy in
+    """What the memory system gives kernels that only move bytes (tests/native/calibrate_stream.hip): a 1 GiB copy in
     add_m's shape (the counter calibration) and, at the scan's size of 4 GiB per buffer, the copy in add_m's
     shape, the copy in the scan's tile shape, a read-only and a write-only stream."""
     import torch
-    lib, st = _capi()
+    import calibrate_stream
+    lib, st = calibrate_stream.load(), torch.cuda.current_stream().cuda_stream
     n = 1 << 30
     x = torch.randint(-1000, 1001, (n,), dtype=torch.int32, device="cuda")
     y = torch.empty_like(x)
     out = {}
     one_gib = 1 << 30
-    ms = time_steps(lambda: lib.prism_calibrate_stream(0, x.data_ptr(), y.data_ptr(), one_gib, st), steps, warmup)
+    ms = time_steps(lambda: lib.calibrate_stream(0, x.data_ptr(), y.data_ptr(), one_gib, st), steps, warmup)
     if not torch.equal(x[: one_gib // 4], y[: one_gib // 4]):
         raise RuntimeError("calibration copy is wrong")
     out["copy_1GiB"] = {"kernel": "calibrate_copy_packet_kernel", "bytes_read": one_gib, "bytes_written": one_gib,
                         "ms": ms, "GBps": 2.0 * one_gib / ms / 1e6}
     for kind, name in CALIBRATION_KINDS.items():
-        ms = time_steps(lambda: lib.prism_calibrate_stream(kind, x.data_ptr(), y.data_ptr(), 4 * n, st), steps, warmup)
+        ms = time_steps(lambda: lib.calibrate_stream(kind, x.data_ptr(), y.data_ptr(), 4 * n, st), steps, warmup)
         moved = (2 if kind < 2 else 1) * 4.0 * n
         out[name] = {"ms": ms, "GBps": moved / ms / 1e6, "frac_of_peak": moved / ms / 1e6 / PEAK["hbm_GBps"]}
     return out
@@ -349,73 +308,6 @@ def cpu_baseline_add_m(n=1 << 24):
             "sample": f"oracle_add_m on n=2^24, {dt * 1e3:.1f} ms", "numpy_GBps": 8.0 * n / dt_np / 1e9}
 
 
-# ------------------------------------------------- HBM-side traffic table --
-
-TRAFFIC_KERNELS = [  # (workload, size, substring of the kernel name, threads in the grid)
-    ("sgemm", 8192, "sgemm_wave_tile_dma_kernel", 1024 * 1024),
-    ("scan", 1 << 30, "scan_lookback_kernel", (1 << 30) // 65536 * 1024),
-    ("gemm_bf16", 8192, "gemm_bf16_early_kernel", 1024 * 256),
-    ("add_m", 1 << 24, "add_m_vec4_kernel", (1 << 24) // 4),
-    ("add_m", 1 << 28, "add_m_vec4_kernel", (1 << 28) // 4),
-]
-
-
-def write_traffic_table(pmc_dir: str) -> int:
-    """Summarises four `rocprofv3 --pmc` runs of this script into profiles/hbm_traffic.md, the table
-    measured_traffic() reads. Expected in pmc_dir (rocprofv3 -d pmc_dir -o NAME --output-format csv):
-    bench_FETCH_SIZE, bench_WRITE_SIZE (`bench.py --no-configs --no-cpu-baseline --steps 3 --warmup 1`) and
-    calib_FETCH_SIZE, calib_WRITE_SIZE (`bench.py --workload calibrate --steps 3 --warmup 1`)."""
-    import csv
-
-    def readings(name, counter, match, grid=None):
-        vals = []
-        with open(os.path.join(pmc_dir, f"{name}_{counter}_counter_collection.csv"), newline="") as f:
-            for r in csv.DictReader(f):
-                if r["Counter_Name"] == counter and match in r["Kernel_Name"] and (grid is None or int(r["Grid_Size"]) == grid):
-                    vals.append(float(r["Counter_Value"]))
-        return vals
-
-    scale = {}
-    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
-        v = readings("calib", counter, "calibrate_copy_packet_kernel", (1 << 30) // 16)
-        if not v:
-            print(f"no copy kernel in calib_{counter}", file=sys.stderr)
-            return 1
-        scale[counter] = (1 << 20) / (sum(v) / len(v))  # the copy moves 1 GiB = 2^20 KiB each way
-    lines = ["# HBM-side traffic per launch (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)", "",
-             "Written by `python bench.py --traffic-summary $OUT/pmc_traffic` from four counter runs (from /tmp with TMPDIR=/tmp on",
-             "the GPU box, R = repo root, OUT = a scratch directory, C = FETCH_SIZE, then WRITE_SIZE; each run its own process):", "",
-             "    rocprofv3 --pmc $C --kernel-trace -d $OUT/pmc_traffic -o bench_$C --output-format csv -- \\",
-             "        python3 $R/bench.py --steps 3 --warmup 1 --no-configs --no-cpu-baseline",
-             "    rocprofv3 --pmc $C --kernel-trace -d $OUT/pmc_traffic -o calib_$C --output-format csv -- \\",
-             "        python3 $R/bench.py --workload calibrate --steps 3 --warmup 1", "",
-             "`bench.py` reads the table back for `roofline.traffic`. A row counts only while the hash of its kernel source",
-             "(first 16 hex digits of the SHA-256 of `prism_amd/csrc/<file>`) is the one in the tree; otherwise the bench line",
-             "says `null`. The counters sit at the L2's memory side, so they include what the 256 MiB memory-side cache serves.",
-             "", f"Scale factors from the 1 GiB copy (calibrate_copy_packet_kernel): FETCH_SIZE x {scale['FETCH_SIZE']:.3f}, WRITE_SIZE x {scale['WRITE_SIZE']:.3f}"
-             " (KiB per dispatch -> KiB moved).", "",
-             "| workload | size | bytes read | bytes written | source hash | launches averaged | algorithmic bytes | ratio |",
-             "|---|---:|---:|---:|---|---:|---:|---:|"]
-    algorithmic = {("sgemm", 8192): 4 * 4 * 8192 ** 2, ("scan", 1 << 30): 8 << 30, ("gemm_bf16", 8192): (2 * 2 + 4) * 8192 ** 2,
-                   ("add_m", 1 << 24): 8 << 24, ("add_m", 1 << 28): 8 << 28}
-    for workload, size, match, grid in TRAFFIC_KERNELS:
-        f, w = readings("bench", "FETCH_SIZE", match, grid), readings("bench", "WRITE_SIZE", match, grid)
-        if not f or not w:
-            print(f"no readings for {workload} {size}", file=sys.stderr)
-            continue
-        rd = int(sum(f) / len(f) * scale["FETCH_SIZE"] * 1024)
-        wr = int(sum(w) / len(w) * scale["WRITE_SIZE"] * 1024)
-        alg = algorithmic[(workload, size)]
-        lines.append(f"| {workload} | {size} | {rd} | {wr} | {source_hash(workload)} | {min(len(f), len(w))} | {alg} | {(rd + wr) / alg:.3f} |")
-    lines += ["", "The streaming kernels move their algorithmic bytes and nothing else (the scan's status words and polls are",
-              "0.1 %). The GEMMs are compute-bound; their HBM-side reads are L2 misses of re-used A / B panels: with 256 x 256",
-              "tiles and an 8 x 4 tile patch per XCD, 12 of the 64 panel reads of a patch miss, which is what an XCD's 32 CUs",
-              "working in step can reach at best with that patch shape."]
-    TRAFFIC_FILE.write_text("\n".join(lines) + "\n")
-    print("\n".join(lines))
-    return 0
-
-
 # ------------------------------------------------------------------- main --
 
 def main() -> int:
@@ -429,9 +321,14 @@ def main() -> int:
                     help="skip the table of the other BASELINE configurations (also.configs)")
     ap.add_argument("--traffic-summary", metavar="DIR", default=None,
                     help="no GPU work: summarise the rocprofv3 --pmc outputs in DIR into profiles/hbm_traffic.md")
+    ap.add_argument("--trace-summary", metavar="DIR", default=None,
+                    help="no GPU work: summarise the rocprofv3 --kernel-trace --stats output in DIR into "
+                         "profiles/bench_all_kernels_kernel_trace.md")
     args = ap.parse_args()
     if args.traffic_summary:
         return write_traffic_table(args.traffic_summary)
+    if args.trace_summary:
+        return write_kernel_trace_table(args.trace_summary)
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no multi-GPU part); run with --gpus 1",
               file=sys.stderr)
@@ -448,7 +345,7 @@ def main() -> int:
     want = lambda w: args.workload in ("all", w)
 
     if args.workload == "calibrate":
-        # Plain streaming kernels of known size (prism_calibrate_stream): the copy of 1 GiB (kind 0) is what the
+        # Plain streaming kernels of known size (tests/native/calibrate_stream.hip): the copy of 1 GiB (kind 0) is what the
         # FETCH_SIZE / WRITE_SIZE counters of a `rocprofv3 --pmc` run of this script are scaled by; all four kinds
         # at 4 GiB are the ceiling the streaming workloads are compared with.
         print(json.dumps({"workload": "calibrate", **bench_calibration(K, W)}), flush=True)

@@ -52,18 +52,6 @@ int prism_device_info(int* cu_count, int* clock_khz, int* wavefront_size,
  */
 int prism_tile_coords(int workgroup_id, int tiles_m, int tiles_n, int* tile_m, int* tile_n);
 
-/*
- * Measurement aid, no counterpart in the reference: a kernel that only moves
- * `bytes` bytes (a multiple of 16, both buffers 16-byte aligned), in the access
- * shapes the streaming kernels here use. kind 0: copy in -> out, one 16-byte
- * packet per lane (the shape of add_m); 1: copy in the scan's tile shape (a
- * workgroup loads 256 KiB, then stores them); 2: read `in` only (`out` needs
- * 256 bytes); 3: write `out` only. The benchmark times them beside add_m and
- * the scan as the ceiling this GPU's memory system gives such kernels, and
- * scales hardware traffic counters by a copy of known size.
- */
-int prism_calibrate_stream(int kind, const void* in, void* out, size_t bytes, void* stream);
-
 /* ----------------------------------------------------------------- add_m -- */
 
 /*

@@ -16,7 +16,7 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "libprism_amd.so"
-SOURCES = ["capi.hip", "add_m.hip", "scan.hip", "sgemm.hip", "gemm_bf16.hip", "calibrate.hip", "regroup.hip"]
+SOURCES = ["capi.hip", "add_m.hip", "scan.hip", "sgemm.hip", "gemm_bf16.hip", "regroup.hip"]
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_*_f32 out of scalar
 # float code; the kernels here get their fp32 throughput from MFMA instead.
@@ -37,11 +37,7 @@ def hipcc_path() -> str:
     raise RuntimeError("hipcc not found (set HIPCC or add /opt/rocm/bin to PATH)")
 
 
-def build(verbose: bool = False, extra_flags: list[str] | None = None, output: Path | None = None) -> Path:
-    """Compile every kernel source into one shared library; always recompiles."""
-    out = Path(output) if output else LIB_PATH
-    cmd = [hipcc_path(), *HIPCC_FLAGS, *(extra_flags or []), "-shared", "-o", str(out)]
-    cmd += [str(CSRC / s) for s in SOURCES]
+def _run(cmd: list[str], verbose: bool) -> None:
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)
@@ -52,6 +48,25 @@ def build(verbose: bool = False, extra_flags: list[str] | None = None, output: P
         raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{err}")
     if verbose and err.strip():
         print(err, file=sys.stderr)
+
+
+def build(verbose: bool = False, extra_flags: list[str] | None = None, output: Path | None = None,
+          sources: list[str] | None = None) -> Path:
+    """Compile every kernel source into one shared library; always recompiles. The sources are compiled
+    side by side (one hipcc process each) into a scratch directory and linked."""
+    import tempfile
+    from concurrent.futures import ThreadPoolExecutor
+
+    out = Path(output) if output else LIB_PATH
+    hipcc = hipcc_path()
+    flags = [*HIPCC_FLAGS, *(extra_flags or [])]
+    names = sources or SOURCES
+    with tempfile.TemporaryDirectory(prefix="prism_amd_build_") as tmp:
+        objs = [str(Path(tmp) / (Path(s).stem + ".o")) for s in names]
+        jobs = [[hipcc, *flags, "-c", str(CSRC / s), "-o", o] for s, o in zip(names, objs)]
+        with ThreadPoolExecutor(max_workers=min(len(jobs), os.cpu_count() or 1, 16)) as pool:
+            list(pool.map(lambda c: _run(c, verbose), jobs))
+        _run([hipcc, *flags, "-shared", "-o", str(out), *objs], verbose)
     return out
 
 

@@ -51,10 +51,6 @@ int prism_tile_coords(int workgroup_id, int tiles_m, int tiles_n, int* tile_m, i
     return 0;
 }
 
-int prism_calibrate_stream(int kind, const void* in, void* out, size_t bytes, void* stream) {
-    return launch_calibrate_stream(kind, in, out, bytes, static_cast<hipStream_t>(stream));
-}
-
 int prism_wave_regroup_i32(const int32_t* in, int32_t* out, size_t n, int items_per_lane, int direction, void* stream) {
     return launch_wave_regroup(in, out, n, items_per_lane, direction, static_cast<hipStream_t>(stream));
 }

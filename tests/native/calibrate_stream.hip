@@ -1,7 +1,13 @@
 // Streaming calibration kernels: what this GPU's memory system gives a kernel that only moves bytes,
-// in the two access shapes the streaming kernels of this library use. bench.py times them next to
+// in the two access shapes the streaming kernels of libprism_amd.so use. bench.py times them next to
 // add_m and the scan (the ceiling those are measured against besides the published 8 TB/s) and scales
-// the FETCH_SIZE / WRITE_SIZE counters by what they read for a copy of known size.
+// the FETCH_SIZE / WRITE_SIZE counters by what they read for a copy of known size. A measurement aid:
+// built into its own small library (libcalibrate_stream.so, see tests/calibrate_stream.py), not part of
+// the product library or its header.
+//
+//   int calibrate_stream(int kind, const void* in, void* out, size_t bytes, void* stream)
+//       0 = launched; 1 = bad argument; otherwise the hipError_t of the launch. `bytes` is a multiple of
+//       16, both buffers 16-byte aligned.
 //
 //   kind 0  copy, one 16 B packet per lane, 256-thread workgroups (add_m's shape): the workgroups sweep
 //           memory in dispatch order as one compact front
@@ -9,10 +15,14 @@
 //           workgroup loads its whole 256 KiB tile, then stores it
 //   kind 2  read only, shape of kind 0 (4 bytes per workgroup are written so that the loads are kept)
 //   kind 3  write only, shape of kind 0
-#include "common.h"
+#include <hip/hip_runtime.h>
 
-namespace prism {
+#include <cstddef>
+#include <cstdint>
+
 namespace {
+
+constexpr int kWave = 64;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
@@ -56,17 +66,17 @@ __global__ __launch_bounds__(256) void calibrate_write_kernel(u32x4* __restrict_
 
 }  // namespace
 
-int launch_calibrate_stream(int kind, const void* in, void* out, size_t bytes, hipStream_t s) {
-    if (kind < 0 || kind > 3) return fail(1, "prism_calibrate_stream: unknown kind %d", kind);
+extern "C" int calibrate_stream(int kind, const void* in, void* out, size_t bytes, void* stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (kind < 0 || kind > 3) return 1;
     if (bytes == 0) return 0;
-    if ((kind != 3 && in == nullptr) || out == nullptr) return fail(1, "prism_calibrate_stream: null pointer");
-    if (bytes % 16 != 0 || !aligned16(in) || !aligned16(out))
-        return fail(1, "prism_calibrate_stream: buffers must be 16-byte aligned and a multiple of 16 bytes long");
-    if (kind == 2 && bytes < 256) return fail(1, "prism_calibrate_stream: the read-only kind needs 256 bytes of `out`");
+    if ((kind != 3 && in == nullptr) || out == nullptr) return 1;
+    if (bytes % 16 != 0 || (reinterpret_cast<uintptr_t>(in) & 15u) || (reinterpret_cast<uintptr_t>(out) & 15u)) return 1;
+    if (kind == 2 && bytes < 256) return 1;  // the read-only kind writes into the first 256 bytes of `out`
     const size_t n_vec = bytes / 16;
     const size_t per_block = kind == 1 ? static_cast<size_t>(kTileThreads) * kTilePackets : 256;
-    const size_t blocks = ceil_div(n_vec, per_block);
-    if (blocks > 0x7fffffffull) return fail(1, "prism_calibrate_stream: %zu bytes are too many", bytes);
+    const size_t blocks = (n_vec + per_block - 1) / per_block;
+    if (blocks > 0x7fffffffull) return 1;
     const dim3 grid(static_cast<unsigned>(blocks));
     const u32x4* src = static_cast<const u32x4*>(in);
     u32x4* dst = static_cast<u32x4*>(out);
@@ -76,7 +86,5 @@ int launch_calibrate_stream(int kind, const void* in, void* out, size_t bytes, h
         case 2: calibrate_read_kernel<<<grid, dim3(256), 0, s>>>(src, static_cast<uint32_t*>(out), n_vec); break;
         default: calibrate_write_kernel<<<grid, dim3(256), 0, s>>>(dst, n_vec); break;
     }
-    return check_launch("calibrate kernel");
+    return static_cast<int>(hipGetLastError());
 }
-
-}  // namespace prism

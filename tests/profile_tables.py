@@ -1,0 +1,173 @@
+"""The tables under profiles/ that bench.py reads and writes.
+
+profiles/hbm_traffic.md holds the HBM-side bytes per launch of the headline kernels (`roofline.traffic` in the
+benchmark line); profiles/bench_all_kernels_kernel_trace.md the per-kernel durations of a `rocprofv3
+--kernel-trace --stats` run of the benchmark beside the benchmark's own event timing. Both are written from the
+profiler's raw CSV files by the functions below (`python bench.py --traffic-summary DIR`, `python bench.py
+--trace-summary DIR`), never by hand, and tests/test_bench_tables.py checks that the traffic rows belong to the
+kernel sources in the tree. No GPU work happens here.
+"""
+from __future__ import annotations
+
+import hashlib
+import json
+import os
+import re
+import sys
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parents[1]
+TRAFFIC_FILE = ROOT / "profiles" / "hbm_traffic.md"
+KERNEL_SOURCE = {"sgemm": "sgemm.hip", "scan": "scan.hip", "gemm_bf16": "gemm_bf16.hip", "add_m": "add_m.hip"}
+
+
+def source_hash(workload: str) -> str:
+    """First 16 hex digits of the SHA-256 of the kernel source a workload runs."""
+    return hashlib.sha256((ROOT / "prism_amd" / "csrc" / KERNEL_SOURCE[workload]).read_bytes()).hexdigest()[:16]
+
+
+def measured_traffic(workload: str, size: int):
+    """HBM-side bytes per launch (L2 misses: TCC fetches + write-backs) from profiles/hbm_traffic.md, the
+    summary of two `rocprofv3 --pmc` runs of bench.py (FETCH_SIZE, then WRITE_SIZE, scaled by what the same
+    counters read for a copy of known size). Each row records the hash of the kernel source it was measured
+    on; a row whose hash differs from the source now in the tree is stale and gives None."""
+    try:
+        text = TRAFFIC_FILE.read_text()
+    except OSError:
+        return None
+    for m in re.finditer(r"^\|\s*(\w+)\s*\|\s*(\d+)\s*\|\s*(\d+)\s*\|\s*(\d+)\s*\|\s*([0-9a-f]{16})\s*\|", text, re.M):
+        if m.group(1) == workload and int(m.group(2)) == size:
+            return int(m.group(3)) + int(m.group(4)) if m.group(5) == source_hash(workload) else None
+    return None
+
+
+# ------------------------------------------------- HBM-side traffic table --
+
+TRAFFIC_KERNELS = [  # (workload, size, substring of the kernel name, threads in the grid)
+    ("sgemm", 8192, "sgemm_wave_tile_dma_kernel", 1024 * 1024),
+    ("scan", 1 << 30, "scan_lookback_kernel", (1 << 30) // 65536 * 1024),
+    ("gemm_bf16", 8192, "gemm_bf16_early_kernel", 1024 * 256),
+    ("add_m", 1 << 24, "add_m_vec4_kernel", (1 << 24) // 4),
+    ("add_m", 1 << 28, "add_m_vec4_kernel", (1 << 28) // 4),
+]
+
+
+def write_traffic_table(pmc_dir: str) -> int:
+    """Summarises four `rocprofv3 --pmc` runs of bench.py into profiles/hbm_traffic.md, the table
+    measured_traffic() reads. Expected in pmc_dir (rocprofv3 -d pmc_dir -o NAME --output-format csv):
+    bench_FETCH_SIZE, bench_WRITE_SIZE (`bench.py --no-configs --no-cpu-baseline --steps 3 --warmup 1`) and
+    calib_FETCH_SIZE, calib_WRITE_SIZE (`bench.py --workload calibrate --steps 3 --warmup 1`)."""
+    import csv
+
+    def readings(name, counter, match, grid=None):
+        vals = []
+        with open(os.path.join(pmc_dir, f"{name}_{counter}_counter_collection.csv"), newline="") as f:
+            for r in csv.DictReader(f):
+                if r["Counter_Name"] == counter and match in r["Kernel_Name"] and (grid is None or int(r["Grid_Size"]) == grid):
+                    vals.append(float(r["Counter_Value"]))
+        return vals
+
+    scale = {}
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        v = readings("calib", counter, "calibrate_copy_packet_kernel", (1 << 30) // 16)
+        if not v:
+            print(f"no copy kernel in calib_{counter}", file=sys.stderr)
+            return 1
+        scale[counter] = (1 << 20) / (sum(v) / len(v))  # the copy moves 1 GiB = 2^20 KiB each way
+    lines = ["# HBM-side traffic per launch (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)", "",
+             "Written by `python bench.py --traffic-summary $OUT/pmc_traffic` from four counter runs (from /tmp with TMPDIR=/tmp on",
+             "the GPU box, R = repo root, OUT = a scratch directory, C = FETCH_SIZE, then WRITE_SIZE; each run its own process):", "",
+             "    rocprofv3 --pmc $C --kernel-trace -d $OUT/pmc_traffic -o bench_$C --output-format csv -- \\",
+             "        python3 $R/bench.py --steps 3 --warmup 1 --no-configs --no-cpu-baseline",
+             "    rocprofv3 --pmc $C --kernel-trace -d $OUT/pmc_traffic -o calib_$C --output-format csv -- \\",
+             "        python3 $R/bench.py --workload calibrate --steps 3 --warmup 1", "",
+             "`bench.py` reads the table back for `roofline.traffic`. A row counts only while the hash of its kernel source",
+             "(first 16 hex digits of the SHA-256 of `prism_amd/csrc/<file>`) is the one in the tree; otherwise the bench line",
+             "says `null`. The counters sit at the L2's memory side, so they include what the 256 MiB memory-side cache serves.",
+             "", f"Scale factors from the 1 GiB copy (calibrate_copy_packet_kernel): FETCH_SIZE x {scale['FETCH_SIZE']:.3f}, WRITE_SIZE x {scale['WRITE_SIZE']:.3f}"
+             " (KiB per dispatch -> KiB moved).", "",
+             "| workload | size | bytes read | bytes written | source hash | launches averaged | algorithmic bytes | ratio |",
+             "|---|---:|---:|---:|---|---:|---:|---:|"]
+    algorithmic = {("sgemm", 8192): 4 * 4 * 8192 ** 2, ("scan", 1 << 30): 8 << 30, ("gemm_bf16", 8192): (2 * 2 + 4) * 8192 ** 2,
+                   ("add_m", 1 << 24): 8 << 24, ("add_m", 1 << 28): 8 << 28}
+    for workload, size, match, grid in TRAFFIC_KERNELS:
+        f, w = readings("bench", "FETCH_SIZE", match, grid), readings("bench", "WRITE_SIZE", match, grid)
+        if not f or not w:
+            print(f"no readings for {workload} {size}", file=sys.stderr)
+            continue
+        rd = int(sum(f) / len(f) * scale["FETCH_SIZE"] * 1024)
+        wr = int(sum(w) / len(w) * scale["WRITE_SIZE"] * 1024)
+        alg = algorithmic[(workload, size)]
+        lines.append(f"| {workload} | {size} | {rd} | {wr} | {source_hash(workload)} | {min(len(f), len(w))} | {alg} | {(rd + wr) / alg:.3f} |")
+    lines += ["", "The streaming kernels move their algorithmic bytes and nothing else (the scan's status words and polls are",
+              "0.1 %). The GEMMs are compute-bound; their HBM-side reads are L2 misses of re-used A / B panels: with 256 x 256",
+              "tiles and an 8 x 4 tile patch per XCD, 12 of the 64 panel reads of a patch miss, which is what an XCD's 32 CUs",
+              "working in step can reach at best with that patch shape."]
+    TRAFFIC_FILE.write_text("\n".join(lines) + "\n")
+    print("\n".join(lines))
+    return 0
+
+
+# ------------------------------------------------------ kernel-trace table --
+
+TRACE_FILE = ROOT / "profiles" / "bench_all_kernels_kernel_trace.md"
+PEAKS = {"sgemm": (157.3, "TFLOP/s fp32 MFMA"), "gemm_bf16": (2500.0, "TFLOP/s bf16 MFMA"),
+         "scan": (8000.0, "GB/s HBM"), "add_m": (8000.0, "GB/s HBM"), "add_m_2p28": (8000.0, "GB/s HBM")}
+TRACE_KERNELS = [  # (key of the benchmark line, substring of the kernel name, work per launch, unit divisor)
+    ("sgemm", "sgemm_wave_tile_dma_kernel<256, 256, 32, 32, 128, false, false, false>", 2.0 * 8192 ** 3, 1e12),
+    ("scan", "scan_lookback_kernel<prism::(anonymous namespace)::BigCfg", 8.0 * (1 << 30), 1e9),
+    ("gemm_bf16", "gemm_bf16_", 2.0 * 8192 ** 3, 1e12),
+    ("add_m_2p28", "add_m_vec4_kernel<true>", 8.0 * (1 << 28), 1e9),
+    ("add_m", "add_m_vec4_kernel<false>", 8.0 * (1 << 24), 1e9),
+]
+
+
+def write_kernel_trace_table(prof_dir: str) -> int:
+    """Summarises one `rocprofv3 --kernel-trace --stats` run of bench.py into
+    profiles/bench_all_kernels_kernel_trace.md. Expected in prof_dir: bench_kernel_stats.csv (rocprofv3 -d prof_dir
+    -o bench --output-format csv) and bench.json, the line the profiled run printed."""
+    import csv
+
+    with open(os.path.join(prof_dir, "bench_kernel_stats.csv"), newline="") as f:
+        stats = list(csv.DictReader(f))
+    with open(os.path.join(prof_dir, "bench.json")) as f:
+        line = json.loads([l for l in f.read().splitlines() if l.startswith("{")][-1])
+    timed = {"sgemm": line, **{k: v for k, v in line["also"].items() if isinstance(v, dict) and "ms" in v}}
+    out = ["# rocprofv3 kernel-trace summary: bench.py, the headline workloads (MI355X, gfx950)", "",
+           "Written by `python bench.py --trace-summary $OUT/prof_trace` from one profiled run (from /tmp with TMPDIR=/tmp on",
+           "the GPU box, R = repo root, OUT = a scratch directory):", "",
+           "    rocprofv3 --kernel-trace --stats -d $OUT/prof_trace -o bench --output-format csv -- \\",
+           "        python3 $R/bench.py --no-configs --no-cpu-baseline > $OUT/prof_trace/bench.json", "",
+           "Workloads: sgemm 8192^3 (kernel 5, alpha 1, beta 0.5), scan int32 n=2^30, gemm_bf16 8192^3, add_m n=2^24 and 2^28.",
+           f"Each kernel runs once for the parity gate, for {line.get('settle_ms', 150):.0f} ms of untimed settling, {line['warmup']} warm-up and {line['steps']} timed steps,",
+           "hence the call counts; the profiler's average covers all of them (the cold first call is the `max` column), the",
+           "last column is the benchmark's own event timing of the timed steps of the same run.", "",
+           "| kernel (prism::) | calls | avg us | min us | max us | bench.py ms/step | achieved | peak | fraction |",
+           "|---|---:|---:|---:|---:|---:|---:|---|---:|"]
+    for key, match, work, div in TRACE_KERNELS:
+        rows = [r for r in stats if match in r["Name"]]
+        if not rows or key not in timed:
+            print(f"no kernel or no timing for {key}", file=sys.stderr)
+            continue
+        r = max(rows, key=lambda r: float(r["TotalDurationNs"]))
+        name = re.sub(r"^void ", "", r["Name"]).replace("prism::(anonymous namespace)::", "")
+        name = name[: name.index("(")] if "(" in name else name
+        ms = timed[key]["ms_per_step"] if key == "sgemm" else timed[key]["ms"]
+        achieved = work / (ms * 1e-3) / div
+        peak, unit = PEAKS[key]
+        out.append(f"| `{name}` | {r['Calls']} | {float(r['AverageNs']) / 1e3:.2f} | {float(r['MinNs']) / 1e3:.2f} | "
+                   f"{float(r['MaxNs']) / 1e3:.2f} | {ms:.4f} | {achieved:.1f} | {peak:g} {unit} | {achieved / peak:.3f} |")
+    out += ["", "Work per launch: sgemm and gemm_bf16 2 * 8192^3 flop, scan 2 * 4 * 2^30 B, add_m 8 B per element. add_m at 2^24",
+            "re-reads and re-writes the same 128 MiB every step, which the 256 MiB memory-side cache partly serves: the",
+            "HBM-bound add_m figure is the 2^28 one.", "",
+            "All kernels of this library in the run (the streaming calibration copies and PyTorch's own kernels left out):", "",
+            "| kernel | calls | average us | total ms |", "|---|---:|---:|---:|"]
+    for r in sorted(stats, key=lambda r: -float(r["TotalDurationNs"])):
+        if "prism::" not in r["Name"]:
+            continue
+        name = re.sub(r"^void ", "", r["Name"]).replace("prism::(anonymous namespace)::", "")
+        name = name[: name.index("(")] if "(" in name else name
+        out.append(f"| `{name}` | {r['Calls']} | {float(r['AverageNs']) / 1e3:.1f} | {float(r['TotalDurationNs']) / 1e6:.1f} |")
+    TRACE_FILE.write_text("\n".join(out) + "\n")
+    print("\n".join(out))
+    return 0

@@ -4,12 +4,11 @@ import re
 import sys
 from pathlib import Path
 
-ROOT = Path(__file__).resolve().parents[1]
-sys.path.insert(0, str(ROOT))
+sys.path.insert(0, str(Path(__file__).resolve().parent))
 
 
 def test_traffic_table_rows_match_the_kernel_sources_in_the_tree():
-    import bench
+    import profile_tables as bench
     text = bench.TRAFFIC_FILE.read_text()
     rows = re.findall(r"^\|\s*(\w+)\s*\|\s*(\d+)\s*\|\s*\d+\s*\|\s*\d+\s*\|\s*([0-9a-f]{16})\s*\|", text, re.M)
     assert {(w, int(n)) for w, n, _ in rows} >= {("sgemm", 8192), ("scan", 1 << 30), ("gemm_bf16", 8192), ("add_m", 1 << 28)}

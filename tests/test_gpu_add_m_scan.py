@@ -91,25 +91,25 @@ def test_wave_regroup_blocked_and_striped(prism, items):
 
 
 def test_calibration_streams(prism):
-    """prism_calibrate_stream: both copy shapes copy exactly `bytes` bytes and nothing more; the one-way
-    kinds run; bad arguments are refused."""
-    from prism_amd import _lib
-    lib = _lib.load()
+    """The benchmark's calibration kernels (tests/native/calibrate_stream.hip): both copy shapes copy exactly
+    `bytes` bytes and nothing more; the one-way kinds run; bad arguments are refused."""
+    import calibrate_stream
+    lib = calibrate_stream.load()
     n = (1 << 22) + 1024 * 3 + 4  # not a whole number of either kind's workgroups
     x = torch.randint(-2**31, 2**31 - 1, (n + 64,), dtype=torch.int32, device=DEV)
     for kind in (0, 1):
         y = torch.full((n + 64,), 12345, dtype=torch.int32, device=DEV)
-        assert lib.prism_calibrate_stream(kind, x.data_ptr(), y.data_ptr(), 4 * n, None) == 0
+        assert lib.calibrate_stream(kind, x.data_ptr(), y.data_ptr(), 4 * n, None) == 0
         torch.cuda.synchronize()
         assert torch.equal(y[:n], x[:n]) and bool((y[n:] == 12345).all()), kind
     y = torch.zeros(n, dtype=torch.int32, device=DEV)
-    assert lib.prism_calibrate_stream(2, x.data_ptr(), y.data_ptr(), 4 * n, None) == 0
-    assert lib.prism_calibrate_stream(3, None, y.data_ptr(), 4 * n, None) == 0
+    assert lib.calibrate_stream(2, x.data_ptr(), y.data_ptr(), 4 * n, None) == 0
+    assert lib.calibrate_stream(3, None, y.data_ptr(), 4 * n, None) == 0
     torch.cuda.synchronize()
     assert int(y[4]) == 1 and int(y[5]) == 1 and int(y[6]) == 2 and int(y[7]) == 3  # packet 1 = {1, 1, 2, 3}
-    assert lib.prism_calibrate_stream(4, x.data_ptr(), y.data_ptr(), 64, None) == 1
-    assert lib.prism_calibrate_stream(0, x.data_ptr(), y.data_ptr(), 60, None) == 1
-    assert lib.prism_calibrate_stream(0, x[1:].data_ptr(), y.data_ptr(), 64, None) == 1
+    assert lib.calibrate_stream(4, x.data_ptr(), y.data_ptr(), 64, None) == 1
+    assert lib.calibrate_stream(0, x.data_ptr(), y.data_ptr(), 60, None) == 1
+    assert lib.calibrate_stream(0, x[1:].data_ptr(), y.data_ptr(), 64, None) == 1
 
 
 # -------------------------------------------------------------------- scan --

@@ -197,17 +197,19 @@ def test_no_write_outside_and_k_zero(prism, oracle):
 
 
 @pytest.mark.parametrize("n", [4096, 8192, 16384])
-def test_baseline_sizes_full(prism, n):
+def test_baseline_sizes_full(prism, oracle, n):
     """BASELINE sizes: N(0,1) inputs rounded to bf16; EVERY element against an fp64 product of the rounded
-    inputs formed on the device (bench.gemm_bf16_max_err_fp64), bound 1e-3 relative to the largest element."""
-    import bench
+    inputs formed on the device (fp64_referee.gemm_bf16_max_err_fp64), bound 1e-3 relative to the largest element.
+    The device product is itself checked against the CPU oracle on 32 sampled rows."""
+    import fp64_referee
     g = torch.Generator(device=DEV)
     g.manual_seed(0)
     A = torch.randn((n, n), dtype=torch.float32, device=DEV, generator=g).to(torch.bfloat16)
     B = torch.randn((n, n), dtype=torch.float32, device=DEV, generator=g).to(torch.bfloat16)
     D = prism.gemm_bf16(A, B)
-    err, ref_max = bench.gemm_bf16_max_err_fp64(A, B, D)
+    err, ref_max = fp64_referee.gemm_bf16_max_err_fp64(A, B, D)
     assert err <= REL * ref_max, f"n = {n}: max error {err:.3e}, largest element {ref_max:.3e}"
+    assert fp64_referee.pin_gemm_bf16_referee(oracle, A, B) <= 1e-9
     # scaling an input by 2 (exact in bf16) scales the output exactly
     D2 = prism.gemm_bf16((A.float() * 2).to(torch.bfloat16), B)
     assert torch.equal(D2, 2.0 * D)

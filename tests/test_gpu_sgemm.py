@@ -425,12 +425,12 @@ def _bound(K, beta):
 
 def _full_check(prism, M, N, K, alpha, beta, variant, linearity=True):
     """Full-size run; EVERY element is compared with an fp64 product formed on the device
-    (bench.sgemm_max_err_fp64: torch's fp64 GEMM on row blocks), bound 1e-5 * sqrt(K) * max|A| * max|B|."""
-    import bench
+    (fp64_referee.sgemm_max_err_fp64: torch's fp64 GEMM on row blocks), bound 1e-5 * sqrt(K) * max|A| * max|B|."""
+    import fp64_referee
     A, B, C0 = _device_inputs(M, N, K)
     c = C0.clone()
     prism.sgemm(M, N, K, alpha, A, B, beta, c, variant=variant)
-    err = bench.sgemm_max_err_fp64(alpha, A, B, beta, C0, c)
+    err = fp64_referee.sgemm_max_err_fp64(alpha, A, B, beta, C0, c)
     assert err <= _bound(K, beta), f"kernel {variant} {M}x{N}x{K}: max error {err:.3e}"
     if linearity:  # doubling alpha with beta = 0 doubles every element exactly
         c1 = torch.empty_like(c)
@@ -442,10 +442,15 @@ def _full_check(prism, M, N, K, alpha, beta, variant, linearity=True):
 
 
 @pytest.mark.parametrize("n", [4096, 8192])
-def test_baseline_square_all_kernels_full_size(prism, n):
+def test_baseline_square_all_kernels_full_size(prism, oracle, n):
     """BASELINE's square sizes 4096 and 8192 (alpha 1, beta 0.5) for every kernel of the progression: every
     element against the fp64 product, and kernels 1, 2, 3, 4, 6 (one fused multiply-add per k, in order)
-    bit-identical to each other."""
+    bit-identical to each other. The device-side fp64 product that judges them is itself compared with the
+    CPU oracle on 32 sampled rows of the same problem."""
+    import fp64_referee
+    A, B, C0 = _device_inputs(n, n, n)
+    assert fp64_referee.pin_sgemm_referee(oracle, 1.0, A, B, 0.5, C0) <= 1e-9
+    del A, B, C0
     first = None
     for v in ALL:
         c = _full_check(prism, n, n, n, 1.0, 0.5, v, linearity=(v == 5))
@@ -459,8 +464,13 @@ def test_wave_tile_16384x16384x512(prism):
 
 
 @pytest.mark.parametrize("shape", [(4096, 4096, 128), (128, 4096, 4096), (8191, 4097, 1023), (16384, 16384, 512)])
-def test_baseline_tail_shapes_all_kernels_full(prism, shape):
-    """BASELINE's non-square and tail shapes (beta = 0) through every kernel, every element against fp64."""
+def test_baseline_tail_shapes_all_kernels_full(prism, oracle, shape):
+    """BASELINE's non-square and tail shapes (beta = 0) through every kernel, every element against fp64
+    (the device product pinned to the CPU oracle on sampled rows first)."""
+    import fp64_referee
     M, N, K = shape
+    A, B, C0 = _device_inputs(M, N, K)
+    assert fp64_referee.pin_sgemm_referee(oracle, 1.0, A, B, 0.0, C0) <= 1e-9
+    del A, B, C0
     for v in ALL:
         _full_check(prism, M, N, K, 1.0, 0.0, v, linearity=False)
