@@ -1,3 +1,9 @@
+#ifndef PRISM_HANDOVER_REPORT
+#define PRISM_HANDOVER_REPORT
+// written by a hand-over wait that ran out of polls: 1 + 2 * (array number) + (1 when waiting for a filled
+// array) in the low byte, the round above it; the launcher's <name>_status call reads and clears it
+__device__ unsigned int __prism_handover_report = 0;
+#endif
 __global__ void handed_over_gemm(const __bf16* P, const __bf16* Q, float* D, int N, int K, int tiles_n) {
     extern __shared__ __align__(128) char __smem[];
     int __block_id_0 = blockIdx.x;
@@ -53,9 +59,17 @@ __global__ void handed_over_gemm(const __bf16* P, const __bf16* Q, float* D, int
                                                     int lane = __thread_id_3;
                                                     int row = (lane / 4);
                                                     int k8 = (8 * (lane % 4));
-                                                    for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__empty_p_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_p_first * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                    {
+                                                        int __spin = 0;
+                                                        for (; __spin < 65536 && __hip_atomic_load(&__empty_p_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_p_first * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                        if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 1u | (static_cast<unsigned int>(__round_p_first) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                                    }
                                                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-                                                    for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__empty_q_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_q_first * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                    {
+                                                        int __spin = 0;
+                                                        for (; __spin < 65536 && __hip_atomic_load(&__empty_q_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_q_first * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                        if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 5u | (static_cast<unsigned int>(__round_q_first) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                                    }
                                                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                                                     for (int part = 0; part < 4; part++) {
                                                         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&P_rows[(((((16 * part) + row) * K) + k0) + k8)]), (__attribute__((address_space(3))) void*)(&p_first_fill[(512 * part)]), 16, 0, 0);
@@ -69,9 +83,17 @@ __global__ void handed_over_gemm(const __bf16* P, const __bf16* Q, float* D, int
                                                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
                                                     if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__full_q_first, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                                                     __round_q_first += 1;
-                                                    for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__empty_p_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_p_second * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                    {
+                                                        int __spin = 0;
+                                                        for (; __spin < 65536 && __hip_atomic_load(&__empty_p_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_p_second * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                        if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 3u | (static_cast<unsigned int>(__round_p_second) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                                    }
                                                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-                                                    for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__empty_q_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_q_second * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                    {
+                                                        int __spin = 0;
+                                                        for (; __spin < 65536 && __hip_atomic_load(&__empty_q_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_q_second * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                        if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 7u | (static_cast<unsigned int>(__round_q_second) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                                    }
                                                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                                                     for (int part = 0; part < 4; part++) {
                                                         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&P_rows[((((((16 * part) + row) * K) + k0) + 32) + k8)]), (__attribute__((address_space(3))) void*)(&p_second_fill[(512 * part)]), 16, 0, 0);
@@ -99,14 +121,22 @@ __global__ void handed_over_gemm(const __bf16* P, const __bf16* Q, float* D, int
                                                     int lane = __thread_id_3;
                                                     int r = (lane % 16);
                                                     int k8 = (8 * (lane / 16));
-                                                    for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__full_p_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_p_first + 1) * 1); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                    {
+                                                        int __spin = 0;
+                                                        for (; __spin < 65536 && __hip_atomic_load(&__full_p_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_p_first + 1) * 1); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                        if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 2u | (static_cast<unsigned int>(__round_p_first) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                                    }
                                                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                                                     float4 a = reinterpret_cast<float4 *>(&p_first[((((16 * wave) + r) * 32) + k8)])[0];
                                                     __builtin_amdgcn_s_waitcnt(0);
                                                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
                                                     if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__empty_p_first, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                                                     __round_p_first += 1;
-                                                    for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__full_q_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_q_first + 1) * 1); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                    {
+                                                        int __spin = 0;
+                                                        for (; __spin < 65536 && __hip_atomic_load(&__full_q_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_q_first + 1) * 1); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                        if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 6u | (static_cast<unsigned int>(__round_q_first) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                                    }
                                                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                                                     for (int n = 0; n < 4; n++) {
                                                         float4 b = reinterpret_cast<float4 *>(&q_first[((((16 * n) + r) * 32) + k8)])[0];
@@ -125,14 +155,22 @@ __global__ void handed_over_gemm(const __bf16* P, const __bf16* Q, float* D, int
                                                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
                                                     if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__empty_q_first, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                                                     __round_q_first += 1;
-                                                    for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__full_p_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_p_second + 1) * 1); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                    {
+                                                        int __spin = 0;
+                                                        for (; __spin < 65536 && __hip_atomic_load(&__full_p_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_p_second + 1) * 1); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                        if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 4u | (static_cast<unsigned int>(__round_p_second) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                                    }
                                                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                                                     float4 a2 = reinterpret_cast<float4 *>(&p_second[((((16 * wave) + r) * 32) + k8)])[0];
                                                     __builtin_amdgcn_s_waitcnt(0);
                                                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
                                                     if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__empty_p_second, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                                                     __round_p_second += 1;
-                                                    for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__full_q_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_q_second + 1) * 1); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                    {
+                                                        int __spin = 0;
+                                                        for (; __spin < 65536 && __hip_atomic_load(&__full_q_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_q_second + 1) * 1); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                        if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 8u | (static_cast<unsigned int>(__round_q_second) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                                    }
                                                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                                                     for (int n = 0; n < 4; n++) {
                                                         float4 b2 = reinterpret_cast<float4 *>(&q_second[((((16 * n) + r) * 32) + k8)])[0];

@@ -67,6 +67,12 @@ __device__ void multiply_slot(int __block_id, int __thread_id, char* __smem, flo
     return;
 }
 
+#ifndef PRISM_HANDOVER_REPORT
+#define PRISM_HANDOVER_REPORT
+// written by a hand-over wait that ran out of polls: 1 + 2 * (array number) + (1 when waiting for a filled
+// array) in the low byte, the round above it; the launcher's <name>_status call reads and clears it
+__device__ unsigned int __prism_handover_report = 0;
+#endif
 __global__ __launch_bounds__(768) void handed_over_gemm_big(const __bf16* P, const __bf16* Q, float* D, int N, int K, int tiles_m, int tiles_n) {
     extern __shared__ __align__(128) char __smem[];
     int __block_id_0 = blockIdx.x;
@@ -104,14 +110,22 @@ __global__ __launch_bounds__(768) void handed_over_gemm_big(const __bf16* P, con
                                     int __block_id_2 = __block_id_1;
                                     int __thread_id_2 = __thread_id_1;
                                     if (__thread_id_2 >= 0 && __thread_id_2 < 256) {
-                                        for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__empty_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_first * 8); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                        {
+                                            int __spin = 0;
+                                            for (; __spin < 65536 && __hip_atomic_load(&__empty_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_first * 8); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                            if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 1u | (static_cast<unsigned int>(__round_first) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                        }
                                         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                                         fill_slot(__block_id_2, __thread_id_2, __smem, first_fill, P_rows, Q_rows, K, k0);
                                         __builtin_amdgcn_s_waitcnt(0);
                                         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
                                         if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__full_first, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                                         __round_first += 1;
-                                        for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__empty_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_second * 8); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                        {
+                                            int __spin = 0;
+                                            for (; __spin < 65536 && __hip_atomic_load(&__empty_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_second * 8); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                            if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 3u | (static_cast<unsigned int>(__round_second) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                        }
                                         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                                         fill_slot(__block_id_2, __thread_id_2, __smem, second_fill, P_rows, Q_rows, K, (k0 + 64));
                                         __builtin_amdgcn_s_waitcnt(0);
@@ -124,14 +138,22 @@ __global__ __launch_bounds__(768) void handed_over_gemm_big(const __bf16* P, con
                                     int __block_id_2 = __block_id_1;
                                     int __thread_id_2 = __thread_id_1 - 256;
                                     if (__thread_id_2 >= 0 && __thread_id_2 < 512) {
-                                        for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__full_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_first + 1) * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                        {
+                                            int __spin = 0;
+                                            for (; __spin < 65536 && __hip_atomic_load(&__full_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_first + 1) * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                            if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 2u | (static_cast<unsigned int>(__round_first) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                        }
                                         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                                         multiply_slot(__block_id_2, __thread_id_2, __smem, acc, first);
                                         __builtin_amdgcn_s_waitcnt(0);
                                         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
                                         if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__empty_first, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                                         __round_first += 1;
-                                        for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__full_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_second + 1) * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                        {
+                                            int __spin = 0;
+                                            for (; __spin < 65536 && __hip_atomic_load(&__full_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_second + 1) * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                            if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 4u | (static_cast<unsigned int>(__round_second) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                        }
                                         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                                         multiply_slot(__block_id_2, __thread_id_2, __smem, acc, second);
                                         __builtin_amdgcn_s_waitcnt(0);
@@ -185,4 +207,17 @@ extern "C" int handed_over_gemm_big_launch(const __bf16* P, const __bf16* Q, flo
     if (grid_blocks == 0) return 0;
     handed_over_gemm_big<<<dim3(grid_blocks), dim3(768), 0, static_cast<hipStream_t>(stream)>>>(P, Q, D, N, K, tiles_m, tiles_n);
     return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int handed_over_gemm_big_status(void* stream) {
+    hipError_t e = hipStreamSynchronize(static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return static_cast<int>(e);
+    unsigned int word = 0;
+    e = hipMemcpyFromSymbol(&word, HIP_SYMBOL(__prism_handover_report), sizeof(word));
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (word == 0) return 0;
+    const unsigned int zero = 0;
+    e = hipMemcpyToSymbol(HIP_SYMBOL(__prism_handover_report), &zero, sizeof(zero));
+    if (e != hipSuccess) return static_cast<int>(e);
+    return static_cast<int>(0x40000000u | (word & 0x3fffffffu));
 }

@@ -1,3 +1,9 @@
+#ifndef PRISM_HANDOVER_REPORT
+#define PRISM_HANDOVER_REPORT
+// written by a hand-over wait that ran out of polls: 1 + 2 * (array number) + (1 when waiting for a filled
+// array) in the low byte, the round above it; the launcher's <name>_status call reads and clears it
+__device__ unsigned int __prism_handover_report = 0;
+#endif
 __global__ __launch_bounds__(768) void handed_over_sgemm(int M, int N, int K, float alpha, const float* A, const float* B, float beta, float* C, int tiles_n) {
     extern __shared__ __align__(128) char __smem[];
     int __block_id_0 = blockIdx.x;
@@ -35,14 +41,22 @@ __global__ __launch_bounds__(768) void handed_over_sgemm(int M, int N, int K, fl
                                     int __block_id_2 = __block_id_1;
                                     int __thread_id_2 = __thread_id_1;
                                     if (__thread_id_2 >= 0 && __thread_id_2 < 256) {
-                                        for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__empty_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_first * 8); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                        {
+                                            int __spin = 0;
+                                            for (; __spin < 65536 && __hip_atomic_load(&__empty_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_first * 8); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                            if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 1u | (static_cast<unsigned int>(__round_first) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                        }
                                         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                                         fill_slot_f32(__block_id_2, __thread_id_2, __smem, first_fill, A_rows, B_cols, N, K, k0);
                                         __builtin_amdgcn_s_waitcnt(0);
                                         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
                                         if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__full_first, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                                         __round_first += 1;
-                                        for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__empty_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_second * 8); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                        {
+                                            int __spin = 0;
+                                            for (; __spin < 65536 && __hip_atomic_load(&__empty_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_second * 8); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                            if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 3u | (static_cast<unsigned int>(__round_second) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                        }
                                         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                                         fill_slot_f32(__block_id_2, __thread_id_2, __smem, second_fill, A_rows, B_cols, N, K, (k0 + 32));
                                         __builtin_amdgcn_s_waitcnt(0);
@@ -55,14 +69,22 @@ __global__ __launch_bounds__(768) void handed_over_sgemm(int M, int N, int K, fl
                                     int __block_id_2 = __block_id_1;
                                     int __thread_id_2 = __thread_id_1 - 256;
                                     if (__thread_id_2 >= 0 && __thread_id_2 < 512) {
-                                        for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__full_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_first + 1) * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                        {
+                                            int __spin = 0;
+                                            for (; __spin < 65536 && __hip_atomic_load(&__full_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_first + 1) * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                            if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 2u | (static_cast<unsigned int>(__round_first) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                        }
                                         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                                         multiply_slot_f32(__block_id_2, __thread_id_2, __smem, acc, first);
                                         __builtin_amdgcn_s_waitcnt(0);
                                         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
                                         if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__empty_first, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                                         __round_first += 1;
-                                        for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__full_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_second + 1) * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                        {
+                                            int __spin = 0;
+                                            for (; __spin < 65536 && __hip_atomic_load(&__full_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_second + 1) * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                            if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 4u | (static_cast<unsigned int>(__round_second) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                        }
                                         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                                         multiply_slot_f32(__block_id_2, __thread_id_2, __smem, acc, second);
                                         __builtin_amdgcn_s_waitcnt(0);

@@ -453,14 +453,21 @@ def generate(name: str, bounded: bool = False, auto_sync: bool = True, annotate:
     return _Emitter(k, bounded).emit()
 
 
-def generate_launcher(name: str, block_size: int = 256, template: Optional[List[int]] = None) -> str:
+def generate_launcher(name: str, block_size: int = 256, template: Optional[List[int]] = None,
+                      handover_spins: Optional[int] = None) -> str:
     """The kernel plus an `extern "C"` launcher.
 
     Thread-level kernel: bounded kernel and `int <name>_launch(<params>, size_t n, void* stream)`, which
     starts ceil(n / block_size) workgroups. Kernel with a block perspective:
     `int <name>_launch(<params>, unsigned grid_blocks, void* stream)`, which starts grid_blocks workgroups
     of block_size threads with the dynamic LDS the kernel's shared() arrays need; `template` gives the
-    values of its template parameters. block_size is a multiple of the 64-lane wavefront."""
+    values of its template parameters. block_size is a multiple of the 64-lane wavefront.
+
+    A kernel that hands LDS arrays between the cases of a split also gets `int <name>_status(void* stream)`:
+    it waits for the stream and returns 0, or, when a hand-over wait of any launch since the last call ran
+    out of polls (handover_spins of them; the default is the emitter's), 0x40000000 | code, where the code's
+    low byte is 1 + 2 * (number of the array in declaration order) + (1 for a wait for a filled array) and
+    the bits above it the round; the results of that launch are invalid. The call clears the report."""
     if block_size % 64 or not 64 <= block_size <= 1024:
         raise HipgenError("block_size must be a multiple of 64 between 64 and 1024")
     k = _kernel(name)
@@ -470,13 +477,29 @@ def generate_launcher(name: str, block_size: int = 256, template: Optional[List[
         from .hipgen_blocks import BlockEmitter, device_functions_used, generate_blocks
         if k.kind != "global":
             raise HipgenError("only global kernels have launchers")
-        em = BlockEmitter(k, True)
+        em = BlockEmitter(k, True, handover_spins=handover_spins)
         text = em.emit_function()
         if len(template or []) != len(em.template):
             raise HipgenError(f"{name} has {len(em.template)} template parameters, {len(template or [])} values given")
         if k.smem is not None and em.smem_offset > k.smem:
             raise HipgenError(f"{name} declares smem={k.smem} but its shared() arrays take {em.smem_offset} bytes")
-        helpers = "".join(generate_blocks(d) + "\n" for d in device_functions_used(name))
+        from .hipgen_blocks import HANDOVER_REPORT
+        helpers = "".join(generate_blocks(d, handover_spins=handover_spins) + "\n" for d in device_functions_used(name))
+        status = ""
+        if HANDOVER_REPORT in helpers + text:
+            status = (
+                f'\nextern "C" int {name}_status(void* stream) {{\n'
+                "    hipError_t e = hipStreamSynchronize(static_cast<hipStream_t>(stream));\n"
+                "    if (e != hipSuccess) return static_cast<int>(e);\n"
+                "    unsigned int word = 0;\n"
+                f"    e = hipMemcpyFromSymbol(&word, HIP_SYMBOL({HANDOVER_REPORT}), sizeof(word));\n"
+                "    if (e != hipSuccess) return static_cast<int>(e);\n"
+                "    if (word == 0) return 0;\n"
+                "    const unsigned int zero = 0;\n"
+                f"    e = hipMemcpyToSymbol(HIP_SYMBOL({HANDOVER_REPORT}), &zero, sizeof(zero));\n"
+                "    if (e != hipSuccess) return static_cast<int>(e);\n"
+                "    return static_cast<int>(0x40000000u | (word & 0x3fffffffu));\n"
+                "}\n")
         targs = "<" + ", ".join(str(int(v)) for v in template) + ">" if template else ""
         params = ", ".join(f"{t} {n}" for t, n in em.params)
         args = ", ".join(n for _, n in em.params)
@@ -488,7 +511,7 @@ def generate_launcher(name: str, block_size: int = 256, template: Optional[List[
             f"    {name}{targs}<<<dim3(grid_blocks), dim3({block_size}), {em.smem_offset}, static_cast<hipStream_t>(stream)>>>"
             f"({args});\n"
             "    return static_cast<int>(hipGetLastError());\n"
-            "}\n")
+            "}\n" + status)
     if template:
         raise HipgenError("thread-level kernels take no template values")
     em = _Emitter(k, True)
@@ -509,7 +532,7 @@ def generate_launcher(name: str, block_size: int = 256, template: Optional[List[
 
 
 def build(name: str, out_dir: Optional[str] = None, block_size: int = 256,
-          template: Optional[List[int]] = None) -> ctypes.CDLL:
+          template: Optional[List[int]] = None, handover_spins: Optional[int] = None) -> ctypes.CDLL:
     """Compile `generate_launcher(name, block_size, template)` for gfx950 and load it. The handle's
     `<name>_launch` takes the kernel's parameters (device pointers as integers), then the element count
     (thread-level kernels) or the number of workgroups (kernels with a block perspective), then a stream."""
@@ -517,7 +540,7 @@ def build(name: str, out_dir: Optional[str] = None, block_size: int = 256,
     d = Path(out_dir) if out_dir else Path(tempfile.mkdtemp(prefix="prism_hipgen_"))
     d.mkdir(parents=True, exist_ok=True)
     src, lib = d / f"{name}.hip", d / f"lib{name}.so"
-    src.write_text(generate_launcher(name, block_size, template))
+    src.write_text(generate_launcher(name, block_size, template, handover_spins))
     proc = subprocess.run([hipcc_path(), *HIPCC_FLAGS, "-shared", "-o", str(lib), str(src)],
                           capture_output=True, text=True)
     if proc.returncode != 0:

@@ -478,9 +478,22 @@ class _SyncPlan:
 
 # -------------------------------------------------------------------- emitter --
 
+HANDOVER_REPORT = "__prism_handover_report"   # file-scope device word a hand-over wait that gives up writes
+HANDOVER_REPORT_DEFINITION = (
+    "#ifndef PRISM_HANDOVER_REPORT\n#define PRISM_HANDOVER_REPORT\n"
+    "// written by a hand-over wait that ran out of polls: 1 + 2 * (array number) + (1 when waiting for a filled\n"
+    "// array) in the low byte, the round above it; the launcher's <name>_status call reads and clears it\n"
+    f"__device__ unsigned int {HANDOVER_REPORT} = 0;\n#endif\n")
+
+
 class BlockEmitter:
-    def __init__(self, kernel: Kernel, auto_sync: bool = True, annotate: bool = False):
+    def __init__(self, kernel: Kernel, auto_sync: bool = True, annotate: bool = False,
+                 handover_spins: Optional[int] = None):
         self.k = kernel
+        if handover_spins is not None:
+            if not 0 <= handover_spins <= 1 << 30:
+                raise HipgenError("handover_spins must lie between 0 and 2^30")
+            self.HANDOVER_SPINS = handover_spins  # 0: every wait gives up at once (a way to exercise the give-up path)
         self.annotate = annotate          # a comment in front of every barrier says what it is for
         self.auto_sync = auto_sync
         self.out: List[str] = []
@@ -675,11 +688,22 @@ class BlockEmitter:
     HANDOVER_SPINS = 1 << 16   # a wait gives up after this many polls (milliseconds; a real wait takes microseconds), so that a broken protocol cannot hang the GPU
 
     def wait_for(self, array: str, what: str) -> None:
+        """A bounded wait. A wavefront that runs out of polls goes on (the kernel always exits) but says so: it
+        stores a non-zero code into the file-scope word HANDOVER_REPORT, which the launcher's `<name>_status`
+        call turns into an error, because what such a wavefront goes on to read or overwrite is not what the
+        program meant."""
         writers, readers = self.plan.handed[array]
         need = f"(__round_{array} + 1) * {writers}" if what == "full" else f"__round_{array} * {readers}"
-        self.emit(f"for (int __spin = 0; __spin < {self.HANDOVER_SPINS} && __hip_atomic_load(&__{what}_{array}, "
+        code = 1 + 2 * list(self.plan.handed).index(array) + (1 if what == "full" else 0)
+        self.uses_handover_report = True
+        self.open()
+        self.emit("int __spin = 0;")
+        self.emit(f"for (; __spin < {self.HANDOVER_SPINS} && __hip_atomic_load(&__{what}_{array}, "
                   f"__ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>({need}); ++__spin) "
                   "__builtin_amdgcn_s_sleep(1);")
+        self.emit(f"if (__spin == {self.HANDOVER_SPINS} && (threadIdx.x & 63) == 0) __hip_atomic_store(&{HANDOVER_REPORT}, "
+                  f"{code}u | (static_cast<unsigned int>(__round_{array}) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
+        self.close()
         self.emit('__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");')
 
     def signal(self, array: str, what: str) -> None:
@@ -1004,16 +1028,18 @@ class BlockEmitter:
         self.block(fn.body)
         self.indent -= 1
         self.emit("}")
-        return "\n".join(self.out) + "\n"
+        text = "\n".join(self.out) + "\n"
+        # the word the hand-over waits report into is defined once per file, whichever function comes first
+        return (HANDOVER_REPORT_DEFINITION + text) if getattr(self, "uses_handover_report", False) else text
 
 
-def generate_blocks(name: str, auto_sync: bool = True, annotate: bool = False) -> str:
+def generate_blocks(name: str, auto_sync: bool = True, annotate: bool = False, handover_spins: Optional[int] = None) -> str:
     """HIP text of kernel or device function `name` in the structured form described above. annotate=True puts a
     comment in front of every barrier that names the statement's source line and the arrays the barrier is for
     (the reference keeps such a record per barrier as well, SyncReason, prism/sync_analysis.py:40-73)."""
     if name not in _REGISTRY:
         raise HipgenError(f"no kernel named {name!r} has been defined with @prism")
-    return BlockEmitter(_REGISTRY[name], auto_sync, annotate).emit_function()
+    return BlockEmitter(_REGISTRY[name], auto_sync, annotate, handover_spins).emit_function()
 
 
 def explain_barriers(name: str) -> List[str]:

@@ -32,7 +32,7 @@ def test_waits_and_signals_of_the_producer_consumer_gemm():
     def events(start, stop):
         out = []
         for ln in got[start:stop]:
-            if ln.startswith("for (int __spin"):
+            if ln.startswith("for (; __spin"):
                 word = ln.split("__hip_atomic_load(&__")[1].split(",")[0]
                 need = ln.split("static_cast<unsigned int>(")[1].split("); ++__spin")[0]
                 out.append(("wait", word, need))
@@ -64,8 +64,14 @@ def test_waits_and_signals_of_the_producer_consumer_gemm():
     assert got[first_signal + 1] == "__round_p_first += 1;"
     assert ("__builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&P_rows[(((((16 * part) + row) * K) "
             "+ k0) + k8)]), (__attribute__((address_space(3))) void*)(&p_first_fill[(512 * part)]), 16, 0, 0);") in got
-    # every wait is bounded
-    assert all("__spin < 65536 &&" in ln for ln in got if ln.startswith("for (int __spin"))
+    # every wait is bounded, and one that runs out of polls reports it (array and round) into the file-scope word
+    waits = [n for n, ln in enumerate(got) if ln.startswith("for (; __spin")]
+    assert len(waits) == 8 and all("__spin < 65536 &&" in got[n] for n in waits)
+    assert all(got[n - 1] == "int __spin = 0;" and got[n + 1].startswith("if (__spin == 65536 && (threadIdx.x & 63) == 0) "
+               "__hip_atomic_store(&__prism_handover_report, ") for n in waits)
+    n = waits[0]   # first wait of the producer: array 0 (p_first), waiting for "empty" -> code 1
+    assert "1u | (static_cast<unsigned int>(__round_p_first) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);" in got[n + 1]
+    assert got[0] == "#ifndef PRISM_HANDOVER_REPORT" and "__device__ unsigned int __prism_handover_report = 0;" in got[:6]
 
 
 @requires(grid[1], block[1], thread[128])
@@ -140,15 +146,15 @@ def test_hand_over_through_device_functions():
     mults = [n for n, ln in enumerate(got) if ln.startswith("multiply_slot(")]
     assert len(fills) == 2 and len(mults) == 2
     for name, n in zip(("first", "second"), fills):   # wait until the eight readers are done, fill, count in
-        assert got[n - 2].startswith(f"for (int __spin = 0; __spin < 65536 && __hip_atomic_load(&__empty_{name},")
-        assert f"__round_{name} * 8" in got[n - 2]
+        assert got[n - 4].startswith(f"for (; __spin < 65536 && __hip_atomic_load(&__empty_{name},")
+        assert f"__round_{name} * 8" in got[n - 4]
         assert f"__hip_atomic_fetch_add(&__full_{name}, 1u" in got[n + 3] and got[n + 4] == f"__round_{name} += 1;"
     for name, n in zip(("first", "second"), mults):   # wait until the four writers are done, multiply, give back
-        assert f"__hip_atomic_load(&__full_{name}," in got[n - 2] and f"(__round_{name} + 1) * 4" in got[n - 2]
+        assert f"__hip_atomic_load(&__full_{name}," in got[n - 4] and f"(__round_{name} + 1) * 4" in got[n - 4]
         assert f"__hip_atomic_fetch_add(&__empty_{name}, 1u" in got[n + 3]
     loop = got.index("for (int k0 = 0; k0 < K; k0 += 128) {")
     assert got.count("__syncthreads();") == 2 and all(n < loop for n, ln in enumerate(got) if ln == "__syncthreads();")
-    assert "__launch_bounds__(768)" in got[0]
+    assert "__launch_bounds__(768)" in got[6]   # behind the six lines that define the report word
     # a thread group may be a whole number of wavefronts (the callee's group of 256 producer threads)
     assert "int __thread_id_1 = __thread_id_0 % 256;" in lines(generate("fill_slot"))
 
@@ -174,6 +180,52 @@ def test_producer_consumer_gemm_against_the_oracle(built, oracle, shape):
     assert np.all(out[:64] == 777.0) and np.all(out[64 + M * N:] == 777.0)
     ref = oracle.gemm_bf16_f64(p16, q16)
     assert np.max(np.abs(out[64:64 + M * N].reshape(M, N) - ref)) <= 1e-3 * np.abs(ref).max()
+
+
+def test_the_launcher_text_has_a_status_call_and_the_poll_bound_is_an_argument():
+    text = hipgen.generate_launcher("handed_over_gemm", block_size=320)
+    assert 'extern "C" int handed_over_gemm_status(void* stream)' in text
+    assert text.count("__device__ unsigned int __prism_handover_report = 0;") == 1
+    assert "hipMemcpyFromSymbol(&word, HIP_SYMBOL(__prism_handover_report)" in text
+    # the full-size kernel's waits sit in the kernel, its device functions come first in the file: one definition
+    big = hipgen.generate_launcher("handed_over_gemm_big", block_size=768)
+    assert big.count("__device__ unsigned int __prism_handover_report = 0;") == 1 and "handed_over_gemm_big_status" in big
+    # a kernel without hand-over has neither the word nor the call
+    plain = hipgen.generate_launcher("tiled_sgemm", block_size=1024, template=[32])
+    assert "__prism_handover_report" not in plain and "_status" not in plain
+    none = hipgen.generate_launcher("handed_over_gemm", block_size=320, handover_spins=0)
+    assert "for (; __spin < 0 &&" in none and "if (__spin == 0 && (threadIdx.x & 63) == 0)" in none
+    with pytest.raises(HipgenError):
+        hipgen.generate_launcher("handed_over_gemm", block_size=320, handover_spins=-1)
+
+
+@pytest.mark.gpu
+def test_a_wait_that_gives_up_is_reported_and_the_kernel_still_exits(built, tmp_path_factory):
+    """Driven from the host: a build whose waits give up before their first poll (handover_spins = 0). Every
+    wavefront runs through all its rounds without waiting, the kernel exits normally, its result is not
+    trusted, and the status call reports the give-up once and clears it. The ordinary build reports nothing."""
+    import torch
+    impatient = hipgen.build("handed_over_gemm", out_dir=str(tmp_path_factory.mktemp("hipgen_handover_spins0")),
+                             block_size=320, handover_spins=0)
+    M, N, K = 128, 128, 256
+    P = torch.zeros((M, K), dtype=torch.bfloat16, device="cuda:0")
+    Q = torch.zeros((N, K), dtype=torch.bfloat16, device="cuda:0")
+    buf = torch.full((M * N + 128,), 777.0, dtype=torch.float32, device="cuda:0")
+    D = buf[64:64 + M * N]
+    torch.cuda.synchronize()
+    for lib in (impatient, built):
+        lib.handed_over_gemm_launch.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int] * 3 + [ctypes.c_uint, ctypes.c_void_p]
+        lib.handed_over_gemm_status.argtypes = [ctypes.c_void_p]
+    print("handed_over_gemm with handover_spins=0", flush=True)
+    assert impatient.handed_over_gemm_launch(P.data_ptr(), Q.data_ptr(), D.data_ptr(), N, K, N // 64, (M // 64) * (N // 64), None) == 0
+    rc = impatient.handed_over_gemm_status(None)
+    assert rc & 0x40000000 and 1 <= (rc & 0xff) <= 8, hex(rc)   # four arrays, "empty" and "full" waits
+    assert impatient.handed_over_gemm_status(None) == 0             # reported once, then cleared
+    out = buf.cpu().numpy()
+    assert np.all(out[:64] == 777.0) and np.all(out[64 + M * N:] == 777.0)   # stores stayed inside the tile grid
+    assert built.handed_over_gemm_launch(P.data_ptr(), Q.data_ptr(), D.data_ptr(), N, K, N // 64, (M // 64) * (N // 64), None) == 0
+    assert built.handed_over_gemm_status(None) == 0
+    assert bool((D == 0).all())
 
 
 @requires(grid[1], block[1], thread[128])
