@@ -265,22 +265,42 @@ int prism_sgemm(int variant, int M, int N, int K, float alpha, const float* A,
                 const float* B, float beta, float* C, void* stream);
 
 /*
- * prism_sgemm with a workspace, for shapes that have too few tiles for the GPU
- * and a long K (skinny products such as 128 x 4096 x 4096): kernel 5 then cuts K
- * across workgroups, every part writes its M x N partial product into the
- * workspace, and a second kernel adds the parts in a fixed order (the same bits
- * on every run) and applies alpha and beta. prism_sgemm_workspace_bytes says
- * how much a shape can use (0: it would not be cut); with a smaller or NULL
- * workspace (16-byte aligned otherwise), or any other kernel number, the call is
- * prism_sgemm. Calls that share a workspace must be ordered on one stream.
- * No counterpart in the reference, whose launchers (evals/4090_sgemm/runner.cu:
- * 191-243) take no workspace; a harness that wants the split holds one buffer
- * and passes it here.
+ * prism_sgemm with a workspace. Kernel 5 gives every workgroup one whole output
+ * tile, as the reference's launcher does (evals/4090_sgemm/runner.cu:191-243),
+ * so a problem whose tiles are not a whole number of rounds of the GPU's compute
+ * units leaves most of them idle in the last round, and a skinny problem (few
+ * tiles, long K: 128 x 4096 x 4096) leaves them idle throughout. With a
+ * workspace the K ranges of the tiles of the last, partial round (of all tiles,
+ * when there are fewer than compute units or the problem is skinny) are shared
+ * evenly between all compute units: a workgroup that gets part of a tile's K
+ * range stores its partial product into the workspace, and a second kernel adds
+ * a tile's partial products in the order of k (the same bits on every run on
+ * one device) and applies alpha and beta. No workgroup waits for another.
+ * prism_sgemm_workspace_bytes says how much a shape can use on the CURRENT
+ * device (0: nothing would be shared); query it with the device current that
+ * the call will run on. With a smaller or NULL workspace, one that is not
+ * 16-byte aligned, operands that are not 16-byte aligned, N or K not a multiple
+ * of 4, or any other kernel number, the call is prism_sgemm. Arguments are
+ * checked as in prism_sgemm. Calls that share a workspace must be ordered on one
+ * stream. No counterpart in the reference, whose launchers take no workspace; a
+ * harness that wants the sharing holds one buffer and passes it here.
  */
 size_t prism_sgemm_workspace_bytes(int M, int N, int K);
 int prism_sgemm_ws(int variant, int M, int N, int K, float alpha, const float* A,
                    const float* B, float beta, float* C, void* workspace,
                    size_t workspace_bytes, void* stream);
+
+/*
+ * What prism_sgemm_ws does for this shape on the current device, given 16-byte
+ * aligned operands and workspace_bytes of workspace: *workgroups = the number
+ * of workgroups that share K ranges, *shared_tiles = the tiles they share
+ * (256 x 256 ones, or 64 x 256 for skinny shapes); both 0 when the call would
+ * be prism_sgemm. Either pointer may be NULL. Lets a harness or test assert
+ * that the workspace path is the one it measures. No counterpart in the
+ * reference.
+ */
+int prism_sgemm_ws_plan(int M, int N, int K, size_t workspace_bytes, int* workgroups,
+                        int* shared_tiles);
 
 /*
  * The reference dispatcher's own shape: default stream, kernel numbers 1..5.

@@ -23,6 +23,7 @@ from .ops import (  # noqa: F401
     scan_workspace_init,
     segmented_scan,
     sgemm,
+    sgemm_workspace_plan,
     sgemm_workspace_size,
     tile_coords,
     wave_regroup,

@@ -38,6 +38,7 @@ SIGNATURES = {
     "prism_sgemm_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int]),
     "prism_sgemm_ws": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_void_p,
                                  C.c_float, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "prism_sgemm_ws_plan": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_size_t, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "prism_run_my_kernel": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_void_p,
                                       C.c_void_p, C.c_float, C.c_void_p]),
     "prism_gemm_bf16": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),

@@ -142,6 +142,10 @@ int prism_sgemm_ws(int variant, int M, int N, int K, float alpha, const float* A
                            static_cast<hipStream_t>(stream));
 }
 
+int prism_sgemm_ws_plan(int M, int N, int K, size_t workspace_bytes, int* workgroups, int* shared_tiles) {
+    return sgemm_ws_plan(M, N, K, workspace_bytes, workgroups, shared_tiles);
+}
+
 int prism_run_my_kernel(int my_kernel_num, int M, int N, int K, float alpha, float* A, float* B,
                         float beta, float* C) {
     if (my_kernel_num < 1 || my_kernel_num > 5)

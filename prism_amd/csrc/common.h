@@ -74,7 +74,12 @@ int launch_scan_static(const uint32_t* in, uint32_t* out, size_t n, hipStream_t 
 int launch_wave_regroup(const int32_t* in, int32_t* out, size_t n, int items_per_lane, int direction, hipStream_t s);
 int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, const float* B,
                  float beta, float* C, hipStream_t s);
+// 0 if the arguments are ones launch_sgemm accepts, else the error (and the error string is set).
+int check_sgemm_arguments(int variant, int M, int N, int K, const float* A, const float* B, const float* C);
 size_t sgemm_workspace_bytes(int M, int N, int K);
+// What launch_sgemm_ws does for this shape with 16 B-aligned operands and ws_bytes of workspace: the number of
+// workgroups that share K ranges and of the tiles they share (both 0: the call is launch_sgemm).
+int sgemm_ws_plan(int M, int N, int K, size_t ws_bytes, int* groups, int* sk_tiles);
 int launch_sgemm_ws(int variant, int M, int N, int K, float alpha, const float* A, const float* B, float beta,
                     float* C, void* ws, size_t ws_bytes, hipStream_t s);
 int launch_gemm_bf16(int M, int N, int K, const uint16_t* A, const uint16_t* B, float* D_f32,

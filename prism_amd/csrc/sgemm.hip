@@ -453,26 +453,24 @@ __attribute__((amdgpu_waves_per_eu(4))) void sgemm_wave_tile_kernel(
 // into columns >= N, which are never stored. The last K % 4 values of k are added in front of the
 // write-back from ordinary loads, and C is written element by element where a chunk straddles N.
 //
-// SPLIT (whole tiles only): the K range is cut into `first_big` equal parts and the grid holds one workgroup
-// per tile and part; part s multiplies k in [s K / parts, (s + 1) K / parts) and writes its M x N partial
-// product (alpha and beta are not applied) into slice s of the buffer passed as C, for sgemm_add_parts_kernel.
-template <int BM, int BN, int BK, int WM, int WN, bool EDGE, bool RAGGED = false, bool SPLIT = false>
+// STREAMK: the grid is gridDim.x workgroups that share the (tile, K tile) iterations of `sk_tiles` tiles evenly,
+// whatever their number: tile number first_big + t for t < sk_tiles, each K_all / BK (rounded up) iterations long,
+// laid end to end; workgroup w takes iterations [w I / G, (w + 1) I / G) of the I in all. A workgroup's share is
+// a run of segments, each a range of K tiles of one output tile. A segment that covers its tile's whole K range
+// is finished here (alpha, beta, C); any other is stored as a raw BM x BN partial product into a slot of the
+// workspace `ws` (slot 2 w for the segment a workgroup starts with, 2 w + 1 for the one it ends with), and
+// sgemm_stream_k_fixup_kernel adds a tile's partial products in the order of k and finishes the tile. No
+// workgroup waits for another one. (The reference's launcher gives every block one whole tile,
+// evals/4090_sgemm/runner.cu:191-243; this is the same tile loop entered and left in the middle of K.)
+template <int BM, int BN, int BK, int WM, int WN, bool EDGE, bool RAGGED = false, bool STREAMK = false>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile_dma_kernel(
     int M, int N, int K_all, float alpha, const float* __restrict__ A, const float* __restrict__ B,
-    float beta, float* C, int tiles_m, int tiles_n, int first_big) {
+    float beta, float* C, int tiles_m, int tiles_n, int first_big, float* ws = nullptr, int sk_tiles = 0) {
     static_assert(EDGE || !RAGGED, "the ragged form is an edge form");
-    static_assert(!SPLIT || !EDGE, "the K split is written for whole tiles");
-    // lda: elements between A rows. K: the part of the k range the loop covers.
+    static_assert(!STREAMK || !RAGGED, "the shared-K form needs 16 B-aligned rows");
+    // lda: elements between A rows. K: the part of the k range the loops cover.
     const int lda = K_all;
-    const int K = RAGGED ? K_all - K_all % 4 : (SPLIT ? K_all / first_big : K_all);
-    unsigned tile_id = blockIdx.x;
-    if constexpr (SPLIT) {
-        const unsigned tiles = static_cast<unsigned>(tiles_m) * tiles_n, part = blockIdx.x / tiles;
-        tile_id = blockIdx.x % tiles;
-        A += static_cast<size_t>(part) * K;
-        B += static_cast<size_t>(part) * K * N;
-        C += static_cast<size_t>(part) * M * N;
-    }
+    const int K = RAGGED ? K_all - K_all % 4 : K_all;
     constexpr int WAVES_N = BN / WN;
     constexpr int WAVES = (BM / WM) * WAVES_N;
     constexpr int MI = WM / 32, NI = 4;
@@ -497,23 +495,6 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
     __shared__ __attribute__((aligned(1024))) float Bs0[BK * BN];
     __shared__ __attribute__((aligned(1024))) float Bs1[BK * BN];
 
-    // first_big < 0: the grid covers the tiles_m x tiles_n grid of BM x BN tiles. Otherwise this launch
-    // finishes what a launch on 256 x 256 tiles left over: tiles_m x tiles_n is that launch's grid, first_big
-    // the first tile number it did not take, and every leftover tile is cut into 256 / BM row slices.
-    int row0, col0;
-    if (SPLIT || first_big < 0) {
-        int tm, tn;
-        xcd_tile_coords(static_cast<int>(tile_id), tiles_m, tiles_n, tm, tn);
-        row0 = tm * BM;
-        col0 = tn * BN;
-    } else {
-        constexpr int SUB = 256 / BM;
-        int tm, tn;
-        xcd_tile_coords(first_big + blockIdx.x / SUB, tiles_m, tiles_n, tm, tn);
-        row0 = tm * 256 + static_cast<int>(blockIdx.x % SUB) * BM;
-        col0 = tn * 256;
-    }
-
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // wave-uniform, lives in an SGPR
@@ -521,12 +502,6 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
     const int l32 = lane & 31, lhi = lane >> 5;
 
     f32x16 acc[MI][NI];
-#pragma unroll
-    for (int i = 0; i < MI; ++i)
-#pragma unroll
-        for (int j = 0; j < NI; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
     // Load side. A: in pass u this wave fills rows [(u * WAVES + wave) * ROWS_PER_LOAD, + ROWS_PER_LOAD);
     // lane l owns row l / KP of those and slot l % KP. The swizzle term is the same in every pass.
@@ -538,46 +513,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
     const int ld_chunk = (lane % KP) ^ ((ld_row >> SWZ) & (KP - 1));
     const uint32_t a_lane = (static_cast<uint32_t>(lane / KP) * static_cast<uint32_t>(lda) + ld_chunk * 4) * 4u;  // bytes
     const uint32_t b_lane = static_cast<uint32_t>(lane) * 16u;
-    const char* a_wave = reinterpret_cast<const char*>(A + static_cast<size_t>(row0 + wave * ROWS_PER_LOAD) * lda);
-    const char* b_wave = reinterpret_cast<const char*>(B + static_cast<size_t>(wave) * N + col0);
     const size_t a_pass = static_cast<size_t>(ROWS_PER_PASS) * lda * 4;
     const size_t b_pass = static_cast<size_t>(WAVES) * N * 4;
-
-    // EDGE: M, N, K need not be whole tiles (N and K multiples of 4, so that rows stay 16 B aligned and
-    // a 16 B chunk is whole or absent). The loads go through buffer descriptors whose extents end with
-    // the matrices: A rows >= M and B rows >= K lie beyond them and arrive as zeros. What lies past
-    // the end of a row is the next row, so there the lane offset is replaced by one beyond any extent:
-    // B columns >= N (fixed per lane) and, in the partial K tile, A chunks with k >= K.
-    const int a_first = row0 + wave * ROWS_PER_LOAD;              // this wave's first A row
-    const long long a_left = static_cast<long long>(M - a_first) * lda * 4;
-    const long long b_left = (static_cast<long long>(K - wave) * N - col0) * 4;
-    const i32x4 a_rsrc = buffer_descriptor(EDGE && a_left > 0 ? static_cast<const void*>(a_wave) : static_cast<const void*>(A),
-                                           EDGE ? clamped_extent(a_left) : 0u);
-    const i32x4 b_rsrc = buffer_descriptor(EDGE && b_left > 0 ? static_cast<const void*>(b_wave) : static_cast<const void*>(B),
-                                           EDGE ? clamped_extent(b_left) : 0u);
-    const int k_full = K - K % BK;
-    const uint32_t a_tail = (k_full + ld_chunk * 4 < K) ? a_lane : kBeyondExtent;
-    const uint32_t b_edge = (col0 + 4 * lane < N) ? b_lane : kBeyondExtent;
-    // Load number m (0 .. A_PER + B_PER - 1) of the tile that starts at k0.
-    auto issue_load = [&](float* as, float* bs, int k0, int m) {
-        if constexpr (EDGE) {
-            if (m < A_PER)
-                direct_load16_buffer(a_rsrc, k0 < k_full ? a_lane : a_tail,
-                                     static_cast<uint32_t>(k0) * 4u + m * static_cast<uint32_t>(a_pass),
-                                     as + (m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK);
-            else
-                direct_load16_buffer(b_rsrc, b_edge,
-                                     (static_cast<uint32_t>(k0) + (m - A_PER) * WAVES) * static_cast<uint32_t>(N) * 4u,
-                                     bs + ((m - A_PER) * WAVES + wave) * BN);
-        } else {
-            if (m < A_PER)
-                direct_load16(a_wave + static_cast<size_t>(k0) * 4 + m * a_pass, a_lane,
-                              as + (m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK);
-            else
-                direct_load16(b_wave + static_cast<size_t>(k0) * N * 4 + (m - A_PER) * b_pass, b_lane,
-                              bs + ((m - A_PER) * WAVES + wave) * BN);
-        }
-    };
     constexpr int LOADS = A_PER + B_PER;
 
     // Operand side.
@@ -608,166 +545,321 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void sgemm_wave_tile
                 }
     };
     auto nothing = [](int) {};
-
-    // One phase = everything between two barriers. It is entered right after the
-    // barrier that says "tile t is complete in (as, bs), nobody reads (as_n, bs_n)
-    // any more", while operand slot 1 still holds the last group of tile t-1:
-    //   read group 0 of tile t           -> slot 0
-    //   MFMAs of the last group of t-1   <- slot 1, with the direct loads of tile t+1 issued among them
-    //   groups 0 .. KS-2 of tile t, each preceded by the reads of the next group
-    //   wait for this wave's direct loads, barrier
-    auto phase = [&](float* as, float* bs, float* as_n, float* bs_n, int k_next, auto prefetch) {
-        read_frags(as, bs, 0, 0);
-        mfma_all(1, [&](int m) {
-            if constexpr (prefetch) {
-                if (m % LOAD_GAP == 0 && m / LOAD_GAP < LOADS) {
-                    issue_load(as_n, bs_n, k_next, m / LOAD_GAP);
-                    // The scheduler would otherwise bunch the loads together, and a burst of
-                    // them holds the wave (and with it the next MFMA) at the memory pipeline.
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            }
-        });
-#pragma unroll
-        for (int s = 0; s + 1 < KS; ++s) {
-            read_frags(as, bs, s + 1, (s + 1) & 1);
-            mfma_all(s & 1, nothing);
-        }
-        constexpr int G = 4 * MI * NI;  // MFMAs per group
-        constexpr int PLACED = prefetch ? (LOADS - 1) * LOAD_GAP + 1 : 0;  // MFMAs above the last sched_barrier
-        if constexpr (!prefetch) __builtin_amdgcn_sched_group_barrier(0x100, MI + 4, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, G - PLACED, 0);
-#pragma unroll
-        for (int s = 0; s + 1 < KS; ++s) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, MI + 4, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, G - 4, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);  // keep the MFMAs above the barrier: the direct loads get a whole tile to land
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));  // the direct loads are invisible to the compiler's wait counts
-        __syncthreads();
-    };
     using yes = std::integral_constant<bool, true>;
     using no = std::integral_constant<bool, false>;
 
-    // Slot 1 starts as zeros, so the "previous tile" MFMAs of the first phase add nothing.
+    // The product of A[row0 .., k_begin .. k_end) and B[k_begin .. k_end, col0 ..) for one BM x BN tile (k_begin a
+    // multiple of BK). raw == false: written to C as alpha * product + beta * C. raw == true (STREAMK only): the
+    // bare product, stored as a BM x BN array at `part`.
+    auto run_tile = [&](const int row0, const int col0, const int k_begin, const int k_end, const bool raw, float* part) {
 #pragma unroll
-    for (int i = 0; i < MI; ++i) fa[1][i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj) fb[1][jj] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            for (int j = 0; j < NI; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    auto load_tile0 = [&](float* as, float* bs) {
-#pragma unroll
-        for (int m = 0; m < LOADS; ++m) issue_load(as, bs, 0, m);
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));
-        __syncthreads();
-    };
+        const char* a_wave = reinterpret_cast<const char*>(A + static_cast<size_t>(row0 + wave * ROWS_PER_LOAD) * lda);
+        const char* b_wave = reinterpret_cast<const char*>(B + static_cast<size_t>(wave) * N + col0);
 
-    // The launcher guarantees K > 0 and, unless EDGE, K % BK == 0. Tiles alternate between the
-    // two stages such that the last tile always sits in stage 1.
-    const int k_tiles = (K + BK - 1) / BK;
-    int t = 0;
-    if (k_tiles & 1) {
-        load_tile0(As1, Bs1);
-        if (k_tiles > 1) {
-            phase(As1, Bs1, As0, Bs0, BK, yes{});
-            t = 1;
-        }
-    } else {
-        load_tile0(As0, Bs0);
-    }
-    for (; t + 2 < k_tiles; t += 2) {
-        phase(As0, Bs0, As1, Bs1, (t + 1) * BK, yes{});
-        phase(As1, Bs1, As0, Bs0, (t + 2) * BK, yes{});
-    }
-    if (k_tiles > 1) phase(As0, Bs0, As1, Bs1, (t + 1) * BK, yes{});
-    phase(As1, Bs1, As0, Bs0, 0, no{});
-    mfma_all(1, nothing);  // last group of the last tile
-
-    // Epilogue: a lane holds columns 4 l32 .. 4 l32 + 3 of 16 rows per 32-row block.
-    const int c_row = row0 + wave_m * WM + 4 * lhi, c_col = col0 + wave_n * WN + 4 * l32;
-    float* c_lane = C + static_cast<size_t>(c_row) * N + c_col;
-    auto write_back = [&](auto read_c) {
-#pragma unroll
-        for (int i = 0; i < MI; ++i) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int r_in = i * 32 + 8 * (v / 4) + (v % 4);
-                if (EDGE && (c_row + r_in >= M || c_col >= N)) continue;
-                f32x4* c = reinterpret_cast<f32x4*>(c_lane + static_cast<size_t>(r_in) * N);
-                f32x4 r;
-                if constexpr (read_c) {
-                    const f32x4 old = *c;
-#pragma unroll
-                    for (int j = 0; j < NI; ++j) r[j] = __builtin_fmaf(alpha, acc[i][j][v], beta * old[j]);
-                } else {
-#pragma unroll
-                    for (int j = 0; j < NI; ++j) r[j] = alpha * acc[i][j][v];
-                }
-                *c = r;
+        // EDGE: M, N, K need not be whole tiles (N and K multiples of 4, so that rows stay 16 B aligned and
+        // a 16 B chunk is whole or absent). The loads go through buffer descriptors whose extents end with
+        // the matrices: A rows >= M and B rows >= K lie beyond them and arrive as zeros. What lies past
+        // the end of a row is the next row, so there the lane offset is replaced by one beyond any extent:
+        // B columns >= N (fixed per lane) and, in the partial K tile, A chunks with k >= K.
+        const int a_first = row0 + wave * ROWS_PER_LOAD;              // this wave's first A row
+        const long long a_left = static_cast<long long>(M - a_first) * lda * 4;
+        const long long b_left = (static_cast<long long>(k_end - wave) * N - col0) * 4;
+        const i32x4 a_rsrc = buffer_descriptor(EDGE && a_left > 0 ? static_cast<const void*>(a_wave) : static_cast<const void*>(A),
+                                               EDGE ? clamped_extent(a_left) : 0u);
+        const i32x4 b_rsrc = buffer_descriptor(EDGE && b_left > 0 ? static_cast<const void*>(b_wave) : static_cast<const void*>(B),
+                                               EDGE ? clamped_extent(b_left) : 0u);
+        const int k_full = k_end - k_end % BK;
+        const uint32_t a_tail = (k_full + ld_chunk * 4 < k_end) ? a_lane : kBeyondExtent;
+        const uint32_t b_edge = (col0 + 4 * lane < N) ? b_lane : kBeyondExtent;
+        // Load number m (0 .. A_PER + B_PER - 1) of the tile that starts at k0.
+        auto issue_load = [&](float* as, float* bs, int k0, int m) {
+            if constexpr (EDGE) {
+                if (m < A_PER)
+                    direct_load16_buffer(a_rsrc, k0 < k_full ? a_lane : a_tail,
+                                         static_cast<uint32_t>(k0) * 4u + m * static_cast<uint32_t>(a_pass),
+                                         as + (m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK);
+                else
+                    direct_load16_buffer(b_rsrc, b_edge,
+                                         (static_cast<uint32_t>(k0) + (m - A_PER) * WAVES) * static_cast<uint32_t>(N) * 4u,
+                                         bs + ((m - A_PER) * WAVES + wave) * BN);
+            } else {
+                if (m < A_PER)
+                    direct_load16(a_wave + static_cast<size_t>(k0) * 4 + m * a_pass, a_lane,
+                                  as + (m * ROWS_PER_PASS + wave * ROWS_PER_LOAD) * BK);
+                else
+                    direct_load16(b_wave + static_cast<size_t>(k0) * N * 4 + (m - A_PER) * b_pass, b_lane,
+                                  bs + ((m - A_PER) * WAVES + wave) * BN);
             }
-            __builtin_amdgcn_sched_barrier(0);  // at most one 32-row block of C reads in flight (64 registers)
+        };
+
+        // One phase = everything between two barriers. It is entered right after the
+        // barrier that says "tile t is complete in (as, bs), nobody reads (as_n, bs_n)
+        // any more", while operand slot 1 still holds the last group of tile t-1:
+        //   read group 0 of tile t           -> slot 0
+        //   MFMAs of the last group of t-1   <- slot 1, with the direct loads of tile t+1 issued among them
+        //   groups 0 .. KS-2 of tile t, each preceded by the reads of the next group
+        //   wait for this wave's direct loads, barrier
+        auto phase = [&](float* as, float* bs, float* as_n, float* bs_n, int k_next, auto prefetch) {
+            read_frags(as, bs, 0, 0);
+            mfma_all(1, [&](int m) {
+                if constexpr (prefetch) {
+                    if (m % LOAD_GAP == 0 && m / LOAD_GAP < LOADS) {
+                        issue_load(as_n, bs_n, k_next, m / LOAD_GAP);
+                        // The scheduler would otherwise bunch the loads together, and a burst of
+                        // them holds the wave (and with it the next MFMA) at the memory pipeline.
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            });
+#pragma unroll
+            for (int s = 0; s + 1 < KS; ++s) {
+                read_frags(as, bs, s + 1, (s + 1) & 1);
+                mfma_all(s & 1, nothing);
+            }
+            constexpr int G = 4 * MI * NI;  // MFMAs per group
+            constexpr int PLACED = prefetch ? (LOADS - 1) * LOAD_GAP + 1 : 0;  // MFMAs above the last sched_barrier
+            if constexpr (!prefetch) __builtin_amdgcn_sched_group_barrier(0x100, MI + 4, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, G - PLACED, 0);
+#pragma unroll
+            for (int s = 0; s + 1 < KS; ++s) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, MI + 4, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, G - 4, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);  // keep the MFMAs above the barrier: the direct loads get a whole tile to land
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));  // the direct loads are invisible to the compiler's wait counts
+            __syncthreads();
+        };
+
+        // Slot 1 starts as zeros, so the "previous tile" MFMAs of the first phase add nothing.
+#pragma unroll
+        for (int i = 0; i < MI; ++i) fa[1][i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) fb[1][jj] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+        auto load_tile0 = [&](float* as, float* bs) {
+#pragma unroll
+            for (int m = 0; m < LOADS; ++m) issue_load(as, bs, k_begin, m);
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));
+            __syncthreads();
+        };
+
+        // The launcher guarantees k_end > k_begin and, unless EDGE, whole K tiles. Tiles alternate between the
+        // two stages such that the last tile always sits in stage 1.
+        const int k_tiles = (k_end - k_begin + BK - 1) / BK;
+        int t = 0;
+        if (k_tiles & 1) {
+            load_tile0(As1, Bs1);
+            if (k_tiles > 1) {
+                phase(As1, Bs1, As0, Bs0, k_begin + BK, yes{});
+                t = 1;
+            }
+        } else {
+            load_tile0(As0, Bs0);
         }
-    };
-    if constexpr (!RAGGED) {
-        if (beta == 0.0f) write_back(no{}); else write_back(yes{});
-    } else {
-        // The k values the loop left out (K_all % 4 of them): a lane adds them to its 16 rows x 4 columns
-        // per 32-row block from ordinary loads.
-        const int k_tail = K_all - K;
-        if (k_tail > 0 && c_col < N) {
-            float bt[3][NI];
+        for (; t + 2 < k_tiles; t += 2) {
+            phase(As0, Bs0, As1, Bs1, k_begin + (t + 1) * BK, yes{});
+            phase(As1, Bs1, As0, Bs0, k_begin + (t + 2) * BK, yes{});
+        }
+        if (k_tiles > 1) phase(As0, Bs0, As1, Bs1, k_begin + (t + 1) * BK, yes{});
+        phase(As1, Bs1, As0, Bs0, 0, no{});
+        mfma_all(1, nothing);  // last group of the last tile
+
+        // Epilogue: a lane holds columns 4 l32 .. 4 l32 + 3 of 16 rows per 32-row block.
+        const int c_row = row0 + wave_m * WM + 4 * lhi, c_col = col0 + wave_n * WN + 4 * l32;
+        if constexpr (STREAMK) {
+            if (raw) {
+                // The bare product of this segment, every element of the tile (edge tiles hold zeros outside C).
+                float* p_lane = part + static_cast<size_t>(wave_m * WM + 4 * lhi) * BN + wave_n * WN + 4 * l32;
 #pragma unroll
-            for (int t = 0; t < 3; ++t)
+                for (int i = 0; i < MI; ++i) {
 #pragma unroll
-                for (int j = 0; j < NI; ++j)
-                    bt[t][j] = (t < k_tail && c_col + j < N) ? B[static_cast<size_t>(K + t) * N + c_col + j] : 0.0f;
+                    for (int v = 0; v < 16; ++v) {
+                        const int r_in = i * 32 + 8 * (v / 4) + (v % 4);
+                        f32x4 r;
 #pragma unroll
-            for (int i = 0; i < MI; ++i)
+                        for (int j = 0; j < NI; ++j) r[j] = acc[i][j][v];
+                        *reinterpret_cast<f32x4*>(p_lane + static_cast<size_t>(r_in) * BN) = r;
+                    }
+                }
+                return;
+            }
+        }
+        float* c_lane = C + static_cast<size_t>(c_row) * N + c_col;
+        auto write_back = [&](auto read_c) {
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    const int row = c_row + i * 32 + 8 * (v / 4) + (v % 4);
-                    if (row >= M) continue;
-                    const float* a_row = A + static_cast<size_t>(row) * lda + K;
-#pragma unroll
-                    for (int t = 0; t < 3; ++t)
-                        if (t < k_tail) {
-                            const float a = a_row[t];
-#pragma unroll
-                            for (int j = 0; j < NI; ++j) acc[i][j][v] = __builtin_fmaf(a, bt[t][j], acc[i][j][v]);
-                        }
-                }
-        }
-        // C rows are 4 B aligned only: whole chunks as 16 B accesses at that alignment, the chunk that
-        // straddles N element by element.
-        typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
-        const bool read_c = beta != 0.0f;
-#pragma unroll
-        for (int i = 0; i < MI; ++i) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int r_in = i * 32 + 8 * (v / 4) + (v % 4);
-                if (c_row + r_in >= M || c_col >= N) continue;
-                float* c = c_lane + static_cast<size_t>(r_in) * N;
-                if (c_col + NI <= N) {
-                    f32x4_a4* c4 = reinterpret_cast<f32x4_a4*>(c);
-                    f32x4 old = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-                    if (read_c) old = *c4;
+                    const int r_in = i * 32 + 8 * (v / 4) + (v % 4);
+                    if (EDGE && (c_row + r_in >= M || c_col >= N)) continue;
+                    f32x4* c = reinterpret_cast<f32x4*>(c_lane + static_cast<size_t>(r_in) * N);
                     f32x4 r;
+                    if constexpr (read_c) {
+                        const f32x4 old = *c;
 #pragma unroll
-                    for (int j = 0; j < NI; ++j)
-                        r[j] = read_c ? __builtin_fmaf(alpha, acc[i][j][v], beta * old[j]) : alpha * acc[i][j][v];
-                    *c4 = r;
-                } else {
+                        for (int j = 0; j < NI; ++j) r[j] = __builtin_fmaf(alpha, acc[i][j][v], beta * old[j]);
+                    } else {
 #pragma unroll
-                    for (int j = 0; j < NI; ++j)
-                        if (c_col + j < N)
-                            c[j] = read_c ? __builtin_fmaf(alpha, acc[i][j][v], beta * c[j]) : alpha * acc[i][j][v];
+                        for (int j = 0; j < NI; ++j) r[j] = alpha * acc[i][j][v];
+                    }
+                    *c = r;
                 }
+                __builtin_amdgcn_sched_barrier(0);  // at most one 32-row block of C reads in flight (64 registers)
             }
-            __builtin_amdgcn_sched_barrier(0);
+        };
+        if constexpr (!RAGGED) {
+            if (beta == 0.0f) write_back(no{}); else write_back(yes{});
+        } else {
+            // The k values the loop left out (K_all % 4 of them): a lane adds them to its 16 rows x 4 columns
+            // per 32-row block from ordinary loads.
+            const int k_tail = K_all - K;
+            if (k_tail > 0 && c_col < N) {
+                float bt[3][NI];
+#pragma unroll
+                for (int t = 0; t < 3; ++t)
+#pragma unroll
+                    for (int j = 0; j < NI; ++j)
+                        bt[t][j] = (t < k_tail && c_col + j < N) ? B[static_cast<size_t>(K + t) * N + c_col + j] : 0.0f;
+#pragma unroll
+                for (int i = 0; i < MI; ++i)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int row = c_row + i * 32 + 8 * (v / 4) + (v % 4);
+                        if (row >= M) continue;
+                        const float* a_row = A + static_cast<size_t>(row) * lda + K;
+#pragma unroll
+                        for (int t = 0; t < 3; ++t)
+                            if (t < k_tail) {
+                                const float a = a_row[t];
+#pragma unroll
+                                for (int j = 0; j < NI; ++j) acc[i][j][v] = __builtin_fmaf(a, bt[t][j], acc[i][j][v]);
+                            }
+                    }
+            }
+            // C rows are 4 B aligned only: whole chunks as 16 B accesses at that alignment, the chunk that
+            // straddles N element by element.
+            typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+            const bool read_c = beta != 0.0f;
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int r_in = i * 32 + 8 * (v / 4) + (v % 4);
+                    if (c_row + r_in >= M || c_col >= N) continue;
+                    float* c = c_lane + static_cast<size_t>(r_in) * N;
+                    if (c_col + NI <= N) {
+                        f32x4_a4* c4 = reinterpret_cast<f32x4_a4*>(c);
+                        f32x4 old = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                        if (read_c) old = *c4;
+                        f32x4 r;
+#pragma unroll
+                        for (int j = 0; j < NI; ++j)
+                            r[j] = read_c ? __builtin_fmaf(alpha, acc[i][j][v], beta * old[j]) : alpha * acc[i][j][v];
+                        *c4 = r;
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < NI; ++j)
+                            if (c_col + j < N)
+                                c[j] = read_c ? __builtin_fmaf(alpha, acc[i][j][v], beta * c[j]) : alpha * acc[i][j][v];
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+
+    if constexpr (!STREAMK) {
+        // first_big < 0: the grid covers the tiles_m x tiles_n grid of BM x BN tiles. Otherwise this launch
+        // finishes what a launch on 256 x 256 tiles left over: tiles_m x tiles_n is that launch's grid, first_big
+        // the first tile number it did not take, and every leftover tile is cut into 256 / BM row slices.
+        int row0, col0;
+        if (first_big < 0) {
+            int tm, tn;
+            xcd_tile_coords(static_cast<int>(blockIdx.x), tiles_m, tiles_n, tm, tn);
+            row0 = tm * BM;
+            col0 = tn * BN;
+        } else {
+            constexpr int SUB = 256 / BM;
+            int tm, tn;
+            xcd_tile_coords(first_big + blockIdx.x / SUB, tiles_m, tiles_n, tm, tn);
+            row0 = tm * 256 + static_cast<int>(blockIdx.x % SUB) * BM;
+            col0 = tn * 256;
+        }
+        run_tile(row0, col0, 0, K, false, nullptr);
+    } else {
+        // This workgroup's run of iterations, segment by segment. Iteration i is K tile i % kt of tile i / kt.
+        typedef unsigned long long u64;
+        const u64 kt = static_cast<u64>((K + BK - 1) / BK), total = static_cast<u64>(sk_tiles) * kt;
+        const u64 w = blockIdx.x, groups = gridDim.x;
+        u64 it = w * total / groups;
+        const u64 it_end = (w + 1) * total / groups;
+        const u64 first_tile = it / kt;
+        while (it < it_end) {
+            const u64 tile = it / kt, k0 = it - tile * kt;
+            const u64 k1 = (it_end - it < kt - k0) ? k0 + (it_end - it) : kt;
+            int tm, tn;
+            xcd_tile_coords(first_big + static_cast<int>(tile), tiles_m, tiles_n, tm, tn);
+            const bool raw = !(k0 == 0 && k1 == kt);
+            const int k_end = static_cast<int>(k1 * BK) < K ? static_cast<int>(k1 * BK) : K;
+            float* part = ws + (2 * w + (tile != first_tile ? 1u : 0u)) * static_cast<size_t>(BM * BN);
+            run_tile(tm * BM, tn * BN, static_cast<int>(k0 * BK), k_end, raw, part);
+            it += k1 - k0;
         }
     }
+}
+
+// Finishes the tiles whose K range sgemm_wave_tile_dma_kernel<..., STREAMK> shared between workgroups:
+// C = alpha * (the tile's partial products, added in the order of k: the same bits on every run) + beta * C. One
+// thread per 4 consecutive columns; grid = sk_tiles x (BM * BN / 1024) workgroups of 256. The arithmetic that
+// says which workgroup held which part of which tile is the kernel's own.
+template <int BM, int BN, int BK>
+__global__ __launch_bounds__(256) void sgemm_stream_k_fixup_kernel(int M, int N, int K, float alpha, float beta, float* C,
+                                                                   const float* __restrict__ ws, int tiles_m, int tiles_n,
+                                                                   int first_tile_number, int sk_tiles, unsigned groups) {
+    typedef unsigned long long u64;
+    constexpr unsigned PER_TILE = BM * BN / 1024;  // workgroups per tile
+    const unsigned tile = blockIdx.x / PER_TILE;
+    const unsigned q = (blockIdx.x % PER_TILE) * 256 + threadIdx.x;  // which 16 B packet of the tile
+    const int r = static_cast<int>(q / (BN / 4)), c = static_cast<int>(q % (BN / 4)) * 4;
+    const u64 kt = static_cast<u64>((K + BK - 1) / BK), total = static_cast<u64>(sk_tiles) * kt;
+    const u64 lo = tile * kt, hi = lo + kt;  // the tile's iterations
+    // first and last workgroup whose share [w total / groups, (w + 1) total / groups) meets [lo, hi)
+    u64 w0 = (lo * groups) / total, w1 = ((hi - 1) * groups) / total;
+    while (w0 > 0 && w0 * total / groups > lo) --w0;
+    while ((w0 + 1) * total / groups <= lo) ++w0;
+    while (w1 + 1 < groups && (w1 + 1) * total / groups < hi) ++w1;
+    while (w1 * total / groups >= hi) --w1;
+    if (w0 == w1) return;  // one workgroup had the whole K range of this tile and finished it
+    int tm, tn;
+    xcd_tile_coords(first_tile_number + static_cast<int>(tile), tiles_m, tiles_n, tm, tn);
+    const int row = tm * BM + r, col = tn * BN + c;
+    if (row >= M || col >= N) return;  // N is a multiple of 4: a packet is inside or outside
+    f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (u64 w = w0; w <= w1; ++w) {
+        const u64 begins = w * total / groups;
+        if (begins == (w + 1) * total / groups) continue;  // a workgroup without a share wrote nothing
+        const u64 slot = 2 * w + (begins / kt != tile ? 1u : 0u);
+        const f32x4 p = *reinterpret_cast<const f32x4*>(ws + slot * static_cast<size_t>(BM * BN) + static_cast<size_t>(r) * BN + c);
+        sum += p;
+    }
+    f32x4* out = reinterpret_cast<f32x4*>(C + static_cast<size_t>(row) * N + col);
+    f32x4 res;
+    if (beta == 0.0f) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) res[j] = alpha * sum[j];
+    } else {
+        const f32x4 old = *out;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) res[j] = __builtin_fmaf(alpha, sum[j], beta * old[j]);
+    }
+    *out = res;
 }
 
 // -------------------------------------------- kernel 5, one wave per tile --
@@ -1108,28 +1200,75 @@ __global__ __launch_bounds__(kWave * KSPLIT) void sgemm_single_wave_kernel(
     }
 }
 
-// ------------------------------------------------ kernel 5, K split: adding up --
-// C = alpha * (part 0 + part 1 + ... in this order: the same bits on every run) + beta * C, four elements per
-// thread; the parts are the M x N slices the SPLIT form of the workgroup kernel wrote.
-__global__ __launch_bounds__(256) void sgemm_add_parts_kernel(size_t quads, int parts, const f32x4* __restrict__ ws,
-                                                              float alpha, float beta, f32x4* C) {
-    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
-    if (i >= quads) return;
-    f32x4 sum = ws[i];
-    for (int p = 1; p < parts; ++p) sum += ws[static_cast<size_t>(p) * quads + i];
-    f32x4 r;
-    if (beta == 0.0f) {
+// ------------------------------------------------ kernel 5, a thin strip of columns --
+// C[:, n0 .. n0 + r) = alpha * A @ B[:, n0 .. n0 + r) + beta * C[:, n0 .. n0 + r) for r <= R columns: what is left of
+// N beyond a whole number of 256-column tiles when that is a few columns only (N = 4097: a 257th tile column
+// would cost a seventeenth of the whole product for one column of C). Not matrix-instruction work: a
+// wavefront owns a row of A at a time, its lanes walk the row 64 elements apart (256 B per instruction),
+// multiply by the strip of B, which waits in LDS (KC rows of it at a time), and the lanes' sums meet in a
+// butterfly. The summation order differs from the big tiles', within the same tolerance.
+template <int R, int KC, int ROWS>
+__global__ __launch_bounds__(256) void sgemm_thin_columns_kernel(int M, int N, int K, int n0, int r, float alpha,
+                                                                 const float* __restrict__ A, const float* __restrict__ B,
+                                                                 float beta, float* C) {
+    __shared__ float strip[KC * R];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    constexpr int PER_WAVE = ROWS / 4;
+    const int row_first = blockIdx.x * ROWS + wave * PER_WAVE;
+    float acc[PER_WAVE][R];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) r[j] = alpha * sum[j];
-    } else {
-        const f32x4 old = C[i];
+    for (int i = 0; i < PER_WAVE; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) r[j] = __builtin_fmaf(alpha, sum[j], beta * old[j]);
+        for (int j = 0; j < R; ++j) acc[i][j] = 0.0f;
+    for (int k0 = 0; k0 < K; k0 += KC) {
+        const int kc = K - k0 < KC ? K - k0 : KC;
+        __syncthreads();  // the strip of the chunk before is no longer read
+        for (int e = threadIdx.x; e < kc * R; e += 256) {
+            const int k = e / R, j = e % R;
+            strip[e] = j < r ? B[static_cast<size_t>(k0 + k) * N + n0 + j] : 0.0f;
+        }
+        __syncthreads();
+        // four steps of 64 k at a time: 4 * PER_WAVE loads in flight per lane
+        for (int kb = 0; kb < kc; kb += 4 * kWave) {
+            float a[4][PER_WAVE];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int k = kb + u * kWave + lane;
+#pragma unroll
+                for (int i = 0; i < PER_WAVE; ++i)
+                    a[u][i] = (k < kc && row_first + i < M) ? A[static_cast<size_t>(row_first + i) * K + k0 + k] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int k = kb + u * kWave + lane;
+                if (k < kc) {
+#pragma unroll
+                    for (int j = 0; j < R; ++j) {
+                        const float b = strip[k * R + j];
+#pragma unroll
+                        for (int i = 0; i < PER_WAVE; ++i) acc[i][j] = __builtin_fmaf(a[u][i], b, acc[i][j]);
+                    }
+                }
+            }
+        }
     }
-    C[i] = r;
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; ++i)
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            float v = acc[i][j];
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, kWave);
+            if (lane == 0 && row_first + i < M && j < r) {
+                float* c = &C[static_cast<size_t>(row_first + i) * N + n0 + j];
+                *c = epilogue(alpha, v, beta, c);
+            }
+        }
 }
 
 // --------------------------------------------------------------- launchers --
+
+constexpr int kThinColumns = 8;  // up to this many columns beyond whole 256-column tiles go to the thin-strip kernel
 
 template <int BM, int BN, int BK, int TM, int TN, bool VEC>
 int run_thread_tile(int M, int N, int K, float alpha, const float* A, const float* B, float beta,
@@ -1167,13 +1306,15 @@ int run_wave_tile(int M, int N, int K, float alpha, const float* A, const float*
 }
 
 // Whole-tile kernel when the problem is made of 256 x 256 tiles and there are
-// enough of them for three quarters of the CUs.
+// enough of them for three quarters of the CUs. n_cols (a multiple of 256 when given): only the first n_cols
+// columns of C are computed; N stays the row length of B and C.
 template <int BM, int BN, int BK, int WM, int WN, bool ALLOW_EDGES>
 bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const float* B, float beta,
-                       float* C, hipStream_t s, int* rc) {
+                       float* C, hipStream_t s, int* rc, int n_cols = -1) {
     if (K <= 0) return false;
+    if (n_cols < 0) n_cols = N;
     const bool aligned = aligned16(A) && aligned16(B) && aligned16(C);
-    const bool whole = aligned && M % BM == 0 && N % BN == 0 && K % BK == 0;
+    const bool whole = aligned && M % BM == 0 && n_cols % BN == 0 && N % 4 == 0 && K % BK == 0;
     // Edges: the kernel's buffer offsets are 32 bits wide (a 256-row panel of A plus one K tile; all of B
     // plus one K tile). Rows that do not stay 16 B aligned (N or K not a multiple of 4, or matrices that
     // are only 4 B aligned) take the ragged form, whose K loop needs at least one group of 4.
@@ -1182,7 +1323,7 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
                    (static_cast<long long>(BM) + 64) * K * 4 >= (1ll << 31) ||
                    (static_cast<long long>(K) + 64) * N * 4 >= (1ll << 31)))
         return false;
-    const int tiles_m = ceil_div(M, BM), tiles_n = ceil_div(N, BN);
+    const int tiles_m = ceil_div(M, BM), tiles_n = ceil_div(n_cols, BN);
     if (static_cast<long long>(tiles_m) * tiles_n * 4 < 3ll * cu_count()) return false;
     if (static_cast<long long>(tiles_m) * tiles_n < cu_count()) {
         // A single, partial round of big tiles costs a full one: four strips per SIMD on the CUs that have a
@@ -1381,32 +1522,47 @@ bool try_single_wave(int M, int N, int K, float alpha, const float* A, const flo
     return true;
 }
 
-// K split across workgroups, for problems with too few 64 x 256 tiles for the CUs and a long K (skinny
-// problems: 128 x 4096 x 4096 has 32 such tiles for 256 CUs). Needs M x N x parts floats of workspace, which the
-// reference-shaped entry points do not have; prism_sgemm_ws takes one. Returns the number of parts (0: no split).
-int split_parts(int M, int N, int K, const float* A, const float* B, const float* C) {
+// What prism_sgemm_ws does with a workspace: the K ranges of some or all output tiles are shared evenly between
+// `groups` workgroups (the STREAMK form of the workgroup kernel), which takes 2 * groups tile-sized slots of
+// workspace for the partial products.
+//   bm == 256: problems of 256 x 256 tiles whose count is not a whole number of rounds of the CUs. The whole
+//              rounds (main_tiles tiles) run as ever, one tile per workgroup; the sk_tiles tiles of the last,
+//              partial round are shared between all CUs, so that round costs its share of a round instead of a
+//              whole one (or of what the cheaper cuts of launch_sgemm make of it).
+//   bm == 64:  skinny problems (few 64 x 256 tiles, long K; 128 x 4096 x 4096 has 32 such tiles for 256 CUs).
+struct StreamKPlan {
+    int bm = 0;          // 0: no sharing, the call is launch_sgemm
+    int main_tiles = 0;  // tiles of the whole rounds (bm == 256)
+    int sk_tiles = 0;
+    int groups = 0;
+    bool whole = false;  // whole tiles and whole K tiles: the kernel's form without range checks
+    size_t bytes() const { return static_cast<size_t>(2) * groups * bm * 256 * sizeof(float); }
+};
+
+// The skinny case: a small model of the shared and the unshared kernels says whether sharing pays. Returns the
+// number of K parts per tile the model prefers (0: leave it). M, N multiples of 64 and 256, K of 16.
+int skinny_parts(int M, int N, int K) {
     if (M <= 0 || N <= 0 || K < 1024 || M % 64 || N % 256 || K % 16) return 0;
-    if (A != nullptr && !(aligned16(A) && aligned16(B) && aligned16(C))) return 0;
     const long long tiles = static_cast<long long>(M / 64) * (N / 256);
     const int cus = cu_count();
-    if (tiles * 5 > cus) return 0;                       // from about a fifth of the CUs up the unsplit kernels are level
+    if (tiles * 5 > cus) return 0;                       // from about a fifth of the CUs up the unshared kernels are level
     if (static_cast<long long>(K) * 64 >= (1ll << 30) || static_cast<long long>(N) * 64 >= (1ll << 30)) return 0;
-    // The number of parts that a small model of the two kernels prefers: rounds of workgroups, each as long as
-    // its part of K plus a fixed cost worth about 128 k (53 ns per k for a wavefront's strip at the fp32 MFMA
-    // rate), and the adding-up, which moves parts + 2 times the output at about 5 TB/s behind a second launch.
-    // Measured against it on 128 x 4096 x 4096: 4 / 8 / 16 parts 65 / 100 / 93 TFLOP/s (model 65 / 105 / 84).
+    // Rounds of workgroups, each as long as its part of K plus a fixed cost worth about 128 k (53 ns per k for a
+    // wavefront's strip at the fp32 MFMA rate), and the adding-up, which moves parts + 2 times the output at
+    // about 5 TB/s behind a second launch. Measured against it on 128 x 4096 x 4096: 4 / 8 / 16 parts
+    // 65 / 100 / 93 TFLOP/s (model 65 / 105 / 84).
     int parts = 0;
     double best = 0.0;
     for (int p = 2; p <= 64; p *= 2) {
         if (K % (16 * p) != 0 || K / p < 128) break;
-        const double rounds = static_cast<double>((tiles * p + cus - 1) / cus);
-        const double us = rounds * (K / p + 128) * 0.053 + (p + 2) * (static_cast<double>(M) * N * 4.0) / 5.0e6 + 3.0;
+        const double rounds = static_cast<double>(tiles * p) / cus;
+        const double us = (rounds < 1.0 ? 1.0 : rounds) * (K / p + 128) * 0.053 + (p + 2) * (static_cast<double>(M) * N * 4.0) / 5.0e6 + 3.0;
         if (parts == 0 || us < best) {
             best = us;
             parts = p;
         }
     }
-    // Against the unsplit one-wave tiles of 32 x 32, which such shapes take: bound by their L2 traffic (1 B per
+    // Against the unshared one-wave tiles of 32 x 32, which such shapes take: bound by their L2 traffic (1 B per
     // 8 flop at about 9 TB/s) or by the instructions a wavefront issues one after the other (13.3 ns per k and
     // tile, K cut four or two ways inside the workgroup where launch_sgemm does that), plus about 6 us.
     // Measured: 128 x 4096 x 4096 68 us (model 60), 64 x 512 x 2048 12 (13), 64 x 256 x 16384 65 (60).
@@ -1414,39 +1570,102 @@ int split_parts(int M, int N, int K, const float* A, const float* B, const float
     const long long tiles32 = static_cast<long long>(M / 32) * (N / 32), simds = 4ll * cus;
     const int inner = (tiles32 * 8 <= simds && K >= 1024) ? 4 : (tiles32 * 4 <= simds && K >= 512) ? 2 : 1;
     const double chain_us = static_cast<double>((tiles32 * inner + simds - 1) / simds) * (K / inner) * 0.0133;
-    const double unsplit_us = std::max(flop / 8.0 / 9.0e6, chain_us) + 6.0;
-    return (parts >= 2 && best < 0.85 * unsplit_us) ? parts : 0;
+    const double unshared_us = std::max(flop / 8.0 / 9.0e6, chain_us) + 6.0;
+    return (parts >= 2 && best < 0.85 * unshared_us) ? parts : 0;
+}
+
+// aligned: A, B and C are 16 B aligned (a query without pointers assumes so).
+StreamKPlan stream_k_plan(int M, int N, int K, bool aligned) {
+    StreamKPlan plan;
+    if (M <= 0 || N <= 0 || K <= 0 || !aligned || N % 4 || K % 4) return plan;  // rows must stay 16 B aligned
+    const int cus = cu_count();
+    if (const int parts = skinny_parts(M, N, K)) {
+        const long long tiles = static_cast<long long>(M / 64) * (N / 256);
+        plan.bm = 64;
+        plan.sk_tiles = static_cast<int>(tiles);
+        plan.groups = static_cast<int>(std::min<long long>(cus, tiles * parts));
+        plan.whole = true;
+        return plan;
+    }
+    // 256 x 256 tiles: the same limits as try_wave_tile_dma (32-bit buffer offsets in the range-checked form).
+    const bool whole = M % 256 == 0 && N % 256 == 0 && K % 32 == 0;
+    if (!whole && ((256ll + 64) * K * 4 >= (1ll << 31) || (static_cast<long long>(K) + 64) * N * 4 >= (1ll << 31))) return plan;
+    const long long tiles = static_cast<long long>(ceil_div(M, 256)) * ceil_div(N, 256);
+    // Fewer tiles than CUs: sharing all of them was measured level with or behind the smaller tiles launch_sgemm
+    // picks there (3072^3 134 against 149 TFLOP/s, 3584^3 139 against 142, 3200^3 125 against 123): every tile
+    // then pays for partial products.
+    if (tiles <= cus || tiles > 0x3fffffff || K < 256) return plan;
+    const int left = static_cast<int>(tiles % cus);
+    if (left == 0) return plan;
+    // A last round that is nearly full gains nothing from being shared (the partial products cost a few per
+    // cent), and one of just under a quarter of the CUs is as cheap as 64 x 256 slices, one to a CU, which
+    // launch_sgemm makes of it (6144^3, 64 tiles left: 152.7 against 151.4 shared; 4352^3, 33 left: 136.6
+    // against 146.7 shared).
+    if (left * 16 > 15 * cus || (left * 4 <= cus && left * 16 >= 3 * cus)) return plan;
+    plan.bm = 256;
+    plan.main_tiles = static_cast<int>(tiles - left);
+    plan.sk_tiles = left;
+    plan.groups = cus;
+    plan.whole = whole;
+    return plan;
 }
 
 }  // namespace
 
-size_t sgemm_workspace_bytes(int M, int N, int K) {
-    const int parts = split_parts(M, N, K, nullptr, nullptr, nullptr);
-    return static_cast<size_t>(parts) * static_cast<size_t>(M > 0 ? M : 0) * static_cast<size_t>(N > 0 ? N : 0) * sizeof(float);
+size_t sgemm_workspace_bytes(int M, int N, int K) { return stream_k_plan(M, N, K, true).bytes(); }
+
+int sgemm_ws_plan(int M, int N, int K, size_t ws_bytes, int* groups, int* sk_tiles) {
+    const StreamKPlan plan = stream_k_plan(M, N, K, true);
+    const bool taken = plan.bm != 0 && ws_bytes >= plan.bytes();
+    if (groups) *groups = taken ? plan.groups : 0;
+    if (sk_tiles) *sk_tiles = taken ? plan.sk_tiles : 0;
+    return 0;
 }
 
 int launch_sgemm_ws(int variant, int M, int N, int K, float alpha, const float* A, const float* B, float beta,
                     float* C, void* ws, size_t ws_bytes, hipStream_t s) {
-    if (variant == 0 || variant == 5) {
-        const int parts = (C != nullptr && A != nullptr && B != nullptr && M > 0 && N > 0) ? split_parts(M, N, K, A, B, C) : 0;
-        const size_t need = static_cast<size_t>(parts) * static_cast<size_t>(M) * N * sizeof(float);
-        if (parts >= 2 && ws != nullptr && ws_bytes >= need && (reinterpret_cast<uintptr_t>(ws) & 15u) == 0) {
-            const int tiles_m = M / 64, tiles_n = N / 256;
-            const dim3 grid(static_cast<unsigned>(tiles_m) * tiles_n * parts);
-            sgemm_wave_tile_dma_kernel<64, 256, 16, 32, 128, false, false, true><<<grid, dim3(256), 0, s>>>(
-                M, N, K, 1.0f, A, B, 0.0f, static_cast<float*>(ws), tiles_m, tiles_n, parts);
-            if (int rc = check_launch("sgemm_wave_tile_dma_kernel (K split)")) return rc;
-            const size_t quads = static_cast<size_t>(M) * N / 4;
-            sgemm_add_parts_kernel<<<dim3(static_cast<unsigned>(ceil_div(quads, size_t{256}))), dim3(256), 0, s>>>(
-                quads, parts, static_cast<const f32x4*>(ws), alpha, beta, reinterpret_cast<f32x4*>(C));
-            return check_launch("sgemm_add_parts_kernel");
+    if (int rc = check_sgemm_arguments(variant, M, N, K, A, B, C)) return rc;
+    if ((variant == 0 || variant == 5) && M > 0 && N > 0 && K > 0 && ws != nullptr && aligned16(ws)) {
+        const StreamKPlan plan = stream_k_plan(M, N, K, aligned16(A) && aligned16(B) && aligned16(C));
+        if (plan.bm != 0 && ws_bytes >= plan.bytes()) {
+            float* parts = static_cast<float*>(ws);
+            const dim3 grid(static_cast<unsigned>(plan.groups));
+            if (plan.bm == 64) {
+                const int tiles_m = M / 64, tiles_n = N / 256;
+                sgemm_wave_tile_dma_kernel<64, 256, 16, 32, 128, false, false, true><<<grid, dim3(256), 0, s>>>(
+                    M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, 0, parts, plan.sk_tiles);
+                if (int rc = check_launch("sgemm_wave_tile_dma_kernel (K shared, 64 x 256 tiles)")) return rc;
+                sgemm_stream_k_fixup_kernel<64, 256, 16><<<dim3(static_cast<unsigned>(plan.sk_tiles) * 16), dim3(256), 0, s>>>(
+                    M, N, K, alpha, beta, C, parts, tiles_m, tiles_n, 0, plan.sk_tiles, grid.x);
+                return check_launch("sgemm_stream_k_fixup_kernel");
+            }
+            const int tiles_m = ceil_div(M, 256), tiles_n = ceil_div(N, 256);
+            if (plan.main_tiles > 0) {
+                const dim3 main_grid(static_cast<unsigned>(plan.main_tiles));
+                if (plan.whole)
+                    sgemm_wave_tile_dma_kernel<256, 256, 32, 32, 128, false><<<main_grid, dim3(1024), 0, s>>>(
+                        M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
+                else
+                    sgemm_wave_tile_dma_kernel<256, 256, 32, 32, 128, true><<<main_grid, dim3(1024), 0, s>>>(
+                        M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
+                if (int rc = check_launch("sgemm_wave_tile_dma_kernel (whole rounds)")) return rc;
+            }
+            if (plan.whole)
+                sgemm_wave_tile_dma_kernel<256, 256, 32, 32, 128, false, false, true><<<grid, dim3(1024), 0, s>>>(
+                    M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, plan.main_tiles, parts, plan.sk_tiles);
+            else
+                sgemm_wave_tile_dma_kernel<256, 256, 32, 32, 128, true, false, true><<<grid, dim3(1024), 0, s>>>(
+                    M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, plan.main_tiles, parts, plan.sk_tiles);
+            if (int rc = check_launch("sgemm_wave_tile_dma_kernel (K shared, 256 x 256 tiles)")) return rc;
+            sgemm_stream_k_fixup_kernel<256, 256, 32><<<dim3(static_cast<unsigned>(plan.sk_tiles) * 64), dim3(256), 0, s>>>(
+                M, N, K, alpha, beta, C, parts, tiles_m, tiles_n, plan.main_tiles, plan.sk_tiles, grid.x);
+            return check_launch("sgemm_stream_k_fixup_kernel");
         }
     }
     return launch_sgemm(variant, M, N, K, alpha, A, B, beta, C, s);
 }
 
-int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, const float* B,
-                 float beta, float* C, hipStream_t s) {
+int check_sgemm_arguments(int variant, int M, int N, int K, const float* A, const float* B, const float* C) {
     if (variant < 0 || variant > 6) return fail(1, "prism_sgemm: unknown kernel number %d", variant);
     if (M < 0 || N < 0 || K < 0) return fail(1, "prism_sgemm: negative dimension (%d,%d,%d)", M, N, K);
     if (M == 0 || N == 0) return 0;
@@ -1454,6 +1673,13 @@ int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, 
         return fail(1, "prism_sgemm: null matrix pointer");
     if (!aligned4(A) || !aligned4(B) || !aligned4(C))
         return fail(1, "prism_sgemm: matrices must be 4-byte aligned");
+    return 0;
+}
+
+int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, const float* B,
+                 float beta, float* C, hipStream_t s) {
+    if (int rc = check_sgemm_arguments(variant, M, N, K, A, B, C)) return rc;
+    if (M == 0 || N == 0) return 0;
     const size_t mn = static_cast<size_t>(M) * N;
     if (variant == 0) variant = 5;
     // K == 0 leaves C = beta * C; the naive kernel does exactly that.
@@ -1492,6 +1718,16 @@ int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, 
                 // Whole 256 x 256 tiles for at least three quarters of the CUs: the direct-to-LDS kernel,
                 // K tiles of 32 (128 KiB of LDS) when K allows, else of 16.
                 int rc = 0;
+                // A few columns beyond a whole number of 256-column tiles (N = 4097) would cost a whole tile
+                // column: the big tiles take the whole columns, a thin-strip kernel the rest.
+                if (const int r = N % 256; N > 256 && r > 0 && r <= kThinColumns && M >= 64 &&
+                    try_wave_tile_dma<256, 256, 32, 32, 128, true>(M, N, K, alpha, A, B, beta, C, s, &rc, N - r)) {
+                    if (rc != 0) return rc;
+                    constexpr int ROWS = 8;  // two rows per wavefront: a thousand workgroups for M = 8191
+                    sgemm_thin_columns_kernel<kThinColumns, 1024, ROWS><<<dim3(static_cast<unsigned>(ceil_div(M, ROWS))), dim3(256), 0, s>>>(
+                        M, N, K, N - r, r, alpha, A, B, beta, C);
+                    return check_launch("sgemm_thin_columns_kernel");
+                }
                 // Ragged M, N, K take the K-tile-of-32 kernel with zero-filled edges (its ragged form when
                 // rows are not 16 B aligned).
                 if (try_wave_tile_dma<256, 256, 32, 32, 128, true>(M, N, K, alpha, A, B, beta, C, s, &rc)) return rc;

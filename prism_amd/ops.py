@@ -238,17 +238,28 @@ def run_my_kernel(my_kernel_num: int, M: int, N: int, K: int, alpha: float, A: P
 
 
 def sgemm_workspace_size(M: int, N: int, K: int) -> int:
-    """Workspace bytes with which kernel 5 cuts K across workgroups for this shape (0: it would not)."""
+    """Workspace bytes with which kernel 5 shares K ranges between workgroups for this shape on the current
+    device (0: it would not)."""
     return int(_lib.load().prism_sgemm_workspace_bytes(M, N, K))
+
+
+def sgemm_workspace_plan(M: int, N: int, K: int, workspace_bytes: int):
+    """(workgroups that share K ranges, tiles they share) for a call with aligned operands and that much
+    workspace; (0, 0) when the call would be the plain one."""
+    import ctypes
+    groups, tiles = ctypes.c_int(0), ctypes.c_int(0)
+    _check(_lib.load().prism_sgemm_ws_plan(M, N, K, workspace_bytes, ctypes.byref(groups), ctypes.byref(tiles)), "sgemm_ws_plan")
+    return groups.value, tiles.value
 
 
 def sgemm(M: int, N: int, K: int, alpha: float, A: "torch.Tensor", B: "torch.Tensor", beta: float,
           C: "torch.Tensor", variant: int = 5, workspace: Optional["torch.Tensor"] = None) -> "torch.Tensor":
     """sgemm(M,N,K,alpha,A,B,beta,C): the kernel signature of generated/my_sgemm_kernel_*.cu.
 
-    workspace: a device buffer of at least sgemm_workspace_size(M, N, K) bytes lets kernel 5 cut K across
-    workgroups on skinny shapes (deterministic: the parts are added in a fixed order); calls that share one
-    must be ordered on one stream. Without it the call is the reference-shaped one.
+    workspace: a device buffer of at least sgemm_workspace_size(M, N, K) bytes lets kernel 5 share the K ranges
+    of the tiles of a partial last round (or of all tiles of a skinny shape) between all compute units
+    (deterministic: a tile's partial products are added in the order of k); calls that share one must be
+    ordered on one stream. Without it the call is the reference-shaped one.
     """
     if variant not in (0, 1, 2, 3, 4, 5, 6):
         raise ValueError("Unknown my_kernel number")

@@ -48,7 +48,7 @@ def test_every_declaration_cites_the_reference():
                        ("prism_scan_max_i32", "scan.py:106-173"), ("prism_scan_min_i32", "scan.py:106-173"),
                        ("prism_launch_scan", "4090_scan/main.cu"),
                        ("prism_sgemm", "runner.cu"), ("prism_run_my_kernel", "runner.cu"),
-                       ("prism_sgemm_ws", "runner.cu:\n * 191-243"),
+                       ("prism_sgemm_ws", "evals/4090_sgemm/runner.cu:191-243"),
                        ("prism_gemm_bf16", "h100_matmul.py"), ("prism_runmyh100", "utils.cuh")]:
         decl = text.index(name + "(")
         comment = text.rfind("/*", 0, decl)
@@ -68,6 +68,12 @@ def test_argument_checks_run_before_any_gpu_work(lib):
     assert lib.prism_sgemm(7, 4, 4, 4, 1.0, None, None, 0.0, None, None) == 1
     assert lib.prism_sgemm(5, -1, 4, 4, 1.0, None, None, 0.0, None, None) == 1
     assert lib.prism_sgemm(5, 4, 4, 4, 1.0, None, None, 0.0, None, None) == 1  # null matrices
+    # the workspace form checks the same things before it looks at the workspace
+    assert lib.prism_sgemm_ws(7, 4, 4, 4, 1.0, None, None, 0.0, None, None, 0, None) == 1
+    assert b"unknown kernel number" in lib.prism_last_error_string()
+    assert lib.prism_sgemm_ws(5, 128, 4096, -4096, 1.0, None, None, 0.0, None, None, 0, None) == 1
+    assert lib.prism_sgemm_ws(5, 128, 4096, 4096, 1.0, None, None, 0.0, None, None, 0, None) == 1
+    assert b"null matrix pointer" in lib.prism_last_error_string()
     # the workspace form checks like prism_sgemm; the size query needs no device (256 CUs assumed without one)
     assert lib.prism_sgemm_ws(7, 4, 4, 4, 1.0, None, None, 0.0, None, None, 0, None) == 1
     assert lib.prism_sgemm_ws(5, 4, 4, 4, 1.0, None, None, 0.0, None, None, 0, None) == 1

@@ -214,14 +214,16 @@ def test_wave_tile_leftover_round(prism, oracle, shape):
 
 @pytest.mark.parametrize("shape", [(128, 4096, 4096), (64, 2048, 8192), (256, 256, 16384), (192, 768, 8192), (64, 4096, 4096)])
 def test_wave_tile_k_split_with_workspace(prism, oracle, shape):
-    """Skinny products through prism_sgemm_ws: kernel 5 cuts K across workgroups (8, 32, 64, 16 and 16 parts
-    here), every part writes its partial product into the workspace and a second kernel adds the parts in a fixed
-    order. Every element against fp64, with and without reading C (C full of NaN when it is not read), the same
-    bits on a second run, nothing written beyond the bytes prism_sgemm_workspace_bytes names, and with a
-    workspace one byte short the call is the unsplit one, bit for bit."""
+    """Skinny products through prism_sgemm_ws: the K ranges of the few 64 x 256 tiles are shared between all
+    CUs, every workgroup writes its partial products into the workspace and a second kernel adds a tile's parts
+    in the order of k. Every element against fp64, with and without reading C (C full of NaN when it is not
+    read), the same bits on a second run, nothing written beyond the bytes prism_sgemm_workspace_bytes names,
+    and with a workspace one byte short the call is the unshared one, bit for bit."""
     M, N, K = shape
     need = prism.sgemm_workspace_size(M, N, K)
-    assert need >= 2 * M * N * 4 and need % (M * N * 4) == 0
+    groups, shared = prism.sgemm_workspace_plan(M, N, K, need)
+    assert shared == (M // 64) * (N // 256) and 2 * shared <= groups <= prism.device_info()["cu_count"]
+    assert need == 2 * groups * 64 * 256 * 4 and prism.sgemm_workspace_plan(M, N, K, need - 1) == (0, 0)
     A, B, Cm = oracle.gen_sgemm(M, N, K, seed=M + N + K)
     a, b = dev(A), dev(B)
     wsbuf = torch.full((need + 512,), 0x5A, dtype=torch.uint8, device=DEV)
@@ -244,6 +246,56 @@ def test_wave_tile_k_split_with_workspace(prism, oracle, shape):
     prism.sgemm(M, N, K, 1.25, a, b, 0.5, c4, variant=5)
     assert np.array_equal(host(c3), host(c4))
     assert np.max(np.abs(host(c3) - outs[0])) <= 2 * tol(oracle, K, A, B, 0.5, Cm)
+
+
+@pytest.mark.parametrize("shape", [(4352, 4352, 512), (5120, 5120, 288), (5000, 5000, 260), (4608, 4864, 1024), (4100, 4612, 300)])
+def test_wave_tile_last_round_shared_with_workspace(prism, oracle, shape):
+    """256 x 256 tiles that are not a whole number of rounds of the CUs, through prism_sgemm_ws: the whole rounds
+    run one tile per workgroup, the K ranges of the tiles of the last round (33, 144, 144, 86 and 67 here) are
+    shared between all CUs, in shares of two K tiles and up, and a second kernel adds a tile's partial products.
+    Whole tiles and ragged M, N, K (rows 16 B aligned). Every element against an fp64 product formed on the
+    device, with and without reading C (NaN in C when it is not read), the same bits on a second run, nothing
+    written outside the workspace, and the plan query says that the shared form is the one that ran."""
+    import fp64_referee
+    M, N, K = shape
+    cus = prism.device_info()["cu_count"]
+    tiles = -(-M // 256) * -(-N // 256)
+    need = prism.sgemm_workspace_size(M, N, K)
+    assert need == 2 * cus * 256 * 256 * 4
+    assert prism.sgemm_workspace_plan(M, N, K, need) == (cus, tiles % cus)
+    A, B, C0 = _device_inputs(M, N, K)
+    wsbuf = torch.full((need + 512,), 0x5A, dtype=torch.uint8, device=DEV)
+    ws = wsbuf[256:256 + need]
+    for beta in (0.5, 0.0):
+        c = C0.clone() if beta else torch.full((M, N), float("nan"), device=DEV)
+        print(f"prism_sgemm_ws {M}x{N}x{K} beta={beta}", flush=True)
+        prism.sgemm(M, N, K, 1.25, A, B, beta, c, variant=5, workspace=ws)
+        err = fp64_referee.sgemm_max_err_fp64(1.25, A, B, beta, C0, c)
+        assert err <= 1.25 * _bound(K, beta), f"{M}x{N}x{K} beta={beta}: max error {err:.3e}"
+        c2 = C0.clone() if beta else torch.full((M, N), float("nan"), device=DEV)
+        prism.sgemm(M, N, K, 1.25, A, B, beta, c2, variant=5, workspace=ws)
+        assert torch.equal(c, c2)
+    assert bool((wsbuf[:256] == 0x5A).all()) and bool((wsbuf[256 + need:] == 0x5A).all())
+
+
+@pytest.mark.parametrize("shape", [(4096, 3073, 100), (4000, 3080, 67), (4096, 3076, 64), (8191, 4097, 1023), (4096, 3329, 4), (3000, 4099, 2100)])
+def test_wave_tile_thin_strip_of_columns(prism, oracle, shape):
+    """N a few columns (1 to 8) beyond a whole number of 256-column tiles: the big tiles take the whole tile
+    columns, a strip kernel the rest (rows 4 B or 16 B aligned, whole and ragged M and K, K longer than the
+    strip kernel's LDS chunk). Every element against fp64; C poisoned with NaN when it is not read; guard
+    values around C."""
+    import fp64_referee
+    M, N, K = shape
+    A, B, C0 = _device_inputs(M, N, K)
+    for beta in (0.5, 0.0):
+        cbuf = torch.full((M * N + 128,), 777.0, device=DEV)
+        c = cbuf[64:64 + M * N].view(M, N)
+        c.copy_(C0 if beta else torch.full((M, N), float("nan"), device=DEV))
+        print(f"prism_sgemm {M}x{N}x{K} beta={beta}", flush=True)
+        prism.sgemm(M, N, K, 0.75, A, B, beta, c, variant=5)
+        err = fp64_referee.sgemm_max_err_fp64(0.75, A, B, beta, C0, c)
+        assert err <= _bound(K, beta), f"{M}x{N}x{K} beta={beta}: max error {err:.3e}"
+        assert bool((cbuf[:64] == 777.0).all()) and bool((cbuf[64 + M * N:] == 777.0).all())
 
 
 def test_workspace_form_leaves_other_shapes_and_kernels_alone(prism, oracle):
