@@ -138,7 +138,9 @@ def bench_sgemm(prism, M, N, K, alpha, beta, variant, steps, warmup, gate=True, 
 
 # ------------------------------------------------------------------- scan --
 
-def bench_scan(prism, n, steps, warmup, gate=True):
+def bench_scan(prism, n, steps, warmup, gate=True, ticket_order=False):
+    """ticket_order: tiles numbered by the reference's ticket counter (PRISM_SCAN_TICKET_ORDER) instead of by
+    workgroup id, through prism_scan_i32_ex."""
     import torch
     g = torch.Generator(device="cuda")
     g.manual_seed(0)
@@ -164,8 +166,11 @@ def bench_scan(prism, n, steps, warmup, gate=True):
     # evals/4090_scan/main.cu:81-82).
     lib, st = _capi()
     xp, op, wp, wb = x.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel()
-    ms = time_steps(lambda: lib.prism_scan_i32(xp, op, n, wp, wb, st), steps, warmup)
-    prism.scan_status(ws)  # raises if any timed call gave up in its look-back
+    if ticket_order:
+        ms = time_steps(lambda: lib.prism_scan_i32_ex(xp, op, n, wp, wb, 2, -1, st), steps, warmup)
+    else:
+        ms = time_steps(lambda: lib.prism_scan_i32(xp, op, n, wp, wb, st), steps, warmup)
+    prism.scan_status(ws)  # raises if any timed call reported anything
     nbytes = 2.0 * 4 * n  # scan_harness.cuh:161
     gbps = nbytes / (ms * 1e-3) / 1e9
     return {"ms": ms, "GBps": gbps,
@@ -358,6 +363,10 @@ def main() -> int:
     if want("scan"):
         res["scan"] = bench_scan(prism, 1 << 30, K, W)
         log("scan 2^30:", res["scan"])
+        res["scan_ticket_order"] = bench_scan(prism, 1 << 30, K, W, gate=False, ticket_order=True)
+        res["scan_ticket_order"]["note"] = ("the same scan with tiles numbered by the reference's ticket counter "
+                                            "(examples/scan.py:88-99) instead of by workgroup id")
+        log("scan 2^30, ticket order:", res["scan_ticket_order"])
     if want("gemm_bf16"):
         res["gemm_bf16"] = bench_gemm_bf16(prism, 8192, K, W)
         log("gemm_bf16 8192^3:", res["gemm_bf16"])

@@ -93,8 +93,10 @@ int prism_wave_regroup_i32(const int32_t* in, int32_t* out, size_t n, int items_
 size_t prism_scan_workspace_bytes(size_t n);
 
 /*
- * Brings a workspace (16-byte aligned) into its initial state: all zeros. Call
- * it once after allocating (a zero-filled allocation is initialised as well).
+ * Brings a workspace (16-byte aligned) into its initial state (zeros and a
+ * magic word in the header). Call it once after allocating; a scan on a
+ * workspace without the magic word touches nothing in it and
+ * prism_scan_status reports PRISM_ERROR_SCAN_WORKSPACE.
  * The reference clears its workspace with two cudaMemset calls in front of
  * every launch (evals/4090_scan/main.cu:81-82); here every scan leaves the
  * workspace ready for the next one, so no clearing launch sits in front of a
@@ -110,12 +112,15 @@ int prism_scan_workspace_init(void* workspace, size_t workspace_bytes, void* str
  * runs); partial overlap is not. The workspace must be initialised (above) and
  * hold prism_scan_workspace_bytes(n) bytes; calls that share a workspace must
  * be ordered on one stream, and may differ in n and in kind.
- * Tiles are numbered by workgroup id, which relies on workgroups starting in
- * id order; prism_scan_i32_ex can select the reference's ticket counter
- * instead. A tile's wait for its predecessors is bounded, so the kernel always
- * finishes; should a wait ever run out, the output is invalid and
- * prism_scan_status reports it. Callers that must not return a wrong scan call
- * prism_scan_status before they use the output.
+ * Tiles are numbered by workgroup id, which waits least when workgroups start
+ * in id order (prism_scan_i32_ex can select the reference's ticket counter
+ * instead), but the result does not rest on that order: a tile whose
+ * predecessor stays silent for milliseconds forms that predecessor's sum from
+ * the input itself, so every tile finishes on its own and the sums are the
+ * same bits however the workgroups were started. A return value of 0 means the
+ * call was enqueued; what can still invalidate the output is a workspace that
+ * was never initialised, which prism_scan_status reports once the stream has
+ * drained.
  * Replaces scan_kernel + its device helpers (examples/scan.py:23-227,
  * generated/scan_kernel.cu:1-29).
  */
@@ -127,6 +132,9 @@ enum {
     PRISM_SCAN_EXCLUSIVE = 1,     /* prism_scan_exclusive_i32's result                                  */
     PRISM_SCAN_TICKET_ORDER = 2,  /* tiles numbered by get_block_idx_from_global_counter's ticket        */
                                   /* (examples/scan.py:88-99) instead of by workgroup id                 */
+    PRISM_SCAN_NO_HELP = 4,       /* a look-back that runs out of polls reports it (prism_scan_status)   */
+                                  /* and goes on with a wrong sum instead of helping its predecessor:    */
+                                  /* the plain bounded wait, kept to exercise that way out               */
     PRISM_SCAN_OP_SUM = 0x00,
     PRISM_SCAN_OP_MAX = 0x10,     /* prism_scan_max_i32's result (inclusive, workgroup-id order only)    */
     PRISM_SCAN_OP_MIN = 0x20      /* prism_scan_min_i32's result (inclusive, workgroup-id order only)    */
@@ -134,14 +142,18 @@ enum {
 
 /* prism_scan_status: a tile gave up waiting for its predecessors. */
 #define PRISM_ERROR_SCAN_ORDER 10001
+/* prism_scan_status: the workspace was never initialised (or was overwritten). */
+#define PRISM_ERROR_SCAN_WORKSPACE 10002
 
 /*
  * prism_scan_i32 with every choice spelled out as an argument (the library
  * reads no environment variables and keeps no options between calls).
- * spin_limit bounds the polls of one look-back window: negative = the
- * library's default (2^22, seconds), 0 = every look-back gives up at once,
- * which exercises the kernel's way out from the host without a stuck
- * predecessor. The reference's kernel waits without bound
+ * spin_limit bounds the polls of one look-back window before the tile stops
+ * waiting for a silent predecessor and helps it (forms its sum from the
+ * input), or, with PRISM_SCAN_NO_HELP, reports and goes on: negative = the
+ * library's default (2^12 polls, milliseconds; 2^22 with PRISM_SCAN_NO_HELP),
+ * 0 = no waiting at all, which exercises either way out from the host without
+ * a stuck predecessor. The reference's kernel waits without bound
  * (generated/lookback_to_prev_blocks.cu:12-21).
  */
 int prism_scan_i32_ex(const int32_t* in, int32_t* out, size_t n, void* workspace,
@@ -153,22 +165,26 @@ int prism_scan_i32_ex(const int32_t* in, int32_t* out, size_t n, void* workspace
  * status words live in a device array that is part of the library (2 MiB + 256
  * bytes per GPU, held until the process ends), so n is limited to 2^31
  * elements; a larger n returns 1 with an error string. No counterpart in the
- * reference (its launcher takes a workspace the caller allocated,
- * evals/4090_scan/main.cu:68-86). It is for callers that cannot allocate:
- * code under HIP graph capture, tight serving loops, harnesses that forbid
- * hipMalloc. The call makes no hipMalloc / hipFree and uses no allocating
- * library routine. All calls on one GPU share that GPU's array: they must be
- * ordered on one stream, calls that overlap on one GPU race. Same kernels,
- * same result and same bounded look-back as prism_scan_i32;
+ * reference. It is for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc. The call makes
+ * no hipMalloc / hipFree and uses no allocating library routine. The first call
+ * on a device looks the array's address up and fills it once; that call must
+ * be made outside stream capture (prism_scan_status(NULL, 0, stream) serves as
+ * well), later ones may be captured. All calls on one GPU share that GPU's
+ * array: they must be ordered on one stream, calls that overlap on one GPU
+ * race. Same kernels and same result as prism_scan_i32;
  * prism_scan_status(NULL, 0, stream) reports for the library's array.
  */
 int prism_scan_i32_static(const int32_t* in, int32_t* out, size_t n, void* stream);
 
 /*
- * Waits for `stream`, then reports whether any scan on this workspace since
- * the last report gave up waiting in its look-back: 0 = none did;
- * PRISM_ERROR_SCAN_ORDER = one did, the output of that call is invalid, the
- * error string names the tile, and the workspace has been re-initialised.
+ * Waits for `stream`, then reports on the scans that used this workspace
+ * since the last report: 0 = nothing to report; PRISM_ERROR_SCAN_WORKSPACE =
+ * the workspace was not initialised (or something else wrote into it);
+ * PRISM_ERROR_SCAN_ORDER = a look-back gave up waiting (only scans that do not
+ * help: PRISM_SCAN_NO_HELP, the segmented and the 64-bit scan). In both cases
+ * the output of those scans is invalid, the error string says more, and the
+ * workspace has been initialised afresh.
  * workspace == NULL stands for the array prism_scan_i32_static uses on the
  * current device. The reference has no counterpart (its look-back cannot give up); this is what
  * turns a broken tile-order assumption into an error instead of a wrong sum.

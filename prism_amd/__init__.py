@@ -9,6 +9,7 @@ call loads (and, if the file is absent, builds) libprism_amd.so.
 from .ops import (  # noqa: F401
     PrismError,
     ScanOrderError,
+    ScanWorkspaceError,
     SGEMM_KERNELS,
     add_m,
     device_info,

@@ -62,8 +62,8 @@ int prism_add_m(const int32_t* x, int32_t* y, int32_t m, size_t n, void* stream)
 size_t prism_scan_workspace_bytes(size_t n) { return scan_workspace_bytes(n); }
 
 static_assert(PRISM_SCAN_EXCLUSIVE == kFlagExclusive && PRISM_SCAN_TICKET_ORDER == kFlagTicket &&
-                  PRISM_SCAN_OP_MAX == kFlagOpMax && PRISM_SCAN_OP_MIN == kFlagOpMin &&
-                  PRISM_ERROR_SCAN_ORDER == kScanOrderError,
+                  PRISM_SCAN_NO_HELP == kFlagNoHelp && PRISM_SCAN_OP_MAX == kFlagOpMax && PRISM_SCAN_OP_MIN == kFlagOpMin &&
+                  PRISM_ERROR_SCAN_ORDER == kScanOrderError && PRISM_ERROR_SCAN_WORKSPACE == kScanWorkspaceError,
               "include/prism_amd.h and common.h disagree");
 
 static const uint32_t* u32(const int32_t* p) { return reinterpret_cast<const uint32_t*>(p); }

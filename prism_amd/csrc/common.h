@@ -58,12 +58,12 @@ inline int cu_count() {
 // Internal launchers, one per kernel family (defined in the .hip files).
 int launch_add_m(const int32_t* x, int32_t* y, int32_t m, size_t n, hipStream_t s);
 // Scan flags and error code: the values of PRISM_SCAN_* / PRISM_ERROR_SCAN_ORDER in include/prism_amd.h.
-constexpr unsigned kFlagExclusive = 1u, kFlagTicket = 2u;
+constexpr unsigned kFlagExclusive = 1u, kFlagTicket = 2u, kFlagNoHelp = 4u;
 constexpr unsigned kFlagOpMask = 0x30u, kFlagOpSum = 0x00u, kFlagOpMax = 0x10u, kFlagOpMin = 0x20u;
-constexpr int kScanOrderError = 10001;
+constexpr int kScanOrderError = 10001, kScanWorkspaceError = 10002;
 size_t scan_workspace_bytes(size_t n);
 int scan_workspace_init(void* ws, size_t ws_bytes, hipStream_t s);
-// spin_limit < 0: the library's bound on look-back polls; 0: every look-back gives up at once.
+// spin_limit < 0: the library's bound on the polls of a look-back window; 0: a look-back never waits.
 int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, unsigned flags,
                 long long spin_limit, hipStream_t s);
 int scan_status(void* ws, size_t ws_bytes, hipStream_t s);

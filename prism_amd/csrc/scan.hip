@@ -33,22 +33,23 @@
 // with more than one wave per tile was measured slower: the extra status
 // traffic costs more than the round trips it saves.
 //
-// Tile order. A tile may only wait for tiles that are already running. The
-// reference gets that from a ticket counter (examples/scan.py:88-99): tiles are
-// numbered in the order blocks start. The ticket is an agent-scope atomic on one
-// address, and its round trip (about 2 us) sits in front of every block's first
-// load: measured 5 % of the run time at 2^30. The default here is therefore
-// tile = a fixed function of the workgroup id (chunks of 4 consecutive tiles go to
-// workgroups of one XCD, see the kernel), which is deadlock-free as long as the
-// dispatcher starts the workgroups of a 1-D grid in id order on every XCD (then
-// the lowest unfinished tile is always running; this is the same assumption
-// CUB's look-back scan makes on NVIDIA hardware). The flag kFlagTicket selects the
-// reference's ticket order instead. In both modes the look-back wait is bounded
-// (kSpinLimit polls, several seconds): a wave that runs out stores the tile number
-// plus one into the workspace header (kHdrReport) and carries on with a wrong
-// prefix, so that the GPU never hangs; scan_status() reads that word after the
-// stream has drained and turns it into an error, so that a broken ordering
-// assumption is reported, not returned as a wrong result.
+// Tile order. The reference numbers tiles with a ticket counter (examples/scan.py:88-99), in the order blocks
+// start, so that a tile only ever waits for tiles that are already running. The ticket is an agent-scope
+// atomic on one address, and its round trip (about 2 us) sits in front of every block's first load: measured
+// 12 % of the run time at 2^30. The default here is tile = a fixed function of the workgroup id (chunks of 4
+// consecutive tiles go to workgroups of one XCD, see the kernel), which waits least when the dispatcher starts
+// the workgroups of a 1-D grid in id order on every XCD. Correctness does not rest on that order: a look-back
+// that has polled a window kSpinLimit times without an answer (milliseconds; a running predecessor answers in
+// microseconds) stops waiting and HELPS: wave 0 reads the silent predecessor's input itself, reduces it and
+// uses that aggregate. Every tile therefore finishes on its own whatever the others do, the GPU never hangs
+// and the result is the same bits. (In place, a predecessor might finish and overwrite its input while it is
+// being helped: the helper polls the tile's status once more after its reads have returned and, if anything
+// has been published by then, takes the published value instead; a tile's first publication is complete
+// before any of its output stores are issued.) The flag kFlagTicket selects the reference's ticket order
+// instead, kFlagNoHelp the behaviour of a plain bounded wait: a wave that runs out stores the tile number plus
+// one into the workspace header (kHdrReport) and carries on with a wrong prefix; scan_status() reads that word
+// after the stream has drained and turns it into an error. The segmented and the 64-bit scans wait that way
+// always. scan_status() also reports a workspace that was never initialised (the header holds a magic word).
 //
 // Workspace protocol (no reset launch per call). Every tile owns TWO status words,
 // one per parity of the workspace's call counter. A call with parity p publishes
@@ -87,13 +88,17 @@ typedef unsigned long long u64;
 constexpr size_t kHeaderBytes = 256;
 enum : int {                // header fields, as indices of 32-bit words
     kHdrTicket = 0,         // ticket counter (ticket order only); 0 between calls
+    kHdrBadWorkspace = 1,   // a tile found no magic word or an impossible state: tile number + 1, sticky like kHdrReport
     kHdrReport = 2,         // look-back time-out report: tile number + 1, sticky until scan_status() reads it
-    kHdrDone = 3,           // tiles that have finished (segmented scan only); 0 between calls
+    kHdrDone = 3,           // tiles that have read the header (plain scan) / finished (segmented scan); 0 between calls
     kHdrCalls = 4,          // calls completed on this workspace; its low bit is the parity of the next call
     kHdrDirty0 = 5,         // tiles whose parity-0 words may be non-zero
     kHdrDirty1 = 6,         // same for parity 1
+    kHdrMagic = 7,          // kMagic once scan_workspace_init() has run (read together with words 4-6)
 };
-constexpr uint32_t kSpinLimit = 1u << 22;  // polls of one look-back window before giving up
+constexpr uint32_t kMagic = 0x5ca9b10cu;
+constexpr uint32_t kSpinLimit = 1u << 22;  // polls of one look-back window / of the closing tile's wait before giving up
+constexpr uint32_t kHelpAfter = 1u << 12;  // polls of one look-back window before a silent predecessor is helped
 
 // Tile shapes: {threads, 16 B packets per lane}.
 struct SmallCfg { static constexpr int BLOCK = 1024, VPT = 4; };
@@ -241,45 +246,89 @@ __device__ __forceinline__ void close_call(uint32_t* header, u32x4 hdr, uint32_t
     __hip_atomic_store(&header[kHdrCalls], calls + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-__device__ __forceinline__ void finish_status_protocol(uint32_t* header, u64* status, u32x4 hdr, uint32_t tile,
-                                                       uint32_t tiles, int lane) {
-    clear_other_parity(status, hdr, tile, tiles, lane);
-    // The last tile closes the call: every earlier tile has published by now (its look-back saw them
-    // all), so every tile has read the header.
-    if (tile == tiles - 1 && lane == 0) close_call(header, hdr, tiles);
+// The aggregate of one whole tile, formed by one wavefront from the tile's input: what a look-back does for a
+// predecessor that does not answer. Slow (one wavefront reads the whole tile) and rare.
+template <typename Op, bool VEC, int TILE>
+__device__ __forceinline__ uint32_t tile_aggregate(const uint32_t* in, size_t tile_base, int lane) {
+    // Two loads in flight and a loop that stays a loop: this code sits inside the look-back of every tile and
+    // must not cost the common path registers.
+    uint32_t acc = Op::identity;
+    if constexpr (VEC) {
+        const u32x4* src = reinterpret_cast<const u32x4*>(in + tile_base) + lane;
+#pragma unroll 1
+        for (int i = 0; i < TILE / 4 / kWave; i += 2) {
+            const u32x4 x = src[static_cast<size_t>(i) * kWave], y = src[static_cast<size_t>(i + 1) * kWave];
+            acc = Op::apply(acc, Op::apply(Op::apply(x.x, x.y), Op::apply(x.z, x.w)));
+            acc = Op::apply(acc, Op::apply(Op::apply(y.x, y.y), Op::apply(y.z, y.w)));
+        }
+    } else {
+        const uint32_t* src = in + tile_base + lane;
+#pragma unroll 1
+        for (int i = 0; i < TILE / kWave; i += 4) {
+            const uint32_t x0 = src[static_cast<size_t>(i) * kWave], x1 = src[static_cast<size_t>(i + 1) * kWave];
+            const uint32_t x2 = src[static_cast<size_t>(i + 2) * kWave], x3 = src[static_cast<size_t>(i + 3) * kWave];
+            acc = Op::apply(acc, Op::apply(Op::apply(x0, x1), Op::apply(x2, x3)));
+        }
+    }
+    return wave_last_lane(wave_inclusive_scan_op<Op>(acc));
 }
 
 // Exclusive prefix of tile `tile` (> 0): the sum of all earlier tiles. Run by
 // one whole wavefront; lane l inspects tile (window_end - l), whose status word
-// of this call's parity is status[2 * tile + parity]. Every tile below `tile` is
-// running or finished (see "Tile order" above) and will publish without waiting
-// for anything later, so the loop terminates; the spin limit is a guard, and
-// spin_limit == 0 gives up before the first poll (a host-side way to exercise the
-// way out).
-template <typename Op>
+// of this call's parity is status[2 * tile + parity]. A predecessor that is
+// running publishes within microseconds without waiting for anything later. One
+// that has not answered after spin_limit polls of its window is not waited for
+// any longer: with `help` the wavefront forms that tile's aggregate from the
+// input itself (tile_aggregate; see "Tile order" at the top for why that is also
+// right in place), so the loop always ends with the right sum; without `help`
+// it reports tile + 1 into *report and returns what it has. spin_limit == 0
+// skips the waiting altogether, which exercises either way out from the host.
+// A state that no tile ever writes means the workspace holds something else
+// (never initialised, or overwritten): reported into *bad_workspace.
+template <typename Op, bool VEC, int TILE>
 __device__ __forceinline__ uint32_t look_back(const u64* status, uint32_t parity, uint32_t tile, int lane,
-                                              uint32_t spin_limit, uint32_t* report) {
+                                              uint32_t spin_limit, bool help, const uint32_t* in, uint32_t* report,
+                                              uint32_t* bad_workspace) {
     uint32_t sum = Op::identity;
     uint32_t spins = 0;
     long long window_end = static_cast<long long>(tile) - 1;
     while (true) {
-        if (spins >= spin_limit) {
-            if (lane == 0) __hip_atomic_store(report, tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            break;
-        }
         const long long t = window_end - lane;
         // Tiles "before the first" count as a published prefix of nothing.
-        const u64 w = (t >= 0) ? poll(&status[2 * t + parity]) : pack_status(kPrefix, Op::identity);
-        const uint32_t state = static_cast<uint32_t>(w);
-        const uint32_t value = static_cast<uint32_t>(w >> 32);
-        const u64 has_prefix = __ballot(state == kPrefix);
-        const u64 is_invalid = __ballot(state == kInvalid);
-        // Lanes 0..first-prefix-lane are needed; all 64 when no prefix is in the window.
-        const u64 needed = has_prefix ? ((2ull << __builtin_ctzll(has_prefix)) - 1ull) : ~0ull;
-        if (is_invalid & needed) {
-            ++spins;  // no s_sleep: the wait for the poll's answer paces the loop (sleeping measured 1 % slower)
-            continue;
+        u64 w = (t >= 0) ? poll(&status[2 * t + parity]) : pack_status(kPrefix, Op::identity);
+        uint32_t state = static_cast<uint32_t>(w);
+        if (__ballot(state > kPrefix)) {
+            if (lane == 0) __hip_atomic_store(bad_workspace, tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
         }
+        u64 has_prefix = __ballot(state == kPrefix);
+        u64 is_invalid = __ballot(state == kInvalid);
+        // Lanes 0..first-prefix-lane are needed; all 64 when no prefix is in the window.
+        u64 needed = has_prefix ? ((2ull << __builtin_ctzll(has_prefix)) - 1ull) : ~0ull;
+        if (is_invalid & needed) {
+            if (spins < spin_limit) {
+                ++spins;  // no s_sleep: the wait for the poll's answer paces the loop (sleeping measured 1 % slower)
+                continue;
+            }
+            if (!help) {
+                if (lane == 0) __hip_atomic_store(report, tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                break;
+            }
+            for (u64 todo = is_invalid & needed; todo != 0; todo &= todo - 1) {
+                const int l = __builtin_ctzll(todo);
+                const uint32_t formed = tile_aggregate<Op, VEC, TILE>(in, static_cast<size_t>(window_end - l) * TILE, lane);
+                // Every read of that tile's input has returned (the reduction used them). If the tile has
+                // published anything by now, its word is the truth (in place, the input may be turning into
+                // output); if not, it has not stored any output yet and `formed` is the sum of its input.
+                const u64 again = poll(&status[2 * (window_end - l) + parity]);
+                if (lane == l) w = static_cast<uint32_t>(again) != kInvalid ? again : pack_status(kAggregate, formed);
+            }
+            state = static_cast<uint32_t>(w);
+            has_prefix = __ballot(state == kPrefix);
+            needed = has_prefix ? ((2ull << __builtin_ctzll(has_prefix)) - 1ull) : ~0ull;
+        }
+        spins = 0;
+        const uint32_t value = static_cast<uint32_t>(w >> 32);
         const uint32_t contrib = ((needed >> lane) & 1ull) ? value : Op::identity;
         sum = Op::apply(sum, wave_last_lane(wave_inclusive_scan_op<Op>(contrib)));
         if (has_prefix) break;
@@ -305,7 +354,7 @@ __device__ __forceinline__ void stream_store(u32x4* p, u32x4 v) {
 template <typename Cfg, bool VEC, bool TICKET, bool EXCLUSIVE, typename Op = SumOp>
 __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_t* in, uint32_t* out,
                                                                    size_t n, uint32_t* header,
-                                                                   u64* status, uint32_t spin_limit) {
+                                                                   u64* status, uint32_t spin_limit, bool help) {
     constexpr int BLOCK = Cfg::BLOCK, VPT = Cfg::VPT;
     constexpr int WAVES = BLOCK / kWave;
     constexpr int TILE = BLOCK * VPT * 4;
@@ -387,15 +436,42 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan_lookback_kernel(const uint32_
         const uint32_t parity = calls & 1u;
         u64* const mine = &status[2 * static_cast<size_t>(tile) + parity];
         uint32_t prefix = Op::identity;
-        if (tile == 0) {
-            if (lane == 0) publish(mine, kPrefix, aggregate);
+        if (hdr.w != kMagic) {
+            // Not a workspace scan_workspace_init() has seen: nothing in it can be trusted, so nothing is read
+            // or written beyond this report, and the output of the call is invalid.
+            if (lane == 0) __hip_atomic_store(&header[kHdrBadWorkspace], tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         } else {
-            if (lane == 0) publish(mine, kAggregate, aggregate);
-            prefix = look_back<Op>(status, parity, tile, lane, spin_limit, &header[kHdrReport]);
-            if (lane == 0) publish(mine, kPrefix, Op::apply(aggregate, prefix));
+            // Counted in before anything is published: the tile that closes the call waits for this count,
+            // because with helping its look-back can be complete before every tile has read the header.
+            if (lane == 0) __hip_atomic_fetch_add(&header[kHdrDone], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (tile == 0) {
+                if (lane == 0) publish(mine, kPrefix, aggregate);
+            } else {
+                if (lane == 0) publish(mine, kAggregate, aggregate);
+                prefix = look_back<Op, VEC, TILE>(status, parity, tile, lane, spin_limit, help, in, &header[kHdrReport],
+                                                  &header[kHdrBadWorkspace]);
+            }
+            // The first publication is complete (and with it every poll) before the second one and, behind the
+            // barrier below, the output stores are issued: a helper that finds this tile unpublished after its
+            // reads have returned has read input, not output.
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));
+            if (tile != 0 && lane == 0) publish(mine, kPrefix, Op::apply(aggregate, prefix));
+            clear_other_parity(status, hdr, tile, tiles, lane);
+            if (tile == tiles - 1 && lane == 0) {
+                // The last tile closes the call once every tile has read the header (normally all have: its
+                // look-back saw them published; only tiles it helped may be missing, and they need no one).
+                uint32_t spins = 0;
+                while (__hip_atomic_load(&header[kHdrDone], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != tiles) {
+                    if (++spins > kSpinLimit) {
+                        __hip_atomic_store(&header[kHdrReport], tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(8);
+                }
+                close_call(header, hdr, tiles);
+            }
         }
         if (lane == 0) s_tile_prefix = prefix;
-        finish_status_protocol(header, status, hdr, tile, tiles, lane);
     }
     __syncthreads();
     const uint32_t base_sum = Op::apply(s_tile_prefix, wave_prefix);
@@ -471,7 +547,7 @@ __device__ __forceinline__ u64 pack_seg_status(uint32_t state, Seg p) {
 // The pair that everything before tile `tile` (> 0) contributes to it. The walk back ends at the nearest
 // tile that has published a prefix or whose own range holds a head: what lies before a head does not matter.
 __device__ __forceinline__ Seg look_back_seg(const u64* status, uint32_t parity, uint32_t tile, int lane,
-                                             uint32_t spin_limit, uint32_t* report) {
+                                             uint32_t spin_limit, uint32_t* report, uint32_t* bad_workspace) {
     Seg sum{0u, 0u};
     uint32_t spins = 0;
     long long window_end = static_cast<long long>(tile) - 1;
@@ -485,6 +561,10 @@ __device__ __forceinline__ Seg look_back_seg(const u64* status, uint32_t parity,
         const uint32_t state = static_cast<uint32_t>(w) & 0xffu;
         const uint32_t flag = (static_cast<uint32_t>(w) >> 8) & 1u;
         const uint32_t value = static_cast<uint32_t>(w >> 32);
+        if (__ballot(state > kPrefix || (static_cast<uint32_t>(w) >> 9) != 0u)) {  // no tile writes such a word
+            if (lane == 0) __hip_atomic_store(bad_workspace, tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+        }
         const u64 is_invalid = __ballot(state == kInvalid);
         const u64 ends_walk = __ballot(state == kPrefix || flag != 0u);
         const int first_invalid = is_invalid ? __builtin_ctzll(is_invalid) : kWave;
@@ -616,17 +696,19 @@ __global__ __launch_bounds__(Cfg::BLOCK) void segmented_scan_lookback_kernel(con
         const uint32_t parity = hdr.x & 1u;
         u64* const mine = &status[2 * static_cast<size_t>(tile) + parity];
         Seg prefix{0u, 0u};
-        if (tile == 0) {
+        if (hdr.w != kMagic) {  // not an initialised workspace: report, touch nothing else
+            if (lane == 0) __hip_atomic_store(&header[kHdrBadWorkspace], tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else if (tile == 0) {
             if (lane == 0) __hip_atomic_store(mine, pack_seg_status(kPrefix, aggregate), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         } else {
             if (lane == 0) __hip_atomic_store(mine, pack_seg_status(kAggregate, aggregate), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            prefix = look_back_seg(status, parity, tile, lane, spin_limit, &header[kHdrReport]);
+            prefix = look_back_seg(status, parity, tile, lane, spin_limit, &header[kHdrReport], &header[kHdrBadWorkspace]);
             if (lane == 0)
                 __hip_atomic_store(mine, pack_seg_status(kPrefix, seg_combine(prefix, aggregate)), __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
         }
         if (lane == 0) s_tile_prefix_v = prefix.v;
-        clear_other_parity(status, hdr, tile, tiles, lane);
+        if (hdr.w == kMagic) clear_other_parity(status, hdr, tile, tiles, lane);
     }
     __syncthreads();
     // What comes before this wave: the tile's prefix, unless a head in an earlier wave of the tile cuts it off.
@@ -657,7 +739,7 @@ __global__ __launch_bounds__(Cfg::BLOCK) void segmented_scan_lookback_kernel(con
     // A look-back that ended at a head says nothing about the tiles before that head, so the last tile's
     // look-back cannot tell that every tile has read the header. Tiles count themselves off instead, and
     // the one that counts last closes the call.
-    if (tid == 0) {
+    if (tid == 0 && hdr.w == kMagic) {
         const uint32_t done = __hip_atomic_fetch_add(&header[kHdrDone], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (done == tiles - 1) close_call(header, hdr, tiles);
     }
@@ -697,7 +779,7 @@ __device__ __forceinline__ void publish64(u64* lo_word, uint32_t state, u64 valu
 
 // Sum of all tiles before `tile` (> 0). Lane l inspects tile window_end - l: slots 2 t and 2 t + 1.
 __device__ __forceinline__ u64 look_back64(const u64* status, uint32_t parity, uint32_t tile, int lane, uint32_t spin_limit,
-                                           uint32_t* report) {
+                                           uint32_t* report, uint32_t* bad_workspace) {
     u64 sum = 0;
     uint32_t spins = 0;
     long long window_end = static_cast<long long>(tile) - 1;
@@ -710,6 +792,10 @@ __device__ __forceinline__ u64 look_back64(const u64* status, uint32_t parity, u
         const u64 lo = (t >= 0) ? poll(&status[4 * t + parity]) : pack_status(kPrefix, 0u);
         const u64 hi = (t >= 0) ? poll(&status[4 * t + 2 + parity]) : pack_status(kPrefix, 0u);
         const uint32_t state_lo = static_cast<uint32_t>(lo), state_hi = static_cast<uint32_t>(hi);
+        if (__ballot(state_lo > kPrefix || state_hi > kPrefix)) {  // no tile writes such a word
+            if (lane == 0) __hip_atomic_store(bad_workspace, tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+        }
         // halves of two different publications (or one still missing) count as "nothing yet"
         const uint32_t state = state_lo == state_hi ? state_lo : kInvalid;
         const u64 value = (lo >> 32) | (hi & 0xffffffff00000000ull);
@@ -795,18 +881,24 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan64_lookback_kernel(const u64* 
         const uint32_t parity = hdr.x & 1u;
         u64* const mine = &status[4 * static_cast<size_t>(tile) + parity];
         u64 prefix = 0;
-        if (tile == 0) {
-            if (lane == 0) publish64(mine, kPrefix, aggregate);
+        if (hdr.w != kMagic) {  // not an initialised workspace: report, touch nothing else
+            if (lane == 0) __hip_atomic_store(&header[kHdrBadWorkspace], tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         } else {
-            if (lane == 0) publish64(mine, kAggregate, aggregate);
-            prefix = look_back64(status, parity, tile, lane, spin_limit, &header[kHdrReport]);
-            if (lane == 0) publish64(mine, kPrefix, aggregate + prefix);
+            if (tile == 0) {
+                if (lane == 0) publish64(mine, kPrefix, aggregate);
+            } else {
+                if (lane == 0) publish64(mine, kAggregate, aggregate);
+                prefix = look_back64(status, parity, tile, lane, spin_limit, &header[kHdrReport], &header[kHdrBadWorkspace]);
+                if (lane == 0) publish64(mine, kPrefix, aggregate + prefix);
+            }
+            // The workspace protocol counts status slots: this tile's are 2 t and 2 t + 1 of 2 * tiles. The last
+            // tile closes the call: every earlier tile has published by now (its look-back saw them all), so
+            // every tile has read the header.
+            clear_other_parity(status, hdr, 2 * tile, 2 * tiles, lane);
+            clear_other_parity(status, hdr, 2 * tile + 1, 2 * tiles, lane);
+            if (tile == tiles - 1 && lane == 0) close_call(header, hdr, 2 * tiles);
         }
         if (lane == 0) s_tile_prefix = prefix;
-        // The workspace protocol counts status slots: this tile's are 2 t and 2 t + 1 of 2 * tiles.
-        clear_other_parity(status, hdr, 2 * tile, 2 * tiles, lane);
-        clear_other_parity(status, hdr, 2 * tile + 1, 2 * tiles, lane);
-        if (tile == tiles - 1 && lane == 0) close_call(header, hdr, 2 * tiles);
     }
     __syncthreads();
     const u64 base = s_tile_prefix + wave_prefix;
@@ -830,10 +922,11 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan64_lookback_kernel(const u64* 
     }
 }
 
-// Zero fill of a workspace (a kernel, not hipMemsetAsync, so that it can be captured into a graph).
+// Initial state of a workspace: all zeros but for the magic word of the header (a kernel, not hipMemsetAsync, so
+// that it can be captured into a graph). Words 6 and 7 of the header share 64-bit word 3.
 __global__ __launch_bounds__(256) void scan_fill_zero_kernel(u64* words, size_t n_words) {
     const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
-    if (i < n_words) words[i] = 0ull;
+    if (i < n_words) words[i] = (i == kHdrMagic / 2) ? (static_cast<u64>(kMagic) << 32) : 0ull;
 }
 
 inline bool use_small(size_t n, bool vec) { return n <= kSmallMax || !vec; }
@@ -851,15 +944,16 @@ int launch_cfg(const uint32_t* in, uint32_t* out, size_t n, uint32_t* header, u6
     const size_t tiles = ceil_div(n, static_cast<size_t>(tile_elems<Cfg>()));
     const dim3 grid(static_cast<unsigned>(tiles)), block(Cfg::BLOCK);
     const int op = static_cast<int>(flags & kFlagOpMask);
+    const bool help = (flags & kFlagNoHelp) == 0;
     if (op == kFlagOpMax)
-        scan_lookback_kernel<Cfg, VEC, false, false, MaxI32Op><<<grid, block, 0, s>>>(in, out, n, header, status, limit);
+        scan_lookback_kernel<Cfg, VEC, false, false, MaxI32Op><<<grid, block, 0, s>>>(in, out, n, header, status, limit, help);
     else if (op == kFlagOpMin)
-        scan_lookback_kernel<Cfg, VEC, false, false, MinI32Op><<<grid, block, 0, s>>>(in, out, n, header, status, limit);
+        scan_lookback_kernel<Cfg, VEC, false, false, MinI32Op><<<grid, block, 0, s>>>(in, out, n, header, status, limit, help);
     else
         with_flag((flags & kFlagTicket) != 0, [&](auto ticket) {
             with_flag((flags & kFlagExclusive) != 0, [&](auto excl) {
                 scan_lookback_kernel<Cfg, VEC, decltype(ticket)::value, decltype(excl)::value>
-                    <<<grid, block, 0, s>>>(in, out, n, header, status, limit);
+                    <<<grid, block, 0, s>>>(in, out, n, header, status, limit, help);
             });
         });
     return check_launch("scan_lookback_kernel");
@@ -872,7 +966,7 @@ int launch_cfg(const uint32_t* in, uint32_t* out, size_t n, uint32_t* header, u6
 // address hipGetSymbolAddress returns, never the array's name.
 constexpr size_t kStaticMaxElems = size_t{1} << 31;
 constexpr size_t kStaticBytes = kHeaderBytes + 16 * (kStaticMaxElems / kWorkspaceTileElems + 1);
-static __device__ __align__(256) unsigned char scratch[kStaticBytes];  // zero at load = initialised
+static __device__ __align__(256) unsigned char scratch[kStaticBytes];  // initialised by the first call on a device
 
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
@@ -889,6 +983,11 @@ int static_scratch(void** ptr, hipStream_t s) {
     if (dev < 0 || dev >= kMaxDevices) return fail(1, "prism_scan: device %d outside the supported range", dev);
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
     if (g_scratch_ptr[dev] == nullptr) {
+        // The one-time set-up must not end up in a graph (its fill would run again on every replay).
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &capturing) == hipSuccess && capturing != hipStreamCaptureStatusNone)
+            return fail(1, "prism_scan_i32_static: the first call on a device sets the library's scratch array up and must be "
+                           "made outside stream capture (prism_scan_status(NULL, 0, stream) does it as well)");
         void* p = nullptr;
         e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
         if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
@@ -931,7 +1030,7 @@ int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws
     if ((reinterpret_cast<uintptr_t>(ws) & 15u) != 0)
         return fail(1, "prism_scan: workspace must be 16-byte aligned");
     const int op = static_cast<int>(flags & kFlagOpMask);
-    if ((flags & ~(kFlagExclusive | kFlagTicket | kFlagOpMask)) != 0 || op > kFlagOpMin)
+    if ((flags & ~(kFlagExclusive | kFlagTicket | kFlagNoHelp | kFlagOpMask)) != 0 || op > kFlagOpMin)
         return fail(1, "prism_scan: unknown flag bits 0x%x", flags);
     if (op != kFlagOpSum && (flags & (kFlagExclusive | kFlagTicket)) != 0)
         return fail(1, "prism_scan: the running maximum / minimum is inclusive and numbers tiles by workgroup id");
@@ -946,7 +1045,7 @@ int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws
             return fail(1, "prism_scan: in and out overlap without being equal");
     }
     if (ceil_div(n, kWorkspaceTileElems) > 0x7fffffffull) return fail(1, "prism_scan: n=%zu too large", n);
-    const uint32_t limit = spin_limit < 0 ? kSpinLimit
+    const uint32_t limit = spin_limit < 0 ? ((flags & kFlagNoHelp) ? kSpinLimit : kHelpAfter)
                                           : static_cast<uint32_t>(spin_limit > 0xffffffffll ? 0xffffffffll : spin_limit);
 
     uint32_t* header = reinterpret_cast<uint32_t*>(ws);
@@ -1034,18 +1133,24 @@ int scan_status(void* ws, size_t ws_bytes, hipStream_t s) {
     if (ws_bytes < kHeaderBytes + 16) return fail(1, "prism_scan_status: workspace of %zu bytes is too small", ws_bytes);
     hipError_t e = hipStreamSynchronize(s);
     if (e != hipSuccess) return hip_fail(e, "prism_scan_status: hipStreamSynchronize");
-    uint32_t report = 0;
-    e = hipMemcpy(&report, static_cast<const uint32_t*>(ws) + kHdrReport, sizeof(report), hipMemcpyDeviceToHost);
+    uint32_t hdr[8] = {};
+    e = hipMemcpy(hdr, ws, sizeof(hdr), hipMemcpyDeviceToHost);
     if (e != hipSuccess) return hip_fail(e, "prism_scan_status: hipMemcpy");
-    if (report == 0) return 0;
-    // A tile gave up waiting: its call's output is invalid, and the tile that closes a call may have done
-    // so before every tile had started. Bring the workspace back to its initial state.
+    const bool bad_workspace = hdr[kHdrMagic] != kMagic || hdr[kHdrBadWorkspace] != 0;
+    const uint32_t report = hdr[kHdrReport];
+    if (!bad_workspace && report == 0) return 0;
+    // The output of the call that reported is invalid, and the workspace may be in any state (the tile that
+    // closes a call may have done so before every tile had started). Bring it back to its initial state.
     if (int rc = scan_workspace_init(ws, ws_bytes, s)) return rc;
     e = hipStreamSynchronize(s);
     if (e != hipSuccess) return hip_fail(e, "prism_scan_status: hipStreamSynchronize");
+    if (bad_workspace)
+        return fail(kScanWorkspaceError,
+                    "prism_scan: the workspace was not initialised with prism_scan_workspace_init (or something else "
+                    "wrote into it); the output of the scans that used it is invalid. It is initialised now");
     return fail(kScanOrderError,
-                "prism_scan: tile %u gave up waiting for its predecessors (workgroups did not start in the assumed "
-                "order, or the spin limit was set too low); the output of that call is invalid",
+                "prism_scan: tile %u gave up waiting for its predecessors (a scan without helping whose workgroups did "
+                "not start in the assumed order, or a spin limit set too low); the output of that call is invalid",
                 report - 1u);
 }
 

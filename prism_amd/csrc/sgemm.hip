@@ -841,13 +841,22 @@ __global__ __launch_bounds__(256) void sgemm_stream_k_fixup_kernel(int M, int N,
     xcd_tile_coords(first_tile_number + static_cast<int>(tile), tiles_m, tiles_n, tm, tn);
     const int row = tm * BM + r, col = tn * BN + c;
     if (row >= M || col >= N) return;  // N is a multiple of 4: a packet is inside or outside
+    // Four partial products are fetched at a time (the loads are independent of each other), then added in order.
+    const float* mine = ws + static_cast<size_t>(r) * BN + c;
     f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (u64 w = w0; w <= w1; ++w) {
-        const u64 begins = w * total / groups;
-        if (begins == (w + 1) * total / groups) continue;  // a workgroup without a share wrote nothing
-        const u64 slot = 2 * w + (begins / kt != tile ? 1u : 0u);
-        const f32x4 p = *reinterpret_cast<const f32x4*>(ws + slot * static_cast<size_t>(BM * BN) + static_cast<size_t>(r) * BN + c);
-        sum += p;
+    for (u64 w = w0; w <= w1; w += 4) {
+        f32x4 p[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            p[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            const u64 begins = (w + u) * total / groups;
+            // past the tile's last workgroup, or a workgroup without a share (it wrote nothing): adds +0
+            if (w + u > w1 || begins == (w + u + 1) * total / groups) continue;
+            const u64 slot = 2 * (w + u) + (begins / kt != tile ? 1u : 0u);
+            p[u] = *reinterpret_cast<const f32x4*>(mine + slot * static_cast<size_t>(BM * BN));
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) sum += p[u];
     }
     f32x4* out = reinterpret_cast<f32x4*>(C + static_cast<size_t>(row) * N + col);
     f32x4 res;
@@ -1223,9 +1232,19 @@ __global__ __launch_bounds__(256) void sgemm_thin_columns_kernel(int M, int N, i
     for (int k0 = 0; k0 < K; k0 += KC) {
         const int kc = K - k0 < KC ? K - k0 : KC;
         __syncthreads();  // the strip of the chunk before is no longer read
-        for (int e = threadIdx.x; e < kc * R; e += 256) {
-            const int k = e / R, j = e % R;
-            strip[e] = j < r ? B[static_cast<size_t>(k0 + k) * N + n0 + j] : 0.0f;
+        // only the r real columns are fetched (the others' sums are never stored); four loads in flight per thread
+        for (int e0 = threadIdx.x; e0 < kc * r; e0 += 4 * 256) {
+            float b[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int e = e0 + u * 256;
+                b[u] = e < kc * r ? B[static_cast<size_t>(k0 + e / r) * N + n0 + e % r] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int e = e0 + u * 256;
+                if (e < kc * r) strip[(e / r) * R + e % r] = b[u];
+            }
         }
         __syncthreads();
         // four steps of 64 k at a time: 4 * PER_WAVE loads in flight per lane

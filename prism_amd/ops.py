@@ -98,12 +98,18 @@ def wave_regroup(inp: "torch.Tensor", items_per_lane: int, to_striped: bool = Tr
 
 SCAN_EXCLUSIVE = 1       # flag values of include/prism_amd.h
 SCAN_TICKET_ORDER = 2
+SCAN_NO_HELP = 4
 SCAN_OP = {"sum": 0x00, "max": 0x10, "min": 0x20}
 ERROR_SCAN_ORDER = 10001
+ERROR_SCAN_WORKSPACE = 10002
 
 
 class ScanOrderError(PrismError):
     """A tile of a scan gave up waiting for its predecessors; that call's output is invalid."""
+
+
+class ScanWorkspaceError(PrismError):
+    """A scan ran on a workspace that was never initialised (or was overwritten); its output is invalid."""
 
 
 def get_workspace_size(n: int) -> int:
@@ -118,8 +124,8 @@ def _ws_bytes(workspace: "torch.Tensor") -> int:
 
 
 def new_scan_workspace(n: int, device="cuda") -> "torch.Tensor":
-    """An initialised (zero-filled) workspace for scans of up to n elements."""
-    return torch.zeros(get_workspace_size(n), dtype=torch.uint8, device=device)
+    """An initialised workspace for scans of up to n elements (the fill is enqueued on the current stream)."""
+    return scan_workspace_init(torch.empty(get_workspace_size(n), dtype=torch.uint8, device=device))
 
 
 def scan_workspace_init(workspace: "torch.Tensor") -> "torch.Tensor":
@@ -130,10 +136,13 @@ def scan_workspace_init(workspace: "torch.Tensor") -> "torch.Tensor":
 
 
 def scan_status(workspace: "torch.Tensor", stream: Optional[int] = None) -> None:
-    """Wait for the stream and raise ScanOrderError if a scan on this workspace gave up in its look-back."""
+    """Wait for the stream; raise ScanWorkspaceError if a scan found the workspace uninitialised, ScanOrderError
+    if one that does not help its predecessors gave up in its look-back."""
     rc = _lib.load().prism_scan_status(_ptr(workspace), _ws_bytes(workspace), _stream() if stream is None else stream)
     if rc == ERROR_SCAN_ORDER:
         raise ScanOrderError(_lib.last_error())
+    if rc == ERROR_SCAN_WORKSPACE:
+        raise ScanWorkspaceError(_lib.last_error())
     _check(rc, "scan_status")
 
 
@@ -160,21 +169,23 @@ def launch_scan(n: int, x: "torch.Tensor", workspace: "torch.Tensor", check: boo
 
 def scan(inp: "torch.Tensor", out: Optional["torch.Tensor"] = None,
          workspace: Optional["torch.Tensor"] = None, exclusive: bool = False, op: str = "sum",
-         ticket_order: bool = False, spin_limit: int = -1, check: bool = True) -> "torch.Tensor":
+         ticket_order: bool = False, spin_limit: int = -1, check: bool = True, help: bool = True) -> "torch.Tensor":
     """Prefix sum modulo 2^32 of a 1-D int32/uint32 tensor (modulo 2^64 of an int64/uint64 one); out may be inp. Inclusive (out[i] includes
     inp[i]) unless exclusive=True (out[0] = 0, out[i] = inp[0] + ... + inp[i-1]). op="max" / op="min": the
     running maximum / minimum of an int32 tensor instead (inclusive only).
 
     workspace: an initialised workspace (new_scan_workspace / scan_workspace_init) that calls on one stream
     may share; None allocates one. ticket_order numbers tiles by the reference's ticket counter instead of
-    by workgroup id; spin_limit bounds the look-back polls (-1: library default, 0: give up at once).
-    check=True (default) waits for the result and raises ScanOrderError if the look-back gave up;
-    check=False leaves the call asynchronous and the check (scan_status) to the caller.
+    by workgroup id; spin_limit bounds the polls of a look-back window before the tile helps a silent
+    predecessor (-1: library default, 0: no waiting); help=False makes a look-back that runs out of polls
+    report instead (ScanOrderError), the plain bounded wait. check=True (default) waits for the result and
+    raises if the workspace was uninitialised or such a look-back gave up; check=False leaves the call
+    asynchronous and the check (scan_status) to the caller.
     """
     if op not in SCAN_OP:
         raise ValueError("scan: op must be 'sum', 'max' or 'min'")
     if inp.dtype in (torch.int64, torch.uint64):  # 64-bit elements: inclusive sums modulo 2^64 only
-        if op != "sum" or exclusive or ticket_order or spin_limit != -1:
+        if op != "sum" or exclusive or ticket_order or spin_limit != -1 or not help:
             raise ValueError("scan: 64-bit elements support the inclusive sum in workgroup-id order only")
         n = inp.numel()
         if out is None:
@@ -195,7 +206,8 @@ def scan(inp: "torch.Tensor", out: Optional["torch.Tensor"] = None,
     _need(out, (inp.dtype,), n, "out")
     if workspace is None:
         workspace = new_scan_workspace(n, inp.device)
-    flags = SCAN_OP[op] | (SCAN_EXCLUSIVE if exclusive else 0) | (SCAN_TICKET_ORDER if ticket_order else 0)
+    flags = (SCAN_OP[op] | (SCAN_EXCLUSIVE if exclusive else 0) | (SCAN_TICKET_ORDER if ticket_order else 0)
+             | (0 if help else SCAN_NO_HELP))
     _check(_lib.load().prism_scan_i32_ex(_ptr(inp), _ptr(out), n, _ptr(workspace), _ws_bytes(workspace), flags,
                                          int(spin_limit), _stream()), "scan")
     if check and n > 0:

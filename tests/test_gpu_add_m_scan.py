@@ -223,11 +223,40 @@ def test_scan_ticket_order_matches_dispatch_order(prism, oracle, n):
         assert np.array_equal(host(out), want), ticket
 
 
-def test_scan_that_gives_up_is_an_error(prism, oracle):
-    """With the spin limit forced to 0 every look-back gives up before its first poll: the kernel must
-    still finish (the point of the bound), and the failure must be loud: scan() raises, and so does
-    scan_status() after an unchecked call. Afterwards the same workspace serves exact scans again and
-    reports nothing."""
+def test_scan_that_stops_waiting_helps_its_predecessors(prism, oracle):
+    """With the spin limit forced to 0 no look-back waits: a predecessor that has not published when it is polled
+    is helped at once, i.e. wave 0 of the waiting tile forms that tile's sum from the input. Every tile then
+    finishes on its own, so the bits must be exact whatever the tiles' timing: both tile shapes, 16 B- and 4
+    B-aligned views, inclusive, exclusive and running maximum, workgroup-id and ticket order, and IN PLACE, where
+    a helped predecessor may be turning its input into output meanwhile (the helper's second poll decides).
+    Nothing is reported, and the workspace serves ordinary calls in between."""
+    for n in ((1 << 22) + 77, (1 << 26) + 65536 * 5 + 3):
+        x = oracle.gen_scan(n, seed=n % 1000)
+        inc, exc, mx = oracle.scan_cpu(x), oracle.scan_exclusive_cpu(x), oracle.scan_max_cpu(x)
+        xd = dev(x)
+        ws = prism.new_scan_workspace(n)
+        out = torch.empty_like(xd)
+        for kw, want in (({}, inc), ({"ticket_order": True}, inc), ({"exclusive": True}, exc), ({"op": "max"}, mx)):
+            print(f"scan n={n} spin_limit=0 {kw}", flush=True)
+            prism.scan(xd, out, ws, spin_limit=0, **kw)
+            assert np.array_equal(host(out), want), kw
+            prism.scan(xd, out, ws, **kw)
+            assert np.array_equal(host(out), want), kw
+        for _ in range(3):  # in place
+            buf = xd.clone()
+            prism.scan(buf, buf, ws, spin_limit=0)
+            assert np.array_equal(host(buf), inc)
+        view_in, view_out = dev(np.concatenate([[5], x]).astype(np.int32))[1:], torch.empty(n + 3, dtype=torch.int32, device=DEV)[3:]
+        prism.scan(view_in, view_out, ws, spin_limit=0)  # 4-byte-aligned views: the small tile, element-wise loads
+        assert np.array_equal(host(view_out), inc)
+        prism.scan_status(ws)
+
+
+def test_scan_without_helping_that_gives_up_is_an_error(prism, oracle):
+    """The plain bounded wait (help=False, PRISM_SCAN_NO_HELP) with the spin limit forced to 0: every look-back
+    gives up before it has waited at all. The kernel must still finish (the point of the bound), and the failure
+    must be loud: scan() raises, and so does scan_status() after an unchecked call. Afterwards the same workspace
+    serves exact scans again and reports nothing."""
     n = 1 << 26
     x = oracle.gen_scan(n, seed=3)
     want = oracle.scan_cpu(x)
@@ -236,8 +265,8 @@ def test_scan_that_gives_up_is_an_error(prism, oracle):
     ws = prism.new_scan_workspace(n)
     for ticket in (True, False):
         with pytest.raises(prism.ScanOrderError, match="gave up waiting"):
-            prism.scan(xd, out, ws, ticket_order=ticket, spin_limit=0)
-        prism.scan(xd, out, ws, ticket_order=ticket, spin_limit=0, check=False)  # asynchronous, unchecked
+            prism.scan(xd, out, ws, ticket_order=ticket, spin_limit=0, help=False)
+        prism.scan(xd, out, ws, ticket_order=ticket, spin_limit=0, help=False, check=False)  # asynchronous, unchecked
         with pytest.raises(prism.ScanOrderError):
             prism.scan_status(ws)
         prism.scan_status(ws)  # the report was consumed and the workspace re-initialised
@@ -247,6 +276,71 @@ def test_scan_that_gives_up_is_an_error(prism, oracle):
     # the reference-shaped launcher checks as well (through the library: no spin limit to force here)
     prism.launch_scan(n, xd, ws)
     assert np.array_equal(host(xd), want)
+
+
+def test_scan_on_a_workspace_that_was_never_initialised_is_an_error(prism, oracle):
+    """A workspace straight from the allocator (here: filled with 0xFF, and once with zeros, which is not the
+    initial state either): every kind of scan must leave it alone, exit normally and be reported by
+    scan_status() as PRISM_ERROR_SCAN_WORKSPACE; the status call initialises the workspace, after which the same
+    buffer serves exact scans."""
+    n = (1 << 24) + 5
+    x = oracle.gen_scan(n, seed=9)
+    want = oracle.scan_cpu(x)
+    xd = dev(x)
+    out = torch.empty_like(xd)
+    heads = torch.zeros(n, dtype=torch.uint8, device=DEV)
+    for fill in (0xFF, 0x00):
+        ws = torch.full((prism.get_workspace_size(n) + 64,), fill, dtype=torch.uint8, device=DEV)[:prism.get_workspace_size(n)]
+        runs = (lambda: prism.scan(xd, out, ws, check=False), lambda: prism.scan(xd, out, ws, check=False, ticket_order=True),
+                lambda: prism.segmented_scan(xd, heads, out, ws, check=False),
+                lambda: prism.scan(xd.to(torch.int64), None, ws, check=False))
+        for run in runs:
+            ws.fill_(fill)
+            print(f"scan on a workspace filled with {fill:#x}", flush=True)
+            run()
+            torch.cuda.synchronize()
+            body = ws[32:]  # nothing but the report word of the header was written
+            assert bool((body == fill).all())
+            with pytest.raises(prism.ScanWorkspaceError, match="not initialised"):
+                prism.scan_status(ws)
+            prism.scan_status(ws)
+            prism.scan(xd, out, ws)
+            assert np.array_equal(host(out), want)
+
+
+def test_scan_while_another_stream_keeps_the_gpu_busy(prism, oracle):
+    """Scans of 2^28 elements while a second stream (default priority) runs long SGEMMs that compete for every
+    CU: workgroups of the scan then start whenever the other kernel leaves room, in no particular rhythm.
+    The bits must be exact and nothing may be reported, in workgroup-id order (the default) and in ticket order."""
+    n = 1 << 28
+    g = torch.Generator(device=DEV)
+    g.manual_seed(0)
+    xd = torch.randint(-1000, 1001, (n,), dtype=torch.int32, device=DEV, generator=g)
+    out = torch.empty_like(xd)
+    ws = prism.new_scan_workspace(n)
+    prism.scan(xd, out, ws)
+    want = out.clone()
+    assert int(want[-1]) == ((int(xd.sum(dtype=torch.int64)) + 2**31) % 2**32) - 2**31
+    assert bool(torch.equal(want[1:] - want[:-1], xd[1:]))
+    M = 4096
+    A = torch.rand((M, M), device=DEV)
+    B = torch.rand((M, M), device=DEV)
+    C = torch.zeros((M, M), device=DEV)
+    side = torch.cuda.Stream()  # default priority
+    torch.cuda.synchronize()
+    for ticket in (False, True):
+        with torch.cuda.stream(side):
+            for variant in (3, 6, 3, 6, 3, 6):  # 7 ms and 2 ms apiece: about 30 ms of competing work
+                prism.sgemm(M, M, M, 1.0, A, B, 0.0, C, variant=variant)
+        for rep in range(12):
+            out.zero_()
+            print(f"scan 2^28 beside SGEMMs on another stream, ticket_order={ticket}, repeat {rep}", flush=True)
+            prism.scan(xd, out, ws, ticket_order=ticket, check=False)
+        prism.scan_status(ws)
+        assert torch.equal(out, want)
+        side.synchronize()
+        prism.scan(xd, out, ws, ticket_order=ticket)
+        assert torch.equal(out, want)
 
 
 def test_scan_workspace_shared_by_calls_of_any_length_and_kind(prism, oracle):
