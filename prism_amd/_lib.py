@@ -8,7 +8,7 @@ from __future__ import annotations
 import ctypes as C
 import threading
 
-from .build import LIB_PATH, ensure_built
+from .build import LIB_PATH, ensure_built, ensure_vendor_built
 
 # name -> (restype, argtypes); must list every function include/prism_amd.h declares.
 SIGNATURES = {
@@ -64,8 +64,34 @@ def load() -> C.CDLL:
     return _lib
 
 
+# The vendor-baseline library (prism_amd/csrc/vendor/vendor_baselines.hip): hipCUB, rocBLAS and hipBLASLt behind
+# plain C entry points, for the evaluation sweeps and their tests. Not part of include/prism_amd.h.
+VENDOR_SIGNATURES = {
+    "vendor_scan_temp_bytes": (C.c_int, [C.c_size_t, C.POINTER(C.c_size_t)]),
+    "vendor_scan_inclusive_sum": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "vendor_sgemm": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_void_p]),
+    "vendor_gemm_bf16_f32": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "vendor_gemm_bf16_colmajor": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+}
+_vendor = None
+
+
+def load_vendor() -> C.CDLL:
+    """Load (building first if the file is absent) the vendor-baseline library."""
+    global _vendor
+    with _lock:
+        if _vendor is None:
+            lib = C.CDLL(str(ensure_vendor_built()))
+            for name, (restype, argtypes) in VENDOR_SIGNATURES.items():
+                fn = getattr(lib, name)
+                fn.restype = restype
+                fn.argtypes = argtypes
+            _vendor = lib
+    return _vendor
+
+
 def last_error() -> str:
     return load().prism_last_error_string().decode("utf-8", "replace")
 
 
-__all__ = ["load", "last_error", "SIGNATURES", "LIB_PATH"]
+__all__ = ["load", "load_vendor", "last_error", "SIGNATURES", "VENDOR_SIGNATURES", "LIB_PATH"]

@@ -76,5 +76,23 @@ def ensure_built() -> Path:
     return LIB_PATH
 
 
+# The vendor libraries behind plain C entry points (hipCUB, rocBLAS, hipBLASLt called directly): the baselines of
+# the evaluation sweeps. A library of its own, so that libprism_amd.so links nothing but the HIP runtime.
+VENDOR_LIB_PATH = PKG_DIR / "libprism_vendor_baselines.so"
+
+
+def build_vendor_baselines(verbose: bool = False) -> Path:
+    _run([hipcc_path(), *HIPCC_FLAGS, "-shared", "-o", str(VENDOR_LIB_PATH), str(CSRC / "vendor" / "vendor_baselines.hip"),
+          "-lrocblas", "-lhipblaslt"], verbose)
+    return VENDOR_LIB_PATH
+
+
+def ensure_vendor_built() -> Path:
+    if not VENDOR_LIB_PATH.exists():
+        build_vendor_baselines()
+    return VENDOR_LIB_PATH
+
+
 if __name__ == "__main__":
     print(build(verbose=True))
+    print(build_vendor_baselines(verbose=True))

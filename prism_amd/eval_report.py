@@ -15,9 +15,10 @@ prints can be fed to the reference's plotting script unchanged:
   h100   evals/h100_bench/main.cu:112-167     8 back-to-back launches between two events, TFLOPS;
          lines "Kernel: ..." / "cuBLAS: ..." (parsed by plot_results.py:18-34)
 
-The vendor-library slots ("cuBLAS", "CUB") are filled with what the ROCm stack
-offers through PyTorch: rocBLAS/hipBLASLt `torch.matmul` and rocPRIM
-`torch.cumsum`. They are comparison lines, like the reference's.
+The vendor-library slots ("cuBLAS", "CUB") are filled by the ROCm libraries called directly, the way the
+harnesses call theirs: rocblas_sgemm, a hipBLASLt bf16 matmul and hipcub::DeviceScan::InclusiveSum, behind the
+C entry points of prism_amd/csrc/vendor/vendor_baselines.hip (a library of its own, built by prism_amd.build).
+They are comparison lines, like the reference's.
 
 `generated` runs the same protocols over the kernels that prism_amd.hipgen prints from the example programs
 (prism_amd/examples), which is what the reference's figures show for its own back-end: "My Kernel" 1..5 are
@@ -89,10 +90,16 @@ def _best_wall_ms(fn, target_ms: float) -> float:
 
 # ----------------------------------------------------------------- sweeps --
 
+def _ok(rc: int) -> None:
+    if rc != 0:
+        raise RuntimeError(f"a vendor-library call failed with code {rc}")
+
+
 def sweep_sgemm(out=sys.stdout, sizes=SGEMM_SIZES, repeats: int = 10) -> None:
     import torch
     from . import _lib
-    lib = _lib.load()
+    lib, vendor = _lib.load(), _lib.load_vendor()
+    stream = torch.cuda.current_stream().cuda_stream
     alpha, beta = 0.5, 3.0
     top = max(sizes)
     A = torch.rand((top, top), device="cuda") * 2 - 1
@@ -104,10 +111,11 @@ def sweep_sgemm(out=sys.stdout, sizes=SGEMM_SIZES, repeats: int = 10) -> None:
         c = C.flatten()[: n * n].view(n, n).clone()
         flops = 2.0 * n * n * n
         print(f"\n====================================\nSize: {n}x{n}x{n}\n====================================", file=out)
-        print("\n[cuBLAS FP32]", file=out)  # slot of the vendor BLAS: rocBLAS/hipBLASLt through torch
+        print("\n[cuBLAS FP32]", file=out)  # slot of the vendor BLAS: rocblas_sgemm, called as runner.cu:124-132 calls cuBLAS
         ref = c.clone()
-        torch.addmm(ref, a, b, beta=beta, alpha=alpha, out=ref)
-        ms = _events_ms(lambda: torch.addmm(ref, a, b, beta=beta, alpha=alpha, out=ref), repeats)
+        vend = lambda: vendor.vendor_sgemm(n, n, n, alpha, a.data_ptr(), b.data_ptr(), beta, ref.data_ptr(), stream)
+        _ok(vend())
+        ms = _events_ms(vend, repeats)
         print(sgemm_line(ms / 1e3 / repeats, repeats * flops * 1e-9 / (ms / 1e3), n), file=out)
         for k in (1, 2, 3, 4, 5):
             print(f"\n[My Kernel {k}]", file=out)
@@ -120,13 +128,20 @@ def sweep_sgemm(out=sys.stdout, sizes=SGEMM_SIZES, repeats: int = 10) -> None:
 
 
 def sweep_scan(out=sys.stdout, log2_sizes=SCAN_LOG2_SIZES, target_ms: float = 500.0) -> None:
+    import ctypes
+
     import torch
     from . import _lib
-    lib = _lib.load()
+    lib, vendor_lib = _lib.load(), _lib.load_vendor()
     top = 1 << max(log2_sizes)
     x = torch.randint(0, 101, (top,), dtype=torch.int32, device="cuda")  # U{0..100}, scan_harness.cuh:172
     work = torch.empty_like(x)
     ws = torch.empty(lib.prism_scan_workspace_bytes(top), dtype=torch.uint8, device="cuda")
+    # hipcub::DeviceScan::InclusiveSum with its temporary storage allocated once, outside the timed region
+    # (evals/4090_scan/bench.cu:96-116); it scans out of place, from the pristine input into the work buffer
+    need = ctypes.c_size_t(0)
+    _ok(vendor_lib.vendor_scan_temp_bytes(top, ctypes.byref(need)))
+    temp = torch.empty(max(need.value, 16), dtype=torch.uint8, device="cuda")
     print(scan_header(), file=out)
     for p in log2_sizes:
         n = 1 << p
@@ -135,7 +150,7 @@ def sweep_scan(out=sys.stdout, log2_sizes=SCAN_LOG2_SIZES, target_ms: float = 50
         def ours():
             lib.prism_launch_scan(n, buf.data_ptr(), ws.data_ptr())
         def vendor():
-            torch.cumsum(xin, 0, dtype=torch.int32, out=buf)
+            _ok(vendor_lib.vendor_scan_inclusive_sum(xin.data_ptr(), buf.data_ptr(), n, temp.data_ptr(), temp.numel(), None))
         results = []
         for fn in (vendor, ours):
             best, elapsed = float("inf"), 0.0
@@ -158,7 +173,7 @@ def sweep_scan(out=sys.stdout, log2_sizes=SCAN_LOG2_SIZES, target_ms: float = 50
 def sweep_h100(out=sys.stdout, sizes=H100_SIZES, repeats: int = 8) -> None:
     import torch
     from . import _lib
-    lib = _lib.load()
+    lib, vendor = _lib.load(), _lib.load_vendor()
     for n in sizes:
         A = torch.randn((n, n), device="cuda").to(torch.bfloat16)
         B = torch.randn((n, n), device="cuda").to(torch.bfloat16)
@@ -168,12 +183,14 @@ def sweep_h100(out=sys.stdout, sizes=H100_SIZES, repeats: int = 8) -> None:
         fn()
         ms = _events_ms(fn, repeats)
         print(h100_line("Kernel:", ms / 1e3 / repeats, repeats * flops * 1e-9 / ms, n), file=out)
-        vend = lambda: torch.matmul(A, B.T)
-        vend()
+        # hipBLASLt, same operands and the same bf16 column-major result as the harness asks of cuBLAS (main.cu:64-73)
+        Cv = torch.empty_like(Cc)
+        vend = lambda: vendor.vendor_gemm_bf16_colmajor(n, n, n, A.data_ptr(), B.data_ptr(), Cv.data_ptr(), None)
+        _ok(vend())
         ms = _events_ms(vend, repeats)
         print(h100_line("cuBLAS:", ms / 1e3 / repeats, repeats * flops * 1e-9 / ms, n) + "\n", file=out)
         out.flush()
-        del A, B, Cc
+        del A, B, Cc, Cv
 
 
 def sweep_generated(out=sys.stdout, sgemm_sizes=SGEMM_SIZES, scan_log2_sizes=SCAN_LOG2_SIZES, h100_sizes=H100_SIZES,
@@ -184,9 +201,10 @@ def sweep_generated(out=sys.stdout, sgemm_sizes=SGEMM_SIZES, scan_log2_sizes=SCA
 
     import torch
 
-    from . import examples, hipgen
+    from . import _lib, examples, hipgen
     examples.load()
     built = {}
+    vendor_lib = _lib.load_vendor()
 
     def kernel(name):
         if name not in built:
@@ -218,8 +236,9 @@ def sweep_generated(out=sys.stdout, sgemm_sizes=SGEMM_SIZES, scan_log2_sizes=SCA
         print(f"\n====================================\nSize: {n}x{n}x{n}\n====================================", file=out)
         print("\n[cuBLAS FP32]", file=out)
         ref = c.clone()
-        torch.addmm(ref, a, b, beta=beta, alpha=alpha, out=ref)
-        ms = _events_ms(lambda: torch.addmm(ref, a, b, beta=beta, alpha=alpha, out=ref), repeats)
+        vend = lambda: vendor_lib.vendor_sgemm(n, n, n, alpha, a.data_ptr(), b.data_ptr(), beta, ref.data_ptr(), None)
+        _ok(vend())
+        ms = _events_ms(vend, repeats)
         print(sgemm_line(ms / 1e3 / repeats, repeats * flops * 1e-9 / (ms / 1e3), n), file=out)
         for k, (name, smallest, last, blocks) in steps.items():
             if k == 5 and n >= big5[1] and n % 2048 == 0:
@@ -245,6 +264,9 @@ def sweep_generated(out=sys.stdout, sgemm_sizes=SGEMM_SIZES, scan_log2_sizes=SCA
     work = torch.empty_like(x)
     counter = torch.zeros(1, dtype=torch.int32, device="cuda")
     status = torch.zeros(top // 65536, dtype=torch.int64, device="cuda")
+    need = ctypes.c_size_t(0)
+    _ok(vendor_lib.vendor_scan_temp_bytes(top, ctypes.byref(need)))
+    temp = torch.empty(max(need.value, 16), dtype=torch.uint8, device="cuda")
     print("\n" + scan_header(), file=out)
     for p in scan_log2_sizes:
         n = 1 << p
@@ -257,7 +279,7 @@ def sweep_generated(out=sys.stdout, sgemm_sizes=SGEMM_SIZES, scan_log2_sizes=SCA
                 raise RuntimeError("lookback_scan_striped failed to launch")
 
         def vendor():
-            torch.cumsum(xin, 0, dtype=torch.int32, out=buf)
+            _ok(vendor_lib.vendor_scan_inclusive_sum(xin.data_ptr(), buf.data_ptr(), n, temp.data_ptr(), temp.numel(), None))
         results = [_best_wall_ms(fn, target_ms) for fn in (vendor, ours)]
         bytes_ = n * 4 * 2
         print(scan_row(n, results[0], bytes_ / results[0] / 1e6, results[1], bytes_ / results[1] / 1e6), file=out)
@@ -280,8 +302,8 @@ def sweep_generated(out=sys.stdout, sgemm_sizes=SGEMM_SIZES, scan_log2_sizes=SCA
             raise RuntimeError(f"{name} failed to launch at {n}")
         ms = _events_ms(fn, 8)
         print(h100_line("Kernel:", ms / 1e3 / 8, 8 * flops * 1e-9 / ms, n), file=out)
-        vend = lambda: torch.matmul(P, Q.T)
-        vend()
+        vend = lambda: vendor_lib.vendor_gemm_bf16_f32(n, n, n, P.data_ptr(), Q.data_ptr(), D.data_ptr(), None)
+        _ok(vend())
         ms = _events_ms(vend, 8)
         print(h100_line("cuBLAS:", ms / 1e3 / 8, 8 * flops * 1e-9 / ms, n) + "\n", file=out)
         out.flush()

@@ -94,3 +94,58 @@ def test_sweeps_over_generated_kernels_produce_parseable_reports():
     rows = parse_scan_table(text)
     assert [r[0] for r in rows] == [1 << 20, 1 << 22] and all(r[1] > 0 and r[2] > 0 for r in rows)
     assert re.search(H100_KERNEL, text) and re.search(H100_VENDOR, text)
+
+
+def test_vendor_baseline_library_builds_and_exports_its_entry_points():
+    """hipCUB, rocBLAS and hipBLASLt behind plain C entry points: a library of its own, every symbol typed."""
+    from prism_amd import _lib
+    lib = _lib.load_vendor()
+    for name in _lib.VENDOR_SIGNATURES:
+        assert hasattr(lib, name)
+
+
+@pytest.mark.gpu
+def test_vendor_baselines_compute_what_the_sweeps_compare_with(oracle):
+    """The vendor-library calls are handed operands in this repository's layouts (row-major fp32; bf16 A M x K and
+    B N x K; the harness's column-major bf16 result): their results must be the same products the library's own
+    kernels are checked against, or the comparison lines of the sweeps would time something else."""
+    import ctypes
+
+    import numpy as np
+    import torch
+    from prism_amd import _lib
+    v = _lib.load_vendor()
+    dev = "cuda:0"
+    # scan: exact
+    n = (1 << 22) + 1234
+    x = oracle.gen_scan(n, seed=1)
+    xd = torch.from_numpy(x).to(dev)
+    out = torch.empty_like(xd)
+    need = ctypes.c_size_t(0)
+    assert v.vendor_scan_temp_bytes(n, ctypes.byref(need)) == 0
+    temp = torch.empty(max(need.value, 16), dtype=torch.uint8, device=dev)
+    assert v.vendor_scan_inclusive_sum(xd.data_ptr(), out.data_ptr(), n, temp.data_ptr(), temp.numel(), None) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), oracle.scan_cpu(x))
+    # sgemm: a ragged, non-square shape shows a transposed operand or a swapped dimension
+    M, N, K = 200, 328, 136
+    A, B, Cm = oracle.gen_sgemm(M, N, K, seed=2)
+    c = torch.from_numpy(Cm).to(dev)
+    assert v.vendor_sgemm(M, N, K, 0.5, torch.from_numpy(A).to(dev).data_ptr(), torch.from_numpy(B).to(dev).data_ptr(), 3.0,
+                          c.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    assert np.max(np.abs(c.cpu().numpy() - oracle.sgemm_f64(0.5, A, B, 3.0, Cm))) <= oracle.sgemm_tolerance(K, A, B) + 3.0 * 2**-22
+    # bf16: fp32 row-major result and bf16 column-major result
+    M, N, K = 192, 320, 136
+    A16, B16 = oracle.gen_gemm_bf16(M, N, K, seed=3)
+    a = torch.from_numpy(A16.view(np.int16)).to(dev)
+    b = torch.from_numpy(B16.view(np.int16)).to(dev)
+    ref = oracle.gemm_bf16_f64(A16, B16)
+    d = torch.empty((M, N), dtype=torch.float32, device=dev)
+    assert v.vendor_gemm_bf16_f32(M, N, K, a.data_ptr(), b.data_ptr(), d.data_ptr(), None) == 0
+    cc = torch.empty(N * M, dtype=torch.int16, device=dev)
+    assert v.vendor_gemm_bf16_colmajor(M, N, K, a.data_ptr(), b.data_ptr(), cc.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    assert np.max(np.abs(d.cpu().numpy() - ref)) <= 1e-3 * np.abs(ref).max()
+    got = oracle.bf16_to_f32(cc.cpu().numpy().view(np.uint16)).reshape(N, M).T
+    assert np.max(np.abs(got - ref)) <= 2.0**-8 * np.abs(ref).max()
