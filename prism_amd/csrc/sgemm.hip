@@ -1651,6 +1651,16 @@ int launch_sgemm_ws(int variant, int M, int N, int K, float alpha, const float* 
             const dim3 grid(static_cast<unsigned>(plan.groups));
             if (plan.bm == 64) {
                 const int tiles_m = M / 64, tiles_n = N / 256;
+                // K tiles of 32 when K allows: a workgroup streams its whole share of B once, and what it has in
+                // flight (one stage) is what hides the memory latency; 20 KiB (K tiles of 16) do not.
+                if (K % 32 == 0) {
+                    sgemm_wave_tile_dma_kernel<64, 256, 32, 32, 128, false, false, true><<<grid, dim3(256), 0, s>>>(
+                        M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, 0, parts, plan.sk_tiles);
+                    if (int rc = check_launch("sgemm_wave_tile_dma_kernel (K shared, 64 x 256 tiles)")) return rc;
+                    sgemm_stream_k_fixup_kernel<64, 256, 32><<<dim3(static_cast<unsigned>(plan.sk_tiles) * 16), dim3(256), 0, s>>>(
+                        M, N, K, alpha, beta, C, parts, tiles_m, tiles_n, 0, plan.sk_tiles, grid.x);
+                    return check_launch("sgemm_stream_k_fixup_kernel");
+                }
                 sgemm_wave_tile_dma_kernel<64, 256, 16, 32, 128, false, false, true><<<grid, dim3(256), 0, s>>>(
                     M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, 0, parts, plan.sk_tiles);
                 if (int rc = check_launch("sgemm_wave_tile_dma_kernel (K shared, 64 x 256 tiles)")) return rc;
