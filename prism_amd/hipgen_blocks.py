@@ -27,8 +27,10 @@ statement sits in one); a loop whose body would meet such a hazard with its own 
 barrier at the end of the body. What a call does to an array it is handed is read off the callee's signature
 (a pointer to const is only read, :871-940), and a `ptr(shared(T))` parameter is an LDS array of its own
 (:151-158); a pointer that a call returns is not followed. A barrier is never placed inside an `if` (threads
-may disagree on the branch): the hazard is resolved in front of the `if`, and one that lies wholly inside an
-`if` is an error; the reference walks into branches (:424-447). For programs in the shapes of the reference's
+may disagree on the branch): the hazard is resolved in front of the `if`. One that lies wholly inside an `if`
+gets its barrier inside when the condition is the same for every thread of the workgroup (it names nothing but
+numbers, grid- or block-level parameters and variables, and the variables of loops over such ranges), as the
+reference does for any branch (it walks into branches, :424-447); inside any other `if` it is an error. For programs in the shapes of the reference's
 LDS-tiled SGEMMs, its kernel 5 and its scan this gives the barriers the reference prints
 (generated/sgemm_shared_mem_block.cu:38,42, my_sgemm_kernel_4.cu:48,65, my_sgemm_kernel_5.cu:41,46,
 scan_kernel.cu:17,19).
@@ -189,6 +191,20 @@ class _SyncPlan:
                     _is_call(n, "shared") or (_is_call(n, "ptr") and address_space_of(n) == "SHARED")
                     for n in ast.walk(_annotation(a.annotation)[0])):
                 self.root[a.arg] = a.arg
+        # names whose value is the same for every thread of a workgroup: parameters and variables declared at
+        # grid or block perspective (the perspective rules keep thread-level values out of them), and, while the
+        # walk is inside them, the variables of loops over ranges of such values
+        self.uniform: Set[str] = set()
+        for a in fn.args.args:
+            if a.arg != "template" and a.annotation is not None:
+                level = _annotation(a.annotation)[1]
+                if level is not None and level[0] in ("grid", "block"):
+                    self.uniform.add(a.arg)
+        for n in ast.walk(fn):
+            if isinstance(n, ast.AnnAssign) and isinstance(n.target, ast.Name):
+                level = _annotation(n.annotation)[1]
+                if level is not None and level[0] in ("grid", "block"):
+                    self.uniform.add(n.target.id)
         self._collect(fn.body)
         self._plan_handovers(fn.body)
         self._walk(fn.body, (set(), set()), True)
@@ -356,6 +372,23 @@ class _SyncPlan:
                 for case in s.cases:
                     self._plan_handovers(case.body)
 
+    def _block_uniform(self, node: Optional[ast.AST]) -> bool:
+        """True when the expression is built from numbers, names in self.uniform, arithmetic and comparisons
+        only: no call (id() differs from thread to thread), no memory access."""
+        if node is None:
+            return True
+        for n in ast.walk(node):
+            if isinstance(n, ast.Name):
+                if n.id not in self.uniform:
+                    return False
+            elif isinstance(n, ast.Constant):
+                if not isinstance(n.value, (int, float, bool)):
+                    return False
+            elif not isinstance(n, (ast.BinOp, ast.UnaryOp, ast.BoolOp, ast.Compare, ast.operator, ast.unaryop,
+                                    ast.boolop, ast.cmpop, ast.expr_context)):
+                return False
+        return True
+
     @staticmethod
     def _hazard(r: Set[str], w: Set[str], pending: Tuple[Set[str], Set[str]]) -> bool:
         pr, pw = pending
@@ -382,7 +415,15 @@ class _SyncPlan:
                     pr, pw = set(), set()
                 pr |= self._reads(s.iter if isinstance(s, ast.For) else s.test)
                 before_loop = (set(pr), set(pw))
+                # the variable of a loop over a range of workgroup-uniform values is uniform inside the loop
+                loop_var = (s.target.id if isinstance(s, ast.For) and isinstance(s.target, ast.Name) and may_sync
+                            and s.target.id not in self.uniform and _is_call(s.iter, "range")
+                            and all(self._block_uniform(a) for a in s.iter.args) else None)
+                if loop_var is not None:
+                    self.uniform.add(loop_var)
                 pr, pw = self._walk(s.body, (pr, pw), may_sync)
+                if loop_var is not None:
+                    self.uniform.discard(loop_var)
                 if self._probe(s.body, (pr, pw)) == "hazard":
                     if not may_sync:
                         raise HipgenError(f"{_line(s)}: a loop inside an `if` needs a barrier between its iterations")
@@ -399,11 +440,14 @@ class _SyncPlan:
                 if self._hazard(r, w, (pr, pw)):
                     self._mark(s, may_sync, self._reason(r, w, (pr, pw)))
                     pr, pw = set(), set()
-                # Inside the branches (or the cases of a split) no barrier may be placed: not every thread
-                # gets there. Hazards inside are errors.
+                # Inside the cases of a split, and inside an `if` on which the threads of a workgroup may
+                # disagree, no barrier may be placed: not every thread gets there, and a hazard inside is an
+                # error. An `if` whose condition is the same for the whole workgroup is entered by all of its
+                # threads or by none, so a hazard that lies wholly inside gets its barrier inside.
                 bodies = [s.body, s.orelse] if isinstance(s, ast.If) else [c.body for c in s.cases]
+                inside = may_sync and isinstance(s, ast.If) and self._block_uniform(s.test)
                 for body in bodies:
-                    a = self._walk(body, (set(), set()), False)
+                    a = self._walk(body, (set(), set()), inside)
                     pr |= a[0]
                     pw |= a[1]
                 pr |= r
@@ -726,10 +770,34 @@ class BlockEmitter:
         self.emit(f"__builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&{src}), "
                   f"(__attribute__((address_space(3))) void*)(&{dst}), 16, 0, 0);")
 
+    # kinds of instructions a scheduling group may name -> mask bits of __builtin_amdgcn_sched_group_barrier
+    _SCHED_KINDS = {"mfma": 0x008, "valu": 0x002, "salu": 0x004, "vmem": 0x010, "vmem_read": 0x020, "vmem_write": 0x040,
+                    "lds": 0x080, "lds_read": 0x100, "lds_write": 0x200, "any": 0x000}
+
+    def sched_group(self, n: ast.Call) -> None:
+        """`intrinsic.sched_group("lds_read", 4)`: the next scheduling group holds 4 LDS reads. A run of such
+        statements behind a stretch of straight-line code states the order in which the compiler's scheduler is
+        to interleave that stretch's instructions (LDS reads, matrix instructions, loads), which is what the
+        hand-written kernels' pipelines rest on; `intrinsic.sched_group("barrier")` keeps the scheduler from
+        moving anything across the statement. Prints __builtin_amdgcn_sched_group_barrier / sched_barrier; the
+        reference has no counterpart (its tensor-core path issues whole tiles per instruction)."""
+        a = n.args
+        if len(a) == 1 and isinstance(a[0], ast.Constant) and a[0].value == "barrier" and not n.keywords:
+            return self.emit("__builtin_amdgcn_sched_barrier(0);")
+        if (len(a) not in (2, 3) or n.keywords or not all(isinstance(x, ast.Constant) for x in a)
+                or a[0].value not in self._SCHED_KINDS or not isinstance(a[1].value, int) or a[1].value < 1
+                or (len(a) == 3 and not isinstance(a[2].value, int))):
+            raise HipgenError(f"{_line(n)}: intrinsic.sched_group(kind, count[, id]) with kind one of "
+                              f"{', '.join(sorted(self._SCHED_KINDS))}, or intrinsic.sched_group(\"barrier\")")
+        self.emit(f"__builtin_amdgcn_sched_group_barrier({self._SCHED_KINDS[a[0].value]:#05x}, {a[1].value}, "
+                  f"{a[2].value if len(a) == 3 else 0});")
+
     def matrix_instruction(self, n: ast.Call) -> None:
         name = n.func.attr
         if name == "load_to_lds":
             return self.load_to_lds(n)
+        if name == "sched_group":
+            return self.sched_group(n)
         if name not in _MFMA:
             raise HipgenError(f"{_line(n)}: intrinsic.{name} is not an instruction of this target "
                               f"(available: {', '.join(sorted(_MFMA))})")

@@ -17,7 +17,7 @@ from prism_amd import hipgen
 from prism_amd.examples import add_m, basics, mfma, scan, sgemm  # noqa: F401  (define the kernels)
 from prism_amd.hipgen import (HipgenError, block, const, generate, generate_launcher, grid, group, intrinsic, partition, prism,
                               ptr, requires, shared, split, thread)
-from prism_amd.hipgen_blocks import dynamic_lds_bytes
+from prism_amd.hipgen_blocks import dynamic_lds_bytes, explain_barriers
 
 
 @requires(grid[1], block[1], thread[1])
@@ -47,6 +47,24 @@ def split_with_hazard(x: ptr(float) @ grid[1]):
                         with group(thread[1]):
                             buf_mine[t] = x_mine[t]
                             x_mine[t] = buf[127 - t]
+
+
+@requires(grid[1], block[1], thread[1])
+@prism("global")
+def hazard_in_uniform_branch(x: ptr(float) @ grid[1], rounds: int @ grid[1]):
+    """The same write-then-read of LDS, inside an `if` on which all threads of a workgroup agree (a loop variable
+    over a grid-level range against a grid-level parameter), reversed once per round."""
+    with partition(x, p=thread[1], offset=0) as x_mine:
+        with group(block[1]):
+            buf: shared(float[64], static=True) @ block[1]
+            t: int @ thread[1] = id()
+            with partition(buf, p=thread[1], offset=t) as slot:
+                with group(thread[1]):
+                    for r in range(rounds):
+                        if r % 2 == 0:
+                            slot[0] = x_mine[t]
+                            x_mine[t] = buf[63 - t]
+                        intrinsic.sched_group("barrier")
 
 
 @requires(grid[1], block[1], thread[48])
@@ -332,6 +350,45 @@ def test_split_restarts_ids_in_every_case():
         generate("split_with_hazard")  # a barrier inside a case would not be reached by the other threads
 
 
+def test_a_hazard_inside_a_workgroup_uniform_if_gets_its_barrier_inside():
+    """The reference's pass walks into branches and places barriers there (prism/sync_analysis.py:424-447). Here that
+    is done when every thread of the workgroup takes the same side: the condition names only numbers, grid- or
+    block-level values and variables of loops over such ranges. The barrier stands between the store and the
+    read, inside the `if`; the loop then needs one more at the end of its body (the next round's store against
+    this round's read)."""
+    got = lines(generate("hazard_in_uniform_branch"))
+    at = got.index("if (((r % 2) == 0)) {")
+    assert got[at + 1] == "slot[0] = x_mine[t];" and got[at + 2] == "__syncthreads();" and got[at + 3] == "x_mine[t] = buf[(63 - t)];"
+    assert got[at + 4] == "}" and got[at + 5] == "__builtin_amdgcn_sched_barrier(0);" and got[at + 6] == "__syncthreads();"
+    assert got.count("__syncthreads();") == 2
+    why = explain_barriers("hazard_in_uniform_branch")
+    assert len(why) == 2 and "reads buf (written since the last barrier)" in why[0]
+
+
+def test_scheduling_group_statements():
+    @requires(grid[1], block[1], thread[1])
+    @prism("global")
+    def scheduled(x: ptr(float) @ grid[1]):
+        with group(block[1]):
+            intrinsic.sched_group("lds_read", 4)
+            intrinsic.sched_group("mfma", 8, 1)
+            intrinsic.sched_group("vmem_read", 1)
+            intrinsic.sched_group("barrier")
+
+    got = lines(generate("scheduled"))
+    assert got[got.index("__builtin_amdgcn_sched_group_barrier(0x100, 4, 0);") + 1] == "__builtin_amdgcn_sched_group_barrier(0x008, 8, 1);"
+    assert "__builtin_amdgcn_sched_group_barrier(0x020, 1, 0);" in got and "__builtin_amdgcn_sched_barrier(0);" in got
+
+    @requires(grid[1], block[1], thread[1])
+    @prism("global")
+    def badly_scheduled(x: ptr(float) @ grid[1]):
+        with group(block[1]):
+            intrinsic.sched_group("tensor", 4)
+
+    with pytest.raises(HipgenError, match="kind one of"):
+        generate("badly_scheduled")
+
+
 def test_refusals_name_the_construct():
     with pytest.raises(HipgenError, match="inside one `if`"):
         generate("hazard_in_branch")
@@ -577,3 +634,21 @@ def test_generated_lds_tiled_mfma_sgemm(built, oracle, shape):
     """LDS staging with the emitter's barriers around wavefront-wide matrix instructions."""
     M, N, K = shape
     run_sgemm(built["mfma_tile_sgemm"], "mfma_tile_sgemm", oracle, M, N, K, N // 64, (M // 64) * (N // 64))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rounds", [0, 1, 2, 3, 6])
+def test_generated_barrier_inside_a_uniform_if_runs(tmp_path_factory, rounds):
+    """hazard_in_uniform_branch reverses its 64 values through LDS once per even round, behind a barrier that
+    stands inside the `if`: wrong or missing barriers show as values from the wrong round."""
+    import torch
+    from prism_amd import hipgen
+    lib = hipgen.build("hazard_in_uniform_branch", out_dir=str(tmp_path_factory.mktemp("uniform_if")), block_size=64)
+    fn = lib.hazard_in_uniform_branch_launch
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_uint, ctypes.c_void_p]
+    x = np.arange(64, dtype=np.float32) * 1.5
+    xd = torch.from_numpy(x).to("cuda:0")
+    assert fn(xd.data_ptr(), rounds, 1, None) == 0
+    torch.cuda.synchronize()
+    want = x[::-1] if ((rounds + 1) // 2) % 2 else x
+    assert np.array_equal(xd.cpu().numpy(), want)
