@@ -741,7 +741,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
         for (int i = 0; i < MI; ++i)
 #pragma unroll
             for (int j = 0; j < NI; ++j) {
-                mfma_16x16x32_in_place(acc[i][j], fp[set][i], fq[set][j]);
+                mfma_16x16x32_in_place(acc[i][j], fq[set][j], fp[set][i]);  // Q first: see the write-back
                 __builtin_amdgcn_sched_barrier(0);
                 after(i * NI + j);
                 __builtin_amdgcn_sched_barrier(0);
@@ -855,46 +855,64 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < NI; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fp[2][i], fq[2][j], acc[i][j], 0, 0, 0);
-    // Write-back. Tiles that lie wholly inside the matrix (all of them unless EDGE) store without guards.
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fq[2][j], fp[2][i], acc[i][j], 0, 0, 0);
+    // Write-back. The matrix instructions are given the Q fragment first, i.e. they form the transposed
+    // sub-tile (Q rows) x (P rows): register v of lane l then holds OUT[row l % 16][column 4 (l / 16) + v] of
+    // the sub-tile, four consecutive columns, and a lane stores them as one packet (16 B of fp32, 8 B of bf16)
+    // instead of four separate elements. Tiles that lie wholly inside the matrix (all of them unless EDGE)
+    // store without guards; rows need only be aligned like their elements.
+    auto store_packet = [&](OutT* at, const f32x4& r) {
+        if constexpr (std::is_same<OutT, float>::value) {
+            typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+            *reinterpret_cast<f32x4_a4*>(at) = r;
+        } else {
+            typedef uint16_t u16x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+            *reinterpret_cast<u16x4_a2*>(at) = u16x4_a2{f32_to_bf16_rne(r[0]), f32_to_bf16_rne(r[1]), f32_to_bf16_rne(r[2]), f32_to_bf16_rne(r[3])};
+        }
+    };
     auto write_back = [&](auto guarded) {
 #pragma unroll
         for (int i = 0; i < MI; ++i) {
+            const int row = row0 + wave_m * WM + i * 16 + l16;
 #pragma unroll
             for (int j = 0; j < NI; ++j) {
-                const int col = col0 + wave_n * WN + j * 16 + l16;
+                const int col = col0 + wave_n * WN + j * 16 + 4 * lq;
+                OutT* at = &OUT[static_cast<size_t>(row) * Cn + col];
+                if constexpr (!guarded) {
+                    store_packet(at, acc[i][j]);
+                } else {  // tiles that hang over an edge: element by element
 #pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const int row = row0 + wave_m * WM + i * 16 + 4 * lq + v;
-                    if (!guarded || (row < R && col < Cn)) store_out(&OUT[static_cast<size_t>(row) * Cn + col], acc[i][j][v]);
+                    for (int v = 0; v < 4; ++v)
+                        if (row < R && col + v < Cn) store_out(at + v, acc[i][j][v]);
                 }
             }
         }
     };
     if constexpr (RAGGED) {
         // The k values the loop left out (K_all % 8 of them, at most 7) are added on the way out (load_k_tail
-        // above): a lane holds 32 rows x 8 columns. The product of two bf16 values is exact in fp32.
-        float qt[NI][7];
+        // above): a lane holds 8 rows x 32 columns (four consecutive ones per sub-tile). The product of two bf16
+        // values is exact in fp32.
+        float pt[MI][7];
 #pragma unroll
-        for (int j = 0; j < NI; ++j) load_k_tail(Q, ld, col0, Cn, col0 + wave_n * WN + j * 16 + l16, K, K_all, qt[j]);
+        for (int i = 0; i < MI; ++i) load_k_tail(P, ld, row0, R, row0 + wave_m * WM + i * 16 + l16, K, K_all, pt[i]);
 #pragma unroll
-        for (int i = 0; i < MI; ++i) {
-            float pt[4][7];
+        for (int j = 0; j < NI; ++j) {
+            const int col = col0 + wave_n * WN + j * 16 + 4 * lq;
+            float qt[4][7];
 #pragma unroll
-            for (int v = 0; v < 4; ++v) load_k_tail(P, ld, row0, R, row0 + wave_m * WM + i * 16 + 4 * lq + v, K, K_all, pt[v]);
+            for (int v = 0; v < 4; ++v) load_k_tail(Q, ld, col0, Cn, col + v, K, K_all, qt[v]);
 #pragma unroll
-            for (int j = 0; j < NI; ++j) {
-                const int col = col0 + wave_n * WN + j * 16 + l16;
+            for (int i = 0; i < MI; ++i) {
+                const int row = row0 + wave_m * WM + i * 16 + l16;
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
-                    const int row = row0 + wave_m * WM + i * 16 + 4 * lq + v;
                     float r = acc[i][j][v];
 #pragma unroll
-                    for (int t = 0; t < 7; ++t) r = __builtin_fmaf(pt[v][t], qt[j][t], r);
-                    if (row < R && col < Cn) store_out(&OUT[static_cast<size_t>(row) * Cn + col], r);
+                    for (int t = 0; t < 7; ++t) r = __builtin_fmaf(pt[i][t], qt[v][t], r);
+                    if (row < R && col + v < Cn) store_out(&OUT[static_cast<size_t>(row) * Cn + col + v], r);
                 }
             }
-            __builtin_amdgcn_sched_barrier(0);  // one row block at a time: its 28 P values and no more
+            __builtin_amdgcn_sched_barrier(0);  // one column block at a time: its 28 Q values and no more
         }
     } else {
         if (!EDGE || (row0 + BM <= R && col0 + BN <= Cn)) write_back(std::false_type{});

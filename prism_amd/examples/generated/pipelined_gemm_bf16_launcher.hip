@@ -92,11 +92,37 @@ __global__ __launch_bounds__(512) void pipelined_gemm_bf16(const __bf16* P, cons
                     for (int k0 = 0; k0 < K; k0 += 128) {
                         fill_stage_bf16(__block_id_1, __thread_id_1, __smem, second, P_rows, Q_rows, K, (k0 + 64));
                         multiply_stage_bf16(__block_id_1, __thread_id_1, __smem, acc, first);
-                        __syncthreads();
-                        if (((k0 + 128) < K)) {
-                            fill_stage_bf16(__block_id_1, __thread_id_1, __smem, first, P_rows, Q_rows, K, (k0 + 128));
+                        __builtin_amdgcn_sched_group_barrier(0x100, 5, 0);
+                        for (int g = 0; g < 7; g++) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
                         }
+                        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x100, 5, 0);
+                        for (int g = 0; g < 7; g++) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                        }
+                        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                        __syncthreads();
+                        fill_stage_bf16(__block_id_1, __thread_id_1, __smem, first, P_rows, Q_rows, K, ((k0 + 128) % K));
                         multiply_stage_bf16(__block_id_1, __thread_id_1, __smem, acc, second);
+                        __builtin_amdgcn_sched_group_barrier(0x100, 5, 0);
+                        for (int g = 0; g < 7; g++) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                        }
+                        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x100, 5, 0);
+                        for (int g = 0; g < 7; g++) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                        }
+                        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
                         __syncthreads();
                     }
                     {

@@ -174,11 +174,43 @@ def pipelined_gemm_bf16(P: ptr(const(bf16)) @ grid[1], Q: ptr(const(bf16)) @ gri
                     acc: float[128] @ thread[1] = {0}
                     fill_stage_bf16(first, P_rows, Q_rows, K, 0)
                     for k0 in range(0, K, 128):
+                        # A fill and the multiplication behind it are one stretch of straight-line code, and the
+                        # scheduling groups say how its instructions are to be interleaved: the 4 + 1 operand
+                        # reads the first matrix instructions need, then groups of four matrix instructions with
+                        # the next operand read and, in the first k-step, one of the fill's eight global loads
+                        # behind each (a burst of loads holds the wavefront, and the matrix pipe with it, at the
+                        # memory pipeline). Measured at 8192^3: 1156 TFLOP/s as the compiler orders it, 1280 so.
                         fill_stage_bf16(second, P_rows, Q_rows, K, k0 + 64)
                         multiply_stage_bf16(acc, first)
-                        if k0 + 128 < K:
-                            fill_stage_bf16(first, P_rows, Q_rows, K, k0 + 128)
+                        intrinsic.sched_group("lds_read", 5)
+                        for g in range(7):
+                            intrinsic.sched_group("mfma", 4)
+                            intrinsic.sched_group("lds_read", 1)
+                            intrinsic.sched_group("vmem_read", 1)
+                        intrinsic.sched_group("mfma", 4)
+                        intrinsic.sched_group("vmem_read", 1)
+                        intrinsic.sched_group("lds_read", 5)
+                        for g in range(7):
+                            intrinsic.sched_group("mfma", 4)
+                            intrinsic.sched_group("lds_read", 1)
+                        intrinsic.sched_group("mfma", 4)
+                        # The refill is not put under `if k0 + 128 < K`: a branch would end the stretch of code the
+                        # groups order. The last trip fetches the first K tile once more, into a stage nobody
+                        # reads again; the barrier at the end of the body waits for those loads as for all others.
+                        fill_stage_bf16(first, P_rows, Q_rows, K, (k0 + 128) % K)
                         multiply_stage_bf16(acc, second)
+                        intrinsic.sched_group("lds_read", 5)
+                        for g in range(7):
+                            intrinsic.sched_group("mfma", 4)
+                            intrinsic.sched_group("lds_read", 1)
+                            intrinsic.sched_group("vmem_read", 1)
+                        intrinsic.sched_group("mfma", 4)
+                        intrinsic.sched_group("vmem_read", 1)
+                        intrinsic.sched_group("lds_read", 5)
+                        for g in range(7):
+                            intrinsic.sched_group("mfma", 4)
+                            intrinsic.sched_group("lds_read", 1)
+                        intrinsic.sched_group("mfma", 4)
                     with partition(D_tile, p=thread[1], offset=0) as D_mine:
                         wave: int @ thread[64] = id()
                         with group(thread[64]):
