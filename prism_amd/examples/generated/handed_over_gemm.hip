@@ -61,13 +61,17 @@ __global__ void handed_over_gemm(const __bf16* P, const __bf16* Q, float* D, int
                                                     int k8 = (8 * (lane % 4));
                                                     {
                                                         int __spin = 0;
-                                                        for (; __spin < 65536 && __hip_atomic_load(&__empty_p_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_p_first * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                        const unsigned int __need = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__round_p_first * 4)));
+                                                        #pragma nounroll
+                                                        for (; __spin < 65536 && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__hip_atomic_load(&__empty_p_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)))) < __need; ++__spin) __builtin_amdgcn_s_sleep(1);
                                                         if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 1u | (static_cast<unsigned int>(__round_p_first) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                                                     }
                                                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                                                     {
                                                         int __spin = 0;
-                                                        for (; __spin < 65536 && __hip_atomic_load(&__empty_q_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_q_first * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                        const unsigned int __need = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__round_q_first * 4)));
+                                                        #pragma nounroll
+                                                        for (; __spin < 65536 && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__hip_atomic_load(&__empty_q_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)))) < __need; ++__spin) __builtin_amdgcn_s_sleep(1);
                                                         if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 5u | (static_cast<unsigned int>(__round_q_first) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                                                     }
                                                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -85,13 +89,17 @@ __global__ void handed_over_gemm(const __bf16* P, const __bf16* Q, float* D, int
                                                     __round_q_first += 1;
                                                     {
                                                         int __spin = 0;
-                                                        for (; __spin < 65536 && __hip_atomic_load(&__empty_p_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_p_second * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                        const unsigned int __need = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__round_p_second * 4)));
+                                                        #pragma nounroll
+                                                        for (; __spin < 65536 && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__hip_atomic_load(&__empty_p_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)))) < __need; ++__spin) __builtin_amdgcn_s_sleep(1);
                                                         if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 3u | (static_cast<unsigned int>(__round_p_second) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                                                     }
                                                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                                                     {
                                                         int __spin = 0;
-                                                        for (; __spin < 65536 && __hip_atomic_load(&__empty_q_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_q_second * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                        const unsigned int __need = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__round_q_second * 4)));
+                                                        #pragma nounroll
+                                                        for (; __spin < 65536 && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__hip_atomic_load(&__empty_q_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)))) < __need; ++__spin) __builtin_amdgcn_s_sleep(1);
                                                         if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 7u | (static_cast<unsigned int>(__round_q_second) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                                                     }
                                                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -123,7 +131,9 @@ __global__ void handed_over_gemm(const __bf16* P, const __bf16* Q, float* D, int
                                                     int k8 = (8 * (lane / 16));
                                                     {
                                                         int __spin = 0;
-                                                        for (; __spin < 65536 && __hip_atomic_load(&__full_p_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_p_first + 1) * 1); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                        const unsigned int __need = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>((__round_p_first + 1) * 1)));
+                                                        #pragma nounroll
+                                                        for (; __spin < 65536 && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__hip_atomic_load(&__full_p_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)))) < __need; ++__spin) __builtin_amdgcn_s_sleep(1);
                                                         if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 2u | (static_cast<unsigned int>(__round_p_first) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                                                     }
                                                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -134,7 +144,9 @@ __global__ void handed_over_gemm(const __bf16* P, const __bf16* Q, float* D, int
                                                     __round_p_first += 1;
                                                     {
                                                         int __spin = 0;
-                                                        for (; __spin < 65536 && __hip_atomic_load(&__full_q_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_q_first + 1) * 1); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                        const unsigned int __need = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>((__round_q_first + 1) * 1)));
+                                                        #pragma nounroll
+                                                        for (; __spin < 65536 && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__hip_atomic_load(&__full_q_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)))) < __need; ++__spin) __builtin_amdgcn_s_sleep(1);
                                                         if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 6u | (static_cast<unsigned int>(__round_q_first) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                                                     }
                                                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -157,7 +169,9 @@ __global__ void handed_over_gemm(const __bf16* P, const __bf16* Q, float* D, int
                                                     __round_q_first += 1;
                                                     {
                                                         int __spin = 0;
-                                                        for (; __spin < 65536 && __hip_atomic_load(&__full_p_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_p_second + 1) * 1); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                        const unsigned int __need = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>((__round_p_second + 1) * 1)));
+                                                        #pragma nounroll
+                                                        for (; __spin < 65536 && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__hip_atomic_load(&__full_p_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)))) < __need; ++__spin) __builtin_amdgcn_s_sleep(1);
                                                         if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 4u | (static_cast<unsigned int>(__round_p_second) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                                                     }
                                                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -168,7 +182,9 @@ __global__ void handed_over_gemm(const __bf16* P, const __bf16* Q, float* D, int
                                                     __round_p_second += 1;
                                                     {
                                                         int __spin = 0;
-                                                        for (; __spin < 65536 && __hip_atomic_load(&__full_q_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_q_second + 1) * 1); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                        const unsigned int __need = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>((__round_q_second + 1) * 1)));
+                                                        #pragma nounroll
+                                                        for (; __spin < 65536 && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__hip_atomic_load(&__full_q_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)))) < __need; ++__spin) __builtin_amdgcn_s_sleep(1);
                                                         if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 8u | (static_cast<unsigned int>(__round_q_second) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                                                     }
                                                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");

@@ -125,7 +125,9 @@ __global__ __launch_bounds__(768) void handed_over_sgemm(int M, int N, int K, fl
                                     if (__thread_id_2 >= 0 && __thread_id_2 < 256) {
                                         {
                                             int __spin = 0;
-                                            for (; __spin < 65536 && __hip_atomic_load(&__empty_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_first * 8); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                            const unsigned int __need = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__round_first * 8)));
+                                            #pragma nounroll
+                                            for (; __spin < 65536 && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__hip_atomic_load(&__empty_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)))) < __need; ++__spin) __builtin_amdgcn_s_sleep(1);
                                             if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 1u | (static_cast<unsigned int>(__round_first) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                                         }
                                         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -136,7 +138,9 @@ __global__ __launch_bounds__(768) void handed_over_sgemm(int M, int N, int K, fl
                                         __round_first += 1;
                                         {
                                             int __spin = 0;
-                                            for (; __spin < 65536 && __hip_atomic_load(&__empty_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>(__round_second * 8); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                            const unsigned int __need = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__round_second * 8)));
+                                            #pragma nounroll
+                                            for (; __spin < 65536 && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__hip_atomic_load(&__empty_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)))) < __need; ++__spin) __builtin_amdgcn_s_sleep(1);
                                             if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 3u | (static_cast<unsigned int>(__round_second) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                                         }
                                         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -153,7 +157,9 @@ __global__ __launch_bounds__(768) void handed_over_sgemm(int M, int N, int K, fl
                                     if (__thread_id_2 >= 0 && __thread_id_2 < 512) {
                                         {
                                             int __spin = 0;
-                                            for (; __spin < 65536 && __hip_atomic_load(&__full_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_first + 1) * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                            const unsigned int __need = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>((__round_first + 1) * 4)));
+                                            #pragma nounroll
+                                            for (; __spin < 65536 && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__hip_atomic_load(&__full_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)))) < __need; ++__spin) __builtin_amdgcn_s_sleep(1);
                                             if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 2u | (static_cast<unsigned int>(__round_first) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                                         }
                                         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -164,7 +170,9 @@ __global__ __launch_bounds__(768) void handed_over_sgemm(int M, int N, int K, fl
                                         __round_first += 1;
                                         {
                                             int __spin = 0;
-                                            for (; __spin < 65536 && __hip_atomic_load(&__full_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < static_cast<unsigned int>((__round_second + 1) * 4); ++__spin) __builtin_amdgcn_s_sleep(1);
+                                            const unsigned int __need = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>((__round_second + 1) * 4)));
+                                            #pragma nounroll
+                                            for (; __spin < 65536 && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__hip_atomic_load(&__full_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)))) < __need; ++__spin) __builtin_amdgcn_s_sleep(1);
                                             if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 4u | (static_cast<unsigned int>(__round_second) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                                         }
                                         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");

@@ -32,9 +32,10 @@ def test_waits_and_signals_of_the_producer_consumer_gemm():
     def events(start, stop):
         out = []
         for ln in got[start:stop]:
-            if ln.startswith("for (; __spin"):
+            if ln.startswith("const unsigned int __need = "):
+                need = ln.split("static_cast<int>(")[1].split(")));")[0]
+            elif ln.startswith("for (; __spin"):
                 word = ln.split("__hip_atomic_load(&__")[1].split(",")[0]
-                need = ln.split("static_cast<unsigned int>(")[1].split("); ++__spin")[0]
                 out.append(("wait", word, need))
             elif "__hip_atomic_fetch_add(&__" in ln:
                 out.append(("signal", ln.split("__hip_atomic_fetch_add(&__")[1].split(",")[0]))
@@ -67,8 +68,9 @@ def test_waits_and_signals_of_the_producer_consumer_gemm():
     # every wait is bounded, and one that runs out of polls reports it (array and round) into the file-scope word
     waits = [n for n, ln in enumerate(got) if ln.startswith("for (; __spin")]
     assert len(waits) == 8 and all("__spin < 65536 &&" in got[n] for n in waits)
-    assert all(got[n - 1] == "int __spin = 0;" and got[n + 1].startswith("if (__spin == 65536 && (threadIdx.x & 63) == 0) "
-               "__hip_atomic_store(&__prism_handover_report, ") for n in waits)
+    assert all(got[n - 3] == "int __spin = 0;" and got[n - 1] == "#pragma nounroll" and "__builtin_amdgcn_readfirstlane(" in got[n]
+               and got[n + 1].startswith("if (__spin == 65536 && (threadIdx.x & 63) == 0) "
+                                         "__hip_atomic_store(&__prism_handover_report, ") for n in waits)
     n = waits[0]   # first wait of the producer: array 0 (p_first), waiting for "empty" -> code 1
     assert "1u | (static_cast<unsigned int>(__round_p_first) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);" in got[n + 1]
     assert got[0] == "#ifndef PRISM_HANDOVER_REPORT" and "__device__ unsigned int __prism_handover_report = 0;" in got[:6]
@@ -146,11 +148,11 @@ def test_hand_over_through_device_functions():
     mults = [n for n, ln in enumerate(got) if ln.startswith("multiply_slot(")]
     assert len(fills) == 2 and len(mults) == 2
     for name, n in zip(("first", "second"), fills):   # wait until the eight readers are done, fill, count in
-        assert got[n - 4].startswith(f"for (; __spin < 65536 && __hip_atomic_load(&__empty_{name},")
-        assert f"__round_{name} * 8" in got[n - 4]
+        assert got[n - 4].startswith("for (; __spin < 65536 && ") and f"__hip_atomic_load(&__empty_{name}," in got[n - 4]
+        assert f"__round_{name} * 8" in got[n - 6]
         assert f"__hip_atomic_fetch_add(&__full_{name}, 1u" in got[n + 3] and got[n + 4] == f"__round_{name} += 1;"
     for name, n in zip(("first", "second"), mults):   # wait until the four writers are done, multiply, give back
-        assert f"__hip_atomic_load(&__full_{name}," in got[n - 4] and f"(__round_{name} + 1) * 4" in got[n - 4]
+        assert f"__hip_atomic_load(&__full_{name}," in got[n - 4] and f"(__round_{name} + 1) * 4" in got[n - 6]
         assert f"__hip_atomic_fetch_add(&__empty_{name}, 1u" in got[n + 3]
     loop = got.index("for (int k0 = 0; k0 < K; k0 += 128) {")
     assert got.count("__syncthreads();") == 2 and all(n < loop for n, ln in enumerate(got) if ln == "__syncthreads();")
@@ -191,6 +193,8 @@ def test_the_launcher_text_has_a_status_call_and_the_poll_bound_is_an_argument()
     big = hipgen.generate_launcher("handed_over_gemm_big", block_size=768)
     assert big.count("__device__ unsigned int __prism_handover_report = 0;") == 1 and "handed_over_gemm_big_status" in big
     # a kernel without hand-over has neither the word nor the call
+    from prism_amd import examples
+    examples.load()
     plain = hipgen.generate_launcher("tiled_sgemm", block_size=1024, template=[32])
     assert "__prism_handover_report" not in plain and "_status" not in plain
     none = hipgen.generate_launcher("handed_over_gemm", block_size=320, handover_spins=0)
