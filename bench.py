@@ -45,7 +45,7 @@ ROOT = Path(__file__).resolve().parent
 # Helpers shared with the tests live in tests/: the parity gate (fp64_referee), the tables under profiles/
 # (profile_tables) and the streaming calibration kernels (calibrate_stream).
 sys.path.insert(0, str(ROOT / "tests"))
-from profile_tables import measured_traffic, write_kernel_trace_table, write_traffic_table  # noqa: E402
+from profile_tables import measured_traffic, write_eval_tables, write_kernel_trace_table, write_traffic_table  # noqa: E402
 
 
 def log(*a):
@@ -252,6 +252,59 @@ def bench_gemm_bf16(prism, n, steps, warmup, gate=True):
                          "frac": tflops / PEAK["bf16_mfma_TFLOPs"], "traffic": measured_traffic("gemm_bf16", n)}}
 
 
+# ------------------------------------------------------- vendor libraries --
+
+def bench_vendor(steps, warmup):
+    """The ROCm libraries called directly (prism_amd/csrc/vendor/vendor_baselines.hip) on the headline problems,
+    timed like the workloads above, in the same run: rocblas_sgemm at 8192^3 (alpha 1, beta 0.5),
+    hipcub::DeviceScan::InclusiveSum at 2^30, hipBLASLt's bf16 matmul at 8192^3 with the fp32 row-major result of
+    prism_gemm_bf16 and with the bf16 column-major result of the reference's harness (prism_runmyh100's).
+    Comparison lines, like the cuBLAS / CUB lines of the reference's harnesses."""
+    import ctypes
+
+    import torch
+    from prism_amd import _lib
+    v, lib = _lib.load_vendor(), _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    out = {}
+
+    def checked(fn):
+        def call():
+            rc = fn()
+            return 0 if rc == 0 else 1
+        return call
+    n = 8192
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0)
+    A = torch.rand((n, n), device="cuda", generator=g) * 2 - 1
+    B = torch.rand((n, n), device="cuda", generator=g) * 2 - 1
+    C = torch.rand((n, n), device="cuda", generator=g) * 2 - 1
+    ms = time_steps(checked(lambda: v.vendor_sgemm(n, n, n, 1.0, A.data_ptr(), B.data_ptr(), 0.5, C.data_ptr(), st)), steps, warmup)
+    out["rocblas_sgemm_8192"] = {"ms": ms, "tflops": 2.0 * n ** 3 / ms / 1e9}
+    del A, B, C
+    P = torch.randn((n, n), device="cuda", generator=g).to(torch.bfloat16)
+    Q = torch.randn((n, n), device="cuda", generator=g).to(torch.bfloat16)
+    D = torch.empty((n, n), dtype=torch.float32, device="cuda")
+    Cc = torch.empty((n, n), dtype=torch.bfloat16, device="cuda")
+    ms = time_steps(checked(lambda: v.vendor_gemm_bf16_f32(n, n, n, P.data_ptr(), Q.data_ptr(), D.data_ptr(), st)), steps, warmup)
+    out["hipblaslt_bf16_8192_f32_out"] = {"ms": ms, "tflops": 2.0 * n ** 3 / ms / 1e9}
+    ms = time_steps(checked(lambda: v.vendor_gemm_bf16_colmajor(n, n, n, P.data_ptr(), Q.data_ptr(), Cc.data_ptr(), st)), steps, warmup)
+    out["hipblaslt_bf16_8192_bf16_colmajor_out"] = {"ms": ms, "tflops": 2.0 * n ** 3 / ms / 1e9}
+    ms = time_steps(lambda: lib.prism_runmyh100(n, n, n, P.data_ptr(), Q.data_ptr(), Cc.data_ptr(), None), steps, warmup)
+    out["ours_bf16_8192_bf16_colmajor_out"] = {"ms": ms, "tflops": 2.0 * n ** 3 / ms / 1e9, "entry": "prism_runmyh100"}
+    del P, Q, D, Cc
+    m = 1 << 30
+    x = torch.randint(-1000, 1001, (m,), dtype=torch.int32, device="cuda")
+    y = torch.empty_like(x)
+    need = ctypes.c_size_t(0)
+    if v.vendor_scan_temp_bytes(m, ctypes.byref(need)) != 0:
+        raise RuntimeError("vendor_scan_temp_bytes failed")
+    temp = torch.empty(max(need.value, 16), dtype=torch.uint8, device="cuda")
+    ms = time_steps(checked(lambda: v.vendor_scan_inclusive_sum(x.data_ptr(), y.data_ptr(), m, temp.data_ptr(), temp.numel(), st)), steps, warmup)
+    out["hipcub_inclusive_sum_2p30"] = {"ms": ms, "GBps": 8.0 * m / ms / 1e6}
+    return out
+
+
 # ----------------------------------------------------------- CPU baselines --
 
 def cpu_baseline_sgemm(n=8192, rows=4):
@@ -322,6 +375,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="all", choices=["all", "sgemm", "scan", "gemm_bf16", "add_m", "calibrate"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-vendor", action="store_true", help="skip the vendor-library comparison lines (also.vendor_libraries)")
     ap.add_argument("--no-configs", action="store_true",
                     help="skip the table of the other BASELINE configurations (also.configs)")
     ap.add_argument("--traffic-summary", metavar="DIR", default=None,
@@ -329,7 +383,12 @@ def main() -> int:
     ap.add_argument("--trace-summary", metavar="DIR", default=None,
                     help="no GPU work: summarise the rocprofv3 --kernel-trace --stats output in DIR into "
                          "profiles/bench_all_kernels_kernel_trace.md")
+    ap.add_argument("--eval-summary", metavar="DIR", default=None,
+                    help="no GPU work: summarise eval_report.txt / eval_generated.txt in DIR (outputs of "
+                         "`python -m prism_amd.eval_report [generated]`) into profiles/eval_sweeps.md")
     args = ap.parse_args()
+    if args.eval_summary:
+        return write_eval_tables(args.eval_summary)
     if args.traffic_summary:
         return write_traffic_table(args.traffic_summary)
     if args.trace_summary:
@@ -383,6 +442,10 @@ def main() -> int:
         res["add_m"]["note"] = "x and y are 128 MiB together and fit the 256 MiB memory-side cache: not an HBM-bound figure"
         log("add_m 2^28:", res["add_m_2p28"])
 
+    if args.workload == "all" and not args.no_vendor:
+        res["vendor_libraries"] = bench_vendor(K, W)
+        log("vendor libraries:", res["vendor_libraries"])
+
     # Every other BASELINE configuration, with fewer steps (kernel 1 at 8192^3 takes 0.35 s a step): a table
     # under "also.configs" of the JSON line, each entry parity-gated like the headline workloads.
     configs = {}
@@ -400,11 +463,23 @@ def main() -> int:
             r = bench_sgemm(prism, M, N, Kd, 1.0, 0.0, 5, 10, 2)
             configs[f"sgemm_k5_{M}x{N}x{Kd}"] = {"ms": r["ms"], "tflops": r["tflops"], "frac": r["roofline"]["frac"], "steps": 10}
             log(f"  sgemm kernel 5 {M}x{N}x{Kd}: {r['ms']:.3f} ms  {r['tflops']:.2f} TFLOP/s")
-        # the skinny tail shape once more through the workspace form (K cut across workgroups)
-        r = bench_sgemm(prism, 128, 4096, 4096, 1.0, 0.0, 5, 10, 2, with_workspace=True)
-        configs["sgemm_k5_128x4096x4096_with_workspace"] = {"ms": r["ms"], "tflops": r["tflops"], "frac": r["roofline"]["frac"],
-                                                            "steps": 10, "entry": "prism_sgemm_ws"}
-        log(f"  sgemm kernel 5 128x4096x4096 with workspace: {r['ms']:.3f} ms  {r['tflops']:.2f} TFLOP/s")
+        # Shapes whose tiles do not fill whole rounds of the CUs, through the reference-shaped entry and through the
+        # workspace form (prism_sgemm_ws: K ranges shared between all CUs); the plan query says that the shared
+        # form is what the "with_workspace" rows measured.
+        for (M, N, Kd) in ((128, 4096, 4096), (5120, 5120, 5120), (4352, 4352, 4352), (3200, 3200, 3200)):
+            name = f"sgemm_k5_{M}x{N}x{Kd}"
+            if name not in configs:
+                r = bench_sgemm(prism, M, N, Kd, 1.0, 0.0, 5, 10, 2)
+                configs[name] = {"ms": r["ms"], "tflops": r["tflops"], "frac": r["roofline"]["frac"], "steps": 10}
+                log(f"  sgemm kernel 5 {M}x{N}x{Kd}: {r['ms']:.3f} ms  {r['tflops']:.2f} TFLOP/s")
+            groups, shared = prism.sgemm_workspace_plan(M, N, Kd, prism.sgemm_workspace_size(M, N, Kd))
+            if groups == 0:
+                continue  # nothing would be shared for this shape (3200^3: fewer tiles than CUs)
+            r = bench_sgemm(prism, M, N, Kd, 1.0, 0.0, 5, 10, 2, with_workspace=True)
+            configs[name + "_with_workspace"] = {"ms": r["ms"], "tflops": r["tflops"], "frac": r["roofline"]["frac"], "steps": 10,
+                                                 "entry": "prism_sgemm_ws", "workgroups_sharing": groups, "tiles_shared": shared}
+            log(f"  sgemm kernel 5 {M}x{N}x{Kd} with workspace ({shared} tiles shared by {groups} workgroups): "
+                f"{r['ms']:.3f} ms  {r['tflops']:.2f} TFLOP/s")
         for p in (20, 24, 28):
             r = bench_scan(prism, 1 << p, 20, 3)
             configs[f"scan_2p{p}"] = {"ms": r["ms"], "GBps": r["GBps"], "frac": r["roofline"]["frac"], "steps": 20}

@@ -171,3 +171,86 @@ def write_kernel_trace_table(prof_dir: str) -> int:
     TRACE_FILE.write_text("\n".join(out) + "\n")
     print("\n".join(out))
     return 0
+
+
+# ------------------------------------------- sweeps of the evaluation report --
+
+def parse_eval_report(text: str):
+    """The three sweeps of `python -m prism_amd.eval_report ...` (the reference harnesses' text formats) as
+    ({size: {"vendor" | kernel number: GFLOPS}}, [(n, vendor GB/s, ours GB/s)], {size: {"Kernel" | "cuBLAS": TFLOPS}})."""
+    sgemm, scan, h100 = {}, [], {}
+    size = kernel = None
+    in_table = False
+    for line in text.splitlines():
+        t = line.strip()
+        m = re.match(r"Size:\s+(\d+)x\d+x\d+", t)
+        if m:
+            size = int(m.group(1))
+        if t == "[cuBLAS FP32]":
+            kernel = "vendor"
+        m = re.match(r"\[My Kernel (\d+)\]", t)
+        if m:
+            kernel = int(m.group(1))
+        m = re.search(r"performance:\s+\(\s*([\d.]+)\)\s+GFLOPS", t)
+        if m and kernel is not None and size is not None:
+            sgemm.setdefault(size, {})[kernel] = float(m.group(1))
+            kernel = None
+        m = re.match(r"(Kernel|cuBLAS):\s+.*performance:\s+\(\s*([\d.]+)\)\s+TFLOPS.*size:\s+\((\d+)\)", t)
+        if m:
+            h100.setdefault(int(m.group(3)), {})[m.group(1)] = float(m.group(2))
+        if "Size" in t and "CUB (GB/s)" in t:
+            in_table = True
+            continue
+        if in_table and t.startswith("---"):
+            continue
+        if in_table and t:
+            parts = re.split(r"\s*\|\s*", t)
+            scan.append((int(parts[0]), float(parts[1].split()[1]), float(parts[2].split()[1])))
+        elif in_table:
+            in_table = False
+    return sgemm, scan, h100
+
+
+def write_eval_tables(report_dir: str) -> int:
+    """Summarises two runs of the evaluation sweeps into profiles/eval_sweeps.md. Expected in report_dir:
+    eval_report.txt (`python -m prism_amd.eval_report`) and eval_generated.txt (`python -m prism_amd.eval_report
+    generated`)."""
+    out = ["# The reference harnesses' sweeps on one MI355X: hand-written kernels, DSL-generated kernels, vendor libraries", "",
+           "Written by `python bench.py --eval-summary $OUT` from two runs on the GPU box (R = repo root, OUT = a scratch",
+           "directory):", "",
+           "    python3 -m prism_amd.eval_report > $OUT/eval_report.txt", "    python3 -m prism_amd.eval_report generated > $OUT/eval_generated.txt", "",
+           "Protocols and text formats are the reference's (evals/4090_sgemm/main.cu:154-217: 10 launches between two events,",
+           "alpha 0.5, beta 3.0; evals/4090_scan/bench.cu:157-262: best wall-clock of launch + sync; evals/h100_bench/main.cu:112-167:",
+           "8 launches between two events). The vendor columns are rocblas_sgemm, hipcub::DeviceScan::InclusiveSum and a hipBLASLt",
+           "bf16 matmul called directly (prism_amd/csrc/vendor/vendor_baselines.hip). The large GEMMs are timed right after the",
+           "first call, while the clocks still settle, and read a few per cent below the sustained figures of bench.py.", ""]
+    for name, title in (("eval_report.txt", "Hand-written kernels (libprism_amd.so)"), ("eval_generated.txt", "Kernels printed by the DSL back-end (prism_amd/examples)")):
+        path = os.path.join(report_dir, name)
+        if not os.path.exists(path):
+            print(f"no {name} in {report_dir}", file=sys.stderr)
+            continue
+        sgemm, scan, h100 = parse_eval_report(open(path).read())
+        out += [f"## {title}", ""]
+        if sgemm:
+            kernels = sorted({k for row in sgemm.values() for k in row if k != "vendor"})
+            out += ["SGEMM, TFLOP/s (fraction of the 157.3 TFLOP/s fp32 MFMA peak for kernel 5):", "",
+                    "| size | rocBLAS | " + " | ".join(f"kernel {k}" for k in kernels) + " |", "|---:|---:|" + "---:|" * len(kernels)]
+            for size in sorted(sgemm):
+                row = sgemm[size]
+                cells = []
+                for k in kernels:
+                    v = row.get(k)
+                    cells.append("-" if v is None else f"{v / 1e3:.1f}" + (f" ({v / 1e3 / 157.3:.2f})" if k == 5 else ""))
+                out.append(f"| {size} | {row.get('vendor', 0) / 1e3:.1f} | " + " | ".join(cells) + " |")
+            out.append("")
+        if scan:
+            out += ["Inclusive scan of uint32, GB/s (fraction of the 8 TB/s HBM peak):", "", "| n | hipCUB | ours |", "|---:|---:|---:|"]
+            out += [f"| 2^{n.bit_length() - 1} | {v:.0f} | {o:.0f} ({o / 8000:.2f}) |" for n, v, o in scan]
+            out.append("")
+        if h100:
+            out += ["bf16 GEMM, TFLOP/s (fraction of the 2.5 PFLOP/s bf16 MFMA peak):", "", "| size | hipBLASLt | ours |", "|---:|---:|---:|"]
+            out += [f"| {n} | {r.get('cuBLAS', 0):.0f} | {r.get('Kernel', 0):.0f} ({r.get('Kernel', 0) / 2500:.2f}) |" for n, r in sorted(h100.items())]
+            out.append("")
+    (ROOT / "profiles" / "eval_sweeps.md").write_text("\n".join(out) + "\n")
+    print("\n".join(out))
+    return 0
