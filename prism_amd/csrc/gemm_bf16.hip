@@ -736,14 +736,17 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
             fq[set][r - MI] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(&Qs[stage][q_off[kk] + (r - MI) * 16 * BK]));
     };
     // The 64 instructions of one k-step from fragment set `set`; `after(m)` is issued right behind the m-th.
+    // The sub-tiles are walked row by row, every other row backwards, so that consecutive instructions always
+    // share one operand (measured 0.5-1 % over always walking forwards).
     auto mfma_block = [&](int set, auto after) {
 #pragma unroll
         for (int i = 0; i < MI; ++i)
 #pragma unroll
-            for (int j = 0; j < NI; ++j) {
+            for (int jj = 0; jj < NI; ++jj) {
+                const int j = (i & 1) ? NI - 1 - jj : jj;
                 mfma_16x16x32_in_place(acc[i][j], fq[set][j], fp[set][i]);  // Q first: see the write-back
                 __builtin_amdgcn_sched_barrier(0);
-                after(i * NI + j);
+                after(i * NI + jj);
                 __builtin_amdgcn_sched_barrier(0);
             }
     };
