@@ -45,7 +45,8 @@ ROOT = Path(__file__).resolve().parent
 # Helpers shared with the tests live in tests/: the parity gate (fp64_referee), the tables under profiles/
 # (profile_tables) and the streaming calibration kernels (calibrate_stream).
 sys.path.insert(0, str(ROOT / "tests"))
-from profile_tables import measured_traffic, write_eval_tables, write_kernel_trace_table, write_traffic_table  # noqa: E402
+from profile_tables import (measured_traffic, write_counter_table, write_eval_tables, write_kernel_trace_table,  # noqa: E402
+                            write_traffic_table)
 
 
 def log(*a):
@@ -383,12 +384,16 @@ def main() -> int:
     ap.add_argument("--trace-summary", metavar="DIR", default=None,
                     help="no GPU work: summarise the rocprofv3 --kernel-trace --stats output in DIR into "
                          "profiles/bench_all_kernels_kernel_trace.md")
+    ap.add_argument("--counter-summary", metavar="DIR", default=None,
+                    help="no GPU work: summarise three rocprofv3 --pmc runs (p1, p2, p3) in DIR into profiles/kernel_counters.md")
     ap.add_argument("--eval-summary", metavar="DIR", default=None,
                     help="no GPU work: summarise eval_report.txt / eval_generated.txt in DIR (outputs of "
                          "`python -m prism_amd.eval_report [generated]`) into profiles/eval_sweeps.md")
     args = ap.parse_args()
     if args.eval_summary:
         return write_eval_tables(args.eval_summary)
+    if args.counter_summary:
+        return write_counter_table(args.counter_summary)
     if args.traffic_summary:
         return write_traffic_table(args.traffic_summary)
     if args.trace_summary:

@@ -2,10 +2,12 @@
 
 profiles/hbm_traffic.md holds the HBM-side bytes per launch of the headline kernels (`roofline.traffic` in the
 benchmark line); profiles/bench_all_kernels_kernel_trace.md the per-kernel durations of a `rocprofv3
---kernel-trace --stats` run of the benchmark beside the benchmark's own event timing. Both are written from the
-profiler's raw CSV files by the functions below (`python bench.py --traffic-summary DIR`, `python bench.py
---trace-summary DIR`), never by hand, and tests/test_bench_tables.py checks that the traffic rows belong to the
-kernel sources in the tree. No GPU work happens here.
+--kernel-trace --stats` run of the benchmark beside the benchmark's own event timing; profiles/kernel_counters.md
+the hardware counters of the same kernels beside the vendor libraries' kernels and plain streaming kernels of the
+same run; profiles/eval_sweeps.md the reference harnesses' sweeps. All are written from raw output files by the
+functions below (`python bench.py --traffic-summary | --trace-summary | --counter-summary | --eval-summary DIR`),
+never by hand, and tests/test_bench_tables.py checks that the traffic rows belong to the kernel sources in the
+tree. No GPU work happens here.
 """
 from __future__ import annotations
 
@@ -168,7 +170,161 @@ def write_kernel_trace_table(prof_dir: str) -> int:
         name = re.sub(r"^void ", "", r["Name"]).replace("prism::(anonymous namespace)::", "")
         name = name[: name.index("(")] if "(" in name else name
         out.append(f"| `{name}` | {r['Calls']} | {float(r['AverageNs']) / 1e3:.1f} | {float(r['TotalDurationNs']) / 1e6:.1f} |")
+    configs = os.path.join(prof_dir, "configs_kernel_stats.csv")
+    if os.path.exists(configs):
+        with open(configs, newline="") as f:
+            stats = list(csv.DictReader(f))
+        out += ["", "## The default run, configuration table included", "",
+                "    rocprofv3 --kernel-trace --stats -d $OUT/prof_trace -o configs --output-format csv -- \\",
+                "        python3 $R/bench.py --no-cpu-baseline", "",
+                "`also.configs` adds SGEMM kernels 1, 2, 3, 6, 4, 5 at 1024^3 .. 8192^3, kernel 5 at the tail shapes (with and",
+                "without a workspace where one is used), the scans of 2^20, 2^24 and 2^28 elements and the bf16 product at 4096^3 and",
+                "16384^3. This table names the kernel each of them lands on; averages mix the sizes a kernel was launched at.", "",
+                "| kernel | calls | average us | total ms |", "|---|---:|---:|---:|"]
+        for r in sorted(stats, key=lambda r: -float(r["TotalDurationNs"])):
+            if "prism::" not in r["Name"]:
+                continue
+            name = re.sub(r"^void ", "", r["Name"]).replace("prism::(anonymous namespace)::", "")
+            name = name[: name.index("(")] if "(" in name else name
+            out.append(f"| `{name}` | {r['Calls']} | {float(r['AverageNs']) / 1e3:.1f} | {float(r['TotalDurationNs']) / 1e6:.1f} |")
     TRACE_FILE.write_text("\n".join(out) + "\n")
+    print("\n".join(out))
+    return 0
+
+
+# ------------------------------------------------ hardware counter tables --
+
+COUNTER_FILE = ROOT / "profiles" / "kernel_counters.md"
+COUNTER_PASSES = {
+    "p1": "SQ_BUSY_CYCLES SQ_VALU_MFMA_BUSY_CYCLES SQ_WAVE_CYCLES SQ_INSTS_VALU SQ_INSTS_LDS SQ_ACTIVE_INST_LDS SQ_LDS_BANK_CONFLICT SQ_WAIT_INST_ANY",
+    "p2": "GRBM_GUI_ACTIVE TCC_HIT_sum TCC_MISS_sum TCP_PENDING_STALL_CYCLES_sum",
+    "p3": "SQ_WAVES SQ_WAVE_CYCLES SQ_WAIT_ANY SQ_INSTS_VMEM_RD SQ_INSTS_VMEM_WR SQ_INSTS_SALU SQ_ACTIVE_INST_ANY GRBM_GUI_ACTIVE",
+}
+GEMM_ROWS = [  # (label, substrings that must all occur in the kernel name, grid size in threads)
+    ("ours, SGEMM kernel 5 (fp32)", ["sgemm_wave_tile_dma_kernel<256, 256, 32, 32, 128, false, false, false>"], 1024 * 1024),
+    ("rocBLAS `rocblas_sgemm` (fp32)", ["Cijk_Ailk_Bljk_SB_"], None),
+    ("ours, bf16 in, fp32 out", ["gemm_bf16_early_kernel<256, 256, 128, 128, false, float"], 256 * 1024),
+    ("hipBLASLt, bf16 in, fp32 out", ["Cijk_Alik_Bljk_BSS_BH"], None),
+    ("ours, bf16 in, bf16 column-major out", ["gemm_bf16_early_kernel<256, 256, 128, 128, false, unsigned short"], 256 * 1024),
+    ("hipBLASLt, bf16 in, bf16 column-major out", ["Cijk_Alik_Bljk_BBS_BH"], None),
+]
+STREAM_ROWS = [
+    ("ours, scan 2^30 (tiles by workgroup id)", ["scan_lookback_kernel<", "BigCfg, true, false, false"], (1 << 30) // 64),
+    ("ours, scan 2^30 (ticket order)", ["scan_lookback_kernel<", "BigCfg, true, true, false"], (1 << 30) // 64),
+    ("hipCUB `DeviceScan::InclusiveSum` 2^30 (its scan kernel)", ["rocprim", "trampoline_kernel"], None),
+    ("copy 2^30 x 4 B, the scan's tile shape", ["calibrate_copy_tile_kernel"], (1 << 30) // 64),
+    ("copy 2^30 x 4 B, one packet per lane", ["calibrate_copy_packet_kernel"], (1 << 30) // 4),
+    ("read only, 4 GiB", ["calibrate_read_kernel"], None),
+    ("write only, 4 GiB", ["calibrate_write_kernel"], None),
+    ("ours, add_m 2^28", ["add_m_vec4_kernel<true>"], (1 << 28) // 4),
+]
+
+
+def write_counter_table(pmc_dir: str) -> int:
+    """Summarises three `rocprofv3 --pmc` runs of bench.py (COUNTER_PASSES, outputs p1, p2, p3 in pmc_dir) into
+    profiles/kernel_counters.md: per kernel the mean over its dispatches of every counter, and what follows
+    from them (clock, matrix-pipe duty, L2 hit rate, waves resident, share of cycles the vector L1 waits)."""
+    import csv
+    from collections import defaultdict
+
+    def load(name):
+        per = defaultdict(lambda: defaultdict(list))  # (kernel name, grid) -> counter -> values
+        dur = defaultdict(dict)                       # (kernel name, grid) -> dispatch id -> ns
+        path = os.path.join(pmc_dir, f"{name}_counter_collection.csv")
+        with open(path, newline="") as f:
+            for r in csv.DictReader(f):
+                key = (r["Kernel_Name"], int(r["Grid_Size"]))
+                per[key][r["Counter_Name"]].append(float(r["Counter_Value"]))
+                dur[key][r["Dispatch_Id"]] = int(r["End_Timestamp"]) - int(r["Start_Timestamp"])
+        return per, dur
+
+    try:
+        passes = {name: load(name) for name in COUNTER_PASSES}
+    except OSError as e:
+        print(f"{e}", file=sys.stderr)
+        return 1
+
+    def row_values(match, grid):
+        """Counter means of the kernel (the one with most dispatches among those that match), from all passes."""
+        vals, n, us = {}, 0, 0.0
+        for name, (per, dur) in passes.items():
+            keys = [k for k in per if all(m in k[0] for m in match) and (grid is None or k[1] == grid)]
+            if not keys:
+                continue
+            k = max(keys, key=lambda k: len(dur[k]))
+            d = sorted(dur[k].values())
+            d = d[: max(1, len(d) * 9 // 10)]  # the cold first dispatches out
+            if name == "p2":
+                n, us = len(dur[k]), sum(d) / len(d) / 1e3
+                vals["_name"], vals["_grid"] = k
+            for c, v in per[k].items():
+                vals.setdefault(f"{name}:{c}", sum(v) / len(v))
+                vals.setdefault(c, sum(v) / len(v))
+        return vals, n, us
+
+    def short(name):
+        name = re.sub(r"^void ", "", name).replace("prism::(anonymous namespace)::", "").replace("(anonymous namespace)::", "")
+        name = name[: name.index("(")] if "(" in name else name
+        return name if len(name) <= 72 else name[:69] + "..."
+
+    out = ["# rocprofv3 --pmc: hardware counters of the headline kernels beside the vendor libraries' and plain streaming kernels", "",
+           "Written by `python bench.py --counter-summary $OUT/pmc_counters` from three counter runs of the same program (from /tmp",
+           "with TMPDIR=/tmp on the GPU box, R = repo root, OUT = a scratch directory; each pass its own process, because one pass",
+           "holds at most 8 SQ, 4 TCC and 2 GRBM counters):", ""]
+    for name, counters in COUNTER_PASSES.items():
+        out += [f"    rocprofv3 --pmc {counters} \\",
+                f"        --kernel-trace -d $OUT/pmc_counters -o {name} --output-format csv -- python3 $R/bench.py --steps 5 --warmup 1 --no-configs --no-cpu-baseline"]
+    out += ["", "`bench.py` runs, in one process, our kernels at the headline sizes (8192^3, 2^30, 2^28), the vendor libraries called directly",
+            "on the same operands (rocblas_sgemm, hipBLASLt matmul, hipcub::DeviceScan::InclusiveSum) and the plain streaming kernels of",
+            "tests/native/calibrate_stream.hip on 4 GiB buffers. Every figure is the mean over a kernel's dispatches in the run; counters",
+            "are sums over the 8 XCDs. Derived: shader cycles = GRBM_GUI_ACTIVE / 8; clock = cycles / duration (both of pass p2);",
+            "matrix-pipe duty = SQ_VALU_MFMA_BUSY_CYCLES (p1) / 1024 SIMDs / cycles; L2 hit rate = TCC_HIT / (TCC_HIT + TCC_MISS);",
+            "waves resident = 4 x SQ_WAVE_CYCLES / cycles (p3, cycles of p3); vector L1 waiting = TCP_PENDING_STALL_CYCLES / 256 CUs / cycles.",
+            "Durations under counter collection are a few per cent above the untraced ones.", "",
+            "## GEMM kernels at 8192^3", "",
+            "| kernel | dispatches | duration us | clock GHz | matrix-pipe duty | duty x clock / 2.4 GHz | SQ_INSTS_VALU | SQ_INSTS_LDS | SQ_ACTIVE_INST_LDS | LDS bank conflict cycles | SQ_WAIT_INST_ANY / SQ_WAVE_CYCLES | L2 hit |",
+            "|---|---:|---:|---:|---:|---:|---:|---:|---:|---:|---:|---:|"]
+    names = []
+    for label, match, grid in GEMM_ROWS:
+        v, n, us = row_values(match, grid)
+        if not n or "GRBM_GUI_ACTIVE" not in v:
+            print(f"no dispatches for {label}", file=sys.stderr)
+            continue
+        cycles = v["p2:GRBM_GUI_ACTIVE"] / 8
+        clock = cycles / (us * 1e3)
+        duty = v.get("SQ_VALU_MFMA_BUSY_CYCLES", 0) / 1024 / cycles
+        hit = v.get("TCC_HIT_sum", 0) / max(1.0, v.get("TCC_HIT_sum", 0) + v.get("TCC_MISS_sum", 0))
+        names.append(f"* {label}: `{short(v['_name'])}`, {v['_grid'] // 256 if 'prism' not in v['_name'] else v['_grid']} "
+                     + ("workgroups of 256 threads" if "prism" not in v["_name"] else "threads"))
+        out.append(f"| {label} | {n} | {us:.1f} | {clock:.2f} | {duty:.3f} | {duty * clock / 2.4:.3f} | {v.get('SQ_INSTS_VALU', 0):.3g} | "
+                   f"{v.get('SQ_INSTS_LDS', 0):.3g} | {v.get('SQ_ACTIVE_INST_LDS', 0):.3g} | {v.get('SQ_LDS_BANK_CONFLICT', 0):.3g} | "
+                   f"{v.get('SQ_WAIT_INST_ANY', 0) / max(1.0, v.get('p1:SQ_WAVE_CYCLES', 1)):.3f} | {hit:.2f} |")
+    out += ["", "Kernel names:", ""] + names
+    out += ["", "The fp32 kernels run near the nominal 2.4 GHz and their duty x clock is the fraction of the 157.3 TFLOP/s peak that bench.py",
+            "reports. The bf16 kernels, ours and the library's alike, are power-limited: the clock column is what the part holds under",
+            "them, and the published 2.5 PFLOP/s assumes 2.4 GHz.", "",
+            "## Streaming kernels", "",
+            "| kernel | dispatches | duration us | GB/s | fraction of 8 TB/s | waves launched | waves resident | SQ_WAIT_ANY / SQ_WAVE_CYCLES | SQ_ACTIVE_INST_ANY / SQ_WAVE_CYCLES | vector-memory reads | writes | vector L1 waiting | L2 hit |",
+            "|---|---:|---:|---:|---:|---:|---:|---:|---:|---:|---:|---:|---:|"]
+    moved = {"scan": 8.0 * (1 << 30), "hipCUB": 8.0 * (1 << 30), "copy": 8.0 * (1 << 30), "read": 4.0 * (1 << 30), "write": 4.0 * (1 << 30), "add_m": 8.0 * (1 << 28)}
+    for label, match, grid in STREAM_ROWS:
+        v, n, us = row_values(match, grid)
+        if not n or "p3:GRBM_GUI_ACTIVE" not in v:
+            print(f"no dispatches for {label}", file=sys.stderr)
+            continue
+        nbytes = next(b for k, b in moved.items() if k in label)
+        cycles2, cycles3 = v["p2:GRBM_GUI_ACTIVE"] / 8, v["p3:GRBM_GUI_ACTIVE"] / 8
+        wc = max(1.0, v.get("p3:SQ_WAVE_CYCLES", 1))
+        hit = v.get("TCC_HIT_sum", 0) / max(1.0, v.get("TCC_HIT_sum", 0) + v.get("TCC_MISS_sum", 0))
+        out.append(f"| {label} | {n} | {us:.1f} | {nbytes / us / 1e3:.0f} | {nbytes / us / 1e3 / 8000:.3f} | {v.get('SQ_WAVES', 0):.0f} | "
+                   f"{4 * wc / cycles3:.0f} | {v.get('SQ_WAIT_ANY', 0) / wc:.3f} | {v.get('SQ_ACTIVE_INST_ANY', 0) / wc:.3f} | "
+                   f"{v.get('SQ_INSTS_VMEM_RD', 0):.0f} | {v.get('SQ_INSTS_VMEM_WR', 0):.0f} | "
+                   f"{v.get('TCP_PENDING_STALL_CYCLES_sum', 0) / 256 / cycles2:.3f} | {hit:.2f} |")
+    out += ["", "A scan tile of 65536 elements issues 16 x 16 data loads and as many stores; what the scan's vector-memory counts exceed",
+            "the tile-shaped copy's by is its status traffic (header read, look-back polls, aggregate / prefix / cleared word). The scan",
+            "stands beside the copy in its own tile shape, the copy with one packet per lane is the shape add_m uses, and the one-way",
+            "streams show what the memory system gives in each direction."]
+    COUNTER_FILE.write_text("\n".join(out) + "\n")
     print("\n".join(out))
     return 0
 
