@@ -134,7 +134,8 @@ enum {
                                   /* (examples/scan.py:88-99) instead of by workgroup id                 */
     PRISM_SCAN_NO_HELP = 4,       /* a look-back that runs out of polls reports it (prism_scan_status)   */
                                   /* and goes on with a wrong sum instead of helping its predecessor:    */
-                                  /* the plain bounded wait, kept to exercise that way out               */
+                                  /* the plain bounded wait, kept to exercise that way out (every kind   */
+                                  /* of scan takes this flag through its _ex entry point)                */
     PRISM_SCAN_OP_SUM = 0x00,
     PRISM_SCAN_OP_MAX = 0x10,     /* prism_scan_max_i32's result (inclusive, workgroup-id order only)    */
     PRISM_SCAN_OP_MIN = 0x20      /* prism_scan_min_i32's result (inclusive, workgroup-id order only)    */
@@ -181,8 +182,8 @@ int prism_scan_i32_static(const int32_t* in, int32_t* out, size_t n, void* strea
  * Waits for `stream`, then reports on the scans that used this workspace
  * since the last report: 0 = nothing to report; PRISM_ERROR_SCAN_WORKSPACE =
  * the workspace was not initialised (or something else wrote into it);
- * PRISM_ERROR_SCAN_ORDER = a look-back gave up waiting (only scans that do not
- * help: PRISM_SCAN_NO_HELP, the segmented and the 64-bit scan). In both cases
+ * PRISM_ERROR_SCAN_ORDER = a look-back gave up waiting (only scans that were
+ * told not to help, PRISM_SCAN_NO_HELP). In both cases
  * the output of those scans is invalid, the error string says more, and the
  * workspace has been initialised afresh.
  * workspace == NULL stands for the array prism_scan_i32_static uses on the
@@ -233,6 +234,18 @@ int prism_segmented_scan_i32(const int32_t* in, const uint8_t* heads, int32_t* o
                              void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * prism_segmented_scan_i32 with the look-back's choices as arguments, as
+ * prism_scan_i32_ex has them: flags is 0 or PRISM_SCAN_NO_HELP, spin_limit the
+ * bound on the polls of one look-back window (negative = the library's
+ * default, 0 = no waiting). A tile that helps forms its predecessor's (head
+ * seen, sum) pair from that tile's input and head bytes. The reference's
+ * look-back waits without bound (generated/lookback_to_prev_blocks.cu:12-21).
+ */
+int prism_segmented_scan_i32_ex(const int32_t* in, const uint8_t* heads, int32_t* out, size_t n,
+                                void* workspace, size_t workspace_bytes, unsigned flags,
+                                long long spin_limit, void* stream);
+
+/*
  * Inclusive prefix sum of 64-bit elements, out[i] = in[0] + ... + in[i] modulo
  * 2^64 (identical bit patterns for int64 and uint64): scan_kernel's
  * decomposition (examples/scan.py:106-227) on wider elements. A tile publishes
@@ -245,6 +258,15 @@ int prism_segmented_scan_i32(const int32_t* in, const uint8_t* heads, int32_t* o
  */
 int prism_scan_i64(const int64_t* in, int64_t* out, size_t n, void* workspace,
                    size_t workspace_bytes, void* stream);
+
+/*
+ * prism_scan_i64 with the look-back's choices as arguments (flags 0 or
+ * PRISM_SCAN_NO_HELP, spin_limit as for prism_scan_i32_ex). The reference's
+ * look-back waits without bound (generated/lookback_to_prev_blocks.cu:12-21).
+ */
+int prism_scan_i64_ex(const int64_t* in, int64_t* out, size_t n, void* workspace,
+                      size_t workspace_bytes, unsigned flags, long long spin_limit,
+                      void* stream);
 
 /*
  * The reference launcher's own shape: in-place on x, default stream, returns

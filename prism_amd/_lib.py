@@ -31,7 +31,11 @@ SIGNATURES = {
     "prism_scan_min_i32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p]),
     "prism_segmented_scan_i32": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t,
                                            C.c_void_p]),
+    "prism_segmented_scan_i32_ex": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t,
+                                              C.c_uint, C.c_longlong, C.c_void_p]),
     "prism_scan_i64": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "prism_scan_i64_ex": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_uint, C.c_longlong,
+                                    C.c_void_p]),
     "prism_launch_scan": (C.c_void_p, [C.c_size_t, C.c_void_p, C.c_void_p]),
     "prism_sgemm": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_void_p,
                               C.c_float, C.c_void_p, C.c_void_p]),

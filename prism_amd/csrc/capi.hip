@@ -112,12 +112,24 @@ int prism_scan_min_i32(const int32_t* in, int32_t* out, size_t n, void* workspac
 
 int prism_segmented_scan_i32(const int32_t* in, const uint8_t* heads, int32_t* out, size_t n, void* workspace,
                              size_t workspace_bytes, void* stream) {
-    return launch_segmented_scan(u32(in), heads, u32(out), n, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+    return launch_segmented_scan(u32(in), heads, u32(out), n, workspace, workspace_bytes, 0u, -1, static_cast<hipStream_t>(stream));
+}
+
+int prism_segmented_scan_i32_ex(const int32_t* in, const uint8_t* heads, int32_t* out, size_t n, void* workspace,
+                                size_t workspace_bytes, unsigned flags, long long spin_limit, void* stream) {
+    return launch_segmented_scan(u32(in), heads, u32(out), n, workspace, workspace_bytes, flags, spin_limit,
+                                 static_cast<hipStream_t>(stream));
 }
 
 int prism_scan_i64(const int64_t* in, int64_t* out, size_t n, void* workspace, size_t workspace_bytes, void* stream) {
     return launch_scan64(reinterpret_cast<const unsigned long long*>(in), reinterpret_cast<unsigned long long*>(out), n,
-                         workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+                         workspace, workspace_bytes, 0u, -1, static_cast<hipStream_t>(stream));
+}
+
+int prism_scan_i64_ex(const int64_t* in, int64_t* out, size_t n, void* workspace, size_t workspace_bytes, unsigned flags,
+                      long long spin_limit, void* stream) {
+    return launch_scan64(reinterpret_cast<const unsigned long long*>(in), reinterpret_cast<unsigned long long*>(out), n,
+                         workspace, workspace_bytes, flags, spin_limit, static_cast<hipStream_t>(stream));
 }
 
 uint32_t* prism_launch_scan(size_t n, uint32_t* x, void* workspace) {

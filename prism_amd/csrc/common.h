@@ -67,9 +67,11 @@ int scan_workspace_init(void* ws, size_t ws_bytes, hipStream_t s);
 int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws_bytes, unsigned flags,
                 long long spin_limit, hipStream_t s);
 int scan_status(void* ws, size_t ws_bytes, hipStream_t s);
+// flags: kFlagNoHelp or 0; spin_limit as for launch_scan.
 int launch_segmented_scan(const uint32_t* in, const uint8_t* heads, uint32_t* out, size_t n, void* ws, size_t ws_bytes,
-                          hipStream_t s);
-int launch_scan64(const unsigned long long* in, unsigned long long* out, size_t n, void* ws, size_t ws_bytes, hipStream_t s);
+                          unsigned flags, long long spin_limit, hipStream_t s);
+int launch_scan64(const unsigned long long* in, unsigned long long* out, size_t n, void* ws, size_t ws_bytes, unsigned flags,
+                  long long spin_limit, hipStream_t s);
 int launch_scan_static(const uint32_t* in, uint32_t* out, size_t n, hipStream_t s);
 int launch_wave_regroup(const int32_t* in, int32_t* out, size_t n, int items_per_lane, int direction, hipStream_t s);
 int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, const float* B,

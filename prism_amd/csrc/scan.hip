@@ -39,7 +39,7 @@
 // 12 % of the run time at 2^30. The default here is tile = a fixed function of the workgroup id (chunks of 4
 // consecutive tiles go to workgroups of one XCD, see the kernel), which waits least when the dispatcher starts
 // the workgroups of a 1-D grid in id order on every XCD. Correctness does not rest on that order: a look-back
-// that has polled a window kSpinLimit times without an answer (milliseconds; a running predecessor answers in
+// that has polled a window kHelpAfter times without an answer (milliseconds; a running predecessor answers in
 // microseconds) stops waiting and HELPS: wave 0 reads the silent predecessor's input itself, reduces it and
 // uses that aggregate. Every tile therefore finishes on its own whatever the others do, the GPU never hangs
 // and the result is the same bits. (In place, a predecessor might finish and overwrite its input while it is
@@ -48,8 +48,8 @@
 // before any of its output stores are issued.) The flag kFlagTicket selects the reference's ticket order
 // instead, kFlagNoHelp the behaviour of a plain bounded wait: a wave that runs out stores the tile number plus
 // one into the workspace header (kHdrReport) and carries on with a wrong prefix; scan_status() reads that word
-// after the stream has drained and turns it into an error. The segmented and the 64-bit scans wait that way
-// always. scan_status() also reports a workspace that was never initialised (the header holds a magic word).
+// after the stream has drained and turns it into an error. The segmented and the 64-bit scans help in the same
+// way. scan_status() also reports a workspace that was never initialised (the header holds a magic word).
 //
 // Workspace protocol (no reset launch per call). Every tile owns TWO status words,
 // one per parity of the workspace's call counter. A call with parity p publishes
@@ -544,23 +544,61 @@ __device__ __forceinline__ u64 pack_seg_status(uint32_t state, Seg p) {
     return static_cast<u64>(state | (p.f << 8)) | (static_cast<u64>(p.v) << 32);
 }
 
+// The pair of one whole tile, formed by one wavefront from the tile's input and head bytes: what a look-back
+// does for a predecessor that does not answer (see tile_aggregate). Two commutative reductions stand in for the
+// ordered one: the position of the tile's last head, then the sum of everything from there on.
+template <bool VEC, int TILE>
+__device__ __forceinline__ Seg tile_aggregate_seg(const uint32_t* in, const uint8_t* heads, size_t tile_base, int lane) {
+    int last = -1;  // index within the tile of the last head this lane has seen
+    uint32_t acc = 0u;
+    if constexpr (VEC) {
+        const uint32_t* hsrc = reinterpret_cast<const uint32_t*>(heads + tile_base) + lane;
+#pragma unroll 1
+        for (int i = 0; i < TILE / 4 / kWave; ++i) {
+            const uint32_t hb = hsrc[static_cast<size_t>(i) * kWave];
+            if (hb != 0u) last = 4 * (i * kWave + lane) + (31 - __builtin_clz(hb)) / 8;  // increasing with i
+        }
+        last = static_cast<int>(wave_last_lane(wave_inclusive_scan_op<MaxI32Op>(static_cast<uint32_t>(last))));
+        const u32x4* src = reinterpret_cast<const u32x4*>(in + tile_base) + lane;
+#pragma unroll 1
+        for (int i = 0; i < TILE / 4 / kWave; ++i) {
+            const u32x4 x = src[static_cast<size_t>(i) * kWave];
+            const int at = 4 * (i * kWave + lane);
+            acc += (at >= last ? x.x : 0u) + (at + 1 >= last ? x.y : 0u) + (at + 2 >= last ? x.z : 0u) + (at + 3 >= last ? x.w : 0u);
+        }
+    } else {
+        const uint8_t* hsrc = heads + tile_base + lane;
+#pragma unroll 1
+        for (int i = 0; i < TILE / kWave; ++i)
+            if (hsrc[static_cast<size_t>(i) * kWave] != 0) last = i * kWave + lane;
+        last = static_cast<int>(wave_last_lane(wave_inclusive_scan_op<MaxI32Op>(static_cast<uint32_t>(last))));
+        const uint32_t* src = in + tile_base + lane;
+#pragma unroll 1
+        for (int i = 0; i < TILE / kWave; ++i) {
+            const uint32_t x = src[static_cast<size_t>(i) * kWave];
+            acc += (i * kWave + lane >= last) ? x : 0u;
+        }
+    }
+    return Seg{last >= 0 ? 1u : 0u, wave_last_lane(wave_inclusive_scan(acc))};
+}
+
 // The pair that everything before tile `tile` (> 0) contributes to it. The walk back ends at the nearest
 // tile that has published a prefix or whose own range holds a head: what lies before a head does not matter.
+// A predecessor that has not answered after spin_limit polls is helped (tile_aggregate_seg) or, without
+// `help`, reported, as in look_back.
+template <bool VEC, int TILE>
 __device__ __forceinline__ Seg look_back_seg(const u64* status, uint32_t parity, uint32_t tile, int lane,
-                                             uint32_t spin_limit, uint32_t* report, uint32_t* bad_workspace) {
+                                             uint32_t spin_limit, bool help, const uint32_t* in, const uint8_t* heads,
+                                             uint32_t* report, uint32_t* bad_workspace) {
     Seg sum{0u, 0u};
     uint32_t spins = 0;
     long long window_end = static_cast<long long>(tile) - 1;
     while (true) {
-        if (spins >= spin_limit) {
-            if (lane == 0) __hip_atomic_store(report, tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            break;
-        }
         const long long t = window_end - lane;
         const u64 w = (t >= 0) ? poll(&status[2 * t + parity]) : pack_status(kPrefix, 0u);
-        const uint32_t state = static_cast<uint32_t>(w) & 0xffu;
-        const uint32_t flag = (static_cast<uint32_t>(w) >> 8) & 1u;
-        const uint32_t value = static_cast<uint32_t>(w >> 32);
+        uint32_t state = static_cast<uint32_t>(w) & 0xffu;
+        uint32_t flag = (static_cast<uint32_t>(w) >> 8) & 1u;
+        uint32_t value = static_cast<uint32_t>(w >> 32);
         if (__ballot(state > kPrefix || (static_cast<uint32_t>(w) >> 9) != 0u)) {  // no tile writes such a word
             if (lane == 0) __hip_atomic_store(bad_workspace, tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             break;
@@ -568,13 +606,37 @@ __device__ __forceinline__ Seg look_back_seg(const u64* status, uint32_t parity,
         const u64 is_invalid = __ballot(state == kInvalid);
         const u64 ends_walk = __ballot(state == kPrefix || flag != 0u);
         const int first_invalid = is_invalid ? __builtin_ctzll(is_invalid) : kWave;
-        const int first_end = ends_walk ? __builtin_ctzll(ends_walk) : kWave;
-        if (first_end >= first_invalid) {  // no end of the walk among the lanes known so far
-            if (first_invalid < kWave) {
+        int first_end = ends_walk ? __builtin_ctzll(ends_walk) : kWave;
+        if (first_end >= first_invalid && first_invalid < kWave) {  // a tile that has not answered is needed
+            if (spins < spin_limit) {
                 ++spins;
                 continue;
             }
+            if (!help) {
+                if (lane == 0) __hip_atomic_store(report, tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                break;
+            }
+            // Nearest first, until the end of the walk is known: a helped tile that holds a head ends it.
+            for (u64 todo = is_invalid; todo != 0; todo &= todo - 1) {
+                const int l = __builtin_ctzll(todo);
+                if (l > first_end) break;
+                const Seg formed = tile_aggregate_seg<VEC, TILE>(in, heads, static_cast<size_t>(window_end - l) * TILE, lane);
+                // As in look_back: all reads of that tile's input have returned; a word it has published by now
+                // is the truth, otherwise it has stored no output yet and `formed` is the pair of its input.
+                const u64 again = poll(&status[2 * (window_end - l) + parity]);
+                const uint32_t st = static_cast<uint32_t>(again) & 0xffu;
+                const uint32_t s_l = st != kInvalid ? st : kAggregate;
+                const uint32_t f_l = st != kInvalid ? (static_cast<uint32_t>(again) >> 8) & 1u : formed.f;
+                const uint32_t v_l = st != kInvalid ? static_cast<uint32_t>(again >> 32) : formed.v;
+                if (lane == l) {
+                    state = s_l;
+                    flag = f_l;
+                    value = v_l;
+                }
+                if ((s_l == kPrefix || f_l != 0u) && l < first_end) first_end = l;
+            }
         }
+        spins = 0;
         // Lanes 0 .. last are valid; none before `last` holds a head, so their values simply add up
         // (lane 0 is the nearest tile; the order does not matter for flagless pairs).
         const int last = first_end < kWave ? first_end : kWave - 1;
@@ -594,7 +656,7 @@ __device__ __forceinline__ Seg look_back_seg(const u64* status, uint32_t parity,
 template <typename Cfg, bool VEC>
 __global__ __launch_bounds__(Cfg::BLOCK) void segmented_scan_lookback_kernel(const uint32_t* in, const uint8_t* heads,
                                                                              uint32_t* out, size_t n, uint32_t* header,
-                                                                             u64* status, uint32_t spin_limit) {
+                                                                             u64* status, uint32_t spin_limit, bool help) {
     constexpr int BLOCK = Cfg::BLOCK, VPT = Cfg::VPT;
     constexpr int WAVES = BLOCK / kWave;
     constexpr int TILE = BLOCK * VPT * 4;
@@ -702,11 +764,16 @@ __global__ __launch_bounds__(Cfg::BLOCK) void segmented_scan_lookback_kernel(con
             if (lane == 0) __hip_atomic_store(mine, pack_seg_status(kPrefix, aggregate), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         } else {
             if (lane == 0) __hip_atomic_store(mine, pack_seg_status(kAggregate, aggregate), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            prefix = look_back_seg(status, parity, tile, lane, spin_limit, &header[kHdrReport], &header[kHdrBadWorkspace]);
-            if (lane == 0)
-                __hip_atomic_store(mine, pack_seg_status(kPrefix, seg_combine(prefix, aggregate)), __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
+            prefix = look_back_seg<VEC, TILE>(status, parity, tile, lane, spin_limit, help, in, heads, &header[kHdrReport],
+                                              &header[kHdrBadWorkspace]);
         }
+        // The first publication is complete before the second one and, behind the barrier below, the output
+        // stores are issued: a helper that finds this tile unpublished after its reads have returned has read
+        // input, not output.
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));
+        if (hdr.w == kMagic && tile != 0 && lane == 0)
+            __hip_atomic_store(mine, pack_seg_status(kPrefix, seg_combine(prefix, aggregate)), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
         if (lane == 0) s_tile_prefix_v = prefix.v;
         if (hdr.w == kMagic) clear_other_parity(status, hdr, tile, tiles, lane);
     }
@@ -777,17 +844,35 @@ __device__ __forceinline__ void publish64(u64* lo_word, uint32_t state, u64 valu
     publish(lo_word + 2, state, static_cast<uint32_t>(value >> 32));
 }
 
-// Sum of all tiles before `tile` (> 0). Lane l inspects tile window_end - l: slots 2 t and 2 t + 1.
+// The sum of one whole tile of 64-bit elements, formed by one wavefront from the tile's input (see tile_aggregate).
+template <bool VEC, int TILE>
+__device__ __forceinline__ u64 tile_aggregate64(const u64* in, size_t tile_base, int lane) {
+    u64 acc = 0;
+    if constexpr (VEC) {
+        const u64x2* src = reinterpret_cast<const u64x2*>(in + tile_base) + lane;
+#pragma unroll 1
+        for (int i = 0; i < TILE / 2 / kWave; i += 2) {
+            const u64x2 x = src[static_cast<size_t>(i) * kWave], y = src[static_cast<size_t>(i + 1) * kWave];
+            acc += (x.x + x.y) + (y.x + y.y);
+        }
+    } else {
+        const u64* src = in + tile_base + lane;
+#pragma unroll 1
+        for (int i = 0; i < TILE / kWave; i += 2) acc += src[static_cast<size_t>(i) * kWave] + src[static_cast<size_t>(i + 1) * kWave];
+    }
+    return wave_last_lane64(wave_inclusive_scan64(acc));
+}
+
+// Sum of all tiles before `tile` (> 0). Lane l inspects tile window_end - l: slots 2 t and 2 t + 1. A
+// predecessor that has not answered after spin_limit polls is helped (tile_aggregate64) or, without `help`,
+// reported, as in look_back.
+template <bool VEC, int TILE>
 __device__ __forceinline__ u64 look_back64(const u64* status, uint32_t parity, uint32_t tile, int lane, uint32_t spin_limit,
-                                           uint32_t* report, uint32_t* bad_workspace) {
+                                           bool help, const u64* in, uint32_t* report, uint32_t* bad_workspace) {
     u64 sum = 0;
     uint32_t spins = 0;
     long long window_end = static_cast<long long>(tile) - 1;
     while (true) {
-        if (spins >= spin_limit) {
-            if (lane == 0) __hip_atomic_store(report, tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            break;
-        }
         const long long t = window_end - lane;
         const u64 lo = (t >= 0) ? poll(&status[4 * t + parity]) : pack_status(kPrefix, 0u);
         const u64 hi = (t >= 0) ? poll(&status[4 * t + 2 + parity]) : pack_status(kPrefix, 0u);
@@ -797,15 +882,37 @@ __device__ __forceinline__ u64 look_back64(const u64* status, uint32_t parity, u
             break;
         }
         // halves of two different publications (or one still missing) count as "nothing yet"
-        const uint32_t state = state_lo == state_hi ? state_lo : kInvalid;
-        const u64 value = (lo >> 32) | (hi & 0xffffffff00000000ull);
-        const u64 has_prefix = __ballot(state == kPrefix);
+        uint32_t state = state_lo == state_hi ? state_lo : kInvalid;
+        u64 value = (lo >> 32) | (hi & 0xffffffff00000000ull);
+        u64 has_prefix = __ballot(state == kPrefix);
         const u64 is_invalid = __ballot(state == kInvalid);
-        const u64 needed = has_prefix ? ((2ull << __builtin_ctzll(has_prefix)) - 1ull) : ~0ull;
+        u64 needed = has_prefix ? ((2ull << __builtin_ctzll(has_prefix)) - 1ull) : ~0ull;
         if (is_invalid & needed) {
-            ++spins;
-            continue;
+            if (spins < spin_limit) {
+                ++spins;
+                continue;
+            }
+            if (!help) {
+                if (lane == 0) __hip_atomic_store(report, tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                break;
+            }
+            for (u64 todo = is_invalid & needed; todo != 0; todo &= todo - 1) {
+                const int l = __builtin_ctzll(todo);
+                const u64 formed = tile_aggregate64<VEC, TILE>(in, static_cast<size_t>(window_end - l) * TILE, lane);
+                // As in look_back. A tile stores output only after both halves of its prefix are published, so a
+                // pair that is still missing or mixed here means that `formed` is the sum of its input.
+                const u64 lo2 = poll(&status[4 * (window_end - l) + parity]), hi2 = poll(&status[4 * (window_end - l) + 2 + parity]);
+                const uint32_t s2 = static_cast<uint32_t>(lo2);
+                const bool published = s2 == static_cast<uint32_t>(hi2) && s2 != kInvalid;
+                if (lane == l) {
+                    state = published ? s2 : kAggregate;
+                    value = published ? ((lo2 >> 32) | (hi2 & 0xffffffff00000000ull)) : formed;
+                }
+            }
+            has_prefix = __ballot(state == kPrefix);
+            needed = has_prefix ? ((2ull << __builtin_ctzll(has_prefix)) - 1ull) : ~0ull;
         }
+        spins = 0;
         const u64 contrib = ((needed >> lane) & 1ull) ? value : 0ull;
         sum += wave_last_lane64(wave_inclusive_scan64(contrib));
         if (has_prefix) break;
@@ -818,7 +925,7 @@ __device__ __forceinline__ u64 look_back64(const u64* status, uint32_t parity, u
 // which is what the workspace holds per 32768 elements.
 template <typename Cfg, bool VEC>
 __global__ __launch_bounds__(Cfg::BLOCK) void scan64_lookback_kernel(const u64* in, u64* out, size_t n, uint32_t* header,
-                                                                     u64* status, uint32_t spin_limit) {
+                                                                     u64* status, uint32_t spin_limit, bool help) {
     constexpr int BLOCK = Cfg::BLOCK, VPT = Cfg::VPT;
     constexpr int WAVES = BLOCK / kWave;
     constexpr int TILE = BLOCK * VPT * 2;
@@ -884,19 +991,34 @@ __global__ __launch_bounds__(Cfg::BLOCK) void scan64_lookback_kernel(const u64* 
         if (hdr.w != kMagic) {  // not an initialised workspace: report, touch nothing else
             if (lane == 0) __hip_atomic_store(&header[kHdrBadWorkspace], tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         } else {
+            // Counted in before anything is published, as in scan_lookback_kernel: with helping the last tile's
+            // look-back can be complete before every tile has read the header.
+            if (lane == 0) __hip_atomic_fetch_add(&header[kHdrDone], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (tile == 0) {
                 if (lane == 0) publish64(mine, kPrefix, aggregate);
             } else {
                 if (lane == 0) publish64(mine, kAggregate, aggregate);
-                prefix = look_back64(status, parity, tile, lane, spin_limit, &header[kHdrReport], &header[kHdrBadWorkspace]);
-                if (lane == 0) publish64(mine, kPrefix, aggregate + prefix);
+                prefix = look_back64<VEC, TILE>(status, parity, tile, lane, spin_limit, help, in, &header[kHdrReport],
+                                                &header[kHdrBadWorkspace]);
             }
-            // The workspace protocol counts status slots: this tile's are 2 t and 2 t + 1 of 2 * tiles. The last
-            // tile closes the call: every earlier tile has published by now (its look-back saw them all), so
-            // every tile has read the header.
+            // The first publication is complete before the second one and the output stores are issued (see
+            // scan_lookback_kernel).
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));
+            if (tile != 0 && lane == 0) publish64(mine, kPrefix, aggregate + prefix);
+            // The workspace protocol counts status slots: this tile's are 2 t and 2 t + 1 of 2 * tiles.
             clear_other_parity(status, hdr, 2 * tile, 2 * tiles, lane);
             clear_other_parity(status, hdr, 2 * tile + 1, 2 * tiles, lane);
-            if (tile == tiles - 1 && lane == 0) close_call(header, hdr, 2 * tiles);
+            if (tile == tiles - 1 && lane == 0) {  // closes the call once every tile has read the header
+                uint32_t waited = 0;
+                while (__hip_atomic_load(&header[kHdrDone], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != tiles) {
+                    if (++waited > kSpinLimit) {
+                        __hip_atomic_store(&header[kHdrReport], tile + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(8);
+                }
+                close_call(header, hdr, 2 * tiles);
+            }
         }
         if (lane == 0) s_tile_prefix = prefix;
     }
@@ -1056,8 +1178,20 @@ int launch_scan(const uint32_t* in, uint32_t* out, size_t n, void* ws, size_t ws
     return launch_cfg<BigCfg, true>(in, out, n, header, status, flags, limit, s);
 }
 
+// The limit on the polls of one look-back window for the kinds of scan that take only the no-help flag.
+static int help_and_limit(const char* who, unsigned flags, long long spin_limit, bool* help, uint32_t* limit) {
+    if ((flags & ~kFlagNoHelp) != 0) return fail(1, "%s: unknown flag bits 0x%x (only PRISM_SCAN_NO_HELP applies)", who, flags);
+    *help = (flags & kFlagNoHelp) == 0;
+    *limit = spin_limit < 0 ? (*help ? kHelpAfter : kSpinLimit)
+                            : static_cast<uint32_t>(spin_limit > 0xffffffffll ? 0xffffffffll : spin_limit);
+    return 0;
+}
+
 int launch_segmented_scan(const uint32_t* in, const uint8_t* heads, uint32_t* out, size_t n, void* ws, size_t ws_bytes,
-                          hipStream_t s) {
+                          unsigned flags, long long spin_limit, hipStream_t s) {
+    bool help = true;
+    uint32_t limit = 0;
+    if (int rc = help_and_limit("prism_segmented_scan", flags, spin_limit, &help, &limit)) return rc;
     if (n == 0) return 0;
     if (in == nullptr || out == nullptr || heads == nullptr || ws == nullptr)
         return fail(1, "prism_segmented_scan: null pointer with n=%zu", n);
@@ -1081,15 +1215,19 @@ int launch_segmented_scan(const uint32_t* in, const uint8_t* heads, uint32_t* ou
     const size_t tiles = ceil_div(n, static_cast<size_t>(small ? tile_elems<SmallCfg>() : tile_elems<BigCfg>()));
     const dim3 grid(static_cast<unsigned>(tiles));
     if (!vec)
-        segmented_scan_lookback_kernel<SmallCfg, false><<<grid, dim3(SmallCfg::BLOCK), 0, s>>>(in, heads, out, n, header, status, kSpinLimit);
+        segmented_scan_lookback_kernel<SmallCfg, false><<<grid, dim3(SmallCfg::BLOCK), 0, s>>>(in, heads, out, n, header, status, limit, help);
     else if (small)
-        segmented_scan_lookback_kernel<SmallCfg, true><<<grid, dim3(SmallCfg::BLOCK), 0, s>>>(in, heads, out, n, header, status, kSpinLimit);
+        segmented_scan_lookback_kernel<SmallCfg, true><<<grid, dim3(SmallCfg::BLOCK), 0, s>>>(in, heads, out, n, header, status, limit, help);
     else
-        segmented_scan_lookback_kernel<BigCfg, true><<<grid, dim3(BigCfg::BLOCK), 0, s>>>(in, heads, out, n, header, status, kSpinLimit);
+        segmented_scan_lookback_kernel<BigCfg, true><<<grid, dim3(BigCfg::BLOCK), 0, s>>>(in, heads, out, n, header, status, limit, help);
     return check_launch("segmented_scan_lookback_kernel");
 }
 
-int launch_scan64(const unsigned long long* in, unsigned long long* out, size_t n, void* ws, size_t ws_bytes, hipStream_t s) {
+int launch_scan64(const unsigned long long* in, unsigned long long* out, size_t n, void* ws, size_t ws_bytes, unsigned flags,
+                  long long spin_limit, hipStream_t s) {
+    bool help = true;
+    uint32_t limit = 0;
+    if (int rc = help_and_limit("prism_scan_i64", flags, spin_limit, &help, &limit)) return rc;
     if (n == 0) return 0;
     if (in == nullptr || out == nullptr || ws == nullptr) return fail(1, "prism_scan_i64: null pointer with n=%zu", n);
     if ((reinterpret_cast<uintptr_t>(in) & 7u) != 0 || (reinterpret_cast<uintptr_t>(out) & 7u) != 0)
@@ -1109,9 +1247,9 @@ int launch_scan64(const unsigned long long* in, unsigned long long* out, size_t 
     u64* status = reinterpret_cast<u64*>(static_cast<char*>(ws) + kHeaderBytes);
     const dim3 grid(static_cast<unsigned>(tiles)), block(BigCfg::BLOCK);
     if (aligned16(in) && aligned16(out))
-        scan64_lookback_kernel<BigCfg, true><<<grid, block, 0, s>>>(in, out, n, header, status, kSpinLimit);
+        scan64_lookback_kernel<BigCfg, true><<<grid, block, 0, s>>>(in, out, n, header, status, limit, help);
     else
-        scan64_lookback_kernel<BigCfg, false><<<grid, block, 0, s>>>(in, out, n, header, status, kSpinLimit);
+        scan64_lookback_kernel<BigCfg, false><<<grid, block, 0, s>>>(in, out, n, header, status, limit, help);
     return check_launch("scan64_lookback_kernel");
 }
 

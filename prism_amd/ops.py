@@ -185,7 +185,7 @@ def scan(inp: "torch.Tensor", out: Optional["torch.Tensor"] = None,
     if op not in SCAN_OP:
         raise ValueError("scan: op must be 'sum', 'max' or 'min'")
     if inp.dtype in (torch.int64, torch.uint64):  # 64-bit elements: inclusive sums modulo 2^64 only
-        if op != "sum" or exclusive or ticket_order or spin_limit != -1 or not help:
+        if op != "sum" or exclusive or ticket_order:
             raise ValueError("scan: 64-bit elements support the inclusive sum in workgroup-id order only")
         n = inp.numel()
         if out is None:
@@ -193,7 +193,8 @@ def scan(inp: "torch.Tensor", out: Optional["torch.Tensor"] = None,
         _need(out, (inp.dtype,), n, "out")
         if workspace is None:
             workspace = new_scan_workspace(n, inp.device)
-        _check(_lib.load().prism_scan_i64(_ptr(inp), _ptr(out), n, _ptr(workspace), _ws_bytes(workspace), _stream()), "scan")
+        _check(_lib.load().prism_scan_i64_ex(_ptr(inp), _ptr(out), n, _ptr(workspace), _ws_bytes(workspace),
+                                             0 if help else SCAN_NO_HELP, int(spin_limit), _stream()), "scan")
         if check and n > 0:
             scan_status(workspace)
         return out
@@ -216,9 +217,11 @@ def scan(inp: "torch.Tensor", out: Optional["torch.Tensor"] = None,
 
 
 def segmented_scan(inp: "torch.Tensor", heads: "torch.Tensor", out: Optional["torch.Tensor"] = None,
-                   workspace: Optional["torch.Tensor"] = None, check: bool = True) -> "torch.Tensor":
+                   workspace: Optional["torch.Tensor"] = None, check: bool = True, spin_limit: int = -1,
+                   help: bool = True) -> "torch.Tensor":
     """Inclusive sums modulo 2^32 that start again at every element whose byte in `heads` (uint8 / bool, one per
-    element) is non-zero; element 0 always starts a segment. out may be inp. workspace and check as for scan()."""
+    element) is non-zero; element 0 always starts a segment. out may be inp. workspace, check, spin_limit and help
+    as for scan()."""
     _need(inp, (torch.int32, torch.uint32), 0, "inp")
     n = inp.numel()
     _need(heads, (torch.uint8, torch.bool), n, "heads")
@@ -227,8 +230,8 @@ def segmented_scan(inp: "torch.Tensor", heads: "torch.Tensor", out: Optional["to
     _need(out, (inp.dtype,), n, "out")
     if workspace is None:
         workspace = new_scan_workspace(n, inp.device)
-    _check(_lib.load().prism_segmented_scan_i32(_ptr(inp), _ptr(heads), _ptr(out), n, _ptr(workspace),
-                                                _ws_bytes(workspace), _stream()), "segmented_scan")
+    _check(_lib.load().prism_segmented_scan_i32_ex(_ptr(inp), _ptr(heads), _ptr(out), n, _ptr(workspace), _ws_bytes(workspace),
+                                                   0 if help else SCAN_NO_HELP, int(spin_limit), _stream()), "segmented_scan")
     if check and n > 0:
         scan_status(workspace)
     return out

@@ -487,6 +487,59 @@ def test_scan_of_64_bit_elements_2pow29_properties(prism):
     assert int(out[-1]) == ((total + 2**63) % 2**64) - 2**63
 
 
+def test_segmented_and_64_bit_scans_help_their_predecessors_too(prism, oracle):
+    """The spin limit forced to 0, as in test_scan_that_stops_waiting_helps_its_predecessors, for the other two
+    kinds of scan. Segmented: the helper forms a tile's (head seen, sum) pair from its input and head bytes, for
+    segments much shorter than a tile (nearly every tile holds a head and ends the walk), about a tile long and
+    many tiles long (walks across helped, flagless tiles), none at all; both tile shapes, unaligned views, in
+    place. 64-bit: values that use all 64 bits, both alignments, in place. Bit for bit against the serial loops;
+    nothing is reported, and without helping the same calls are errors."""
+    for n in ((1 << 22) + 77, (1 << 25) + 65536 * 5 + 3):
+        x = oracle.gen_scan(n, seed=n % 1000)
+        xd = dev(x)
+        ws = prism.new_scan_workspace(n)
+        for mean in (6, 40_000, 3_000_000):
+            h = oracle.gen_heads(n, mean, seed=int(mean) % 97)
+            hd = dev(h)
+            want = oracle.segmented_scan_cpu(x, h)
+            print(f"segmented scan n={n} mean segment {mean} spin_limit=0", flush=True)
+            out = prism.segmented_scan(xd, hd, workspace=ws, spin_limit=0)
+            assert np.array_equal(host(out), want), mean
+            buf = xd.clone()
+            prism.segmented_scan(buf, hd, buf, workspace=ws, spin_limit=0)  # in place
+            assert np.array_equal(host(buf), want), mean
+        assert np.array_equal(host(prism.segmented_scan(xd, dev(np.zeros(n, np.uint8)), workspace=ws, spin_limit=0)), oracle.scan_cpu(x))
+        h = oracle.gen_heads(n, 500, seed=5)
+        x1 = dev(np.concatenate([[0], x]).astype(np.int32))[1:]
+        h1 = dev(np.concatenate([[9], h]).astype(np.uint8))[1:]
+        y = torch.zeros(n + 1, dtype=torch.int32, device=DEV)
+        prism.segmented_scan(x1, h1, y[1:], workspace=ws, spin_limit=0)  # element-wise loads, the small tile
+        assert np.array_equal(host(y)[1:], oracle.segmented_scan_cpu(x, h))
+        with pytest.raises(prism.ScanOrderError, match="gave up waiting"):
+            prism.segmented_scan(xd, dev(np.zeros(n, np.uint8)), workspace=ws, spin_limit=0, help=False)
+        assert np.array_equal(host(prism.segmented_scan(xd, dev(h), workspace=ws)), oracle.segmented_scan_cpu(x, h))
+
+        rng = np.random.default_rng(n % 211)
+        m = n // 2
+        x64 = rng.integers(-2**62, 2**62, m, dtype=np.int64)
+        want64 = oracle.scan_i64_cpu(x64)
+        x64d = dev(x64)
+        print(f"64-bit scan n={m} spin_limit=0", flush=True)
+        assert np.array_equal(host(prism.scan(x64d, workspace=ws, spin_limit=0)), want64)
+        for _ in range(2):
+            buf = x64d.clone()
+            prism.scan(buf, buf, workspace=ws, spin_limit=0)
+            assert np.array_equal(host(buf), want64)
+        x1 = dev(np.concatenate([[0], x64]).astype(np.int64))[1:]
+        y = torch.zeros(m + 1, dtype=torch.int64, device=DEV)
+        prism.scan(x1, y[1:], workspace=ws, spin_limit=0)  # 8-byte-aligned views
+        assert np.array_equal(host(y)[1:], want64)
+        with pytest.raises(prism.ScanOrderError, match="gave up waiting"):
+            prism.scan(x64d, workspace=ws, spin_limit=0, help=False)
+        assert np.array_equal(host(prism.scan(x64d, workspace=ws)), want64)
+        prism.scan_status(ws)
+
+
 def test_scan_2pow30_properties(prism):
     """Full BASELINE size (4 GiB in, 4 GiB out): checked on the device through
     size-independent properties - first element, the difference invariant
