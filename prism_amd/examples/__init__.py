@@ -35,7 +35,7 @@ KERNELS: Dict[str, Tuple[str, int, Optional[List[int]]]] = {
     "two_roles": ("basics", 256, None),
     "gather_columns": ("basics", 256, None),
     "handed_over_gemm": ("handover", 320, None),
-    "handed_over_gemm_big": ("handover", 768, None),
+    "handed_over_gemm_big": ("handover", 512, None),
     "handed_over_sgemm": ("handover", 768, None),
     "pipelined_sgemm": ("pipelined", 1024, None),
     "pipelined_gemm_bf16": ("pipelined", 512, None),

@@ -8,6 +8,19 @@
 // array) in the low byte, the round above it; the launcher's <name>_status call reads and clears it
 __device__ unsigned int __prism_handover_report = 0;
 #endif
+#ifndef PRISM_LDS_WORD_HELPERS
+#define PRISM_LDS_WORD_HELPERS
+// one LDS word read / counted up without the compiler seeing an LDS access (the address is the low half of the
+// generic one); the memory clobber keeps every memory operation on its side of the call
+__device__ __forceinline__ unsigned int __prism_lds_peek(const unsigned int* word) {
+    unsigned int value;
+    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(value) : "v"((unsigned int)(unsigned long long)word) : "memory");
+    return value;
+}
+__device__ __forceinline__ void __prism_lds_count(unsigned int* word) {
+    asm volatile("ds_add_u32 %0, %1" :: "v"((unsigned int)(unsigned long long)word), "v"(1u) : "memory");
+}
+#endif
 __global__ void handed_over_gemm(const __bf16* P, const __bf16* Q, float* D, int N, int K, int tiles_n) {
     extern __shared__ __align__(128) char __smem[];
     int __block_id_0 = blockIdx.x;
@@ -26,21 +39,25 @@ __global__ void handed_over_gemm(const __bf16* P, const __bf16* Q, float* D, int
                     __shared__ __bf16 p_first[2048];
                     __shared__ unsigned int __full_p_first, __empty_p_first;
                     int __round_p_first = 0;
+                    bool __pending_p_first = false;  // filled by this wavefront and not announced yet
                     if (threadIdx.x == 0) { __full_p_first = 0; __empty_p_first = 0; }
                     __syncthreads();
                     __shared__ __bf16 q_first[2048];
                     __shared__ unsigned int __full_q_first, __empty_q_first;
                     int __round_q_first = 0;
+                    bool __pending_q_first = false;  // filled by this wavefront and not announced yet
                     if (threadIdx.x == 0) { __full_q_first = 0; __empty_q_first = 0; }
                     __syncthreads();
                     __shared__ __bf16 p_second[2048];
                     __shared__ unsigned int __full_p_second, __empty_p_second;
                     int __round_p_second = 0;
+                    bool __pending_p_second = false;  // filled by this wavefront and not announced yet
                     if (threadIdx.x == 0) { __full_p_second = 0; __empty_p_second = 0; }
                     __syncthreads();
                     __shared__ __bf16 q_second[2048];
                     __shared__ unsigned int __full_q_second, __empty_q_second;
                     int __round_q_second = 0;
+                    bool __pending_q_second = false;  // filled by this wavefront and not announced yet
                     if (threadIdx.x == 0) { __full_q_second = 0; __empty_q_second = 0; }
                     __syncthreads();
                     float acc[16] = {0};
@@ -66,59 +83,155 @@ __global__ void handed_over_gemm(const __bf16* P, const __bf16* Q, float* D, int
                                                     {
                                                         int __spin = 0;
                                                         const unsigned int __need = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__round_p_first * 4)));
+                                                        if (static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__prism_lds_peek(&__empty_p_first)))) < __need) {
+                                                            if (__pending_p_first) {
+                                                                __builtin_amdgcn_s_waitcnt(0);
+                                                                if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_p_first);
+                                                                __pending_p_first = false;
+                                                            }
+                                                            if (__pending_p_second) {
+                                                                __builtin_amdgcn_s_waitcnt(0);
+                                                                if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_p_second);
+                                                                __pending_p_second = false;
+                                                            }
+                                                            if (__pending_q_first) {
+                                                                __builtin_amdgcn_s_waitcnt(0);
+                                                                if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_q_first);
+                                                                __pending_q_first = false;
+                                                            }
+                                                            if (__pending_q_second) {
+                                                                __builtin_amdgcn_s_waitcnt(0);
+                                                                if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_q_second);
+                                                                __pending_q_second = false;
+                                                            }
+                                                        }
                                                         #pragma nounroll
-                                                        for (; __spin < 65536 && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__hip_atomic_load(&__empty_p_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)))) < __need; ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                        for (; __spin < 65536 && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__prism_lds_peek(&__empty_p_first)))) < __need; ++__spin) __builtin_amdgcn_s_sleep(1);
                                                         if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 1u | (static_cast<unsigned int>(__round_p_first) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                                                     }
-                                                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                                                     {
                                                         int __spin = 0;
                                                         const unsigned int __need = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__round_q_first * 4)));
+                                                        if (static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__prism_lds_peek(&__empty_q_first)))) < __need) {
+                                                            if (__pending_p_first) {
+                                                                __builtin_amdgcn_s_waitcnt(0);
+                                                                if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_p_first);
+                                                                __pending_p_first = false;
+                                                            }
+                                                            if (__pending_p_second) {
+                                                                __builtin_amdgcn_s_waitcnt(0);
+                                                                if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_p_second);
+                                                                __pending_p_second = false;
+                                                            }
+                                                            if (__pending_q_first) {
+                                                                __builtin_amdgcn_s_waitcnt(0);
+                                                                if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_q_first);
+                                                                __pending_q_first = false;
+                                                            }
+                                                            if (__pending_q_second) {
+                                                                __builtin_amdgcn_s_waitcnt(0);
+                                                                if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_q_second);
+                                                                __pending_q_second = false;
+                                                            }
+                                                        }
                                                         #pragma nounroll
-                                                        for (; __spin < 65536 && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__hip_atomic_load(&__empty_q_first, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)))) < __need; ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                        for (; __spin < 65536 && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__prism_lds_peek(&__empty_q_first)))) < __need; ++__spin) __builtin_amdgcn_s_sleep(1);
                                                         if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 5u | (static_cast<unsigned int>(__round_q_first) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                                                     }
-                                                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                                                     for (int part = 0; part < 4; part++) {
-                                                        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&P_rows[(((((16 * part) + row) * K) + k0) + k8)]), (__attribute__((address_space(3))) void*)(&p_first_fill[(512 * part)]), 16, 0, 0);
-                                                        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&Q_rows[(((((16 * part) + row) * K) + k0) + k8)]), (__attribute__((address_space(3))) void*)(&q_first_fill[(512 * part)]), 16, 0, 0);
+                                                        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&P_rows[(((((16 * part) + row) * K) + k0) + k8)]), (__attribute__((address_space(3))) void*)(unsigned int)(unsigned long long)(&p_first_fill[(512 * part)]), 16, 0, 0);
+                                                        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&Q_rows[(((((16 * part) + row) * K) + k0) + k8)]), (__attribute__((address_space(3))) void*)(unsigned int)(unsigned long long)(&q_first_fill[(512 * part)]), 16, 0, 0);
                                                     }
-                                                    __builtin_amdgcn_s_waitcnt(0);
-                                                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-                                                    if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__full_p_first, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                                                     __round_p_first += 1;
-                                                    __builtin_amdgcn_s_waitcnt(0);
-                                                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-                                                    if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__full_q_first, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                                                     __round_q_first += 1;
+                                                    if (__pending_p_second) {
+                                                        __builtin_amdgcn_s_waitcnt(3960);  // vmcnt(8)
+                                                        if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_p_second);
+                                                        __pending_p_second = false;
+                                                    }
+                                                    if (__pending_q_second) {
+                                                        __builtin_amdgcn_s_waitcnt(3960);  // vmcnt(8)
+                                                        if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_q_second);
+                                                        __pending_q_second = false;
+                                                    }
+                                                    __pending_p_first = true;
+                                                    __pending_q_first = true;
                                                     {
                                                         int __spin = 0;
                                                         const unsigned int __need = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__round_p_second * 4)));
+                                                        if (static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__prism_lds_peek(&__empty_p_second)))) < __need) {
+                                                            if (__pending_p_first) {
+                                                                __builtin_amdgcn_s_waitcnt(0);
+                                                                if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_p_first);
+                                                                __pending_p_first = false;
+                                                            }
+                                                            if (__pending_p_second) {
+                                                                __builtin_amdgcn_s_waitcnt(0);
+                                                                if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_p_second);
+                                                                __pending_p_second = false;
+                                                            }
+                                                            if (__pending_q_first) {
+                                                                __builtin_amdgcn_s_waitcnt(0);
+                                                                if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_q_first);
+                                                                __pending_q_first = false;
+                                                            }
+                                                            if (__pending_q_second) {
+                                                                __builtin_amdgcn_s_waitcnt(0);
+                                                                if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_q_second);
+                                                                __pending_q_second = false;
+                                                            }
+                                                        }
                                                         #pragma nounroll
-                                                        for (; __spin < 65536 && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__hip_atomic_load(&__empty_p_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)))) < __need; ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                        for (; __spin < 65536 && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__prism_lds_peek(&__empty_p_second)))) < __need; ++__spin) __builtin_amdgcn_s_sleep(1);
                                                         if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 3u | (static_cast<unsigned int>(__round_p_second) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                                                     }
-                                                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                                                     {
                                                         int __spin = 0;
                                                         const unsigned int __need = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__round_q_second * 4)));
+                                                        if (static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__prism_lds_peek(&__empty_q_second)))) < __need) {
+                                                            if (__pending_p_first) {
+                                                                __builtin_amdgcn_s_waitcnt(0);
+                                                                if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_p_first);
+                                                                __pending_p_first = false;
+                                                            }
+                                                            if (__pending_p_second) {
+                                                                __builtin_amdgcn_s_waitcnt(0);
+                                                                if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_p_second);
+                                                                __pending_p_second = false;
+                                                            }
+                                                            if (__pending_q_first) {
+                                                                __builtin_amdgcn_s_waitcnt(0);
+                                                                if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_q_first);
+                                                                __pending_q_first = false;
+                                                            }
+                                                            if (__pending_q_second) {
+                                                                __builtin_amdgcn_s_waitcnt(0);
+                                                                if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_q_second);
+                                                                __pending_q_second = false;
+                                                            }
+                                                        }
                                                         #pragma nounroll
-                                                        for (; __spin < 65536 && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__hip_atomic_load(&__empty_q_second, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)))) < __need; ++__spin) __builtin_amdgcn_s_sleep(1);
+                                                        for (; __spin < 65536 && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__prism_lds_peek(&__empty_q_second)))) < __need; ++__spin) __builtin_amdgcn_s_sleep(1);
                                                         if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 7u | (static_cast<unsigned int>(__round_q_second) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                                                     }
-                                                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                                                     for (int part = 0; part < 4; part++) {
-                                                        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&P_rows[((((((16 * part) + row) * K) + k0) + 32) + k8)]), (__attribute__((address_space(3))) void*)(&p_second_fill[(512 * part)]), 16, 0, 0);
-                                                        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&Q_rows[((((((16 * part) + row) * K) + k0) + 32) + k8)]), (__attribute__((address_space(3))) void*)(&q_second_fill[(512 * part)]), 16, 0, 0);
+                                                        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&P_rows[((((((16 * part) + row) * K) + k0) + 32) + k8)]), (__attribute__((address_space(3))) void*)(unsigned int)(unsigned long long)(&p_second_fill[(512 * part)]), 16, 0, 0);
+                                                        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&Q_rows[((((((16 * part) + row) * K) + k0) + 32) + k8)]), (__attribute__((address_space(3))) void*)(unsigned int)(unsigned long long)(&q_second_fill[(512 * part)]), 16, 0, 0);
                                                     }
-                                                    __builtin_amdgcn_s_waitcnt(0);
-                                                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-                                                    if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__full_p_second, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                                                     __round_p_second += 1;
-                                                    __builtin_amdgcn_s_waitcnt(0);
-                                                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-                                                    if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_add(&__full_q_second, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                                                     __round_q_second += 1;
+                                                    if (__pending_p_first) {
+                                                        __builtin_amdgcn_s_waitcnt(3960);  // vmcnt(8)
+                                                        if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_p_first);
+                                                        __pending_p_first = false;
+                                                    }
+                                                    if (__pending_q_first) {
+                                                        __builtin_amdgcn_s_waitcnt(3960);  // vmcnt(8)
+                                                        if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_q_first);
+                                                        __pending_q_first = false;
+                                                    }
+                                                    __pending_p_second = true;
+                                                    __pending_q_second = true;
                                                 }
                                             }
                                         }
@@ -216,6 +329,26 @@ __global__ void handed_over_gemm(const __bf16* P, const __bf16* Q, float* D, int
                                 }
                             }
                         }
+                    }
+                    if (__pending_p_first) {
+                        __builtin_amdgcn_s_waitcnt(0);
+                        if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_p_first);
+                        __pending_p_first = false;
+                    }
+                    if (__pending_p_second) {
+                        __builtin_amdgcn_s_waitcnt(0);
+                        if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_p_second);
+                        __pending_p_second = false;
+                    }
+                    if (__pending_q_first) {
+                        __builtin_amdgcn_s_waitcnt(0);
+                        if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_q_first);
+                        __pending_q_first = false;
+                    }
+                    if (__pending_q_second) {
+                        __builtin_amdgcn_s_waitcnt(0);
+                        if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_q_second);
+                        __pending_q_second = false;
                     }
                     {
                         float* D_mine = D_tile + (0);

@@ -84,8 +84,12 @@ def handed_over_gemm(P: ptr(const(bf16)) @ grid[1], Q: ptr(const(bf16)) @ grid[1
                                                 D_mine[(16 * wave + 4 * (lane / 16) + v) * N + 16 * n + lane % 16] = acc[4 * n + v]
 
 
-# The same hand-over at full size: a 128 x 256 tile per workgroup, four producer and eight consumer wavefronts,
-# two slots of 64 k (48 KiB each: 128 rows of P, then 256 rows of Q, 128-byte rows).
+# The same hand-over at full size: a 128 x 256 tile per workgroup, four producer and four consumer wavefronts,
+# three slots of 64 k (48 KiB each: 128 rows of P, then 256 rows of Q, 128-byte rows). The producers fill the
+# slots in turn; because one case fills several arrays, the generator announces a filling only when the next
+# one's loads are on their way, so that two fillings are in flight while the consumers multiply the third.
+# Measured at 8192^3: eight consumers of 64 x 64 and two slots 1000 TFLOP/s, four of 64 x 128 and two slots
+# 1030, four of 64 x 128 and three slots 1120.
 
 @requires(thread[256])
 @prism("device")
@@ -110,15 +114,15 @@ def fill_slot(slot: ptr(bf16) @ thread[256], P_from: ptr(const(bf16)) @ block[1]
     return
 
 
-@requires(thread[512])
+@requires(thread[256])
 @prism("device")
 def multiply_slot(acc: ptr(float) @ thread[1], slot: ptr(const(bf16)) @ block[1]):
-    """Eight wavefronts, two down and four across, each adding its 64 x 64 part of (P part)(Q part)^T to acc: two
-    k-steps of 4 x 4 matrix instructions of 16 x 16 x 32, acc[(4 i + j) * 4 + v] = D[16 i + 4 (lane / 16) + v][16 j + lane % 16]."""
-    with group(thread[512]):
+    """Four wavefronts, two down and two across, each adding its 64 x 128 part of (P part)(Q part)^T to acc: two
+    k-steps of 4 x 8 matrix instructions of 16 x 16 x 32, acc[(8 i + j) * 4 + v] = D[16 i + 4 (lane / 16) + v][16 j + lane % 16]."""
+    with group(thread[256]):
         wave: int @ thread[64] = id()
-        row0: int @ thread[64] = 64 * (wave / 4)
-        col0: int @ thread[64] = 64 * (wave % 4)
+        row0: int @ thread[64] = 64 * (wave / 2)
+        col0: int @ thread[64] = 128 * (wave % 2)
         with group(thread[64]):
             lane: int @ thread[1] = id()
             r: int @ thread[1] = lane % 16
@@ -127,24 +131,27 @@ def multiply_slot(acc: ptr(float) @ thread[1], slot: ptr(const(bf16)) @ block[1]
                 k8: int @ thread[1] = 8 * ((4 * kk + lane / 16) ^ ((r / 2) % 8))
                 for i in range(4):
                     a[i] = float4_cast(slot[(row0 + 16 * i + r) * 64 + k8])
-                for j in range(4):
+                for j in range(8):
                     b: float4 @ thread[1] = float4_cast(slot[8192 + (col0 + 16 * j + r) * 64 + k8])
                     for i in range(4):
                         intrinsic.mfma_f32_16x16x32_bf16(
-                            a[i], b, acc[(4 * i + j) * 4], acc[(4 * i + j) * 4 + 1], acc[(4 * i + j) * 4 + 2], acc[(4 * i + j) * 4 + 3],
-                            out=[acc[(4 * i + j) * 4], acc[(4 * i + j) * 4 + 1], acc[(4 * i + j) * 4 + 2], acc[(4 * i + j) * 4 + 3]])
+                            a[i], b, acc[(8 * i + j) * 4], acc[(8 * i + j) * 4 + 1], acc[(8 * i + j) * 4 + 2], acc[(8 * i + j) * 4 + 3],
+                            out=[acc[(8 * i + j) * 4], acc[(8 * i + j) * 4 + 1], acc[(8 * i + j) * 4 + 2], acc[(8 * i + j) * 4 + 3]])
     return
 
 
-@attr("__launch_bounds__(768)")
-@requires(grid[1], block[1], thread[768])
+@attr("__launch_bounds__(512)")
+@requires(grid[1], block[1], thread[512])
 @prism("global")
 def handed_over_gemm_big(P: ptr(const(bf16)) @ grid[1], Q: ptr(const(bf16)) @ grid[1], D: ptr(float) @ grid[1],
                          N: int @ grid[1], K: int @ grid[1], tiles_m: int @ grid[1], tiles_n: int @ grid[1]):
-    """D = P Q^T on 128 x 256 tiles: 256 producer threads keep two slots filled, 512 consumer threads multiply
-    them. K is a multiple of 128, M of 1024 and N of 256 (tiles_m = M / 128 a multiple of 8, tiles_n = N / 256).
+    """D = P Q^T on 128 x 256 tiles: 256 producer threads keep three slots filled, 256 consumer threads multiply
+    them. K is a multiple of 64, M of 1024 and N of 256 (tiles_m = M / 128 a multiple of 8, tiles_n = N / 256).
     Workgroups are dealt to the eight XCDs in turn; the tile order gives the workgroups that run on one XCD at the
-    same time a patch of eight tile rows by four tile columns, so that they share their panels in its L2."""
+    same time a patch of eight tile rows by four tile columns, so that they share their panels in its L2.
+    A trip of the loop covers 192 k. Where K ends inside a trip the producers fill the remaining slots with the
+    first K tiles once more (every trip issues the same loads, which is what lets the generator count them) and
+    the consumers leave those slots out."""
     per_xcd: const(int) @ block[1] = (tiles_m * tiles_n) / 8
     t: const(int) @ block[1] = (id() % 8) * per_xcd + id() / 8
     tile_r: const(int) @ block[1] = 8 * (t / (8 * tiles_n)) + t % 8
@@ -155,31 +162,39 @@ def handed_over_gemm_big(P: ptr(const(bf16)) @ grid[1], Q: ptr(const(bf16)) @ gr
                 with group(block[1]):
                     first: shared(bf16[24576], static=True) @ block[1]
                     second: shared(bf16[24576], static=True) @ block[1]
-                    acc: float[64] @ thread[1] = {0}
-                    for k0 in range(0, K, 128):
+                    third: shared(bf16[24576], static=True) @ block[1]
+                    acc: float[128] @ thread[1] = {0}
+                    for k0 in range(0, K, 192):
+                        k1: const(int) @ block[1] = (k0 + 64) % K
+                        k2: const(int) @ block[1] = (k0 + 128) % K
                         with claim(first, p=thread[256], offset=0) as first_fill:
                             with claim(second, p=thread[256], offset=0) as second_fill:
-                                match split(thread):
-                                    case 256:
-                                        fill_slot(first_fill, P_rows, Q_rows, K, k0)
-                                        fill_slot(second_fill, P_rows, Q_rows, K, k0 + 64)
-                                    case 512:
-                                        multiply_slot(acc, first)
-                                        multiply_slot(acc, second)
+                                with claim(third, p=thread[256], offset=0) as third_fill:
+                                    match split(thread):
+                                        case 256:
+                                            fill_slot(first_fill, P_rows, Q_rows, K, k0)
+                                            fill_slot(second_fill, P_rows, Q_rows, K, k1)
+                                            fill_slot(third_fill, P_rows, Q_rows, K, k2)
+                                        case 256:
+                                            multiply_slot(acc, first)
+                                            if k0 + 64 < K:
+                                                multiply_slot(acc, second)
+                                            if k0 + 128 < K:
+                                                multiply_slot(acc, third)
                     with partition(D_tile, p=thread[1], offset=0) as D_mine:
                         match split(thread):
                             case 256:
                                 pass
-                            case 512:
+                            case 256:
                                 wave: int @ thread[64] = id()
                                 with group(thread[64]):
                                     lane: int @ thread[1] = id()
                                     with group(thread[1]):
                                         for i in range(4):
-                                            for j in range(4):
+                                            for j in range(8):
                                                 for v in range(4):
-                                                    D_mine[(64 * (wave / 4) + 16 * i + 4 * (lane / 16) + v) * N
-                                                           + 64 * (wave % 4) + 16 * j + lane % 16] = acc[(4 * i + j) * 4 + v]
+                                                    D_mine[(64 * (wave / 2) + 16 * i + 4 * (lane / 16) + v) * N
+                                                           + 128 * (wave % 2) + 16 * j + lane % 16] = acc[(8 * i + j) * 4 + v]
 
 
 # SGEMM the same way: C = alpha A B + beta C (row-major fp32) on the fp32 matrix instruction, 128 x 256 tiles,

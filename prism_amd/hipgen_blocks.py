@@ -172,6 +172,58 @@ def _const_pointer_params(name: str) -> Set[int]:
 
 # --------------------------------------------------------------- barrier plan --
 
+def _static_load_count(stmts: List[ast.stmt], depth: int = 0) -> Optional[int]:
+    """How many vector memory operations a thread issues in `stmts`, when the text alone says so: direct-to-LDS
+    loads under loops over constant ranges, `with` scopes and calls of device functions of the same kind, and
+    besides them only declarations and assignments of index arithmetic (no element access, no other call than
+    id()). None for anything else."""
+    total = 0
+    for s in stmts:
+        if isinstance(s, ast.Expr) and isinstance(s.value, ast.Constant):
+            continue
+        if isinstance(s, ast.Return) and s.value is None:
+            continue
+        if isinstance(s, ast.Pass):
+            continue
+        if isinstance(s, ast.Expr) and isinstance(s.value, ast.Call):
+            call = s.value
+            if _is_intrinsic(call, "load_to_lds"):
+                if any(isinstance(n, ast.Call) for a in call.args for n in ast.walk(a)):
+                    return None
+                total += 1
+                continue
+            if isinstance(call.func, ast.Name) and call.func.id in _REGISTRY and depth < 8:
+                inner = _static_load_count(ast.parse(_REGISTRY[call.func.id].source).body[0].body, depth + 1)
+                if inner is None or any(isinstance(n, (ast.Subscript, ast.Call)) for a in call.args for n in ast.walk(a)):
+                    return None
+                total += inner
+                continue
+            return None
+        if isinstance(s, (ast.AnnAssign, ast.Assign)):
+            value = s.value
+            if value is not None and any(isinstance(n, ast.Subscript) or (isinstance(n, ast.Call) and not _is_call(n, "id"))
+                                         for n in ast.walk(value)):
+                return None
+            if isinstance(s, ast.Assign) and any(isinstance(n, ast.Subscript) for t in s.targets for n in ast.walk(t)):
+                return None
+            continue
+        if isinstance(s, ast.With):
+            inner = _static_load_count(s.body, depth)
+            if inner is None:
+                return None
+            total += inner
+            continue
+        if isinstance(s, ast.For) and _is_call(s.iter, "range") and 1 <= len(s.iter.args) <= 3 \
+                and all(isinstance(a, ast.Constant) and isinstance(a.value, int) for a in s.iter.args) and not s.orelse:
+            inner = _static_load_count(s.body, depth)
+            if inner is None:
+                return None
+            total += len(range(*[a.value for a in s.iter.args])) * inner
+            continue
+        return None
+    return total
+
+
 class _SyncPlan:
     """Which statements get a barrier in front of them / at the end of their body."""
 
@@ -186,6 +238,9 @@ class _SyncPlan:
         self.covered: Dict[int, Set[str]] = {}                     # id(match) -> arrays handed over inside it
         self.wait_before: Dict[int, List[Tuple[str, str]]] = {}    # id(stmt) -> [(array, "full" | "empty")]
         self.signal_after: Dict[int, List[Tuple[str, str]]] = {}
+        self.filled_together: Dict[str, List[str]] = {}            # array -> the arrays its writing case fills (itself included)
+        self.flush_after: Dict[int, List[str]] = {}                # id(loop or match) -> arrays whose last filling is announced behind it
+        self.flush_in_case: Dict[int, Tuple[List[str], Optional[ast.stmt]]] = {}  # id(last stmt of the writing case) -> (arrays, loop)
         for a in fn.args.args:            # a parameter declared ptr(shared(T)) or ptr(T, SHARED) points into LDS
             if a.arg != "template" and a.annotation is not None and any(   # (prism/sync_analysis.py:151-158)
                     _is_call(n, "shared") or (_is_call(n, "ptr") and address_space_of(n) == "SHARED")
@@ -321,7 +376,7 @@ class _SyncPlan:
             w |= b
         return r, w
 
-    def _plan_handovers(self, stmts: List[ast.stmt]) -> None:
+    def _plan_handovers(self, stmts: List[ast.stmt], enclosing: Optional[ast.stmt] = None, alone: bool = False) -> None:
         """An LDS array that one case of `match split(thread)` writes and other cases read is handed from case
         to case: the writing wavefronts wait until the array is empty, fill it and signal that it is full; the
         reading wavefronts wait until it is full, read it and signal that it is empty (the reference's split
@@ -329,7 +384,18 @@ class _SyncPlan:
         sides count rounds in two LDS words per array). In each case the wait goes in front of the first
         statement that touches the array and the signal behind the last one, in the innermost statement list
         that `with` scopes alone lead to. No workgroup
-        barrier is involved, so a writer may run as many arrays ahead of the readers as there are arrays."""
+        barrier is involved, so a writer may run as many arrays ahead of the readers as there are arrays.
+
+        A case that fills several arrays announces a filling late (BlockEmitter.announce_later): `filled_together`
+        names the arrays of such a case, and `flush_after` the statement (the innermost loop around the split, or
+        the split itself) behind which the last filling is announced at the latest. A filling stays unannounced
+        from one trip of that loop to the next only when the split is all the loop does (`alone`: declarations
+        and `with` scopes aside) and the loop ends without a workgroup barrier; otherwise the writing case
+        announces it before it leaves the split (`flush_in_case`), because a barrier further down would wait for
+        readers that wait for the announcement."""
+        doing = [t for t in stmts if not isinstance(t, (ast.AnnAssign, ast.Pass))
+                 and not (isinstance(t, ast.Expr) and isinstance(t.value, ast.Constant))]
+        sole = len(doing) == 1
         for s in stmts:
             if isinstance(s, ast.Match) and _is_call(s.subject, "split") and s.subject.args \
                     and isinstance(s.subject.args[0], ast.Name) and s.subject.args[0].id == "thread":
@@ -366,11 +432,27 @@ class _SyncPlan:
                         wait, signal = ("empty", "full") if i in writers else ("full", "empty")
                         self.wait_before.setdefault(id(touching[0]), []).append((array, wait))
                         self.signal_after.setdefault(id(touching[-1]), []).append((array, signal))
-            for field in ("body", "orelse"):
-                self._plan_handovers(getattr(s, field, []) or [])
-            if isinstance(s, ast.Match):
+                by_case: Dict[int, List[str]] = {}
+                for array in self.covered.get(id(s), ()):
+                    by_case.setdefault(next(i for i, (_, w) in enumerate(access) if array in w), []).append(array)
+                for i, arrays in by_case.items():
+                    if len(arrays) > 1:
+                        for array in arrays:
+                            self.filled_together[array] = sorted(arrays)
+                        self.flush_after.setdefault(id(enclosing if enclosing is not None else s), []).extend(sorted(arrays))
+                        carried = enclosing if alone and sole else None
+                        self.flush_in_case[id(s.cases[i].body[-1])] = (sorted(arrays), carried)
+            if isinstance(s, (ast.For, ast.While)):
+                self._plan_handovers(s.body, s, True)
+                self._plan_handovers(getattr(s, "orelse", []) or [], enclosing, False)
+            elif isinstance(s, ast.With):
+                self._plan_handovers(s.body, enclosing, alone and sole)
+            elif isinstance(s, ast.Match):
                 for case in s.cases:
-                    self._plan_handovers(case.body)
+                    self._plan_handovers(case.body, enclosing, False)
+            else:
+                for field in ("body", "orelse"):
+                    self._plan_handovers(getattr(s, field, []) or [], enclosing, False)
 
     def _block_uniform(self, node: Optional[ast.AST]) -> bool:
         """True when the expression is built from numbers, names in self.uniform, arithmetic and comparisons
@@ -528,6 +610,21 @@ HANDOVER_REPORT_DEFINITION = (
     "// written by a hand-over wait that ran out of polls: 1 + 2 * (array number) + (1 when waiting for a filled\n"
     "// array) in the low byte, the round above it; the launcher's <name>_status call reads and clears it\n"
     f"__device__ unsigned int {HANDOVER_REPORT} = 0;\n#endif\n")
+# A wavefront with direct-to-LDS loads in flight touches its hand-over words through these: in front of every LDS
+# access it can see, the compiler waits for all such loads (it does not know which part of LDS they write), and
+# a wavefront that announces fillings late (BlockEmitter.announce_later) lives on having loads in flight.
+LATE_ANNOUNCEMENT_HELPERS = (
+    "#ifndef PRISM_LDS_WORD_HELPERS\n#define PRISM_LDS_WORD_HELPERS\n"
+    "// one LDS word read / counted up without the compiler seeing an LDS access (the address is the low half of the\n"
+    "// generic one); the memory clobber keeps every memory operation on its side of the call\n"
+    "__device__ __forceinline__ unsigned int __prism_lds_peek(const unsigned int* word) {\n"
+    "    unsigned int value;\n"
+    "    asm volatile(\"ds_read_b32 %0, %1\\n\\ts_waitcnt lgkmcnt(0)\" : \"=v\"(value) : \"v\"((unsigned int)(unsigned long long)word) : \"memory\");\n"
+    "    return value;\n"
+    "}\n"
+    "__device__ __forceinline__ void __prism_lds_count(unsigned int* word) {\n"
+    "    asm volatile(\"ds_add_u32 %0, %1\" :: \"v\"((unsigned int)(unsigned long long)word), \"v\"(1u) : \"memory\");\n"
+    "}\n#endif\n")
 
 
 class BlockEmitter:
@@ -668,8 +765,20 @@ class BlockEmitter:
             for array, what in (self.plan.wait_before.get(id(s), []) if self.plan is not None else []):
                 self.wait_for(array, what)
             self.stmt(s)
-            for array, what in (self.plan.signal_after.get(id(s), []) if self.plan is not None else []):
-                self.signal(array, what)
+            signals = self.plan.signal_after.get(id(s), []) if self.plan is not None else []
+            late = [array for array, what in signals if what == "full" and array in self.plan.filled_together]
+            if late:
+                self.announce_later(late, s)
+            for array, what in signals:
+                if array not in late:
+                    self.signal(array, what)
+            if self.plan is not None and id(s) in self.plan.flush_in_case:
+                arrays, loop = self.plan.flush_in_case[id(s)]
+                if loop is None or id(loop) in self.plan.at_end:   # nothing stays unannounced beyond this case
+                    for array in arrays:
+                        self.announce_pending(array, None)
+            for array in (self.plan.flush_after.get(id(s), []) if self.plan is not None else []):
+                self.announce_pending(array, None)
 
     def stmt(self, s: ast.stmt) -> None:
         if isinstance(s, ast.AnnAssign) and isinstance(s.target, ast.Name):
@@ -744,17 +853,32 @@ class BlockEmitter:
         # it with the same count, and said so (readfirstlane) the compiler branches on scalar registers. Left to
         # itself it treats the exit as per-lane, unrolls eight polls and threads the live poll counter through
         # every exit with execution-mask bookkeeping: measured 12 % of a producer / consumer GEMM's time.
+        late = what == "empty" and array in self.plan.filled_together   # a wavefront that may have loads in flight
+        word = f"&__{what}_{array}"
+        peek = (f"__prism_lds_peek({word})" if late else
+                f"static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__hip_atomic_load({word}, "
+                "__ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP))))")
+        if late:
+            peek = f"static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>({peek})))"
         self.open()
         self.emit("int __spin = 0;")
         self.emit(f"const unsigned int __need = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>({need})));")
+        if late:
+            # About to block: whatever this wavefront has filled and not announced yet is announced first (the
+            # readers may need it before they give this array back), see announce_later.
+            self.emit(f"if ({peek} < __need) {{")
+            self.indent += 1
+            for other in self.plan.filled_together[array]:
+                self.announce_pending(other, None)
+            self.indent -= 1
+            self.emit("}")
         self.emit("#pragma nounroll")
-        self.emit(f"for (; __spin < {self.HANDOVER_SPINS} && static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>("
-                  f"__hip_atomic_load(&__{what}_{array}, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)))) < __need; ++__spin) "
-                  "__builtin_amdgcn_s_sleep(1);")
+        self.emit(f"for (; __spin < {self.HANDOVER_SPINS} && {peek} < __need; ++__spin) __builtin_amdgcn_s_sleep(1);")
         self.emit(f"if (__spin == {self.HANDOVER_SPINS} && (threadIdx.x & 63) == 0) __hip_atomic_store(&{HANDOVER_REPORT}, "
                   f"{code}u | (static_cast<unsigned int>(__round_{array}) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
         self.close()
-        self.emit('__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");')
+        if not late:   # (the peek's memory clobber orders the late form: the loads that follow are issued behind it)
+            self.emit('__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");')
 
     def signal(self, array: str, what: str) -> None:
         # every memory operation of the wavefront is complete (direct-to-LDS loads count as vector memory
@@ -765,6 +889,40 @@ class BlockEmitter:
                   "__HIP_MEMORY_SCOPE_WORKGROUP);")
         self.emit(f"__round_{array} += 1;")
 
+    def announce_later(self, arrays: List[str], filling: ast.stmt) -> None:
+        """Behind a statement that fills `arrays`, in a case that fills several arrays: the filling is counted
+        (its round) but announced ("full") only when the wavefront has issued the loads of the NEXT filling,
+        or is about to block in a wait, or leaves the loop, whichever comes first. The announcement needs the
+        filling's loads to have landed; made right away, as signal() does, it keeps a wavefront from having
+        more than one filling's loads in flight, and a filling then costs the whole memory latency. Behind the
+        next filling it waits only until at most that filling's loads are outstanding (a wavefront's loads
+        complete in order, so everything older has landed then), when their number is known from the program
+        text."""
+        for array in arrays:
+            self.emit(f"__round_{array} += 1;")
+        n = _static_load_count([filling])
+        for other in self.plan.filled_together[arrays[0]]:
+            if other not in arrays:   # filled by an earlier statement
+                self.announce_pending(other, n)
+        for array in arrays:
+            self.emit(f"__pending_{array} = true;")
+
+    def announce_pending(self, array: str, may_fly: Optional[int]) -> None:
+        """Announces the last filling of `array` if that is still to do. may_fly: how many of the wavefront's
+        latest vector memory operations may still be in flight (None: none)."""
+        if may_fly is None or not 0 < may_fly < 64:
+            wait = "__builtin_amdgcn_s_waitcnt(0);"
+        else:  # s_waitcnt immediate of gfx9: vmcnt in bits 3:0 and 15:14, expcnt 6:4 and lgkmcnt 11:8 left at "no wait"
+            wait = f"__builtin_amdgcn_s_waitcnt({(may_fly & 15) | ((may_fly >> 4) << 14) | (7 << 4) | (15 << 8)});  // vmcnt({may_fly})"
+        self.uses_late_announcements = True
+        self.emit(f"if (__pending_{array}) {{")
+        self.indent += 1
+        self.emit(wait)   # the filling has landed in LDS; the count below is issued behind it
+        self.emit(f"if ((threadIdx.x & 63) == 0) __prism_lds_count(&__full_{array});")
+        self.emit(f"__pending_{array} = false;")
+        self.indent -= 1
+        self.emit("}")
+
     def load_to_lds(self, n: ast.Call) -> None:
         """`intrinsic.load_to_lds(dst[i], src[j])`: the wavefront copies 64 x 16 bytes from global memory into LDS
         without staging registers: lane l's 16 bytes at &src[j] (j is the lane's own) land at &dst[i] + 16 l
@@ -773,8 +931,12 @@ class BlockEmitter:
         if len(n.args) != 2 or n.keywords or not all(isinstance(a, ast.Subscript) for a in n.args):
             raise HipgenError(f"{_line(n)}: intrinsic.load_to_lds(dst[i], src[j])")
         dst, src = self.expr(n.args[0]), self.expr(n.args[1])
+        # The LDS address is the low half of the generic one. Taken that way, and not by a pointer conversion,
+        # because the conversion carries a null check that the compiler cannot fold when the device function
+        # is not inlined (it then fails in its back end: "Operand has incorrect register class" on a compare
+        # with the LDS aperture base).
         self.emit(f"__builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&{src}), "
-                  f"(__attribute__((address_space(3))) void*)(&{dst}), 16, 0, 0);")
+                  f"(__attribute__((address_space(3))) void*)(unsigned int)(unsigned long long)(&{dst}), 16, 0, 0);")
 
     # kinds of instructions a scheduling group may name -> mask bits of __builtin_amdgcn_sched_group_barrier
     _SCHED_KINDS = {"mfma": 0x008, "valu": 0x002, "salu": 0x004, "vmem": 0x010, "vmem_read": 0x020, "vmem_write": 0x040,
@@ -965,6 +1127,8 @@ class BlockEmitter:
             # the array is handed between the cases of a split: its two round counters, cleared before anyone waits
             self.emit(f"__shared__ unsigned int __full_{name}, __empty_{name};")
             self.emit(f"int __round_{name} = 0;")
+            if name in self.plan.filled_together:
+                self.emit(f"bool __pending_{name} = false;  // filled by this wavefront and not announced yet")
             self.emit(f"if (threadIdx.x == 0) {{ __full_{name} = 0; __empty_{name} = 0; }}")
             self.emit("__syncthreads();")
 
@@ -1104,6 +1268,8 @@ class BlockEmitter:
         self.emit("}")
         text = "\n".join(self.out) + "\n"
         # the word the hand-over waits report into is defined once per file, whichever function comes first
+        if getattr(self, "uses_late_announcements", False):
+            text = LATE_ANNOUNCEMENT_HELPERS + text
         return (HANDOVER_REPORT_DEFINITION + text) if getattr(self, "uses_handover_report", False) else text
 
 
