@@ -11,10 +11,10 @@ __device__ void fill_slot_f32(int __block_id, int __thread_id, char* __smem, flo
             int lane = __thread_id_2;
             for (int part = 0; part < 4; part++) {
                 int arow = ((8 * ((4 * part) + w)) + (lane / 8));
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&A_from[(((arow * K) + k_at) + (4 * ((lane % 8) ^ ((arow / 2) % 8))))]), (__attribute__((address_space(3))) void*)(unsigned int)(unsigned long long)(&slot[(256 * ((4 * part) + w))]), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&A_from[(((arow * K) + k_at) + (4 * ((lane % 8) ^ ((arow / 2) % 8))))]), (__attribute__((address_space(3))) void*)(&slot[(256 * ((4 * part) + w))]), 16, 0, 0);
             }
             for (int part = 0; part < 8; part++) {
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&B_from[((((k_at + (4 * part)) + w) * N) + (4 * lane))]), (__attribute__((address_space(3))) void*)(unsigned int)(unsigned long long)(&slot[(4096 + (256 * ((4 * part) + w)))]), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&B_from[((((k_at + (4 * part)) + w) * N) + (4 * lane))]), (__attribute__((address_space(3))) void*)(&slot[(4096 + (256 * ((4 * part) + w)))]), 16, 0, 0);
             }
         }
     }

@@ -135,8 +135,8 @@ __global__ void handed_over_gemm(const __bf16* P, const __bf16* Q, float* D, int
                                                         if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 5u | (static_cast<unsigned int>(__round_q_first) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                                                     }
                                                     for (int part = 0; part < 4; part++) {
-                                                        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&P_rows[(((((16 * part) + row) * K) + k0) + k8)]), (__attribute__((address_space(3))) void*)(unsigned int)(unsigned long long)(&p_first_fill[(512 * part)]), 16, 0, 0);
-                                                        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&Q_rows[(((((16 * part) + row) * K) + k0) + k8)]), (__attribute__((address_space(3))) void*)(unsigned int)(unsigned long long)(&q_first_fill[(512 * part)]), 16, 0, 0);
+                                                        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&P_rows[(((((16 * part) + row) * K) + k0) + k8)]), (__attribute__((address_space(3))) void*)(&p_first_fill[(512 * part)]), 16, 0, 0);
+                                                        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&Q_rows[(((((16 * part) + row) * K) + k0) + k8)]), (__attribute__((address_space(3))) void*)(&q_first_fill[(512 * part)]), 16, 0, 0);
                                                     }
                                                     __round_p_first += 1;
                                                     __round_q_first += 1;
@@ -211,8 +211,8 @@ __global__ void handed_over_gemm(const __bf16* P, const __bf16* Q, float* D, int
                                                         if (__spin == 65536 && (threadIdx.x & 63) == 0) __hip_atomic_store(&__prism_handover_report, 7u | (static_cast<unsigned int>(__round_q_second) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                                                     }
                                                     for (int part = 0; part < 4; part++) {
-                                                        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&P_rows[((((((16 * part) + row) * K) + k0) + 32) + k8)]), (__attribute__((address_space(3))) void*)(unsigned int)(unsigned long long)(&p_second_fill[(512 * part)]), 16, 0, 0);
-                                                        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&Q_rows[((((((16 * part) + row) * K) + k0) + 32) + k8)]), (__attribute__((address_space(3))) void*)(unsigned int)(unsigned long long)(&q_second_fill[(512 * part)]), 16, 0, 0);
+                                                        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&P_rows[((((((16 * part) + row) * K) + k0) + 32) + k8)]), (__attribute__((address_space(3))) void*)(&p_second_fill[(512 * part)]), 16, 0, 0);
+                                                        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&Q_rows[((((((16 * part) + row) * K) + k0) + 32) + k8)]), (__attribute__((address_space(3))) void*)(&q_second_fill[(512 * part)]), 16, 0, 0);
                                                     }
                                                     __round_p_second += 1;
                                                     __round_q_second += 1;

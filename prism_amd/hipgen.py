@@ -544,5 +544,9 @@ def build(name: str, out_dir: Optional[str] = None, block_size: int = 256,
     proc = subprocess.run([hipcc_path(), *HIPCC_FLAGS, "-shared", "-o", str(lib), str(src)],
                           capture_output=True, text=True)
     if proc.returncode != 0:
-        raise HipgenError(f"hipcc failed for {name}:\n{proc.stderr}")
+        hint = ""
+        if "Operand has incorrect register class" in proc.stderr and "global_load_lds" in src.read_text():
+            hint = ("\n(a device function that calls intrinsic.load_to_lds was probably not inlined: the compiler cannot "
+                    "turn its pointer into an LDS address then; make the function smaller or call it from fewer places)")
+        raise HipgenError(f"hipcc failed for {name}:\n{proc.stderr}{hint}")
     return ctypes.CDLL(str(lib))

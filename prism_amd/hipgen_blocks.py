@@ -931,12 +931,13 @@ class BlockEmitter:
         if len(n.args) != 2 or n.keywords or not all(isinstance(a, ast.Subscript) for a in n.args):
             raise HipgenError(f"{_line(n)}: intrinsic.load_to_lds(dst[i], src[j])")
         dst, src = self.expr(n.args[0]), self.expr(n.args[1])
-        # The LDS address is the low half of the generic one. Taken that way, and not by a pointer conversion,
-        # because the conversion carries a null check that the compiler cannot fold when the device function
-        # is not inlined (it then fails in its back end: "Operand has incorrect register class" on a compare
-        # with the LDS aperture base).
+        # The LDS address comes from a pointer conversion, which the compiler folds into the array's LDS offset once
+        # the device function is inlined (taking the low half of the generic address instead keeps the 64-bit
+        # address arithmetic alive: measured 8 % of a GEMM whose wavefronts all load). A device function that is
+        # NOT inlined keeps the conversion's null check, and this compiler then fails in its back end ("Operand
+        # has incorrect register class"); build() says so when it sees that message.
         self.emit(f"__builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&{src}), "
-                  f"(__attribute__((address_space(3))) void*)(unsigned int)(unsigned long long)(&{dst}), 16, 0, 0);")
+                  f"(__attribute__((address_space(3))) void*)(&{dst}), 16, 0, 0);")
 
     # kinds of instructions a scheduling group may name -> mask bits of __builtin_amdgcn_sched_group_barrier
     _SCHED_KINDS = {"mfma": 0x008, "valu": 0x002, "salu": 0x004, "vmem": 0x010, "vmem_read": 0x020, "vmem_write": 0x040,

@@ -91,9 +91,8 @@ def test_waits_and_signals_of_the_producer_consumer_gemm():
     first_signal = next(n for n, ln in enumerate(got) if "__hip_atomic_fetch_add(&__empty_p_first" in ln)
     assert got[first_signal - 2:first_signal] == ["__builtin_amdgcn_s_waitcnt(0);", '__builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");']
     assert got[first_signal + 1] == "__round_p_first += 1;"
-    # the LDS address of a direct load is the low half of the generic address (no pointer conversion with its null check)
     assert ("__builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(&P_rows[(((((16 * part) + row) * K) "
-            "+ k0) + k8)]), (__attribute__((address_space(3))) void*)(unsigned int)(unsigned long long)(&p_first_fill[(512 * part)]), 16, 0, 0);") in got
+            "+ k0) + k8)]), (__attribute__((address_space(3))) void*)(&p_first_fill[(512 * part)]), 16, 0, 0);") in got
     # the writer reads and counts its hand-over words through helpers the compiler does not see into: it would
     # otherwise wait for all direct loads in front of every LDS access
     assert "__device__ __forceinline__ unsigned int __prism_lds_peek(const unsigned int* word) {" in got
