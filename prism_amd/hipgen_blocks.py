@@ -241,6 +241,7 @@ class _SyncPlan:
         self.filled_together: Dict[str, List[str]] = {}            # array -> the arrays its writing case fills (itself included)
         self.flush_after: Dict[int, List[str]] = {}                # id(loop or match) -> arrays whose last filling is announced behind it
         self.flush_in_case: Dict[int, Tuple[List[str], Optional[ast.stmt]]] = {}  # id(last stmt of the writing case) -> (arrays, loop)
+        self.announce_before_wait: Dict[int, List[str]] = {}       # id(stmt with a wait in front) -> arrays its case announces late
         for a in fn.args.args:            # a parameter declared ptr(shared(T)) or ptr(T, SHARED) points into LDS
             if a.arg != "template" and a.annotation is not None and any(   # (prism/sync_analysis.py:151-158)
                     _is_call(n, "shared") or (_is_call(n, "ptr") and address_space_of(n) == "SHARED")
@@ -402,6 +403,7 @@ class _SyncPlan:
                 access = [self._whole(c.body) for c in s.cases]
                 counts = [c.pattern.value.value if isinstance(c.pattern, ast.MatchValue)
                           and isinstance(c.pattern.value, ast.Constant) else 0 for c in s.cases]
+                wait_sites: Dict[int, List[int]] = {}   # case -> id(stmt) of every statement of it with a wait in front
                 for array in sorted(set().union(*(r | w for r, w in access))):
                     writers = [i for i, (_, w) in enumerate(access) if array in w]
                     readers = [i for i, (r, w) in enumerate(access) if array in r and array not in w]
@@ -432,6 +434,7 @@ class _SyncPlan:
                         wait, signal = ("empty", "full") if i in writers else ("full", "empty")
                         self.wait_before.setdefault(id(touching[0]), []).append((array, wait))
                         self.signal_after.setdefault(id(touching[-1]), []).append((array, signal))
+                        wait_sites.setdefault(i, []).append(id(touching[0]))
                 by_case: Dict[int, List[str]] = {}
                 for array in self.covered.get(id(s), ()):
                     by_case.setdefault(next(i for i, (_, w) in enumerate(access) if array in w), []).append(array)
@@ -442,6 +445,8 @@ class _SyncPlan:
                         self.flush_after.setdefault(id(enclosing if enclosing is not None else s), []).extend(sorted(arrays))
                         carried = enclosing if alone and sole else None
                         self.flush_in_case[id(s.cases[i].body[-1])] = (sorted(arrays), carried)
+                        for site in wait_sites.get(i, []):   # whatever this case waits for, filled arrays or others
+                            self.announce_before_wait[site] = sorted(arrays)
             if isinstance(s, (ast.For, ast.While)):
                 self._plan_handovers(s.body, s, True)
                 self._plan_handovers(getattr(s, "orelse", []) or [], enclosing, False)
@@ -763,7 +768,7 @@ class BlockEmitter:
                     self.emit(f"// {_line(s)} {self.plan.why.get(id(s), '')}")
                 self.emit("__syncthreads();")
             for array, what in (self.plan.wait_before.get(id(s), []) if self.plan is not None else []):
-                self.wait_for(array, what)
+                self.wait_for(array, what, self.plan.announce_before_wait.get(id(s)))
             self.stmt(s)
             signals = self.plan.signal_after.get(id(s), []) if self.plan is not None else []
             late = [array for array, what in signals if what == "full" and array in self.plan.filled_together]
@@ -840,11 +845,13 @@ class BlockEmitter:
     # -- hand-over of an LDS array between the cases of a split: two words per array count the rounds
     HANDOVER_SPINS = 1 << 16   # a wait gives up after this many polls (milliseconds; a real wait takes microseconds), so that a broken protocol cannot hang the GPU
 
-    def wait_for(self, array: str, what: str) -> None:
+    def wait_for(self, array: str, what: str, unannounced: Optional[List[str]] = None) -> None:
         """A bounded wait. A wavefront that runs out of polls goes on (the kernel always exits) but says so: it
         stores a non-zero code into the file-scope word HANDOVER_REPORT, which the launcher's `<name>_status`
         call turns into an error, because what such a wavefront goes on to read or overwrite is not what the
-        program meant."""
+        program meant. unannounced: the arrays this wavefront's case fills and announces late; whatever of them
+        is still unannounced is announced before the wavefront blocks, in any wait, because the other side may
+        need it before it lets this wait go."""
         writers, readers = self.plan.handed[array]
         need = f"(__round_{array} + 1) * {writers}" if what == "full" else f"__round_{array} * {readers}"
         code = 1 + 2 * list(self.plan.handed).index(array) + (1 if what == "full" else 0)
@@ -853,7 +860,7 @@ class BlockEmitter:
         # it with the same count, and said so (readfirstlane) the compiler branches on scalar registers. Left to
         # itself it treats the exit as per-lane, unrolls eight polls and threads the live poll counter through
         # every exit with execution-mask bookkeeping: measured 12 % of a producer / consumer GEMM's time.
-        late = what == "empty" and array in self.plan.filled_together   # a wavefront that may have loads in flight
+        late = unannounced is not None   # a wavefront that may have direct-to-LDS loads in flight
         word = f"&__{what}_{array}"
         peek = (f"__prism_lds_peek({word})" if late else
                 f"static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>(__hip_atomic_load({word}, "
@@ -864,11 +871,11 @@ class BlockEmitter:
         self.emit("int __spin = 0;")
         self.emit(f"const unsigned int __need = static_cast<unsigned int>(__builtin_amdgcn_readfirstlane(static_cast<int>({need})));")
         if late:
-            # About to block: whatever this wavefront has filled and not announced yet is announced first (the
-            # readers may need it before they give this array back), see announce_later.
+            # About to block: whatever this wavefront has filled and not announced yet is announced first, see
+            # announce_later.
             self.emit(f"if ({peek} < __need) {{")
             self.indent += 1
-            for other in self.plan.filled_together[array]:
+            for other in unannounced:
                 self.announce_pending(other, None)
             self.indent -= 1
             self.emit("}")
@@ -877,7 +884,7 @@ class BlockEmitter:
         self.emit(f"if (__spin == {self.HANDOVER_SPINS} && (threadIdx.x & 63) == 0) __hip_atomic_store(&{HANDOVER_REPORT}, "
                   f"{code}u | (static_cast<unsigned int>(__round_{array}) << 8), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
         self.close()
-        if not late:   # (the peek's memory clobber orders the late form: the loads that follow are issued behind it)
+        if not late:   # (the peek's memory clobber orders the late form: what follows is issued behind it)
             self.emit('__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");')
 
     def signal(self, array: str, what: str) -> None:

@@ -203,6 +203,66 @@ def test_what_is_refused_and_what_needs_no_handover():
     assert "__full_buf" not in generate("one_side_only")      # read by both cases, written by none
 
 
+@requires(grid[1], block[1], thread[128])
+@prism("global")
+def there_and_back(x: ptr(int) @ grid[1], trips: int @ grid[1]):
+    with group(block[1]):
+        one: shared(int[256], static=True) @ block[1]
+        two: shared(int[256], static=True) @ block[1]
+        back: shared(int[64], static=True) @ block[1]
+        for i in range(trips):
+            with claim(one, p=thread[64], offset=0) as one_fill:
+                with claim(two, p=thread[64], offset=0) as two_fill:
+                    with claim(back, p=thread[64], offset=0) as back_fill:
+                        match split(thread):
+                            case 64:
+                                with group(thread[64]):
+                                    lane: int @ thread[1] = id()
+                                    intrinsic.load_to_lds(one_fill[0], x[4 * lane])
+                                    intrinsic.load_to_lds(two_fill[0], x[4 * lane + 256])
+                                t: int @ thread[1] = back[3]
+                            case 64:
+                                u: int @ thread[1] = one[0] + two[1]
+                                with partition(back_fill, p=thread[1], offset=0) as mine:
+                                    mine[0] = u
+
+
+def test_a_late_announcing_case_announces_before_it_blocks_in_any_wait():
+    """The first case fills two arrays (announced late) and then waits for an array the second case fills from
+    them: blocked in that wait with the second filling unannounced, both cases would wait for each other. Every
+    wait of a late-announcing case, for whichever array, announces first when it has to block; and its polls go
+    through the helper (the wavefront may have direct loads in flight)."""
+    got = lines(generate("there_and_back"))
+    wait = next(n for n, ln in enumerate(got) if ln.startswith("for (; __spin") and "__full_back" in ln)
+    assert "__prism_lds_peek(&__full_back)" in got[wait]
+    block = [n for n, ln in enumerate(got[:wait]) if ln.startswith("if (static_cast<unsigned int>(") and "__prism_lds_peek(&__full_back)" in ln][-1]
+    between = got[block:wait]
+    assert "if (__pending_one) {" in between and "if (__pending_two) {" in between
+    assert between.count("__builtin_amdgcn_s_waitcnt(0);") == 2
+    # the other case fills one array only: it announces at once, the ordinary way
+    assert any("__hip_atomic_fetch_add(&__full_back, 1u" in ln for ln in got) and "__pending_back" not in "\n".join(got)
+
+
+def test_loads_of_a_filling_are_counted_from_the_program_text():
+    import ast
+    from prism_amd.hipgen_blocks import _static_load_count
+    from prism_amd import examples
+    examples.load()
+
+    def count(text):
+        return _static_load_count(ast.parse(text).body)
+
+    assert count("fill_slot(a, P, Q, K, k0)") == 12           # four and eight direct loads per thread
+    assert count("fill_slot(a, P, Q, K, k0)\nfill_slot(b, P, Q, K, k1)") == 24
+    assert count("for part in range(3):\n    intrinsic.load_to_lds(a[512 * part], P[part * K + lane])") == 3
+    assert count("row: int @ thread[1] = lane / 4\nintrinsic.load_to_lds(a[0], P[row])") == 1
+    # anything the text does not settle: a condition, a loop whose trips are not constants, an element read or written
+    assert count("if k0 + 64 < K:\n    fill_slot(a, P, Q, K, k0)") is None
+    assert count("for part in range(n):\n    intrinsic.load_to_lds(a[0], P[part])") is None
+    assert count("v: int @ thread[1] = P[0]\nintrinsic.load_to_lds(a[0], P[v])") is None
+    assert count("fill_slot(a, P, Q, K, table[0])") is None
+
+
 @pytest.fixture(scope="module")
 def built(tmp_path_factory):
     return hipgen.build("handed_over_gemm", out_dir=str(tmp_path_factory.mktemp("hipgen_handover")), block_size=320)
