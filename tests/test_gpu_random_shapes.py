@@ -84,6 +84,51 @@ def test_sgemm_kernel_5_random_shapes(prism, seed):
             assert err <= 1e-5 * np.sqrt(K) + abs(beta) * 2**-22, f"{M}x{N}x{K} with a workspace: max error {err:.3e}"
 
 
+@pytest.mark.parametrize("seed", [11, 12])
+def test_sgemm_random_shapes_with_more_tiles_than_cus(prism, seed):
+    """Draws the ones above do not reach: more 256 x 256 tiles than CUs with a K long enough for the workspace form
+    to share the last round's K loops between all workgroups (ragged M and any start; N, K multiples of 4 or not:
+    the shared form needs 16 B-aligned rows and is asked for only then), and a thin strip of columns beyond a whole
+    number of tiles. Both entry points, every element, guard values around C, a workspace full of NaN. (The same
+    draws over 28 000 more seeds were run once.)"""
+    rng = np.random.default_rng(seed)
+    g = torch.Generator(device=DEV)
+    g.manual_seed(seed)
+    taken = 0
+    for i in range(9):
+        kind = i % 3
+        if kind == 0:
+            M, N, K = int(rng.integers(4100, 6200)), int(rng.integers(4100, 6200)), int(rng.integers(256, 900))
+        elif kind == 1:
+            M, N, K = int(rng.integers(4100, 6200)), 4 * int(rng.integers(1025, 1550)), 4 * int(rng.integers(64, 225))
+        else:
+            M, N, K = int(rng.integers(64, 3000)), 256 * int(rng.integers(1, 12)) + int(rng.integers(1, 9)), int(rng.integers(16, 1200))
+        sa, sb, sc = (int(rng.integers(0, 4)) for _ in range(3))
+        if kind == 1 and i % 2:
+            sa = sb = sc = 0
+        A = torch.rand((M, K), device=DEV, generator=g) * 2 - 1
+        B = torch.rand((K, N), device=DEV, generator=g) * 2 - 1
+        C0 = torch.rand((M, N), device=DEV, generator=g) * 2 - 1
+        beta = 0.5 if i % 2 else 0.0
+        a, b = _fenced(A, sa, float("nan")), _fenced(B, sb, float("nan"))
+        cbuf = torch.full((M * N + 64,), 777.0, device=DEV)
+        c = cbuf[8 + sc:8 + sc + M * N].view(M, N)
+        want = 1.25 * (A.double() @ B.double()) + beta * C0.double()
+        ws_bytes = prism.sgemm_workspace_size(M, N, K)
+        ws = torch.full((max(ws_bytes, 4) // 4,), float("nan"), device=DEV)
+        for use_ws in (False, True):
+            c.copy_(C0)
+            print(f"sgemm M={M} N={N} K={K} starts {sa} {sb} {8 + sc} beta={beta} workspace={use_ws and ws_bytes}", flush=True)
+            prism.sgemm(M, N, K, 1.25, a, b, beta, c, variant=5, workspace=ws if use_ws else None)
+            torch.cuda.synchronize()
+            assert bool((cbuf[:8 + sc] == 777.0).all()) and bool((cbuf[8 + sc + M * N:] == 777.0).all())
+            err = float((c.double() - want).abs().max())
+            assert err <= 1e-5 * np.sqrt(K) + abs(beta) * 2**-22, f"{M}x{N}x{K} workspace={use_ws}: max error {err:.3e}"
+        if sa == 0 and sb == 0 and (8 + sc) % 4 == 0:
+            taken += prism.sgemm_workspace_plan(M, N, K, ws_bytes)[0] > 0
+    assert taken >= 1   # at least one draw went through the shared form
+
+
 @pytest.mark.parametrize("seed", [4, 5, 6])
 def test_gemm_bf16_random_shapes(prism, seed):
     g = torch.Generator(device=DEV)
@@ -143,3 +188,8 @@ def test_scans_random_lengths_and_alignments(prism, seed):
         assert torch.equal(got, want), f"n={n} start={start} kind={kind}"
         if not in_place:
             assert torch.equal(x, keep)
+        if i % 4 == 0:   # the same call with look-backs that never wait: every silent predecessor is helped
+            if in_place:
+                x.copy_(keep)
+            kw = {"exclusive": True} if kind == 2 else {"op": "max"} if kind == 3 else {}
+            assert torch.equal(prism.scan(x, out=out, workspace=ws, spin_limit=0, **kw), want), f"n={n} start={start} kind={kind} helping"
