@@ -306,6 +306,22 @@ def bench_vendor(steps, warmup):
     return out
 
 
+def vendor_sgemm_tflops(M, N, K, alpha, beta, steps, warmup):
+    """rocblas_sgemm called directly on one shape (seeded operands like bench_sgemm's), timed like a workload."""
+    import torch
+    from prism_amd import _lib
+    v = _lib.load_vendor()
+    st = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0)
+    A = torch.rand((M, K), device="cuda", generator=g) * 2 - 1
+    B = torch.rand((K, N), device="cuda", generator=g) * 2 - 1
+    C = torch.rand((M, N), device="cuda", generator=g) * 2 - 1
+    ms = time_steps(lambda: 0 if v.vendor_sgemm(M, N, K, alpha, A.data_ptr(), B.data_ptr(), beta, C.data_ptr(), st) == 0 else 1,
+                    steps, warmup)
+    return 2.0 * M * N * K / ms / 1e9
+
+
 # ----------------------------------------------------------- CPU baselines --
 
 def cpu_baseline_sgemm(n=8192, rows=4):
@@ -485,6 +501,11 @@ def main() -> int:
                                                  "entry": "prism_sgemm_ws", "workgroups_sharing": groups, "tiles_shared": shared}
             log(f"  sgemm kernel 5 {M}x{N}x{Kd} with workspace ({shared} tiles shared by {groups} workgroups): "
                 f"{r['ms']:.3f} ms  {r['tflops']:.2f} TFLOP/s")
+        if not args.no_vendor:   # rocblas_sgemm on the same shapes, same run and protocol
+            for (M, N, Kd) in ((4096, 4096, 128), (128, 4096, 4096), (8191, 4097, 1023), (16384, 16384, 512),
+                               (5120, 5120, 5120), (4352, 4352, 4352), (3200, 3200, 3200)):
+                configs[f"sgemm_k5_{M}x{N}x{Kd}"]["rocblas_sgemm_tflops"] = vendor_sgemm_tflops(M, N, Kd, 1.0, 0.0, 10, 2)
+                log(f"  rocblas_sgemm {M}x{N}x{Kd}: {configs[f'sgemm_k5_{M}x{N}x{Kd}']['rocblas_sgemm_tflops']:.2f} TFLOP/s")
         for p in (20, 24, 28):
             r = bench_scan(prism, 1 << p, 20, 3)
             configs[f"scan_2p{p}"] = {"ms": r["ms"], "GBps": r["GBps"], "frac": r["roofline"]["frac"], "steps": 20}

@@ -1288,6 +1288,7 @@ __global__ __launch_bounds__(256) void sgemm_thin_columns_kernel(int M, int N, i
 // --------------------------------------------------------------- launchers --
 
 constexpr int kThinColumns = 8;  // up to this many columns beyond whole 256-column tiles go to the thin-strip kernel
+constexpr int kShortK = 2048;    // up to this K the 256 x 256 tiles of a problem that fills the CUs run as 128 x 256 halves, two to a CU
 
 template <int BM, int BN, int BK, int TM, int TN, bool VEC>
 int run_thread_tile(int M, int N, int K, float alpha, const float* A, const float* B, float beta,
@@ -1361,6 +1362,13 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
     const int tiles = tiles_m * tiles_n, cus = cu_count();
     int main_tiles = tiles, leftover_wt = 0;
     const bool lane_offsets_fit = static_cast<long long>(K) * 64 < (1ll << 30) && static_cast<long long>(N) * 64 < (1ll << 30);
+    // Short K: a tile's write-back (and the read of C in front of it) is a large part of its time, and with one
+    // workgroup per CU nothing runs beside it. As 128 x 256 halves (K tiles of 16, 48 KiB of LDS, eight waves) two
+    // workgroups share a CU and drift apart, so that one's write-back overlaps the other's K loop:
+    // 4096 x 4096 x 128 95 -> 106 TFLOP/s (81 -> 90 with beta), 8192 x 8192 x 256 126 -> 132 (108 -> 121),
+    // 16384 x 16384 x 512 142 -> 144 (130 -> 140); level from K = 4096 up (8192^3 152.3 / 152.2).
+    // (The tiles of whole rounds only; a partial last round is cut as for any K, below.)
+    const bool short_k = K <= kShortK && tiles >= cus && lane_offsets_fit;
     if (ragged && lane_offsets_fit && tiles > cus && tiles % cus != 0 && K >= 64) {
         // The one-wave kernels have no ragged form: 64 x 256 slices, which cost about 0.27 of a round per
         // slice on the fullest CU (128 x 256 halves cost 0.58 per half, never less), when three to a CU do.
@@ -1400,11 +1408,17 @@ bool try_wave_tile_dma(int M, int N, int K, float alpha, const float* A, const f
     // `edge` selects the zero-filling variants of both kernels (sub-tiles that lie wholly outside C exit at once).
     auto launch = [&](auto edge, auto ragged_rows) {
         constexpr bool EDGE = decltype(edge)::value, RAGGED = decltype(ragged_rows)::value;
-        sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, EDGE, RAGGED><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
-            M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
-        *rc = check_launch("sgemm_wave_tile_dma_kernel");
+        if (short_k) {
+            sgemm_wave_tile_dma_kernel<128, 256, 16, 32, 128, EDGE, RAGGED><<<dim3(static_cast<unsigned>(main_tiles) * 2), dim3(512), 0, s>>>(
+                M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, 0);
+            *rc = check_launch("sgemm_wave_tile_dma_kernel (halves, two to a CU)");
+        } else {
+            sgemm_wave_tile_dma_kernel<BM, BN, BK, WM, WN, EDGE, RAGGED><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
+                M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
+            *rc = check_launch("sgemm_wave_tile_dma_kernel");
+        }
         if (*rc == 0 && leftover_wt == 128) {
-            // 128 x 256 halves of the same kernel, one workgroup to a CU
+            // 128 x 256 halves of the same kernel (one workgroup to a CU for a partial round, two for short K)
             sgemm_wave_tile_dma_kernel<128, 256, 16, 32, 128, EDGE, RAGGED><<<dim3(static_cast<unsigned>(tiles - main_tiles) * 2), dim3(512), 0, s>>>(
                 M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, main_tiles);
             *rc = check_launch("sgemm_wave_tile_dma_kernel (leftover halves)");
@@ -1613,7 +1627,9 @@ StreamKPlan stream_k_plan(int M, int N, int K, bool aligned) {
     // Fewer tiles than CUs: sharing all of them was measured level with or behind the smaller tiles launch_sgemm
     // picks there (3072^3 134 against 149 TFLOP/s, 3584^3 139 against 142, 3200^3 125 against 123): every tile
     // then pays for partial products.
-    if (tiles <= cus || tiles > 0x3fffffff || K < 256) return plan;
+    // A short K leaves too little work per tile to pay for partial products and the second launch (5120 x 5120 x K,
+    // plain / shared: K = 512 124 / 111, 1024 131 / 128 (4352^2), 2048 134 / 140, 5120 136 / 148 TFLOP/s).
+    if (tiles <= cus || tiles > 0x3fffffff || K < kShortK) return plan;
     const int left = static_cast<int>(tiles % cus);
     if (left == 0) return plan;
     // A last round that is nearly full gains nothing from being shared (the partial products cost a few per
@@ -1671,7 +1687,14 @@ int launch_sgemm_ws(int variant, int M, int N, int K, float alpha, const float* 
             const int tiles_m = ceil_div(M, 256), tiles_n = ceil_div(N, 256);
             if (plan.main_tiles > 0) {
                 const dim3 main_grid(static_cast<unsigned>(plan.main_tiles));
-                if (plan.whole)
+                const dim3 halves_grid(static_cast<unsigned>(plan.main_tiles) * 2);  // short K: see try_wave_tile_dma
+                if (K <= kShortK && plan.whole)
+                    sgemm_wave_tile_dma_kernel<128, 256, 16, 32, 128, false><<<halves_grid, dim3(512), 0, s>>>(
+                        M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, 0);
+                else if (K <= kShortK)
+                    sgemm_wave_tile_dma_kernel<128, 256, 16, 32, 128, true><<<halves_grid, dim3(512), 0, s>>>(
+                        M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, 0);
+                else if (plan.whole)
                     sgemm_wave_tile_dma_kernel<256, 256, 32, 32, 128, false><<<main_grid, dim3(1024), 0, s>>>(
                         M, N, K, alpha, A, B, beta, C, tiles_m, tiles_n, -1);
                 else

@@ -86,8 +86,9 @@ def test_sgemm_kernel_5_random_shapes(prism, seed):
 
 @pytest.mark.parametrize("seed", [11, 12])
 def test_sgemm_random_shapes_with_more_tiles_than_cus(prism, seed):
-    """Draws the ones above do not reach: more 256 x 256 tiles than CUs with a K long enough for the workspace form
-    to share the last round's K loops between all workgroups (ragged M and any start; N, K multiples of 4 or not:
+    """Draws the ones above do not reach: more 256 x 256 tiles than CUs, K on both sides of 2048 (up to there the whole
+    rounds run as 128 x 256 halves; from there on the workspace form shares the last round's K loops between all
+    workgroups (ragged M and any start; N, K multiples of 4 or not:
     the shared form needs 16 B-aligned rows and is asked for only then), and a thin strip of columns beyond a whole
     number of tiles. Both entry points, every element, guard values around C, a workspace full of NaN. (The same
     draws over 28 000 more seeds were run once.)"""
@@ -98,9 +99,9 @@ def test_sgemm_random_shapes_with_more_tiles_than_cus(prism, seed):
     for i in range(9):
         kind = i % 3
         if kind == 0:
-            M, N, K = int(rng.integers(4100, 6200)), int(rng.integers(4100, 6200)), int(rng.integers(256, 900))
+            M, N, K = int(rng.integers(4100, 6200)), int(rng.integers(4100, 6200)), int(rng.integers(1500, 2600))
         elif kind == 1:
-            M, N, K = int(rng.integers(4100, 6200)), 4 * int(rng.integers(1025, 1550)), 4 * int(rng.integers(64, 225))
+            M, N, K = int(rng.integers(4100, 6200)), 4 * int(rng.integers(1025, 1550)), 4 * int(rng.integers(512, 650))
         else:
             M, N, K = int(rng.integers(64, 3000)), 256 * int(rng.integers(1, 12)) + int(rng.integers(1, 9)), int(rng.integers(16, 1200))
         sa, sb, sc = (int(rng.integers(0, 4)) for _ in range(3))

@@ -248,12 +248,13 @@ def test_wave_tile_k_split_with_workspace(prism, oracle, shape):
     assert np.max(np.abs(host(c3) - outs[0])) <= 2 * tol(oracle, K, A, B, 0.5, Cm)
 
 
-@pytest.mark.parametrize("shape", [(4352, 4352, 512), (5120, 5120, 288), (5000, 5000, 260), (4608, 4864, 1024), (4100, 4612, 300)])
+@pytest.mark.parametrize("shape", [(4352, 4352, 2048), (5120, 5120, 2080), (5000, 5000, 2052), (4608, 4864, 3072), (4100, 4612, 2060)])
 def test_wave_tile_last_round_shared_with_workspace(prism, oracle, shape):
     """256 x 256 tiles that are not a whole number of rounds of the CUs, through prism_sgemm_ws: the whole rounds
     run one tile per workgroup, the K ranges of the tiles of the last round (33, 144, 144, 86 and 67 here) are
-    shared between all CUs, in shares of two K tiles and up, and a second kernel adds a tile's partial products.
-    Whole tiles and ragged M, N, K (rows 16 B aligned). Every element against an fp64 product formed on the
+    shared between all CUs, and a second kernel adds a tile's partial products (K of 2048 and up: below that the
+    entry point leaves the product to prism_sgemm, see test_short_k_is_not_shared). Whole tiles and ragged M, N, K
+    (rows 16 B aligned). Every element against an fp64 product formed on the
     device, with and without reading C (NaN in C when it is not read), the same bits on a second run, nothing
     written outside the workspace, and the plan query says that the shared form is the one that ran."""
     import fp64_referee
@@ -276,6 +277,39 @@ def test_wave_tile_last_round_shared_with_workspace(prism, oracle, shape):
         prism.sgemm(M, N, K, 1.25, A, B, beta, c2, variant=5, workspace=ws)
         assert torch.equal(c, c2)
     assert bool((wsbuf[:256] == 0x5A).all()) and bool((wsbuf[256 + need:] == 0x5A).all())
+
+
+def test_short_k_is_not_shared(prism):
+    """With a short K a tile holds too little work to pay for partial products: no workspace is asked for, and
+    the workspace entry point gives the bits of the plain one."""
+    for (M, N, K) in ((5120, 5120, 512), (4352, 4352, 1024), (4100, 4612, 300)):
+        assert prism.sgemm_workspace_size(M, N, K) == 0 and prism.sgemm_workspace_plan(M, N, K, 1 << 30) == (0, 0)
+    M, N, K = 4352, 4352, 1024
+    A, B, C0 = _device_inputs(M, N, K)
+    ws = torch.empty(1 << 20, device=DEV)
+    c1, c2 = C0.clone(), C0.clone()
+    prism.sgemm(M, N, K, 1.25, A, B, 0.5, c1, variant=5, workspace=ws)
+    prism.sgemm(M, N, K, 1.25, A, B, 0.5, c2, variant=5)
+    assert torch.equal(c1, c2)
+
+
+@pytest.mark.parametrize("shape", [(4096, 4096, 128), (8192, 4096, 256), (4100, 4612, 300), (8190, 4098, 1000), (4097, 4097, 1025), (5120, 5120, 512), (4096, 8192, 2048)])
+def test_wave_tile_short_k_runs_as_halves(prism, oracle, shape):
+    """K up to 2048 on problems with at least as many 256 x 256 tiles as CUs: the tiles of the whole rounds run as
+    128 x 256 halves, two workgroups to a CU (whole tiles, ragged edges, rows that are only 4 B aligned, a partial
+    last round beside them). Every element against fp64, with and without reading C, guard values around C."""
+    import fp64_referee
+    M, N, K = shape
+    A, B, C0 = _device_inputs(M, N, K)
+    for beta in (0.5, 0.0):
+        cbuf = torch.full((M * N + 128,), 777.0, device=DEV)
+        c = cbuf[64:64 + M * N].view(M, N)
+        c.copy_(C0 if beta else torch.full((M, N), float("nan"), device=DEV))
+        print(f"prism_sgemm {M}x{N}x{K} beta={beta}", flush=True)
+        prism.sgemm(M, N, K, 0.75, A, B, beta, c, variant=5)
+        err = fp64_referee.sgemm_max_err_fp64(0.75, A, B, beta, C0, c)
+        assert err <= _bound(K, beta), f"{M}x{N}x{K} beta={beta}: max error {err:.3e}"
+        assert bool((cbuf[:64] == 777.0).all()) and bool((cbuf[64 + M * N:] == 777.0).all())
 
 
 @pytest.mark.parametrize("shape", [(4096, 3073, 100), (4000, 3080, 67), (4096, 3076, 64), (8191, 4097, 1023), (4096, 3329, 4), (3000, 4099, 2100)])
