@@ -1285,9 +1285,79 @@ __global__ __launch_bounds__(256) void sgemm_thin_columns_kernel(int M, int N, i
         }
 }
 
+// --------------------------------------------------- kernel 5, a thin strip of rows --
+// C[m0 .. m0 + r, :) = alpha * A[m0 .. m0 + r, :) @ B + beta * C[m0 .. m0 + r, :) for r <= R rows: what is left of M
+// beyond a whole number of 256-row tiles when that is a few rows only (M = 4097: a 17th tile row would cost a
+// seventeenth of the whole product, or a round of its own, for one row of C). A vector-matrix product that reads
+// all of B once. A workgroup owns 16 columns (N = 4096 gives every CU one); a wavefront's lanes are four rows of k
+// by sixteen columns, so that one load instruction fetches 64 B of four rows of B; its sixteen wavefronts take a
+// sixteenth of K each. Lane l fetches A[row][k0 + l] for 64 values of k at a time, and the value a lane needs
+// (k0 + 4 u + its row of k) comes to it through the LDS crossbar. The sums meet in a fixed order: the wavefronts'
+// in LDS, then the four rows of k. The summation order differs from the big tiles', within the same tolerance.
+// (With a lane per column and 64 columns per workgroup the kernel kept a quarter of the CUs busy with one multiply
+// and one broadcast per lane, k and row: 56 us for 8 x 4096 x 4096 against 17 this way.)
+constexpr int kThinRowsCols = 16;  // columns of C per workgroup of the strip kernel (32: 52 us against 32 for 8 x 4096 x 4096)
+template <int R>
+__global__ __launch_bounds__(1024) void sgemm_thin_rows_kernel(int N, int K, int m0, int r, float alpha,
+                                                               const float* __restrict__ A, const float* __restrict__ B,
+                                                               float beta, float* C) {
+    constexpr int WAVES = 16, COLS = kThinRowsCols, KQ = kWave / COLS;
+    __shared__ float part[WAVES][R][kWave];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) / kWave);
+    const int kq = lane / COLS, c = lane % COLS;
+    const int col = blockIdx.x * COLS + c;
+    const bool live = col < N;
+    const int per = (K + WAVES - 1) / WAVES;
+    const int k_begin = wave * per, k_end = (k_begin + per < K) ? k_begin + per : K;
+    const float* a_rows = A + static_cast<size_t>(m0) * K;
+    const float* b_col = B + (live ? col : 0);
+    float acc[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) acc[i] = 0.0f;
+    for (int k0 = k_begin; k0 < k_end; k0 += kWave) {
+        float a[R], b[kWave / KQ];
+#pragma unroll
+        for (int i = 0; i < R; ++i) a[i] = (i < r && k0 + lane < k_end) ? a_rows[static_cast<size_t>(i) * K + k0 + lane] : 0.0f;
+#pragma unroll
+        for (int u = 0; u < kWave / KQ; ++u) {
+            const int k = k0 + KQ * u + kq;
+            b[u] = (live && k < k_end) ? b_col[static_cast<size_t>(k) * N] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < kWave / KQ; ++u)
+#pragma unroll
+            for (int i = 0; i < R; ++i) acc[i] = __builtin_fmaf(__shfl(a[i], KQ * u + kq, kWave), b[u], acc[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < R; ++i) part[wave][i][lane] = acc[i];
+    __syncthreads();
+    if (wave < r) {   // wavefront i adds up row i: the wavefronts' shares in the order of k, then the four rows of k
+        float v = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) v += part[w][wave][lane];
+        float sum = v;
+#pragma unroll
+        for (int q = 1; q < KQ; ++q) sum += __shfl(v, c + q * COLS, kWave);
+        if (kq == 0 && live) {
+            float* out = &C[static_cast<size_t>(m0 + wave) * N + col];
+            *out = epilogue(alpha, sum, beta, out);
+        }
+    }
+}
+
 // --------------------------------------------------------------- launchers --
 
 constexpr int kThinColumns = 8;  // up to this many columns beyond whole 256-column tiles go to the thin-strip kernel
+constexpr int kThinRows = 8;     // and up to this many rows beyond whole 256-row tiles to its counterpart
+
+// How many of the last rows of an M x N product kernel 5 leaves to the thin-strip kernel (0: none): a few rows
+// beyond a whole number of 256-row tiles, when the rows before still fill three quarters of the CUs with tiles.
+int thin_rows_of(int M, int N) {
+    const int r = M % 256;
+    if (M <= 256 || r == 0 || r > kThinRows || N < 256) return 0;
+    return static_cast<long long>(M / 256) * ceil_div(N, 256) * 4 >= 3ll * cu_count() ? r : 0;
+}
 constexpr int kShortK = 2048;    // up to this K the 256 x 256 tiles of a problem that fills the CUs run as 128 x 256 halves, two to a CU
 
 template <int BM, int BN, int BK, int TM, int TN, bool VEC>
@@ -1611,6 +1681,7 @@ int skinny_parts(int M, int N, int K) {
 StreamKPlan stream_k_plan(int M, int N, int K, bool aligned) {
     StreamKPlan plan;
     if (M <= 0 || N <= 0 || K <= 0 || !aligned || N % 4 || K % 4) return plan;  // rows must stay 16 B aligned
+    M -= thin_rows_of(M, N);   // the plan is for the rows the tiles keep (launch_sgemm_ws hands the rest to the strip kernel)
     const int cus = cu_count();
     if (const int parts = skinny_parts(M, N, K)) {
         const long long tiles = static_cast<long long>(M / 64) * (N / 256);
@@ -1662,6 +1733,12 @@ int launch_sgemm_ws(int variant, int M, int N, int K, float alpha, const float* 
     if (int rc = check_sgemm_arguments(variant, M, N, K, A, B, C)) return rc;
     if ((variant == 0 || variant == 5) && M > 0 && N > 0 && K > 0 && ws != nullptr && aligned16(ws)) {
         const StreamKPlan plan = stream_k_plan(M, N, K, aligned16(A) && aligned16(B) && aligned16(C));
+        if (const int r = thin_rows_of(M, N); r != 0 && plan.bm != 0 && ws_bytes >= plan.bytes()) {
+            if (int rc = launch_sgemm_ws(variant, M - r, N, K, alpha, A, B, beta, C, ws, ws_bytes, s)) return rc;
+            sgemm_thin_rows_kernel<kThinRows><<<dim3(static_cast<unsigned>(ceil_div(N, kThinRowsCols))), dim3(1024), 0, s>>>(
+                N, K, M - r, r, alpha, A, B, beta, C);
+            return check_launch("sgemm_thin_rows_kernel");
+        }
         if (plan.bm != 0 && ws_bytes >= plan.bytes()) {
             float* parts = static_cast<float*>(ws);
             const dim3 grid(static_cast<unsigned>(plan.groups));
@@ -1767,6 +1844,15 @@ int launch_sgemm(int variant, int M, int N, int K, float alpha, const float* A, 
             // run_my_sgemm_5 (evals/4090_sgemm/runner.cu:194-202), with four
             // 64-lane waves in place of four 32-lane warps.
             {
+                // A few rows beyond a whole number of 256-row tiles (M = 4097) would cost a whole tile row: the
+                // product of the rows before runs as ever (the same call on M - r rows), a thin-strip kernel
+                // takes the rest (4097 x 4097 x 1025: 108 -> 131 TFLOP/s).
+                if (const int r = thin_rows_of(M, N)) {
+                    if (int rc = launch_sgemm(5, M - r, N, K, alpha, A, B, beta, C, s)) return rc;
+                    sgemm_thin_rows_kernel<kThinRows><<<dim3(static_cast<unsigned>(ceil_div(N, kThinRowsCols))), dim3(1024), 0, s>>>(
+                        N, K, M - r, r, alpha, A, B, beta, C);
+                    return check_launch("sgemm_thin_rows_kernel");
+                }
                 // Whole 256 x 256 tiles for at least three quarters of the CUs: the direct-to-LDS kernel,
                 // K tiles of 32 (128 KiB of LDS) when K allows, else of 16.
                 int rc = 0;

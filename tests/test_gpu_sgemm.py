@@ -248,10 +248,10 @@ def test_wave_tile_k_split_with_workspace(prism, oracle, shape):
     assert np.max(np.abs(host(c3) - outs[0])) <= 2 * tol(oracle, K, A, B, 0.5, Cm)
 
 
-@pytest.mark.parametrize("shape", [(4352, 4352, 2048), (5120, 5120, 2080), (5000, 5000, 2052), (4608, 4864, 3072), (4100, 4612, 2060)])
+@pytest.mark.parametrize("shape", [(4352, 4352, 2048), (5120, 5120, 2080), (5000, 5000, 2052), (4608, 4864, 3072), (4228, 4612, 2060), (4100, 5376, 2052)])
 def test_wave_tile_last_round_shared_with_workspace(prism, oracle, shape):
     """256 x 256 tiles that are not a whole number of rounds of the CUs, through prism_sgemm_ws: the whole rounds
-    run one tile per workgroup, the K ranges of the tiles of the last round (33, 144, 144, 86 and 67 here) are
+    run one tile per workgroup, the K ranges of the tiles of the last round (33, 144, 144, 86, 67 and 80 beside a strip of four rows here) are
     shared between all CUs, and a second kernel adds a tile's partial products (K of 2048 and up: below that the
     entry point leaves the product to prism_sgemm, see test_short_k_is_not_shared). Whole tiles and ragged M, N, K
     (rows 16 B aligned). Every element against an fp64 product formed on the
@@ -260,7 +260,7 @@ def test_wave_tile_last_round_shared_with_workspace(prism, oracle, shape):
     import fp64_referee
     M, N, K = shape
     cus = prism.device_info()["cu_count"]
-    tiles = -(-M // 256) * -(-N // 256)
+    tiles = (M // 256 if 0 < M % 256 <= 8 else -(-M // 256)) * -(-N // 256)   # up to 8 rows beyond whole tiles go to the strip kernel
     need = prism.sgemm_workspace_size(M, N, K)
     assert need == 2 * cus * 256 * 256 * 4
     assert prism.sgemm_workspace_plan(M, N, K, need) == (cus, tiles % cus)
@@ -310,6 +310,31 @@ def test_wave_tile_short_k_runs_as_halves(prism, oracle, shape):
         err = fp64_referee.sgemm_max_err_fp64(0.75, A, B, beta, C0, c)
         assert err <= _bound(K, beta), f"{M}x{N}x{K} beta={beta}: max error {err:.3e}"
         assert bool((cbuf[:64] == 777.0).all()) and bool((cbuf[64 + M * N:] == 777.0).all())
+
+
+@pytest.mark.parametrize("shape", [(4097, 4097, 1025), (4100, 4096, 512), (8193, 4100, 300), (4104, 4104, 2100), (4098, 6000, 17), (4097, 4096, 4096)])
+def test_wave_tile_thin_strip_of_rows(prism, oracle, shape):
+    """M a few rows (1 to 8) beyond a whole number of 256-row tiles: the rows before run as ever, a strip kernel
+    takes the rest (with a thin strip of columns at the same time, ragged N and K, K shorter than its sixteen
+    wavefronts' shares and longer than one trip of their loops). Every element against fp64; C poisoned with
+    NaN when it is not read; guard values around C; operands that start at an odd element."""
+    import fp64_referee
+    M, N, K = shape
+    A0, B0, C0 = _device_inputs(M, N, K)
+    for beta, shift in ((0.5, 0), (0.0, 1)):
+        abuf = torch.full((M * K + 8,), float("nan"), device=DEV)
+        bbuf = torch.full((K * N + 8,), float("nan"), device=DEV)
+        A, B = abuf[shift:shift + M * K].view(M, K), bbuf[shift:shift + K * N].view(K, N)
+        A.copy_(A0)
+        B.copy_(B0)
+        cbuf = torch.full((M * N + 128,), 777.0, device=DEV)
+        c = cbuf[64 + shift:64 + shift + M * N].view(M, N)
+        c.copy_(C0 if beta else torch.full((M, N), float("nan"), device=DEV))
+        print(f"prism_sgemm {M}x{N}x{K} beta={beta} operands start at element {shift}", flush=True)
+        prism.sgemm(M, N, K, 0.75, A, B, beta, c, variant=5)
+        err = fp64_referee.sgemm_max_err_fp64(0.75, A0, B0, beta, C0, c)
+        assert err <= _bound(K, beta), f"{M}x{N}x{K} beta={beta}: max error {err:.3e}"
+        assert bool((cbuf[:64 + shift] == 777.0).all()) and bool((cbuf[64 + shift + M * N:] == 777.0).all())
 
 
 @pytest.mark.parametrize("shape", [(4096, 3073, 100), (4000, 3080, 67), (4096, 3076, 64), (8191, 4097, 1023), (4096, 3329, 4), (3000, 4099, 2100)])
