@@ -396,6 +396,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_ring_
     const uint32_t lane_off = (static_cast<uint32_t>(lane / KP) * static_cast<uint32_t>(ld) + ld_chunk * 8) * 2u;  // bytes
     const char* p_wave = reinterpret_cast<const char*>(P + static_cast<size_t>(row0 + wave * ROWS_PER_LOAD) * ld);
     const char* q_wave = reinterpret_cast<const char*>(Q + static_cast<size_t>(col0 + wave * ROWS_PER_LOAD) * ld);
+
     const size_t pass_bytes = static_cast<size_t>(ROWS_PER_PASS) * ld * 2;
     // Load number m (0 .. LOADS - 1) of the tile that starts at k0, into stage `stage`.
     const int p_first = row0 + wave * ROWS_PER_LOAD, q_first = col0 + wave * ROWS_PER_LOAD;
@@ -618,11 +619,17 @@ __device__ __forceinline__ void mfma_results_settle() {
 // start at 2 B-aligned addresses, which the memory path accepts (measured on gfx950, for the lane offset and
 // for the descriptor's base). The K loop covers K rounded down to a multiple of 8, where every chunk lies
 // inside its row, and the last K % 8 values of k are added in front of the write-back from ordinary loads.
-template <int BM, int BN, int WM, int WN, bool EDGE, typename OutT, bool RAGGED = false>
+//
+// PERSIST (whole tiles only): a workgroup takes tiles blockIdx.x, blockIdx.x + gridDim.x, ... of n_tiles one after
+// the other. The sixteen loads every phase issues, which in the last two phases of a tile have nothing left to
+// fetch, then fetch the first two K tiles of the workgroup's NEXT tile: the next tile starts with its operands in
+// LDS, the write-back's stores drain while it multiplies, and no workgroup is launched or retired in between.
+template <int BM, int BN, int WM, int WN, bool EDGE, typename OutT, bool RAGGED = false, bool PERSIST = false>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early_kernel(
     int R, int Cn, int K_all, const uint16_t* __restrict__ P, const uint16_t* __restrict__ Q,
-    OutT* __restrict__ OUT, int tiles_m, int tiles_n) {
+    OutT* __restrict__ OUT, int tiles_m, int tiles_n, int n_tiles = 0) {
     static_assert(EDGE || !RAGGED, "the ragged form is an edge form");
+    static_assert(!PERSIST || !EDGE, "the persistent form takes whole tiles");
     // ld: elements between rows of P and of Q. K: the part of the k range the loop covers.
     const int ld = K_all;
     const int K = RAGGED ? K_all - K_all % 8 : K_all;
@@ -639,9 +646,10 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
 
     __shared__ __attribute__((aligned(1024))) uint16_t Ps[2][BM * BK];
     __shared__ __attribute__((aligned(1024))) uint16_t Qs[2][BN * BK];
+    int tile = blockIdx.x;
     int tm, tn;
-    xcd_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
-    const int row0 = tm * BM, col0 = tn * BN;
+    xcd_tile_coords(tile, tiles_m, tiles_n, tm, tn);
+    int row0 = tm * BM, col0 = tn * BN;
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -650,17 +658,12 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     const int l16 = lane & 15, lq = lane >> 4;
 
     f32x4 acc[MI][NI];
-#pragma unroll
-    for (int i = 0; i < MI; ++i)
-#pragma unroll
-        for (int j = 0; j < NI; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
     // Load side, as in gemm_bf16_ring_kernel.
     const int ld_row = wave * ROWS_PER_LOAD + lane / KP;
     const int ld_chunk = (lane % KP) ^ ((ld_row >> SWZ) & (KP - 1));
     const uint32_t lane_off = (static_cast<uint32_t>(lane / KP) * static_cast<uint32_t>(ld) + ld_chunk * 8) * 2u;
-    const char* p_wave = reinterpret_cast<const char*>(P + static_cast<size_t>(row0 + wave * ROWS_PER_LOAD) * ld);
-    const char* q_wave = reinterpret_cast<const char*>(Q + static_cast<size_t>(col0 + wave * ROWS_PER_LOAD) * ld);
+
     // The loads go through two buffer descriptors (this wave's first P row, its first Q row) for their
     // addressing mode, not for range checks: descriptor base + scalar offset + lane offset, where the scalar
     // offset (load number x rows per pass) and the lane offset are loop-invariant and only the two bases
@@ -676,10 +679,17 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     // (Forced into a scalar register here: direct_load16_buffer_to_destination takes its scalar operands as
     // they are, so that no v_readfirstlane ends up right in front of a load.)
     const uint32_t pass_bytes = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(ROWS_PER_PASS) * static_cast<uint32_t>(ld) * 2u);  // the launcher keeps BM * K * 2 below 2^31
-    const int p_first = row0 + wave * ROWS_PER_LOAD, q_first = col0 + wave * ROWS_PER_LOAD;
-    const long long p_left = static_cast<long long>(R - p_first) * ld * 2, q_left = static_cast<long long>(Cn - q_first) * ld * 2;
-    const i32x4 p_rsrc = buffer_descriptor(EDGE && p_left <= 0 ? reinterpret_cast<const char*>(P) : p_wave, EDGE ? clamped_extent(p_left) : 0x7fffffffu);
-    const i32x4 q_rsrc = buffer_descriptor(EDGE && q_left <= 0 ? reinterpret_cast<const char*>(Q) : q_wave, EDGE ? clamped_extent(q_left) : 0x7fffffffu);
+    // The two descriptors of the tile whose first row / column is r0 / c0.
+    auto descriptors_of = [&](int r0, int c0, i32x4& p_desc, i32x4& q_desc) {
+        const char* p_wave = reinterpret_cast<const char*>(P + static_cast<size_t>(r0 + wave * ROWS_PER_LOAD) * ld);
+        const char* q_wave = reinterpret_cast<const char*>(Q + static_cast<size_t>(c0 + wave * ROWS_PER_LOAD) * ld);
+        const int p_first = r0 + wave * ROWS_PER_LOAD, q_first = c0 + wave * ROWS_PER_LOAD;
+        const long long p_left = static_cast<long long>(R - p_first) * ld * 2, q_left = static_cast<long long>(Cn - q_first) * ld * 2;
+        p_desc = buffer_descriptor(EDGE && p_left <= 0 ? reinterpret_cast<const char*>(P) : p_wave, EDGE ? clamped_extent(p_left) : 0x7fffffffu);
+        q_desc = buffer_descriptor(EDGE && q_left <= 0 ? reinterpret_cast<const char*>(Q) : q_wave, EDGE ? clamped_extent(q_left) : 0x7fffffffu);
+    };
+    i32x4 p_rsrc, q_rsrc;
+    descriptors_of(row0, col0, p_rsrc, q_rsrc);
     auto advanced = [](i32x4 d, uint32_t bytes) {  // the descriptor with its base moved up
         const uint64_t a = ((static_cast<uint64_t>(static_cast<uint32_t>(d[1])) << 32) | static_cast<uint32_t>(d[0])) + bytes;
         d[0] = static_cast<int>(a & 0xffffffffu);
@@ -764,14 +774,14 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     // code for the last two phases it moved accumulators between registers right behind matrix
     // instructions whose latency it does not know, see mfma_16x16x32_in_place, and read them too early;
     // with the loads under a run-time condition the branches cost 5 %.)
-    auto phase = [&](auto stage_c, uint32_t k_next_bytes) {
+    auto phase = [&](auto stage_c, const i32x4& p_from, const i32x4& q_from, uint32_t k_next_bytes) {
         constexpr int S = decltype(stage_c)::value;
         constexpr int MINE = 1 + S, OTHER = 2 - S;  // fragment sets of k-step 1: this stage's, the other stage's
         // Load number n goes behind instruction BARRIER_AT + n * GAP of the phase's 128 (counted from the
         // start of the first block); the barrier that frees the stage sits behind instruction BARRIER_AT - 1.
         constexpr int BARRIER_AT = kEarlyBarrierAt, GAP = kEarlyLoadGap;
         static_assert(BARRIER_AT >= 33 && BARRIER_AT <= 64 && BARRIER_AT + (LOADS - 1) * GAP < 128, "loads fit the phase");
-        const i32x4 pd = advanced(p_rsrc, k_next_bytes), qd = advanced(q_rsrc, k_next_bytes);
+        const i32x4 pd = advanced(p_from, k_next_bytes), qd = advanced(q_from, k_next_bytes);
         const uint32_t off = lane_offset_at(static_cast<int>(k_next_bytes / 2));
         auto maybe_load = [&](int at) {  // `at` = number of the instruction just issued, 0..127
             if (at + 1 >= BARRIER_AT && (at + 1 - BARRIER_AT) % GAP == 0 && (at + 1 - BARRIER_AT) / GAP < LOADS)
@@ -797,12 +807,6 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     };
     using s0 = std::integral_constant<int, 0>;
     using s1 = std::integral_constant<int, 1>;
-
-    // "k-step 1 of the tile before the first" multiplies zeros (set 2 is what the first phase, stage 0, uses).
-#pragma unroll
-    for (int i = 0; i < MI; ++i) fp[2][i] = bf16x8{};
-#pragma unroll
-    for (int j = 0; j < NI; ++j) fq[2][j] = bf16x8{};
 
     // Tile t lives in stage t % 2. Whole tiles: the launcher guarantees an even number of K tiles, at least 4;
     // EDGE: the count is padded to one (the padding tiles load zeros).
@@ -836,6 +840,28 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
+  while (true) {   // one output tile per trip (a single trip unless PERSIST)
+    // Entered with the tile's first K tile complete in stage 0 and its second one on the way into stage 1.
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    // "k-step 1 of the tile before the first" multiplies zeros (set 2 is what the first phase, stage 0, uses).
+#pragma unroll
+    for (int i = 0; i < MI; ++i) fp[2][i] = bf16x8{};
+#pragma unroll
+    for (int j = 0; j < NI; ++j) fq[2][j] = bf16x8{};
+    // The workgroup's next tile, if it has one: what the last two phases fetch.
+    const int next_tile = PERSIST ? tile + static_cast<int>(gridDim.x) : 0;
+    const bool has_next = PERSIST && next_tile < n_tiles;
+    int next_row0 = row0, next_col0 = col0;
+    i32x4 p_next = p_rsrc, q_next = q_rsrc;
+    if (has_next) {
+        xcd_tile_coords(next_tile, tiles_m, tiles_n, tm, tn);
+        next_row0 = tm * BM;
+        next_col0 = tn * BN;
+        descriptors_of(next_row0, next_col0, p_next, q_next);
+    }
     for (int t = 0; t < k_tiles; t += 2) {
         // Fragment registers that the vector ALU has written (the zeros of set 2 above, and the copies the
         // compiler makes of them in front of the loop) need wait states before a matrix instruction reads
@@ -845,15 +871,31 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
         // call only). Here scalar instructions happen to sit in between; the five wait states make that
         // independent of what the compiler puts at the head of the loop, and cost nothing measurable.
         asm volatile("s_nop 4");
-        const int next = t + 2 < k_tiles ? t + 2 : k_tiles - 2;
+        // What this pair of phases fetches: K tiles t + 2 and t + 3 of this tile; in the last trip the first two K
+        // tiles of the next tile, or, without one, the last two of this tile once more. Selected, not branched
+        // on: the trips stay the same straight-line code.
+        const bool last = t + 2 >= k_tiles;
+        const int next = last ? (has_next ? 0 : k_tiles - 2) : t + 2;
         const uint32_t k_next_bytes = k_bytes_of(next);  // k_first and next are even: next + 1 does not wrap
-        phase(s0{}, k_next_bytes);
-        phase(s1{}, k_next_bytes + BK * 2);
+        i32x4 p_from = p_rsrc, q_from = q_rsrc;
+        if (last) {
+            p_from = p_next;
+            q_from = q_next;
+        }
+        phase(s0{}, p_from, q_from, k_next_bytes);
+        phase(s1{}, p_from, q_from, k_next_bytes + BK * 2);
     }
     // k-step 1 of the last tile (stage 1 -> set 2). Outside the loop the compiler is free to move accumulators
     // to other registers; it does so between these instructions, so here they are issued through the builtin,
     // whose result latency it knows.
     mfma_results_settle();
+    // Every later use of an accumulator takes it from here, behind the wait states: without this the compiler is
+    // free to copy accumulators in front of them (they are no memory operation, which is all the settling
+    // assembly orders), and in the persistent form it did.
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) asm volatile("" : "+a"(acc[i][j]));
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
@@ -921,6 +963,13 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
         if (!EDGE || (row0 + BM <= R && col0 + BN <= Cn)) write_back(std::false_type{});
         else write_back(std::true_type{});
     }
+    if (!has_next) break;
+    tile = next_tile;
+    row0 = next_row0;
+    col0 = next_col0;
+    p_rsrc = p_next;
+    q_rsrc = q_next;
+  }
     // The last, redundant loads write LDS: they must have landed before the wave ends and its LDS goes to
     // the next workgroup. Behind the write-back the wait is covered by the stores.
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));
@@ -953,8 +1002,12 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
         const int left = tiles % cus;
         const bool cut = tiles > cus && left != 0 && left * 4 <= 2 * cus;
         const int main_tiles = cut ? tiles - left : tiles;
-        gemm_bf16_early_kernel<BM, BN, WM, WN, false, OutT><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
-            R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
+        if (main_tiles > cus && cus % 8 == 0)   // more than one round: one workgroup per CU walks its tiles (see PERSIST)
+            gemm_bf16_early_kernel<BM, BN, WM, WN, false, OutT, false, true><<<dim3(static_cast<unsigned>(cus)), block, 0, s>>>(
+                R, Cn, K, P, Q, OUT, tiles_m, tiles_n, main_tiles);
+        else
+            gemm_bf16_early_kernel<BM, BN, WM, WN, false, OutT><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
+                R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
         if (int rc = check_launch("gemm_bf16_early_kernel")) return rc;
         if (cut) {
             if (left * 4 <= cus)  // one per CU: the four-deep ring, as below
