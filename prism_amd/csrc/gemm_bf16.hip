@@ -774,7 +774,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     // code for the last two phases it moved accumulators between registers right behind matrix
     // instructions whose latency it does not know, see mfma_16x16x32_in_place, and read them too early;
     // with the loads under a run-time condition the branches cost 5 %.)
-    auto phase = [&](auto stage_c, const i32x4& p_from, const i32x4& q_from, uint32_t k_next_bytes) {
+    auto phase = [&](auto stage_c, const i32x4& p_from, const i32x4& q_from, uint32_t k_next_bytes, bool wait_at_end) {
         constexpr int S = decltype(stage_c)::value;
         constexpr int MINE = 1 + S, OTHER = 2 - S;  // fragment sets of k-step 1: this stage's, the other stage's
         // Load number n goes behind instruction BARRIER_AT + n * GAP of the phase's 128 (counted from the
@@ -800,7 +800,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
             maybe_load(m);
         });
         mfma_block(0, [&](int m) { maybe_load(64 + m); });
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(LOADS, kLgkmMax));
+        if (wait_at_end) __builtin_amdgcn_s_waitcnt(waitcnt_imm(LOADS, kLgkmMax));
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");  // the compiler does not know that the loads write LDS: no read moves above the barrier
         __builtin_amdgcn_sched_barrier(0);
@@ -836,7 +836,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
 #pragma unroll
         for (int m = 0; m < LOADS; ++m) issue_load(1, pd, qd, off, m);
     }
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(LOADS, kLgkmMax));
+    // PERSIST: both K tiles have landed at the head of every tile (see the wait in front of the write-back).
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(PERSIST ? 0 : LOADS, kLgkmMax));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
@@ -882,8 +883,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
             p_from = p_next;
             q_from = q_next;
         }
-        phase(s0{}, p_from, q_from, k_next_bytes);
-        phase(s1{}, p_from, q_from, k_next_bytes + BK * 2);
+        // PERSIST: the first phase of a tile does not wait at its end. What that wait is for, the tile's second K
+        // tile, has landed already, and the loads are counted in order: it would wait for the 64 stores of the
+        // tile before, which sit in front of this phase's loads. They get one more phase to drain.
+        phase(s0{}, p_from, q_from, k_next_bytes, !PERSIST || t != 0);
+        phase(s1{}, p_from, q_from, k_next_bytes + BK * 2, true);
     }
     // k-step 1 of the last tile (stage 1 -> set 2). Outside the loop the compiler is free to move accumulators
     // to other registers; it does so between these instructions, so here they are issued through the builtin,
@@ -960,6 +964,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
             __builtin_amdgcn_sched_barrier(0);  // one column block at a time: its 28 Q values and no more
         }
     } else {
+        // PERSIST: the next tile's first two K tiles (fetched by the last two phases) land before the stores queue up
+        // behind them; its first phase relies on that.
+        if constexpr (PERSIST) __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));
         if (!EDGE || (row0 + BM <= R && col0 + BN <= Cn)) write_back(std::false_type{});
         else write_back(std::true_type{});
     }
@@ -973,6 +980,96 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
     // The last, redundant loads write LDS: they must have landed before the wave ends and its LDS goes to
     // the next workgroup. Behind the write-back the wait is covered by the stores.
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));
+}
+
+// Up to 16 rows of one operand against all rows of the other: D[f][g] = sum_k F[f][k] * G[g][k], f < f_count <= 16.
+// The strips that a matrix leaves beyond whole 256 x 256 tiles when it hangs over them by a few rows or columns go
+// here instead of into a round of edge tiles of their own (4097 x 4097 x 4096: one round of whole tiles plus two
+// strips instead of 289 guarded tiles in two rounds). Reading G bounds it: one 16 x 16 x 32 matrix instruction per 1 KB
+// of G, both fragments straight from global memory (F stays in the caches). A workgroup takes 16 rows of G; its eight
+// waves split K and add their parts in a fixed order. K is a multiple of 8 and both operands are 16 B aligned.
+// ALONG_G: OUT[f * ldo + g] (extra rows of P: F = those rows, G = Q); else OUT[g * ldo + f] (extra rows of Q, i.e.
+// extra columns of OUT: F = those rows, G = P). The instruction gets the operand first whose index runs along OUT's
+// rows, so that a lane's four results are neighbours in memory (see the write-back of gemm_bf16_early_kernel).
+constexpr int kThinMax = 16, kThinWaves = 8;
+template <bool ALONG_G, typename OutT>
+__global__ __launch_bounds__(kThinWaves * kWave) void gemm_bf16_thin_kernel(
+    int f_count, int g_count, int K, const uint16_t* __restrict__ F, const uint16_t* __restrict__ G,
+    OutT* __restrict__ OUT, long long ldo) {
+    __shared__ f32x4 part[kThinWaves][kWave];
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int l16 = lane % 16, lq = lane / 16;
+    const int g0 = static_cast<int>(blockIdx.x) * 16;
+    const bool f_ok = l16 < f_count, g_ok = g0 + l16 < g_count;
+    const uint16_t* f_at = F + static_cast<size_t>(f_ok ? l16 : 0) * K + 8 * lq;
+    const uint16_t* g_at = G + static_cast<size_t>(g_ok ? g0 + l16 : 0) * K + 8 * lq;
+    // Steps of 32 along K; wave w takes steps [w * per, (w + 1) * per). The last step may be short: packets of
+    // 8 that begin at or beyond K are zeros.
+    const int steps = ceil_div(K, 32), per = ceil_div(steps, kThinWaves);
+    const int first = wave * per, last = first + per < steps ? first + per : steps;
+    constexpr int U = 4;
+    f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int step = first; step < last; step += U) {
+        bf16x8 fv[U], gv[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int k = (step + u) * 32;
+            const bool in = step + u < last && k + 8 * lq < K;
+            fv[u] = in && f_ok ? *reinterpret_cast<const bf16x8*>(f_at + k) : bf16x8{};
+            gv[u] = in && g_ok ? *reinterpret_cast<const bf16x8*>(g_at + k) : bf16x8{};
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            acc = ALONG_G ? __builtin_amdgcn_mfma_f32_16x16x32_bf16(gv[u], fv[u], acc, 0, 0, 0)
+                          : __builtin_amdgcn_mfma_f32_16x16x32_bf16(fv[u], gv[u], acc, 0, 0, 0);
+    }
+    part[wave][lane] = acc;
+    __syncthreads();
+    if (wave != 0) return;
+    f32x4 sum = part[0][lane];
+#pragma unroll
+    for (int w = 1; w < kThinWaves; ++w) sum += part[w][lane];
+    // ALONG_G: the lane holds D[f = l16][g = g0 + 4 lq + v]; else D[f = 4 lq + v][g = g0 + l16].
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const int f = ALONG_G ? l16 : 4 * lq + v, g = ALONG_G ? g0 + 4 * lq + v : g0 + l16;
+        if (f < f_count && g < g_count)
+            store_out(&OUT[ALONG_G ? f * ldo + g : g * ldo + f], sum[v]);
+    }
+}
+
+// Whole 256 x 256 tiles with K a multiple of 128, at least 384: tiles_m x tiles_n of them from the top left corner
+// of OUT (R and Cn bound the operands and give OUT's row length; they may reach beyond the tiles).
+template <int BM, int BN, int WM, int WN, typename OutT>
+int run_whole_tiles(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, OutT* OUT, int tiles_m, int tiles_n,
+                    hipStream_t s) {
+    const dim3 block((BM / WM) * (BN / WN) * kWave);
+
+    // Tile counts that do not fill whole rounds of CUs: the 256 x 256 kernel takes the whole rounds and
+    // the tiles of the last, partial round are cut into 128 x 128 tiles (two workgroups per CU), when
+    // that gives every CU at most two of them (6144^3: 2 rounds + 64 tiles instead of 3 rounds).
+    static_assert(BM == 256 && BN == 256, "the leftover launch cuts 256 x 256 tiles");
+    const int tiles = tiles_m * tiles_n, cus = cu_count();
+    const int left = tiles % cus;
+    const bool cut = tiles > cus && left != 0 && left * 4 <= 2 * cus;
+    const int main_tiles = cut ? tiles - left : tiles;
+    if (main_tiles > cus && cus % 8 == 0)   // more than one round: one workgroup per CU walks its tiles (see PERSIST)
+        gemm_bf16_early_kernel<BM, BN, WM, WN, false, OutT, false, true><<<dim3(static_cast<unsigned>(cus)), block, 0, s>>>(
+            R, Cn, K, P, Q, OUT, tiles_m, tiles_n, main_tiles);
+    else
+        gemm_bf16_early_kernel<BM, BN, WM, WN, false, OutT><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
+            R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
+    if (int rc = check_launch("gemm_bf16_early_kernel")) return rc;
+    if (cut) {
+        if (left * 4 <= cus)  // one per CU: the four-deep ring, as below
+            gemm_bf16_ring_kernel<128, 128, 64, 4, 64, 64, false, OutT><<<dim3(static_cast<unsigned>(left) * 4), dim3(256), 0, s>>>(
+                R, Cn, K, P, Q, OUT, tiles_m, tiles_n, main_tiles);
+        else
+            gemm_bf16_ring_kernel<128, 128, 64, 2, 64, 64, false, OutT><<<dim3(static_cast<unsigned>(left) * 4), dim3(256), 0, s>>>(
+                R, Cn, K, P, Q, OUT, tiles_m, tiles_n, main_tiles);
+        return check_launch("gemm_bf16_ring_kernel (leftover)");
+    }
+    return 0;
 }
 
 // Kernel choice. Whole 256 x 256 x 64 tiles: the early-read pipeline whenever the K tile count is even and
@@ -993,33 +1090,28 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
     const bool panel_ok = static_cast<long long>(BM > BN ? BM : BN) * (static_cast<long long>(K) + 6 * 64) * 2 < (1ll << 31);
     const bool few_tiles = static_cast<long long>(tiles_m) * tiles_n * 2 < cu_count();
     const bool lane_offsets_ok = static_cast<long long>(K) * 2 * 64 < (1ll << 32);  // 32-bit lane offsets inside a load's rows
-    if (whole && !few_tiles && K % 128 == 0 && K >= 6 * 64 && panel_ok && lane_offsets_ok) {
-        // Tile counts that do not fill whole rounds of CUs: the 256 x 256 kernel takes the whole rounds and
-        // the tiles of the last, partial round are cut into 128 x 128 tiles (two workgroups per CU), when
-        // that gives every CU at most two of them (6144^3: 2 rounds + 64 tiles instead of 3 rounds).
-        static_assert(BM == 256 && BN == 256, "the leftover launch cuts 256 x 256 tiles");
-        const int tiles = tiles_m * tiles_n, cus = cu_count();
-        const int left = tiles % cus;
-        const bool cut = tiles > cus && left != 0 && left * 4 <= 2 * cus;
-        const int main_tiles = cut ? tiles - left : tiles;
-        if (main_tiles > cus && cus % 8 == 0)   // more than one round: one workgroup per CU walks its tiles (see PERSIST)
-            gemm_bf16_early_kernel<BM, BN, WM, WN, false, OutT, false, true><<<dim3(static_cast<unsigned>(cus)), block, 0, s>>>(
-                R, Cn, K, P, Q, OUT, tiles_m, tiles_n, main_tiles);
-        else
-            gemm_bf16_early_kernel<BM, BN, WM, WN, false, OutT><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
-                R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
-        if (int rc = check_launch("gemm_bf16_early_kernel")) return rc;
-        if (cut) {
-            if (left * 4 <= cus)  // one per CU: the four-deep ring, as below
-                gemm_bf16_ring_kernel<128, 128, 64, 4, 64, 64, false, OutT><<<dim3(static_cast<unsigned>(left) * 4), dim3(256), 0, s>>>(
-                    R, Cn, K, P, Q, OUT, tiles_m, tiles_n, main_tiles);
-            else
-                gemm_bf16_ring_kernel<128, 128, 64, 2, 64, 64, false, OutT><<<dim3(static_cast<unsigned>(left) * 4), dim3(256), 0, s>>>(
-                    R, Cn, K, P, Q, OUT, tiles_m, tiles_n, main_tiles);
-            return check_launch("gemm_bf16_ring_kernel (leftover)");
+    // A few rows or columns beyond whole tiles (at most kThinMax each way) over at least half a round of whole
+    // tiles: the whole tiles as below, the rest as strips (gemm_bf16_thin_kernel).
+    const int r_thin = R % BM, c_thin = Cn % BN;
+    if ((r_thin != 0 || c_thin != 0) && r_thin <= kThinMax && c_thin <= kThinMax && aligned && K % 128 == 0 && K >= 6 * 64 &&
+        panel_ok && lane_offsets_ok && static_cast<long long>(R / BM) * (Cn / BN) * 2 >= cu_count()) {
+        const int Rw = R - r_thin, Cw = Cn - c_thin;
+        if (int rc = run_whole_tiles<BM, BN, WM, WN, OutT>(R, Cn, K, P, Q, OUT, Rw / BM, Cw / BN, s)) return rc;
+        const dim3 thin_block(kThinWaves * kWave);
+        if (r_thin != 0) {  // rows Rw.. of OUT, all columns
+            gemm_bf16_thin_kernel<true, OutT><<<dim3(static_cast<unsigned>(ceil_div(Cn, 16))), thin_block, 0, s>>>(
+                r_thin, Cn, K, P + static_cast<size_t>(Rw) * K, Q, OUT + static_cast<size_t>(Rw) * Cn, Cn);
+            if (int rc = check_launch("gemm_bf16_thin_kernel (rows)")) return rc;
+        }
+        if (c_thin != 0) {  // columns Cw.. of OUT, the rows of the whole tiles
+            gemm_bf16_thin_kernel<false, OutT><<<dim3(static_cast<unsigned>(ceil_div(Rw, 16))), thin_block, 0, s>>>(
+                c_thin, Rw, K, Q + static_cast<size_t>(Cw) * K, P, OUT + Cw, Cn);
+            if (int rc = check_launch("gemm_bf16_thin_kernel (columns)")) return rc;
         }
         return 0;
     }
+    if (whole && !few_tiles && K % 128 == 0 && K >= 6 * 64 && panel_ok && lane_offsets_ok)
+        return run_whole_tiles<BM, BN, WM, WN, OutT>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n, s);
     // The same for rows that are not 16 B aligned (K not a multiple of 8, operands at an odd element).
     if (few_tiles && !(aligned && K % 8 == 0) && K >= 8 && panel_ok) {
         const int tm = ceil_div(R, 128), tn = ceil_div(Cn, 128);

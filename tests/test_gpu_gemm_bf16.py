@@ -98,6 +98,22 @@ def test_ragged_shapes_with_aligned_rows(prism, oracle, shape):
     starting points, and the five shapes before the last two: K tile counts of 7, 2, 1, 5 and 6 before
     padding to an even count of at least 4). The matrices sit between NaNs, so one element read from outside a
     matrix, or from the next row in the partial K tile, would poison the output; stores are fenced too."""
+    check_between_fences(prism, oracle, shape)
+
+
+@pytest.mark.parametrize("shape", [(2817, 3088, 384), (3072, 3073, 512), (3080, 3072, 640), (4097, 4100, 768), (3088, 2832, 1152),
+                                   (2829, 3074, 2048)])
+def test_thin_strips_beyond_whole_tiles(prism, oracle, shape):
+    """Up to 16 rows and up to 16 columns beyond whole 256 x 256 tiles, over at least half a round of whole tiles, K
+    a multiple of 128 from 384 up: the whole tiles run unguarded (one launch, or one workgroup per CU walking
+    several tiles in the fourth shape) and the rest as strips, 16 rows of the long operand to a workgroup whose eight
+    waves split K (3, 4, 5, 6, 9 and 16 steps of 32 to a wave, with fewer or none for the last waves). fp32 output and the
+    transposed bf16 output, where rows and columns change places. Operands and outputs sit between NaNs and
+    fences."""
+    check_between_fences(prism, oracle, shape)
+
+
+def check_between_fences(prism, oracle, shape):
     M, N, K = shape
     A16, B16 = oracle.gen_gemm_bf16(M, N, K, seed=3 * M + N + K)
     buf = torch.full((M * N + 512,), 777.0, dtype=torch.float32, device=DEV)
