@@ -1075,7 +1075,7 @@ int run_whole_tiles(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, 
 // Kernel choice. Whole 256 x 256 x 64 tiles: the early-read pipeline whenever the K tile count is even and
 // at least 6, else the direct-to-LDS ring (any count from 2). Ragged M, N or K with K a multiple of 8 and
 // 16 B-aligned operands: the early-read pipeline's edge variant (K tiles padded with zeros to an even count).
-// Rows that are not 16 B aligned: its ragged form. Fewer than 128 tiles: 128 x 128 tiles of the ring, with the
+// Rows that are not 16 B aligned: its ragged form. At most 128 tiles: 128 x 128 tiles of the ring, with the
 // same edge and ragged forms. Everything else: the general kernel.
 template <int BM, int BN, int BK, int WM, int WN, typename OutT>
 int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, OutT* OUT,
@@ -1088,7 +1088,9 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
     const bool whole = (R % BM == 0) && (Cn % BN == 0) && aligned;
     // A 256-row panel (plus up to six K tiles of padding) is addressed with 32-bit offsets.
     const bool panel_ok = static_cast<long long>(BM > BN ? BM : BN) * (static_cast<long long>(K) + 6 * 64) * 2 < (1ll << 31);
-    const bool few_tiles = static_cast<long long>(tiles_m) * tiles_n * 2 < cu_count();
+    // Up to half as many 256 x 256 tiles as CUs: as 128 x 128 tiles they still all run at once, two to a CU
+    // (1024 x 8192 x 8192, 128 tiles: 1050 -> 1190 TFLOP/s; with more tiles the small ones lose, 160: 1170 -> 900).
+    const bool few_tiles = static_cast<long long>(tiles_m) * tiles_n * 2 <= cu_count();
     const bool lane_offsets_ok = static_cast<long long>(K) * 2 * 64 < (1ll << 32);  // 32-bit lane offsets inside a load's rows
     // A few rows or columns beyond whole tiles (at most kThinMax each way) over at least half a round of whole
     // tiles: the whole tiles as below, the rest as strips (gemm_bf16_thin_kernel).

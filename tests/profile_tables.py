@@ -48,7 +48,7 @@ def measured_traffic(workload: str, size: int):
 TRAFFIC_KERNELS = [  # (workload, size, substring of the kernel name, threads in the grid)
     ("sgemm", 8192, "sgemm_wave_tile_dma_kernel", 1024 * 1024),
     ("scan", 1 << 30, "scan_lookback_kernel", (1 << 30) // 65536 * 1024),
-    ("gemm_bf16", 8192, "gemm_bf16_early_kernel", 1024 * 256),
+    ("gemm_bf16", 8192, "gemm_bf16_early_kernel", 256 * 256),  # one workgroup per CU walks four tiles
     ("add_m", 1 << 24, "add_m_vec4_kernel", (1 << 24) // 4),
     ("add_m", 1 << 28, "add_m_vec4_kernel", (1 << 28) // 4),
 ]
@@ -203,9 +203,9 @@ COUNTER_PASSES = {
 GEMM_ROWS = [  # (label, substrings that must all occur in the kernel name, grid size in threads)
     ("ours, SGEMM kernel 5 (fp32)", ["sgemm_wave_tile_dma_kernel<256, 256, 32, 32, 128, false, false, false>"], 1024 * 1024),
     ("rocBLAS `rocblas_sgemm` (fp32)", ["Cijk_Ailk_Bljk_SB_"], None),
-    ("ours, bf16 in, fp32 out", ["gemm_bf16_early_kernel<256, 256, 128, 128, false, float"], 256 * 1024),
+    ("ours, bf16 in, fp32 out", ["gemm_bf16_early_kernel<256, 256, 128, 128, false, float"], 256 * 256),
     ("hipBLASLt, bf16 in, fp32 out", ["Cijk_Alik_Bljk_BSS_BH"], None),
-    ("ours, bf16 in, bf16 column-major out", ["gemm_bf16_early_kernel<256, 256, 128, 128, false, unsigned short"], 256 * 1024),
+    ("ours, bf16 in, bf16 column-major out", ["gemm_bf16_early_kernel<256, 256, 128, 128, false, unsigned short"], 256 * 256),
     ("hipBLASLt, bf16 in, bf16 column-major out", ["Cijk_Alik_Bljk_BBS_BH"], None),
 ]
 STREAM_ROWS = [

@@ -51,12 +51,12 @@ def test_fp32_output_vs_fp64_oracle(prism, oracle, shape):
                                    (256, 512, 6144), (512, 256, 6208), (128, 384, 6272),
                                    (3072, 3072, 384), (3072, 3072, 192), (2816, 3328, 448), (3072, 3328, 512),
                                    (4352, 4352, 384), (4608, 4608, 384), (2560, 2304, 320), (2304, 2560, 448),
-                                   (3072, 3072, 1280)])
+                                   (3072, 3072, 1280), (2048, 4096, 384)])
 def test_whole_tile_paths(prism, oracle, shape):
-    """Problems made of whole tiles leave the general kernel. Fewer than 128 tiles of 256 x 256 (the first
-    ten shapes and the last two): 128 x 128 tiles, direct-to-LDS ring, four K tiles deep where every CU gets at
+    """Problems made of whole tiles leave the general kernel. Up to 128 tiles of 256 x 256, half the CUs (the first
+    ten shapes, the two before the last two, and the last with exactly 128): 128 x 128 tiles, direct-to-LDS ring, four K tiles deep where every CU gets at
     most one tile and K has four tiles (K tile counts of 4, 5, 6, 7, 16, 96, 97 and 98 here), two deep otherwise
-    (K of 128 and 192; the two shapes before the last with 360 tiles). From 128 tiles up: an even K tile count from 6 up
+    (K of 128 and 192; the two shapes with 360 tiles, the last with 512). From 129 tiles up: an even K tile count from 6 up
     takes the direct-to-LDS pipeline with early fragment reads (6 and 8 K tiles here), the others the
     direct-to-LDS ring of 256 x 256 tiles (3 and 7 K tiles). Two shapes have 289 and 324 tiles for 256 CUs: the 33 or
     68 tiles of the partial second round are cut into 128 x 128 tiles by a second launch (the four-deep ring for
