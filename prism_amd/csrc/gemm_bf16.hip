@@ -1180,17 +1180,36 @@ int run_gemm_bf16(int R, int Cn, int K, const uint16_t* P, const uint16_t* Q, Ou
             <<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n, -1);
         return check_launch("gemm_bf16_ring_kernel");
     }
+    // The edge forms of the early-read kernel. As with whole tiles, the tiles of a partial last round (at most half
+    // the CUs' worth) are cut into 128 x 128 tiles of the ring, two workgroups per CU (8190^3: 1089 tiles, 4 rounds
+    // and 65 tiles cut into 260 instead of 5 rounds).
+    auto edge_tiles = [&](auto ragged, const char* what) -> int {
+        constexpr bool RG = decltype(ragged)::value;
+        const int tiles = tiles_m * tiles_n, cus = cu_count();
+        const int left = tiles % cus;
+        const bool cut = tiles > cus && left != 0 && left * 4 <= 2 * cus;
+        const int main_tiles = cut ? tiles - left : tiles;
+        gemm_bf16_early_kernel<BM, BN, WM, WN, true, OutT, RG><<<dim3(static_cast<unsigned>(main_tiles)), block, 0, s>>>(
+            R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
+        if (int rc = check_launch(what)) return rc;
+        if (cut) {
+            if (left * 4 <= cus && K >= 256)
+                gemm_bf16_ring_kernel<128, 128, 64, 4, 64, 64, true, OutT, RG><<<dim3(static_cast<unsigned>(left) * 4), dim3(256), 0, s>>>(
+                    R, Cn, K, P, Q, OUT, tiles_m, tiles_n, main_tiles);
+            else
+                gemm_bf16_ring_kernel<128, 128, 64, 2, 64, 64, true, OutT, RG><<<dim3(static_cast<unsigned>(left) * 4), dim3(256), 0, s>>>(
+                    R, Cn, K, P, Q, OUT, tiles_m, tiles_n, main_tiles);
+            return check_launch("gemm_bf16_ring_kernel (leftover, edges)");
+        }
+        return 0;
+    };
     // Ragged M, N or K with 16 B-aligned rows: the early-read kernel with zero-filled edges.
-    if (aligned && K % 8 == 0 && K > 0 && panel_ok && lane_offsets_ok) {
-        gemm_bf16_early_kernel<BM, BN, WM, WN, true, OutT><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
-        return check_launch("gemm_bf16_early_kernel (edges)");
-    }
+    if (aligned && K % 8 == 0 && K > 0 && panel_ok && lane_offsets_ok)
+        return edge_tiles(std::false_type{}, "gemm_bf16_early_kernel (edges)");
     // Rows that are not 16 B aligned (K not a multiple of 8, or operands at an odd element): its ragged form,
     // when there are enough tiles for the CUs and at least one group of 8 along K.
-    if (!few_tiles && K >= 8 && panel_ok && lane_offsets_ok) {
-        gemm_bf16_early_kernel<BM, BN, WM, WN, true, OutT, true><<<grid, block, 0, s>>>(R, Cn, K, P, Q, OUT, tiles_m, tiles_n);
-        return check_launch("gemm_bf16_early_kernel (ragged rows)");
-    }
+    if (!few_tiles && K >= 8 && panel_ok && lane_offsets_ok)
+        return edge_tiles(std::true_type{}, "gemm_bf16_early_kernel (ragged rows)");
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<BM, BN, BK, WM, WN, true, OutT>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(gemm_bf16_kernel)");

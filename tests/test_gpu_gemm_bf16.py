@@ -88,7 +88,7 @@ def nan_fenced(a16: np.ndarray, start: int = 1024) -> torch.Tensor:
 @pytest.mark.parametrize("shape", [(1, 1, 8), (257, 255, 8), (300, 520, 392), (255, 513, 456), (512, 512, 72), (1000, 1000, 1000),
                                    (256, 256, 64), (8, 8, 1032), (264, 24, 6152), (777, 300, 128),
                                    (3000, 3080, 392), (2900, 3100, 72), (3072, 3072, 8), (3000, 3072, 264), (2816, 3000, 328),
-                                   (2500, 2300, 264), (3000, 3072, 1288)])
+                                   (2500, 2300, 264), (3000, 3072, 1288), (4200, 4300, 392), (4600, 4700, 136)])
 def test_ragged_shapes_with_aligned_rows(prism, oracle, shape):
     """M, N not whole tiles or K not a multiple of 64, K a multiple of 8: the kernels' edge variants
     (rows beyond the matrix and K tiles beyond K read as zeros through the buffer descriptor's range
@@ -96,7 +96,8 @@ def test_ragged_shapes_with_aligned_rows(prism, oracle, shape):
     deep for K below that and for the 360 tiles of the shape before the last), the direct-to-LDS pipeline with early fragment
     reads from 128 tiles of 256 x 256 up (the last shape, 21 K tiles padded to 22 and walked from staggered
     starting points, and the five shapes before the last two: K tile counts of 7, 2, 1, 5 and 6 before
-    padding to an even count of at least 4). The matrices sit between NaNs, so one element read from outside a
+    padding to an even count of at least 4); the last two shapes have 289 and 342 tiles for 256 CUs, whose partial
+    second round (33 and 86 tiles) is cut into 128 x 128 edge tiles of the ring, four and two deep. The matrices sit between NaNs, so one element read from outside a
     matrix, or from the next row in the partial K tile, would poison the output; stores are fenced too."""
     check_between_fences(prism, oracle, shape)
 
@@ -134,13 +135,15 @@ def check_between_fences(prism, oracle, shape):
 
 @pytest.mark.parametrize("shape", [(3000, 3080, 393), (2900, 3100, 75), (3072, 3072, 9), (3000, 3072, 647), (3072, 3072, 15),
                                    (3072, 3072, 264), (2817, 3001, 406),
-                                   (1001, 1001, 1001), (300, 520, 395), (257, 255, 9), (64, 64, 8), (2001, 1999, 130), (1000, 1000, 264)])
+                                   (1001, 1001, 1001), (300, 520, 395), (257, 255, 9), (64, 64, 8), (2001, 1999, 130), (1000, 1000, 264),
+                                   (4200, 4290, 393), (4700, 4600, 139)])
 def test_rows_not_16_byte_aligned(prism, oracle, shape):
     """K not a multiple of 8, or operands that start at an odd element: rows are then only 2 B or 4 B aligned
     and, from 128 tiles of 256 x 256 up, the early-read kernel runs in its ragged form: 16 B direct loads from
     2 B-aligned addresses, a K loop over K rounded down to a multiple of 8 (1 to 11 tiles here, padded to an
-    even count of at least 4), and the last K % 8 values of k added on the way out; the last six shapes are small
-    problems for the ragged form of the ring of 128 x 128 tiles (two and four deep). The matrices sit between
+    even count of at least 4), and the last K % 8 values of k added on the way out; the six shapes before the last two are
+    small problems for the ragged form of the ring of 128 x 128 tiles (two and four deep), and the last two leave a
+    partial second round (33 and 86 tiles of 256 x 256) that the same ring finishes. The matrices sit between
     NaNs at an even and at an odd element; stores are fenced; fp32 and bf16 outputs."""
     M, N, K = shape
     A16, B16 = oracle.gen_gemm_bf16(M, N, K, seed=5 * M + N + K)
