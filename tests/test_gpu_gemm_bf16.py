@@ -77,6 +77,29 @@ def test_whole_tile_paths(prism, oracle, shape):
     assert np.all(np.abs(c - ref) <= 2.0**-8 * np.abs(ref) + REL * np.abs(ref).max())
 
 
+@pytest.mark.parametrize("shape", [(3072, 3072, 384), (4352, 4352, 384)])
+def test_whole_tiles_with_outputs_at_odd_elements(prism, oracle, shape):
+    """Whole tiles write unguarded 16 B packets: fp32 rows in packets of four values, bf16 rows as runs of 16 B that
+    went through LDS. The interface asks only element alignment of the outputs, so here D starts at an odd float
+    and C at an odd bf16 element, between fences. One launch of one tile per workgroup (144 tiles) and the walking
+    launch with a cut partial round (289 tiles)."""
+    M, N, K = shape
+    A16, B16 = oracle.gen_gemm_bf16(M, N, K, seed=K + 3 * M)
+    ref = oracle.gemm_bf16_f64(A16, B16)
+    buf = torch.full((M * N + 512,), 777.0, dtype=torch.float32, device=DEV)
+    prism.gemm_bf16(dev16(A16), dev16(B16), buf[255:255 + M * N].view(M, N))
+    out = host(buf)
+    assert np.all(out[:255] == 777.0) and np.all(out[255 + M * N:] == 777.0)
+    check_f32(oracle, out[255:255 + M * N].reshape(M, N), A16, B16, ref)
+    Cc = torch.full((N * M + 64,), -7.0, dtype=torch.bfloat16, device=DEV)
+    prism.runmyh100(M, N, K, dev16(A16), dev16(B16), Cc[31:31 + N * M])
+    got = host(Cc.view(torch.int16)).view(np.uint16)
+    guard = np.float32(-7.0).view(np.uint32) >> 16
+    assert np.all(got[:31] == guard) and np.all(got[31 + N * M:] == guard)
+    c = oracle.bf16_to_f32(got[31:31 + N * M]).reshape(N, M).T
+    assert np.all(np.abs(c - ref) <= 2.0**-8 * np.abs(ref) + REL * np.abs(ref).max())
+
+
 def nan_fenced(a16: np.ndarray, start: int = 1024) -> torch.Tensor:
     """The matrix as a view into a device buffer whose other elements are bf16 NaN patterns; `start` is its
     first element's index (a multiple of 8 keeps it 16 B aligned)."""
