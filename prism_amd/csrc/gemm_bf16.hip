@@ -646,8 +646,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
 
     __shared__ __attribute__((aligned(1024))) uint16_t Ps[2][BM * BK];
     __shared__ __attribute__((aligned(1024))) uint16_t Qs[2][BN * BK];
-    // bf16 output of whole tiles: 16 rows x WN columns per wave on their way out (see write_back_bf16_rows below).
-    constexpr bool ROWS_OUT = !EDGE && std::is_same<OutT, uint16_t>::value;
+    // Whole tiles: 16 rows x WN columns of bf16, or x WN / 2 columns of fp32, per wave on their way out (see
+    // write_back_rows below).
+    constexpr bool ROWS_OUT = !EDGE;
     constexpr int OUT_LD = WN + 8;  // 272 B rows: the sixteen lanes of a 16-row column of packets hit 16 different bank pairs
     __shared__ __attribute__((aligned(16))) uint16_t Out_s[ROWS_OUT ? WAVES : 1][ROWS_OUT ? 16 * OUT_LD : 8];
     int tile = blockIdx.x;
@@ -941,13 +942,36 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
             }
         }
     };
-    // bf16 output, whole tiles: a lane's packet is 8 B, and its neighbours' packets lie in other rows (lane l holds row
-    // l % 16), so one store instruction would be 64 separate 8 B writes, which cost the memory pipeline as much as 64
-    // wider ones: 8 us per tile and CU against 2.3 us for the same bytes written as 256 B runs. So 16 rows at a time
-    // go through LDS: packets in (a wave's own 16 x 128 patch, rows padded by 16 B), rows out, 16 B per lane, sixteen
+    // Whole tiles: a lane's packet of four results is 8 B of bf16 or 16 B of fp32, and its neighbours' packets lie in
+    // other rows (lane l holds row l % 16), so one store instruction would be 64 separate writes, which cost the memory
+    // pipeline as much as 64 wider ones: in a store-only loop 8 us per bf16 tile and CU against 2.3 us for the same
+    // bytes written as 256 B runs (fp32, with output that stays in L2: 7.2 against 4.6). So 16 rows at a time go through
+    // LDS: packets in (a wave's own patch of 16 rows x 256 B, rows padded by 16 B), rows out, 16 B per lane, sixteen
     // lanes to a row, four rows to a store. LDS executes a wave's accesses in order: no waits between the two.
-    auto write_back_bf16_rows = [&]() {
-        if constexpr (ROWS_OUT) {
+    // fp32 gains 1-3 % (16384 x 16384 x 1024: 14 %): a round's 67 MB from all CUs at once are bound by the write
+    // bandwidth whatever the pattern. bf16, together with the hardware's conversion: 17-30 % at K up to 1024.
+    auto write_back_rows = [&]() {
+        if constexpr (ROWS_OUT && std::is_same<OutT, float>::value) {
+            typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+            char* mine = reinterpret_cast<char*>(Out_s[wave]);
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+#pragma unroll
+                for (int jh = 0; jh < 2; ++jh) {
+#pragma unroll
+                    for (int jj = 0; jj < 4; ++jj)
+                        *reinterpret_cast<f32x4*>(mine + l16 * (OUT_LD * 2) + jj * 64 + lq * 16) = acc[i][4 * jh + jj];
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) {
+                        const int in_block = 4 * p + lq;
+                        const f32x4 v = *reinterpret_cast<const f32x4*>(mine + in_block * (OUT_LD * 2) + 16 * l16);
+                        const int row = row0 + wave_m * WM + i * 16 + in_block;
+                        const int col = col0 + wave_n * WN + jh * 64 + 4 * l16;
+                        *reinterpret_cast<f32x4_a4*>(&OUT[static_cast<size_t>(row) * Cn + col]) = v;
+                    }
+                }
+            }
+        } else if constexpr (ROWS_OUT) {
             typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
             typedef uint32_t u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
             uint16_t* mine = Out_s[wave];
@@ -1000,7 +1024,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * kWave) void gemm_bf16_early
         // PERSIST: the next tile's first two K tiles (fetched by the last two phases) land before the stores queue up
         // behind them; its first phase relies on that.
         if constexpr (PERSIST) __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kLgkmMax));
-        if constexpr (ROWS_OUT) write_back_bf16_rows();
+        if constexpr (ROWS_OUT) write_back_rows();
         else if (!EDGE || (row0 + BM <= R && col0 + BN <= Cn)) write_back(std::false_type{});
         else write_back(std::true_type{});
     }
