@@ -12,8 +12,15 @@
 //                                               counts: direct-to-LDS ring of two stages
 //                                               (gemm_bf16_ring_kernel)
 //   1 producer + 2 consumer warpgroups      ->  every wave loads and multiplies
-//   persistent CTAs + 16x8 super-tiles      ->  one workgroup per tile, 16x16 super-blocks with an
-//                                               8x4 patch per XCD (tile_map.h)
+//   persistent CTAs + 16x8 super-tiles      ->  with more tiles than CUs one workgroup per CU that walks
+//                                               its tiles and fetches the next tile's first K tiles in
+//                                               the last phases of the current one, else one workgroup
+//                                               per tile; 16x16 super-blocks with an 8x4 patch per XCD
+//                                               (tile_map.h)
+//   epilogue: registers -> global           ->  whole tiles leave as 256 B runs of rows through a wave's
+//                                               own LDS patch, bf16 converted in hardware; a few rows or
+//                                               columns beyond whole tiles run as strips
+//                                               (gemm_bf16_thin_kernel)
 //   K tail dropped, M/N multiples required  ->  any M, N, K. Ragged M, N, K with K a multiple of 8
 //                                               (16 B-aligned rows): the same kernels, edges zero-filled
 //                                               by the buffer loads' range check. K not a multiple of 8
