@@ -253,6 +253,30 @@ def bench_gemm_bf16(prism, n, steps, warmup, gate=True):
                          "frac": tflops / PEAK["bf16_mfma_TFLOPs"], "traffic": measured_traffic("gemm_bf16", n)}}
 
 
+def bench_runmyh100(prism, n, steps, warmup):
+    """The same product through the reference harness's entry (evals/h100_bench/utils.cuh:504-533): bf16 column-major
+    C[n * M + m], gated against the fp64 product at bf16's rounding step."""
+    import torch
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0)
+    A = torch.randn((n, n), dtype=torch.float32, device="cuda", generator=g).to(torch.bfloat16)
+    B = torch.randn((n, n), dtype=torch.float32, device="cuda", generator=g).to(torch.bfloat16)
+    Cc = torch.empty((n, n), dtype=torch.bfloat16, device="cuda")
+    lib, st = _capi()
+    a, b, c = A.data_ptr(), B.data_ptr(), Cc.data_ptr()
+    if lib.prism_runmyh100(n, n, n, a, b, c, None) != 0:
+        raise RuntimeError("prism_runmyh100 failed")
+    torch.cuda.synchronize()
+    err, ref_max = gemm_bf16_max_err_fp64(A, B, Cc.T)   # C is column-major: its transpose view is M x N
+    if not err <= 2.0 ** -8 * ref_max:
+        raise RuntimeError(f"runmyh100 n={n} failed the parity gate: err {err}")
+    ms = time_steps(lambda: lib.prism_runmyh100(n, n, n, a, b, c, None), steps, warmup)
+    tflops = 2.0 * n * n * n / (ms * 1e-3) / 1e12
+    return {"ms": ms, "tflops": tflops, "entry": "prism_runmyh100", "output": "bf16, column-major (the reference's)",
+            "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK["bf16_mfma_TFLOPs"], "unit": "TFLOP/s",
+                         "frac": tflops / PEAK["bf16_mfma_TFLOPs"], "traffic": None}}
+
+
 # ------------------------------------------------------- vendor libraries --
 
 def bench_vendor(steps, warmup):
@@ -450,6 +474,8 @@ def main() -> int:
     if want("gemm_bf16"):
         res["gemm_bf16"] = bench_gemm_bf16(prism, 8192, K, W)
         log("gemm_bf16 8192^3:", res["gemm_bf16"])
+        res["gemm_bf16_runmyh100"] = bench_runmyh100(prism, 8192, K, W)
+        log("gemm_bf16 8192^3 through prism_runmyh100:", res["gemm_bf16_runmyh100"])
     if want("add_m"):
         res["add_m"] = bench_add_m(prism, 1 << 24, max(K, 50), W)
         log("add_m 2^24:", res["add_m"])
