@@ -114,11 +114,14 @@ def write_traffic_table(pmc_dir: str) -> int:
 
 TRACE_FILE = ROOT / "profiles" / "bench_all_kernels_kernel_trace.md"
 PEAKS = {"sgemm": (157.3, "TFLOP/s fp32 MFMA"), "gemm_bf16": (2500.0, "TFLOP/s bf16 MFMA"),
-         "scan": (8000.0, "GB/s HBM"), "add_m": (8000.0, "GB/s HBM"), "add_m_2p28": (8000.0, "GB/s HBM")}
+         "gemm_bf16_runmyh100": (2500.0, "TFLOP/s bf16 MFMA"), "scan": (8000.0, "GB/s HBM"),
+         "scan_ticket_order": (8000.0, "GB/s HBM"), "add_m": (8000.0, "GB/s HBM"), "add_m_2p28": (8000.0, "GB/s HBM")}
 TRACE_KERNELS = [  # (key of the benchmark line, substring of the kernel name, work per launch, unit divisor)
     ("sgemm", "sgemm_wave_tile_dma_kernel<256, 256, 32, 32, 128, false, false, false>", 2.0 * 8192 ** 3, 1e12),
-    ("scan", "scan_lookback_kernel<prism::(anonymous namespace)::BigCfg", 8.0 * (1 << 30), 1e9),
-    ("gemm_bf16", "gemm_bf16_", 2.0 * 8192 ** 3, 1e12),
+    ("scan", "scan_lookback_kernel<prism::(anonymous namespace)::BigCfg, true, false, false", 8.0 * (1 << 30), 1e9),
+    ("scan_ticket_order", "scan_lookback_kernel<prism::(anonymous namespace)::BigCfg, true, true, false", 8.0 * (1 << 30), 1e9),
+    ("gemm_bf16", "gemm_bf16_early_kernel<256, 256, 128, 128, false, float", 2.0 * 8192 ** 3, 1e12),
+    ("gemm_bf16_runmyh100", "gemm_bf16_early_kernel<256, 256, 128, 128, false, unsigned short", 2.0 * 8192 ** 3, 1e12),
     ("add_m_2p28", "add_m_vec4_kernel<true>", 8.0 * (1 << 28), 1e9),
     ("add_m", "add_m_vec4_kernel<false>", 8.0 * (1 << 24), 1e9),
 ]
@@ -140,7 +143,8 @@ def write_kernel_trace_table(prof_dir: str) -> int:
            "the GPU box, R = repo root, OUT = a scratch directory):", "",
            "    rocprofv3 --kernel-trace --stats -d $OUT/prof_trace -o bench --output-format csv -- \\",
            "        python3 $R/bench.py --no-configs --no-cpu-baseline > $OUT/prof_trace/bench.json", "",
-           "Workloads: sgemm 8192^3 (kernel 5, alpha 1, beta 0.5), scan int32 n=2^30, gemm_bf16 8192^3, add_m n=2^24 and 2^28.",
+           "Workloads: sgemm 8192^3 (kernel 5, alpha 1, beta 0.5), scan int32 n=2^30 (tiles by workgroup id, and by ticket), gemm_bf16 8192^3 (fp32 output, and",
+           "the reference harness's entry with bf16 column-major output), add_m n=2^24 and 2^28.",
            f"Each kernel runs once for the parity gate, for {line.get('settle_ms', 150):.0f} ms of untimed settling, {line['warmup']} warm-up and {line['steps']} timed steps,",
            "hence the call counts; the profiler's average covers all of them (the cold first call is the `max` column), the",
            "last column is the benchmark's own event timing of the timed steps of the same run.", "",
