@@ -48,7 +48,7 @@ def measured_traffic(workload: str, size: int):
 TRAFFIC_KERNELS = [  # (workload, size, substring of the kernel name, threads in the grid)
     ("sgemm", 8192, "sgemm_wave_tile_dma_kernel", 1024 * 1024),
     ("scan", 1 << 30, "scan_lookback_kernel", (1 << 30) // 65536 * 1024),
-    ("gemm_bf16", 8192, "gemm_bf16_early_kernel", 256 * 256),  # one workgroup per CU walks four tiles
+    ("gemm_bf16", 8192, "gemm_bf16_early_kernel<256, 256, 128, 128, false, float", 256 * 256),  # fp32 output; one workgroup per CU walks four tiles
     ("add_m", 1 << 24, "add_m_vec4_kernel", (1 << 24) // 4),
     ("add_m", 1 << 28, "add_m_vec4_kernel", (1 << 28) // 4),
 ]
