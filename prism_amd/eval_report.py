@@ -180,13 +180,24 @@ def sweep_h100(out=sys.stdout, sizes=H100_SIZES, repeats: int = 8) -> None:
         Cc = torch.empty((n, n), dtype=torch.bfloat16, device="cuda")  # column-major M x N, as the reference
         flops = 2.0 * n * n * n
         fn = lambda: lib.prism_runmyh100(n, n, n, A.data_ptr(), B.data_ptr(), Cc.data_ptr(), None)
-        fn()
-        ms = _events_ms(fn, repeats)
-        print(h100_line("Kernel:", ms / 1e3 / repeats, repeats * flops * 1e-9 / ms, n), file=out)
         # hipBLASLt, same operands and the same bf16 column-major result as the harness asks of cuBLAS (main.cu:64-73)
         Cv = torch.empty_like(Cc)
         vend = lambda: vendor.vendor_gemm_bf16_colmajor(n, n, n, A.data_ptr(), B.data_ptr(), Cv.data_ptr(), None)
+        # The harness's order (main.cu:122-167): the library once, the kernel once, the two results compared, then
+        # the kernel's timed launches, then the library's. The harness allows 0.1 absolute; here that, or one rounding
+        # step of bf16 where a step is larger (from |C| = 16 up: two correct roundings of sums that differ in their last
+        # fp32 bits may be a step apart).
         _ok(vend())
+        _ok(fn())
+        torch.cuda.synchronize()
+        worst = 0.0
+        for r0 in range(0, n, 2048):
+            a, b = Cc[r0:r0 + 2048].float(), Cv[r0:r0 + 2048].float()
+            worst = max(worst, float(((a - b).abs() - (2.0 ** -7 * torch.maximum(a.abs(), b.abs())).clamp(min=0.1)).max()))
+        print("Passed correctness verification!" if worst <= 0.0 else
+              f"Failed to pass correctness verification against hipBLASLt (beyond 0.1 and one bf16 step by {worst:g}).", file=out)
+        ms = _events_ms(fn, repeats)
+        print(h100_line("Kernel:", ms / 1e3 / repeats, repeats * flops * 1e-9 / ms, n), file=out)
         ms = _events_ms(vend, repeats)
         print(h100_line("cuBLAS:", ms / 1e3 / repeats, repeats * flops * 1e-9 / ms, n) + "\n", file=out)
         out.flush()

@@ -76,9 +76,11 @@ def test_sweeps_produce_parseable_reports():
     assert [r[0] for r in rows] == [1 << 20, 1 << 22] and all(r[1] > 0 and r[2] > 0 for r in rows)
 
     buf = io.StringIO()
-    er.sweep_h100(buf, sizes=(2048,), repeats=3)
+    er.sweep_h100(buf, sizes=(2048, 4352), repeats=3)
     text = buf.getvalue()
     assert re.search(H100_KERNEL, text) and re.search(H100_VENDOR, text)
+    # the harness's comparison with the vendor library (evals/h100_bench/main.cu:122-135), once per size
+    assert text.count("Passed correctness verification!") == 2 and "Failed" not in text
 
 
 @pytest.mark.gpu
